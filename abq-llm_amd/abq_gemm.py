@@ -1,0 +1,220 @@
+"""ctypes binding of libabq_gemm.so (the C ABI in include/abq_gemm.h).
+
+Plumbing for the tests, the smoke check and the benchmark: device buffers are torch tensors,
+their data_ptr() goes straight through the C ABI.  There is no CPU fallback here: if the
+shared library is missing or the HIP launch fails, the call raises.
+
+Import torch before this module so that the library binds to the HIP runtime torch loaded.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libabq_gemm.so")
+
+ABQ_OK = 0
+STATUS_NAMES = {
+    0: "ABQ_OK", 1: "ABQ_ERR_INVALID_ARG", 2: "ABQ_ERR_BAD_K", 3: "ABQ_ERR_UNSUPPORTED",
+    4: "ABQ_ERR_NOT_INITIALIZED", 5: "ABQ_ERR_LAUNCH", 6: "ABQ_ERR_NO_DEVICE", 7: "ABQ_ERR_TOO_LARGE",
+}
+OUT_I32, OUT_F16_TENSOR, OUT_F16_SCALED = 0, 1, 2
+STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC = range(5)
+STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic"]
+
+# every symbol include/abq_gemm.h declares
+EXPORTED = [
+    "abq_status_string", "abq_last_hip_error", "abq_version",
+    "abq_pack_i32", "abq_pack_u4", "abq_pack_f16",
+    "abq_parse_kernel_name", "abq_format_kernel_name",
+    "abq_native_config_count", "abq_native_config_get",
+    "abq_gemm_init", "abq_gemm_set_scales", "abq_gemm_exec", "abq_gemm_launch",
+]
+
+
+class TileConfig(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int) for n in (
+        "x_bits", "w_bits", "is_signed", "block_m", "block_n", "block_k",
+        "warp_m", "warp_n", "warp_k", "mma_m", "mma_n", "mma_k", "nstage")]
+
+    def as_tuple(self):
+        return tuple(getattr(self, n) for n, _ in self._fields_)
+
+    def __repr__(self):
+        return "TileConfig(%s)" % ", ".join("%s=%d" % (n, getattr(self, n)) for n, _ in self._fields_)
+
+
+class Dim3(ctypes.Structure):
+    _fields_ = [("x", ctypes.c_uint), ("y", ctypes.c_uint), ("z", ctypes.c_uint)]
+
+
+class GemmState(ctypes.Structure):
+    _fields_ = [
+        ("shared_mem_size", ctypes.c_size_t),
+        ("grid_dim", Dim3), ("block_dim", Dim3),
+        ("init_success", ctypes.c_int),
+        ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int),
+        ("X", ctypes.c_void_p), ("W", ctypes.c_void_p), ("C", ctypes.c_void_p), ("D", ctypes.c_void_p),
+        ("bias", ctypes.c_int),
+        ("cfg", TileConfig),
+        ("strategy", ctypes.c_int), ("variant", ctypes.c_int), ("out_kind", ctypes.c_int),
+        ("x_scale", ctypes.c_void_p), ("w_scale", ctypes.c_void_p),
+        ("group_size", ctypes.c_int),
+        ("reserved", ctypes.c_int * 5),
+    ]
+
+
+class AbqError(RuntimeError):
+    def __init__(self, status, what):
+        self.status = status
+        super().__init__("%s failed: %s (%d)" % (what, STATUS_NAMES.get(status, "?"), status))
+
+
+_lib = None
+
+
+def lib():
+    """Loads libabq_gemm.so; raises if it has not been built (no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libabq_gemm.so is not built: run `make -C %s` (or __graft_entry__.build())" % _HERE)
+        L = ctypes.CDLL(LIB_PATH)
+        vp, ci = ctypes.c_void_p, ctypes.c_int
+        L.abq_status_string.restype = ctypes.c_char_p
+        L.abq_status_string.argtypes = [ci]
+        L.abq_last_hip_error.restype = ci
+        L.abq_version.restype = ci
+        L.abq_pack_i32.argtypes = [vp, vp, ci, ci, ci, vp]
+        L.abq_pack_u4.argtypes = [vp, vp, ci, ci, ci, vp]
+        L.abq_pack_f16.argtypes = [vp, vp, vp, ci, ci, ci, vp]
+        L.abq_parse_kernel_name.argtypes = [ctypes.c_char_p, ctypes.POINTER(TileConfig), ctypes.POINTER(ci)]
+        L.abq_format_kernel_name.argtypes = [ctypes.POINTER(TileConfig), ci, ctypes.c_char_p, ctypes.c_size_t]
+        L.abq_native_config_count.argtypes = [ci, ci, ci]
+        L.abq_native_config_count.restype = ci
+        L.abq_native_config_get.argtypes = [ci, ci, ci, ci, ctypes.POINTER(TileConfig)]
+        L.abq_gemm_init.argtypes = [ctypes.POINTER(TileConfig), ci, ci, ci, vp, vp, ci, ci, ci, vp, vp, ci, ci,
+                                    ctypes.POINTER(GemmState)]
+        L.abq_gemm_set_scales.argtypes = [ctypes.POINTER(GemmState), vp, vp, ci]
+        L.abq_gemm_exec.argtypes = [ctypes.POINTER(GemmState), vp]
+        L.abq_gemm_launch.argtypes = [ctypes.POINTER(TileConfig), vp, vp, vp, vp, ci, ci, ci, ci, vp]
+        _lib = L
+    return _lib
+
+
+def _check(status, what):
+    if status != ABQ_OK:
+        raise AbqError(status, what)
+
+
+def _stream_ptr(stream):
+    if stream is None:
+        import torch
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    if isinstance(stream, int):
+        return ctypes.c_void_p(stream)
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def parse_kernel_name(name):
+    cfg, wmma = TileConfig(), ctypes.c_int(0)
+    _check(lib().abq_parse_kernel_name(name.encode(), ctypes.byref(cfg), ctypes.byref(wmma)), "abq_parse_kernel_name")
+    return cfg, bool(wmma.value)
+
+
+def format_kernel_name(cfg, is_wmma=False):
+    buf = ctypes.create_string_buffer(160)
+    _check(lib().abq_format_kernel_name(ctypes.byref(cfg), int(is_wmma), buf, 160), "abq_format_kernel_name")
+    return buf.value.decode()
+
+
+def native_configs(x_bits, w_bits, signed):
+    n = lib().abq_native_config_count(x_bits, w_bits, int(signed))
+    out = []
+    for i in range(n):
+        c = TileConfig()
+        _check(lib().abq_native_config_get(x_bits, w_bits, int(signed), i, ctypes.byref(c)), "abq_native_config_get")
+        out.append(c)
+    return out
+
+
+def planes_empty(bits, rows, k, device="cuda"):
+    import torch
+    return torch.empty((bits, rows, k // 32), dtype=torch.int32, device=device)
+
+
+def pack_i32(values, bits, out=None, stream=None):
+    """values: int32 device tensor [rows, k] -> planes int32 tensor [bits, rows, k/32]."""
+    import torch
+    assert values.dtype == torch.int32 and values.is_cuda and values.is_contiguous()
+    rows, k = values.shape
+    if out is None:
+        out = planes_empty(bits, rows, k, values.device)
+    _check(lib().abq_pack_i32(values.data_ptr(), out.data_ptr(), rows, k, bits, _stream_ptr(stream)), "abq_pack_i32")
+    return out
+
+
+def pack_u4(words, rows, k, bits=4, out=None, stream=None):
+    import torch
+    assert words.dtype == torch.int32 and words.is_cuda and words.is_contiguous()
+    assert words.numel() == rows * k // 8
+    if out is None:
+        out = planes_empty(bits, rows, k, words.device)
+    _check(lib().abq_pack_u4(words.data_ptr(), out.data_ptr(), rows, k, bits, _stream_ptr(stream)), "abq_pack_u4")
+    return out
+
+
+def pack_f16(values, scale, bits, out=None, stream=None):
+    """values: fp16 device tensor [rows, k]; scale: float32 device tensor with one element."""
+    import torch
+    assert values.dtype == torch.float16 and values.is_cuda and values.is_contiguous()
+    assert scale.dtype == torch.float32 and scale.is_cuda
+    rows, k = values.shape
+    if out is None:
+        out = planes_empty(bits, rows, k, values.device)
+    _check(lib().abq_pack_f16(values.data_ptr(), scale.data_ptr(), out.data_ptr(), rows, k, bits,
+                              _stream_ptr(stream)), "abq_pack_f16")
+    return out
+
+
+class Gemm:
+    """One initialised GEMM (the role of AqBMMAOpState + InitFn/ExecFn in the reference)."""
+
+    def __init__(self, x_planes, w_planes, signed, out=None, cfg=None, out_kind=OUT_I32, c_scale=None,
+                 x_scale=None, w_scale=None, group_size=0):
+        import torch
+        q, M, kw = x_planes.shape
+        p, N, kw2 = w_planes.shape
+        assert kw == kw2 and x_planes.is_cuda and w_planes.is_cuda
+        assert x_planes.is_contiguous() and w_planes.is_contiguous()
+        K = kw * 32
+        if out is None:
+            out = torch.empty((M, N), dtype=torch.int32 if out_kind == OUT_I32 else torch.float16,
+                              device=x_planes.device)
+        self.out, self.x_planes, self.w_planes = out, x_planes, w_planes
+        self.c_scale, self.x_scale, self.w_scale = c_scale, x_scale, w_scale
+        self.state = GemmState()
+        cfg_ptr = ctypes.byref(cfg) if cfg is not None else None
+        st = lib().abq_gemm_init(cfg_ptr, q, p, int(bool(signed)), x_planes.data_ptr(), w_planes.data_ptr(),
+                                 M, N, K, out.data_ptr(), c_scale.data_ptr() if c_scale is not None else None,
+                                 0, out_kind, ctypes.byref(self.state))
+        _check(st, "abq_gemm_init")
+        if out_kind == OUT_F16_SCALED:
+            _check(lib().abq_gemm_set_scales(ctypes.byref(self.state), x_scale.data_ptr(), w_scale.data_ptr(),
+                                             group_size), "abq_gemm_set_scales")
+
+    @property
+    def strategy(self):
+        return STRATEGY_NAMES[self.state.strategy]
+
+    @property
+    def config_name(self):
+        return format_kernel_name(self.state.cfg)
+
+    def run(self, stream=None):
+        _check(lib().abq_gemm_exec(ctypes.byref(self.state), _stream_ptr(stream)), "abq_gemm_exec")
+        return self.out
+
+
+def gemm(x_planes, w_planes, signed, **kw):
+    return Gemm(x_planes, w_planes, signed, **kw).run()

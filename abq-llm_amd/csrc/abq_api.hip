@@ -1,0 +1,510 @@
+// Host side of the C ABI declared in include/abq_gemm.h: argument checking, the kernel
+// registry (tile tuple -> instantiation), the default strategy choice and the launches.
+// No entry point allocates device or host memory.
+#include "abq_gemm.h"
+
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "abq_kernels.h"
+
+namespace abq {
+
+hipError_t launch_pack_i32(const int32_t *, uint32_t *, int, int, int, hipStream_t);
+hipError_t launch_pack_f16(const void *, const float *, uint32_t *, int, int, int, hipStream_t);
+hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
+
+// (x_bits, w_bits) pairs with specialised kernels: the twelve of the reference library
+// (engine/mma_any/aq_bmma_impl/aq_bmma_w{2a2,...,8a8}.h).
+#define ABQ_FOR_EACH_COMBO(F) \
+    F(2, 2) F(4, 2) F(6, 2) F(8, 2) F(3, 3) F(8, 3) F(4, 4) F(8, 4) F(5, 5) F(6, 6) F(7, 7) F(8, 8)
+#define ABQ_NUM_COMBOS 12
+
+#define ABQ_DECL(Q, P)                                \
+    void abq_mfma_register_##Q##_##P(KernelTable *);  \
+    void abq_bcnt_register_##Q##_##P(KernelTable *);
+ABQ_FOR_EACH_COMBO(ABQ_DECL)
+#undef ABQ_DECL
+
+struct Registry {
+    KernelTable mfma[2 * ABQ_NUM_COMBOS];
+    KernelTable bcnt[2 * ABQ_NUM_COMBOS];
+    Registry()
+    {
+        int i = 0;
+#define ABQ_REG(Q, P)                                  \
+    abq_mfma_register_##Q##_##P(&mfma[i]);             \
+    abq_bcnt_register_##Q##_##P(&bcnt[i]);             \
+    i += 2;
+        ABQ_FOR_EACH_COMBO(ABQ_REG)
+#undef ABQ_REG
+    }
+};
+
+static const Registry &registry()
+{
+    static const Registry r;
+    return r;
+}
+
+static const KernelTable *find_table(const KernelTable *tables, int x_bits, int w_bits, int is_signed)
+{
+    for (int i = 0; i < 2 * ABQ_NUM_COMBOS; ++i)
+        if (tables[i].x_bits == x_bits && tables[i].w_bits == w_bits &&
+            tables[i].is_signed == (is_signed ? 1 : 0))
+            return &tables[i];
+    return nullptr;
+}
+
+static thread_local int g_last_hip_error = 0;
+
+static abq_status hip_status(hipError_t e)
+{
+    if (e == hipSuccess)
+        return ABQ_OK;
+    g_last_hip_error = (int)e;
+    return e == hipErrorNoDevice || e == hipErrorInvalidDevice ? ABQ_ERR_NO_DEVICE : ABQ_ERR_LAUNCH;
+}
+
+// ---- tile tuple <-> kernel entry ---------------------------------------------------------
+
+static void entry_to_config(const KernelEntry &e, int strategy, int x_bits, int w_bits,
+                            int is_signed, int lpr_log2, abq_tile_config *c)
+{
+    c->x_bits = x_bits;
+    c->w_bits = w_bits;
+    c->is_signed = is_signed ? 1 : 0;
+    if (strategy == ABQ_STRATEGY_BCNT) {
+        const int lpr = 1 << lpr_log2;
+        c->block_m = e.tm;
+        c->block_n = 4 * (64 / lpr);
+        c->block_k = lpr * 128;
+        c->warp_m = e.tm;
+        c->warp_n = 64 / lpr;
+        c->warp_k = lpr * 128;
+        c->mma_m = 1;
+        c->mma_n = 1;
+        c->mma_k = 128;
+        c->nstage = 1;
+    } else {
+        const int stepk = (64 / e.mi) * 4 * 32;
+        c->block_m = e.mi * e.tm * e.wm;
+        c->block_n = e.mi * e.tn * e.wn;
+        c->block_k = stepk * e.wk;
+        c->warp_m = e.mi * e.tm;
+        c->warp_n = e.mi * e.tn;
+        c->warp_k = stepk;
+        c->mma_m = e.mi;
+        c->mma_n = e.mi;
+        c->mma_k = 1024 / e.mi;
+        c->nstage = e.nstage;
+    }
+}
+
+static int strategy_of_mma(const abq_tile_config &c)
+{
+    if (c.mma_m == 1 && c.mma_n == 1 && c.mma_k == 128)
+        return ABQ_STRATEGY_BCNT;
+    if (c.mma_m == 16 && c.mma_n == 16 && c.mma_k == 64)
+        return ABQ_STRATEGY_MFMA16;
+    if (c.mma_m == 32 && c.mma_n == 32 && c.mma_k == 32)
+        return ABQ_STRATEGY_MFMA32;
+    return ABQ_STRATEGY_AUTO;
+}
+
+// Lanes per weight row for the popcount kernels: the power of two in [16, 64] that wastes
+// the fewest lanes for this K (a row has K/128 sixteen-byte units).
+static int best_lpr_log2(int K)
+{
+    const int units = K / 128;
+    int best = 6;
+    double best_eff = 0;
+    for (int l = 4; l <= 6; ++l) {
+        const int lpr = 1 << l;
+        const int iters = (units + lpr - 1) / lpr;
+        const double eff = (double)units / (iters * lpr);
+        if (eff > best_eff + 1e-9 || (eff > best_eff - 1e-9 && l > best)) {
+            best_eff = eff;
+            best = l;
+        }
+    }
+    return best;
+}
+
+static int find_mfma_variant(const KernelTable &t, int mi, int tm, int tn, int wm, int wn, int wk)
+{
+    for (int i = 0; i < t.count; ++i) {
+        const KernelEntry &e = t.entries[i];
+        if (e.mi == mi && e.tm == tm && e.tn == tn && e.wm == wm && e.wn == wn && e.wk == wk)
+            return i;
+    }
+    return -1;
+}
+
+// Default choice when the caller names no native tile: popcount for one or two activation
+// rows, 16-row MFMA tiles with K split over the waves up to 16 rows, 32-row MFMA tiles above.
+static void choose_default(int M, int N, int *strategy, int *mi, int *tm, int *tn, int *wm, int *wn,
+                           int *wk)
+{
+    if (M <= 2) {
+        *strategy = ABQ_STRATEGY_BCNT;
+        *mi = 1; *tm = M; *tn = 1; *wm = 1; *wn = 4; *wk = 1;
+    } else if (M <= 16) {
+        *strategy = ABQ_STRATEGY_MFMA16;
+        *mi = 16; *tm = 1; *tn = 1; *wm = 1; *wn = 1; *wk = 8;
+    } else {
+        *strategy = ABQ_STRATEGY_MFMA32;
+        *mi = 32; *wm = 2; *wn = 2; *wk = 1;
+        const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+        if (M > 64 && tiles128 >= 256) {
+            *tm = 2; *tn = 2;
+        } else if (M > 32) {
+            *tm = 1; *tn = 2;
+        } else {
+            *tm = 1; *tn = 1;
+        }
+    }
+}
+
+static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, int is_signed, int M,
+                          int N, int K, abq_gemm_state *st)
+{
+    const Registry &reg = registry();
+    int strategy = cfg ? strategy_of_mma(*cfg) : ABQ_STRATEGY_AUTO;
+    const KernelTable *tm_ = find_table(reg.mfma, x_bits, w_bits, is_signed);
+    const KernelTable *tb_ = find_table(reg.bcnt, x_bits, w_bits, is_signed);
+    if (!tm_ || !tb_) {
+        // no specialised instantiation: run-time loop kernel, one activation row per grid row
+        if (x_bits < 1 || x_bits > 16 || w_bits < 1 || w_bits > 16)
+            return ABQ_ERR_UNSUPPORTED;
+        if (M > 65535)
+            return ABQ_ERR_TOO_LARGE;
+        st->strategy = ABQ_STRATEGY_GENERIC;
+        st->variant = 0;
+        st->cfg = abq_tile_config{ x_bits, w_bits, is_signed ? 1 : 0, 1, 4, 2048, 1, 1, 2048, 1, 1, 32, 1 };
+        st->grid_dim = abq_dim3{ (unsigned)((N + 3) / 4 > 65536 ? 65536 : (N + 3) / 4), (unsigned)M, 1 };
+        st->block_dim = abq_dim3{ 256, 1, 1 };
+        st->shared_mem_size = 0;
+        return ABQ_OK;
+    }
+
+    int mi = 0, tm = 0, tn = 0, wm = 0, wn = 0, wk = 0;
+    int lpr_log2 = best_lpr_log2(K);
+    if (strategy == ABQ_STRATEGY_AUTO) {
+        choose_default(M, N, &strategy, &mi, &tm, &tn, &wm, &wn, &wk);
+    } else if (strategy == ABQ_STRATEGY_BCNT) {
+        mi = 1; tm = cfg->block_m; tn = 1; wm = 1; wn = 4; wk = 1;
+        // block_k = lanes per row * 128; accept 16, 32 or 64 lanes, else keep the best fit
+        const int lpr = cfg->block_k / 128;
+        if (cfg->block_k % 128 == 0 && (lpr == 16 || lpr == 32 || lpr == 64))
+            lpr_log2 = lpr == 16 ? 4 : lpr == 32 ? 5 : 6;
+    } else {
+        mi = cfg->mma_m;
+        const int stepk = (64 / mi) * 4 * 32;
+        if (cfg->warp_m <= 0 || cfg->warp_n <= 0 || cfg->warp_m % mi || cfg->warp_n % mi ||
+            cfg->block_m % cfg->warp_m || cfg->block_n % cfg->warp_n || cfg->warp_k != stepk ||
+            cfg->block_k % stepk)
+            return ABQ_ERR_UNSUPPORTED;
+        tm = cfg->warp_m / mi; tn = cfg->warp_n / mi;
+        wm = cfg->block_m / cfg->warp_m; wn = cfg->block_n / cfg->warp_n;
+        wk = cfg->block_k / stepk;
+    }
+
+    if (strategy == ABQ_STRATEGY_BCNT) {
+        int v = -1;
+        for (int i = 0; i < tb_->count; ++i)
+            if (tb_->entries[i].tm == tm)
+                v = i;
+        if (v < 0)
+            return ABQ_ERR_UNSUPPORTED;
+        const KernelEntry &e = tb_->entries[v];
+        const int rpp = 64 >> lpr_log2;
+        const int npass = (N + rpp - 1) / rpp;
+        if ((M + e.tm - 1) / e.tm > 65535)
+            return ABQ_ERR_TOO_LARGE;
+        st->strategy = strategy;
+        st->variant = v;
+        entry_to_config(e, strategy, x_bits, w_bits, is_signed, lpr_log2, &st->cfg);
+        st->grid_dim = abq_dim3{ (unsigned)((npass + 3) / 4 > 65536 ? 65536 : (npass + 3) / 4),
+                                 (unsigned)((M + e.tm - 1) / e.tm), 1 };
+        st->block_dim = abq_dim3{ 256, 1, 1 };
+        st->shared_mem_size = 0;
+        st->reserved[0] = lpr_log2;
+        return ABQ_OK;
+    }
+
+    const int v = find_mfma_variant(*tm_, mi, tm, tn, wm, wn, wk);
+    if (v < 0)
+        return ABQ_ERR_UNSUPPORTED;
+    const KernelEntry &e = tm_->entries[v];
+    // The signed path scales both operands to the top of the byte: |acc| <= K * 2^14.
+    if (K >= (1 << 17))
+        return ABQ_ERR_TOO_LARGE;
+    const int bm = e.mi * e.tm * e.wm, bn = e.mi * e.tn * e.wn;
+    if ((M + bm - 1) / bm > 65535)
+        return ABQ_ERR_TOO_LARGE;
+    st->strategy = strategy;
+    st->variant = v;
+    entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
+    st->grid_dim = abq_dim3{ (unsigned)((N + bn - 1) / bn), (unsigned)((M + bm - 1) / bm), 1 };
+    st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn * e.wk), 1, 1 };
+    const int acc = e.mi == 16 ? 4 : 16;
+    st->shared_mem_size = e.wk > 1 ? (size_t)e.wm * e.wn * (e.wk - 1) * (e.tm * e.tn * acc + e.tm + e.tn) * 64 * 4 : 0;
+    return ABQ_OK;
+}
+
+} // namespace abq
+
+using namespace abq;
+
+extern "C" {
+
+const char *abq_status_string(abq_status s)
+{
+    switch (s) {
+    case ABQ_OK: return "ok";
+    case ABQ_ERR_INVALID_ARG: return "invalid argument";
+    case ABQ_ERR_BAD_K: return "K must be >= 128 and a multiple of 128";
+    case ABQ_ERR_UNSUPPORTED: return "unsupported bit combination, tile tuple or option";
+    case ABQ_ERR_NOT_INITIALIZED: return "state not initialised";
+    case ABQ_ERR_LAUNCH: return "HIP launch failed";
+    case ABQ_ERR_NO_DEVICE: return "no usable HIP device";
+    case ABQ_ERR_TOO_LARGE: return "size exceeds a documented limit";
+    }
+    return "unknown status";
+}
+
+int abq_last_hip_error(void) { return g_last_hip_error; }
+int abq_version(void) { return ABQ_VERSION; }
+
+// ---- packing -----------------------------------------------------------------------------
+
+static abq_status check_pack(const void *in, const void *out, int rows, int k, int bits)
+{
+    if (!in || !out || rows <= 0 || k <= 0 || bits < 1 || bits > 32)
+        return ABQ_ERR_INVALID_ARG;
+    if (k % 32 != 0)
+        return ABQ_ERR_BAD_K;
+    return ABQ_OK;
+}
+
+abq_status abq_pack_i32(const int32_t *in, uint32_t *planes, int rows, int k, int bits, void *stream)
+{
+    abq_status s = check_pack(in, planes, rows, k, bits);
+    if (s != ABQ_OK)
+        return s;
+    return hip_status(launch_pack_i32(in, planes, rows, k, bits, (hipStream_t)stream));
+}
+
+abq_status abq_pack_u4(const uint32_t *in, uint32_t *planes, int rows, int k, int bits, void *stream)
+{
+    abq_status s = check_pack(in, planes, rows, k, bits);
+    if (s != ABQ_OK)
+        return s;
+    return hip_status(launch_pack_u4(in, planes, rows, k, bits, (hipStream_t)stream));
+}
+
+abq_status abq_pack_f16(const void *in_f16, const float *scale_dev, uint32_t *planes, int rows,
+                        int k, int bits, void *stream)
+{
+    abq_status s = check_pack(in_f16, planes, rows, k, bits);
+    if (s != ABQ_OK)
+        return s;
+    if (!scale_dev)
+        return ABQ_ERR_INVALID_ARG;
+    return hip_status(launch_pack_f16(in_f16, scale_dev, planes, rows, k, bits, (hipStream_t)stream));
+}
+
+// ---- names -------------------------------------------------------------------------------
+
+abq_status abq_parse_kernel_name(const char *name, abq_tile_config *cfg, int *is_wmma)
+{
+    if (!name || !cfg)
+        return ABQ_ERR_INVALID_ARG;
+    const char *p = name;
+    int wmma = 0;
+    if (strncmp(p, "AqBWMMA_", 8) == 0) {
+        wmma = 1;
+        p += 8;
+    } else if (strncmp(p, "AqBMMA_", 7) == 0) {
+        p += 7;
+    } else {
+        return ABQ_ERR_INVALID_ARG;
+    }
+    abq_tile_config c;
+    char sign[8] = { 0 };
+    int consumed = 0;
+    // 8x2xtrue_1x48x512_8x24x128_8x8x128_4
+    if (sscanf(p, "%dx%dx%5[a-z]_%dx%dx%d_%dx%dx%d_%dx%dx%d_%d%n", &c.x_bits, &c.w_bits, sign,
+               &c.block_m, &c.block_n, &c.block_k, &c.warp_m, &c.warp_n, &c.warp_k, &c.mma_m,
+               &c.mma_n, &c.mma_k, &c.nstage, &consumed) != 13)
+        return ABQ_ERR_INVALID_ARG;
+    if (strcmp(sign, "true") == 0)
+        c.is_signed = 1;
+    else if (strcmp(sign, "false") == 0)
+        c.is_signed = 0;
+    else
+        return ABQ_ERR_INVALID_ARG;
+    const char *rest = p + consumed;
+    if (*rest != '\0' && strcmp(rest, "_InitFn") != 0 && strcmp(rest, "_ExecFn") != 0)
+        return ABQ_ERR_INVALID_ARG;
+    *cfg = c;
+    if (is_wmma)
+        *is_wmma = wmma;
+    return ABQ_OK;
+}
+
+abq_status abq_format_kernel_name(const abq_tile_config *c, int is_wmma, char *buf, size_t n)
+{
+    if (!c || !buf || n == 0)
+        return ABQ_ERR_INVALID_ARG;
+    int w = snprintf(buf, n, "%s_%dx%dx%s_%dx%dx%d_%dx%dx%d_%dx%dx%d_%d", is_wmma ? "AqBWMMA" : "AqBMMA",
+                     c->x_bits, c->w_bits, c->is_signed ? "true" : "false", c->block_m, c->block_n,
+                     c->block_k, c->warp_m, c->warp_n, c->warp_k, c->mma_m, c->mma_n, c->mma_k,
+                     c->nstage);
+    return (w < 0 || (size_t)w >= n) ? ABQ_ERR_TOO_LARGE : ABQ_OK;
+}
+
+// Native tile space: popcount entries for 16/32/64 lanes per row, then the MFMA entries.
+int abq_native_config_count(int x_bits, int w_bits, int is_signed)
+{
+    const Registry &reg = registry();
+    const KernelTable *tb = find_table(reg.bcnt, x_bits, w_bits, is_signed);
+    const KernelTable *tm = find_table(reg.mfma, x_bits, w_bits, is_signed);
+    if (!tb || !tm)
+        return 0;
+    return tb->count * 3 + tm->count;
+}
+
+abq_status abq_native_config_get(int x_bits, int w_bits, int is_signed, int index, abq_tile_config *cfg)
+{
+    if (!cfg || index < 0)
+        return ABQ_ERR_INVALID_ARG;
+    const Registry &reg = registry();
+    const KernelTable *tb = find_table(reg.bcnt, x_bits, w_bits, is_signed);
+    const KernelTable *tm = find_table(reg.mfma, x_bits, w_bits, is_signed);
+    if (!tb || !tm)
+        return ABQ_ERR_UNSUPPORTED;
+    if (index < tb->count * 3) {
+        entry_to_config(tb->entries[index / 3], ABQ_STRATEGY_BCNT, x_bits, w_bits, is_signed,
+                        4 + index % 3, cfg);
+        return ABQ_OK;
+    }
+    index -= tb->count * 3;
+    if (index >= tm->count)
+        return ABQ_ERR_INVALID_ARG;
+    const KernelEntry &e = tm->entries[index];
+    entry_to_config(e, e.mi == 16 ? ABQ_STRATEGY_MFMA16 : ABQ_STRATEGY_MFMA32, x_bits, w_bits,
+                    is_signed, 0, cfg);
+    return ABQ_OK;
+}
+
+// ---- GEMM --------------------------------------------------------------------------------
+
+abq_status abq_gemm_init(const abq_tile_config *cfg, int x_bits, int w_bits, int is_signed,
+                         const uint32_t *X, const uint32_t *W, int M, int N, int K, void *D,
+                         const void *C, int bias, int out_kind, abq_gemm_state *state)
+{
+    if (!state)
+        return ABQ_ERR_INVALID_ARG;
+    memset(state, 0, sizeof(*state));
+    if (cfg) {
+        x_bits = cfg->x_bits;
+        w_bits = cfg->w_bits;
+        is_signed = cfg->is_signed;
+    }
+    if (!X || !W || !D || M <= 0 || N <= 0 || K <= 0)
+        return ABQ_ERR_INVALID_ARG;
+    if (x_bits < 1 || w_bits < 1)
+        return ABQ_ERR_INVALID_ARG;
+    if (bias) // the reference asserts !bias (engine/mma_any/aq_bmma_op.h:79)
+        return ABQ_ERR_UNSUPPORTED;
+    if (K < 128 || K % 128 != 0)
+        return ABQ_ERR_BAD_K;
+    if (out_kind != ABQ_OUT_I32 && out_kind != ABQ_OUT_F16_TENSOR && out_kind != ABQ_OUT_F16_SCALED)
+        return ABQ_ERR_INVALID_ARG;
+    if (out_kind == ABQ_OUT_F16_TENSOR && !C)
+        return ABQ_ERR_INVALID_ARG;
+    if ((long)M * N >= (1L << 31) || (long)M * (K / 32) >= (1L << 31) || (long)N * (K / 32) >= (1L << 31))
+        return ABQ_ERR_TOO_LARGE;
+
+    abq_status s = resolve(cfg, x_bits, w_bits, is_signed, M, N, K, state);
+    if (s != ABQ_OK)
+        return s;
+    state->M = M;
+    state->N = N;
+    state->K = K;
+    state->X = X;
+    state->W = W;
+    state->C = C;
+    state->D = D;
+    state->bias = 0;
+    state->out_kind = out_kind;
+    state->init_success = 1;
+    return ABQ_OK;
+}
+
+abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, const float *w_scale,
+                               int group_size)
+{
+    if (!state || !state->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    if (!x_scale || !w_scale)
+        return ABQ_ERR_INVALID_ARG;
+    if (group_size != 0) // grouped scales need a K-blocked main loop; not built yet
+        return ABQ_ERR_UNSUPPORTED;
+    state->x_scale = x_scale;
+    state->w_scale = w_scale;
+    state->group_size = group_size;
+    return ABQ_OK;
+}
+
+abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
+{
+    if (!st || !st->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    if (st->out_kind == ABQ_OUT_F16_SCALED && (!st->x_scale || !st->w_scale))
+        return ABQ_ERR_INVALID_ARG;
+    GemmArgs a;
+    a.X = st->X;
+    a.W = st->W;
+    a.D = st->D;
+    a.C = st->C;
+    a.x_scale = st->x_scale;
+    a.w_scale = st->w_scale;
+    a.M = st->M;
+    a.N = st->N;
+    a.K = st->K;
+    a.KW = st->K / 32;
+    a.out_kind = st->out_kind;
+    a.group_size = st->group_size;
+    a.lpr_log2 = st->reserved[0];
+    const Registry &reg = registry();
+    const abq_tile_config &c = st->cfg;
+    hipError_t e;
+    if (st->strategy == ABQ_STRATEGY_GENERIC) {
+        e = launch_bcnt_generic(a, c.x_bits, c.w_bits, c.is_signed, (hipStream_t)stream);
+    } else {
+        const KernelTable *t = find_table(st->strategy == ABQ_STRATEGY_BCNT ? reg.bcnt : reg.mfma,
+                                          c.x_bits, c.w_bits, c.is_signed);
+        if (!t || st->variant < 0 || st->variant >= t->count)
+            return ABQ_ERR_NOT_INITIALIZED;
+        e = t->entries[st->variant].launch(a, (hipStream_t)stream);
+    }
+    return hip_status(e);
+}
+
+abq_status abq_gemm_launch(const abq_tile_config *cfg, const uint32_t *X, const uint32_t *W,
+                           const void *C, int32_t *D, int bias, int M, int N, int K, void *stream)
+{
+    if (!cfg)
+        return ABQ_ERR_INVALID_ARG;
+    abq_gemm_state st;
+    abq_status s = abq_gemm_init(cfg, 0, 0, 0, X, W, M, N, K, D, C, bias, ABQ_OUT_I32, &st);
+    if (s != ABQ_OK)
+        return s;
+    return abq_gemm_exec(&st, stream);
+}
+
+} // extern "C"

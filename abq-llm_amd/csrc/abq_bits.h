@@ -1,0 +1,133 @@
+// Bit-plane <-> byte helpers shared by the pack and GEMM kernels.
+//
+// Everything here is plain integer C++ so the same code compiles for the device (hipcc)
+// and for the host (g++), where the unit tests drive it against the CPU oracle.
+//
+// Plane layout (engine/common/pack.cu:54-62 of the reference): element e of a group of 32
+// consecutive K elements sits at bit (31 - e) of the plane word; plane b holds bit b.
+#pragma once
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define ABQ_HD __host__ __device__ __forceinline__
+#else
+#define ABQ_HD inline
+#endif
+
+namespace abq {
+
+// One delta swap of a butterfly bit-matrix transpose: rows a (even) and b (odd) exchange
+// the blocks selected by mask m / shift s.
+ABQ_HD void delta_swap(uint32_t &a, uint32_t &b, uint32_t m, int s)
+{
+    uint32_t na = (a & m) | ((b << s) & ~m);
+    uint32_t nb = ((a >> s) & m) | (b & ~m);
+    a = na;
+    b = nb;
+}
+
+// In-place transpose of the 8x8 bit matrices formed by r[0..7] (rows) and the 8 bit
+// positions of each of the 4 byte lanes (columns).  After the call, byte c of r[s] has at
+// bit j what bit (8c + s) of the old r[j] was.
+ABQ_HD void transpose8x8x4(uint32_t (&r)[8])
+{
+    delta_swap(r[0], r[1], 0x55555555u, 1);
+    delta_swap(r[2], r[3], 0x55555555u, 1);
+    delta_swap(r[4], r[5], 0x55555555u, 1);
+    delta_swap(r[6], r[7], 0x55555555u, 1);
+    delta_swap(r[0], r[2], 0x33333333u, 2);
+    delta_swap(r[1], r[3], 0x33333333u, 2);
+    delta_swap(r[4], r[6], 0x33333333u, 2);
+    delta_swap(r[5], r[7], 0x33333333u, 2);
+    delta_swap(r[0], r[4], 0x0F0F0F0Fu, 4);
+    delta_swap(r[1], r[5], 0x0F0F0F0Fu, 4);
+    delta_swap(r[2], r[6], 0x0F0F0F0Fu, 4);
+    delta_swap(r[3], r[7], 0x0F0F0F0Fu, 4);
+}
+
+// How a BITS-wide operand is laid into an int8 lane for the matrix cores.
+//   kTop    signed operand: plane j goes to byte bit (8-BITS+j), so the MSB plane lands on the
+//           int8 sign bit and the byte equals value * 2^(8-BITS) in two's complement.
+//   kLow    unsigned operand of at most 7 bits: plane j goes to byte bit j.
+//   kFlip   unsigned 8-bit operand: bit 7 is inverted, the byte reads as value - 128.
+enum Int8Mode { kTop = 0, kLow = 1, kFlip = 2 };
+
+template <int BITS, bool SIGNED> struct Int8ModeOf {
+    static constexpr Int8Mode value = SIGNED ? kTop : (BITS == 8 ? kFlip : kLow);
+};
+
+// Expand BITS plane words (32 K elements) into 32 int8 values, as 8 dwords.
+// out[s] byte c is the element at bit position (8c + s) of the plane words, i.e. element
+// e = 31 - (8c + s) of the 32-group.  The element order does not depend on BITS or MODE, so
+// an activation word and a weight word expanded by this routine pair up element by element.
+template <int BITS, Int8Mode MODE> ABQ_HD void planes_to_int8(const uint32_t (&w)[BITS], uint32_t (&out)[8])
+{
+    static_assert(BITS >= 1 && BITS <= 8, "1..8 planes");
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        out[j] = 0u;
+#pragma unroll
+    for (int j = 0; j < BITS; ++j)
+        out[MODE == kTop ? 8 - BITS + j : j] = w[j];
+    if (MODE == kFlip)
+        out[7] = ~out[7];
+    transpose8x8x4(out);
+}
+
+// Sum of the unsigned values of the 32 elements held by BITS plane words.
+template <int BITS> ABQ_HD int planes_value_sum(const uint32_t (&w)[BITS])
+{
+    int s = 0;
+#pragma unroll
+    for (int j = 0; j < BITS; ++j)
+        s += __builtin_popcount(w[j]) << j;
+    return s;
+}
+
+// 8x8 bit-matrix transpose of a 64-bit word (byte r, bit c) -> (byte c, bit r).
+ABQ_HD uint64_t transpose8x8(uint64_t x)
+{
+    uint64_t t;
+    t = (x ^ (x >> 7)) & 0x00AA00AA00AA00AAull;
+    x = x ^ t ^ (t << 7);
+    t = (x ^ (x >> 14)) & 0x0000CCCC0000CCCCull;
+    x = x ^ t ^ (t << 14);
+    t = (x ^ (x >> 28)) & 0x00000000F0F0F0F0ull;
+    x = x ^ t ^ (t << 28);
+    return x;
+}
+
+// Eight consecutive K elements (low 8 bits of each used) -> eight plane bytes.
+// Byte b of the result is the 8-bit slice of plane b covering these elements, first
+// element at the byte's bit 7 (the plane words are MSB first).
+ABQ_HD uint64_t eight_values_to_plane_bytes(const int (&v)[8])
+{
+    uint64_t x = 0;
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+        x |= (uint64_t)((uint32_t)v[c] & 0xFFu) << (8 * (7 - c));
+    return transpose8x8(x);
+}
+
+// Multiplier of the popcount of (activation plane i AND weight plane j):
+// +/- 2^(i+j), negative when exactly one of the two is the MSB plane of a signed operand
+// (engine/test_any_mma.cu:64-68 and engine/mma_any/aq_bmma_kernel.h:549-561 of the reference).
+ABQ_HD int plane_pair_weight(int i, int j, int x_bits, int w_bits, bool is_signed)
+{
+    int mag = 1 << (i + j);
+    bool neg = is_signed && ((i == x_bits - 1) != (j == w_bits - 1));
+    return neg ? -mag : mag;
+}
+
+// Nibble-packed input word (8 elements, first element in the top nibble) -> for plane b the
+// 8-bit slice, first element at bit 7 (engine/common/pack.cu:26-40 of the reference).
+ABQ_HD uint32_t nibble_word_plane_byte(uint32_t word, int b)
+{
+    uint32_t y = (word >> b) & 0x11111111u; // bit 4t <- bit b of nibble t (t = 7 - element)
+    y = (y | (y >> 3)) & 0x03030303u;
+    y = (y | (y >> 6)) & 0x000F000Fu;
+    y = (y | (y >> 12)) & 0xFFu;
+    return y;
+}
+
+} // namespace abq

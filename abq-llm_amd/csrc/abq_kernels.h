@@ -1,0 +1,68 @@
+// Internal interface between the host API (abq_api.cpp) and the HIP kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "abq_bits.h"
+
+namespace abq {
+
+// Arguments of every GEMM kernel (the reference passes AqBMMAOpState::Argument_t,
+// engine/mma_any/aq_bmma_op.h:24-31).
+struct GemmArgs {
+    const uint32_t *X; // planes [x_bits][M][KW]
+    const uint32_t *W; // planes [w_bits][N][KW]
+    void *D;           // [M][N] int32 or fp16
+    const void *C;     // one fp16 scale (ABQ_OUT_F16_TENSOR) or null
+    const float *x_scale;
+    const float *w_scale;
+    int M, N, K, KW; // KW = K / 32 plane words per row
+    int out_kind;
+    int group_size;
+    int lpr_log2;    // popcount kernels: log2(lanes that share one weight row)
+};
+
+typedef hipError_t (*GemmLauncher)(const GemmArgs &, hipStream_t);
+
+// One kernel instantiation together with the tile tuple that names it.
+struct KernelEntry {
+    int mi;                 // MFMA rows (16 / 32); 1 for the popcount kernels
+    int tm, tn;             // MFMA tiles per wave (popcount: tm = activation rows per pass)
+    int wm, wn, wk;         // waves per workgroup along M, N, K
+    int nstage;
+    GemmLauncher launch;
+};
+
+struct KernelTable {
+    int x_bits, w_bits, is_signed;
+    const KernelEntry *entries;
+    int count;
+};
+
+// Defined once per (x_bits, w_bits) translation unit; looked up by abq_api.cpp.
+const KernelTable *mfma_tables(int *count);
+const KernelTable *bcnt_tables(int *count);
+hipError_t launch_bcnt_generic(const GemmArgs &, int x_bits, int w_bits, int is_signed, hipStream_t);
+
+// ---- output stage shared by all kernels ------------------------------------------------
+// out_kind values mirror abq_out_kind in include/abq_gemm.h.
+__device__ __forceinline__ void store_result(const GemmArgs &a, int m, int n, int acc)
+{
+    const size_t idx = (size_t)m * a.N + n;
+    if (a.out_kind == 0) {
+        reinterpret_cast<int *>(a.D)[idx] = acc;
+    } else if (a.out_kind == 1) {
+        // half(acc) * scale, both steps rounding to fp16
+        // (fastertransformer/.../abqgemm/mma_any/aq_bmma_kernel.h:516-519 of the reference).
+        // int -> float -> half rounds once: beyond 2^24, where the first step is inexact,
+        // the half result is infinity either way.
+        const _Float16 scale = *reinterpret_cast<const _Float16 *>(a.C);
+        const _Float16 h = (_Float16)(float)acc;
+        reinterpret_cast<_Float16 *>(a.D)[idx] = h * scale;
+    } else {
+        const float r = (float)acc * a.x_scale[m] * a.w_scale[n];
+        reinterpret_cast<_Float16 *>(a.D)[idx] = (_Float16)r;
+    }
+}
+
+} // namespace abq

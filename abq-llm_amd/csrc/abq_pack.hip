@@ -1,0 +1,143 @@
+// Bit-plane packing kernels.
+//
+// Replace pack / pack4 (engine/common/pack.cu:18-64 of the reference) and pack_int / pack_half
+// (fastertransformer/src/fastertransformer/kernels/abqgemm/abq_gemm_wrapper.cu:9-54).
+// Output layout is the reference's: planes[b][r][j], element e of a 32-group at bit 31-e.
+//
+// The reference launches one thread per output word per plane, so its input is re-read once
+// per plane.  Here a lane reads 8 consecutive elements once (32 bytes of int32 or 16 bytes of
+// fp16), turns them into one byte per plane with an 8x8 bit transpose, and the four lanes of
+// a quad assemble the bytes into one word per plane with DPP moves.  Input bytes are read
+// once, every load is 16 bytes wide and consecutive lanes touch consecutive memory.
+#include "abq_kernels.h"
+
+namespace abq {
+
+// OR across the 4 lanes of a quad (all lanes end with the result).
+__device__ __forceinline__ uint32_t quad_or(uint32_t v)
+{
+    v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true); // quad_perm [1,0,3,2]
+    v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true); // quad_perm [2,3,0,1]
+    return v;
+}
+
+// Emits the plane words of one 32-element group; the quad's lane q holds elements 8q..8q+7.
+__device__ __forceinline__ void emit_planes(const int (&v)[8], uint32_t *planes, size_t plane_words,
+                                            size_t word_idx, int bits, int quad_lane, bool active)
+{
+    for (int base = 0; base < bits; base += 8) {
+        int vs[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            vs[c] = active ? (int)((uint32_t)v[c] >> base) : 0;
+        const uint64_t bytes = eight_values_to_plane_bytes(vs);
+        const int nb = min(8, bits - base);
+        for (int b = 0; b < nb; ++b) {
+            uint32_t word = (uint32_t)((bytes >> (8 * b)) & 0xFFu) << (24 - 8 * quad_lane);
+            word = quad_or(word);
+            if (active && quad_lane == 0)
+                planes[(size_t)(base + b) * plane_words + word_idx] = word;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void pack_i32_kernel(const int4 *__restrict__ in,
+                                                       uint32_t *__restrict__ planes,
+                                                       size_t n_units, int bits)
+{
+    const size_t plane_words = n_units / 4;
+    // n_units is a multiple of 4 and the stride a multiple of 256, so a quad is active as one.
+    const size_t rounded = (n_units + 255) / 256 * 256;
+    for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < rounded; t += (size_t)gridDim.x * 256) {
+        const bool active = t < n_units;
+        int v[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
+        if (active) {
+            const int4 lo = in[2 * t], hi = in[2 * t + 1];
+            v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
+            v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+        }
+        emit_planes(v, planes, plane_words, t / 4, bits, (int)(t & 3), active);
+    }
+}
+
+__global__ __launch_bounds__(256) void pack_f16_kernel(const uint4 *__restrict__ in,
+                                                       const float *__restrict__ scale,
+                                                       uint32_t *__restrict__ planes,
+                                                       size_t n_units, int bits)
+{
+    const size_t plane_words = n_units / 4;
+    const _Float16 hs = (_Float16)scale[0];
+    const size_t rounded = (n_units + 255) / 256 * 256;
+    for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < rounded; t += (size_t)gridDim.x * 256) {
+        const bool active = t < n_units;
+        int v[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
+        if (active) {
+            union {
+                uint4 u;
+                _Float16 h[8];
+            } raw;
+            raw.u = in[t];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const _Float16 p = raw.h[c] * hs; // fp16 product, rounded to nearest even
+                v[c] = (int)p;                    // truncation
+            }
+        }
+        emit_planes(v, planes, plane_words, t / 4, bits, (int)(t & 3), active);
+    }
+}
+
+__global__ __launch_bounds__(256) void pack_u4_kernel(const uint4 *__restrict__ in,
+                                                      uint32_t *__restrict__ planes, size_t n_words,
+                                                      int bits)
+{
+    for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < n_words; t += (size_t)gridDim.x * 256) {
+        const uint4 v = in[t];
+        for (int b = 0; b < bits; ++b) {
+            // For b >= 4 the reference's shifts reach into the neighbouring nibble
+            // (pack.cu:28 shifts the whole word); the helper does the same.
+            const uint32_t word = (nibble_word_plane_byte(v.x, b) << 24) | (nibble_word_plane_byte(v.y, b) << 16) |
+                                  (nibble_word_plane_byte(v.z, b) << 8) | nibble_word_plane_byte(v.w, b);
+            planes[(size_t)b * n_words + t] = word;
+        }
+    }
+}
+
+static int grid_for(size_t items)
+{
+    size_t blocks = (items + 255) / 256;
+    if (blocks > 256 * 16)
+        blocks = 256 * 16;
+    if (blocks < 1)
+        blocks = 1;
+    return (int)blocks;
+}
+
+hipError_t launch_pack_i32(const int32_t *in, uint32_t *planes, int rows, int k, int bits,
+                           hipStream_t stream)
+{
+    const size_t n_units = (size_t)rows * k / 8;
+    hipLaunchKernelGGL(pack_i32_kernel, dim3(grid_for(n_units)), dim3(256), 0, stream,
+                       reinterpret_cast<const int4 *>(in), planes, n_units, bits);
+    return hipGetLastError();
+}
+
+hipError_t launch_pack_f16(const void *in, const float *scale, uint32_t *planes, int rows, int k,
+                           int bits, hipStream_t stream)
+{
+    const size_t n_units = (size_t)rows * k / 8;
+    hipLaunchKernelGGL(pack_f16_kernel, dim3(grid_for(n_units)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint4 *>(in), scale, planes, n_units, bits);
+    return hipGetLastError();
+}
+
+hipError_t launch_pack_u4(const uint32_t *in, uint32_t *planes, int rows, int k, int bits,
+                          hipStream_t stream)
+{
+    const size_t n_words = (size_t)rows * k / 32;
+    hipLaunchKernelGGL(pack_u4_kernel, dim3(grid_for(n_words)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint4 *>(in), planes, n_words, bits);
+    return hipGetLastError();
+}
+
+} // namespace abq

@@ -1,0 +1,184 @@
+/*
+ * abq_gemm.h -- C ABI of the MI355X (gfx950) arbitrary-bit quantized GEMM engine.
+ *
+ * Every entry point takes plain pointers and sizes.  Device pointers must be valid on the
+ * current HIP device; `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ * The library allocates nothing in any entry point declared here and keeps no mutable
+ * global state, so calls are stream ordered and thread safe on distinct states.
+ *
+ * Data layout (identical to the reference engine, see engine/common/pack.cu:46-64 there):
+ *   planes   uint32 words, K-major, MSB first: bit (31-e) of planes[b][r][j] is bit b of
+ *            element in[r][32*j+e].   X planes [x_bits][M][K/32], W planes [w_bits][N][K/32].
+ *   D        row-major [M][N], int32 or fp16 depending on the output kind.
+ *   The GEMM computes D = Xint . Wint^T, i.e.
+ *   D[m][n] = sum_{i<x_bits, j<w_bits} s_i s_j 2^(i+j) popcount(Xp[i][m][:] & Wp[j][n][:])
+ *   with s = -1 only for the MSB plane of a signed operand.
+ *   K must be a multiple of 128 and at least 128 (engine/test_any_mma.cu:99).
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to the
+ * reference tree).
+ */
+#ifndef ABQ_GEMM_H
+#define ABQ_GEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ABQ_VERSION 1
+
+/* Status codes.  The reference reports errors as cudaError_t from the pack launchers
+ * (engine/common/pack.cu:82,102), an initSuccess flag (engine/mma_any/aq_bmma_op.h:23,102,114)
+ * and printf + early return in the FT wrapper (abq_gemm_wrapper.cu:100-103,128-136). */
+typedef enum abq_status {
+    ABQ_OK = 0,
+    ABQ_ERR_INVALID_ARG = 1, /* null pointer, non-positive size, bits out of range        */
+    ABQ_ERR_BAD_K = 2,       /* K < 128 or K % 128 != 0                                    */
+    ABQ_ERR_UNSUPPORTED = 3, /* bit combination / tile tuple / option not implemented      */
+    ABQ_ERR_NOT_INITIALIZED = 4, /* exec called on a state whose init failed               */
+    ABQ_ERR_LAUNCH = 5,      /* the HIP runtime rejected the launch (see abq_last_hip_error) */
+    ABQ_ERR_NO_DEVICE = 6,   /* no usable gfx950 device                                    */
+    ABQ_ERR_TOO_LARGE = 7    /* a size exceeds a documented limit                          */
+} abq_status;
+
+const char *abq_status_string(abq_status s);
+/* hipError_t of the last failed launch on this thread, 0 if none. */
+int abq_last_hip_error(void);
+int abq_version(void);
+
+/* ---------------------------------------------------------------------------------------
+ * Bit-plane packing
+ * ------------------------------------------------------------------------------------- */
+
+/* Replaces launch_pack (engine/common/pack.h:23-24, pack.cu:46-64,93-104) and
+ * ABQGEMMWrapper::pack(const int*, ...) (abq_gemm_wrapper.cu:9-27,71-77).
+ * in: int32 [rows][k] on the device; planes: uint32 [bits][rows][k/32]. k % 32 == 0. */
+abq_status abq_pack_i32(const int32_t *in, uint32_t *planes, int rows, int k, int bits,
+                        void *stream);
+
+/* Replaces launch_pack4 (engine/common/pack.h:20-21, pack.cu:18-44,73-84).
+ * in: uint32 [rows*k/8], eight 4-bit elements per word, first element in the top nibble. */
+abq_status abq_pack_u4(const uint32_t *in, uint32_t *planes, int rows, int k, int bits,
+                       void *stream);
+
+/* Replaces pack_half / ABQGEMMWrapper::pack(const half*, const float*, ...)
+ * (fastertransformer/src/fastertransformer/kernels/abqgemm/abq_gemm_wrapper.cu:29-69).
+ * in: fp16 [rows][k]; scale: one float on the device; value = (int)(half(x) * half(scale)),
+ * the product rounded to fp16, the conversion truncating, no clamp. */
+abq_status abq_pack_f16(const void *in_f16, const float *scale_dev, uint32_t *planes, int rows,
+                        int k, int bits, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Tile configuration = the tuple encoded in the reference's kernel symbol names
+ * (engine/common/base.h:144-146): X_BITS x W_BITS x SIGNED _ BM x BN x BK _ WM x WN x WK _
+ * MMA_M x MMA_N x MMA_K _ NSTAGE.
+ *
+ * The MMA triple selects the gfx950 strategy:
+ *   1 x 1 x 128   VALU AND + popcount, K along the lanes, wavefront reduction
+ *   16 x 16 x 64  planes re-assembled to int8 in registers, v_mfma_i32_16x16x64_i8
+ *   32 x 32 x 32  the same feeding v_mfma_i32_32x32x32_i8
+ * Any other triple (the reference's 8x8x128, 16x8x128, 16x8x256 tensor-core shapes) asks the
+ * library to choose strategy and tile itself from (bits, M, N, K).
+ * ------------------------------------------------------------------------------------- */
+typedef struct abq_tile_config {
+    int x_bits, w_bits, is_signed;
+    int block_m, block_n, block_k;
+    int warp_m, warp_n, warp_k;
+    int mma_m, mma_n, mma_k;
+    int nstage;
+} abq_tile_config;
+
+typedef enum abq_strategy {
+    ABQ_STRATEGY_AUTO = 0,
+    ABQ_STRATEGY_BCNT = 1,   /* VALU popcount          */
+    ABQ_STRATEGY_MFMA16 = 2, /* int8 MFMA 16x16x64     */
+    ABQ_STRATEGY_MFMA32 = 3, /* int8 MFMA 32x32x32     */
+    ABQ_STRATEGY_GENERIC = 4 /* any 1..16 bit pair, runtime loops (slow, always available) */
+} abq_strategy;
+
+/* Parses "AqBMMA_8x2xtrue_1x48x512_8x24x128_8x8x128_4" (an optional _InitFn/_ExecFn suffix is
+ * accepted).  *is_wmma is set for the AqBWMMA family (engine/mma_any/aq_wmma_op.h), which maps
+ * to the same kernels.  Replaces the named globals declared by AQ_DECL_FUN
+ * (engine/common/base.h:159-166). */
+abq_status abq_parse_kernel_name(const char *name, abq_tile_config *cfg, int *is_wmma);
+/* Inverse of the above; writes at most n bytes including the terminator. */
+abq_status abq_format_kernel_name(const abq_tile_config *cfg, int is_wmma, char *buf, size_t n);
+
+/* Number of native gfx950 tile configurations for a bit combination, and the i-th one.
+ * This is the search space the autotuner walks (the role of engine/gen_kernel.cpp:24-157). */
+int abq_native_config_count(int x_bits, int w_bits, int is_signed);
+abq_status abq_native_config_get(int x_bits, int w_bits, int is_signed, int index,
+                                 abq_tile_config *cfg);
+
+/* ---------------------------------------------------------------------------------------
+ * GEMM
+ * ------------------------------------------------------------------------------------- */
+typedef struct abq_dim3 {
+    unsigned x, y, z;
+} abq_dim3;
+
+typedef enum abq_out_kind {
+    ABQ_OUT_I32 = 0,        /* int32 D (engine/mma_any/aq_bmma_kernel.h:485-580)                 */
+    ABQ_OUT_F16_TENSOR = 1, /* fp16 D = half(acc) * C[0], C one fp16 on the device
+                               (FT abqgemm/mma_any/aq_bmma_kernel.h:479,516-519)               */
+    ABQ_OUT_F16_SCALED = 2  /* fp16 D = acc * x_scale[m] * w_scale[n] (fp32 math), per-token
+                               and per-channel scales; see abq_gemm_set_scales                 */
+} abq_out_kind;
+
+/* Launch state, the POD returned by the reference's InitFn (AqBMMAOpState,
+ * engine/mma_any/aq_bmma_op.h:19-32).  Caller owned; init fills it, exec only reads it. */
+typedef struct abq_gemm_state {
+    size_t shared_mem_size;
+    abq_dim3 grid_dim;
+    abq_dim3 block_dim;
+    int init_success;
+    /* Argument_t */
+    int M, N, K;
+    const uint32_t *X;
+    const uint32_t *W;
+    const void *C;
+    void *D;
+    int bias;
+    /* resolved configuration */
+    abq_tile_config cfg;
+    int strategy; /* abq_strategy actually used */
+    int variant;  /* index into the strategy's kernel table */
+    int out_kind; /* abq_out_kind */
+    /* optional dequantization operands (ABQ_OUT_F16_SCALED) */
+    const float *x_scale;  /* [M] per token            */
+    const float *w_scale;  /* [N] or [N][K/group_size] */
+    int group_size;        /* 0 = per channel          */
+    int reserved[5];
+} abq_gemm_state;
+
+/* Replaces AqBMMAInitFn / AqBWMMAInitFn (engine/mma_any/aq_bmma_op.h:141-147,163 and
+ * aq_wmma_op.h) and AqBMMAOp::initialize (:76-115).  cfg may be NULL (library chooses).
+ * x_bits / w_bits / is_signed are read from cfg when given, else from the three ints.
+ * `bias` must be 0 (the reference asserts the same, aq_bmma_op.h:79).
+ * On failure state->init_success is 0 and the status says why. */
+abq_status abq_gemm_init(const abq_tile_config *cfg, int x_bits, int w_bits, int is_signed,
+                         const uint32_t *X, const uint32_t *W, int M, int N, int K, void *D,
+                         const void *C, int bias, int out_kind, abq_gemm_state *state);
+
+/* Attaches per-token / per-channel scales to an initialised state (ABQ_OUT_F16_SCALED).
+ * New behaviour with respect to the reference kernels; the semantics follow
+ * algorithm/quantize/quantizer.py:111-179 (scale per row of X, per row of W). */
+abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, const float *w_scale,
+                               int group_size);
+
+/* Replaces AqBMMAExecFn / AqBWMMAExecFn (engine/mma_any/aq_bmma_op.h:155-161,164): one
+ * asynchronous launch on `stream`. */
+abq_status abq_gemm_exec(const abq_gemm_state *state, void *stream);
+
+/* Replaces launchWmmaAnyKernel (engine/wmma_any/wmma_any.h:18-38, wmma_any.cu:28-87): the
+ * first-generation entry point, init + exec in one call, int32 D. */
+abq_status abq_gemm_launch(const abq_tile_config *cfg, const uint32_t *X, const uint32_t *W,
+                           const void *C, int32_t *D, int bias, int M, int N, int K, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ABQ_GEMM_H */

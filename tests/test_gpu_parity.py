@@ -1,0 +1,241 @@
+"""GPU parity tests: every kernel is called through the C ABI (libabq_gemm.so) and compared
+bit for bit with the CPU oracle on the same seeded inputs.  Inputs are packed by the oracle on
+the host, so the GEMM tests do not depend on the pack kernels."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+pytestmark = pytest.mark.gpu
+
+COMBOS = [(2, 2), (3, 3), (4, 4), (5, 5), (6, 6), (7, 7), (8, 8), (4, 2), (6, 2), (8, 2), (8, 4), (8, 3)]
+BASELINE_COMBOS = [c for c in COMBOS if c != (8, 3)]  # the 11 of BASELINE.json configs[3]
+
+
+def rand_vals(rng, rows, k, bits, signed):
+    lo, hi = (-(1 << (bits - 1)), (1 << (bits - 1)) - 1) if signed else (0, (1 << bits) - 1)
+    return rng.integers(lo, hi + 1, size=(rows, k), dtype=np.int32)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int32) if a.dtype == np.uint32 else np.ascontiguousarray(a)).cuda()
+
+
+def planes_dev(planes):
+    return torch.from_numpy(np.ascontiguousarray(planes).view(np.int32)).cuda()
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    if not torch.cuda.is_available():
+        pytest.fail("marked gpu but no GPU is visible")
+
+
+# ------------------------------------------------------------------ packing
+
+@pytest.mark.parametrize("rows,k,bits", [(1, 128, 8), (3, 128, 2), (8, 4096, 8), (17, 384, 5), (64, 4096, 4),
+                                         (5, 11008, 8), (2, 256, 13), (1, 128, 32), (130, 1152, 7)])
+def test_pack_i32_bit_exact(abq, oracle, rows, k, bits):
+    rng = np.random.default_rng(rows * 1000 + k + bits)
+    v = rng.integers(-(1 << 31), (1 << 31) - 1, size=(rows, k), dtype=np.int64).astype(np.int32) if bits > 8 \
+        else rand_vals(rng, rows, k, 8, True)  # values wider than `bits` must alias like the reference
+    got = abq.pack_i32(dev(v), bits).cpu().numpy().view(np.uint32)
+    assert np.array_equal(got, oracle.pack_i32(v, bits))
+
+
+def test_pack_i32_large_and_round_trip(abq, oracle):
+    rng = np.random.default_rng(11)
+    v = rand_vals(rng, 2048, 4096, 8, True)
+    got = abq.pack_i32(dev(v), 8).cpu().numpy().view(np.uint32)
+    assert np.array_equal(got, oracle.pack_i32(v, 8))
+    assert np.array_equal(oracle.unpack(got, True), v)
+
+
+@pytest.mark.parametrize("rows,k", [(1, 128), (16, 256), (64, 4096)])
+def test_pack_u4_bit_exact(abq, oracle, rows, k):
+    rng = np.random.default_rng(rows + k)
+    words = rng.integers(0, 1 << 32, size=rows * k // 8, dtype=np.uint64).astype(np.uint32)
+    got = abq.pack_u4(dev(words), rows, k, 4).cpu().numpy().view(np.uint32)
+    assert np.array_equal(got, oracle.pack_u4(words, rows, k, 4))
+
+
+@pytest.mark.parametrize("scale", [1.0, 0.5, 127.0 / 6.0, 100.0, 1e-3])
+def test_pack_f16_all_finite_bit_patterns(abq, oracle, scale):
+    x = np.arange(65536, dtype=np.uint16).view(np.float16)
+    x = np.where(np.isfinite(x), x, np.float16(0)).astype(np.float16).reshape(512, 128)
+    s = torch.tensor([scale], dtype=torch.float32, device="cuda")
+    for bits in (8, 17):
+        got = abq.pack_f16(torch.from_numpy(x).cuda(), s, bits).cpu().numpy().view(np.uint32)
+        want = oracle.pack_f16(x, scale, bits)
+        with np.errstate(over="ignore"):
+            finite = np.isfinite((x * np.float16(scale)).astype(np.float16))  # inf -> int is device defined
+        mask = np.packbits(finite.reshape(512, 4, 32), axis=2, bitorder="big").view(">u4").astype(np.uint32).reshape(512, 4)
+        assert np.array_equal(got & mask, want & mask)
+
+
+# ------------------------------------------------------------------ GEMM: every native tile, every combination
+
+SMALL_SHAPES = [(1, 64, 128), (3, 37, 384), (8, 130, 1152), (17, 64, 512), (33, 96, 256)]
+
+
+@pytest.mark.parametrize("q,p", COMBOS)
+@pytest.mark.parametrize("signed", [True, False])
+def test_gemm_every_native_config_small_shapes(abq, oracle, q, p, signed):
+    rng = np.random.default_rng(97 * q + 13 * p + int(signed))
+    cfgs = abq.native_configs(q, p, signed)
+    assert cfgs
+    for (M, N, K) in SMALL_SHAPES:
+        x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+        xp, wp = oracle.pack_i32(x, q), oracle.pack_i32(w, p)
+        want = oracle.np_gemm(x, w)
+        assert np.array_equal(oracle.gemm_popc(xp, wp, signed)[0], want)
+        xd, wd = planes_dev(xp), planes_dev(wp)
+        for cfg in cfgs:
+            out = torch.full((M, N), -12345, dtype=torch.int32, device="cuda")
+            g = abq.Gemm(xd, wd, signed, out=out, cfg=cfg)
+            got = g.run().cpu().numpy()
+            assert np.array_equal(got, want), (abq.format_kernel_name(cfg), M, N, K)
+        got = abq.gemm(xd, wd, signed).cpu().numpy()  # library's own choice
+        assert np.array_equal(got, want)
+
+
+def test_gemm_extreme_values_do_not_overflow(abq, oracle):
+    """All operands at the range ends, K = 13824 (the longest K of the baseline configurations)."""
+    K = 13824
+    for q, p, signed in [(8, 8, False), (8, 8, True), (8, 2, True), (4, 4, False), (7, 7, False)]:
+        xlo, xhi = oracle.value_range(q, signed)
+        wlo, whi = oracle.value_range(p, signed)
+        x = np.array([[xlo] * K, [xhi] * K, [xlo, xhi] * (K // 2)], dtype=np.int32)
+        w = np.array([[wlo] * K, [whi] * K, [whi, wlo] * (K // 2), [0] * K], dtype=np.int32)
+        xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
+        want = oracle.np_gemm(x, w)
+        for cfg in abq.native_configs(q, p, signed):
+            got = abq.gemm(xd, wd, signed, cfg=cfg).cpu().numpy()
+            assert np.array_equal(got, want), (q, p, signed, abq.format_kernel_name(cfg))
+
+
+def test_gemm_generic_bit_widths(abq, oracle):
+    """Bit pairs without a specialised kernel (the W1A1 / W1A4 / W1A8 / W1A16 / W2A16 samples)."""
+    rng = np.random.default_rng(5)
+    for q, p, signed in [(1, 1, False), (4, 1, False), (8, 1, False), (16, 1, False), (16, 2, True), (5, 3, True)]:
+        M, N, K = 3, 70, 256
+        x = rand_vals(rng, M, K, q, signed and q > 1)
+        w = rand_vals(rng, N, K, p, signed and p > 1)
+        xp, wp = oracle.pack_i32(x, q), oracle.pack_i32(w, p)
+        g = abq.Gemm(planes_dev(xp), planes_dev(wp), signed)
+        assert g.strategy == "generic"
+        assert np.array_equal(g.run().cpu().numpy(), oracle.gemm_bitserial(xp, wp, signed))
+
+
+def test_reference_kernel_names_run(abq, oracle):
+    """The two production tiles of the FT wrapper (abq_gemm_wrapper.cu:106-124) by name."""
+    rng = np.random.default_rng(6)
+    for name, M in (("AqBMMA_8x2xtrue_1x48x512_8x24x128_8x8x128_4", 1), ("AqBMMA_8x2xtrue_8x48x256_32x48x128_8x8x128_5", 8),
+                    ("AqBWMMA_8x2xfalse_8x48x256_32x48x128_8x8x128_5", 6)):
+        cfg, _ = abq.parse_kernel_name(name)
+        signed = bool(cfg.is_signed)
+        x, w = rand_vals(rng, M, 4096, 8, signed), rand_vals(rng, 1000, 4096, 2, signed)
+        got = abq.gemm(planes_dev(oracle.pack_i32(x, 8)), planes_dev(oracle.pack_i32(w, 2)), signed, cfg=cfg)
+        assert np.array_equal(got.cpu().numpy(), oracle.np_gemm(x, w))
+
+
+# ------------------------------------------------------------------ output stages
+
+def test_fp16_per_tensor_epilogue_matches_reference_rounding(abq, oracle):
+    rng = np.random.default_rng(7)
+    M, N, K = 8, 256, 1024
+    x, w = rand_vals(rng, M, K, 8, True), rand_vals(rng, N, K, 2, True)
+    xd, wd = planes_dev(oracle.pack_i32(x, 8)), planes_dev(oracle.pack_i32(w, 2))
+    acc = oracle.np_gemm(x, w)
+    for scale in (np.float16(0.0123), np.float16(1.0), np.float16(3.5e-3)):
+        c = torch.tensor([float(scale)], dtype=torch.float16, device="cuda")
+        for cfg in [None] + abq.native_configs(8, 2, True):
+            got = abq.gemm(xd, wd, True, cfg=cfg, out_kind=abq.OUT_F16_TENSOR, c_scale=c).cpu().numpy()
+            want = oracle.epilogue_f16(acc, scale)
+            assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+def test_fp16_per_token_per_channel_epilogue(abq, oracle):
+    """out = acc * x_scale[m] * w_scale[n]; tolerance 1e-2 relative (BASELINE.json north_star)."""
+    rng = np.random.default_rng(8)
+    for M in (1, 8, 48):
+        N, K = 384, 2048
+        x, w = rand_vals(rng, M, K, 8, True), rand_vals(rng, N, K, 2, True)
+        sx = rng.uniform(0.01, 0.05, M).astype(np.float32)
+        sw = rng.uniform(0.005, 0.02, N).astype(np.float32)
+        xd, wd = planes_dev(oracle.pack_i32(x, 8)), planes_dev(oracle.pack_i32(w, 2))
+        got = abq.gemm(xd, wd, True, out_kind=abq.OUT_F16_SCALED, x_scale=torch.from_numpy(sx).cuda(),
+                       w_scale=torch.from_numpy(sw).cuda()).cpu().numpy().astype(np.float64)
+        want = (x.astype(np.float64) * sx[:, None]) @ (w.astype(np.float64) * sw[:, None]).T
+        denom = np.maximum(np.abs(want), np.abs(want).mean())
+        assert np.max(np.abs(got - want) / denom) < 1e-2
+
+
+# ------------------------------------------------------------------ BASELINE.json configurations at full size
+
+def _sampled_oracle_check(oracle, xp, wp, signed, got, rng, rows=4):
+    M = xp.shape[1]
+    pick = np.sort(rng.choice(M, size=min(rows, M), replace=False))
+    want = oracle.gemm_popc(np.ascontiguousarray(xp[:, pick]), wp, signed)[0]
+    assert np.array_equal(got[pick], want)
+
+
+def test_config0_w4a4_unsigned_m64(abq, oracle):
+    rng = np.random.default_rng(0)
+    M, N, K = 64, 4096, 4096
+    x, w = rand_vals(rng, M, K, 4, False), rand_vals(rng, N, K, 4, False)
+    xp, wp = oracle.pack_i32(x, 4), oracle.pack_i32(w, 4)
+    got = abq.gemm(planes_dev(xp), planes_dev(wp), False).cpu().numpy()
+    assert np.array_equal(got, oracle.gemm_popc(xp, wp, False)[0])
+
+
+@pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (4096, 11008)])
+def test_config1_w2a8_decode_full_size(abq, oracle, N, K):
+    rng = np.random.default_rng(N + K)
+    w = rand_vals(rng, N, K, 2, True)
+    wp = oracle.pack_i32(w, 2)
+    wd = planes_dev(wp)
+    for M in (1, 4, 8):
+        x = np.clip(np.rint(rng.normal(0, 32, (M, K))), -128, 127).astype(np.int32)
+        xp = oracle.pack_i32(x, 8)
+        want = oracle.gemm_popc(xp, wp, True)[0]
+        xd = planes_dev(xp)
+        for cfg in [None] + abq.native_configs(8, 2, True):
+            if cfg is not None and cfg.mma_m == 32:
+                continue
+            got = abq.gemm(xd, wd, True, cfg=cfg).cpu().numpy()
+            assert np.array_equal(got, want), (M, cfg)
+
+
+@pytest.mark.parametrize("q,p,signed", [(4, 4, True), (4, 4, False), (8, 8, True), (8, 8, False)])
+def test_config2_prefill_full_size(abq, oracle, q, p, signed):
+    """M in {512, 2048} on the LLaMA-7B shapes: exact against the fp64 closed form X.W^T
+    (every product and sum is an integer below 2^53) and against the CPU oracle on sampled rows."""
+    rng = np.random.default_rng(1000 + q + int(signed))
+    for (N, K) in [(4096, 4096), (11008, 4096), (4096, 11008)]:
+        w = rand_vals(rng, N, K, p, signed)
+        wp = oracle.pack_i32(w, p)
+        wd = planes_dev(wp)
+        wf = torch.from_numpy(w).cuda().double()
+        for M in (512, 2048):
+            x = rand_vals(rng, M, K, q, signed)
+            xp = oracle.pack_i32(x, q)
+            got_d = abq.gemm(planes_dev(xp), wd, signed)
+            ref = torch.from_numpy(x).cuda().double() @ wf.T
+            assert torch.equal(got_d.double(), ref), (q, p, signed, M, N, K)
+            _sampled_oracle_check(oracle, xp, wp, signed, got_d.cpu().numpy(), rng, rows=2)
+            del ref
+
+
+@pytest.mark.parametrize("q,p", BASELINE_COMBOS)
+def test_config3_bit_combo_sweep_m128(abq, oracle, q, p):
+    rng = np.random.default_rng(3000 + 10 * q + p)
+    M = 128
+    for (N, K) in [(5120, 5120), (13824, 5120), (5120, 13824)]:
+        for signed in (True, False):
+            x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+            xp, wp = oracle.pack_i32(x, q), oracle.pack_i32(w, p)
+            got_d = abq.gemm(planes_dev(xp), planes_dev(wp), signed)
+            ref = torch.from_numpy(x).cuda().double() @ torch.from_numpy(w).cuda().double().T
+            assert torch.equal(got_d.double(), ref), (q, p, signed, N, K)
+            _sampled_oracle_check(oracle, xp, wp, signed, got_d.cpu().numpy(), rng, rows=2)

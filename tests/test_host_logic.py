@@ -1,0 +1,278 @@
+"""CPU tests of the host-side logic that ships: the bit helpers the kernels are built from
+(compiled for the host), the C ABI's argument checking / naming / tile registry, and the tile
+generator.  No GPU compute is called here."""
+import ctypes
+import hashlib
+import json
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from conftest import PKG, ROOT
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+COMBOS = [(2, 2), (3, 3), (4, 4), (5, 5), (6, 6), (7, 7), (8, 8), (4, 2), (6, 2), (8, 2), (8, 4), (8, 3)]
+
+
+@pytest.fixture(scope="module")
+def shim(tmp_path_factory):
+    out = str(tmp_path_factory.mktemp("shim") / "libshim.so")
+    subprocess.check_call(["g++", "-O2", "-std=c++17", "-shared", "-fPIC", "-I" + os.path.join(PKG, "csrc"),
+                           os.path.join(HERE, "host_shim.cpp"), "-o", out])
+    L = ctypes.CDLL(out)
+    L.shim_planes_to_int8.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long]
+    L.shim_eight_values_to_plane_bytes.argtypes = [ctypes.c_void_p]
+    L.shim_eight_values_to_plane_bytes.restype = ctypes.c_uint64
+    L.shim_nibble_word_plane_byte.argtypes = [ctypes.c_uint32, ctypes.c_int]
+    L.shim_nibble_word_plane_byte.restype = ctypes.c_uint32
+    return L
+
+
+def expand(shim, planes, mode):
+    """planes uint32 [bits, rows, kw] -> int8 [rows, kw, 32] in the kernels' element order."""
+    bits, rows, kw = planes.shape
+    words = np.ascontiguousarray(planes.transpose(1, 2, 0))  # [rows, kw, bits]
+    out = np.zeros((rows, kw, 8), dtype=np.uint32)
+    shim.shim_planes_to_int8(bits, mode, words.ctypes.data, out.ctypes.data, rows * kw)
+    return out.view(np.int8).reshape(rows, kw, 32)
+
+
+def rand_vals(rng, rows, k, bits, signed):
+    lo, hi = (-(1 << (bits - 1)), (1 << (bits - 1)) - 1) if signed else (0, (1 << bits) - 1)
+    return rng.integers(lo, hi + 1, size=(rows, k), dtype=np.int32)
+
+
+@pytest.mark.parametrize("bits", range(1, 9))
+def test_planes_to_int8_values_and_order(shim, oracle, bits):
+    rng = np.random.default_rng(bits)
+    K = 128
+    for signed in (True, False):
+        if signed and bits == 1:
+            continue
+        v = rand_vals(rng, 4, K, bits, signed)
+        planes = oracle.pack_i32(v, bits)
+        mode = shim.shim_int8_mode(bits, int(signed))
+        got = expand(shim, planes, mode).astype(np.int32)
+        # byte (4*s + c) of the 32 is the element at bit position 8c+s, i.e. element 31-(8c+s)
+        s, c = np.divmod(np.arange(32), 4)
+        elem = 31 - (8 * c + s)
+        want = v.reshape(4, K // 32, 32)[:, :, elem]
+        if signed:
+            want = want << (8 - bits)      # top-aligned two's complement
+        elif bits == 8:
+            want = want - 128              # bit 7 flipped
+        assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("q,p", COMBOS)
+@pytest.mark.parametrize("signed", [True, False])
+def test_int8_route_reproduces_oracle(shim, oracle, q, p, signed):
+    """The arithmetic of the matrix-core kernels, emulated on the host: expand both operands,
+    int8 dot products, then the shift (signed) or the row-sum correction (8-bit unsigned)."""
+    rng = np.random.default_rng(31 * q + p)
+    M, N, K = 6, 10, 384
+    x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+    xp, wp = oracle.pack_i32(x, q), oracle.pack_i32(w, p)
+    xm, wm = shim.shim_int8_mode(q, int(signed)), shim.shim_int8_mode(p, int(signed))
+    a = expand(shim, xp, xm).reshape(M, K).astype(np.int64)
+    b = expand(shim, wp, wm).reshape(N, K).astype(np.int64)
+    acc = a @ b.T
+    assert np.abs(acc).max() < 2 ** 31
+    if signed:
+        assert np.all(acc % (1 << (16 - q - p)) == 0)
+        d = acc >> (16 - q - p)
+    else:
+        d = acc.copy()
+        sx = (x.astype(np.int64)).sum(axis=1)
+        sw = (w.astype(np.int64)).sum(axis=1)
+        if p == 8:
+            d += 128 * sx[:, None]
+        if q == 8:
+            d += 128 * sw[None, :]
+        if p == 8 and q == 8:
+            d -= 16384 * K
+    assert np.array_equal(d.astype(np.int32), oracle.gemm_popc(xp, wp, signed)[0])
+
+
+def test_eight_values_to_plane_bytes(shim, oracle):
+    rng = np.random.default_rng(2)
+    for _ in range(200):
+        v = rng.integers(-128, 256, 8).astype(np.int32)
+        got = shim.shim_eight_values_to_plane_bytes(v.ctypes.data)
+        for b in range(8):
+            byte = (got >> (8 * b)) & 0xFF
+            want = sum(((int(v[c]) >> b) & 1) << (7 - c) for c in range(8))
+            assert byte == want
+
+
+def test_nibble_word_plane_byte(shim):
+    rng = np.random.default_rng(3)
+    for word in rng.integers(0, 2 ** 32, 200, dtype=np.uint64):
+        word = int(word)
+        for b in range(4):
+            want = sum((((word >> (4 * (7 - e))) >> b) & 1) << (7 - e) for e in range(8))
+            assert shim.shim_nibble_word_plane_byte(word, b) == want
+
+
+def test_plane_pair_weight_matches_reference_rule(shim):
+    # engine/test_any_mma.cu:64-68: multiplier of plane b is -2^b only for the MSB of a signed operand
+    for q, p in COMBOS:
+        for signed in (0, 1):
+            for i in range(q):
+                for j in range(p):
+                    xm = -(1 << i) if signed and i == q - 1 else (1 << i)
+                    wm = -(1 << j) if signed and j == p - 1 else (1 << j)
+                    assert shim.shim_plane_pair_weight(i, j, q, p, signed) == xm * wm
+
+
+# ------------------------------------------------------------------ C ABI (no compute)
+
+def test_library_exports_every_declared_symbol(abq):
+    header = open(os.path.join(ROOT, "include", "abq_gemm.h")).read()
+    declared = set(re.findall(r"\b(abq_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(abq.EXPORTED)
+    L = abq.lib()
+    for name in declared:
+        assert hasattr(L, name), name
+    assert L.abq_version() == 1
+    assert L.abq_status_string(2).decode().startswith("K must")
+
+
+def test_state_struct_matches_header_size(abq):
+    # sizeof(abq_gemm_state) as the C compiler sees it
+    src = '#include "abq_gemm.h"\n#include <stdio.h>\nint main(){printf("%zu %zu", sizeof(abq_gemm_state), sizeof(abq_tile_config));return 0;}'
+    exe = "/tmp/abq_sizeof"
+    subprocess.run(["gcc", "-x", "c", "-", "-I" + os.path.join(ROOT, "include"), "-o", exe], input=src.encode(), check=True)
+    a, b = subprocess.check_output([exe]).decode().split()
+    assert int(a) == ctypes.sizeof(abq.GemmState) and int(b) == ctypes.sizeof(abq.TileConfig)
+
+
+def test_kernel_name_round_trip(abq):
+    name = "AqBMMA_8x2xtrue_1x48x512_8x24x128_8x8x128_4"  # the FT M==1 configuration
+    cfg, wmma = abq.parse_kernel_name(name)
+    assert not wmma and cfg.as_tuple() == (8, 2, 1, 1, 48, 512, 8, 24, 128, 8, 8, 128, 4)
+    assert abq.format_kernel_name(cfg) == name
+    cfg2, wmma2 = abq.parse_kernel_name("AqBWMMA_4x4xfalse_8x32x256_32x64x128_8x8x128_2_ExecFn")
+    assert wmma2 and cfg2.is_signed == 0 and cfg2.nstage == 2
+    for bad in ("AqBMMA_8x2xmaybe_1x48x512_8x24x128_8x8x128_4", "Foo_1", "AqBMMA_8x2xtrue_1x48x512"):
+        with pytest.raises(abq.AbqError):
+            abq.parse_kernel_name(bad)
+
+
+def _init(abq, cfg=None, q=8, p=2, signed=1, X=0x1000, W=0x2000, M=1, N=64, K=4096, D=0x3000, C=None, bias=0,
+          out_kind=0):
+    st = abq.GemmState()
+    rc = abq.lib().abq_gemm_init(ctypes.byref(cfg) if cfg is not None else None, q, p, signed, X, W, M, N, K, D, C,
+                                 bias, out_kind, ctypes.byref(st))
+    return rc, st
+
+
+def test_init_error_paths(abq):
+    # the host-forcible failures of the reference: K constraint, bias, null pointers, unknown tuple
+    assert _init(abq)[0] == 0
+    for K in (0, 64, 127, 200, 4096 + 32):
+        rc, st = _init(abq, K=K)
+        assert rc in (1, 2) and st.init_success == 0
+    assert _init(abq, K=96)[0] == 2
+    assert _init(abq, bias=1)[0] == 3
+    assert _init(abq, X=None)[0] == 1 and _init(abq, W=None)[0] == 1 and _init(abq, D=None)[0] == 1
+    assert _init(abq, M=0)[0] == 1 and _init(abq, N=-1)[0] == 1
+    assert _init(abq, out_kind=1)[0] == 1  # fp16 per-tensor output without a scale pointer
+    assert _init(abq, out_kind=7)[0] == 1
+    assert _init(abq, q=17, p=2)[0] == 3
+    rc, st = _init(abq, q=16, p=1)  # a W1A16 sample of the reference library: run-time loop kernel
+    assert rc == 0 and st.strategy == abq.STRATEGY_GENERIC
+    # exec on a failed state is refused before any launch
+    rc, st = _init(abq, K=100)
+    assert abq.lib().abq_gemm_exec(ctypes.byref(st), None) == 4
+    # a native MMA triple with a tile that is not instantiated
+    cfg, _ = abq.parse_kernel_name("AqBMMA_8x2xtrue_16x48x4096_16x48x512_16x16x64_2")
+    assert _init(abq, cfg=cfg)[0] == 3
+    # K too large for the top-aligned signed int8 route
+    cfg, _ = abq.parse_kernel_name("AqBMMA_8x2xtrue_16x16x4096_16x16x512_16x16x64_2")
+    assert _init(abq, cfg=cfg, K=1 << 17)[0] == 7
+
+
+def test_default_strategy_choice_and_reference_tuples(abq):
+    for M, want in ((1, abq.STRATEGY_BCNT), (2, abq.STRATEGY_BCNT), (4, abq.STRATEGY_MFMA16),
+                    (8, abq.STRATEGY_MFMA16), (16, abq.STRATEGY_MFMA16), (128, abq.STRATEGY_MFMA32),
+                    (2048, abq.STRATEGY_MFMA32)):
+        rc, st = _init(abq, M=M, N=4096)
+        assert rc == 0 and st.strategy == want, M
+    # a reference (tensor-core) tuple is accepted and resolved to a native tile
+    cfg, _ = abq.parse_kernel_name("AqBMMA_8x2xtrue_8x48x256_32x48x128_8x8x128_5")
+    rc, st = _init(abq, cfg=cfg, M=8)
+    assert rc == 0 and st.strategy == abq.STRATEGY_MFMA16 and st.cfg.mma_k == 64
+    assert st.grid_dim.x == 4 and st.block_dim.x == 512
+
+
+@pytest.mark.parametrize("q,p", COMBOS)
+def test_native_configs_resolve_to_themselves(abq, q, p):
+    for signed in (0, 1):
+        cfgs = abq.native_configs(q, p, signed)
+        assert len(cfgs) >= 12
+        seen = set()
+        for c in cfgs:
+            rc, st = _init(abq, cfg=c, M=8, N=512, K=4096)
+            assert rc == 0, c
+            assert st.cfg.as_tuple() == c.as_tuple()
+            seen.add(abq.format_kernel_name(c))
+        assert len(seen) == len(cfgs)
+    assert abq.native_configs(9, 9, 1) == []
+
+
+# ------------------------------------------------------------------ tile generator
+
+@pytest.fixture(scope="module")
+def gen_kernel(tmp_path_factory):
+    exe = str(tmp_path_factory.mktemp("gen") / "gen_kernel")
+    subprocess.check_call(["g++", "-O2", "-std=c++17", os.path.join(PKG, "engine", "gen_kernel.cpp"), "-o", exe])
+    return exe
+
+
+def _tuples(text):
+    pat = re.compile(r"AQ_INSTANTIATE_FUN\(AqBMMA,\s*(\d+),\s*(\d+),\s*(true|false),\s*" + r",\s*".join([r"(\d+)"] * 10) + r"\)")
+    return [(int(g[0]), int(g[1]), 1 if g[2] == "true" else 0) + tuple(int(v) for v in g[3:]) for g in pat.findall(text)]
+
+
+def test_gen_kernel_sm80_space_matches_reference_tile_lists(gen_kernel):
+    """The four tile lists the reference ships that its own generator reproduces (as digests)."""
+    fx = json.load(open(os.path.join(HERE, "golden", "generator_fixture.json")))
+    for name, info in fx["lists"].items():
+        out = subprocess.check_output([gen_kernel, str(info["x_bits"]), str(info["w_bits"]), "1", str(fx["k_stage"]),
+                                       "--space", "sm80"]).decode()
+        tuples = _tuples(out)
+        assert len(tuples) == info["count"], name
+        h = hashlib.sha256()
+        for t in sorted(tuples):
+            h.update((",".join(str(v) for v in t) + "\n").encode())
+        assert h.hexdigest() == info["sha256_sorted"], name
+        assert list(tuples[0]) == info["first"] and list(tuples[-1]) == info["last"]
+
+
+def test_gen_kernel_sm80_space_matches_reference_generator(gen_kernel):
+    ref = os.path.join(ROOT, "oracle", "_ref", "gen_kernel_ref")
+    if not os.path.exists(ref):
+        pytest.skip("oracle/_ref not built (reference tree not mounted)")
+    for q, p in COMBOS:
+        for signed in ("0", "1"):
+            for ks in ("2", "4", "6"):
+                mine = subprocess.check_output([gen_kernel, str(q), str(p), signed, ks, "--space", "sm80"])
+                theirs = subprocess.check_output([ref, str(q), str(p), signed, ks])
+                assert mine == theirs, (q, p, signed, ks)
+
+
+def test_gen_kernel_native_space_is_what_the_library_instantiates(gen_kernel, abq):
+    inc = open(os.path.join(PKG, "csrc", "abq_mfma_variants.inc")).read()
+    committed = [l for l in inc.splitlines() if l.startswith("V(")]
+    out = subprocess.check_output([gen_kernel, "8", "8", "1", "4", "--format", "variants"]).decode().splitlines()
+    assert out == committed
+    for q, p in COMBOS:
+        for signed in (0, 1):
+            text = subprocess.check_output([gen_kernel, str(q), str(p), str(signed), "4"]).decode()
+            gen = set(_tuples(text))
+            native = set(c.as_tuple() for c in abq.native_configs(q, p, signed))
+            assert gen == native, (q, p, signed)
