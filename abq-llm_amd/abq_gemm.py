@@ -18,8 +18,8 @@ STATUS_NAMES = {
     4: "ABQ_ERR_NOT_INITIALIZED", 5: "ABQ_ERR_LAUNCH", 6: "ABQ_ERR_NO_DEVICE", 7: "ABQ_ERR_TOO_LARGE",
 }
 OUT_I32, OUT_F16_TENSOR, OUT_F16_SCALED = 0, 1, 2
-STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC = range(5)
-STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic"]
+STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC, STRATEGY_DECODE = range(6)
+STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic", "decode"]
 
 # every symbol include/abq_gemm.h declares
 EXPORTED = [

@@ -23,19 +23,22 @@ hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream
 
 #define ABQ_DECL(Q, P)                                \
     void abq_mfma_register_##Q##_##P(KernelTable *);  \
-    void abq_bcnt_register_##Q##_##P(KernelTable *);
+    void abq_bcnt_register_##Q##_##P(KernelTable *);  \
+    void abq_decode_register_##Q##_##P(KernelTable *);
 ABQ_FOR_EACH_COMBO(ABQ_DECL)
 #undef ABQ_DECL
 
 struct Registry {
     KernelTable mfma[2 * ABQ_NUM_COMBOS];
     KernelTable bcnt[2 * ABQ_NUM_COMBOS];
+    KernelTable decode[2 * ABQ_NUM_COMBOS];
     Registry()
     {
         int i = 0;
 #define ABQ_REG(Q, P)                                  \
     abq_mfma_register_##Q##_##P(&mfma[i]);             \
     abq_bcnt_register_##Q##_##P(&bcnt[i]);             \
+    abq_decode_register_##Q##_##P(&decode[i]);         \
     i += 2;
         ABQ_FOR_EACH_COMBO(ABQ_REG)
 #undef ABQ_REG
@@ -143,7 +146,8 @@ static int find_mfma_variant(const KernelTable &t, int mi, int tm, int tn, int w
 }
 
 // Default choice when the caller names no native tile: popcount for one or two activation
-// rows, 16-row MFMA tiles with K split over the waves up to 16 rows, 32-row MFMA tiles above.
+// rows, the decode kernel (16-row MFMA tiles, activations staged in LDS) up to 16 rows,
+// 32-row MFMA tiles above.
 static void choose_default(int M, int N, int *strategy, int *mi, int *tm, int *tn, int *wm, int *wn,
                            int *wk)
 {
@@ -151,7 +155,7 @@ static void choose_default(int M, int N, int *strategy, int *mi, int *tm, int *t
         *strategy = ABQ_STRATEGY_BCNT;
         *mi = 1; *tm = M; *tn = 1; *wm = 1; *wn = 4; *wk = 1;
     } else if (M <= 16) {
-        *strategy = ABQ_STRATEGY_MFMA16;
+        *strategy = ABQ_STRATEGY_DECODE;
         *mi = 16; *tm = 1; *tn = 1; *wm = 1; *wn = 1; *wk = 8;
     } else {
         *strategy = ABQ_STRATEGY_MFMA32;
@@ -174,7 +178,8 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
     int strategy = cfg ? strategy_of_mma(*cfg) : ABQ_STRATEGY_AUTO;
     const KernelTable *tm_ = find_table(reg.mfma, x_bits, w_bits, is_signed);
     const KernelTable *tb_ = find_table(reg.bcnt, x_bits, w_bits, is_signed);
-    if (!tm_ || !tb_) {
+    const KernelTable *td_ = find_table(reg.decode, x_bits, w_bits, is_signed);
+    if (!tm_ || !tb_ || !td_) {
         // no specialised instantiation: run-time loop kernel, one activation row per grid row
         if (x_bits < 1 || x_bits > 16 || w_bits < 1 || w_bits > 16)
             return ABQ_ERR_UNSUPPORTED;
@@ -209,6 +214,33 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         tm = cfg->warp_m / mi; tn = cfg->warp_n / mi;
         wm = cfg->block_m / cfg->warp_m; wn = cfg->block_n / cfg->warp_n;
         wk = cfg->block_k / stepk;
+        if (strategy == ABQ_STRATEGY_MFMA16 && cfg->nstage == 3)
+            strategy = ABQ_STRATEGY_DECODE;
+    }
+
+    if (strategy == ABQ_STRATEGY_DECODE) {
+        if (mi != 16 || tm != 1 || tn != 1 || wm != 1 || wn != 1)
+            return ABQ_ERR_UNSUPPORTED;
+        int v = -1;
+        for (int i = 0; i < td_->count; ++i)
+            if (td_->entries[i].wk == wk)
+                v = i;
+        if (v < 0)
+            return ABQ_ERR_UNSUPPORTED;
+        if (K >= (1 << 17) || (M + 15) / 16 > 65535)
+            return ABQ_ERR_TOO_LARGE;
+        const KernelEntry &e = td_->entries[v];
+        const int tiles = (N + 15) / 16;
+        int gx = tiles < 256 ? tiles : 256;
+        if ((tiles + gx - 1) / gx > 8)
+            gx = (tiles + 7) / 8;
+        st->strategy = strategy;
+        st->variant = v;
+        entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
+        st->grid_dim = abq_dim3{ (unsigned)gx, (unsigned)((M + 15) / 16), 1 };
+        st->block_dim = abq_dim3{ (unsigned)(64 * e.wk), 1, 1 };
+        st->shared_mem_size = 0; // sized at launch from M and K (dynamic LDS)
+        return ABQ_OK;
     }
 
     if (strategy == ABQ_STRATEGY_BCNT) {
@@ -372,9 +404,10 @@ int abq_native_config_count(int x_bits, int w_bits, int is_signed)
     const Registry &reg = registry();
     const KernelTable *tb = find_table(reg.bcnt, x_bits, w_bits, is_signed);
     const KernelTable *tm = find_table(reg.mfma, x_bits, w_bits, is_signed);
-    if (!tb || !tm)
+    const KernelTable *td = find_table(reg.decode, x_bits, w_bits, is_signed);
+    if (!tb || !tm || !td)
         return 0;
-    return tb->count * 3 + tm->count;
+    return tb->count * 3 + td->count + tm->count;
 }
 
 abq_status abq_native_config_get(int x_bits, int w_bits, int is_signed, int index, abq_tile_config *cfg)
@@ -384,7 +417,8 @@ abq_status abq_native_config_get(int x_bits, int w_bits, int is_signed, int inde
     const Registry &reg = registry();
     const KernelTable *tb = find_table(reg.bcnt, x_bits, w_bits, is_signed);
     const KernelTable *tm = find_table(reg.mfma, x_bits, w_bits, is_signed);
-    if (!tb || !tm)
+    const KernelTable *td = find_table(reg.decode, x_bits, w_bits, is_signed);
+    if (!tb || !tm || !td)
         return ABQ_ERR_UNSUPPORTED;
     if (index < tb->count * 3) {
         entry_to_config(tb->entries[index / 3], ABQ_STRATEGY_BCNT, x_bits, w_bits, is_signed,
@@ -392,6 +426,11 @@ abq_status abq_native_config_get(int x_bits, int w_bits, int is_signed, int inde
         return ABQ_OK;
     }
     index -= tb->count * 3;
+    if (index < td->count) {
+        entry_to_config(td->entries[index], ABQ_STRATEGY_DECODE, x_bits, w_bits, is_signed, 0, cfg);
+        return ABQ_OK;
+    }
+    index -= td->count;
     if (index >= tm->count)
         return ABQ_ERR_INVALID_ARG;
     const KernelEntry &e = tm->entries[index];
@@ -486,8 +525,10 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     if (st->strategy == ABQ_STRATEGY_GENERIC) {
         e = launch_bcnt_generic(a, c.x_bits, c.w_bits, c.is_signed, (hipStream_t)stream);
     } else {
-        const KernelTable *t = find_table(st->strategy == ABQ_STRATEGY_BCNT ? reg.bcnt : reg.mfma,
-                                          c.x_bits, c.w_bits, c.is_signed);
+        const KernelTable *tables = st->strategy == ABQ_STRATEGY_BCNT     ? reg.bcnt
+                                    : st->strategy == ABQ_STRATEGY_DECODE ? reg.decode
+                                                                          : reg.mfma;
+        const KernelTable *t = find_table(tables, c.x_bits, c.w_bits, c.is_signed);
         if (!t || st->variant < 0 || st->variant >= t->count)
             return ABQ_ERR_NOT_INITIALIZED;
         e = t->entries[st->variant].launch(a, (hipStream_t)stream);

@@ -1,0 +1,398 @@
+// GEMM core for decode-sized M (at most 16 activation rows per grid row): matrix-core strategy
+// with the activations expanded once per workgroup.
+//
+// Replaces AqBMMAKernel::mainLoop + ::epilogue of the reference
+// (engine/mma_any/aq_bmma_kernel.h:109-271, :485-580) for one (x_bits, w_bits) pair per
+// translation unit: compile with -DABQ_Q=<x_bits> -DABQ_P=<w_bits>.
+//
+// The weights are the only large operand: every weight word is read exactly once, with 16-byte
+// loads straight from the reference layout, by the lane that expands it to int8 and feeds it to
+// v_mfma_i32_16x16x64_i8 as the B operand (no LDS round trip for weights).
+// The activations are a few KiB.  Expanding them per wave costs more VALU time than the whole
+// weight stream takes from HBM, so the workgroup expands them once into LDS
+// (xs[row][K bytes], the byte order the expansion routine produces) and every wave reads its A
+// operands from there with ds_read_b128.
+//
+// Work split.  The grid is persistent: at most one workgroup per compute unit, workgroup b owns
+// the 16-row weight tiles b, b+G, b+2G, ...  Inside a workgroup the work items are
+// (tile, K step) pairs, a step being 16 plane words (512 K elements) per row; wave w takes
+// items w, w+NW, ...  Partial 16x16 results meet in LDS with ds_add (integer, so the order does
+// not matter) and are written out once at the end.  K is processed in chunks sized so that the
+// expanded activations fit the LDS budget; one chunk covers all baseline shapes up to M = 8.
+#include "abq_kernels.h"
+
+#ifndef ABQ_Q
+#error "compile with -DABQ_Q=<x_bits> -DABQ_P=<w_bits>"
+#endif
+
+namespace abq {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr int kDecodeMaxTiles = 8;            // weight tiles per workgroup
+constexpr int kDecodeXBudget = 128 * 1024;    // bytes of LDS for the expanded activations
+constexpr int kDecodeFixedLds = kDecodeMaxTiles * (256 + 16) * 4 + 16 * 4;
+
+__device__ __forceinline__ uint32_t comp4(const uint4 &v, int i)
+{
+    return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
+}
+
+// Loads the P plane words [word, word+4) of weight row (tile*16 + r); all-zero when the item or
+// the words are out of range (one predicated region for all planes).
+template <int P>
+__device__ __forceinline__ void load_weight_words(uint4 (&dst)[P], const uint32_t *W, size_t wplane, int KW,
+                                                  int N, int tile, int r, int word, int word_end, bool item_valid)
+{
+#pragma unroll
+    for (int b = 0; b < P; ++b)
+        dst[b] = make_uint4(0u, 0u, 0u, 0u);
+    if (item_valid && word < word_end) {
+        const uint32_t *p = W + (size_t)min(tile * 16 + r, N - 1) * KW + word;
+#pragma unroll
+        for (int b = 0; b < P; ++b) {
+            dst[b] = *reinterpret_cast<const uint4 *>(p);
+            p += wplane;
+        }
+    }
+}
+
+// Expands the four plane words per plane held in wv into the eight B operands of one K step.
+template <int P, Int8Mode MODE, bool SUM>
+__device__ __forceinline__ void expand_weight_words(const uint4 (&wv)[P], v4i (&bops)[8], int &value_sum)
+{
+    value_sum = 0;
+#pragma unroll
+    for (int ws = 0; ws < 4; ++ws) {
+        uint32_t w[P], bop[8];
+#pragma unroll
+        for (int b = 0; b < P; ++b)
+            w[b] = comp4(wv[b], ws);
+        if (SUM)
+            value_sum += planes_value_sum<P>(w);
+        planes_to_int8<P, MODE>(w, bop);
+        bops[ws * 2] = v4i{ (int)bop[0], (int)bop[1], (int)bop[2], (int)bop[3] };
+        bops[ws * 2 + 1] = v4i{ (int)bop[4], (int)bop[5], (int)bop[6], (int)bop[7] };
+    }
+}
+
+template <int Q, int P, bool SIGNED, int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, int chunk_words, int row_words,
+                                                            int tw_base, int tw_rem)
+{
+    constexpr int NT = 64 * NW;
+    constexpr Int8Mode XMODE = Int8ModeOf<Q, SIGNED>::value;
+    constexpr Int8Mode WMODE = Int8ModeOf<P, SIGNED>::value;
+    constexpr bool NEED_SX = WMODE == kFlip; // see abq_gemm_mfma.hip: row-sum corrections for
+    constexpr bool NEED_SW = XMODE == kFlip; // 8-bit unsigned operands fed as value - 128
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    int *tacc = reinterpret_cast<int *>(smem);                 // [kDecodeMaxTiles][16][16]
+    int *tsw = tacc + kDecodeMaxTiles * 256;                   // [kDecodeMaxTiles][16]
+    int *sxs = tsw + kDecodeMaxTiles * 16;                     // [16]
+    unsigned char *xs = smem + kDecodeFixedLds;                // [Mb][RS]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    // wave-uniform: everything derived from it (item -> tile / step) runs on the scalar unit
+    const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int M = a.M, N = a.N, KW = a.KW;
+    const int m0 = blockIdx.y * 16;
+    const int Mb = min(16, M - m0);
+    const int RS = row_words * 32 + 16; // row stride of xs in bytes (row_words = chunk rounded up to a step)
+    const size_t xplane = (size_t)M * KW;
+    const size_t wplane = (size_t)N * KW;
+    const int G = gridDim.x;
+    const int TW = tw_base + ((int)blockIdx.x < tw_rem ? 1 : 0); // tiles b, b+G, ... of this workgroup
+
+    // Work items of this wave: j = wid, wid+NW, ... over (tile, step) pairs of the chunk, step
+    // fastest.  (tl, st) is the item being computed, (tl1, st1) the next one.
+    uint4 w1[P], w2[P];     // raw weight words of the next item and of the one after it
+    uint32_t xcur[Q], xnext[Q];
+    v4i bops[8];            // expanded weights of the item being computed
+    int bsum = 0;
+    int tl = 0, st = wid, tl1, st1;
+
+    // Load order at entry: first the activation words this wave will expand (a few KiB in all,
+    // but the expansion, the LDS write and a barrier hang off them, so they must not queue
+    // behind the weight stream), then the weight words of the wave's first two items.
+    // Everything up to the first MFMA overlaps the weight latency.  The scheduling barrier keeps
+    // the compiler from hoisting loop-invariant setup in front of the loads.
+    {
+        const int cw = min(chunk_words, KW);
+        const int bpr = (cw + 63) >> 6;
+        int m = 0, kb = wid;
+        while (kb >= bpr) {
+            kb -= bpr;
+            ++m;
+        }
+        const int kw = kb * 64 + lane;
+#pragma unroll
+        for (int b = 0; b < Q; ++b)
+            xcur[b] = 0u;
+        if (m < Mb && kw < cw) {
+            const uint32_t *xp = a.X + (size_t)(m0 + m) * KW + kw;
+#pragma unroll
+            for (int b = 0; b < Q; ++b) {
+                xcur[b] = *xp;
+                xp += xplane;
+            }
+        }
+        const int csteps = (cw + 15) >> 4;
+        while (st >= csteps) {
+            st -= csteps;
+            ++tl;
+        }
+        st1 = st + NW;
+        tl1 = tl;
+        while (st1 >= csteps) {
+            st1 -= csteps;
+            ++tl1;
+        }
+        uint4 w0[P];
+        load_weight_words<P>(w0, a.W, wplane, KW, N, blockIdx.x + tl * G, r, st * 16 + 4 * g, cw, tl < TW);
+        load_weight_words<P>(w1, a.W, wplane, KW, N, blockIdx.x + tl1 * G, r, st1 * 16 + 4 * g, cw, tl1 < TW);
+        __builtin_amdgcn_sched_barrier(0);
+        for (int i = tid; i < kDecodeMaxTiles * (256 + 16) + 16; i += NT)
+            tacc[i] = 0; // ordered before the first ds_add by the barrier that ends the expansion
+        if (NEED_SX)
+            __syncthreads(); // the activation row sums are accumulated during the expansion itself
+        // The first item's weights are expanded while other waves expand activations.
+        if (Mb * bpr <= wid)
+            expand_weight_words<P, WMODE, NEED_SW>(w0, bops, bsum);
+        else {
+#pragma unroll
+            for (int b = 0; b < P; ++b)
+                w2[b] = w0[b]; // this wave expands activations first; weights right after
+        }
+    }
+
+    int k_fed = 0;
+    for (int c0 = 0; c0 < KW; c0 += chunk_words) {
+        const int cw = min(chunk_words, KW - c0);
+        const int csteps = (cw + 15) >> 4;
+        const int bpr = (cw + 63) >> 6;
+        const int wend = c0 + cw;
+        k_fed += csteps * 512;
+        const bool has_x_work = wid < Mb * bpr;
+
+        if (c0 != 0) { // later chunks (long K with many activation rows): same first loads, in place
+            const int m = wid / bpr;
+            const int kw = (wid - m * bpr) * 64 + lane;
+#pragma unroll
+            for (int b = 0; b < Q; ++b)
+                xcur[b] = 0u;
+            if (m < Mb && kw < cw) {
+                const uint32_t *xp = a.X + (size_t)(m0 + m) * KW + c0 + kw;
+#pragma unroll
+                for (int b = 0; b < Q; ++b) {
+                    xcur[b] = *xp;
+                    xp += xplane;
+                }
+            }
+            tl = wid / csteps;
+            st = wid - tl * csteps;
+            st1 = st + NW;
+            tl1 = tl;
+            while (st1 >= csteps) {
+                st1 -= csteps;
+                ++tl1;
+            }
+            load_weight_words<P>(w2, a.W, wplane, KW, N, blockIdx.x + tl * G, r, c0 + st * 16 + 4 * g, wend, tl < TW);
+            load_weight_words<P>(w1, a.W, wplane, KW, N, blockIdx.x + tl1 * G, r, c0 + st1 * 16 + 4 * g, wend, tl1 < TW);
+            __syncthreads(); // previous chunk fully consumed before xs is overwritten
+            if (!has_x_work)
+                expand_weight_words<P, WMODE, NEED_SW>(w2, bops, bsum);
+        }
+
+        // Activation expansion: wave-sized blocks of 64 consecutive plane words of one row,
+        // the words of the next block in flight while this one is expanded.
+        for (int blk = wid; blk < Mb * bpr; blk += NW) {
+            const int m = blk / bpr;
+            const int kw = (blk - m * bpr) * 64 + lane;
+            {
+                const int bn = blk + NW;
+                const int mn = bn / bpr;
+                const int kwn = (bn - mn * bpr) * 64 + lane;
+#pragma unroll
+                for (int b = 0; b < Q; ++b)
+                    xnext[b] = 0u;
+                if (mn < Mb && kwn < cw) {
+                    const uint32_t *xp = a.X + (size_t)(m0 + mn) * KW + c0 + kwn;
+#pragma unroll
+                    for (int b = 0; b < Q; ++b) {
+                        xnext[b] = *xp;
+                        xp += xplane;
+                    }
+                }
+            }
+            if (kw < cw) {
+                uint32_t o[8];
+                if (NEED_SX)
+                    atomicAdd(&sxs[m], planes_value_sum<Q>(xcur));
+                planes_to_int8<Q, XMODE>(xcur, o);
+                uint4 *dst = reinterpret_cast<uint4 *>(xs + (size_t)m * RS + kw * 32);
+                dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+                dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+            }
+#pragma unroll
+            for (int b = 0; b < Q; ++b)
+                xcur[b] = xnext[b];
+        }
+        // The tail of a partial last step must hold what all-zero planes expand to (weights
+        // past K are fed as zero planes; the row-sum correction counts these elements).
+        if (cw & 15) {
+            const int pad = csteps * 16 - cw;
+            const uint32_t fill = XMODE == kFlip ? 0x80808080u : 0u;
+            for (int u = tid; u < Mb * pad * 2; u += NT) {
+                const int m = u / (pad * 2), q16 = u - m * (pad * 2);
+                reinterpret_cast<uint4 *>(xs + (size_t)m * RS + cw * 32)[q16] = make_uint4(fill, fill, fill, fill);
+            }
+        }
+        if (has_x_work)
+            expand_weight_words<P, WMODE, NEED_SW>(w2, bops, bsum);
+        __syncthreads();
+
+        v4i acc = { 0, 0, 0, 0 };
+        int sw_part = 0;
+        int cur_tl = tl < TW ? tl : -1;
+        const unsigned char *xrow = xs + (size_t)min(r, Mb - 1) * RS + g * 128;
+
+        while (tl < TW) {
+            // A operands of this step: 8 x 16 bytes per lane
+            v4i aop[8];
+            {
+                const unsigned char *xw = xrow + st * 512;
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    aop[i] = *reinterpret_cast<const v4i *>(xw + i * 16);
+            }
+            // weights of the item after next go in flight now
+            int st2 = st1 + NW, tl2 = tl1;
+            while (st2 >= csteps) {
+                st2 -= csteps;
+                ++tl2;
+            }
+            load_weight_words<P>(w2, a.W, wplane, KW, N, blockIdx.x + tl2 * G, r, c0 + st2 * 16 + 4 * g, wend, tl2 < TW);
+            if (tl != cur_tl) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (4 * g + e < Mb)
+                        atomicAdd(&tacc[cur_tl * 256 + (4 * g + e) * 16 + r], acc[e]);
+                if (NEED_SW)
+                    atomicAdd(&tsw[cur_tl * 16 + r], sw_part);
+                acc = v4i{ 0, 0, 0, 0 };
+                sw_part = 0;
+                cur_tl = tl;
+            }
+            sw_part += bsum;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[i], bops[i], acc, 0, 0, 0);
+            // expand the next item's weights (loaded one iteration ago) for the next round
+            if (tl1 < TW)
+                expand_weight_words<P, WMODE, NEED_SW>(w1, bops, bsum);
+#pragma unroll
+            for (int b = 0; b < P; ++b)
+                w1[b] = w2[b];
+            st = st1;
+            tl = tl1;
+            st1 = st2;
+            tl1 = tl2;
+        }
+        if (cur_tl >= 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (4 * g + e < Mb)
+                    atomicAdd(&tacc[cur_tl * 256 + (4 * g + e) * 16 + r], acc[e]);
+            if (NEED_SW)
+                atomicAdd(&tsw[cur_tl * 16 + r], sw_part);
+        }
+    }
+    __syncthreads();
+
+    // Output: 16 lanes per row of a tile; thread (s = tid / 16, c = tid % 16) serves row s % 16 of
+    // tiles s / 16, s / 16 + NT / 256, ...
+    {
+        const int c = tid & 15, i = (tid >> 4) & 15;
+        for (int t = tid >> 8; t < TW; t += NT / 256) {
+            const int n = (blockIdx.x + t * G) * 16 + c;
+            if (i < Mb && n < N) {
+                unsigned v = (unsigned)tacc[t * 256 + i * 16 + c];
+                if (SIGNED) {
+                    v = (unsigned)((int)v >> (16 - Q - P));
+                } else {
+                    if (NEED_SX)
+                        v += 128u * (unsigned)sxs[i];
+                    if (NEED_SW)
+                        v += 128u * (unsigned)tsw[t * 16 + c];
+                    if (NEED_SX && NEED_SW)
+                        v -= 16384u * (unsigned)k_fed;
+                }
+                store_result(a, m0 + i, n, (int)v);
+            }
+        }
+    }
+}
+
+// K chunking: the whole K in one chunk if the expanded activations fit the LDS budget, else
+// the largest multiple of 16 plane words that does.  row_words is the chunk rounded up to a
+// whole step (16 words), the length each LDS row is laid out for.
+static void decode_chunking(int M, int KW, int *chunk_words, int *row_words)
+{
+    const int mb = M < 16 ? M : 16;
+    const int kwp = (KW + 15) / 16 * 16;
+    if ((long)mb * (kwp * 32 + 16) <= kDecodeXBudget) {
+        *chunk_words = KW;
+        *row_words = kwp;
+        return;
+    }
+    int cw = (kDecodeXBudget / mb - 16) / 32;
+    cw -= cw % 16;
+    *chunk_words = cw;
+    *row_words = cw;
+}
+
+template <int Q, int P, bool SIGNED, int NW>
+static hipError_t launch_mfma_decode(const GemmArgs &a, hipStream_t stream)
+{
+    const int tiles = (a.N + 15) / 16;
+    int gx = tiles < 256 ? tiles : 256; // one workgroup per MI355X compute unit
+    if ((tiles + gx - 1) / gx > kDecodeMaxTiles)
+        gx = (tiles + kDecodeMaxTiles - 1) / kDecodeMaxTiles;
+    int cw, rw;
+    decode_chunking(a.M, a.KW, &cw, &rw);
+    const int mb = a.M < 16 ? a.M : 16;
+    const size_t lds = kDecodeFixedLds + (size_t)mb * (rw * 32 + 16);
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void *>(&gemm_mfma_decode<Q, P, SIGNED, NW>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, kDecodeFixedLds + kDecodeXBudget);
+    if (attr != hipSuccess)
+        return attr;
+    const dim3 grid(gx, (a.M + 15) / 16);
+    hipLaunchKernelGGL((gemm_mfma_decode<Q, P, SIGNED, NW>), grid, dim3(64 * NW), lds, stream, a, cw, rw, tiles / gx, tiles % gx);
+    return hipGetLastError();
+}
+
+// Native tile space of this kernel: waves per workgroup.  Entries reuse the MFMA tuple
+// (16-row tiles, K split over the waves) with nstage = 3 marking the LDS-staged activations.
+#define ABQ_DECODE_VARIANTS(V) V(4) V(8) V(16)
+
+#define ABQ_ENTRY_T(NW) { 16, 1, 1, 1, 1, NW, 3, &launch_mfma_decode<ABQ_Q, ABQ_P, true, NW> },
+#define ABQ_ENTRY_F(NW) { 16, 1, 1, 1, 1, NW, 3, &launch_mfma_decode<ABQ_Q, ABQ_P, false, NW> },
+
+static const KernelEntry kSigned[] = { ABQ_DECODE_VARIANTS(ABQ_ENTRY_T) };
+static const KernelEntry kUnsigned[] = { ABQ_DECODE_VARIANTS(ABQ_ENTRY_F) };
+
+#define ABQ_CAT_(a, b, c, d) a##b##c##d
+#define ABQ_CAT(a, b, c, d) ABQ_CAT_(a, b, c, d)
+
+void ABQ_CAT(abq_decode_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)
+{
+    out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSigned, (int)(sizeof(kSigned) / sizeof(kSigned[0])) };
+    out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, kUnsigned, (int)(sizeof(kUnsigned) / sizeof(kUnsigned[0])) };
+}
+
+} // namespace abq

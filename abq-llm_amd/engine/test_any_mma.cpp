@@ -1,0 +1,276 @@
+// Autotune / benchmark harness: the MI355X counterpart of the reference's
+// engine/test_any_mma.cu (main, :86-272) and engine/test/test_mma/test_mma.h (benchmark, TEST,
+// :21-160).
+//
+//     test_any_mma M N K X_BITS W_BITS SIGNED [--repeat R] [--warmup W] [--rotate-mib MiB]
+//                  [--stream] [--only SUBSTR] [--seed S]
+//
+// Like the reference it builds random operands, packs them on the GPU, computes the expected
+// result on the CPU, then runs EVERY tile configuration of the bit combination, checks each
+// result for exact equality and prints one line per configuration
+//     <arch> <WxAy int|uint> BM BN BK WM WN WK MM MN MK NSTAGE packing _ (us) exec _ (us)
+//     _ TOPS | _ B-TOPS | PASSED|ERROR|FAILED
+// followed by "The best kernel config is ... with ... TOPS".  TOPS = 2*M*N*K / t and
+// B-TOPS = TOPS * X_BITS * W_BITS as in engine/test/test_mma/test_mma_w2a8.cu:37-38.
+//
+// Differences that matter on this hardware:
+//  * the search space is the library's native gfx950 tile list (abq_native_config_*), plus the
+//    library's own default choice as the last line;
+//  * weights rotate through --rotate-mib of distinct buffers (default 512) so that the 256 MB
+//    Infinity Cache cannot serve them; all buffers hold the same data, so one CPU result
+//    checks them all;
+//  * the timed loop is replayed from a HIP graph unless --stream is given, so the host launch
+//    rate does not bound the figure; in addition to the roofline fractions it prints
+//    (HBM 8 TB/s on the packed bytes, int8 MFMA 5 POP/s on 2*M*N*K);
+//  * inputs come from std::mt19937_64 with a fixed seed instead of unseeded rand().
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "abq_gemm.h"
+
+#define HIP_OK(x)                                                                        \
+    do {                                                                                 \
+        hipError_t e_ = (x);                                                             \
+        if (e_ != hipSuccess) {                                                          \
+            std::fprintf(stderr, "HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+            std::exit(1);                                                                \
+        }                                                                                \
+    } while (0)
+
+namespace {
+
+// Expected result, computed from the packed planes the way compute_ref does
+// (engine/test_any_mma.cu:58-84) but with one popcount per word pair.
+void expected_result(const std::vector<uint32_t> &w, const std::vector<uint32_t> &x, std::vector<int> &d, int M,
+                     int N, int K, int w_bits, int x_bits, bool is_signed)
+{
+    const long KW = K / 32;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int m = 0; m < M; ++m) {
+        for (int n = 0; n < N; ++n) {
+            long acc = 0;
+            for (int xb = 0; xb < x_bits; ++xb) {
+                for (int wb = 0; wb < w_bits; ++wb) {
+                    const uint32_t *xr = &x[((long)xb * M + m) * KW];
+                    const uint32_t *wr = &w[((long)wb * N + n) * KW];
+                    long cnt = 0;
+                    for (long k = 0; k < KW; ++k)
+                        cnt += __builtin_popcount(xr[k] & wr[k]);
+                    const bool neg = is_signed && ((xb == x_bits - 1) != (wb == w_bits - 1));
+                    acc += (neg ? -cnt : cnt) << (xb + wb);
+                }
+            }
+            d[(long)m * N + n] = (int)acc;
+        }
+    }
+}
+
+struct Timing {
+    float exec_us = 0, pack_us = 0;
+    int status = -1; // 0 PASSED, -1 ERROR, -2 FAILED (test_mma.h:114-159)
+};
+
+} // namespace
+
+int main(int argc, char **argv)
+{
+    if (argc < 7) {
+        std::printf("Usage: ./test_any_mma M N K X_BITS W_BITS SIGNED [--repeat R] [--warmup W] [--rotate-mib MiB] [--stream] [--only SUBSTR] [--seed S]\n");
+        return -1;
+    }
+    const int M = std::atoi(argv[1]), N = std::atoi(argv[2]), K = std::atoi(argv[3]);
+    const int x_bits = std::atoi(argv[4]), w_bits = std::atoi(argv[5]);
+    const bool is_signed = std::atoi(argv[6]) == 1;
+    int repeat = 1000, warmup = 10, rotate_mib = 512;
+    bool use_graph = true;
+    unsigned long seed = 0;
+    std::string only;
+    for (int i = 7; i < argc; ++i) {
+        if (!std::strcmp(argv[i], "--stream"))
+            use_graph = false;
+        else if (i + 1 < argc && !std::strcmp(argv[i], "--repeat"))
+            repeat = std::atoi(argv[++i]);
+        else if (i + 1 < argc && !std::strcmp(argv[i], "--warmup"))
+            warmup = std::atoi(argv[++i]);
+        else if (i + 1 < argc && !std::strcmp(argv[i], "--rotate-mib"))
+            rotate_mib = std::atoi(argv[++i]);
+        else if (i + 1 < argc && !std::strcmp(argv[i], "--only"))
+            only = argv[++i];
+        else if (i + 1 < argc && !std::strcmp(argv[i], "--seed"))
+            seed = std::strtoul(argv[++i], nullptr, 10);
+    }
+    if (K < 128 || K % 128 != 0) { // engine/test_any_mma.cu:99
+        std::printf("Error, k must >= 128 and k %% 128 == 0!");
+        return -1;
+    }
+
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+
+    // ---- host operands: uniform over the full range of the bit width
+    std::mt19937_64 rng(seed);
+    auto fill = [&](std::vector<int> &v, int bits) {
+        const int lo = is_signed ? -(1 << (bits - 1)) : 0;
+        const int span = 1 << bits;
+        for (auto &e : v)
+            e = lo + (int)(rng() % (unsigned long)span);
+    };
+    std::vector<int> h_x((size_t)M * K), h_w((size_t)N * K);
+    fill(h_x, x_bits);
+    fill(h_w, w_bits);
+
+    const size_t KW = K / 32;
+    const size_t xp_words = (size_t)x_bits * M * KW, wp_words = (size_t)w_bits * N * KW;
+    const size_t wp_bytes = wp_words * 4;
+    size_t nbuf = std::max<size_t>(1, ((size_t)rotate_mib << 20) / wp_bytes);
+    nbuf = std::min<size_t>(nbuf, 4096);
+
+    int *d_x, *d_w, *d_out;
+    uint32_t *d_xp, *d_wp;
+    HIP_OK(hipMalloc(&d_x, h_x.size() * 4));
+    HIP_OK(hipMalloc(&d_w, h_w.size() * 4));
+    HIP_OK(hipMalloc(&d_xp, xp_words * 4));
+    HIP_OK(hipMalloc(&d_wp, wp_bytes * nbuf));
+    HIP_OK(hipMalloc(&d_out, (size_t)M * N * 4));
+    HIP_OK(hipMemcpy(d_x, h_x.data(), h_x.size() * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d_w, h_w.data(), h_w.size() * 4, hipMemcpyHostToDevice));
+
+    if (abq_pack_i32(d_w, d_wp, N, K, w_bits, stream) != ABQ_OK || abq_pack_i32(d_x, d_xp, M, K, x_bits, stream) != ABQ_OK) {
+        std::printf("launch_pack failed (hip error %d)\n", abq_last_hip_error());
+        return -1;
+    }
+    HIP_OK(hipStreamSynchronize(stream));
+    for (size_t b = 1; b < nbuf; ++b)
+        HIP_OK(hipMemcpyAsync((char *)d_wp + b * wp_bytes, d_wp, wp_bytes, hipMemcpyDeviceToDevice, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+
+    std::vector<uint32_t> h_xp(xp_words), h_wp(wp_words);
+    HIP_OK(hipMemcpy(h_xp.data(), d_xp, xp_words * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(h_wp.data(), d_wp, wp_words * 4, hipMemcpyDeviceToHost));
+    std::vector<int> h_ref((size_t)M * N), h_out((size_t)M * N);
+    expected_result(h_wp, h_xp, h_ref, M, N, K, w_bits, x_bits, is_signed);
+
+    // ---- activation packing time (reported separately, test_mma.h:141-152)
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    float pack_us = 0;
+    {
+        for (int i = 0; i < warmup; ++i)
+            abq_pack_i32(d_x, d_xp, M, K, x_bits, stream);
+        HIP_OK(hipEventRecord(e0, stream));
+        const int reps = std::max(10, repeat / 10);
+        for (int i = 0; i < reps; ++i)
+            abq_pack_i32(d_x, d_xp, M, K, x_bits, stream);
+        HIP_OK(hipEventRecord(e1, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        float ms;
+        HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+        pack_us = ms * 1e3f / reps;
+    }
+
+    const double ops = 2.0 * M * N * K;
+    const double alg_bytes = (double)w_bits * N * K / 8 + (double)x_bits * M * K / 8 + 4.0 * M * N;
+    char config_str[32];
+    std::snprintf(config_str, sizeof config_str, "W%dA%d %s", w_bits, x_bits, is_signed ? "int" : "uint");
+
+    auto run_one = [&](const abq_tile_config *cfg, Timing &t, abq_gemm_state &st0) {
+        std::vector<abq_gemm_state> states(nbuf);
+        for (size_t b = 0; b < nbuf; ++b) {
+            abq_status s = abq_gemm_init(cfg, x_bits, w_bits, is_signed, d_xp, (const uint32_t *)((char *)d_wp + b * wp_bytes),
+                                         M, N, K, d_out, nullptr, 0, ABQ_OUT_I32, &states[b]);
+            if (s != ABQ_OK || !states[b].init_success) {
+                t.status = -1;
+                return;
+            }
+        }
+        st0 = states[0];
+        HIP_OK(hipMemsetAsync(d_out, 0xff, (size_t)M * N * 4, stream));
+        if (abq_gemm_exec(&states[0], stream) != ABQ_OK || hipStreamSynchronize(stream) != hipSuccess) {
+            t.status = -1;
+            return;
+        }
+        HIP_OK(hipMemcpy(h_out.data(), d_out, (size_t)M * N * 4, hipMemcpyDeviceToHost));
+        t.status = std::memcmp(h_out.data(), h_ref.data(), (size_t)M * N * 4) == 0 ? 0 : -2;
+        for (int i = 0; i < warmup; ++i)
+            abq_gemm_exec(&states[i % nbuf], stream);
+        HIP_OK(hipStreamSynchronize(stream));
+        float ms = 0;
+        if (use_graph) {
+            hipGraph_t g;
+            hipGraphExec_t ge;
+            HIP_OK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+            for (int i = 0; i < repeat; ++i)
+                abq_gemm_exec(&states[i % nbuf], stream);
+            HIP_OK(hipStreamEndCapture(stream, &g));
+            HIP_OK(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0));
+            HIP_OK(hipEventRecord(e0, stream));
+            HIP_OK(hipGraphLaunch(ge, stream));
+            HIP_OK(hipEventRecord(e1, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+            HIP_OK(hipGraphExecDestroy(ge));
+            HIP_OK(hipGraphDestroy(g));
+        } else {
+            HIP_OK(hipEventRecord(e0, stream));
+            for (int i = 0; i < repeat; ++i)
+                abq_gemm_exec(&states[i % nbuf], stream);
+            HIP_OK(hipEventRecord(e1, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+        }
+        t.exec_us = ms * 1e3f / repeat;
+        t.pack_us = pack_us;
+    };
+
+    double best_tops = 0;
+    std::string best;
+    const int ncfg = abq_native_config_count(x_bits, w_bits, is_signed);
+    for (int i = 0; i <= ncfg; ++i) {
+        abq_tile_config cfg;
+        const bool library_default = i == ncfg;
+        if (!library_default && abq_native_config_get(x_bits, w_bits, is_signed, i, &cfg) != ABQ_OK)
+            continue;
+        char name[160] = "library default";
+        if (!library_default)
+            abq_format_kernel_name(&cfg, 0, name, sizeof name);
+        if (!only.empty() && std::string(name).find(only) == std::string::npos)
+            continue;
+        Timing t;
+        abq_gemm_state st;
+        std::memset(&st, 0, sizeof st);
+        run_one(library_default ? nullptr : &cfg, t, st);
+        const abq_tile_config &c = st.cfg;
+        const double tops = t.status == 0 ? ops / (t.exec_us * 1e-6) / 1e12 : 0;
+        std::printf("gfx950 %s %d %d %d %d %d %d %d %d %d %d ", config_str, c.block_m, c.block_n, c.block_k, c.warp_m,
+                    c.warp_n, c.warp_k, c.mma_m, c.mma_n, c.mma_k, c.nstage);
+        std::printf("packing %f (us) exec %f (us) %f TOPS | %f B-TOPS | %s | %.1f%% HBM %.1f%% MFMA%s\n", t.pack_us,
+                    t.exec_us, tops, tops * x_bits * w_bits, t.status == 0 ? "PASSED" : t.status == -1 ? "ERROR" : "FAILED",
+                    t.status == 0 ? 100.0 * alg_bytes / (t.exec_us * 1e-6) / 8e12 : 0.0, 100.0 * tops / 5000.0,
+                    library_default ? " | library default" : "");
+        if (t.status == 0 && !library_default && tops > best_tops) {
+            best_tops = tops;
+            char buf[128];
+            std::snprintf(buf, sizeof buf, "%d, %d, %d, %d, %d, %d, %d, %d, %d, %d", c.block_m, c.block_n, c.block_k, c.warp_m,
+                          c.warp_n, c.warp_k, c.mma_m, c.mma_n, c.mma_k, c.nstage);
+            best = buf;
+        }
+        std::fflush(stdout);
+    }
+    std::printf("The best kernel config is %s with %f TOPS\n", best.c_str(), best_tops);
+
+    (void)hipFree(d_x);
+    (void)hipFree(d_w);
+    (void)hipFree(d_xp);
+    (void)hipFree(d_wp);
+    (void)hipFree(d_out);
+    (void)hipStreamDestroy(stream);
+    return 0;
+}

@@ -79,6 +79,8 @@ abq_status abq_pack_f16(const void *in_f16, const float *scale_dev, uint32_t *pl
  * The MMA triple selects the gfx950 strategy:
  *   1 x 1 x 128   VALU AND + popcount, K along the lanes, wavefront reduction
  *   16 x 16 x 64  planes re-assembled to int8 in registers, v_mfma_i32_16x16x64_i8
+ *                 (NSTAGE = 3: decode kernel, activations staged in LDS; NSTAGE = 2: every wave
+ *                 expands its own activations)
  *   32 x 32 x 32  the same feeding v_mfma_i32_32x32x32_i8
  * Any other triple (the reference's 8x8x128, 16x8x128, 16x8x256 tensor-core shapes) asks the
  * library to choose strategy and tile itself from (bits, M, N, K).
@@ -96,7 +98,9 @@ typedef enum abq_strategy {
     ABQ_STRATEGY_BCNT = 1,   /* VALU popcount          */
     ABQ_STRATEGY_MFMA16 = 2, /* int8 MFMA 16x16x64     */
     ABQ_STRATEGY_MFMA32 = 3, /* int8 MFMA 32x32x32     */
-    ABQ_STRATEGY_GENERIC = 4 /* any 1..16 bit pair, runtime loops (slow, always available) */
+    ABQ_STRATEGY_GENERIC = 4, /* any 1..16 bit pair, runtime loops (slow, always available) */
+    ABQ_STRATEGY_DECODE = 5   /* int8 MFMA 16x16x64, activations expanded once per workgroup
+                                 into LDS, persistent grid; tile tuples with NSTAGE = 3       */
 } abq_strategy;
 
 /* Parses "AqBMMA_8x2xtrue_1x48x512_8x24x128_8x8x128_4" (an optional _InitFn/_ExecFn suffix is

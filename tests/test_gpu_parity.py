@@ -114,6 +114,22 @@ def test_gemm_extreme_values_do_not_overflow(abq, oracle):
             assert np.array_equal(got, want), (q, p, signed, abq.format_kernel_name(cfg))
 
 
+def test_decode_kernel_k_chunking_and_many_tiles(abq, oracle):
+    """Decode kernel corner cases: activations too large for one LDS chunk (M=16, long K), a
+    partial last K step, more weight tiles than workgroups, and several 16-row blocks of M."""
+    rng = np.random.default_rng(21)
+    for q, p, signed, M, N, K in [(8, 2, True, 16, 100, 11008), (8, 8, False, 13, 70, 13824), (4, 4, False, 16, 333, 8320),
+                                  (8, 2, True, 8, 16 * 256 * 3 + 5, 128), (8, 8, False, 40, 4200, 384)]:
+        x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+        xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
+        want = oracle.np_gemm(x, w)
+        for cfg in abq.native_configs(q, p, signed):
+            if cfg.nstage != 3:
+                continue
+            got = abq.gemm(xd, wd, signed, cfg=cfg).cpu().numpy()
+            assert np.array_equal(got, want), (abq.format_kernel_name(cfg), M, N, K)
+
+
 def test_gemm_generic_bit_widths(abq, oracle):
     """Bit pairs without a specialised kernel (the W1A1 / W1A4 / W1A8 / W1A16 / W2A16 samples)."""
     rng = np.random.default_rng(5)
