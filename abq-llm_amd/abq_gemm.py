@@ -17,7 +17,7 @@ STATUS_NAMES = {
     0: "ABQ_OK", 1: "ABQ_ERR_INVALID_ARG", 2: "ABQ_ERR_BAD_K", 3: "ABQ_ERR_UNSUPPORTED",
     4: "ABQ_ERR_NOT_INITIALIZED", 5: "ABQ_ERR_LAUNCH", 6: "ABQ_ERR_NO_DEVICE", 7: "ABQ_ERR_TOO_LARGE",
 }
-OUT_I32, OUT_F16_TENSOR, OUT_F16_SCALED = 0, 1, 2
+OUT_I32, OUT_F16_TENSOR, OUT_F16_SCALED, OUT_F16_TENSOR_F32SCALE = 0, 1, 2, 3
 STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC, STRATEGY_DECODE = range(6)
 STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic", "decode"]
 

@@ -145,18 +145,17 @@ static int find_mfma_variant(const KernelTable &t, int mi, int tm, int tn, int w
     return -1;
 }
 
-// Default choice when the caller names no native tile: popcount for one or two activation
-// rows, the decode kernel (16-row MFMA tiles, activations staged in LDS) up to 16 rows,
-// 32-row MFMA tiles above.
+// Default choice when the caller names no native tile: the decode kernel (16-row MFMA tiles,
+// activations staged in LDS) up to 16 activation rows, 32-row MFMA tiles above.  The popcount
+// kernels stay reachable through their tile tuples (MMA 1x1x128).
 static void choose_default(int M, int N, int *strategy, int *mi, int *tm, int *tn, int *wm, int *wn,
                            int *wk)
 {
-    if (M <= 2) {
-        *strategy = ABQ_STRATEGY_BCNT;
-        *mi = 1; *tm = M; *tn = 1; *wm = 1; *wn = 4; *wk = 1;
-    } else if (M <= 16) {
+    if (M <= 16) {
+        // Measured on MI355X (W2A8, LLaMA-7B shapes, M = 1, 4, 8): the decode kernel with 16
+        // waves beats the popcount kernel at every M including M = 1, and the other MFMA tiles.
         *strategy = ABQ_STRATEGY_DECODE;
-        *mi = 16; *tm = 1; *tn = 1; *wm = 1; *wn = 1; *wk = 8;
+        *mi = 16; *tm = 1; *tn = 1; *wm = 1; *wn = 1; *wk = 16;
     } else {
         *strategy = ABQ_STRATEGY_MFMA32;
         *mi = 32; *wm = 2; *wn = 2; *wk = 1;
@@ -461,9 +460,9 @@ abq_status abq_gemm_init(const abq_tile_config *cfg, int x_bits, int w_bits, int
         return ABQ_ERR_UNSUPPORTED;
     if (K < 128 || K % 128 != 0)
         return ABQ_ERR_BAD_K;
-    if (out_kind != ABQ_OUT_I32 && out_kind != ABQ_OUT_F16_TENSOR && out_kind != ABQ_OUT_F16_SCALED)
+    if (out_kind < ABQ_OUT_I32 || out_kind > ABQ_OUT_F16_TENSOR_F32SCALE)
         return ABQ_ERR_INVALID_ARG;
-    if (out_kind == ABQ_OUT_F16_TENSOR && !C)
+    if ((out_kind == ABQ_OUT_F16_TENSOR || out_kind == ABQ_OUT_F16_TENSOR_F32SCALE) && !C)
         return ABQ_ERR_INVALID_ARG;
     if ((long)M * N >= (1L << 31) || (long)M * (K / 32) >= (1L << 31) || (long)N * (K / 32) >= (1L << 31))
         return ABQ_ERR_TOO_LARGE;

@@ -59,6 +59,11 @@ __device__ __forceinline__ void store_result(const GemmArgs &a, int m, int n, in
         const _Float16 scale = *reinterpret_cast<const _Float16 *>(a.C);
         const _Float16 h = (_Float16)(float)acc;
         reinterpret_cast<_Float16 *>(a.D)[idx] = h * scale;
+    } else if (a.out_kind == 3) {
+        // the same with the scale held as one float: converted to fp16 first, then as above
+        const _Float16 scale = (_Float16)*reinterpret_cast<const float *>(a.C);
+        const _Float16 h = (_Float16)(float)acc;
+        reinterpret_cast<_Float16 *>(a.D)[idx] = h * scale;
     } else {
         const float r = (float)acc * a.x_scale[m] * a.w_scale[n];
         reinterpret_cast<_Float16 *>(a.D)[idx] = (_Float16)r;

@@ -1,0 +1,83 @@
+// See abq_gemm_wrapper.h.  Follows the decision table of the reference's
+// ABQGEMMWrapper::gemm (abq_gemm_wrapper.cu:79-138): quantise + pack A, check K, pick a kernel,
+// init, check initSuccess, exec.
+#include "abq_gemm_wrapper.h"
+
+#include <stdint.h>
+#include <stdio.h>
+
+#include "abq_gemm.h"
+
+ABQGEMMWrapper::ABQGEMMWrapper(int X_BITS, int W_BITS, bool SIGNED) : x_bits_(X_BITS), w_bits_(W_BITS), signed_(SIGNED) {}
+
+ABQGEMMWrapper::~ABQGEMMWrapper() {}
+
+void ABQGEMMWrapper::pack(const _Float16 *in_data, const float *scale, int *packed_data, int M, int K, int BIT,
+                          hipStream_t stream)
+{
+    const abq_status rc = abq_pack_f16(in_data, scale, reinterpret_cast<uint32_t *>(packed_data), M, K, BIT, stream);
+    if (rc != ABQ_OK)
+        printf("[ABQ][Error] pack failed: %s\n", abq_status_string(rc));
+}
+
+void ABQGEMMWrapper::pack(const int *in_data, int *packed_data, int M, int K, int BIT, hipStream_t stream)
+{
+    const abq_status rc = abq_pack_i32(in_data, reinterpret_cast<uint32_t *>(packed_data), M, K, BIT, stream);
+    if (rc != ABQ_OK)
+        printf("[ABQ][Error] pack failed: %s\n", abq_status_string(rc));
+}
+
+void ABQGEMMWrapper::gemm(const int M, const int N, const int K, const _Float16 *A, const int *B, const _Float16 *C,
+                          _Float16 *D, const float *scale, const float *scale_inter, const float *scale_out, bool bias,
+                          char *abq_gemm_workspace, size_t abq_gemm_ws_bytes, hipStream_t stream)
+{
+    (void)C;
+    (void)scale_inter;
+    if (K < 128 || K % 128 != 0) {
+        printf("[ABQ][Error] unsupport K = %d\n", K);
+        return;
+    }
+    if (abq_gemm_ws_bytes < (size_t)x_bits_ * M * K / 8) {
+        printf("[ABQ][Error] workspace too small: %zu bytes for M,K,bits = %d,%d,%d\n", abq_gemm_ws_bytes, M, K, x_bits_);
+        return;
+    }
+    // quant + packing
+    pack(A, scale, reinterpret_cast<int *>(abq_gemm_workspace), M, K, x_bits_, stream);
+    abq_gemm_state state;
+    const abq_status rc = abq_gemm_init(nullptr, x_bits_, w_bits_, signed_ ? 1 : 0,
+                                        reinterpret_cast<const uint32_t *>(abq_gemm_workspace),
+                                        reinterpret_cast<const uint32_t *>(B), M, N, K, D, scale_out, bias ? 1 : 0,
+                                        ABQ_OUT_F16_TENSOR_F32SCALE, &state);
+    if (rc == ABQ_ERR_UNSUPPORTED) {
+        printf("[ABQ][Error] unsupport w%da%d\n", w_bits_, x_bits_);
+        return;
+    }
+    if (rc != ABQ_OK || !state.init_success) {
+        printf("[ABQ][Error] return due to unsuccessful initialization.\n");
+        return;
+    }
+    const abq_status ex = abq_gemm_exec(&state, stream);
+    if (ex != ABQ_OK)
+        printf("[ABQ][Error] launch failed: %s\n", abq_status_string(ex));
+}
+
+void ABQGEMMWrapper::gemm_scaled(const int M, const int N, const int K, const int *X_packed, const int *B, _Float16 *D,
+                                 const float *x_scale, const float *w_scale, hipStream_t stream)
+{
+    if (K < 128 || K % 128 != 0) {
+        printf("[ABQ][Error] unsupport K = %d\n", K);
+        return;
+    }
+    abq_gemm_state state;
+    abq_status rc = abq_gemm_init(nullptr, x_bits_, w_bits_, signed_ ? 1 : 0, reinterpret_cast<const uint32_t *>(X_packed),
+                                  reinterpret_cast<const uint32_t *>(B), M, N, K, D, nullptr, 0, ABQ_OUT_F16_SCALED, &state);
+    if (rc == ABQ_OK)
+        rc = abq_gemm_set_scales(&state, x_scale, w_scale, 0);
+    if (rc != ABQ_OK || !state.init_success) {
+        printf("[ABQ][Error] return due to unsuccessful initialization.\n");
+        return;
+    }
+    const abq_status ex = abq_gemm_exec(&state, stream);
+    if (ex != ABQ_OK)
+        printf("[ABQ][Error] launch failed: %s\n", abq_status_string(ex));
+}

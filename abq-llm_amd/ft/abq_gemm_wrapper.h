@@ -1,0 +1,43 @@
+// ABQGEMMWrapper: the class the FasterTransformer LLaMA layers call when int8_mode == 5
+// (reference: fastertransformer/src/fastertransformer/kernels/abqgemm/abq_gemm_wrapper.h:6-32;
+// call sites FfnLayer.cc:341-374,489-505, DecoderSelfAttentionLayer.cc:605-621,746-761,
+// GptContextAttentionLayer.cc:150-166,519-535).  Same constructor and method signatures with
+// hipStream_t / _Float16 in place of cudaStream_t / half.
+//
+// Behaviour kept: activation quantisation value = (int)(half(x) * half(scale[0])) with no
+// rounding and no clamp; K must be >= 128 and a multiple of 128; failures print
+// "[ABQ][Error] ..." and return.  Behaviour changed on purpose:
+//  * every bit combination the library has kernels for is accepted, not only W2A8, and the tile
+//    is the library's choice for (M, N, K) instead of the two hard-coded tiles;
+//  * scale_out[0] is read as the float it is (the reference reinterprets the pointer as half*
+//    and reads the low 16 bits of the float, abq_gemm_wrapper.cu:126);
+//  * the workspace size is checked.
+// gemm_scaled() is new: per-token activation scales and per-channel weight scales.
+#pragma once
+#include <hip/hip_runtime_api.h>
+#include <stddef.h>
+
+class ABQGEMMWrapper {
+private:
+    int x_bits_;
+    int w_bits_;
+    bool signed_;
+
+public:
+    ABQGEMMWrapper(int X_BITS, int W_BITS, bool SIGNED);
+    ~ABQGEMMWrapper();
+
+    void pack(const int *in_data, int *packed_data, int M, int K, int BIT, hipStream_t stream);
+    void pack(const _Float16 *in_data, const float *scale, int *packed_data, int M, int K, int BIT,
+              hipStream_t stream);
+    // A: fp16 activations [M][K]; B: packed weight planes [w_bits][N][K/32]; C unused;
+    // D: fp16 [M][N]; scale: activation quantisation scale (1 float, device);
+    // scale_inter unused; scale_out: output scale (1 float, device);
+    // abq_gemm_workspace: at least X_BITS * M * K / 8 bytes of device memory.
+    void gemm(const int M, const int N, const int K, const _Float16 *A, const int *B, const _Float16 *C,
+              _Float16 *D, const float *scale, const float *scale_inter, const float *scale_out, bool bias,
+              char *abq_gemm_workspace, size_t abq_gemm_ws_bytes, hipStream_t stream);
+    // D[m][n] = acc[m][n] * x_scale[m] * w_scale[n]; X given as already packed planes.
+    void gemm_scaled(const int M, const int N, const int K, const int *X_packed, const int *B, _Float16 *D,
+                     const float *x_scale, const float *w_scale, hipStream_t stream);
+};

@@ -128,8 +128,12 @@ typedef enum abq_out_kind {
     ABQ_OUT_I32 = 0,        /* int32 D (engine/mma_any/aq_bmma_kernel.h:485-580)                 */
     ABQ_OUT_F16_TENSOR = 1, /* fp16 D = half(acc) * C[0], C one fp16 on the device
                                (FT abqgemm/mma_any/aq_bmma_kernel.h:479,516-519)               */
-    ABQ_OUT_F16_SCALED = 2  /* fp16 D = acc * x_scale[m] * w_scale[n] (fp32 math), per-token
+    ABQ_OUT_F16_SCALED = 2, /* fp16 D = acc * x_scale[m] * w_scale[n] (fp32 math), per-token
                                and per-channel scales; see abq_gemm_set_scales                 */
+    ABQ_OUT_F16_TENSOR_F32SCALE = 3 /* as ABQ_OUT_F16_TENSOR, but C points to one float on the
+                               device, converted to fp16 first: what the FT wrapper means when it
+                               hands `const float* scale_out` to the kernel
+                               (abq_gemm_wrapper.cu:125-126)                                   */
 } abq_out_kind;
 
 /* Launch state, the POD returned by the reference's InitFn (AqBMMAOpState,

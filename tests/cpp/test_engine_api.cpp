@@ -1,0 +1,198 @@
+// Exercises the C++ face of the library the way the reference's own harness and the FT layers
+// use theirs: named Init/Exec globals (engine/test/test_mma/test_mma.h:68-160), launch_pack,
+// launchWmmaAnyKernel and ABQGEMMWrapper::gemm.  Results are compared with the CPU oracle
+// (oracle/abq_oracle.h) bit for bit.  `--no-gpu` runs only the host-side error paths.
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#define ABQ_ALL_COMBOS
+#include "common/pack.h"
+#include "common/timer.h"
+#include "mma_any/aq_bmma_library.h"
+#include "mma_any/aq_wmma_library.h"
+#include "wmma_any/wmma_any.h"
+#include "abq_gemm_wrapper.h"
+#include "abq_oracle.h"
+
+// reference (tensor-core) tuples, declared here the way a user of the reference would
+AQ_DECL_FUN(AqBMMA, 8, 2, true, 1, 48, 512, 8, 24, 128, 8, 8, 128, 4)
+AQ_DECL_FUN(AqBMMA, 8, 2, true, 8, 48, 256, 32, 48, 128, 8, 8, 128, 5)
+AQ_DECL_FUN(AqBWMMA, 8, 2, false, 8, 48, 256, 32, 48, 128, 8, 8, 128, 5)
+
+static int failures = 0;
+#define CHECK(cond)                                                        \
+    do {                                                                   \
+        if (!(cond)) {                                                     \
+            std::printf("CHECK FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+            ++failures;                                                    \
+        }                                                                  \
+    } while (0)
+#define HIP_OK(x) CHECK((x) == hipSuccess)
+
+static void host_paths()
+{
+    int *fake = reinterpret_cast<int *>(0x1000);
+    // K constraint (engine/test_any_mma.cu:99): init reports failure, nothing is launched
+    AqBMMAOpState st = (*AqBMMA_8x2xtrue_16x16x4096_16x16x512_16x16x64_3_InitFn)(fake, fake, 1, 64, 100, fake, nullptr, false);
+    CHECK(!st.initSuccess);
+    st = (*AqBMMA_8x2xtrue_16x16x4096_16x16x512_16x16x64_3_InitFn)(fake, fake, 8, 4096, 4096, fake, nullptr, false);
+    CHECK(st.initSuccess && st.args.M == 8 && st.args.N == 4096 && st.args.K == 4096);
+    CHECK(st.gridDim.x == 256 && st.blockDim.x == 512); // the named 8-wave decode tile
+    CHECK(st.native.strategy == ABQ_STRATEGY_DECODE);
+    // a reference tuple resolves to the library's choice
+    st = (*AqBMMA_8x2xtrue_1x48x512_8x24x128_8x8x128_4_InitFn)(fake, fake, 1, 4096, 4096, fake, nullptr, false);
+    CHECK(st.initSuccess && st.native.strategy != ABQ_STRATEGY_AUTO);
+    AqBWMMAOpState sw = (*AqBWMMA_8x2xfalse_8x48x256_32x48x128_8x8x128_5_InitFn)(fake, fake, 8, 512, 1024, fake, nullptr, false);
+    CHECK(sw.initSuccess);
+    // the wrapper refuses bad K and short workspaces before touching the device
+    ABQGEMMWrapper wrap(8, 2, true);
+    wrap.gemm(1, 64, 100, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, false, nullptr, 0, nullptr);
+    wrap.gemm(4, 64, 256, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, false, nullptr, 16, nullptr);
+}
+
+struct Case {
+    int M, N, K, q, p;
+    bool is_signed;
+};
+
+static void fill(std::vector<int> &v, int bits, bool is_signed, std::mt19937_64 &rng)
+{
+    const int lo = is_signed ? -(1 << (bits - 1)) : 0;
+    for (auto &e : v)
+        e = lo + (int)(rng() % (1u << bits));
+}
+
+template <typename InitFn, typename ExecFn, typename State>
+static bool run_config(InitFn init_fn, ExecFn exec_fn, const Case &c, int *d_xp, int *d_wp, int *d_out,
+                       const std::vector<int> &ref, hipStream_t stream)
+{
+    HIP_OK(hipMemsetAsync(d_out, 0xff, (size_t)c.M * c.N * 4, stream));
+    State state = (*init_fn)(d_xp, d_wp, c.M, c.N, c.K, d_out, nullptr, false);
+    if (!state.initSuccess)
+        return false;
+    (*exec_fn)(state, stream);
+    if (hipStreamSynchronize(stream) != hipSuccess || hipGetLastError() != hipSuccess)
+        return false;
+    std::vector<int> out((size_t)c.M * c.N);
+    HIP_OK(hipMemcpy(out.data(), d_out, out.size() * 4, hipMemcpyDeviceToHost));
+    return std::memcmp(out.data(), ref.data(), out.size() * 4) == 0;
+}
+
+static void gpu_paths()
+{
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+    std::mt19937_64 rng(7);
+    const Case c{ 8, 1000, 1152, 8, 2, true };
+    std::vector<int> hx((size_t)c.M * c.K), hw((size_t)c.N * c.K);
+    fill(hx, c.q, c.is_signed, rng);
+    fill(hw, c.p, c.is_signed, rng);
+    const size_t KW = c.K / 32, xw = (size_t)c.q * c.M * KW, ww = (size_t)c.p * c.N * KW;
+    int *d_x, *d_w, *d_xp, *d_wp, *d_out;
+    HIP_OK(hipMalloc(&d_x, hx.size() * 4));
+    HIP_OK(hipMalloc(&d_w, hw.size() * 4));
+    HIP_OK(hipMalloc(&d_xp, xw * 4));
+    HIP_OK(hipMalloc(&d_wp, ww * 4));
+    HIP_OK(hipMalloc(&d_out, (size_t)c.M * c.N * 4));
+    HIP_OK(hipMemcpy(d_x, hx.data(), hx.size() * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d_w, hw.data(), hw.size() * 4, hipMemcpyHostToDevice));
+    HIP_OK(launch_pack(d_w, d_wp, c.N, c.K, c.p, stream));
+    HIP_OK(launch_pack(d_x, d_xp, c.M, c.K, c.q, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+
+    // packed planes against the oracle's pack, expected GEMM from the oracle's compute_ref
+    std::vector<uint32_t> xp(xw), wp(ww), xp_ref(xw), wp_ref(ww);
+    HIP_OK(hipMemcpy(xp.data(), d_xp, xw * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(wp.data(), d_wp, ww * 4, hipMemcpyDeviceToHost));
+    abq_oracle_pack_i32(hx.data(), xp_ref.data(), c.M, c.K, c.q);
+    abq_oracle_pack_i32(hw.data(), wp_ref.data(), c.N, c.K, c.p);
+    CHECK(xp == xp_ref && wp == wp_ref);
+    std::vector<int> ref((size_t)c.M * c.N);
+    abq_oracle_gemm_bitserial(wp_ref.data(), xp_ref.data(), ref.data(), c.M, c.N, c.K, c.p, c.q, c.is_signed);
+
+#define RUN(type, ...)                                                                                        \
+    CHECK((run_config<AQ_INIT_FUN(type), AQ_EXEC_FUN(type), AQ_OP_STATE(type)>(                               \
+        AQ_NAME_FUN(type, Init, __VA_ARGS__), AQ_NAME_FUN(type, Exec, __VA_ARGS__), c, d_xp, d_wp, d_out, ref, stream)))
+    RUN(AqBMMA, 8, 2, true, 1, 8, 4096, 1, 2, 4096, 1, 1, 128, 1);          // VALU popcount
+    RUN(AqBMMA, 8, 2, true, 16, 16, 4096, 16, 16, 512, 16, 16, 64, 3);      // decode kernel
+    RUN(AqBMMA, 8, 2, true, 16, 16, 4096, 16, 16, 512, 16, 16, 64, 2);      // int8 MFMA 16x16x64
+    RUN(AqBMMA, 8, 2, true, 128, 128, 256, 64, 64, 256, 32, 32, 32, 2);     // int8 MFMA 32x32x32
+    RUN(AqBWMMA, 8, 2, true, 16, 16, 8192, 16, 16, 512, 16, 16, 64, 3);     // same kernels, wmma names
+    RUN(AqBMMA, 8, 2, true, 8, 48, 256, 32, 48, 128, 8, 8, 128, 5);         // FT tile by its reference name
+#undef RUN
+
+    {   // first-generation entry point
+        HIP_OK(hipMemsetAsync(d_out, 0xff, (size_t)c.M * c.N * 4, stream));
+        AnyQuantParams params{ d_xp, d_wp, nullptr, d_out, false, c.M, c.N, c.K };
+        hipError_t e = launchWmmaAnyKernel<QuantType<8, 2, true>, ShapeBase<16, 16, 4096>, ShapeBase<16, 16, 512>,
+                                           ShapeBase<16, 16, 64>, 3>(params, stream);
+        CHECK(e == hipSuccess);
+        std::vector<int> out((size_t)c.M * c.N);
+        HIP_OK(hipStreamSynchronize(stream));
+        HIP_OK(hipMemcpy(out.data(), d_out, out.size() * 4, hipMemcpyDeviceToHost));
+        CHECK(out == ref);
+    }
+
+    {   // FT wrapper: fp16 activations, static scale, fp16 output scaled by scale_out
+        const float in_scale = 21.0f, out_scale = 0.0123f;
+        std::vector<uint16_t> ha((size_t)c.M * c.K);
+        std::normal_distribution<float> nd(0.f, 2.f);
+        std::mt19937 r32(3);
+        for (auto &h : ha)
+            h = abq_oracle_f32_to_f16(nd(r32));
+        _Float16 *d_a, *d_d;
+        float *d_scales;
+        char *d_ws;
+        const size_t ws_bytes = (size_t)c.q * c.M * c.K / 8;
+        HIP_OK(hipMalloc(&d_a, ha.size() * 2));
+        HIP_OK(hipMalloc(&d_d, (size_t)c.M * c.N * 2));
+        HIP_OK(hipMalloc(&d_scales, 8));
+        HIP_OK(hipMalloc(&d_ws, ws_bytes));
+        HIP_OK(hipMemcpy(d_a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
+        const float scales[2] = { in_scale, out_scale };
+        HIP_OK(hipMemcpy(d_scales, scales, 8, hipMemcpyHostToDevice));
+        ABQGEMMWrapper wrap(c.q, c.p, c.is_signed);
+        wrap.gemm(c.M, c.N, c.K, d_a, d_wp, nullptr, d_d, d_scales, nullptr, d_scales + 1, false, d_ws, ws_bytes, stream);
+        HIP_OK(hipStreamSynchronize(stream));
+        std::vector<uint16_t> got((size_t)c.M * c.N), want((size_t)c.M * c.N);
+        HIP_OK(hipMemcpy(got.data(), d_d, got.size() * 2, hipMemcpyDeviceToHost));
+        std::vector<uint32_t> ap(xw);
+        abq_oracle_pack_f16(ha.data(), in_scale, ap.data(), c.M, c.K, c.q);
+        std::vector<int> acc((size_t)c.M * c.N);
+        abq_oracle_gemm_bitserial(wp_ref.data(), ap.data(), acc.data(), c.M, c.N, c.K, c.p, c.q, c.is_signed);
+        abq_oracle_epilogue_f16(acc.data(), abq_oracle_f32_to_f16(out_scale), want.data(), (int)acc.size());
+        CHECK(got == want);
+        HIP_OK(hipFree(d_a));
+        HIP_OK(hipFree(d_d));
+        HIP_OK(hipFree(d_scales));
+        HIP_OK(hipFree(d_ws));
+    }
+
+    {   // timer interface
+        CudaTimer t(stream);
+        t.start();
+        t.stop();
+        CHECK(t.elapsed_msecs() >= 0.f);
+    }
+    HIP_OK(hipFree(d_x));
+    HIP_OK(hipFree(d_w));
+    HIP_OK(hipFree(d_xp));
+    HIP_OK(hipFree(d_wp));
+    HIP_OK(hipFree(d_out));
+    HIP_OK(hipStreamDestroy(stream));
+}
+
+int main(int argc, char **argv)
+{
+    const bool no_gpu = argc > 1 && !std::strcmp(argv[1], "--no-gpu");
+    host_paths();
+    if (!no_gpu)
+        gpu_paths();
+    std::printf("%s (%d failed checks)\n", failures ? "FAILED" : "PASSED", failures);
+    return failures ? 1 : 0;
+}

@@ -197,7 +197,7 @@ def test_init_error_paths(abq):
 
 
 def test_default_strategy_choice_and_reference_tuples(abq):
-    for M, want in ((1, abq.STRATEGY_BCNT), (2, abq.STRATEGY_BCNT), (4, abq.STRATEGY_DECODE),
+    for M, want in ((1, abq.STRATEGY_DECODE), (2, abq.STRATEGY_DECODE), (4, abq.STRATEGY_DECODE),
                     (8, abq.STRATEGY_DECODE), (16, abq.STRATEGY_DECODE), (128, abq.STRATEGY_MFMA32),
                     (2048, abq.STRATEGY_MFMA32)):
         rc, st = _init(abq, M=M, N=4096)
@@ -206,7 +206,7 @@ def test_default_strategy_choice_and_reference_tuples(abq):
     cfg, _ = abq.parse_kernel_name("AqBMMA_8x2xtrue_8x48x256_32x48x128_8x8x128_5")
     rc, st = _init(abq, cfg=cfg, M=8)
     assert rc == 0 and st.strategy == abq.STRATEGY_DECODE and st.cfg.mma_k == 64 and st.cfg.nstage == 3
-    assert st.grid_dim.x == 4 and st.block_dim.x == 512
+    assert st.grid_dim.x == 4 and st.block_dim.x == 1024
 
 
 @pytest.mark.parametrize("q,p", COMBOS)
