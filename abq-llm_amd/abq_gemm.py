@@ -18,8 +18,9 @@ STATUS_NAMES = {
     4: "ABQ_ERR_NOT_INITIALIZED", 5: "ABQ_ERR_LAUNCH", 6: "ABQ_ERR_NO_DEVICE", 7: "ABQ_ERR_TOO_LARGE",
 }
 OUT_I32, OUT_F16_TENSOR, OUT_F16_SCALED, OUT_F16_TENSOR_F32SCALE = 0, 1, 2, 3
-STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC, STRATEGY_DECODE = range(6)
-STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic", "decode"]
+STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC, STRATEGY_DECODE, STRATEGY_TILED = range(7)
+STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic", "decode", "tiled"]
+LAYOUT_PLANES, LAYOUT_TILED = 0, 1
 
 # every symbol include/abq_gemm.h declares
 EXPORTED = [
@@ -28,6 +29,8 @@ EXPORTED = [
     "abq_parse_kernel_name", "abq_format_kernel_name",
     "abq_native_config_count", "abq_native_config_get",
     "abq_gemm_init", "abq_gemm_set_scales", "abq_gemm_exec", "abq_gemm_launch",
+    "abq_planes_bytes", "abq_relayout_planes", "abq_gemm_set_operand_layout", "abq_gemm_workspace_bytes",
+    "abq_gemm_set_workspace",
 ]
 
 
@@ -60,6 +63,8 @@ class GemmState(ctypes.Structure):
         ("x_scale", ctypes.c_void_p), ("w_scale", ctypes.c_void_p),
         ("group_size", ctypes.c_int),
         ("reserved", ctypes.c_int * 5),
+        ("x_layout", ctypes.c_int), ("w_layout", ctypes.c_int), ("auto_chosen", ctypes.c_int),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
     ]
 
 
@@ -98,6 +103,13 @@ def lib():
         L.abq_gemm_set_scales.argtypes = [ctypes.POINTER(GemmState), vp, vp, ci]
         L.abq_gemm_exec.argtypes = [ctypes.POINTER(GemmState), vp]
         L.abq_gemm_launch.argtypes = [ctypes.POINTER(TileConfig), vp, vp, vp, vp, ci, ci, ci, ci, vp]
+        L.abq_planes_bytes.argtypes = [ci, ci, ci]
+        L.abq_planes_bytes.restype = ctypes.c_size_t
+        L.abq_relayout_planes.argtypes = [vp, vp, ci, ci, ci, vp]
+        L.abq_gemm_set_operand_layout.argtypes = [ctypes.POINTER(GemmState), ci, ci]
+        L.abq_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GemmState)]
+        L.abq_gemm_workspace_bytes.restype = ctypes.c_size_t
+        L.abq_gemm_set_workspace.argtypes = [ctypes.POINTER(GemmState), vp, ctypes.c_size_t]
         _lib = L
     return _lib
 
@@ -177,14 +189,37 @@ def pack_f16(values, scale, bits, out=None, stream=None):
     return out
 
 
+def relayout_planes(planes, out=None, stream=None):
+    """planes int32 tensor [bits, rows, k/32] -> K-tiled tensor [k/128, rows, bits, 4]."""
+    import torch
+    bits, rows, kw = planes.shape
+    assert planes.is_cuda and planes.is_contiguous() and kw % 4 == 0
+    if out is None:
+        out = torch.empty((kw // 4, rows, bits, 4), dtype=torch.int32, device=planes.device)
+    _check(lib().abq_relayout_planes(planes.data_ptr(), out.data_ptr(), rows, kw * 32, bits, _stream_ptr(stream)),
+           "abq_relayout_planes")
+    return out
+
+
 class Gemm:
-    """One initialised GEMM (the role of AqBMMAOpState + InitFn/ExecFn in the reference)."""
+    """One initialised GEMM (the role of AqBMMAOpState + InitFn/ExecFn in the reference).
+
+    x_planes / w_planes are in the reference layout [bits, rows, k/32] unless x_tiled / w_tiled
+    say they were converted with relayout_planes ([k/128, rows, bits, 4])."""
 
     def __init__(self, x_planes, w_planes, signed, out=None, cfg=None, out_kind=OUT_I32, c_scale=None,
-                 x_scale=None, w_scale=None, group_size=0):
+                 x_scale=None, w_scale=None, group_size=0, x_tiled=False, w_tiled=False, workspace=None):
         import torch
-        q, M, kw = x_planes.shape
-        p, N, kw2 = w_planes.shape
+        if x_tiled:
+            kt, M, q, _ = x_planes.shape
+            kw = kt * 4
+        else:
+            q, M, kw = x_planes.shape
+        if w_tiled:
+            kt2, N, p, _ = w_planes.shape
+            kw2 = kt2 * 4
+        else:
+            p, N, kw2 = w_planes.shape
         assert kw == kw2 and x_planes.is_cuda and w_planes.is_cuda
         assert x_planes.is_contiguous() and w_planes.is_contiguous()
         K = kw * 32
@@ -202,6 +237,17 @@ class Gemm:
         if out_kind == OUT_F16_SCALED:
             _check(lib().abq_gemm_set_scales(ctypes.byref(self.state), x_scale.data_ptr(), w_scale.data_ptr(),
                                              group_size), "abq_gemm_set_scales")
+        if x_tiled or w_tiled:
+            _check(lib().abq_gemm_set_operand_layout(ctypes.byref(self.state), int(x_tiled), int(w_tiled)),
+                   "abq_gemm_set_operand_layout")
+        self.workspace = workspace
+        if workspace is not None:
+            _check(lib().abq_gemm_set_workspace(ctypes.byref(self.state), workspace.data_ptr(),
+                                                workspace.numel() * workspace.element_size()), "abq_gemm_set_workspace")
+
+    @property
+    def workspace_bytes(self):
+        return lib().abq_gemm_workspace_bytes(ctypes.byref(self.state))
 
     @property
     def strategy(self):

@@ -14,6 +14,7 @@ namespace abq {
 hipError_t launch_pack_i32(const int32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_pack_f16(const void *, const float *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
+hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 
 // (x_bits, w_bits) pairs with specialised kernels: the twelve of the reference library
 // (engine/mma_any/aq_bmma_impl/aq_bmma_w{2a2,...,8a8}.h).
@@ -24,7 +25,8 @@ hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream
 #define ABQ_DECL(Q, P)                                \
     void abq_mfma_register_##Q##_##P(KernelTable *);  \
     void abq_bcnt_register_##Q##_##P(KernelTable *);  \
-    void abq_decode_register_##Q##_##P(KernelTable *);
+    void abq_decode_register_##Q##_##P(KernelTable *); \
+    void abq_tiled_register_##Q##_##P(KernelTable *);
 ABQ_FOR_EACH_COMBO(ABQ_DECL)
 #undef ABQ_DECL
 
@@ -32,6 +34,7 @@ struct Registry {
     KernelTable mfma[2 * ABQ_NUM_COMBOS];
     KernelTable bcnt[2 * ABQ_NUM_COMBOS];
     KernelTable decode[2 * ABQ_NUM_COMBOS];
+    KernelTable tiled[2 * ABQ_NUM_COMBOS];
     Registry()
     {
         int i = 0;
@@ -39,6 +42,7 @@ struct Registry {
     abq_mfma_register_##Q##_##P(&mfma[i]);             \
     abq_bcnt_register_##Q##_##P(&bcnt[i]);             \
     abq_decode_register_##Q##_##P(&decode[i]);         \
+    abq_tiled_register_##Q##_##P(&tiled[i]);           \
     i += 2;
         ABQ_FOR_EACH_COMBO(ABQ_REG)
 #undef ABQ_REG
@@ -91,7 +95,7 @@ static void entry_to_config(const KernelEntry &e, int strategy, int x_bits, int 
         c->mma_k = 128;
         c->nstage = 1;
     } else {
-        const int stepk = (64 / e.mi) * 4 * 32;
+        const int stepk = e.nstage == 4 ? 128 : (64 / e.mi) * 4 * 32; // NSTAGE 4: K-tiled layout, 128-element K tiles
         c->block_m = e.mi * e.tm * e.wm;
         c->block_n = e.mi * e.tn * e.wn;
         c->block_k = stepk * e.wk;
@@ -205,7 +209,7 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
             lpr_log2 = lpr == 16 ? 4 : lpr == 32 ? 5 : 6;
     } else {
         mi = cfg->mma_m;
-        const int stepk = (64 / mi) * 4 * 32;
+        const int stepk = (strategy == ABQ_STRATEGY_MFMA32 && cfg->nstage == 4) ? 128 : (64 / mi) * 4 * 32;
         if (cfg->warp_m <= 0 || cfg->warp_n <= 0 || cfg->warp_m % mi || cfg->warp_n % mi ||
             cfg->block_m % cfg->warp_m || cfg->block_n % cfg->warp_n || cfg->warp_k != stepk ||
             cfg->block_k % stepk)
@@ -215,6 +219,32 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         wk = cfg->block_k / stepk;
         if (strategy == ABQ_STRATEGY_MFMA16 && cfg->nstage == 3)
             strategy = ABQ_STRATEGY_DECODE;
+        if (strategy == ABQ_STRATEGY_MFMA32 && cfg->nstage == 4)
+            strategy = ABQ_STRATEGY_TILED;
+    }
+
+    if (strategy == ABQ_STRATEGY_TILED) {
+        const KernelTable *tt_ = find_table(reg.tiled, x_bits, w_bits, is_signed);
+        if (!tt_ || mi != 32 || wm != 2 || wn != 2 || wk != 1)
+            return ABQ_ERR_UNSUPPORTED;
+        int v = -1;
+        for (int i = 0; i < tt_->count; ++i)
+            if (tt_->entries[i].tm == tm && tt_->entries[i].tn == tn)
+                v = i;
+        if (v < 0)
+            return ABQ_ERR_UNSUPPORTED;
+        if (K >= (1 << 17))
+            return ABQ_ERR_TOO_LARGE;
+        const KernelEntry &e = tt_->entries[v];
+        const int bm = 64 * e.tm, bn = 64 * e.tn;
+        const int mblocks = (M + bm - 1) / bm, npx = ((N + bn - 1) / bn + 7) / 8;
+        st->strategy = strategy;
+        st->variant = v;
+        entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
+        st->grid_dim = abq_dim3{ (unsigned)(8 * npx * mblocks), 1, 1 };
+        st->block_dim = abq_dim3{ 256, 1, 1 };
+        st->shared_mem_size = 2 * (size_t)(bm + bn) * 144 + (bm + bn) * 4;
+        return ABQ_OK;
     }
 
     if (strategy == ABQ_STRATEGY_DECODE) {
@@ -404,9 +434,10 @@ int abq_native_config_count(int x_bits, int w_bits, int is_signed)
     const KernelTable *tb = find_table(reg.bcnt, x_bits, w_bits, is_signed);
     const KernelTable *tm = find_table(reg.mfma, x_bits, w_bits, is_signed);
     const KernelTable *td = find_table(reg.decode, x_bits, w_bits, is_signed);
-    if (!tb || !tm || !td)
+    const KernelTable *tt = find_table(reg.tiled, x_bits, w_bits, is_signed);
+    if (!tb || !tm || !td || !tt)
         return 0;
-    return tb->count * 3 + td->count + tm->count;
+    return tb->count * 3 + td->count + tm->count + tt->count;
 }
 
 abq_status abq_native_config_get(int x_bits, int w_bits, int is_signed, int index, abq_tile_config *cfg)
@@ -430,8 +461,14 @@ abq_status abq_native_config_get(int x_bits, int w_bits, int is_signed, int inde
         return ABQ_OK;
     }
     index -= td->count;
-    if (index >= tm->count)
-        return ABQ_ERR_INVALID_ARG;
+    if (index >= tm->count) {
+        const KernelTable *tt = find_table(reg.tiled, x_bits, w_bits, is_signed);
+        index -= tm->count;
+        if (!tt || index >= tt->count)
+            return ABQ_ERR_INVALID_ARG;
+        entry_to_config(tt->entries[index], ABQ_STRATEGY_TILED, x_bits, w_bits, is_signed, 0, cfg);
+        return ABQ_OK;
+    }
     const KernelEntry &e = tm->entries[index];
     entry_to_config(e, e.mi == 16 ? ABQ_STRATEGY_MFMA16 : ABQ_STRATEGY_MFMA32, x_bits, w_bits,
                     is_signed, 0, cfg);
@@ -479,7 +516,41 @@ abq_status abq_gemm_init(const abq_tile_config *cfg, int x_bits, int w_bits, int
     state->D = D;
     state->bias = 0;
     state->out_kind = out_kind;
+    state->auto_chosen = (!cfg || strategy_of_mma(*cfg) == ABQ_STRATEGY_AUTO) ? 1 : 0;
     state->init_success = 1;
+    return ABQ_OK;
+}
+
+// ---- K-tiled layout, workspace -------------------------------------------------------------
+
+static size_t planes_bytes(int rows, int k, int bits) { return (size_t)bits * rows * (k / 32) * 4; }
+
+// Picks the tiled-kernel tile for a shape: the largest tile that still gives every compute unit
+// work, preferring 256x256 (best operand reuse) when at least one full wave of tiles exists.
+static abq_status switch_to_tiled(abq_gemm_state *st)
+{
+    const Registry &reg = registry();
+    const abq_tile_config &c = st->cfg;
+    const KernelTable *tt = find_table(reg.tiled, c.x_bits, c.w_bits, c.is_signed);
+    if (!tt)
+        return ABQ_ERR_UNSUPPORTED;
+    static const int order[][2] = { { 4, 4 }, { 2, 4 }, { 2, 2 }, { 2, 1 }, { 1, 1 } };
+    int pick = -1;
+    for (const auto &o : order) {
+        const long tiles = (long)((st->M + 64 * o[0] - 1) / (64 * o[0])) * ((st->N + 64 * o[1] - 1) / (64 * o[1]));
+        for (int i = 0; i < tt->count; ++i)
+            if (tt->entries[i].tm == o[0] && tt->entries[i].tn == o[1] && (tiles >= 200 || (o[0] == 1 && o[1] == 1)) && pick < 0)
+                pick = i;
+    }
+    if (pick < 0)
+        return ABQ_ERR_UNSUPPORTED;
+    abq_tile_config cfg;
+    entry_to_config(tt->entries[pick], ABQ_STRATEGY_TILED, c.x_bits, c.w_bits, c.is_signed, 0, &cfg);
+    abq_gemm_state tmp = *st;
+    const abq_status rc = resolve(&cfg, c.x_bits, c.w_bits, c.is_signed, st->M, st->N, st->K, &tmp);
+    if (rc != ABQ_OK)
+        return rc;
+    *st = tmp;
     return ABQ_OK;
 }
 
@@ -523,6 +594,29 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     hipError_t e;
     if (st->strategy == ABQ_STRATEGY_GENERIC) {
         e = launch_bcnt_generic(a, c.x_bits, c.w_bits, c.is_signed, (hipStream_t)stream);
+    } else if (st->strategy == ABQ_STRATEGY_TILED) {
+        // operands still in the reference layout are converted into the caller's workspace
+        const size_t xb = st->x_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->M, st->K, c.x_bits);
+        const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, c.w_bits);
+        if (xb + wb > st->workspace_bytes || ((xb + wb) && !st->workspace))
+            return ABQ_ERR_INVALID_ARG;
+        char *ws = static_cast<char *>(st->workspace);
+        if (xb) {
+            e = launch_relayout_planes(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, c.x_bits, (hipStream_t)stream);
+            if (e != hipSuccess)
+                return hip_status(e);
+            a.X = reinterpret_cast<const uint32_t *>(ws);
+        }
+        if (wb) {
+            e = launch_relayout_planes(st->W, reinterpret_cast<uint32_t *>(ws + xb), st->N, st->K, c.w_bits, (hipStream_t)stream);
+            if (e != hipSuccess)
+                return hip_status(e);
+            a.W = reinterpret_cast<const uint32_t *>(ws + xb);
+        }
+        const KernelTable *t = find_table(reg.tiled, c.x_bits, c.w_bits, c.is_signed);
+        if (!t || st->variant < 0 || st->variant >= t->count)
+            return ABQ_ERR_NOT_INITIALIZED;
+        e = t->entries[st->variant].launch(a, (hipStream_t)stream);
     } else {
         const KernelTable *tables = st->strategy == ABQ_STRATEGY_BCNT     ? reg.bcnt
                                     : st->strategy == ABQ_STRATEGY_DECODE ? reg.decode
@@ -533,6 +627,64 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
         e = t->entries[st->variant].launch(a, (hipStream_t)stream);
     }
     return hip_status(e);
+}
+
+size_t abq_planes_bytes(int rows, int k, int bits)
+{
+    if (rows <= 0 || k <= 0 || bits <= 0 || k % 32)
+        return 0;
+    return planes_bytes(rows, k, bits);
+}
+
+abq_status abq_relayout_planes(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits, void *stream)
+{
+    if (!planes || !tiled || rows <= 0 || bits < 1 || bits > 8)
+        return ABQ_ERR_INVALID_ARG;
+    if (k < 128 || k % 128 != 0)
+        return ABQ_ERR_BAD_K;
+    return hip_status(launch_relayout_planes(planes, tiled, rows, k, bits, (hipStream_t)stream));
+}
+
+size_t abq_gemm_workspace_bytes(const abq_gemm_state *st)
+{
+    if (!st || !st->init_success)
+        return 0;
+    const size_t xb = st->x_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->M, st->K, st->cfg.x_bits);
+    const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, st->cfg.w_bits);
+    return xb + wb;
+}
+
+abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_layout)
+{
+    if (!st || !st->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    if ((x_layout != ABQ_LAYOUT_PLANES && x_layout != ABQ_LAYOUT_TILED) ||
+        (w_layout != ABQ_LAYOUT_PLANES && w_layout != ABQ_LAYOUT_TILED))
+        return ABQ_ERR_INVALID_ARG;
+    if ((x_layout == ABQ_LAYOUT_TILED || w_layout == ABQ_LAYOUT_TILED) && st->strategy != ABQ_STRATEGY_TILED) {
+        if (!st->auto_chosen)
+            return ABQ_ERR_UNSUPPORTED;
+        const abq_status rc = switch_to_tiled(st);
+        if (rc != ABQ_OK)
+            return rc;
+    }
+    st->x_layout = x_layout;
+    st->w_layout = w_layout;
+    return ABQ_OK;
+}
+
+abq_status abq_gemm_set_workspace(abq_gemm_state *st, void *workspace, size_t bytes)
+{
+    if (!st || !st->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    if (!workspace && bytes)
+        return ABQ_ERR_INVALID_ARG;
+    st->workspace = workspace;
+    st->workspace_bytes = bytes;
+    if (st->strategy != ABQ_STRATEGY_TILED && st->auto_chosen && st->M > 16 && workspace &&
+        bytes >= abq_gemm_workspace_bytes(st))
+        return switch_to_tiled(st);
+    return ABQ_OK;
 }
 
 abq_status abq_gemm_launch(const abq_tile_config *cfg, const uint32_t *X, const uint32_t *W,

@@ -103,6 +103,47 @@ __global__ __launch_bounds__(256) void pack_u4_kernel(const uint4 *__restrict__ 
     }
 }
 
+// planes[b][row][KW] -> tiled[kt][row][b][4]; one workgroup moves 32 rows x 8 K tiles through
+// LDS so that both the reads (128 contiguous bytes per row and plane) and the writes
+// (32 * bits * 16 contiguous bytes per K tile) are coalesced.
+__global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__restrict__ planes,
+                                                              uint32_t *__restrict__ tiled, int rows, int KW, int bits)
+{
+    __shared__ uint4 buf[8][32][9]; // [kt][row][plane], one spare column against bank conflicts
+    const int tid = threadIdx.x;
+    const int kt_tiles = KW / 4;
+    const int row0 = blockIdx.x * 32, kt0 = blockIdx.y * 8;
+    const size_t plane_stride = (size_t)rows * KW;
+    {
+        const int i = tid >> 3, j = tid & 7; // row, K tile: 8 threads read 128 contiguous bytes
+        const int row = row0 + i, kt = kt0 + j;
+        if (row < rows && kt < kt_tiles) {
+            const uint32_t *p = planes + (size_t)row * KW + 4 * kt;
+            for (int b = 0; b < bits; ++b)
+                buf[j][i][b] = *reinterpret_cast<const uint4 *>(p + b * plane_stride);
+        }
+    }
+    __syncthreads();
+    const int nrow = min(32, rows - row0);
+    for (int j = 0; j < 8; ++j) {
+        const int kt = kt0 + j;
+        if (kt >= kt_tiles)
+            break;
+        uint4 *dst = reinterpret_cast<uint4 *>(tiled) + ((size_t)kt * rows + row0) * bits;
+        for (int u = tid; u < nrow * bits; u += 256) // u = row * bits + plane: contiguous in memory
+            dst[u] = buf[j][u / bits][u % bits];
+    }
+}
+
+hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits,
+                                  hipStream_t stream)
+{
+    const int KW = k / 32;
+    const dim3 grid((rows + 31) / 32, (KW / 4 + 7) / 8);
+    hipLaunchKernelGGL(relayout_planes_kernel, grid, dim3(256), 0, stream, planes, tiled, rows, KW, bits);
+    return hipGetLastError();
+}
+
 static int grid_for(size_t items)
 {
     size_t blocks = (items + 255) / 256;

@@ -177,6 +177,15 @@ std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits)
         out.push_back(Tile{ v.mi * v.tm * v.wm, v.mi * v.tn * v.wn, stepk * v.wk, v.mi * v.tm, v.mi * v.tn,
                             stepk, v.mi, v.mi, 1024 / v.mi, v.wm, v.wn * v.wk, { 2 } });
     }
+    // LDS-staged prefill kernel on the K-tiled layout (NSTAGE = 4): 2 x 2 waves, TM x TN MFMA
+    // tiles of 32 x 32 per wave, K tile 128.  Double-buffered int8 tiles must fit 160 KiB of LDS.
+    const int tiled[][2] = { { 4, 4 }, { 2, 4 }, { 2, 2 }, { 2, 1 }, { 1, 1 } };
+    for (const auto &t : tiled) {
+        const int bm = 64 * t[0], bn = 64 * t[1];
+        if (2 * (bm + bn) * 144 + (bm + bn) * 4 > 160 * 1024)
+            continue;
+        out.push_back(Tile{ bm, bn, 128, 32 * t[0], 32 * t[1], 128, 32, 32, 32, 2, 2, { 4 } });
+    }
     return out;
 }
 

@@ -99,8 +99,10 @@ typedef enum abq_strategy {
     ABQ_STRATEGY_MFMA16 = 2, /* int8 MFMA 16x16x64     */
     ABQ_STRATEGY_MFMA32 = 3, /* int8 MFMA 32x32x32     */
     ABQ_STRATEGY_GENERIC = 4, /* any 1..16 bit pair, runtime loops (slow, always available) */
-    ABQ_STRATEGY_DECODE = 5   /* int8 MFMA 16x16x64, activations expanded once per workgroup
+    ABQ_STRATEGY_DECODE = 5,  /* int8 MFMA 16x16x64, activations expanded once per workgroup
                                  into LDS, persistent grid; tile tuples with NSTAGE = 3       */
+    ABQ_STRATEGY_TILED = 6    /* int8 MFMA 32x32x32, LDS-staged, operands in the K-tiled plane
+                                 layout (see abq_relayout_planes); tile tuples with NSTAGE = 4 */
 } abq_strategy;
 
 /* Parses "AqBMMA_8x2xtrue_1x48x512_8x24x128_8x8x128_4" (an optional _InitFn/_ExecFn suffix is
@@ -160,6 +162,11 @@ typedef struct abq_gemm_state {
     const float *w_scale;  /* [N] or [N][K/group_size] */
     int group_size;        /* 0 = per channel          */
     int reserved[5];
+    /* K-tiled operands (ABQ_STRATEGY_TILED) */
+    int x_layout, w_layout;  /* abq_layout of X and W as handed to init                    */
+    int auto_chosen;         /* 1 if the tile was the library's choice                     */
+    void *workspace;         /* caller-owned device scratch for the layout conversions     */
+    size_t workspace_bytes;
 } abq_gemm_state;
 
 /* Replaces AqBMMAInitFn / AqBWMMAInitFn (engine/mma_any/aq_bmma_op.h:141-147,163 and
@@ -176,6 +183,44 @@ abq_status abq_gemm_init(const abq_tile_config *cfg, int x_bits, int w_bits, int
  * algorithm/quantize/quantizer.py:111-179 (scale per row of X, per row of W). */
 abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, const float *w_scale,
                                int group_size);
+
+/* ---------------------------------------------------------------------------------------
+ * K-tiled plane layout (no counterpart in the reference; its kernels only exist for M <= 8).
+ *
+ * The prefill kernels (ABQ_STRATEGY_TILED) read the same bits in the order
+ *     tiled[kt][row][plane][4 words],   kt = K / 128 tiles,
+ * so that the rows of a workgroup tile are contiguous and every cache line fetched is used in
+ * full.  Same size as the reference layout.  Weights are static: convert them once with
+ * abq_relayout_planes and declare the layout with abq_gemm_set_operand_layout.  Operands left in
+ * the reference layout are converted inside abq_gemm_exec on every call into the caller's
+ * workspace (abq_gemm_set_workspace): activations always are unless the caller packs them
+ * tiled, weights only if they were not prepared.
+ * ------------------------------------------------------------------------------------- */
+typedef enum abq_layout {
+    ABQ_LAYOUT_PLANES = 0, /* the reference's wire format */
+    ABQ_LAYOUT_TILED = 1
+} abq_layout;
+
+/* bytes of a packed operand in either layout */
+size_t abq_planes_bytes(int rows, int k, int bits);
+
+/* planes [bits][rows][k/32] -> tiled [k/128][rows][bits][4]; k % 128 == 0. */
+abq_status abq_relayout_planes(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits,
+                               void *stream);
+
+/* Declares the layout of X and W of an initialised state.  A tiled operand moves a state whose
+ * tile was the library's choice to ABQ_STRATEGY_TILED; a state initialised with an explicit
+ * non-tiled tile tuple is refused (ABQ_ERR_UNSUPPORTED). */
+abq_status abq_gemm_set_operand_layout(abq_gemm_state *state, int x_layout, int w_layout);
+
+/* Workspace needed by abq_gemm_exec if the state ran as ABQ_STRATEGY_TILED with its current
+ * operand layouts (0 if both operands are tiled). */
+size_t abq_gemm_workspace_bytes(const abq_gemm_state *state);
+
+/* Hands a caller-owned device buffer to the state.  If the tile was the library's choice, M > 16
+ * and the buffer is large enough, the state moves to ABQ_STRATEGY_TILED; otherwise it keeps
+ * its kernel (which needs no workspace). */
+abq_status abq_gemm_set_workspace(abq_gemm_state *state, void *workspace, size_t bytes);
 
 /* Replaces AqBMMAExecFn / AqBWMMAExecFn (engine/mma_any/aq_bmma_op.h:155-161,164): one
  * asynchronous launch on `stream`. */

@@ -25,6 +25,15 @@ def planes_dev(planes):
     return torch.from_numpy(np.ascontiguousarray(planes).view(np.int32)).cuda()
 
 
+def run_cfg(abq, xd, wd, signed, cfg=None, **kw):
+    """Runs one configuration; kernels on the K-tiled layout get the workspace they ask for."""
+    g = abq.Gemm(xd, wd, signed, cfg=cfg, **kw)
+    if g.strategy == "tiled" and g.workspace_bytes and "workspace" not in kw:
+        ws = torch.empty(g.workspace_bytes, dtype=torch.uint8, device="cuda")
+        g = abq.Gemm(xd, wd, signed, cfg=cfg, workspace=ws, **kw)
+    return g.run()
+
+
 @pytest.fixture(scope="module", autouse=True)
 def _need_gpu():
     if not torch.cuda.is_available():
@@ -73,6 +82,38 @@ def test_pack_f16_all_finite_bit_patterns(abq, oracle, scale):
         assert np.array_equal(got & mask, want & mask)
 
 
+def test_relayout_planes_matches_closed_form(abq):
+    rng = np.random.default_rng(12)
+    for bits, rows, k in [(2, 1, 128), (8, 37, 1152), (4, 300, 4096), (3, 64, 13824)]:
+        planes = rng.integers(0, 1 << 32, size=(bits, rows, k // 32), dtype=np.uint64).astype(np.uint32)
+        got = abq.relayout_planes(planes_dev(planes)).cpu().numpy().view(np.uint32)
+        want = planes.reshape(bits, rows, k // 128, 4).transpose(2, 1, 0, 3)  # tiled[kt, r, b, :] = planes[b, r, 4kt:4kt+4]
+        assert np.array_equal(got, want)
+
+
+def test_tiled_kernels_with_prepared_operands(abq, oracle):
+    """K-tiled kernels fed tiled activations and/or tiled weights directly, ragged shapes."""
+    rng = np.random.default_rng(13)
+    for q, p, signed, M, N, K in [(8, 2, True, 300, 200, 640), (4, 4, False, 70, 513, 1152), (8, 8, False, 257, 129, 384)]:
+        x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+        xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
+        xt, wt = abq.relayout_planes(xd), abq.relayout_planes(wd)
+        want = oracle.np_gemm(x, w)
+        for cfg in [c for c in abq.native_configs(q, p, signed) if c.nstage == 4]:
+            got = abq.gemm(xt, wt, signed, cfg=cfg, x_tiled=True, w_tiled=True).cpu().numpy()
+            assert np.array_equal(got, want), abq.format_kernel_name(cfg)
+            ws = torch.empty(xd.numel() * 4, dtype=torch.uint8, device="cuda")
+            got = abq.gemm(xd, wt, signed, cfg=cfg, w_tiled=True, workspace=ws).cpu().numpy()
+            assert np.array_equal(got, want), abq.format_kernel_name(cfg)
+        # a state with an explicit non-tiled tile refuses tiled operands; exec without workspace is refused
+        cfg = [c for c in abq.native_configs(q, p, signed) if c.nstage == 2][0]
+        with pytest.raises(abq.AbqError):
+            abq.Gemm(xd, wt, signed, cfg=cfg, w_tiled=True)
+        cfg = [c for c in abq.native_configs(q, p, signed) if c.nstage == 4][0]
+        with pytest.raises(abq.AbqError):
+            abq.Gemm(xd, wd, signed, cfg=cfg).run()
+
+
 # ------------------------------------------------------------------ GEMM: every native tile, every combination
 
 SMALL_SHAPES = [(1, 64, 128), (3, 37, 384), (8, 130, 1152), (17, 64, 512), (33, 96, 256)]
@@ -92,8 +133,7 @@ def test_gemm_every_native_config_small_shapes(abq, oracle, q, p, signed):
         xd, wd = planes_dev(xp), planes_dev(wp)
         for cfg in cfgs:
             out = torch.full((M, N), -12345, dtype=torch.int32, device="cuda")
-            g = abq.Gemm(xd, wd, signed, out=out, cfg=cfg)
-            got = g.run().cpu().numpy()
+            got = run_cfg(abq, xd, wd, signed, cfg=cfg, out=out).cpu().numpy()
             assert np.array_equal(got, want), (abq.format_kernel_name(cfg), M, N, K)
         got = abq.gemm(xd, wd, signed).cpu().numpy()  # library's own choice
         assert np.array_equal(got, want)
@@ -110,7 +150,7 @@ def test_gemm_extreme_values_do_not_overflow(abq, oracle):
         xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
         want = oracle.np_gemm(x, w)
         for cfg in abq.native_configs(q, p, signed):
-            got = abq.gemm(xd, wd, signed, cfg=cfg).cpu().numpy()
+            got = run_cfg(abq, xd, wd, signed, cfg=cfg).cpu().numpy()
             assert np.array_equal(got, want), (q, p, signed, abq.format_kernel_name(cfg))
 
 
@@ -166,7 +206,7 @@ def test_fp16_per_tensor_epilogue_matches_reference_rounding(abq, oracle):
     for scale in (np.float16(0.0123), np.float16(1.0), np.float16(3.5e-3)):
         c = torch.tensor([float(scale)], dtype=torch.float16, device="cuda")
         for cfg in [None] + abq.native_configs(8, 2, True):
-            got = abq.gemm(xd, wd, True, cfg=cfg, out_kind=abq.OUT_F16_TENSOR, c_scale=c).cpu().numpy()
+            got = run_cfg(abq, xd, wd, True, cfg=cfg, out_kind=abq.OUT_F16_TENSOR, c_scale=c).cpu().numpy()
             want = oracle.epilogue_f16(acc, scale)
             assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
 
@@ -219,7 +259,7 @@ def test_config1_w2a8_decode_full_size(abq, oracle, N, K):
         for cfg in [None] + abq.native_configs(8, 2, True):
             if cfg is not None and cfg.mma_m == 32:
                 continue
-            got = abq.gemm(xd, wd, True, cfg=cfg).cpu().numpy()
+            got = run_cfg(abq, xd, wd, True, cfg=cfg).cpu().numpy()
             assert np.array_equal(got, want), (M, cfg)
 
 
@@ -232,14 +272,23 @@ def test_config2_prefill_full_size(abq, oracle, q, p, signed):
         w = rand_vals(rng, N, K, p, signed)
         wp = oracle.pack_i32(w, p)
         wd = planes_dev(wp)
+        wt = abq.relayout_planes(wd)  # weights prepared once in the K-tiled layout
         wf = torch.from_numpy(w).cuda().double()
         for M in (512, 2048):
             x = rand_vals(rng, M, K, q, signed)
             xp = oracle.pack_i32(x, q)
-            got_d = abq.gemm(planes_dev(xp), wd, signed)
+            xd = planes_dev(xp)
+            ws = torch.empty(xd.numel() * 4, dtype=torch.uint8, device="cuda")
+            g = abq.Gemm(xd, wt, signed, w_tiled=True, workspace=ws)
+            assert g.strategy == "tiled"
+            got_d = g.run()
             ref = torch.from_numpy(x).cuda().double() @ wf.T
             assert torch.equal(got_d.double(), ref), (q, p, signed, M, N, K)
             _sampled_oracle_check(oracle, xp, wp, signed, got_d.cpu().numpy(), rng, rows=2)
+            if M == 512:  # the kernel that needs no workspace
+                g2 = abq.Gemm(xd, wd, signed)
+                assert g2.strategy == "mfma32"
+                assert torch.equal(g2.run().double(), ref)
             del ref
 
 
@@ -251,7 +300,8 @@ def test_config3_bit_combo_sweep_m128(abq, oracle, q, p):
         for signed in (True, False):
             x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
             xp, wp = oracle.pack_i32(x, q), oracle.pack_i32(w, p)
-            got_d = abq.gemm(planes_dev(xp), planes_dev(wp), signed)
+            got_d = run_cfg(abq, planes_dev(xp), planes_dev(wp), signed,
+                            workspace=torch.empty((xp.size + wp.size) * 4, dtype=torch.uint8, device="cuda"))
             ref = torch.from_numpy(x).cuda().double() @ torch.from_numpy(w).cuda().double().T
             assert torch.equal(got_d.double(), ref), (q, p, signed, N, K)
             _sampled_oracle_check(oracle, xp, wp, signed, got_d.cpu().numpy(), rng, rows=2)
