@@ -525,8 +525,10 @@ abq_status abq_gemm_init(const abq_tile_config *cfg, int x_bits, int w_bits, int
 
 static size_t planes_bytes(int rows, int k, int bits) { return (size_t)bits * rows * (k / 32) * 4; }
 
-// Picks the tiled-kernel tile for a shape: the largest tile that still gives every compute unit
-// work, preferring 256x256 (best operand reuse) when at least one full wave of tiles exists.
+// Picks the tiled-kernel tile for a shape.  Measured on MI355X (W4A4 / W8A8 / W2A8, LLaMA shapes):
+// 128x128 is the fastest tile whenever it yields at least one workgroup per compute unit
+// (larger tiles lose to register pressure in the compiled inner loop, smaller ones to LDS
+// traffic); below that, smaller tiles win by filling the chip.
 static abq_status switch_to_tiled(abq_gemm_state *st)
 {
     const Registry &reg = registry();
@@ -534,7 +536,7 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
     const KernelTable *tt = find_table(reg.tiled, c.x_bits, c.w_bits, c.is_signed);
     if (!tt)
         return ABQ_ERR_UNSUPPORTED;
-    static const int order[][2] = { { 4, 4 }, { 2, 4 }, { 2, 2 }, { 2, 1 }, { 1, 1 } };
+    static const int order[][2] = { { 2, 2 }, { 2, 1 }, { 1, 1 } };
     int pick = -1;
     for (const auto &o : order) {
         const long tiles = (long)((st->M + 64 * o[0] - 1) / (64 * o[0])) * ((st->N + 64 * o[1] - 1) / (64 * o[1]));

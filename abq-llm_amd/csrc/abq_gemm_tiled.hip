@@ -15,16 +15,15 @@
 // relayout_planes_kernel below.
 //
 // Work split.  256 threads = 2 x 2 waves; a wave owns TM x TN MFMA tiles of 32 x 32, the
-// workgroup tile is (64*TM) x (64*TN), the K tile 128.  Per K tile each thread expands the
-// plane words of at most one activation row and one weight row to int8 (abq_bits.h) and
-// writes them to LDS, so every row is expanded once per workgroup; the waves read their MFMA
+// workgroup tile is (64*TM) x (64*TN), the K tile 128.  Per K tile each thread expands TM
+// word-sets (32 K elements each) of one activation row and TN of one weight row to int8
+// (abq_bits.h) and writes them to LDS, so every row is expanded once per workgroup and all
+// threads do the same amount of work without divergence; the waves read their MFMA
 // operands with ds_read_b128 (row stride 144 bytes: conflict free).  LDS is double buffered
 // and the plane words of the next two K tiles are in flight in registers, so the expansion
 // of tile i+1 and the loads of tile i+2 overlap the MFMAs of tile i; one barrier per K tile.
 // Workgroups are numbered so that the 8 XCDs (workgroup id modulo 8) each work on a
 // contiguous band of N with M fastest: a band's weight panels stay in that XCD's L2.
-#include <type_traits>
-
 #include "abq_kernels.h"
 
 #ifndef ABQ_Q
@@ -39,34 +38,40 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 constexpr int kTileK = 128;        // K elements per tile
 constexpr int kLdsRow = 144;       // bytes per expanded row in LDS (128 + 16 padding)
 
-template <int BITS>
-__device__ __forceinline__ void load_tile_row(uint4 (&dst)[BITS], const uint32_t *tiled, int rows, int row, int kt)
+// Loads WPT consecutive plane words per plane of one row of one K tile (tiled layout).
+template <int BITS, int WPT>
+__device__ __forceinline__ void load_tile_words(uint32_t (&dst)[BITS][WPT], const uint32_t *tiled, int rows, int row,
+                                                int kt, int first_word)
 {
-    const uint4 *p = reinterpret_cast<const uint4 *>(tiled) + ((size_t)kt * rows + row) * BITS;
+    const uint32_t *p = tiled + (((size_t)kt * rows + row) * BITS) * 4 + first_word;
 #pragma unroll
-    for (int b = 0; b < BITS; ++b)
-        dst[b] = p[b];
+    for (int b = 0; b < BITS; ++b) {
+        if (WPT == 4) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(p + 4 * b);
+            dst[b][0] = v.x; dst[b][1 % WPT] = v.y; dst[b][2 % WPT] = v.z; dst[b][3 % WPT] = v.w;
+        } else if (WPT == 2) {
+            const uint2 v = *reinterpret_cast<const uint2 *>(p + 4 * b);
+            dst[b][0] = v.x; dst[b][1 % WPT] = v.y;
+        } else {
+            dst[b][0] = p[4 * b];
+        }
+    }
 }
 
-__device__ __forceinline__ uint32_t comp_t(const uint4 &v, int i)
-{
-    return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
-}
-
-// Expands the 4 word-sets of one row (128 K elements) and writes 128 int8 to LDS.
-template <int BITS, Int8Mode MODE, bool SUM>
-__device__ __forceinline__ void expand_row_to_lds(const uint4 (&raw)[BITS], unsigned char *lds_row, int &value_sum)
+// Expands WPT word-sets (32 K elements each) of one row and writes the int8 values to LDS.
+template <int BITS, int WPT, Int8Mode MODE, bool SUM>
+__device__ __forceinline__ void expand_words_to_lds(const uint32_t (&raw)[BITS][WPT], unsigned char *lds, int &value_sum)
 {
 #pragma unroll
-    for (int ws = 0; ws < 4; ++ws) {
+    for (int ws = 0; ws < WPT; ++ws) {
         uint32_t w[BITS], o[8];
 #pragma unroll
         for (int b = 0; b < BITS; ++b)
-            w[b] = comp_t(raw[b], ws);
+            w[b] = raw[b][ws];
         if (SUM)
             value_sum += planes_value_sum<BITS>(w);
         planes_to_int8<BITS, MODE>(w, o);
-        uint4 *dst = reinterpret_cast<uint4 *>(lds_row + ws * 32);
+        uint4 *dst = reinterpret_cast<uint4 *>(lds + ws * 32);
         dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
         dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
     }
@@ -77,15 +82,17 @@ __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const u
                                                         int m_blocks, int n_blocks_per_xcd)
 {
     constexpr int BM = 64 * TM, BN = 64 * TN;
-    constexpr int UNITS = BM + BN;                 // rows expanded per K tile
-    constexpr bool SPLIT = UNITS <= 256;           // each thread expands one row: A rows first, then B rows
-    constexpr int NA = SPLIT ? 1 : (BM + 255) / 256; // else every thread expands NA rows of A and NB of B
-    constexpr int NB = SPLIT ? 1 : (BN + 255) / 256;
+    // every thread expands WA word-sets of one activation row and WB word-sets of one weight row
+    // per K tile (a row has 4 word-sets): uniform work, no divergence
+    constexpr int WA = BM / 64, WB = BN / 64;
+    constexpr int TPRA = 4 / WA, TPRB = 4 / WB; // threads per row
+    static_assert(WA == 1 || WA == 2 || WA == 4, "BM in {64, 128, 256}");
+    static_assert(WB == 1 || WB == 2 || WB == 4, "BN in {64, 128, 256}");
     constexpr Int8Mode XMODE = Int8ModeOf<Q, SIGNED>::value;
     constexpr Int8Mode WMODE = Int8ModeOf<P, SIGNED>::value;
     constexpr bool NEED_SX = WMODE == kFlip; // see abq_gemm_mfma.hip
     constexpr bool NEED_SW = XMODE == kFlip;
-    constexpr int BUF_BYTES = UNITS * kLdsRow;
+    constexpr int BUF_BYTES = (BM + BN) * kLdsRow;
 
     extern __shared__ __align__(16) unsigned char smem[];
     // [2][BM + BN][144] expanded rows, then row sums [BM + BN]
@@ -107,58 +114,16 @@ __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const u
     if (n0 >= N)
         return; // uniform over the workgroup, before any barrier
 
-    // the rows this thread expands (fixed for the whole K loop; activity is uniform per wave)
-    bool act_a[NA], act_b[NB];
-    int la[NA], lb[NB];   // row within the tile
-    int ga[NA], gb[NB];   // row in the operand (clamped at the edge, dropped at the store)
-#pragma unroll
-    for (int u = 0; u < NA; ++u) {
-        la[u] = tid + u * 256;
-        act_a[u] = la[u] < BM;
-        ga[u] = min(m0 + la[u], M - 1);
-    }
-#pragma unroll
-    for (int u = 0; u < NB; ++u) {
-        lb[u] = SPLIT ? tid - BM : tid + u * 256;
-        act_b[u] = lb[u] >= 0 && lb[u] < BN;
-        gb[u] = min(n0 + max(lb[u], 0), N - 1);
-    }
+    // the words this thread expands (fixed for the whole K loop); rows past the edge are clamped
+    // for loading and dropped at the store
+    const int la = tid / TPRA, fa = (tid % TPRA) * WA; // tile row, first word-set
+    const int lb = tid / TPRB, fb = (tid % TPRB) * WB;
+    const int ga = min(m0 + la, M - 1), gb = min(n0 + lb, N - 1);
+    unsigned char *lds_a = smem + la * kLdsRow + fa * 32;
+    unsigned char *lds_b = smem + (BM + lb) * kLdsRow + fb * 32;
 
-    uint4 rawx[2][NA][Q], raww[2][NB][P]; // plane words of the next two K tiles
-    int sum_a[NA], sum_b[NB];
-#pragma unroll
-    for (int u = 0; u < NA; ++u)
-        sum_a[u] = 0;
-#pragma unroll
-    for (int u = 0; u < NB; ++u)
-        sum_b[u] = 0;
-
-    // register slots are named at compile time (S0 / S1) so that the arrays stay in registers
-    auto load_tile = [&](int kt, auto slot_c) __attribute__((always_inline)) {
-        constexpr int slot_ = decltype(slot_c)::value;
-        if (kt < ktiles) {
-#pragma unroll
-            for (int u = 0; u < NA; ++u)
-                if (act_a[u])
-                    load_tile_row<Q>(rawx[slot_][u], xt, M, ga[u], kt);
-#pragma unroll
-            for (int u = 0; u < NB; ++u)
-                if (act_b[u])
-                    load_tile_row<P>(raww[slot_][u], wt, N, gb[u], kt);
-        }
-    };
-    auto expand_tile = [&](auto slot_c, int buf) __attribute__((always_inline)) {
-        constexpr int slot_ = decltype(slot_c)::value;
-        unsigned char *base = smem + buf * BUF_BYTES;
-#pragma unroll
-        for (int u = 0; u < NA; ++u)
-            if (act_a[u])
-                expand_row_to_lds<Q, XMODE, NEED_SX>(rawx[slot_][u], base + la[u] * kLdsRow, sum_a[u]);
-#pragma unroll
-        for (int u = 0; u < NB; ++u)
-            if (act_b[u])
-                expand_row_to_lds<P, WMODE, NEED_SW>(raww[slot_][u], base + (BM + lb[u]) * kLdsRow, sum_b[u]);
-    };
+    uint32_t rx0[Q][WA], rx1[Q][WA], rw0[P][WB], rw1[P][WB]; // plane words of the next two K tiles
+    int sum_a = 0, sum_b = 0;
 
     v16i acc[TM][TN];
 #pragma unroll
@@ -169,57 +134,64 @@ __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const u
             for (int e = 0; e < 16; ++e)
                 acc[i][j][e] = 0;
 
-    const std::integral_constant<int, 0> S0;
-    const std::integral_constant<int, 1> S1;
-    load_tile(0, S0);
-    load_tile(1, S1);
-    expand_tile(S0, 0);
+#define ABQ_LOAD_TILE(KT, RX, RW)                                   \
+    if ((KT) < ktiles) {                                            \
+        load_tile_words<Q, WA>(RX, xt, M, ga, (KT), fa);            \
+        load_tile_words<P, WB>(RW, wt, N, gb, (KT), fb);            \
+    }
+#define ABQ_EXPAND_TILE(RX, RW, BUF)                                                                  \
+    expand_words_to_lds<Q, WA, XMODE, NEED_SX>(RX, lds_a + (BUF) * BUF_BYTES, sum_a);                 \
+    expand_words_to_lds<P, WB, WMODE, NEED_SW>(RW, lds_b + (BUF) * BUF_BYTES, sum_b);
+
+    ABQ_LOAD_TILE(0, rx0, rw0)
+    ABQ_LOAD_TILE(1, rx1, rw1)
+    if (NEED_SX || NEED_SW)
+        for (int i = tid; i < BM + BN; i += 256)
+            rowsum[i] = 0;
+    ABQ_EXPAND_TILE(rx0, rw0, 0)
     __syncthreads();
 
     const unsigned char *a_lane = smem + (wm * 32 * TM + r) * kLdsRow + g * 16;
     const unsigned char *b_lane = smem + (BM + wn * 32 * TN + r) * kLdsRow + g * 16;
 
-    // One K tile: MFMAs on LDS buffer `buf` (tile kt), loads of tile kt+2 into the register slot
+    // One K tile: MFMAs on LDS buffer BUF (tile kt), loads of tile kt+2 into the register slot
     // tile kt used, expansion of tile kt+1 (other register slot) into the other LDS buffer.
-    auto k_tile = [&](int kt, auto cur_c, auto nxt_c) __attribute__((always_inline)) {
-        constexpr int buf = decltype(cur_c)::value;
-        load_tile(kt + 2, cur_c);
-        const unsigned char *ab = a_lane + buf * BUF_BYTES;
-        const unsigned char *bb = b_lane + buf * BUF_BYTES;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            v4i av[TM], bv[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                av[i] = *reinterpret_cast<const v4i *>(ab + i * 32 * kLdsRow + ks * 32);
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                bv[j] = *reinterpret_cast<const v4i *>(bb + j * 32 * kLdsRow + ks * 32);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < ktiles)
-            expand_tile(nxt_c, buf ^ 1);
-        __syncthreads();
-    };
-    for (int kt = 0; kt < ktiles; kt += 2) {
-        k_tile(kt, S0, S1);
-        if (kt + 1 < ktiles)
-            k_tile(kt + 1, S1, S0);
+#define ABQ_K_TILE(KT, BUF, RXC, RWC, RXN, RWN)                                                        \
+    {                                                                                                  \
+        ABQ_LOAD_TILE((KT) + 2, RXC, RWC)                                                              \
+        const unsigned char *ab = a_lane + (BUF) * BUF_BYTES;                                          \
+        const unsigned char *bb = b_lane + (BUF) * BUF_BYTES;                                          \
+        _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                               \
+        {                                                                                              \
+            v4i av[TM], bv[TN];                                                                        \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i)                                             \
+                av[i] = *reinterpret_cast<const v4i *>(ab + i * 32 * kLdsRow + ks * 32);               \
+            _Pragma("unroll") for (int j = 0; j < TN; ++j)                                             \
+                bv[j] = *reinterpret_cast<const v4i *>(bb + j * 32 * kLdsRow + ks * 32);               \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i)                                             \
+                _Pragma("unroll") for (int j = 0; j < TN; ++j)                                         \
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j], acc[i][j], 0, 0, 0); \
+        }                                                                                              \
+        if ((KT) + 1 < ktiles) {                                                                       \
+            ABQ_EXPAND_TILE(RXN, RWN, (BUF) ^ 1)                                                       \
+        }                                                                                              \
+        __syncthreads();                                                                               \
     }
 
+    for (int kt = 0; kt < ktiles; kt += 2) {
+        ABQ_K_TILE(kt, 0, rx0, rw0, rx1, rw1)
+        if (kt + 1 < ktiles)
+            ABQ_K_TILE(kt + 1, 1, rx1, rw1, rx0, rw0)
+    }
+#undef ABQ_K_TILE
+#undef ABQ_EXPAND_TILE
+#undef ABQ_LOAD_TILE
+
     if (NEED_SX || NEED_SW) {
-#pragma unroll
-        for (int u = 0; u < NA; ++u)
-            if (act_a[u])
-                rowsum[la[u]] = sum_a[u];
-#pragma unroll
-        for (int u = 0; u < NB; ++u)
-            if (act_b[u])
-                rowsum[BM + lb[u]] = sum_b[u];
+        if (NEED_SX)
+            atomicAdd(&rowsum[la], sum_a);
+        if (NEED_SW)
+            atomicAdd(&rowsum[BM + lb], sum_b);
         __syncthreads();
     }
 
@@ -246,7 +218,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const u
                         v -= 16384u * (unsigned)k_fed;
                 }
                 if (m < M && n < N)
-                    store_result(a, m, n, (int)v);
+                    store_result_compact(a, m, n, (int)v);
             }
         }
     }

@@ -70,4 +70,19 @@ __device__ __forceinline__ void store_result(const GemmArgs &a, int m, int n, in
     }
 }
 
+// Out-of-line copy for kernels whose epilogue stores hundreds of elements per lane: keeps the
+// unrolled epilogue small (the int32 store is inlined, the fp16 variants are a call).
+__device__ __attribute__((noinline)) static void store_result_call(const GemmArgs &a, int m, int n, int acc)
+{
+    store_result(a, m, n, acc);
+}
+
+__device__ __forceinline__ void store_result_compact(const GemmArgs &a, int m, int n, int acc)
+{
+    if (a.out_kind == 0)
+        reinterpret_cast<int *>(a.D)[(size_t)m * a.N + n] = acc;
+    else
+        store_result_call(a, m, n, acc);
+}
+
 } // namespace abq

@@ -207,9 +207,11 @@ def main():
         for (q, p, signed) in [(4, 4, True), (4, 4, False), (8, 8, True), (8, 8, False)]:
             for (N, K) in SHAPES:
                 wpl = random_planes(torch, (p, N, K // 32))
+                wtl = abq.relayout_planes(wpl)  # weights prepared once in the K-tiled layout
                 for M in (512, 2048):
                     xpl = random_planes(torch, (q, M, K // 32))
-                    gm = abq.Gemm(xpl, wpl, signed)
+                    ws = torch.empty(xpl.numel() * 4, dtype=torch.uint8, device="cuda")
+                    gm = abq.Gemm(xpl, wtl, signed, w_tiled=True, workspace=ws)  # activations converted per call
                     gm.run()
                     torch.cuda.synchronize()
                     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -223,8 +225,8 @@ def main():
                     prefill.append(dict(w_bits=p, x_bits=q, signed=signed, M=M, N=N, K=K, us=round(us, 1),
                                         tops=round(tops, 2), mfma_frac=round(tops / INT8_MFMA_PEAK_TOPS, 4),
                                         kernel="%s:%s" % (gm.strategy, gm.config_name)))
-                    del gm, xpl
-                del wpl
+                    del gm, xpl, ws
+                del wpl, wtl
         extra["prefill"] = prefill
         for r in prefill:
             log("prefill W%dA%d %s M=%d N=%d K=%d  %.1f us  %.1f TOPS (%.1f%% of int8 MFMA peak)"
