@@ -17,6 +17,7 @@ STATUS_NAMES = {
     0: "ABQ_OK", 1: "ABQ_ERR_INVALID_ARG", 2: "ABQ_ERR_BAD_K", 3: "ABQ_ERR_UNSUPPORTED",
     4: "ABQ_ERR_NOT_INITIALIZED", 5: "ABQ_ERR_LAUNCH", 6: "ABQ_ERR_NO_DEVICE", 7: "ABQ_ERR_TOO_LARGE",
 }
+globals().update({name: code for code, name in STATUS_NAMES.items()})
 OUT_I32, OUT_F16_TENSOR, OUT_F16_SCALED, OUT_F16_TENSOR_F32SCALE = 0, 1, 2, 3
 STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC, STRATEGY_DECODE, STRATEGY_TILED = range(7)
 STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic", "decode", "tiled"]
@@ -31,6 +32,7 @@ EXPORTED = [
     "abq_gemm_init", "abq_gemm_set_scales", "abq_gemm_exec", "abq_gemm_launch",
     "abq_planes_bytes", "abq_relayout_planes", "abq_gemm_set_operand_layout", "abq_gemm_workspace_bytes",
     "abq_gemm_set_workspace",
+    "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16",
 ]
 
 
@@ -65,6 +67,8 @@ class GemmState(ctypes.Structure):
         ("reserved", ctypes.c_int * 5),
         ("x_layout", ctypes.c_int), ("w_layout", ctypes.c_int), ("auto_chosen", ctypes.c_int),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("x_zero", ctypes.c_void_p), ("w_zero", ctypes.c_void_p),
+        ("x_group_sums", ctypes.c_void_p), ("w_zero_term", ctypes.c_void_p),
     ]
 
 
@@ -110,6 +114,9 @@ def lib():
         L.abq_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GemmState)]
         L.abq_gemm_workspace_bytes.restype = ctypes.c_size_t
         L.abq_gemm_set_workspace.argtypes = [ctypes.POINTER(GemmState), vp, ctypes.c_size_t]
+        L.abq_gemm_set_zero_points.argtypes = [ctypes.POINTER(GemmState), vp, vp, vp, vp]
+        L.abq_weight_zero_term.argtypes = [vp, ci, ci, ci, ci, vp, vp, ci, vp, vp]
+        L.abq_quant_pack_f16.argtypes = [vp, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, vp]
         _lib = L
     return _lib
 
@@ -201,6 +208,38 @@ def relayout_planes(planes, out=None, stream=None):
     return out
 
 
+def quant_pack_f16(x, bits, symmetric=True, tiled=False, group_size=0, stream=None):
+    """Per-token dynamic quantisation + packing of fp16 activations [rows, k].
+
+    Returns (planes, scale[rows], zero[rows] or None, group_sums[rows, k/group_size] or None);
+    planes hold signed codes, [bits, rows, k/32] or K-tiled [k/128, rows, bits, 4]."""
+    import torch
+    assert x.dtype == torch.float16 and x.is_cuda and x.is_contiguous()
+    rows, k = x.shape
+    shape = (k // 128, rows, bits, 4) if tiled else (bits, rows, k // 32)
+    planes = torch.empty(shape, dtype=torch.int32, device=x.device)
+    scale = torch.empty(rows, dtype=torch.float32, device=x.device)
+    zero = None if symmetric else torch.empty(rows, dtype=torch.float32, device=x.device)
+    sums = torch.empty((rows, k // group_size), dtype=torch.int32, device=x.device) if group_size else None
+    _check(lib().abq_quant_pack_f16(x.data_ptr(), rows, k, bits, int(bool(symmetric)), int(bool(tiled)),
+                                    planes.data_ptr(), scale.data_ptr(),
+                                    zero.data_ptr() if zero is not None else None,
+                                    sums.data_ptr() if sums is not None else None, group_size,
+                                    _stream_ptr(stream)), "abq_quant_pack_f16")
+    return planes, scale, zero, sums
+
+
+def weight_zero_term(w_planes, signed, w_scale, w_zero, group_size, stream=None):
+    """[N] rank-one term of the activation zero-point correction, from reference-layout planes."""
+    import torch
+    bits, n, kw = w_planes.shape
+    out = torch.empty(n, dtype=torch.float32, device=w_planes.device)
+    _check(lib().abq_weight_zero_term(w_planes.data_ptr(), n, kw * 32, bits, int(bool(signed)), w_scale.data_ptr(),
+                                      w_zero.data_ptr() if w_zero is not None else None, group_size,
+                                      out.data_ptr(), _stream_ptr(stream)), "abq_weight_zero_term")
+    return out
+
+
 class Gemm:
     """One initialised GEMM (the role of AqBMMAOpState + InitFn/ExecFn in the reference).
 
@@ -208,7 +247,8 @@ class Gemm:
     say they were converted with relayout_planes ([k/128, rows, bits, 4])."""
 
     def __init__(self, x_planes, w_planes, signed, out=None, cfg=None, out_kind=OUT_I32, c_scale=None,
-                 x_scale=None, w_scale=None, group_size=0, x_tiled=False, w_tiled=False, workspace=None):
+                 x_scale=None, w_scale=None, group_size=0, x_tiled=False, w_tiled=False, workspace=None,
+                 x_zero=None, w_zero=None, x_group_sums=None, w_zero_term=None):
         import torch
         if x_tiled:
             kt, M, q, _ = x_planes.shape
@@ -237,6 +277,11 @@ class Gemm:
         if out_kind == OUT_F16_SCALED:
             _check(lib().abq_gemm_set_scales(ctypes.byref(self.state), x_scale.data_ptr(), w_scale.data_ptr(),
                                              group_size), "abq_gemm_set_scales")
+        self.zero_operands = (x_zero, w_zero, x_group_sums, w_zero_term)
+        if any(t is not None for t in self.zero_operands):
+            _check(lib().abq_gemm_set_zero_points(ctypes.byref(self.state),
+                                                  *[t.data_ptr() if t is not None else None
+                                                    for t in self.zero_operands]), "abq_gemm_set_zero_points")
         if x_tiled or w_tiled:
             _check(lib().abq_gemm_set_operand_layout(ctypes.byref(self.state), int(x_tiled), int(w_tiled)),
                    "abq_gemm_set_operand_layout")

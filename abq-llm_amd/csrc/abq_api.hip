@@ -15,6 +15,10 @@ hipError_t launch_pack_i32(const int32_t *, uint32_t *, int, int, int, hipStream
 hipError_t launch_pack_f16(const void *, const float *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
+hipError_t launch_quant_pack_rows(const void *, uint32_t *, float *, float *, int *, int, int, int, int, int, int,
+                                  hipStream_t);
+hipError_t launch_weight_zero_term(const uint32_t *, int, int, int, int, const float *, const float *, int, float *,
+                                   hipStream_t);
 
 // (x_bits, w_bits) pairs with specialised kernels: the twelve of the reference library
 // (engine/mma_any/aq_bmma_impl/aq_bmma_w{2a2,...,8a8}.h).
@@ -26,7 +30,8 @@ hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, h
     void abq_mfma_register_##Q##_##P(KernelTable *);  \
     void abq_bcnt_register_##Q##_##P(KernelTable *);  \
     void abq_decode_register_##Q##_##P(KernelTable *); \
-    void abq_tiled_register_##Q##_##P(KernelTable *);
+    void abq_tiled_register_##Q##_##P(KernelTable *);  \
+    void abq_tiled_grouped_register_##Q##_##P(KernelTable *);
 ABQ_FOR_EACH_COMBO(ABQ_DECL)
 #undef ABQ_DECL
 
@@ -35,6 +40,7 @@ struct Registry {
     KernelTable bcnt[2 * ABQ_NUM_COMBOS];
     KernelTable decode[2 * ABQ_NUM_COMBOS];
     KernelTable tiled[2 * ABQ_NUM_COMBOS];
+    KernelTable tiled_grouped[2 * ABQ_NUM_COMBOS];
     Registry()
     {
         int i = 0;
@@ -43,6 +49,7 @@ struct Registry {
     abq_bcnt_register_##Q##_##P(&bcnt[i]);             \
     abq_decode_register_##Q##_##P(&decode[i]);         \
     abq_tiled_register_##Q##_##P(&tiled[i]);           \
+    abq_tiled_grouped_register_##Q##_##P(&tiled_grouped[i]); \
     i += 2;
         ABQ_FOR_EACH_COMBO(ABQ_REG)
 #undef ABQ_REG
@@ -563,12 +570,94 @@ abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, cons
         return ABQ_ERR_NOT_INITIALIZED;
     if (!x_scale || !w_scale)
         return ABQ_ERR_INVALID_ARG;
-    if (group_size != 0) // grouped scales need a K-blocked main loop; not built yet
-        return ABQ_ERR_UNSUPPORTED;
+    if (group_size != 0) {
+        // w_scale is [N][K / group_size]: only the tiled kernel folds scales inside the K loop
+        const abq_tile_config &c = state->cfg;
+        if (group_size != 64 && group_size != 128)
+            return ABQ_ERR_UNSUPPORTED;
+        if (state->out_kind != ABQ_OUT_F16_SCALED)
+            return ABQ_ERR_INVALID_ARG;
+        if (!c.is_signed && (c.x_bits == 8 || c.w_bits == 8))
+            return ABQ_ERR_UNSUPPORTED;
+        if (state->strategy != ABQ_STRATEGY_TILED) {
+            if (!state->auto_chosen)
+                return ABQ_ERR_UNSUPPORTED;
+            const abq_status rc = switch_to_tiled(state);
+            if (rc != ABQ_OK)
+                return rc;
+        }
+        const KernelTable *tg = find_table(registry().tiled_grouped, c.x_bits, c.w_bits, c.is_signed);
+        if (!tg)
+            return ABQ_ERR_UNSUPPORTED;
+        int pick = -1;
+        for (int i = 0; i < tg->count; ++i)
+            if (tg->entries[i].mi * tg->entries[i].tm * tg->entries[i].wm == c.block_m &&
+                tg->entries[i].mi * tg->entries[i].tn * tg->entries[i].wn == c.block_n)
+                pick = i;
+        if (pick < 0) {
+            // no group-scale build of this tile: fall back to the smallest one when the library chose
+            if (!state->auto_chosen)
+                return ABQ_ERR_UNSUPPORTED;
+            pick = tg->count - 1;
+            entry_to_config(tg->entries[pick], ABQ_STRATEGY_TILED, c.x_bits, c.w_bits, c.is_signed, 0, &state->cfg);
+        }
+        state->variant = pick;
+    } else if (state->group_size != 0) {
+        return ABQ_ERR_INVALID_ARG; // a state switched to group scales stays there
+    }
     state->x_scale = x_scale;
     state->w_scale = w_scale;
     state->group_size = group_size;
     return ABQ_OK;
+}
+
+abq_status abq_gemm_set_zero_points(abq_gemm_state *state, const float *x_zero, const float *w_zero,
+                                    const int32_t *x_group_sums, const float *w_zero_term)
+{
+    if (!state || !state->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    if (state->group_size == 0) // only the group-scale kernel carries the correction terms
+        return ABQ_ERR_UNSUPPORTED;
+    if ((w_zero && !x_group_sums) || (x_zero && !w_zero_term))
+        return ABQ_ERR_INVALID_ARG;
+    state->x_zero = x_zero;
+    state->w_zero = w_zero;
+    state->x_group_sums = x_group_sums;
+    state->w_zero_term = w_zero_term;
+    return ABQ_OK;
+}
+
+abq_status abq_weight_zero_term(const uint32_t *w_planes, int n, int k, int bits, int is_signed,
+                                const float *w_scale, const float *w_zero, int group_size,
+                                float *w_zero_term, void *stream)
+{
+    if (!w_planes || !w_scale || !w_zero_term || n <= 0 || bits < 1 || bits > 8)
+        return ABQ_ERR_INVALID_ARG;
+    if (k < 128 || k % 128 != 0)
+        return ABQ_ERR_BAD_K;
+    if (group_size != 64 && group_size != 128)
+        return ABQ_ERR_UNSUPPORTED;
+    return hip_status(launch_weight_zero_term(w_planes, n, k, bits, is_signed, w_scale, w_zero, group_size,
+                                              w_zero_term, (hipStream_t)stream));
+}
+
+abq_status abq_quant_pack_f16(const void *x_f16, int rows, int k, int bits, int symmetric, int layout,
+                              uint32_t *planes, float *scale, float *zero, int32_t *group_sums,
+                              int group_size, void *stream)
+{
+    if (!x_f16 || !planes || !scale || rows <= 0 || bits < 2 || bits > 8)
+        return ABQ_ERR_INVALID_ARG;
+    if (!symmetric && !zero)
+        return ABQ_ERR_INVALID_ARG;
+    if (layout != ABQ_LAYOUT_PLANES && layout != ABQ_LAYOUT_TILED)
+        return ABQ_ERR_INVALID_ARG;
+    if (k < 128 || k % 128 != 0)
+        return ABQ_ERR_BAD_K;
+    if (group_sums && group_size != 64 && group_size != 128)
+        return ABQ_ERR_UNSUPPORTED;
+    return hip_status(launch_quant_pack_rows(x_f16, planes, scale, zero, group_sums, rows, k, bits, symmetric ? 1 : 0,
+                                             group_sums ? group_size : 128, layout == ABQ_LAYOUT_TILED,
+                                             (hipStream_t)stream));
 }
 
 abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
@@ -591,6 +680,10 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     a.out_kind = st->out_kind;
     a.group_size = st->group_size;
     a.lpr_log2 = st->reserved[0];
+    a.w_zero = st->w_zero;
+    a.x_zero = st->x_zero;
+    a.x_group_sums = st->x_group_sums;
+    a.w_zero_term = st->w_zero_term;
     const Registry &reg = registry();
     const abq_tile_config &c = st->cfg;
     hipError_t e;
@@ -615,7 +708,7 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
                 return hip_status(e);
             a.W = reinterpret_cast<const uint32_t *>(ws + xb);
         }
-        const KernelTable *t = find_table(reg.tiled, c.x_bits, c.w_bits, c.is_signed);
+        const KernelTable *t = find_table(st->group_size ? reg.tiled_grouped : reg.tiled, c.x_bits, c.w_bits, c.is_signed);
         if (!t || st->variant < 0 || st->variant >= t->count)
             return ABQ_ERR_NOT_INITIALIZED;
         e = t->entries[st->variant].launch(a, (hipStream_t)stream);

@@ -77,7 +77,12 @@ __device__ __forceinline__ void expand_words_to_lds(const uint32_t (&raw)[BITS][
     }
 }
 
-template <int Q, int P, bool SIGNED, int TM, int TN>
+// GROUPED: group-wise weight scales (group size 64 or 128 along K, w_scale[N][K/group]) and
+// per-token activation scales, fp16 output.  The int32 accumulators then cover one scale group
+// and are folded into fp32 accumulators with the group's scale at every group boundary
+// (semantics: algorithm/quantize/quantizer.py:111-179 of the reference, scales per row of W
+// after reshaping to [-1, group_size]).  Not available for 8-bit unsigned operands.
+template <int Q, int P, bool SIGNED, int TM, int TN, bool GROUPED>
 __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt,
                                                         int m_blocks, int n_blocks_per_xcd)
 {
@@ -126,13 +131,26 @@ __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const u
     int sum_a = 0, sum_b = 0;
 
     v16i acc[TM][TN];
+    float facc[GROUPED ? TM : 1][GROUPED ? TN : 1][16];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e)
+            for (int e = 0; e < 16; ++e) {
                 acc[i][j][e] = 0;
+                if (GROUPED)
+                    facc[i][j][e] = 0.f;
+            }
+    // GROUPED: this lane's output columns and where their scales live.  The signed route feeds
+    // value * 2^(8-bits) to the MFMA: the exact power of two that undoes it rides on the scale.
+    const float unshift = SIGNED ? 1.0f / (float)(1 << (16 - Q - P)) : 1.0f;
+    const bool g64 = GROUPED && a.group_size == 64;
+    const int groups = GROUPED ? a.K / a.group_size : 0;
+    const float *wsc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+        wsc[j] = GROUPED ? a.w_scale + (size_t)min(n0 + wn * 32 * TN + j * 32 + r, N - 1) * groups : nullptr;
 
 #define ABQ_LOAD_TILE(KT, RX, RW)                                   \
     if ((KT) < ktiles) {                                            \
@@ -159,6 +177,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const u
 #define ABQ_K_TILE(KT, BUF, RXC, RWC, RXN, RWN)                                                        \
     {                                                                                                  \
         ABQ_LOAD_TILE((KT) + 2, RXC, RWC)                                                              \
+        float gsc[TN][2];                                                                              \
+        if (GROUPED) {                                                                                 \
+            _Pragma("unroll") for (int j = 0; j < TN; ++j)                                             \
+            {                                                                                          \
+                gsc[j][0] = (g64 ? wsc[j][2 * (KT)] : wsc[j][(KT)]) * unshift;                         \
+                gsc[j][1] = g64 ? wsc[j][2 * (KT) + 1] * unshift : gsc[j][0];                          \
+            }                                                                                          \
+        }                                                                                              \
         const unsigned char *ab = a_lane + (BUF) * BUF_BYTES;                                          \
         const unsigned char *bb = b_lane + (BUF) * BUF_BYTES;                                          \
         _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                               \
@@ -171,6 +197,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const u
             _Pragma("unroll") for (int i = 0; i < TM; ++i)                                             \
                 _Pragma("unroll") for (int j = 0; j < TN; ++j)                                         \
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j], acc[i][j], 0, 0, 0); \
+            if (GROUPED && (ks == 3 || (ks == 1 && g64))) {                                            \
+                _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
+                    _Pragma("unroll") for (int j = 0; j < TN; ++j)                                     \
+                        _Pragma("unroll") for (int e = 0; e < 16; ++e)                                 \
+                        {                                                                              \
+                            facc[i][j][e] += (float)acc[i][j][e] * gsc[j][ks >> 1];                    \
+                            acc[i][j][e] = 0;                                                          \
+                        }                                                                              \
+            }                                                                                          \
         }                                                                                              \
         if ((KT) + 1 < ktiles) {                                                                       \
             ABQ_EXPAND_TILE(RXN, RWN, (BUF) ^ 1)                                                       \
@@ -195,6 +230,48 @@ __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const u
         __syncthreads();
     }
 
+    if (GROUPED && a.w_zero) {
+        // Weight zero points: out -= sum_g w_scale[n][g] * w_zero[n][g] * (sum of the activation codes
+        // of row m in group g).  The two factors are staged through LDS 32 groups at a time.
+        constexpr int GC = 32;
+        float *zs_x = reinterpret_cast<float *>(smem); // [GC][BM]
+        float *zs_w = zs_x + GC * BM;                  // [GC][BN]
+        static_assert(GC * (BM + BN) * 4 <= 2 * BUF_BYTES, "staging fits the tile buffers");
+        for (int g0 = 0; g0 < groups; g0 += GC) {
+            __syncthreads();
+            for (int u = tid; u < GC * BM; u += 256) {
+                const int rr = u / GC, gl = u % GC;
+                const int m = min(m0 + rr, M - 1);
+                zs_x[gl * BM + rr] = g0 + gl < groups ? (float)a.x_group_sums[(size_t)m * groups + g0 + gl] : 0.f;
+            }
+            for (int u = tid; u < GC * BN; u += 256) {
+                const int rr = u / GC, gl = u % GC;
+                const size_t idx = (size_t)min(n0 + rr, N - 1) * groups + g0 + gl;
+                zs_w[gl * BN + rr] = g0 + gl < groups ? a.w_scale[idx] * a.w_zero[idx] : 0.f;
+            }
+            __syncthreads();
+            for (int gl = 0; gl < GC; ++gl) {
+                float wz[TN];
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    wz[j] = zs_w[gl * BN + wn * 32 * TN + j * 32 + r];
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4) {
+                        const float4 sx4 = *reinterpret_cast<const float4 *>(&zs_x[gl * BM + wm * 32 * TM + i * 32 + 8 * e4 + 4 * g]);
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) {
+                            facc[i][j][4 * e4 + 0] -= wz[j] * sx4.x;
+                            facc[i][j][4 * e4 + 1] -= wz[j] * sx4.y;
+                            facc[i][j][4 * e4 + 2] -= wz[j] * sx4.z;
+                            facc[i][j][4 * e4 + 3] -= wz[j] * sx4.w;
+                        }
+                    }
+            }
+        }
+    }
+
     const int k_fed = ktiles * kTileK;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -206,6 +283,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const u
             for (int e = 0; e < 16; ++e) {
                 const int ml = wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4);
                 const int m = m0 + ml;
+                if (GROUPED) {
+                    if (m < M && n < N) {
+                        float v = facc[i][j][e];
+                        if (a.x_zero) // activation zero points: a rank-one term
+                            v -= a.x_zero[m] * a.w_zero_term[n];
+                        reinterpret_cast<_Float16 *>(a.D)[(size_t)m * N + n] = (_Float16)(v * a.x_scale[m]);
+                    }
+                    continue;
+                }
                 unsigned v = (unsigned)acc[i][j][e];
                 if (SIGNED) {
                     v = (unsigned)((int)v >> (16 - Q - P));
@@ -224,31 +310,40 @@ __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const u
     }
 }
 
-template <int Q, int P, bool SIGNED, int TM, int TN>
+template <int Q, int P, bool SIGNED, int TM, int TN, bool GROUPED>
 static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 {
     constexpr int BM = 64 * TM, BN = 64 * TN;
+    if (GROUPED && (Int8ModeOf<Q, SIGNED>::value == kFlip || Int8ModeOf<P, SIGNED>::value == kFlip))
+        return hipErrorInvalidValue; // group scales with 8-bit unsigned operands: not built
     const int m_blocks = (a.M + BM - 1) / BM, n_blocks = (a.N + BN - 1) / BN;
     const int npx = (n_blocks + 7) / 8;
     const size_t lds = 2 * (size_t)(BM + BN) * kLdsRow + (BM + BN) * sizeof(int);
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_tiled<Q, P, SIGNED, TM, TN>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void *>(&gemm_mfma_tiled<Q, P, SIGNED, TM, TN, GROUPED>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess)
         return attr;
     const dim3 grid(8 * npx * m_blocks);
-    hipLaunchKernelGGL((gemm_mfma_tiled<Q, P, SIGNED, TM, TN>), grid, dim3(256), lds, stream, a, a.X, a.W, m_blocks, npx);
+    hipLaunchKernelGGL((gemm_mfma_tiled<Q, P, SIGNED, TM, TN, GROUPED>), grid, dim3(256), lds, stream, a, a.X, a.W, m_blocks, npx);
     return hipGetLastError();
 }
 
 // Native tile space of this kernel: MFMA tiles per wave (TM, TN); nstage 4 marks the K-tiled
-// operand layout.
+// operand layout.  The group-scale variants sit in a table of their own and exist for the tiles
+// the default choice uses.
 #define ABQ_TILED_VARIANTS(V) V(4, 4) V(2, 4) V(2, 2) V(2, 1) V(1, 1)
+#define ABQ_GROUPED_VARIANTS(V) V(2, 2) V(1, 1)
 
-#define ABQ_ENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN> },
-#define ABQ_ENTRY_F(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN> },
+#define ABQ_ENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, false> },
+#define ABQ_ENTRY_F(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN, false> },
+#define ABQ_GENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, true> },
+#define ABQ_GENTRY_F(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN, true> },
 
 static const KernelEntry kSigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_T) };
 static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) };
+static const KernelEntry kSignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_T) };
+static const KernelEntry kUnsignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_F) };
 
 #define ABQ_CAT_(a, b, c, d) a##b##c##d
 #define ABQ_CAT(a, b, c, d) ABQ_CAT_(a, b, c, d)
@@ -257,6 +352,12 @@ void ABQ_CAT(abq_tiled_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)
 {
     out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSigned, (int)(sizeof(kSigned) / sizeof(kSigned[0])) };
     out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, kUnsigned, (int)(sizeof(kUnsigned) / sizeof(kUnsigned[0])) };
+}
+
+void ABQ_CAT(abq_tiled_grouped_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)
+{
+    out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSignedGrouped, (int)(sizeof(kSignedGrouped) / sizeof(kSignedGrouped[0])) };
+    out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, kUnsignedGrouped, (int)(sizeof(kUnsignedGrouped) / sizeof(kUnsignedGrouped[0])) };
 }
 
 } // namespace abq

@@ -20,6 +20,11 @@ struct GemmArgs {
     int out_kind;
     int group_size;
     int lpr_log2;    // popcount kernels: log2(lanes that share one weight row)
+    // zero points of the group-scale path (all optional)
+    const float *w_zero;       // [N][K/group_size], in units of weight codes
+    const float *x_zero;       // [M], in units of activation codes
+    const int *x_group_sums;   // [M][K/group_size] sums of activation codes (needed with w_zero)
+    const float *w_zero_term;  // [N] sum_g w_scale * (sum of weight codes - group_size * w_zero) (needed with x_zero)
 };
 
 typedef hipError_t (*GemmLauncher)(const GemmArgs &, hipStream_t);

@@ -144,6 +144,179 @@ hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int r
     return hipGetLastError();
 }
 
+// ---- per-token dynamic quantisation fused with packing ------------------------------------
+//
+// One workgroup per token row of fp16 activations [M][K]: min / max of the row, scale and zero
+// point as the reference's per_token_dynamic_calibration derives them
+// (algorithm/quantize/quantizer.py:149-179), integer codes as its fake_quant rounds and clamps
+// them (:120-123), then the bit planes of the codes.  Codes leave as signed two's complement:
+//   symmetric : scale = clamp(absmax / (2^(n-1)-1), 1e-5, 1e4), code = clamp(rint(x/scale), -2^(n-1), 2^(n-1)-1)
+//   asymmetric: scale = clamp((max-min) / (2^n-1), 1e-5, 1e4), zp = rint(clamp(-min/scale, -1e4, 1e4)),
+//               u = clamp(rint(x/scale) + zp, 0, 2^n-1); stored code = u - 2^(n-1), zero = zp - 2^(n-1)
+// so that x ~ scale * (code - zero) either way (zero = 0 when symmetric).  Arithmetic is fp32.
+// Optionally writes the sum of the codes over every group of group_size elements (the GEMM's
+// zero-point correction needs them).
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+template <bool TILED>
+__global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__restrict__ x, uint32_t *__restrict__ planes,
+                                                              float *__restrict__ scale_out, float *__restrict__ zero_out,
+                                                              int *__restrict__ group_sums, int M, int K, int bits,
+                                                              int symmetric, int group_size)
+{
+    __shared__ float red[2][4];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const int units = K / 8; // 8 halves per 16-byte load
+    const uint4 *xr = x + (size_t)row * units;
+
+    float mx = -INFINITY, mn = INFINITY;
+    for (int u = tid; u < units; u += 256) {
+        union {
+            uint4 q;
+            _Float16 h[8];
+        } raw;
+        raw.q = xr[u];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const float f = (float)raw.h[c];
+            mx = fmaxf(mx, f);
+            mn = fminf(mn, f);
+        }
+    }
+    mx = wave_max(mx);
+    mn = -wave_max(-mn);
+    if ((tid & 63) == 0) {
+        red[0][tid >> 6] = mx;
+        red[1][tid >> 6] = mn;
+    }
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+    mn = fminf(fminf(red[1][0], red[1][1]), fminf(red[1][2], red[1][3]));
+
+    const int half_range = 1 << (bits - 1);
+    float scale, zp;
+    int lo, hi;
+    if (symmetric) {
+        scale = fmaxf(fabsf(mx), fabsf(mn)) / (float)(half_range - 1);
+        scale = fminf(fmaxf(scale, 1e-5f), 1e4f);
+        zp = 0.f;
+        lo = -half_range;
+        hi = half_range - 1;
+    } else {
+        scale = (mx - mn) / (float)(2 * half_range - 1);
+        scale = fminf(fmaxf(scale, 1e-5f), 1e4f);
+        zp = rintf(fminf(fmaxf(-mn / scale, -1e4f), 1e4f));
+        lo = 0;
+        hi = 2 * half_range - 1;
+    }
+    if (tid == 0) {
+        scale_out[row] = scale;
+        if (zero_out)
+            zero_out[row] = symmetric ? 0.f : zp - (float)half_range;
+    }
+
+    const int KW = K / 32;
+    const int rounded = (units + 255) / 256 * 256;
+    const int lanes_per_group = group_size / 8;
+    for (int u = tid; u < rounded; u += 256) {
+        const bool active = u < units; // units is a multiple of 16: quads and groups are active as one
+        int v[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
+        int sum = 0;
+        if (active) {
+            union {
+                uint4 q;
+                _Float16 h[8];
+            } raw;
+            raw.q = xr[u];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                float r = rintf((float)raw.h[c] / scale) + zp;
+                r = fminf(fmaxf(r, (float)lo), (float)hi);
+                v[c] = (int)r - (symmetric ? 0 : half_range);
+                sum += v[c];
+            }
+        }
+        if (group_sums) {
+            for (int o = 1; o < lanes_per_group; o <<= 1)
+                sum += __shfl_xor(sum, o);
+            if (active && (u % lanes_per_group) == 0)
+                group_sums[(size_t)row * (K / group_size) + u / lanes_per_group] = sum;
+        }
+        const uint64_t bytes = eight_values_to_plane_bytes(v);
+        const int quad_lane = u & 3, w = u >> 2; // w: plane word within the row
+        for (int b = 0; b < bits; ++b) {
+            uint32_t word = (uint32_t)((bytes >> (8 * b)) & 0xFFu) << (24 - 8 * quad_lane);
+            word = quad_or(word);
+            if (active && quad_lane == 0) {
+                const size_t idx = TILED ? ((((size_t)(w >> 2) * M + row) * bits + b) * 4 + (w & 3))
+                                         : ((size_t)b * M + row) * KW + w;
+                planes[idx] = word;
+            }
+        }
+    }
+}
+
+hipError_t launch_quant_pack_rows(const void *x, uint32_t *planes, float *scale, float *zero, int *group_sums,
+                                  int M, int K, int bits, int symmetric, int group_size, int tiled,
+                                  hipStream_t stream)
+{
+    if (tiled)
+        hipLaunchKernelGGL(quant_pack_rows_kernel<true>, dim3(M), dim3(256), 0, stream,
+                           reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits,
+                           symmetric, group_size);
+    else
+        hipLaunchKernelGGL(quant_pack_rows_kernel<false>, dim3(M), dim3(256), 0, stream,
+                           reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits,
+                           symmetric, group_size);
+    return hipGetLastError();
+}
+
+// w_zero_term[n] = sum_g w_scale[n][g] * (sum of the weight codes of row n in group g
+//                                         - group_size * w_zero[n][g]);
+// one wave per weight row, lanes over the row's groups.
+__global__ __launch_bounds__(256) void weight_zero_term_kernel(const uint32_t *__restrict__ planes, int N, int KW, int bits,
+                                                               int is_signed, const float *__restrict__ w_scale,
+                                                               const float *__restrict__ w_zero, int group_size,
+                                                               float *__restrict__ out)
+{
+    const int n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (n >= N)
+        return; // whole waves leave; no barrier below
+    const int wpg = group_size / 32, groups = KW / wpg;
+    float t = 0.f;
+    for (int gi = lane; gi < groups; gi += 64) {
+        int sum = 0;
+        for (int b = 0; b < bits; ++b) {
+            int c = 0;
+            for (int w = 0; w < wpg; ++w)
+                c += __popc(planes[((size_t)b * N + n) * KW + gi * wpg + w]);
+            sum += (is_signed && b == bits - 1) ? -(c << b) : (c << b);
+        }
+        const size_t idx = (size_t)n * groups + gi;
+        t += w_scale[idx] * ((float)sum - (float)group_size * (w_zero ? w_zero[idx] : 0.f));
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        t += __shfl_xor(t, o);
+    if (lane == 0)
+        out[n] = t;
+}
+
+hipError_t launch_weight_zero_term(const uint32_t *planes, int n, int k, int bits, int is_signed, const float *w_scale,
+                                   const float *w_zero, int group_size, float *out, hipStream_t stream)
+{
+    hipLaunchKernelGGL(weight_zero_term_kernel, dim3((n + 3) / 4), dim3(256), 0, stream, planes, n, k / 32, bits,
+                       is_signed, w_scale, w_zero, group_size, out);
+    return hipGetLastError();
+}
+
 static int grid_for(size_t items)
 {
     size_t blocks = (items + 255) / 256;

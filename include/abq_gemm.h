@@ -167,6 +167,11 @@ typedef struct abq_gemm_state {
     int auto_chosen;         /* 1 if the tile was the library's choice                     */
     void *workspace;         /* caller-owned device scratch for the layout conversions     */
     size_t workspace_bytes;
+    /* zero points of the group-scale path, see abq_gemm_set_zero_points */
+    const float *x_zero;
+    const float *w_zero;
+    const int32_t *x_group_sums;
+    const float *w_zero_term;
 } abq_gemm_state;
 
 /* Replaces AqBMMAInitFn / AqBWMMAInitFn (engine/mma_any/aq_bmma_op.h:141-147,163 and
@@ -183,6 +188,49 @@ abq_status abq_gemm_init(const abq_tile_config *cfg, int x_bits, int w_bits, int
  * algorithm/quantize/quantizer.py:111-179 (scale per row of X, per row of W). */
 abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, const float *w_scale,
                                int group_size);
+/* group_size 0: w_scale is [N] and D = acc * x_scale[m] * w_scale[n].
+ * group_size 64 or 128: w_scale is [N][K/group_size] (the reference reshapes W to
+ * [-1, group_size] before calibrating, quantizer.py:151-156) and
+ *     D[m][n] = x_scale[m] * sum_g w_scale[n][g] * (sum_{k in g} x[m][k] * w[n][k]).
+ * Group scales run on ABQ_STRATEGY_TILED only: a state whose tile was the library's choice is
+ * moved there (and needs the workspace / layouts of that strategy); a state pinned to another
+ * tile tuple, or 8-bit unsigned operands, return ABQ_ERR_UNSUPPORTED. */
+
+/* Zero points for a state with group scales (asymmetric quantisation, quantizer.py:120-128:
+ * x ~ scale * (code - zero)).  Codes are the integers in the bit planes, read with the
+ * state's signedness; a caller holding unsigned codes u in [0, 2^n) and zero point z may store
+ * u - 2^(n-1) in signed planes and pass z - 2^(n-1).
+ *   w_zero       [N][K/group_size]  weight zero points, or NULL
+ *   x_group_sums [M][K/group_size]  sums of the activation codes per group; required with w_zero
+ *                                   (abq_quant_pack_f16 writes them)
+ *   x_zero       [M]                activation zero points, or NULL
+ *   w_zero_term  [N]                required with x_zero (abq_weight_zero_term computes it once
+ *                                   per weight matrix)
+ *     D[m][n] = x_scale[m] * ( sum_g w_scale[n][g] * (acc_g - w_zero[n][g] * x_group_sums[m][g])
+ *                              - x_zero[m] * w_zero_term[n] ). */
+abq_status abq_gemm_set_zero_points(abq_gemm_state *state, const float *x_zero, const float *w_zero,
+                                    const int32_t *x_group_sums, const float *w_zero_term);
+
+/* w_zero_term[n] = sum_g w_scale[n][g] * (sum_{k in g} w[n][k] - group_size * w_zero[n][g]),
+ * from weight planes in the reference layout.  w_zero may be NULL (all zero). */
+abq_status abq_weight_zero_term(const uint32_t *w_planes, int n, int k, int bits, int is_signed,
+                                const float *w_scale, const float *w_zero, int group_size,
+                                float *w_zero_term, void *stream);
+
+/* Per-token dynamic quantisation of fp16 activations [rows][k] fused with bit-plane packing:
+ * the device-side counterpart of the reference's per_token_dynamic_calibration + fake_quant
+ * rounding (algorithm/quantize/quantizer.py:111-179) followed by pack.  Writes signed codes
+ * (two's complement planes, `bits` planes) in the layout asked for, scale[rows], and
+ * optionally zero[rows] (NULL allowed when symmetric) and group_sums[rows][k/group_size]
+ * (NULL, or group_size 64 / 128).
+ *   symmetric != 0: scale = clamp(absmax / (2^(bits-1) - 1), 1e-5, 1e4), zero = 0
+ *   symmetric == 0: scale = clamp((max - min) / (2^bits - 1), 1e-5, 1e4),
+ *                   zp = round(clamp(-min / scale, -1e4, 1e4)), stored code = u - 2^(bits-1),
+ *                   zero = zp - 2^(bits-1)
+ * fp32 arithmetic, round half to even.  2 <= bits <= 8, k % 128 == 0. */
+abq_status abq_quant_pack_f16(const void *x_f16, int rows, int k, int bits, int symmetric, int layout,
+                              uint32_t *planes, float *scale, float *zero, int32_t *group_sums,
+                              int group_size, void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * K-tiled plane layout (no counterpart in the reference; its kernels only exist for M <= 8).

@@ -83,3 +83,60 @@ def dequantize(xi, qp, scale, zp):
 def fake_quant(x, qp):
     scale, zp = calibrate(x, qp)
     return dequantize(quantize(x, qp, scale, zp), qp, scale, zp)
+
+
+def per_token_codes_f32(x, n_bits, symmetric):
+    """calibrate + quantize for one scale per row (no groups), in float32 round-half-even
+    arithmetic, with codes expressed as signed integers: x ~ scale * (code - zero).
+
+    symmetric: the disable_zero_point range [-2^(n-1), 2^(n-1)-1], zero = 0.
+    asymmetric: unsigned code u in [0, 2^n - 1] and zero point zp as the reference derives them
+    (quantizer.py:165-179, without the 1-/2-bit "bit balance" widening), returned shifted by
+    2^(n-1): code = u - 2^(n-1), zero = zp - 2^(n-1).
+    Returns (codes int32 [rows, cols], scale float32 [rows], zero float32 [rows])."""
+    f = np.float32
+    x = np.asarray(x).astype(f)
+    xmin = x.min(axis=-1, keepdims=True)
+    xmax = x.max(axis=-1, keepdims=True)
+    half = 1 << (n_bits - 1)
+    if symmetric:
+        scale = np.maximum(np.abs(xmax), np.abs(xmin)) / f(half - 1)
+        scale = np.clip(scale, f(CLIPMIN), f(1e4)).astype(f)
+        codes = np.clip(np.rint(x / scale), -half, half - 1)
+        zero = np.zeros_like(scale)
+    else:
+        scale = (xmax - xmin) / f(2 * half - 1)
+        scale = np.clip(scale, f(CLIPMIN), f(1e4)).astype(f)
+        zp = np.rint(np.clip(-xmin / scale, f(-1e4), f(1e4))).astype(f)
+        codes = np.clip(np.rint(x / scale) + zp, 0, 2 * half - 1) - half
+        zero = zp - f(half)
+    return codes.astype(np.int32), scale[:, 0].astype(f), zero[:, 0].astype(f)
+
+
+def group_affine_codes(w, n_bits, group_size):
+    """Weights [N, K] -> asymmetric codes per (row, group of group_size along K), the reference's
+    weight configuration (per_channel_axes=[0] + group_size, main.py:280-288 of the reference)
+    with the plain 2^n - 1 level range.  Signed representation as in per_token_codes_f32.
+    Returns (codes int32 [N, K], scale float64 [N, K/g], zero float64 [N, K/g])."""
+    w = np.asarray(w, dtype=np.float64)
+    n, k = w.shape
+    g = w.reshape(n, k // group_size, group_size)
+    wmin = g.min(axis=-1, keepdims=True)
+    wmax = g.max(axis=-1, keepdims=True)
+    half = 1 << (n_bits - 1)
+    scale = np.clip((wmax - wmin) / (2 * half - 1), CLIPMIN, 1e4)
+    zp = np.round(np.clip(-wmin / scale, -1e4, 1e4))
+    codes = np.clip(np.round(g / scale) + zp, 0, 2 * half - 1) - half
+    return codes.reshape(n, k).astype(np.int32), scale[..., 0], zp[..., 0] - half
+
+
+def dequant_matmul(x_codes, x_scale, x_zero, w_codes, w_scale, w_zero, group_size):
+    """fp64 x_dq @ w_dq.T of the dequantised operands (the reference's fake-quant forward,
+    int_linear.py:25-84 with quantizer.py:124-128).  w_scale / w_zero are [N, K/g] (or [N, 1]
+    with group_size = K); x_scale / x_zero are [M]."""
+    xd = (x_codes.astype(np.float64) - np.asarray(x_zero, dtype=np.float64)[:, None]) * \
+        np.asarray(x_scale, dtype=np.float64)[:, None]
+    ws = np.repeat(np.asarray(w_scale, dtype=np.float64), group_size, axis=1)
+    wz = np.repeat(np.asarray(w_zero, dtype=np.float64), group_size, axis=1)
+    wd = (w_codes.astype(np.float64) - wz) * ws
+    return xd @ wd.T

@@ -1,0 +1,189 @@
+"""GPU tests of the dequantisation side of the path: per-token dynamic quantisation fused with
+packing, group-wise weight scales, zero-point corrections, and the decoder-layer linears of
+BASELINE.json configs[4].  Expected values are fp64 matmuls of the dequantised operands; the
+tolerance is the 1e-2 relative error the task states for the fp16 output."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    if not torch.cuda.is_available():
+        pytest.fail("marked gpu but no GPU is visible")
+
+
+def planes_dev(planes):
+    return torch.from_numpy(np.ascontiguousarray(planes).view(np.int32)).cuda()
+
+
+def fdev(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def assert_close_rel(got, want):
+    """|got - want| <= REL_TOL * |want| elementwise, with an absolute floor of REL_TOL times the
+    matrix's RMS for entries that cancel to nearly zero; plus a much tighter norm-wise bound."""
+    got = got.astype(np.float64)
+    rms = np.sqrt(np.mean(want ** 2))
+    err = np.abs(got - want)
+    assert np.all(np.isfinite(got))
+    assert np.all(err <= REL_TOL * np.abs(want) + REL_TOL * rms), float((err / (np.abs(want) + rms)).max())
+    assert np.linalg.norm(got - want) <= 2e-3 * np.linalg.norm(want)
+
+
+def run_grouped(abq, xp, wp, signed, **kw):
+    g = abq.Gemm(xp, wp, signed, out_kind=abq.OUT_F16_SCALED, **kw)
+    assert g.strategy == "tiled"
+    if g.workspace_bytes:
+        ws = torch.empty(g.workspace_bytes, dtype=torch.uint8, device="cuda")
+        g = abq.Gemm(xp, wp, signed, out_kind=abq.OUT_F16_SCALED, workspace=ws, **kw)
+    out = g.run()
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+# ------------------------------------------------------------------ quantise + pack
+
+@pytest.mark.parametrize("rows,k,bits,symmetric", [(1, 128, 8, True), (5, 4096, 8, True), (33, 11008, 8, False),
+                                                   (7, 256, 4, True), (16, 1152, 4, False), (3, 384, 2, True),
+                                                   (64, 4096, 6, False)])
+def test_quant_pack_matches_the_restated_quantizer(abq, oracle, rows, k, bits, symmetric):
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(rows + k + bits)
+    x = (rng.normal(0, 1, (rows, k)) * rng.uniform(0.1, 8, (rows, 1))).astype(np.float16)
+    x[0, :7] = [0, -0.0, 1, -1, 0.5, 65504, -3]  # an outlier row
+    codes, scale, zero = Q.per_token_codes_f32(x, bits, symmetric)
+    for gs in (64, 128):
+        planes, s, z, sums = abq.quant_pack_f16(torch.from_numpy(x).cuda(), bits, symmetric=symmetric, group_size=gs)
+        torch.cuda.synchronize()
+        assert np.array_equal(s.cpu().numpy(), scale)
+        if not symmetric:
+            assert np.array_equal(z.cpu().numpy(), zero)
+        assert np.array_equal(planes.cpu().numpy().view(np.uint32), oracle.pack_i32(codes, bits))
+        assert np.array_equal(sums.cpu().numpy(), codes.reshape(rows, k // gs, gs).sum(axis=2))
+    # K-tiled output equals the relayout of the plane output
+    tiled, _, _, _ = abq.quant_pack_f16(torch.from_numpy(x).cuda(), bits, symmetric=symmetric, tiled=True)
+    assert torch.equal(tiled, abq.relayout_planes(planes))
+
+
+# ------------------------------------------------------------------ group scales, zero points
+
+@pytest.mark.parametrize("q,p,signed", [(8, 2, True), (4, 4, True), (8, 4, True), (4, 4, False), (6, 2, False),
+                                        (2, 2, True), (7, 7, False)])
+@pytest.mark.parametrize("group_size", [128, 64])
+def test_group_scale_epilogue(abq, oracle, q, p, signed, group_size):
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(q * 10 + p + group_size)
+    for (M, N, K) in [(70, 200, 384), (256, 1024, 1024)]:
+        lo_x, hi_x = (-(1 << (q - 1)), 1 << (q - 1)) if signed else (0, 1 << q)
+        lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed else (0, 1 << p)
+        x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        xs = rng.uniform(0.01, 0.05, M)
+        wsc = rng.uniform(0.001, 0.02, (N, K // group_size))
+        want = Q.dequant_matmul(x, xs, np.zeros(M), w, wsc, np.zeros_like(wsc), group_size)
+        got = run_grouped(abq, planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p)), signed,
+                          x_scale=fdev(xs), w_scale=fdev(wsc), group_size=group_size)
+        assert_close_rel(got, want)
+
+
+@pytest.mark.parametrize("group_size", [128, 64])
+@pytest.mark.parametrize("with_x_zero", [False, True])
+def test_zero_point_corrections(abq, oracle, group_size, with_x_zero):
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(group_size + with_x_zero)
+    for (q, p, signed) in [(8, 2, True), (4, 4, False)]:
+        M, N, K = 150, 330, 5 * 1152  # 45 (or 90) groups: more than one LDS staging pass
+        lo_x, hi_x = (-(1 << (q - 1)), 1 << (q - 1)) if signed else (0, 1 << q)
+        lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed else (0, 1 << p)
+        x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        xs = rng.uniform(0.01, 0.05, M)
+        xz = rng.integers(lo_x // 2, hi_x // 2, M).astype(np.float64) if with_x_zero else np.zeros(M)
+        wsc = rng.uniform(0.001, 0.02, (N, K // group_size))
+        wz = rng.integers(lo_w, hi_w, (N, K // group_size)).astype(np.float64)
+        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, group_size)
+        wp = planes_dev(oracle.pack_i32(w, p))
+        kw = dict(x_scale=fdev(xs), w_scale=fdev(wsc), group_size=group_size, w_zero=fdev(wz),
+                  x_group_sums=torch.from_numpy(x.reshape(M, K // group_size, group_size).sum(axis=2).astype(np.int32)).cuda())
+        if with_x_zero:
+            term = abq.weight_zero_term(wp, signed, kw["w_scale"], kw["w_zero"], group_size)
+            want_term = (wsc * (w.reshape(N, -1, group_size).sum(axis=2) - group_size * wz)).sum(axis=1)
+            assert np.allclose(term.cpu().numpy(), want_term, rtol=1e-5, atol=1e-5)
+            kw.update(x_zero=fdev(xz), w_zero_term=term)
+        got = run_grouped(abq, planes_dev(oracle.pack_i32(x, q)), wp, signed, **kw)
+        assert_close_rel(got, want)
+
+
+def test_group_scale_argument_checks(abq, oracle):
+    rng = np.random.default_rng(0)
+    x = planes_dev(oracle.pack_i32(rng.integers(0, 256, (32, 256)).astype(np.int32), 8))
+    w = planes_dev(oracle.pack_i32(rng.integers(0, 256, (64, 256)).astype(np.int32), 8))
+    s = torch.ones(64 * 4, dtype=torch.float32, device="cuda")
+    with pytest.raises(abq.AbqError) as e:  # 8-bit unsigned operands have no group-scale kernel
+        abq.Gemm(x, w, False, out_kind=abq.OUT_F16_SCALED, x_scale=s, w_scale=s, group_size=128)
+    assert e.value.status == abq.ABQ_ERR_UNSUPPORTED
+    with pytest.raises(abq.AbqError) as e:  # only 64 and 128
+        abq.Gemm(x, w, True, out_kind=abq.OUT_F16_SCALED, x_scale=s, w_scale=s, group_size=32)
+    assert e.value.status == abq.ABQ_ERR_UNSUPPORTED
+    with pytest.raises(abq.AbqError) as e:  # zero points need group scales
+        abq.Gemm(x, w, True, out_kind=abq.OUT_F16_SCALED, x_scale=s, w_scale=s, group_size=0, w_zero=s, x_group_sums=s)
+    assert e.value.status == abq.ABQ_ERR_UNSUPPORTED
+    with pytest.raises(abq.AbqError) as e:  # w_zero without the activation group sums
+        abq.Gemm(x, w, True, out_kind=abq.OUT_F16_SCALED, x_scale=s, w_scale=s, group_size=128, w_zero=s)
+    assert e.value.status == abq.ABQ_ERR_INVALID_ARG
+
+
+# ------------------------------------------------------------------ BASELINE.json configs[4]
+
+LAYER_LINEARS = [("qkv", 12288, 4096), ("o", 4096, 4096), ("gate_up", 2 * 11008, 4096), ("down", 4096, 11008)]
+
+
+def _layer_linear(abq, oracle, name, N, K, tokens, x_symmetric, seed, sample_rows):
+    """One W2A8 linear: fp16 weights N(0, 0.02) quantised to 2 bits per (channel, group of 128),
+    fp16 activations quantised per token on the device; checks `sample_rows` output rows."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(seed)
+    w = rng.normal(0, 0.02, (N, K)).astype(np.float16)
+    w_codes, w_scale, w_zero = Q.group_affine_codes(w, 2, 128)
+    wp = planes_dev(oracle.pack_i32(w_codes, 2))
+    wt = abq.relayout_planes(wp)
+    ws_d, wz_d = fdev(w_scale), fdev(w_zero)
+
+    xg = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.randn((tokens, K), generator=xg, device="cuda", dtype=torch.float32)
+    x[:, ::97] *= 8.0  # a few outlier channels, as LLM activations have
+    x = x.to(torch.float16)
+    xt, xs, xz, sums = abq.quant_pack_f16(x, 8, symmetric=x_symmetric, tiled=True, group_size=128)
+    kw = dict(x_scale=xs, w_scale=ws_d, group_size=128, w_zero=wz_d, x_group_sums=sums, x_tiled=True, w_tiled=True)
+    if not x_symmetric:
+        kw.update(x_zero=xz, w_zero_term=abq.weight_zero_term(wp, True, ws_d, wz_d, 128))
+    got = run_grouped(abq, xt, wt, True, **kw)
+
+    rows = np.sort(rng.choice(tokens, size=min(sample_rows, tokens), replace=False))
+    x_rows = x[torch.from_numpy(rows).cuda()].cpu().numpy()
+    codes, scale, zero = Q.per_token_codes_f32(x_rows, 8, x_symmetric)
+    assert np.array_equal(xs.cpu().numpy()[rows], scale)
+    want = Q.dequant_matmul(codes, scale, zero, w_codes, w_scale, w_zero, 128)
+    assert_close_rel(got[rows], want)
+    # and the quantised result tracks the unquantised fp16 linear as 2-bit weights allow: the
+    # dequantised weights are within scale/2 of the originals, so this is only a sanity bound
+    full = x_rows.astype(np.float64) @ w.astype(np.float64).T
+    assert np.linalg.norm(want - full) < 0.7 * np.linalg.norm(full)
+
+
+@pytest.mark.parametrize("name,N,K", LAYER_LINEARS)
+@pytest.mark.parametrize("x_symmetric", [True, False])
+def test_config4_decoder_layer_linears_batch1(abq, oracle, name, N, K, x_symmetric):
+    _layer_linear(abq, oracle, name, N, K, 1024, x_symmetric, seed=len(name) + N % 97, sample_rows=48)
+
+
+@pytest.mark.parametrize("name,N,K", LAYER_LINEARS)
+def test_config4_decoder_layer_linears_batch16(abq, oracle, name, N, K):
+    _layer_linear(abq, oracle, name, N, K, 16 * 1024, True, seed=7 + len(name), sample_rows=32)

@@ -220,3 +220,57 @@ def test_quantizer_closed_forms():
     # two-bit "bit balance": asymmetric 2-bit range is widened to five levels (quantizer.py:66-68)
     qp = Q.QuantParams(2)
     assert (qp.qmin, qp.qmax) == (0, 4)
+
+
+def test_per_token_codes_f32_agrees_with_the_fp64_restatement():
+    rng = np.random.default_rng(21)
+    x = rng.normal(0, 1, (8, 512)).astype(np.float16)
+    # symmetric: same codes as calibrate/quantize in fp64 except where x/scale sits on a rounding tie
+    codes, scale, zero = Q.per_token_codes_f32(x, 8, True)
+    qp = Q.QuantParams(8, symmetric=True, disable_zero_point=True)
+    s64, _ = Q.calibrate(x, qp)
+    c64 = Q.quantize(x, qp, s64, None)
+    assert np.allclose(scale, s64[:, 0], rtol=1e-6) and not zero.any()
+    assert np.abs(codes - c64).max() <= 1 and (codes != c64).mean() < 1e-3
+    assert np.all(np.abs(codes).max(axis=1) == 127)
+    # asymmetric: unsigned code = code + 2^(n-1), zero point = zero + 2^(n-1)
+    for bits in (8, 4):
+        codes, scale, zero = Q.per_token_codes_f32(x, bits, False)
+        qp = Q.QuantParams(bits)
+        s64, z64 = Q.calibrate(x, qp)
+        c64 = Q.quantize(x, qp, s64, z64)
+        half = 1 << (bits - 1)
+        assert np.allclose(scale, s64[:, 0], rtol=1e-6)
+        assert np.array_equal(zero + half, z64[:, 0])
+        assert np.abs(codes + half - c64).max() <= 1 and (codes + half != c64).mean() < 2e-3
+        assert (codes + half).min() == 0 and (codes + half).max() == 2 * half - 1
+        # dequantisation error at most scale / 2 inside the clamp range
+        deq = (codes - zero[:, None]) * scale[:, None]
+        assert np.all(np.abs(deq - x.astype(np.float32)) <= scale[:, None] * 0.5001)
+
+
+def test_group_affine_codes_and_dequant_matmul():
+    rng = np.random.default_rng(22)
+    w = rng.normal(0, 0.02, (12, 256))
+    codes, scale, zero = Q.group_affine_codes(w, 2, 128)
+    assert codes.shape == (12, 256) and scale.shape == (12, 2) and zero.shape == (12, 2)
+    assert codes.min() == -2 and codes.max() == 1
+    # every group's min and max land on the ends of the code range
+    g = codes.reshape(12, 2, 128)
+    assert np.all(g.min(axis=2) == -2) and np.all(g.max(axis=2) == 1)
+    # same codes as the general restatement with a 4-level range (bit balance switched off)
+    qp = Q.QuantParams(2, group_size=128)
+    qp.qmax = 3
+    s = np.clip((w.reshape(-1, 128).max(1) - w.reshape(-1, 128).min(1)) / 3, Q.CLIPMIN, 1e4)[:, None]
+    z = np.round(-w.reshape(-1, 128).min(1)[:, None] / s)
+    assert np.array_equal(Q.quantize(w, qp, s, z), codes + 2)
+    # dequant_matmul against an element-by-element loop
+    xc = rng.integers(-128, 128, (3, 256)).astype(np.int32)
+    xs, xz = rng.uniform(0.01, 0.1, 3), rng.integers(-5, 5, 3).astype(np.float64)
+    got = Q.dequant_matmul(xc, xs, xz, codes, scale, zero, 128)
+    want = np.zeros((3, 12))
+    for m in range(3):
+        for n in range(12):
+            for k in range(256):
+                want[m, n] += (xc[m, k] - xz[m]) * xs[m] * (codes[n, k] - zero[n, k // 128]) * scale[n, k // 128]
+    assert np.allclose(got, want, rtol=1e-12, atol=1e-12)
