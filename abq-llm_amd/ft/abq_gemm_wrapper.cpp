@@ -81,3 +81,59 @@ void ABQGEMMWrapper::gemm_scaled(const int M, const int N, const int K, const in
     if (ex != ABQ_OK)
         printf("[ABQ][Error] launch failed: %s\n", abq_status_string(ex));
 }
+
+// workspace: activation planes | scale[M] | zero[M] | group sums [M][K/group_size]
+size_t ABQGEMMWrapper::dynamic_workspace_bytes(int M, int K, int group_size) const
+{
+    const size_t planes = ((size_t)x_bits_ * M * K / 8 + 255) / 256 * 256;
+    return planes + (size_t)M * 8 + (size_t)M * (K / group_size) * 4;
+}
+
+void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _Float16 *A, const ABQGroupedWeight &W,
+                                  _Float16 *D, bool x_symmetric, char *abq_gemm_workspace, size_t abq_gemm_ws_bytes,
+                                  hipStream_t stream)
+{
+    if (K < 128 || K % 128 != 0) {
+        printf("[ABQ][Error] unsupport K = %d\n", K);
+        return;
+    }
+    if (!signed_ || (W.group_size != 64 && W.group_size != 128) || (!x_symmetric && !W.zero_term)) {
+        printf("[ABQ][Error] unsupport dynamic quantisation setup\n");
+        return;
+    }
+    if (abq_gemm_ws_bytes < dynamic_workspace_bytes(M, K, W.group_size)) {
+        printf("[ABQ][Error] workspace too small: %zu bytes for M,K,bits = %d,%d,%d\n", abq_gemm_ws_bytes, M, K, x_bits_);
+        return;
+    }
+    const size_t planes_bytes = ((size_t)x_bits_ * M * K / 8 + 255) / 256 * 256;
+    uint32_t *planes = reinterpret_cast<uint32_t *>(abq_gemm_workspace);
+    float *x_scale = reinterpret_cast<float *>(abq_gemm_workspace + planes_bytes);
+    float *x_zero = x_scale + M;
+    int32_t *sums = reinterpret_cast<int32_t *>(x_zero + M);
+    abq_status rc = abq_quant_pack_f16(A, M, K, x_bits_, x_symmetric ? 1 : 0, ABQ_LAYOUT_TILED, planes, x_scale, x_zero,
+                                       sums, W.group_size, stream);
+    if (rc != ABQ_OK) {
+        printf("[ABQ][Error] pack failed: %s\n", abq_status_string(rc));
+        return;
+    }
+    abq_gemm_state state;
+    rc = abq_gemm_init(nullptr, x_bits_, w_bits_, 1, planes, reinterpret_cast<const uint32_t *>(W.planes_tiled), M, N, K,
+                       D, nullptr, 0, ABQ_OUT_F16_SCALED, &state);
+    if (rc == ABQ_OK)
+        rc = abq_gemm_set_scales(&state, x_scale, W.scale, W.group_size);
+    if (rc == ABQ_OK)
+        rc = abq_gemm_set_operand_layout(&state, ABQ_LAYOUT_TILED, ABQ_LAYOUT_TILED);
+    if (rc == ABQ_OK && (W.zero || !x_symmetric))
+        rc = abq_gemm_set_zero_points(&state, x_symmetric ? nullptr : x_zero, W.zero, sums, W.zero_term);
+    if (rc == ABQ_ERR_UNSUPPORTED) {
+        printf("[ABQ][Error] unsupport w%da%d\n", w_bits_, x_bits_);
+        return;
+    }
+    if (rc != ABQ_OK || !state.init_success) {
+        printf("[ABQ][Error] return due to unsuccessful initialization.\n");
+        return;
+    }
+    const abq_status ex = abq_gemm_exec(&state, stream);
+    if (ex != ABQ_OK)
+        printf("[ABQ][Error] launch failed: %s\n", abq_status_string(ex));
+}

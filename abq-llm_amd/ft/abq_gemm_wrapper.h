@@ -13,9 +13,20 @@
 //    and reads the low 16 bits of the float, abq_gemm_wrapper.cu:126);
 //  * the workspace size is checked.
 // gemm_scaled() is new: per-token activation scales and per-channel weight scales.
+// gemm_dynamic() is new: per-token dynamic activation quantisation on the device, group-wise
+// weight scales and zero points (the quantiser semantics of algorithm/quantize/quantizer.py).
 #pragma once
 #include <hip/hip_runtime_api.h>
 #include <stddef.h>
+
+// One prepared weight matrix for gemm_dynamic(): device pointers, owned by the caller.
+struct ABQGroupedWeight {
+    const int *planes_tiled;  // K-tiled planes [K/128][N][w_bits][4] (abq_relayout_planes)
+    const float *scale;       // [N][K/group_size]
+    const float *zero;        // [N][K/group_size] in units of (signed) weight codes, or nullptr
+    const float *zero_term;   // [N] from abq_weight_zero_term; needed for asymmetric activations
+    int group_size;           // 64 or 128
+};
 
 class ABQGEMMWrapper {
 private:
@@ -40,4 +51,11 @@ public:
     // D[m][n] = acc[m][n] * x_scale[m] * w_scale[n]; X given as already packed planes.
     void gemm_scaled(const int M, const int N, const int K, const int *X_packed, const int *B, _Float16 *D,
                      const float *x_scale, const float *w_scale, hipStream_t stream);
+    // A: fp16 activations [M][K], quantised per token to X_BITS signed codes inside the call
+    // (symmetric, or asymmetric with a zero point); D: fp16 [M][N].  The wrapper must have been
+    // constructed with SIGNED = true.  Workspace: dynamic_workspace_bytes(M, K, group_size).
+    void gemm_dynamic(const int M, const int N, const int K, const _Float16 *A, const ABQGroupedWeight &W,
+                      _Float16 *D, bool x_symmetric, char *abq_gemm_workspace, size_t abq_gemm_ws_bytes,
+                      hipStream_t stream);
+    size_t dynamic_workspace_bytes(int M, int K, int group_size) const;
 };

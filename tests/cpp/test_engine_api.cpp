@@ -173,6 +173,101 @@ static void gpu_paths()
         HIP_OK(hipFree(d_ws));
     }
 
+    {   // FT wrapper, dynamic path: per-token int8 activations, 2-bit weights with group scales and
+        // zero points; expected values from a double-precision loop over the dequantised operands
+        const int M = 40, N = 192, K = 512, G = 128, groups = K / G;
+        std::mt19937 r32(5);
+        std::normal_distribution<float> nd(0.f, 1.5f);
+        std::uniform_real_distribution<float> ud(0.002f, 0.02f);
+        std::vector<uint16_t> ha((size_t)M * K);
+        for (auto &h : ha)
+            h = abq_oracle_f32_to_f16(nd(r32));
+        std::vector<int> wq((size_t)N * K);
+        for (auto &v : wq)
+            v = (int)(r32() % 4) - 2;
+        std::vector<float> wscale((size_t)N * groups), wzero((size_t)N * groups);
+        for (auto &v : wscale)
+            v = ud(r32);
+        for (auto &v : wzero)
+            v = (float)((int)(r32() % 4) - 2);
+        std::vector<uint32_t> wpl((size_t)2 * N * K / 32);
+        abq_oracle_pack_i32(wq.data(), wpl.data(), N, K, 2);
+        _Float16 *d_a, *d_d;
+        uint32_t *d_wpl, *d_wt;
+        float *d_wscale, *d_wzero, *d_term;
+        char *d_ws;
+        ABQGEMMWrapper wrap(8, 2, true);
+        const size_t ws_bytes = wrap.dynamic_workspace_bytes(M, K, G);
+        HIP_OK(hipMalloc(&d_a, ha.size() * 2));
+        HIP_OK(hipMalloc(&d_d, (size_t)M * N * 2));
+        HIP_OK(hipMalloc(&d_wpl, wpl.size() * 4));
+        HIP_OK(hipMalloc(&d_wt, wpl.size() * 4));
+        HIP_OK(hipMalloc(&d_wscale, wscale.size() * 4));
+        HIP_OK(hipMalloc(&d_wzero, wzero.size() * 4));
+        HIP_OK(hipMalloc(&d_term, N * 4));
+        HIP_OK(hipMalloc(&d_ws, ws_bytes));
+        HIP_OK(hipMemcpy(d_a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(d_wpl, wpl.data(), wpl.size() * 4, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(d_wscale, wscale.data(), wscale.size() * 4, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(d_wzero, wzero.data(), wzero.size() * 4, hipMemcpyHostToDevice));
+        CHECK(abq_relayout_planes(d_wpl, d_wt, N, K, 2, stream) == ABQ_OK);
+        CHECK(abq_weight_zero_term(d_wpl, N, K, 2, 1, d_wscale, d_wzero, G, d_term, stream) == ABQ_OK);
+        const ABQGroupedWeight weight = { reinterpret_cast<const int *>(d_wt), d_wscale, d_wzero, d_term, G };
+        for (int symmetric = 1; symmetric >= 0; --symmetric) {
+            wrap.gemm_dynamic(M, N, K, d_a, weight, d_d, symmetric != 0, d_ws, ws_bytes, stream);
+            HIP_OK(hipStreamSynchronize(stream));
+            std::vector<uint16_t> got((size_t)M * N);
+            HIP_OK(hipMemcpy(got.data(), d_d, got.size() * 2, hipMemcpyDeviceToHost));
+            double worst = 0, ref_sq = 0;
+            std::vector<double> want((size_t)M * N);
+            for (int m = 0; m < M; ++m) {
+                // the per-token quantiser in float, as the kernel defines it
+                float mx = -INFINITY, mn = INFINITY;
+                for (int k = 0; k < K; ++k) {
+                    const float f = abq_oracle_f16_to_f32(ha[(size_t)m * K + k]);
+                    mx = std::fmax(mx, f);
+                    mn = std::fmin(mn, f);
+                }
+                float scale, zp = 0.f;
+                if (symmetric) {
+                    scale = std::fmin(std::fmax(std::fmax(std::fabs(mx), std::fabs(mn)) / 127.f, 1e-5f), 1e4f);
+                } else {
+                    scale = std::fmin(std::fmax((mx - mn) / 255.f, 1e-5f), 1e4f);
+                    zp = std::nearbyint(std::fmin(std::fmax(-mn / scale, -1e4f), 1e4f));
+                }
+                std::vector<double> xd(K);
+                for (int k = 0; k < K; ++k) {
+                    const float f = abq_oracle_f16_to_f32(ha[(size_t)m * K + k]);
+                    float code = std::nearbyint(f / scale) + zp;
+                    code = symmetric ? std::fmin(std::fmax(code, -128.f), 127.f) : std::fmin(std::fmax(code, 0.f), 255.f);
+                    xd[k] = ((double)code - zp) * scale;
+                }
+                for (int n = 0; n < N; ++n) {
+                    double acc = 0;
+                    for (int k = 0; k < K; ++k)
+                        acc += xd[k] * ((double)wq[(size_t)n * K + k] - wzero[(size_t)n * groups + k / G]) *
+                               wscale[(size_t)n * groups + k / G];
+                    want[(size_t)m * N + n] = acc;
+                    ref_sq += acc * acc;
+                }
+            }
+            const double rms = std::sqrt(ref_sq / want.size());
+            for (size_t i = 0; i < want.size(); ++i) {
+                const double err = std::fabs((double)abq_oracle_f16_to_f32(got[i]) - want[i]);
+                worst = std::fmax(worst, err / (std::fabs(want[i]) + rms));
+            }
+            CHECK(worst <= 1e-2); // the 1e-2 relative tolerance of the fp16 dequantised output
+        }
+        HIP_OK(hipFree(d_a));
+        HIP_OK(hipFree(d_d));
+        HIP_OK(hipFree(d_wpl));
+        HIP_OK(hipFree(d_wt));
+        HIP_OK(hipFree(d_wscale));
+        HIP_OK(hipFree(d_wzero));
+        HIP_OK(hipFree(d_term));
+        HIP_OK(hipFree(d_ws));
+    }
+
     {   // timer interface
         CudaTimer t(stream);
         t.start();
