@@ -97,6 +97,107 @@ ABQ_HD uint64_t transpose8x8(uint64_t x)
     return x;
 }
 
+// ---- field-packed K tiles ------------------------------------------------------------------
+//
+// The LDS-staged MFMA kernels keep their operands in a second, library-private format whose
+// unpacking to int8 costs one or two vector instructions per four elements instead of the
+// bit-matrix transpose that plane words need.  A row's K tile of 128 elements is one record of
+// BITS * 4 words; the element order inside a 32-element word-set is the one planes_to_int8
+// produces ("expanded" dword s, byte c = element 31 - (8c + s)).  The BITS-bit pattern of an
+// element is cut into fields, most significant first:
+//     8 bits: one 8-bit field (the bytes themselves);
+//     else  : a 4-bit, a 2-bit and a 1-bit field for every set bit of BITS (7 = 4+2+1, 6 = 4+2,
+//             5 = 4+1, 3 = 2+1).
+// A field of width f holds, per word-set, f words: word j carries in byte c, at bits
+// [f*s, f*s+f), the field of the element at expanded dword (8/f)*j + s, byte c.  In the record
+// the field of width f starts at word 4 * (BITS & ~(2f-1)) and its word-sets follow each other.
+ABQ_HD constexpr uint32_t field_mask(int f) { return 0x01010101u * ((1u << f) - 1u); }
+ABQ_HD constexpr int field_base(int bits, int f) { return bits & (f - 1); }             // lowest value bit of the field
+ABQ_HD constexpr int field_word_offset(int bits, int f) { return 4 * (bits & ~(2 * f - 1)); }
+
+// Expanded bytes (bit pattern in the low BITS bits of each byte) of one word-set -> its BITS
+// field words, ordered [4-bit field: 4 words][2-bit field: 2 words][1-bit field: 1 word].
+template <int BITS> ABQ_HD void compress_fields(const uint32_t (&e)[8], uint32_t (&out)[BITS])
+{
+    static_assert(BITS >= 1 && BITS <= 8, "1..8 bits");
+    if (BITS == 8) {
+#pragma unroll
+        for (int d = 0; d < 8; ++d)
+            out[d % BITS] = e[d];
+        return;
+    }
+    int idx = 0;
+#pragma unroll
+    for (int f = 4; f >= 1; f >>= 1) {
+        if (!(BITS & f))
+            continue;
+        const int per = 8 / f;
+#pragma unroll
+        for (int j = 0; j < f; ++j) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int s = 0; s < per; ++s)
+                v |= ((e[per * j + s] >> field_base(BITS, f)) & field_mask(f)) << (f * s);
+            out[(idx + j) % BITS] = v;
+        }
+        idx += f;
+    }
+}
+
+// The reverse, fused with the placement in the int8 lane (MODE as for planes_to_int8).  `raw`
+// holds the fields of WPT consecutive word-sets of one row, [4-bit field: 4*WPT words][2-bit:
+// 2*WPT][1-bit: WPT] (or 8*WPT bytes-as-words for 8 bits); `ws` selects the word-set.
+template <int BITS, int WPT, Int8Mode MODE>
+ABQ_HD void expand_fields(const uint32_t (&raw)[BITS * WPT], int ws, uint32_t (&e)[8])
+{
+    if (BITS == 8) {
+#pragma unroll
+        for (int d = 0; d < 8; ++d)
+            e[d] = raw[(8 * ws + d) % (BITS * WPT)] ^ (MODE == kFlip ? 0x80808080u : 0u);
+        return;
+    }
+#pragma unroll
+    for (int d = 0; d < 8; ++d)
+        e[d] = 0u;
+    int idx = 0;
+#pragma unroll
+    for (int f = 4; f >= 1; f >>= 1) {
+        if (!(BITS & f))
+            continue;
+        const int per = 8 / f;
+        const int t = field_base(BITS, f) + (MODE == kTop ? 8 - BITS : 0); // where the field lands in the byte
+#pragma unroll
+        for (int j = 0; j < f; ++j) {
+            const uint32_t w = raw[(idx + f * ws + j) % (BITS * WPT)];
+#pragma unroll
+            for (int s = 0; s < per; ++s) {
+                const int net = t - f * s;
+                const uint32_t y = net >= 0 ? (w << (net & 31)) : (w >> ((-net) & 31));
+                e[per * j + s] |= y & (field_mask(f) << t);
+            }
+        }
+        idx += f * WPT;
+    }
+}
+
+// Sum of the four bytes of every dword of an expanded word-set (values fed unsigned, before
+// any kFlip inversion).
+ABQ_HD int expanded_byte_sum(const uint32_t (&e)[8])
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    uint32_t s = 0;
+#pragma unroll
+    for (int d = 0; d < 8; ++d)
+        s = __builtin_amdgcn_sad_u8(e[d], 0u, s); // sum of |byte - 0| over the four bytes
+    return (int)s;
+#else
+    int s = 0;
+    for (int d = 0; d < 8; ++d)
+        s += (int)((e[d] & 0xFFu) + ((e[d] >> 8) & 0xFFu) + ((e[d] >> 16) & 0xFFu) + (e[d] >> 24));
+    return s;
+#endif
+}
+
 // Eight consecutive K elements (low 8 bits of each used) -> eight plane bytes.
 // Byte b of the result is the 8-bit slice of plane b covering these elements, first
 // element at the byte's bit 7 (the plane words are MSB first).

@@ -7,17 +7,19 @@
 //
 // Why a second layout.  In the reference layout a K tile of 128 elements is 16 bytes per
 // (row, plane) and rows are K/8 bytes apart, so a workgroup tile touches one 128-byte cache line
-// per 16 useful bytes; with hundreds of rows per tile the vector L1 fill rate, not the matrix
-// cores, bounds the kernel.  The K-tiled layout keeps the same bits in the order
-//     tiled[kt][row][plane][4 words],  kt = K tile of 128 elements,
-// so the rows of a tile are contiguous (bits*16 bytes each) and every line is used in full.
-// Weights are converted once (they are static), activations once per call; see
-// relayout_planes_kernel below.
+// per 16 useful bytes; and turning plane words into int8 costs a bit-matrix transpose per 32
+// elements, paid again by every workgroup that uses the row: the vector ALUs, not the matrix
+// cores, then bound the kernel.  The K-tiled layout keeps the same number of bits as records
+//     tiled[kt][row][BITS * 4 words],  kt = K tile of 128 elements,
+// so the rows of a tile are contiguous and every line is used in full, and inside a record the
+// bits are grouped into 4-, 2- and 1-bit fields (abq_bits.h) that unpack to int8 with one or
+// two instructions per four elements.  Weights are converted once (they are static),
+// activations once per call; see relayout_planes_kernel.
 //
 // Work split.  256 threads = 2 x 2 waves; a wave owns TM x TN MFMA tiles of 32 x 32, the
-// workgroup tile is (64*TM) x (64*TN), the K tile 128.  Per K tile each thread expands TM
+// workgroup tile is (64*TM) x (64*TN), the K tile 128.  Per K tile each thread unpacks TM
 // word-sets (32 K elements each) of one activation row and TN of one weight row to int8
-// (abq_bits.h) and writes them to LDS, so every row is expanded once per workgroup and all
+// and writes them to LDS, so every row is expanded once per workgroup and all
 // threads do the same amount of work without divergence; the waves read their MFMA
 // operands with ds_read_b128 (row stride 144 bytes: conflict free).  LDS is double buffered
 // and the plane words of the next two K tiles are in flight in registers, so the expansion
@@ -38,39 +40,67 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 constexpr int kTileK = 128;        // K elements per tile
 constexpr int kLdsRow = 144;       // bytes per expanded row in LDS (128 + 16 padding)
 
-// Loads WPT consecutive plane words per plane of one row of one K tile (tiled layout).
-template <int BITS, int WPT>
-__device__ __forceinline__ void load_tile_words(uint32_t (&dst)[BITS][WPT], const uint32_t *tiled, int rows, int row,
-                                                int kt, int first_word)
+// Loads the fields of WPT consecutive word-sets of one row of one K tile (field-packed layout,
+// abq_bits.h) into dst = [4-bit field: 4*WPT words][2-bit: 2*WPT][1-bit: WPT].
+template <int N> __device__ __forceinline__ void load_words(uint32_t *dst, const uint32_t *src)
 {
-    const uint32_t *p = tiled + (((size_t)kt * rows + row) * BITS) * 4 + first_word;
+    if (N % 4 == 0) {
 #pragma unroll
-    for (int b = 0; b < BITS; ++b) {
-        if (WPT == 4) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(p + 4 * b);
-            dst[b][0] = v.x; dst[b][1 % WPT] = v.y; dst[b][2 % WPT] = v.z; dst[b][3 % WPT] = v.w;
-        } else if (WPT == 2) {
-            const uint2 v = *reinterpret_cast<const uint2 *>(p + 4 * b);
-            dst[b][0] = v.x; dst[b][1 % WPT] = v.y;
-        } else {
-            dst[b][0] = p[4 * b];
+        for (int i = 0; i < N / 4; ++i) {
+            const uint4 v = reinterpret_cast<const uint4 *>(src)[i];
+            dst[4 * i] = v.x; dst[4 * i + 1] = v.y; dst[4 * i + 2] = v.z; dst[4 * i + 3] = v.w;
         }
+    } else if (N == 2) {
+        const uint2 v = *reinterpret_cast<const uint2 *>(src);
+        dst[0] = v.x; dst[1] = v.y;
+    } else {
+        dst[0] = src[0];
+    }
+}
+
+template <int BITS, int WPT>
+__device__ __forceinline__ void load_tile_words(uint32_t (&dst)[BITS * WPT], const uint32_t *tiled, int rows, int row,
+                                                int kt, int first_ws)
+{
+    const uint32_t *rec = tiled + ((size_t)kt * rows + row) * (BITS * 4);
+    if (BITS == 8) {
+        load_words<8 * WPT>(dst, rec + 8 * first_ws);
+        return;
+    }
+    int idx = 0;
+#pragma unroll
+    for (int f = 4; f >= 1; f >>= 1) {
+        if (!(BITS & f))
+            continue;
+        if (f == 4)
+            load_words<4 * WPT>(dst + idx, rec + field_word_offset(BITS, 4) + 4 * first_ws);
+        else if (f == 2)
+            load_words<2 * WPT>(dst + idx, rec + field_word_offset(BITS, 2) + 2 * first_ws);
+        else
+            load_words<WPT>(dst + idx, rec + field_word_offset(BITS, 1) + first_ws);
+        idx += f * WPT;
     }
 }
 
 // Expands WPT word-sets (32 K elements each) of one row and writes the int8 values to LDS.
+// SUM (unsigned operands only) also accumulates the sum of the values.
 template <int BITS, int WPT, Int8Mode MODE, bool SUM>
-__device__ __forceinline__ void expand_words_to_lds(const uint32_t (&raw)[BITS][WPT], unsigned char *lds, int &value_sum)
+__device__ __forceinline__ void expand_words_to_lds(const uint32_t (&raw)[BITS * WPT], unsigned char *lds, int &value_sum)
 {
 #pragma unroll
     for (int ws = 0; ws < WPT; ++ws) {
-        uint32_t w[BITS], o[8];
+        uint32_t o[8];
+        if (SUM) {
+            expand_fields<BITS, WPT, kLow>(raw, ws, o);
+            value_sum += expanded_byte_sum(o);
+            if (MODE == kFlip) {
 #pragma unroll
-        for (int b = 0; b < BITS; ++b)
-            w[b] = raw[b][ws];
-        if (SUM)
-            value_sum += planes_value_sum<BITS>(w);
-        planes_to_int8<BITS, MODE>(w, o);
+                for (int d = 0; d < 8; ++d)
+                    o[d] ^= 0x80808080u;
+            }
+        } else {
+            expand_fields<BITS, WPT, MODE>(raw, ws, o);
+        }
         uint4 *dst = reinterpret_cast<uint4 *>(lds + ws * 32);
         dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
         dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
@@ -83,7 +113,7 @@ __device__ __forceinline__ void expand_words_to_lds(const uint32_t (&raw)[BITS][
 // (semantics: algorithm/quantize/quantizer.py:111-179 of the reference, scales per row of W
 // after reshaping to [-1, group_size]).  Not available for 8-bit unsigned operands.
 template <int Q, int P, bool SIGNED, int TM, int TN, bool GROUPED>
-__global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt,
+__global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt,
                                                         int m_blocks, int n_blocks_per_xcd)
 {
     constexpr int BM = 64 * TM, BN = 64 * TN;
@@ -127,7 +157,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_tiled(const GemmArgs a, const u
     unsigned char *lds_a = smem + la * kLdsRow + fa * 32;
     unsigned char *lds_b = smem + (BM + lb) * kLdsRow + fb * 32;
 
-    uint32_t rx0[Q][WA], rx1[Q][WA], rw0[P][WB], rw1[P][WB]; // plane words of the next two K tiles
+    uint32_t rx0[Q * WA], rx1[Q * WA], rw0[P * WB], rw1[P * WB]; // field words of the next two K tiles
     int sum_a = 0, sum_b = 0;
 
     v16i acc[TM][TN];

@@ -103,35 +103,48 @@ __global__ __launch_bounds__(256) void pack_u4_kernel(const uint4 *__restrict__ 
     }
 }
 
-// planes[b][row][KW] -> tiled[kt][row][b][4]; one workgroup moves 32 rows x 8 K tiles through
-// LDS so that both the reads (128 contiguous bytes per row and plane) and the writes
-// (32 * bits * 16 contiguous bytes per K tile) are coalesced.
-__global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__restrict__ planes,
-                                                              uint32_t *__restrict__ tiled, int rows, int KW, int bits)
+// planes[b][row][KW] -> field-packed K tiles tiled[kt][row][bits * 4 words] (abq_bits.h).  One
+// thread converts one word-set (32 elements of one row): reads of a plane row are contiguous
+// across the threads, the four word-sets of a record are written side by side per field.
+template <int BITS>
+__device__ __forceinline__ void store_fields(uint32_t *rec, int ws, const uint32_t (&f)[BITS])
 {
-    __shared__ uint4 buf[8][32][9]; // [kt][row][plane], one spare column against bank conflicts
-    const int tid = threadIdx.x;
-    const int kt_tiles = KW / 4;
-    const int row0 = blockIdx.x * 32, kt0 = blockIdx.y * 8;
-    const size_t plane_stride = (size_t)rows * KW;
-    {
-        const int i = tid >> 3, j = tid & 7; // row, K tile: 8 threads read 128 contiguous bytes
-        const int row = row0 + i, kt = kt0 + j;
-        if (row < rows && kt < kt_tiles) {
-            const uint32_t *p = planes + (size_t)row * KW + 4 * kt;
-            for (int b = 0; b < bits; ++b)
-                buf[j][i][b] = *reinterpret_cast<const uint4 *>(p + b * plane_stride);
-        }
+    if (BITS == 8) {
+        uint4 *dst = reinterpret_cast<uint4 *>(rec + 8 * ws);
+        dst[0] = make_uint4(f[0], f[1 % BITS], f[2 % BITS], f[3 % BITS]);
+        dst[1] = make_uint4(f[4 % BITS], f[5 % BITS], f[6 % BITS], f[7 % BITS]);
+        return;
     }
-    __syncthreads();
-    const int nrow = min(32, rows - row0);
-    for (int j = 0; j < 8; ++j) {
-        const int kt = kt0 + j;
-        if (kt >= kt_tiles)
-            break;
-        uint4 *dst = reinterpret_cast<uint4 *>(tiled) + ((size_t)kt * rows + row0) * bits;
-        for (int u = tid; u < nrow * bits; u += 256) // u = row * bits + plane: contiguous in memory
-            dst[u] = buf[j][u / bits][u % bits];
+    int idx = 0;
+#pragma unroll
+    for (int w = 4; w >= 1; w >>= 1) {
+        if (!(BITS & w))
+            continue;
+        uint32_t *dst = rec + field_word_offset(BITS, w) + w * ws;
+        if (w == 4)
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(f[idx % BITS], f[(idx + 1) % BITS], f[(idx + 2) % BITS], f[(idx + 3) % BITS]);
+        else if (w == 2)
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(f[idx % BITS], f[(idx + 1) % BITS]);
+        else
+            dst[0] = f[idx % BITS];
+        idx += w;
+    }
+}
+
+template <int BITS>
+__global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__restrict__ planes,
+                                                              uint32_t *__restrict__ tiled, int rows, int KW)
+{
+    const size_t total = (size_t)rows * KW;
+    for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (size_t)gridDim.x * 256) {
+        const int row = (int)(t / KW), w = (int)(t % KW);
+        uint32_t pw[BITS], e[8], f[BITS];
+#pragma unroll
+        for (int b = 0; b < BITS; ++b)
+            pw[b] = planes[(size_t)b * total + t];
+        planes_to_int8<BITS, kLow>(pw, e);
+        compress_fields<BITS>(e, f);
+        store_fields<BITS>(tiled + ((size_t)(w >> 2) * rows + row) * (BITS * 4), w & 3, f);
     }
 }
 
@@ -139,9 +152,44 @@ hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int r
                                   hipStream_t stream)
 {
     const int KW = k / 32;
-    const dim3 grid((rows + 31) / 32, (KW / 4 + 7) / 8);
-    hipLaunchKernelGGL(relayout_planes_kernel, grid, dim3(256), 0, stream, planes, tiled, rows, KW, bits);
+    size_t blocks = ((size_t)rows * KW + 255) / 256;
+    if (blocks > 256 * 32)
+        blocks = 256 * 32;
+    const dim3 grid((unsigned)blocks);
+    switch (bits) {
+#define ABQ_RELAYOUT_CASE(B)                                                                                     \
+    case B:                                                                                                      \
+        hipLaunchKernelGGL(relayout_planes_kernel<B>, grid, dim3(256), 0, stream, planes, tiled, rows, KW);      \
+        break;
+        ABQ_RELAYOUT_CASE(1) ABQ_RELAYOUT_CASE(2) ABQ_RELAYOUT_CASE(3) ABQ_RELAYOUT_CASE(4)
+        ABQ_RELAYOUT_CASE(5) ABQ_RELAYOUT_CASE(6) ABQ_RELAYOUT_CASE(7) ABQ_RELAYOUT_CASE(8)
+#undef ABQ_RELAYOUT_CASE
+    default:
+        return hipErrorInvalidValue;
+    }
     return hipGetLastError();
+}
+
+// compress_fields + store_fields for a run-time bit width
+template <int BITS> __device__ __forceinline__ void store_fields_of(uint32_t *rec, int ws, const uint32_t (&e)[8])
+{
+    uint32_t f[BITS];
+    compress_fields<BITS>(e, f);
+    store_fields<BITS>(rec, ws, f);
+}
+
+__device__ __forceinline__ void store_fields_any(uint32_t *rec, int ws, const uint32_t (&e)[8], int bits)
+{
+    switch (bits) {
+    case 1: store_fields_of<1>(rec, ws, e); break;
+    case 2: store_fields_of<2>(rec, ws, e); break;
+    case 3: store_fields_of<3>(rec, ws, e); break;
+    case 4: store_fields_of<4>(rec, ws, e); break;
+    case 5: store_fields_of<5>(rec, ws, e); break;
+    case 6: store_fields_of<6>(rec, ws, e); break;
+    case 7: store_fields_of<7>(rec, ws, e); break;
+    default: store_fields_of<8>(rec, ws, e); break;
+    }
 }
 
 // ---- per-token dynamic quantisation fused with packing ------------------------------------
@@ -249,15 +297,24 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
             if (active && (u % lanes_per_group) == 0)
                 group_sums[(size_t)row * (K / group_size) + u / lanes_per_group] = sum;
         }
-        const uint64_t bytes = eight_values_to_plane_bytes(v);
-        const int quad_lane = u & 3, w = u >> 2; // w: plane word within the row
-        for (int b = 0; b < bits; ++b) {
-            uint32_t word = (uint32_t)((bytes >> (8 * b)) & 0xFFu) << (24 - 8 * quad_lane);
-            word = quad_or(word);
-            if (active && quad_lane == 0) {
-                const size_t idx = TILED ? ((((size_t)(w >> 2) * M + row) * bits + b) * 4 + (w & 3))
-                                         : ((size_t)b * M + row) * KW + w;
-                planes[idx] = word;
+        const int quad_lane = u & 3, w = u >> 2; // w: word-set (32 elements) within the row
+        if (TILED) {
+            // expanded dword s, byte c = element 31 - (8c + s) of the word-set: this lane's element
+            // 7 - s goes to byte 3 - quad_lane
+            const uint32_t pattern_mask = (1u << bits) - 1u;
+            uint32_t e[8];
+#pragma unroll
+            for (int s = 0; s < 8; ++s)
+                e[s] = quad_or(((uint32_t)v[7 - s] & pattern_mask) << (24 - 8 * quad_lane));
+            if (active && quad_lane == 0)
+                store_fields_any(planes + ((size_t)(w >> 2) * M + row) * (bits * 4), w & 3, e, bits);
+        } else {
+            const uint64_t bytes = eight_values_to_plane_bytes(v);
+            for (int b = 0; b < bits; ++b) {
+                uint32_t word = (uint32_t)((bytes >> (8 * b)) & 0xFFu) << (24 - 8 * quad_lane);
+                word = quad_or(word);
+                if (active && quad_lane == 0)
+                    planes[((size_t)b * M + row) * KW + w] = word;
             }
         }
     }

@@ -21,7 +21,49 @@ template <int BITS> static void expand(int mode, const uint32_t *w, uint32_t *ou
         out[i] = o[i];
 }
 
+// one word-set through the field-packed route: planes -> expanded (low) bytes -> fields -> int8
+template <int BITS> static void via_fields(int mode, const uint32_t *w, uint32_t *fields, uint32_t *o, int *sum)
+{
+    uint32_t a[BITS], e[8], f[BITS], r[8];
+    for (int i = 0; i < BITS; ++i)
+        a[i] = w[i];
+    planes_to_int8<BITS, kLow>(a, e);
+    compress_fields<BITS>(e, f);
+    for (int i = 0; i < BITS; ++i)
+        fields[i] = f[i];
+    if (mode == kTop)
+        expand_fields<BITS, 1, kTop>(f, 0, r);
+    else if (mode == kLow)
+        expand_fields<BITS, 1, kLow>(f, 0, r);
+    else
+        expand_fields<BITS, 1, kFlip>(f, 0, r);
+    for (int i = 0; i < 8; ++i)
+        o[i] = r[i];
+    uint32_t plain[8];
+    expand_fields<BITS, 1, kLow>(f, 0, plain);
+    *sum = expanded_byte_sum(plain);
+}
+
 extern "C" {
+
+// words: [n][bits] plane words; fields: [n][bits] field words; out: [n][8] dwords; sums: [n]
+void shim_via_fields(int bits, int mode, const uint32_t *words, uint32_t *fields, uint32_t *out, int *sums, long n)
+{
+    for (long i = 0; i < n; ++i) {
+        const uint32_t *w = words + i * bits;
+        uint32_t *f = fields + i * bits, *o = out + i * 8;
+        switch (bits) {
+        case 1: via_fields<1>(mode, w, f, o, sums + i); break;
+        case 2: via_fields<2>(mode, w, f, o, sums + i); break;
+        case 3: via_fields<3>(mode, w, f, o, sums + i); break;
+        case 4: via_fields<4>(mode, w, f, o, sums + i); break;
+        case 5: via_fields<5>(mode, w, f, o, sums + i); break;
+        case 6: via_fields<6>(mode, w, f, o, sums + i); break;
+        case 7: via_fields<7>(mode, w, f, o, sums + i); break;
+        case 8: via_fields<8>(mode, w, f, o, sums + i); break;
+        }
+    }
+}
 
 // words: [n][bits] plane words of n 32-groups; out: [n][8] dwords = 32 int8 each
 void shim_planes_to_int8(int bits, int mode, const uint32_t *words, uint32_t *out, long n)

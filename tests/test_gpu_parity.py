@@ -82,13 +82,47 @@ def test_pack_f16_all_finite_bit_patterns(abq, oracle, scale):
         assert np.array_equal(got & mask, want & mask)
 
 
-def test_relayout_planes_matches_closed_form(abq):
+def field_packed(patterns, bits):
+    """The K-tiled, field-packed layout written out from its definition: patterns [rows, K] are the
+    elements' bit patterns (low `bits` bits).  A row's K tile of 128 elements is one record of
+    bits*4 words.  Inside a 32-element word-set, "expanded" dword s, byte c is element
+    31 - (8c + s).  8 bits: the expanded dwords themselves.  Otherwise one field per set bit f of
+    `bits` (4, then 2, then 1), covering value bits [bits & (f-1), +f), starting at word
+    4 * (bits & ~(2f-1)) of the record with f words per word-set: word j, byte c, bits
+    [f*s, f*s+f) = field of the element at expanded dword (8/f)*j + s, byte c."""
+    rows, K = patterns.shape
+    kt = K // 128
+    v = patterns.astype(np.uint32).reshape(rows, kt, 4, 32)
+    s_idx, c_idx = np.meshgrid(np.arange(8), np.arange(4), indexing="ij")
+    E = v[..., 31 - (8 * c_idx + s_idx)]  # [rows, kt, ws, s, c]
+    rec = np.zeros((kt, rows, bits * 4), dtype=np.uint32)
+    shifts8 = (8 * np.arange(4)).astype(np.uint32)
+    if bits == 8:
+        words = (E << shifts8).sum(axis=-1, dtype=np.uint32)  # [rows, kt, ws, s]
+        rec[:] = words.reshape(rows, kt, 32).transpose(1, 0, 2)
+        return rec
+    for f in (4, 2, 1):
+        if not bits & f:
+            continue
+        base, off, per = bits & (f - 1), 4 * (bits & ~(2 * f - 1)), 8 // f
+        fv = (E >> np.uint32(base)) & np.uint32((1 << f) - 1)
+        for ws in range(4):
+            for j in range(f):
+                word = np.zeros((rows, kt), dtype=np.uint32)
+                for s in range(per):
+                    word |= (fv[:, :, ws, per * j + s, :] << (shifts8 + np.uint32(f * s))).sum(axis=-1, dtype=np.uint32)
+                rec[:, :, off + f * ws + j] = word.T
+    return rec
+
+
+def test_relayout_planes_matches_closed_form(abq, oracle):
     rng = np.random.default_rng(12)
-    for bits, rows, k in [(2, 1, 128), (8, 37, 1152), (4, 300, 4096), (3, 64, 13824)]:
+    for bits, rows, k in [(2, 1, 128), (8, 37, 1152), (4, 300, 4096), (3, 64, 13824), (1, 5, 256), (5, 33, 384),
+                          (6, 130, 512), (7, 9, 640)]:
         planes = rng.integers(0, 1 << 32, size=(bits, rows, k // 32), dtype=np.uint64).astype(np.uint32)
         got = abq.relayout_planes(planes_dev(planes)).cpu().numpy().view(np.uint32)
-        want = planes.reshape(bits, rows, k // 128, 4).transpose(2, 1, 0, 3)  # tiled[kt, r, b, :] = planes[b, r, 4kt:4kt+4]
-        assert np.array_equal(got, want)
+        want = field_packed(oracle.unpack(planes, False), bits)
+        assert np.array_equal(got.reshape(want.shape), want), (bits, rows, k)
 
 
 def test_tiled_kernels_with_prepared_operands(abq, oracle):

@@ -24,6 +24,7 @@ def shim(tmp_path_factory):
                            os.path.join(HERE, "host_shim.cpp"), "-o", out])
     L = ctypes.CDLL(out)
     L.shim_planes_to_int8.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long]
+    L.shim_via_fields.argtypes = [ctypes.c_int, ctypes.c_int] + [ctypes.c_void_p] * 4 + [ctypes.c_long]
     L.shim_eight_values_to_plane_bytes.argtypes = [ctypes.c_void_p]
     L.shim_eight_values_to_plane_bytes.restype = ctypes.c_uint64
     L.shim_nibble_word_plane_byte.argtypes = [ctypes.c_uint32, ctypes.c_int]
@@ -43,6 +44,30 @@ def expand(shim, planes, mode):
 def rand_vals(rng, rows, k, bits, signed):
     lo, hi = (-(1 << (bits - 1)), (1 << (bits - 1)) - 1) if signed else (0, (1 << bits) - 1)
     return rng.integers(lo, hi + 1, size=(rows, k), dtype=np.int32)
+
+
+@pytest.mark.parametrize("bits", range(1, 9))
+def test_field_packed_route_equals_plane_route(shim, oracle, bits):
+    """planes -> fields -> int8 gives the same bytes as planes -> int8, for every placement mode,
+    and the field words hold exactly the bits of the values (a field word is a permutation of them)."""
+    rng = np.random.default_rng(100 + bits)
+    planes = rng.integers(0, 1 << 32, size=(bits, 6, 16), dtype=np.uint64).astype(np.uint32)
+    words = np.ascontiguousarray(planes.transpose(1, 2, 0))
+    n = 6 * 16
+    for mode in (0, 1, 2):
+        if mode == 2 and bits != 8:
+            continue
+        fields = np.zeros((n, bits), dtype=np.uint32)
+        out = np.zeros((n, 8), dtype=np.uint32)
+        sums = np.zeros(n, dtype=np.int32)
+        shim.shim_via_fields(bits, mode, words.ctypes.data, fields.ctypes.data, out.ctypes.data, sums.ctypes.data, n)
+        want = np.zeros((n, 8), dtype=np.uint32)
+        shim.shim_planes_to_int8(bits, mode, words.ctypes.data, want.ctypes.data, n)
+        assert np.array_equal(out, want)
+        vals = oracle.unpack(planes, False).reshape(n, 32)
+        assert np.array_equal(sums, vals.sum(axis=1))
+        popc = lambda a: np.unpackbits(a.view(np.uint8)).reshape(n, -1).sum(axis=1)
+        assert np.array_equal(popc(fields), popc(np.ascontiguousarray(words.reshape(n, bits))))
 
 
 @pytest.mark.parametrize("bits", range(1, 9))
