@@ -138,8 +138,9 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
     const int wid = tid >> 6;
     const int wm = wid >> 1, wn = wid & 1;
     const int r = lane & 31, g = lane >> 5;
-    const int M = a.M, N = a.N;
-    const int ktiles = a.K / kTileK;
+    // scalar copies of the shape: every branch on them below is a scalar branch
+    const int M = __builtin_amdgcn_readfirstlane(a.M), N = __builtin_amdgcn_readfirstlane(a.N);
+    const int ktiles = __builtin_amdgcn_readfirstlane(a.K) / kTileK;
 
     // workgroup -> tile: XCD x = id % 8 owns n blocks [x * npx, (x+1) * npx), M fastest
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
@@ -182,21 +183,32 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
     for (int j = 0; j < TN; ++j)
         wsc[j] = GROUPED ? a.w_scale + (size_t)min(n0 + wn * 32 * TN + j * 32 + r, N - 1) * groups : nullptr;
 
-#define ABQ_LOAD_TILE(KT, RX, RW)                                   \
-    if ((KT) < ktiles) {                                            \
-        load_tile_words<Q, WA>(RX, xt, M, ga, (KT), fa);            \
-        load_tile_words<P, WB>(RW, wt, N, gb, (KT), fb);            \
+    // Tiles past the end are clamped to the last one instead of branching: the loop body stays one
+    // basic block, so the scheduler can weave loads, unpacking and MFMAs; the duplicate tile lands
+    // in the LDS buffer nobody reads again, and its row sums are masked out.
+#define ABQ_LOAD_TILE(KT, RX, RW)                                                    \
+    {                                                                                \
+        const int kt_ld = min((KT), ktiles - 1);                                     \
+        load_tile_words<Q, WA>(RX, xt, M, ga, kt_ld, fa);                            \
+        load_tile_words<P, WB>(RW, wt, N, gb, kt_ld, fb);                            \
     }
-#define ABQ_EXPAND_TILE(RX, RW, BUF)                                                                  \
-    expand_words_to_lds<Q, WA, XMODE, NEED_SX>(RX, lds_a + (BUF) * BUF_BYTES, sum_a);                 \
-    expand_words_to_lds<P, WB, WMODE, NEED_SW>(RW, lds_b + (BUF) * BUF_BYTES, sum_b);
+#define ABQ_EXPAND_TILE(RX, RW, BUF, LIVE)                                                            \
+    {                                                                                                 \
+        int part_a = 0, part_b = 0;                                                                   \
+        expand_words_to_lds<Q, WA, XMODE, NEED_SX>(RX, lds_a + (BUF) * BUF_BYTES, part_a);            \
+        expand_words_to_lds<P, WB, WMODE, NEED_SW>(RW, lds_b + (BUF) * BUF_BYTES, part_b);            \
+        if (NEED_SX)                                                                                  \
+            sum_a += (LIVE) ? part_a : 0;                                                             \
+        if (NEED_SW)                                                                                  \
+            sum_b += (LIVE) ? part_b : 0;                                                             \
+    }
 
     ABQ_LOAD_TILE(0, rx0, rw0)
     ABQ_LOAD_TILE(1, rx1, rw1)
     if (NEED_SX || NEED_SW)
         for (int i = tid; i < BM + BN; i += 256)
             rowsum[i] = 0;
-    ABQ_EXPAND_TILE(rx0, rw0, 0)
+    ABQ_EXPAND_TILE(rx0, rw0, 0, true)
     __syncthreads();
 
     const unsigned char *a_lane = smem + (wm * 32 * TM + r) * kLdsRow + g * 16;
@@ -237,9 +249,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
                         }                                                                              \
             }                                                                                          \
         }                                                                                              \
-        if ((KT) + 1 < ktiles) {                                                                       \
-            ABQ_EXPAND_TILE(RXN, RWN, (BUF) ^ 1)                                                       \
-        }                                                                                              \
+        ABQ_EXPAND_TILE(RXN, RWN, (BUF) ^ 1, (KT) + 1 < ktiles)                                        \
         __syncthreads();                                                                               \
     }
 
@@ -303,6 +313,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
     }
 
     const int k_fed = ktiles * kTileK;
+    const StoreOperands so = store_operands(a);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -334,7 +345,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
                         v -= 16384u * (unsigned)k_fed;
                 }
                 if (m < M && n < N)
-                    store_result_compact(a, m, n, (int)v);
+                    store_result_compact(so, m, n, (int)v);
             }
         }
     }

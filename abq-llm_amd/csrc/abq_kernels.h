@@ -75,19 +75,44 @@ __device__ __forceinline__ void store_result(const GemmArgs &a, int m, int n, in
     }
 }
 
-// Out-of-line copy for kernels whose epilogue stores hundreds of elements per lane: keeps the
-// unrolled epilogue small (the int32 store is inlined, the fp16 variants are a call).
-__device__ __attribute__((noinline)) static void store_result_call(const GemmArgs &a, int m, int n, int acc)
+// Out-of-line fp16 store for kernels whose epilogue stores hundreds of elements per lane: keeps
+// the unrolled epilogue small (the int32 store is inlined, the fp16 variants are a call).  The
+// operands travel by value so that the kernel's argument block never has its address taken
+// (which would push every later read of it through memory).
+struct StoreOperands {
+    void *D;
+    const void *C;
+    const float *x_scale;
+    const float *w_scale;
+    int N;
+    int out_kind;
+};
+
+__device__ __forceinline__ StoreOperands store_operands(const GemmArgs &a)
 {
+    return StoreOperands{ a.D, a.C, a.x_scale, a.w_scale, a.N, a.out_kind };
+}
+
+__device__ __attribute__((noinline)) static void store_result_call(void *D, const void *C, const float *x_scale,
+                                                                   const float *w_scale, int N, int out_kind, int m,
+                                                                   int n, int acc)
+{
+    GemmArgs a;
+    a.D = D;
+    a.C = C;
+    a.x_scale = x_scale;
+    a.w_scale = w_scale;
+    a.N = N;
+    a.out_kind = out_kind;
     store_result(a, m, n, acc);
 }
 
-__device__ __forceinline__ void store_result_compact(const GemmArgs &a, int m, int n, int acc)
+__device__ __forceinline__ void store_result_compact(const StoreOperands &o, int m, int n, int acc)
 {
-    if (a.out_kind == 0)
-        reinterpret_cast<int *>(a.D)[(size_t)m * a.N + n] = acc;
+    if (o.out_kind == 0)
+        reinterpret_cast<int *>(o.D)[(size_t)m * o.N + n] = acc;
     else
-        store_result_call(a, m, n, acc);
+        store_result_call(o.D, o.C, o.x_scale, o.w_scale, o.N, o.out_kind, m, n, acc);
 }
 
 } // namespace abq

@@ -35,6 +35,15 @@ Q_BITS, P_BITS, SIGNED = 8, 2, True
 ROTATE_BYTES = 512 << 20
 
 
+# HBM bytes per launch of the dominant kernel, averaged over this workload's nine GEMMs, from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled by a plain copy of known size
+# (summary with the commands: profiles/decode_w2a8_bench_hbm_traffic.md).  Reported only for the
+# kernel it was measured on.
+MEASURED_TRAFFIC_BYTES = {
+    "decode:AqBMMA_8x2xtrue_16x16x8192_16x16x512_16x16x64_3": 9358234,
+}
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -66,6 +75,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="plain stream launches instead of HIP graphs")
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill side measurements")
+    ap.add_argument("--pmc-copy-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB (the known-size kernel that "
+                         "calibrates FETCH_SIZE / WRITE_SIZE in a counter run)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "
@@ -127,6 +139,14 @@ def main():
             log("HIP graph capture failed (%r); falling back to plain stream launches" % (e,))
             use_graph, graphs = False, []
             torch.cuda.synchronize()
+
+    if args.pmc_copy_mib:
+        src = torch.empty(args.pmc_copy_mib << 20, dtype=torch.uint8, device="cuda").random_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---------------------------------------------------------------- warmup
     for case in cases:
@@ -244,13 +264,14 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int32 accumulate over 1-bit planes (int8 MFMA / VALU popcount)",
+        "dtype": "int8",  # bit planes unpacked to int8, int8 MFMA with int32 accumulation
         "data": "synthetic",
         "config": {"workload": "BASELINE configs[1]: W2A8 signed decode GEMM, M in {1,4,8} x (N,K) in "
                                "{(4096,4096),(11008,4096),(4096,11008)}, int32 out, packed operands resident in HBM",
                    "gemms_per_step": len(cases), "x_bits": Q_BITS, "w_bits": P_BITS, "signed": SIGNED},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dominant,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(dominant), "kernel": dominant,
                      "launches_per_step": dg["launches"],
                      "algorithmic_bytes_per_launch_avg": round(dg["bytes"] / dg["launches"]),
                      "avg_launch_us": round(dg["us"] / dg["launches"], 3)},
