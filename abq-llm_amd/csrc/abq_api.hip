@@ -102,7 +102,7 @@ static void entry_to_config(const KernelEntry &e, int strategy, int x_bits, int 
         c->mma_k = 128;
         c->nstage = 1;
     } else {
-        const int stepk = e.nstage == 4 ? 128 : (64 / e.mi) * 4 * 32; // NSTAGE 4: K-tiled layout, 128-element K tiles
+        const int stepk = e.nstage == 4 ? e.kb : (64 / e.mi) * 4 * 32; // NSTAGE 4: K-tiled layout, 128- or 64-element stages
         c->block_m = e.mi * e.tm * e.wm;
         c->block_n = e.mi * e.tn * e.wn;
         c->block_k = stepk * e.wk;
@@ -216,7 +216,7 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
             lpr_log2 = lpr == 16 ? 4 : lpr == 32 ? 5 : 6;
     } else {
         mi = cfg->mma_m;
-        const int stepk = (strategy == ABQ_STRATEGY_MFMA32 && cfg->nstage == 4) ? 128 : (64 / mi) * 4 * 32;
+        const int stepk = (strategy == ABQ_STRATEGY_MFMA32 && cfg->nstage == 4) ? cfg->warp_k : (64 / mi) * 4 * 32;
         if (cfg->warp_m <= 0 || cfg->warp_n <= 0 || cfg->warp_m % mi || cfg->warp_n % mi ||
             cfg->block_m % cfg->warp_m || cfg->block_n % cfg->warp_n || cfg->warp_k != stepk ||
             cfg->block_k % stepk)
@@ -232,25 +232,27 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
 
     if (strategy == ABQ_STRATEGY_TILED) {
         const KernelTable *tt_ = find_table(reg.tiled, x_bits, w_bits, is_signed);
-        if (!tt_ || mi != 32 || wm != 2 || wn != 2 || wk != 1)
+        if (!tt_ || mi != 32 || wk != 1)
             return ABQ_ERR_UNSUPPORTED;
         int v = -1;
-        for (int i = 0; i < tt_->count; ++i)
-            if (tt_->entries[i].tm == tm && tt_->entries[i].tn == tn)
+        for (int i = 0; i < tt_->count; ++i) {
+            const KernelEntry &t = tt_->entries[i];
+            if (t.tm == tm && t.tn == tn && t.wm == wm && t.wn == wn && t.kb == cfg->warp_k)
                 v = i;
+        }
         if (v < 0)
             return ABQ_ERR_UNSUPPORTED;
         if (K >= (1 << 17))
             return ABQ_ERR_TOO_LARGE;
         const KernelEntry &e = tt_->entries[v];
-        const int bm = 64 * e.tm, bn = 64 * e.tn;
+        const int bm = 32 * e.tm * e.wm, bn = 32 * e.tn * e.wn;
         const int mblocks = (M + bm - 1) / bm, npx = ((N + bn - 1) / bn + 7) / 8;
         st->strategy = strategy;
         st->variant = v;
         entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
         st->grid_dim = abq_dim3{ (unsigned)(8 * npx * mblocks), 1, 1 };
-        st->block_dim = abq_dim3{ 256, 1, 1 };
-        st->shared_mem_size = 2 * (size_t)(bm + bn) * 144 + (bm + bn) * 4;
+        st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
+        st->shared_mem_size = 2 * (size_t)(bm + bn) * (e.kb + 16) + (bm + bn) * 4;
         return ABQ_OK;
     }
 
@@ -533,9 +535,8 @@ abq_status abq_gemm_init(const abq_tile_config *cfg, int x_bits, int w_bits, int
 static size_t planes_bytes(int rows, int k, int bits) { return (size_t)bits * rows * (k / 32) * 4; }
 
 // Picks the tiled-kernel tile for a shape.  Measured on MI355X (W4A4 / W8A8 / W2A8, LLaMA shapes):
-// 128x128 is the fastest tile whenever it yields at least one workgroup per compute unit
-// (larger tiles lose to register pressure in the compiled inner loop, smaller ones to LDS
-// traffic); below that, smaller tiles win by filling the chip.
+// the 256x128 tile of eight waves (least L2 -> L1 traffic per MFMA) is the fastest once it yields
+// one workgroup per compute unit, then 128x128; below that, smaller tiles win by filling the chip.
 static abq_status switch_to_tiled(abq_gemm_state *st)
 {
     const Registry &reg = registry();
@@ -543,12 +544,15 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
     const KernelTable *tt = find_table(reg.tiled, c.x_bits, c.w_bits, c.is_signed);
     if (!tt)
         return ABQ_ERR_UNSUPPORTED;
-    static const int order[][2] = { { 2, 2 }, { 2, 1 }, { 1, 1 } };
+    // candidates in order of preference: { TM, TN, waves along M, waves along N, workgroups needed }
+    static const int order[][5] = { { 2, 2, 4, 2, 250 }, { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 200 }, { 1, 1, 2, 2, 0 } };
     int pick = -1;
     for (const auto &o : order) {
-        const long tiles = (long)((st->M + 64 * o[0] - 1) / (64 * o[0])) * ((st->N + 64 * o[1] - 1) / (64 * o[1]));
+        const int bm = 32 * o[0] * o[2], bn = 32 * o[1] * o[3];
+        const long tiles = (long)((st->M + bm - 1) / bm) * ((st->N + bn - 1) / bn);
         for (int i = 0; i < tt->count; ++i)
-            if (tt->entries[i].tm == o[0] && tt->entries[i].tn == o[1] && (tiles >= 200 || (o[0] == 1 && o[1] == 1)) && pick < 0)
+            if (tt->entries[i].tm == o[0] && tt->entries[i].tn == o[1] && tt->entries[i].kb == 128 &&
+                tt->entries[i].wm == o[2] && tt->entries[i].wn == o[3] && tiles >= o[4] && pick < 0)
                 pick = i;
     }
     if (pick < 0)
@@ -598,9 +602,17 @@ abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, cons
             // no group-scale build of this tile: fall back to the smallest one when the library chose
             if (!state->auto_chosen)
                 return ABQ_ERR_UNSUPPORTED;
+            // largest group-scale tile that still yields a workgroup per compute unit
             pick = tg->count - 1;
-            entry_to_config(tg->entries[pick], ABQ_STRATEGY_TILED, c.x_bits, c.w_bits, c.is_signed, 0, &state->cfg);
+            for (int i = tg->count - 1; i >= 0; --i) {
+                const int bm = tg->entries[i].mi * tg->entries[i].tm * tg->entries[i].wm;
+                const int bn = tg->entries[i].mi * tg->entries[i].tn * tg->entries[i].wn;
+                if ((long)((state->M + bm - 1) / bm) * ((state->N + bn - 1) / bn) >= 200)
+                    pick = i;
+            }
         }
+        const int xb_ = c.x_bits, wb_ = c.w_bits, sg_ = c.is_signed;
+        entry_to_config(tg->entries[pick], ABQ_STRATEGY_TILED, xb_, wb_, sg_, 0, &state->cfg);
         state->variant = pick;
     } else if (state->group_size != 0) {
         return ABQ_ERR_INVALID_ARG; // a state switched to group scales stays there

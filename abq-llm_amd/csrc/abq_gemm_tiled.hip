@@ -112,22 +112,34 @@ __device__ __forceinline__ void expand_words_to_lds(const uint32_t (&raw)[BITS *
 // and are folded into fp32 accumulators with the group's scale at every group boundary
 // (semantics: algorithm/quantize/quantizer.py:111-179 of the reference, scales per row of W
 // after reshaping to [-1, group_size]).  Not available for 8-bit unsigned operands.
-template <int Q, int P, bool SIGNED, int TM, int TN, bool GROUPED>
-__global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt,
-                                                        int m_blocks, int n_blocks_per_xcd)
+//
+// KB: K elements per LDS stage, 128 (a whole record) or 64 (half a record: half the LDS per
+// stage, so that the 128 x 256 tile still fits two workgroups per compute unit).
+//
+// WM x WN: waves per workgroup along M and N (2 x 2, or 4 x 2 / 4 x 4 for the large tiles that
+// cut the L2 -> L1 traffic per MFMA).
+template <int Q, int P, bool SIGNED, int TM, int TN, bool GROUPED, int KB, int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN, (WM * WN > 4 ? 1 : (TM * TN <= 4 || KB == 64 ? 2 : 1)))
+void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, int m_blocks, int n_blocks_per_xcd)
 {
-    constexpr int BM = 64 * TM, BN = 64 * TN;
+    constexpr int NT = 64 * WM * WN; // threads
+    constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
+    constexpr int WSETS = KB / 32;          // word-sets of a row per stage
+    constexpr int SPR = kTileK / KB;        // stages per record
+    constexpr int LDS_ROW = KB + 16;        // bytes per expanded row in LDS: ds_read_b128 conflict free
+    static_assert(KB == 128 || KB == 64, "a stage is a record or half of one");
+    static_assert(!GROUPED || KB == 128, "group scales are folded per 128-element stage");
     // every thread expands WA word-sets of one activation row and WB word-sets of one weight row
-    // per K tile (a row has 4 word-sets): uniform work, no divergence
-    constexpr int WA = BM / 64, WB = BN / 64;
-    constexpr int TPRA = 4 / WA, TPRB = 4 / WB; // threads per row
-    static_assert(WA == 1 || WA == 2 || WA == 4, "BM in {64, 128, 256}");
-    static_assert(WB == 1 || WB == 2 || WB == 4, "BN in {64, 128, 256}");
+    // per stage: uniform work, no divergence
+    constexpr int WA = BM * WSETS / NT, WB = BN * WSETS / NT;
+    constexpr int TPRA = WSETS / WA, TPRB = WSETS / WB; // threads per row
+    static_assert(WA == 1 || WA == 2 || WA == 4, "BM * KB / 8192 in {1, 2, 4}");
+    static_assert(WB == 1 || WB == 2 || WB == 4, "BN * KB / 8192 in {1, 2, 4}");
     constexpr Int8Mode XMODE = Int8ModeOf<Q, SIGNED>::value;
     constexpr Int8Mode WMODE = Int8ModeOf<P, SIGNED>::value;
     constexpr bool NEED_SX = WMODE == kFlip; // see abq_gemm_mfma.hip
     constexpr bool NEED_SW = XMODE == kFlip;
-    constexpr int BUF_BYTES = (BM + BN) * kLdsRow;
+    constexpr int BUF_BYTES = (BM + BN) * LDS_ROW;
 
     extern __shared__ __align__(16) unsigned char smem[];
     // [2][BM + BN][144] expanded rows, then row sums [BM + BN]
@@ -136,11 +148,11 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wid = tid >> 6;
-    const int wm = wid >> 1, wn = wid & 1;
+    const int wm = wid / WN, wn = wid % WN;
     const int r = lane & 31, g = lane >> 5;
     // scalar copies of the shape: every branch on them below is a scalar branch
     const int M = __builtin_amdgcn_readfirstlane(a.M), N = __builtin_amdgcn_readfirstlane(a.N);
-    const int ktiles = __builtin_amdgcn_readfirstlane(a.K) / kTileK;
+    const int ktiles = __builtin_amdgcn_readfirstlane(a.K) / KB; // stages
 
     // workgroup -> tile: XCD x = id % 8 owns n blocks [x * npx, (x+1) * npx), M fastest
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
@@ -155,8 +167,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
     const int la = tid / TPRA, fa = (tid % TPRA) * WA; // tile row, first word-set
     const int lb = tid / TPRB, fb = (tid % TPRB) * WB;
     const int ga = min(m0 + la, M - 1), gb = min(n0 + lb, N - 1);
-    unsigned char *lds_a = smem + la * kLdsRow + fa * 32;
-    unsigned char *lds_b = smem + (BM + lb) * kLdsRow + fb * 32;
+    unsigned char *lds_a = smem + la * LDS_ROW + fa * 32;
+    unsigned char *lds_b = smem + (BM + lb) * LDS_ROW + fb * 32;
 
     uint32_t rx0[Q * WA], rx1[Q * WA], rw0[P * WB], rw1[P * WB]; // field words of the next two K tiles
     int sum_a = 0, sum_b = 0;
@@ -189,8 +201,8 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
 #define ABQ_LOAD_TILE(KT, RX, RW)                                                    \
     {                                                                                \
         const int kt_ld = min((KT), ktiles - 1);                                     \
-        load_tile_words<Q, WA>(RX, xt, M, ga, kt_ld, fa);                            \
-        load_tile_words<P, WB>(RW, wt, N, gb, kt_ld, fb);                            \
+        load_tile_words<Q, WA>(RX, xt, M, ga, kt_ld / SPR, (kt_ld % SPR) * WSETS + fa); \
+        load_tile_words<P, WB>(RW, wt, N, gb, kt_ld / SPR, (kt_ld % SPR) * WSETS + fb); \
     }
 #define ABQ_EXPAND_TILE(RX, RW, BUF, LIVE)                                                            \
     {                                                                                                 \
@@ -206,13 +218,13 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
     ABQ_LOAD_TILE(0, rx0, rw0)
     ABQ_LOAD_TILE(1, rx1, rw1)
     if (NEED_SX || NEED_SW)
-        for (int i = tid; i < BM + BN; i += 256)
+        for (int i = tid; i < BM + BN; i += NT)
             rowsum[i] = 0;
     ABQ_EXPAND_TILE(rx0, rw0, 0, true)
     __syncthreads();
 
-    const unsigned char *a_lane = smem + (wm * 32 * TM + r) * kLdsRow + g * 16;
-    const unsigned char *b_lane = smem + (BM + wn * 32 * TN + r) * kLdsRow + g * 16;
+    const unsigned char *a_lane = smem + (wm * 32 * TM + r) * LDS_ROW + g * 16;
+    const unsigned char *b_lane = smem + (BM + wn * 32 * TN + r) * LDS_ROW + g * 16;
 
     // One K tile: MFMAs on LDS buffer BUF (tile kt), loads of tile kt+2 into the register slot
     // tile kt used, expansion of tile kt+1 (other register slot) into the other LDS buffer.
@@ -229,13 +241,13 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
         }                                                                                              \
         const unsigned char *ab = a_lane + (BUF) * BUF_BYTES;                                          \
         const unsigned char *bb = b_lane + (BUF) * BUF_BYTES;                                          \
-        _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                               \
+        _Pragma("unroll") for (int ks = 0; ks < WSETS; ++ks)                                           \
         {                                                                                              \
             v4i av[TM], bv[TN];                                                                        \
             _Pragma("unroll") for (int i = 0; i < TM; ++i)                                             \
-                av[i] = *reinterpret_cast<const v4i *>(ab + i * 32 * kLdsRow + ks * 32);               \
+                av[i] = *reinterpret_cast<const v4i *>(ab + i * 32 * LDS_ROW + ks * 32);               \
             _Pragma("unroll") for (int j = 0; j < TN; ++j)                                             \
-                bv[j] = *reinterpret_cast<const v4i *>(bb + j * 32 * kLdsRow + ks * 32);               \
+                bv[j] = *reinterpret_cast<const v4i *>(bb + j * 32 * LDS_ROW + ks * 32);               \
             _Pragma("unroll") for (int i = 0; i < TM; ++i)                                             \
                 _Pragma("unroll") for (int j = 0; j < TN; ++j)                                         \
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j], acc[i][j], 0, 0, 0); \
@@ -279,12 +291,12 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
         static_assert(GC * (BM + BN) * 4 <= 2 * BUF_BYTES, "staging fits the tile buffers");
         for (int g0 = 0; g0 < groups; g0 += GC) {
             __syncthreads();
-            for (int u = tid; u < GC * BM; u += 256) {
+            for (int u = tid; u < GC * BM; u += NT) {
                 const int rr = u / GC, gl = u % GC;
                 const int m = min(m0 + rr, M - 1);
                 zs_x[gl * BM + rr] = g0 + gl < groups ? (float)a.x_group_sums[(size_t)m * groups + g0 + gl] : 0.f;
             }
-            for (int u = tid; u < GC * BN; u += 256) {
+            for (int u = tid; u < GC * BN; u += NT) {
                 const int rr = u / GC, gl = u % GC;
                 const size_t idx = (size_t)min(n0 + rr, N - 1) * groups + g0 + gl;
                 zs_w[gl * BN + rr] = g0 + gl < groups ? a.w_scale[idx] * a.w_zero[idx] : 0.f;
@@ -312,7 +324,7 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
         }
     }
 
-    const int k_fed = ktiles * kTileK;
+    const int k_fed = ktiles * KB;
     const StoreOperands so = store_operands(a);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -351,22 +363,22 @@ __global__ __launch_bounds__(256, (TM * TN <= 4 ? 2 : 1)) void gemm_mfma_tiled(c
     }
 }
 
-template <int Q, int P, bool SIGNED, int TM, int TN, bool GROUPED>
+template <int Q, int P, bool SIGNED, int TM, int TN, bool GROUPED, int KB, int WM = 2, int WN = 2>
 static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 {
-    constexpr int BM = 64 * TM, BN = 64 * TN;
+    constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
     if (GROUPED && (Int8ModeOf<Q, SIGNED>::value == kFlip || Int8ModeOf<P, SIGNED>::value == kFlip))
         return hipErrorInvalidValue; // group scales with 8-bit unsigned operands: not built
     const int m_blocks = (a.M + BM - 1) / BM, n_blocks = (a.N + BN - 1) / BN;
     const int npx = (n_blocks + 7) / 8;
-    const size_t lds = 2 * (size_t)(BM + BN) * kLdsRow + (BM + BN) * sizeof(int);
+    const size_t lds = 2 * (size_t)(BM + BN) * (KB + 16) + (BM + BN) * sizeof(int);
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&gemm_mfma_tiled<Q, P, SIGNED, TM, TN, GROUPED>),
+        reinterpret_cast<const void *>(&gemm_mfma_tiled<Q, P, SIGNED, TM, TN, GROUPED, KB, WM, WN>),
         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess)
         return attr;
     const dim3 grid(8 * npx * m_blocks);
-    hipLaunchKernelGGL((gemm_mfma_tiled<Q, P, SIGNED, TM, TN, GROUPED>), grid, dim3(256), lds, stream, a, a.X, a.W, m_blocks, npx);
+    hipLaunchKernelGGL((gemm_mfma_tiled<Q, P, SIGNED, TM, TN, GROUPED, KB, WM, WN>), grid, dim3(64 * WM * WN), lds, stream, a, a.X, a.W, m_blocks, npx);
     return hipGetLastError();
 }
 
@@ -374,15 +386,23 @@ static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 // operand layout.  The group-scale variants sit in a table of their own and exist for the tiles
 // the default choice uses.
 #define ABQ_TILED_VARIANTS(V) V(4, 4) V(2, 4) V(2, 2) V(2, 1) V(1, 1)
+#define ABQ_TILED_HALF_VARIANTS(V) V(2, 4) V(2, 2)   // K stage of 64
+#define ABQ_TILED_WIDE_VARIANTS(V) V(2, 2, 4, 2) V(2, 2, 4, 4)   // TM, TN, waves along M, N
 #define ABQ_GROUPED_VARIANTS(V) V(2, 2) V(1, 1)
 
-#define ABQ_ENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, false> },
-#define ABQ_ENTRY_F(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN, false> },
-#define ABQ_GENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, true> },
-#define ABQ_GENTRY_F(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN, true> },
+#define ABQ_ENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, false, 128>, 128 },
+#define ABQ_ENTRY_F(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN, false, 128>, 128 },
+#define ABQ_HENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, false, 64>, 64 },
+#define ABQ_HENTRY_F(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN, false, 64>, 64 },
+#define ABQ_WENTRY_T(TM, TN, WM, WN) { 32, TM, TN, WM, WN, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, false, 128, WM, WN>, 128 },
+#define ABQ_WENTRY_F(TM, TN, WM, WN) { 32, TM, TN, WM, WN, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN, false, 128, WM, WN>, 128 },
+#define ABQ_GENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, true, 128>, 128 },
+#define ABQ_GENTRY_F(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN, true, 128>, 128 },
 
-static const KernelEntry kSigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_T) };
-static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) };
+static const KernelEntry kSigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_T) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_T)
+                                       ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_T) };
+static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
+                                         ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_F) };
 static const KernelEntry kSignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_T) };
 static const KernelEntry kUnsignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_F) };
 

@@ -36,6 +36,7 @@ struct KernelEntry {
     int wm, wn, wk;         // waves per workgroup along M, N, K
     int nstage;
     GemmLauncher launch;
+    int kb;                 // K elements per LDS stage (tiled kernel); 0 where it does not apply
 };
 
 struct KernelTable {
