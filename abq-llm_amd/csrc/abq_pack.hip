@@ -103,9 +103,8 @@ __global__ __launch_bounds__(256) void pack_u4_kernel(const uint4 *__restrict__ 
     }
 }
 
-// planes[b][row][KW] -> field-packed K tiles tiled[kt][row][bits * 4 words] (abq_bits.h).  One
-// thread converts one word-set (32 elements of one row): reads of a plane row are contiguous
-// across the threads, the four word-sets of a record are written side by side per field.
+// planes[b][row][KW] -> field-packed K tiles tiled[kt][row][bits * 4 words] (abq_bits.h).
+// store_fields puts the field words of word-set `ws` into the record at `rec`.
 template <int BITS>
 __device__ __forceinline__ void store_fields(uint32_t *rec, int ws, const uint32_t (&f)[BITS])
 {
@@ -131,20 +130,52 @@ __device__ __forceinline__ void store_fields(uint32_t *rec, int ws, const uint32
     }
 }
 
+// One workgroup converts 32 rows x 8 K tiles.  A thread owns one record (one row, one K tile): it
+// reads 16 bytes per plane (eight threads cover 128 contiguous bytes of a plane row), converts its
+// four word-sets in registers, and parks the record in LDS; the records of one K tile are then
+// contiguous in memory over the 32 rows and leave with coalesced 16-byte stores.
 template <int BITS>
 __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__restrict__ planes,
                                                               uint32_t *__restrict__ tiled, int rows, int KW)
 {
-    const size_t total = (size_t)rows * KW;
-    for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (size_t)gridDim.x * 256) {
-        const int row = (int)(t / KW), w = (int)(t % KW);
-        uint32_t pw[BITS], e[8], f[BITS];
+    constexpr int REC = BITS * 4;          // words per record
+    constexpr int SLAB = 32 * REC + 4;     // words per K tile in LDS (+16 bytes against bank conflicts)
+    __shared__ __align__(16) uint32_t buf[8 * SLAB];
+    const int tid = threadIdx.x;
+    const int kt_tiles = KW / 4;
+    const int row0 = blockIdx.x * 32, kt0 = blockIdx.y * 8;
+    const size_t plane_stride = (size_t)rows * KW;
+    {
+        const int i = tid >> 3, j = tid & 7;
+        const int row = row0 + i, kt = kt0 + j;
+        if (row < rows && kt < kt_tiles) {
+            uint32_t pw[4][BITS]; // [word-set][plane]
+            const uint32_t *p = planes + (size_t)row * KW + 4 * kt;
 #pragma unroll
-        for (int b = 0; b < BITS; ++b)
-            pw[b] = planes[(size_t)b * total + t];
-        planes_to_int8<BITS, kLow>(pw, e);
-        compress_fields<BITS>(e, f);
-        store_fields<BITS>(tiled + ((size_t)(w >> 2) * rows + row) * (BITS * 4), w & 3, f);
+            for (int b = 0; b < BITS; ++b) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(p + b * plane_stride);
+                pw[0][b] = v.x; pw[1][b] = v.y; pw[2][b] = v.z; pw[3][b] = v.w;
+            }
+            uint32_t *rec = buf + j * SLAB + i * REC;
+#pragma unroll
+            for (int ws = 0; ws < 4; ++ws) {
+                uint32_t e[8], f[BITS];
+                planes_to_int8<BITS, kLow>(pw[ws], e);
+                compress_fields<BITS>(e, f);
+                store_fields<BITS>(rec, ws, f);
+            }
+        }
+    }
+    __syncthreads();
+    const int nrow = min(32, rows - row0);
+    for (int j = 0; j < 8; ++j) {
+        const int kt = kt0 + j;
+        if (kt >= kt_tiles)
+            break;
+        uint4 *dst = reinterpret_cast<uint4 *>(tiled + ((size_t)kt * rows + row0) * REC);
+        const uint4 *src = reinterpret_cast<const uint4 *>(buf + j * SLAB);
+        for (int u = tid; u < nrow * BITS; u += 256)
+            dst[u] = src[u];
     }
 }
 
@@ -152,10 +183,7 @@ hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int r
                                   hipStream_t stream)
 {
     const int KW = k / 32;
-    size_t blocks = ((size_t)rows * KW + 255) / 256;
-    if (blocks > 256 * 32)
-        blocks = 256 * 32;
-    const dim3 grid((unsigned)blocks);
+    const dim3 grid((rows + 31) / 32, (KW / 4 + 7) / 8);
     switch (bits) {
 #define ABQ_RELAYOUT_CASE(B)                                                                                     \
     case B:                                                                                                      \
