@@ -248,6 +248,39 @@ def main():
                     del gm, xpl, ws
                 del wpl, wtl
         extra["prefill"] = prefill
+
+        # ------------------------------------------------------------ side measurement: several linears per launch
+        # QKV (N = 3 * 4096) and gate + up (N = 2 * 11008) share their activations, so each is one GEMM
+        # over concatenated weight planes: the launch + ramp cost is paid once for 12 or 22 MB.
+        fused = []
+        for name, N, K in (("qkv", 3 * 4096, 4096), ("gate_up", 2 * 11008, 4096)):
+            wbytes = P_BITS * N * K // 8
+            Wr = random_planes(torch, (max(2, math.ceil(ROTATE_BYTES / wbytes)), P_BITS, N, K // 32))
+            for M in MS:
+                out = torch.empty((M, N), dtype=torch.int32, device="cuda")
+                gs = [abq.Gemm(xs[(M, K)], Wr[r], SIGNED, out=out) for r in range(Wr.shape[0])]
+                for r in range(4):
+                    gs[r % len(gs)].run()
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr):
+                    for r in range(100):
+                        gs[r % len(gs)].run()
+                gr.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                gr.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / 100
+                gbs = algorithmic_bytes(M, N, K, Q_BITS, P_BITS) / (us * 1e-6) / 1e9
+                fused.append(dict(linears=name, M=M, N=N, K=K, us=round(us, 3), hbm_gbs=round(gbs, 1),
+                                  hbm_frac=round(gbs / HBM_PEAK_GBS, 4), kernel="%s:%s" % (gs[0].strategy, gs[0].config_name)))
+                log("fused %s M=%d N=%d K=%d  %.2f us  %.0f GB/s (%.1f%% of HBM peak)" % (name, M, N, K, us, gbs, 100 * gbs / HBM_PEAK_GBS))
+                del gr, gs, out
+            del Wr
+        extra["decode_fused_linears"] = fused
         for r in prefill:
             log("prefill W%dA%d %s M=%d N=%d K=%d  %.1f us  %.1f TOPS (%.1f%% of int8 MFMA peak)"
                 % (r["w_bits"], r["x_bits"], "int" if r["signed"] else "uint", r["M"], r["N"], r["K"], r["us"],

@@ -17,6 +17,7 @@
 #include "mma_any/aq_wmma_library.h"
 #include "wmma_any/wmma_any.h"
 #include "abq_gemm_wrapper.h"
+#include "abq_weight_file.h"
 #include "abq_oracle.h"
 
 // reference (tensor-core) tuples, declared here the way a user of the reference would
@@ -265,6 +266,70 @@ static void gpu_paths()
         HIP_OK(hipFree(d_wscale));
         HIP_OK(hipFree(d_wzero));
         HIP_OK(hipFree(d_term));
+        HIP_OK(hipFree(d_ws));
+    }
+
+    {   // weight file -> device weight -> dynamic GEMM: the file round-trips, and the GEMM on the loaded
+        // weight equals a double-precision loop over the blob's own dequantised codes
+        const int M = 24, N = 160, K = 384, G = 64, groups = K / G;
+        std::mt19937 r32(11);
+        std::normal_distribution<float> nd(0.f, 0.05f), xd_(0.f, 1.f);
+        std::vector<float> wf((size_t)N * K);
+        for (auto &v : wf)
+            v = nd(r32);
+        ABQWeightBlob blob, back;
+        std::string err;
+        CHECK(abq_quantize_weights(wf.data(), N, K, 4, false, G, &blob, &err));
+        const std::string path = "/tmp/abq_test_weight.abqw";
+        CHECK(abq_weight_file_write(path, blob, &err));
+        CHECK(abq_weight_file_read(path, &back, &err));
+        CHECK(back.planes == blob.planes && back.scale == blob.scale && back.zero == blob.zero &&
+              std::memcmp(&back.info, &blob.info, sizeof(blob.info)) == 0);
+        CHECK(!abq_weight_file_read("/tmp/abq_no_such_file.abqw", &back, &err));
+        std::remove(path.c_str());
+        ABQDeviceWeight dw;
+        CHECK(dw.load(blob, stream, &err));
+        std::vector<int> codes((size_t)N * K);
+        abq_oracle_unpack(blob.planes.data(), codes.data(), N, K, 4, 1);
+        std::vector<uint16_t> ha((size_t)M * K);
+        for (auto &h : ha)
+            h = abq_oracle_f32_to_f16(xd_(r32));
+        ABQGEMMWrapper wrap(8, 4, true);
+        const size_t ws_bytes = wrap.dynamic_workspace_bytes(M, K, G);
+        _Float16 *d_a, *d_d;
+        char *d_ws;
+        HIP_OK(hipMalloc(&d_a, ha.size() * 2));
+        HIP_OK(hipMalloc(&d_d, (size_t)M * N * 2));
+        HIP_OK(hipMalloc(&d_ws, ws_bytes));
+        HIP_OK(hipMemcpy(d_a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
+        wrap.gemm_dynamic(M, N, K, d_a, dw.grouped(), d_d, true, d_ws, ws_bytes, stream);
+        HIP_OK(hipStreamSynchronize(stream));
+        std::vector<uint16_t> got((size_t)M * N);
+        HIP_OK(hipMemcpy(got.data(), d_d, got.size() * 2, hipMemcpyDeviceToHost));
+        double worst = 0, ref_sq = 0;
+        std::vector<double> want((size_t)M * N);
+        for (int m = 0; m < M; ++m) {
+            float amax = 0.f;
+            for (int k = 0; k < K; ++k)
+                amax = std::fmax(amax, std::fabs(abq_oracle_f16_to_f32(ha[(size_t)m * K + k])));
+            const float scale = std::fmin(std::fmax(amax / 127.f, 1e-5f), 1e4f);
+            for (int n = 0; n < N; ++n) {
+                double acc = 0;
+                for (int k = 0; k < K; ++k) {
+                    const float code = std::fmin(std::fmax(std::nearbyint(abq_oracle_f16_to_f32(ha[(size_t)m * K + k]) / scale), -128.f), 127.f);
+                    acc += (double)code * scale * ((double)codes[(size_t)n * K + k] - blob.zero[(size_t)n * groups + k / G]) *
+                           blob.scale[(size_t)n * groups + k / G];
+                }
+                want[(size_t)m * N + n] = acc;
+                ref_sq += acc * acc;
+            }
+        }
+        const double rms = std::sqrt(ref_sq / want.size());
+        for (size_t i = 0; i < want.size(); ++i)
+            worst = std::fmax(worst, std::fabs((double)abq_oracle_f16_to_f32(got[i]) - want[i]) / (std::fabs(want[i]) + rms));
+        CHECK(worst <= 1e-2);
+        HIP_OK(hipFree(d_a));
+        HIP_OK(hipFree(d_d));
         HIP_OK(hipFree(d_ws));
     }
 
