@@ -30,6 +30,7 @@ hipError_t launch_weight_zero_term(const uint32_t *, int, int, int, int, const f
     void abq_mfma_register_##Q##_##P(KernelTable *);  \
     void abq_bcnt_register_##Q##_##P(KernelTable *);  \
     void abq_decode_register_##Q##_##P(KernelTable *); \
+    void abq_decode_grouped_register_##Q##_##P(KernelTable *); \
     void abq_tiled_register_##Q##_##P(KernelTable *);  \
     void abq_tiled_grouped_register_##Q##_##P(KernelTable *);
 ABQ_FOR_EACH_COMBO(ABQ_DECL)
@@ -39,6 +40,7 @@ struct Registry {
     KernelTable mfma[2 * ABQ_NUM_COMBOS];
     KernelTable bcnt[2 * ABQ_NUM_COMBOS];
     KernelTable decode[2 * ABQ_NUM_COMBOS];
+    KernelTable decode_grouped[2 * ABQ_NUM_COMBOS];
     KernelTable tiled[2 * ABQ_NUM_COMBOS];
     KernelTable tiled_grouped[2 * ABQ_NUM_COMBOS];
     Registry()
@@ -48,6 +50,7 @@ struct Registry {
     abq_mfma_register_##Q##_##P(&mfma[i]);             \
     abq_bcnt_register_##Q##_##P(&bcnt[i]);             \
     abq_decode_register_##Q##_##P(&decode[i]);         \
+    abq_decode_grouped_register_##Q##_##P(&decode_grouped[i]); \
     abq_tiled_register_##Q##_##P(&tiled[i]);           \
     abq_tiled_grouped_register_##Q##_##P(&tiled_grouped[i]); \
     i += 2;
@@ -567,6 +570,44 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
     return ABQ_OK;
 }
 
+// Moves a state with group scales onto the tiled kernel's group-scale variants.
+static abq_status pick_grouped_tiled(abq_gemm_state *state)
+{
+    if (state->strategy != ABQ_STRATEGY_TILED) {
+        if (!state->auto_chosen)
+            return ABQ_ERR_UNSUPPORTED;
+        const abq_status rc = switch_to_tiled(state);
+        if (rc != ABQ_OK)
+            return rc;
+    }
+    const abq_tile_config &c = state->cfg;
+    const KernelTable *tg = find_table(registry().tiled_grouped, c.x_bits, c.w_bits, c.is_signed);
+    if (!tg)
+        return ABQ_ERR_UNSUPPORTED;
+    int pick = -1;
+    for (int i = 0; i < tg->count; ++i)
+        if (tg->entries[i].mi * tg->entries[i].tm * tg->entries[i].wm == c.block_m &&
+            tg->entries[i].mi * tg->entries[i].tn * tg->entries[i].wn == c.block_n)
+            pick = i;
+    if (pick < 0) {
+        // no group-scale build of this tile: when the library chose, take the largest group-scale
+        // tile that still yields a workgroup per compute unit
+        if (!state->auto_chosen)
+            return ABQ_ERR_UNSUPPORTED;
+        pick = tg->count - 1;
+        for (int i = tg->count - 1; i >= 0; --i) {
+            const int bm = tg->entries[i].mi * tg->entries[i].tm * tg->entries[i].wm;
+            const int bn = tg->entries[i].mi * tg->entries[i].tn * tg->entries[i].wn;
+            if ((long)((state->M + bm - 1) / bm) * ((state->N + bn - 1) / bn) >= 200)
+                pick = i;
+        }
+    }
+    const int xb_ = c.x_bits, wb_ = c.w_bits, sg_ = c.is_signed;
+    entry_to_config(tg->entries[pick], ABQ_STRATEGY_TILED, xb_, wb_, sg_, 0, &state->cfg);
+    state->variant = pick;
+    return ABQ_OK;
+}
+
 abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, const float *w_scale,
                                int group_size)
 {
@@ -575,7 +616,8 @@ abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, cons
     if (!x_scale || !w_scale)
         return ABQ_ERR_INVALID_ARG;
     if (group_size != 0) {
-        // w_scale is [N][K / group_size]: only the tiled kernel folds scales inside the K loop
+        // w_scale is [N][K / group_size]: the decode kernel with group scales for M <= 16 on plane
+        // operands, the tiled kernel otherwise; both fold the scales inside the K loop
         const abq_tile_config &c = state->cfg;
         if (group_size != 64 && group_size != 128)
             return ABQ_ERR_UNSUPPORTED;
@@ -583,37 +625,20 @@ abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, cons
             return ABQ_ERR_INVALID_ARG;
         if (!c.is_signed && (c.x_bits == 8 || c.w_bits == 8))
             return ABQ_ERR_UNSUPPORTED;
-        if (state->strategy != ABQ_STRATEGY_TILED) {
-            if (!state->auto_chosen)
-                return ABQ_ERR_UNSUPPORTED;
-            const abq_status rc = switch_to_tiled(state);
-            if (rc != ABQ_OK)
+        state->group_size = group_size;
+        const bool decode_ok = state->strategy == ABQ_STRATEGY_DECODE && state->auto_chosen && state->M <= 16 &&
+                               state->x_layout == ABQ_LAYOUT_PLANES && state->w_layout == ABQ_LAYOUT_PLANES &&
+                               decode_grouped_lds(state->M, state->K, group_size) != 0 &&
+                               find_table(registry().decode_grouped, c.x_bits, c.w_bits, c.is_signed);
+        if (decode_ok) {
+            state->variant = 0;
+        } else {
+            const abq_status rc = pick_grouped_tiled(state);
+            if (rc != ABQ_OK) {
+                state->group_size = 0;
                 return rc;
-        }
-        const KernelTable *tg = find_table(registry().tiled_grouped, c.x_bits, c.w_bits, c.is_signed);
-        if (!tg)
-            return ABQ_ERR_UNSUPPORTED;
-        int pick = -1;
-        for (int i = 0; i < tg->count; ++i)
-            if (tg->entries[i].mi * tg->entries[i].tm * tg->entries[i].wm == c.block_m &&
-                tg->entries[i].mi * tg->entries[i].tn * tg->entries[i].wn == c.block_n)
-                pick = i;
-        if (pick < 0) {
-            // no group-scale build of this tile: fall back to the smallest one when the library chose
-            if (!state->auto_chosen)
-                return ABQ_ERR_UNSUPPORTED;
-            // largest group-scale tile that still yields a workgroup per compute unit
-            pick = tg->count - 1;
-            for (int i = tg->count - 1; i >= 0; --i) {
-                const int bm = tg->entries[i].mi * tg->entries[i].tm * tg->entries[i].wm;
-                const int bn = tg->entries[i].mi * tg->entries[i].tn * tg->entries[i].wn;
-                if ((long)((state->M + bm - 1) / bm) * ((state->N + bn - 1) / bn) >= 200)
-                    pick = i;
             }
         }
-        const int xb_ = c.x_bits, wb_ = c.w_bits, sg_ = c.is_signed;
-        entry_to_config(tg->entries[pick], ABQ_STRATEGY_TILED, xb_, wb_, sg_, 0, &state->cfg);
-        state->variant = pick;
     } else if (state->group_size != 0) {
         return ABQ_ERR_INVALID_ARG; // a state switched to group scales stays there
     }
@@ -725,8 +750,10 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
             return ABQ_ERR_NOT_INITIALIZED;
         e = t->entries[st->variant].launch(a, (hipStream_t)stream);
     } else {
+        if (st->group_size && st->strategy != ABQ_STRATEGY_DECODE)
+            return ABQ_ERR_NOT_INITIALIZED; // group scales live on the decode and tiled kernels only
         const KernelTable *tables = st->strategy == ABQ_STRATEGY_BCNT     ? reg.bcnt
-                                    : st->strategy == ABQ_STRATEGY_DECODE ? reg.decode
+                                    : st->strategy == ABQ_STRATEGY_DECODE ? (st->group_size ? reg.decode_grouped : reg.decode)
                                                                           : reg.mfma;
         const KernelTable *t = find_table(tables, c.x_bits, c.w_bits, c.is_signed);
         if (!t || st->variant < 0 || st->variant >= t->count)
@@ -771,7 +798,7 @@ abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_l
     if ((x_layout == ABQ_LAYOUT_TILED || w_layout == ABQ_LAYOUT_TILED) && st->strategy != ABQ_STRATEGY_TILED) {
         if (!st->auto_chosen)
             return ABQ_ERR_UNSUPPORTED;
-        const abq_status rc = switch_to_tiled(st);
+        const abq_status rc = st->group_size ? pick_grouped_tiled(st) : switch_to_tiled(st);
         if (rc != ABQ_OK)
             return rc;
     }

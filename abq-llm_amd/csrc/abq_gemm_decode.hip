@@ -376,6 +376,224 @@ static hipError_t launch_mfma_decode(const GemmArgs &a, hipStream_t stream)
     return hipGetLastError();
 }
 
+// ---- decode with group-wise weight scales ----------------------------------------------------
+//
+// D[m][n] = x_scale[m] * ( sum_g w_scale[n][g] * (acc_g - w_zero[n][g] * Sx[m][g]) - x_zero[m] * T[n] ),
+// acc_g the integer dot product over scale group g (64 or 128 elements along K); semantics of
+// algorithm/quantize/quantizer.py:111-179 of the reference, fp16 output.
+//
+// Same plan as above: activations expanded once per workgroup into LDS, weights read once with
+// 16-byte loads and fed to v_mfma_i32_16x16x64_i8 as the B operand, work items = (tile, 512-K
+// step).  In a step lane group g = lane / 16 holds the 128-element block 4*step + g of its weight
+// row, and an MFMA sums over the four lane groups, i.e. over four scale groups.  To keep them
+// apart the step is run four times with the A operand of all but one lane group read from a
+// page of zeros: 32 MFMAs per step instead of 8, which a bandwidth-bound kernel can afford.
+// For groups of 64 the two halves of a block (plane words 0-1 and 2-3) go to separate
+// accumulators.  The block sums are folded into fp32 with their scales; the waves' partial
+// tiles meet in LDS in a fixed order (deterministic sums), tiles_per_pass tiles at a time.
+template <int Q, int P, bool SIGNED>
+__global__ __launch_bounds__(64 * kDecodeGroupedWaves) void gemm_decode_grouped(const GemmArgs a, int tiles_per_wg,
+                                                                                int tiles_per_pass)
+{
+    constexpr int NW = kDecodeGroupedWaves, NT = 64 * NW;
+    constexpr Int8Mode XMODE = Int8ModeOf<Q, SIGNED>::value;
+    constexpr Int8Mode WMODE = Int8ModeOf<P, SIGNED>::value;
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    float *part = reinterpret_cast<float *>(smem);              // [tiles_per_pass][NW][16][16] per-wave partial tiles
+    float *sxg = part + tiles_per_pass * NW * 256;              // [16][groups] activation group sums
+    const int M = a.M, N = a.N, KW = a.KW;
+    const int groups = a.K / a.group_size;
+    const bool g64 = a.group_size == 64;
+    const int blocks = KW / 4;                                  // 128-element blocks of K
+    const int steps = (KW + 15) >> 4;                           // 512-element steps, the last one may be partial
+    unsigned char *zero_page = reinterpret_cast<unsigned char *>(sxg + 16 * groups); // 128 bytes
+    unsigned char *xs = zero_page + 128;                        // [Mb][RS]
+    const int RS = steps * 512 + 16;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int m0 = blockIdx.y * 16;
+    const int Mb = min(16, M - m0);
+    const size_t xplane = (size_t)M * KW, wplane = (size_t)N * KW;
+    const int ntiles = (N + 15) / 16;
+    const int G = gridDim.x;
+    // tiles blockIdx.x, blockIdx.x + G, ... of this workgroup
+    const int TW = min(tiles_per_wg, (ntiles - (int)blockIdx.x + G - 1) / G);
+
+    // Work items: (tile, step) pairs, step fastest; wave w takes items w, w + NW, ... of a pass.
+    // The first item's weight words go in flight before the activation work.
+    uint4 wnext[P];
+    {
+        const int tp0 = min(tiles_per_pass, TW);
+        const int tl = wid / steps, st = wid - tl * steps;
+        load_weight_words<P>(wnext, a.W, wplane, KW, N, blockIdx.x + tl * G, r, st * 16 + 4 * g, KW, wid < tp0 * steps);
+    }
+
+    // activations -> int8 in LDS, one wave per 64 plane words of a row; the tail of a partial last
+    // step and the zero page are cleared
+    {
+        const int bpr = (KW + 63) >> 6;
+        for (int blk = wid; blk < Mb * bpr; blk += NW) {
+            const int m = blk / bpr;
+            const int kw = (blk - m * bpr) * 64 + lane;
+            if (kw < KW) {
+                uint32_t xw[Q], o[8];
+                const uint32_t *xp = a.X + (size_t)(m0 + m) * KW + kw;
+#pragma unroll
+                for (int b = 0; b < Q; ++b) {
+                    xw[b] = *xp;
+                    xp += xplane;
+                }
+                planes_to_int8<Q, XMODE>(xw, o);
+                uint4 *dst = reinterpret_cast<uint4 *>(xs + (size_t)m * RS + kw * 32);
+                dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+                dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+            }
+        }
+        const int pad = steps * 16 - KW; // plane words
+        for (int u = tid; u < Mb * pad * 2; u += NT) {
+            const int m = u / (pad * 2), q16 = u - m * (pad * 2);
+            reinterpret_cast<uint4 *>(xs + (size_t)m * RS + KW * 32)[q16] = make_uint4(0u, 0u, 0u, 0u);
+        }
+        if (tid < 8)
+            reinterpret_cast<uint4 *>(zero_page)[tid] = make_uint4(0u, 0u, 0u, 0u);
+        for (int i = tid; i < 16 * groups; i += NT) {
+            const int m = i / groups;
+            sxg[i] = (a.w_zero && m < Mb) ? (float)a.x_group_sums[(size_t)(m0 + m) * groups + (i - m * groups)] : 0.f;
+        }
+    }
+    __syncthreads();
+
+    // the signed route feeds value * 2^(8-bits): the exact power of two that undoes it rides on the scale
+    const float unshift = SIGNED ? 1.0f / (float)(1 << (16 - Q - P)) : 1.0f;
+    const unsigned char *xrow = xs + (size_t)min(r, Mb - 1) * RS + g * 128;
+
+    for (int t0 = 0; t0 < TW; t0 += tiles_per_pass) {
+        const int tp = min(tiles_per_pass, TW - t0);
+        const int items = tp * steps;
+        // this wave's slots start at zero: it writes only the tiles it has items of
+        for (int i = lane; i < tp * 256; i += 64)
+            part[((i >> 8) * NW + wid) * 256 + (i & 255)] = 0.f;
+
+        float facc[4] = { 0.f, 0.f, 0.f, 0.f };
+        int cur_tl = -1;
+        for (int j = wid; j < items; j += NW) {
+            const int tl = j / steps, st = j - tl * steps;
+            uint4 wv[P];
+#pragma unroll
+            for (int b = 0; b < P; ++b)
+                wv[b] = wnext[b];
+            { // weight words of the wave's next item: in this pass, else the first of the next pass
+                int jn = j + NW, tbase = t0;
+                if (jn >= items) {
+                    jn = wid;
+                    tbase = t0 + tiles_per_pass;
+                }
+                const int tpn = min(tiles_per_pass, TW - tbase);
+                const int tln = jn / steps, stn = jn - tln * steps;
+                load_weight_words<P>(wnext, a.W, wplane, KW, N, blockIdx.x + (tbase + tln) * G, r, stn * 16 + 4 * g, KW,
+                                     tpn > 0 && jn < tpn * steps);
+            }
+            if (tl != cur_tl) {
+                if (cur_tl >= 0) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        part[(cur_tl * NW + wid) * 256 + (4 * g + e) * 16 + r] = facc[e];
+                }
+                facc[0] = facc[1] = facc[2] = facc[3] = 0.f;
+                cur_tl = tl;
+            }
+            v4i bops[8];
+            int unused_sum;
+            expand_weight_words<P, WMODE, false>(wv, bops, unused_sum);
+            const int n = min(((int)blockIdx.x + (t0 + tl) * G) * 16 + r, N - 1);
+            const float *wsc = a.w_scale + (size_t)n * groups;
+            const float *wzp = a.w_zero ? a.w_zero + (size_t)n * groups : nullptr;
+#pragma unroll
+            for (int gsel = 0; gsel < 4; ++gsel) {
+                const int blk = 4 * st + gsel; // the 128-element block lane group gsel holds
+                if (blk >= blocks)
+                    break; // uniform: partial last step
+                const unsigned char *xw = (g == gsel) ? xrow + st * 512 : zero_page;
+                v4i lo = { 0, 0, 0, 0 }, hi = { 0, 0, 0, 0 };
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(*reinterpret_cast<const v4i *>(xw + i * 16), bops[i], lo, 0, 0, 0);
+#pragma unroll
+                for (int i = 4; i < 8; ++i)
+                    hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(*reinterpret_cast<const v4i *>(xw + i * 16), bops[i], hi, 0, 0, 0);
+                if (!g64) {
+                    const float sw = wsc[blk];
+                    const float zs = wzp ? sw * wzp[blk] : 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        facc[e] += (sw * unshift) * (float)(lo[e] + hi[e]) - zs * sxg[(4 * g + e) * groups + blk];
+                } else {
+                    const float s0 = wsc[2 * blk], s1 = wsc[2 * blk + 1];
+                    const float z0 = wzp ? s0 * wzp[2 * blk] : 0.f, z1 = wzp ? s1 * wzp[2 * blk + 1] : 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float *sx = sxg + (4 * g + e) * groups + 2 * blk;
+                        facc[e] += (s0 * unshift) * (float)lo[e] + (s1 * unshift) * (float)hi[e] - z0 * sx[0] - z1 * sx[1];
+                    }
+                }
+            }
+        }
+        if (cur_tl >= 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                part[(cur_tl * NW + wid) * 256 + (4 * g + e) * 16 + r] = facc[e];
+        }
+        __syncthreads();
+        // output: thread (tile, row i, column c) sums the waves' partial tiles in a fixed order
+        for (int u = tid; u < tp * 256; u += NT) {
+            const int tl = u >> 8, i = (u >> 4) & 15, c = u & 15;
+            const int nn = ((int)blockIdx.x + (t0 + tl) * G) * 16 + c;
+            if (i < Mb && nn < N) {
+                float v = 0.f;
+#pragma unroll
+                for (int w2 = 0; w2 < NW; ++w2)
+                    v += part[(tl * NW + w2) * 256 + (u & 255)];
+                if (a.x_zero)
+                    v -= a.x_zero[m0 + i] * a.w_zero_term[nn];
+                reinterpret_cast<_Float16 *>(a.D)[(size_t)(m0 + i) * N + nn] = (_Float16)(v * a.x_scale[m0 + i]);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <int Q, int P, bool SIGNED>
+static hipError_t launch_decode_grouped(const GemmArgs &a, hipStream_t stream)
+{
+    if (Int8ModeOf<Q, SIGNED>::value == kFlip || Int8ModeOf<P, SIGNED>::value == kFlip)
+        return hipErrorInvalidValue;
+    const size_t base = decode_grouped_lds(a.M, a.K, a.group_size); // with one tile per pass
+    if (!base || (a.group_size != 64 && a.group_size != 128))
+        return hipErrorInvalidValue;
+    const int tiles = (a.N + 15) / 16;
+    const int gx = tiles < 256 ? tiles : 256;
+    const int tpw = (tiles + gx - 1) / gx;
+    // as many tiles per pass as the rest of the LDS holds (16 KiB of per-wave partial tiles each)
+    int tpp = 1 + (int)((160 * 1024 - base) / ((size_t)kDecodeGroupedWaves * 1024));
+    if (tpp > tpw)
+        tpp = tpw;
+    const size_t lds = base + (size_t)(tpp - 1) * kDecodeGroupedWaves * 1024;
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void *>(&gemm_decode_grouped<Q, P, SIGNED>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr != hipSuccess)
+        return attr;
+    const dim3 grid(gx, (a.M + 15) / 16);
+    hipLaunchKernelGGL((gemm_decode_grouped<Q, P, SIGNED>), grid, dim3(64 * kDecodeGroupedWaves), lds, stream, a, tpw, tpp);
+    return hipGetLastError();
+}
+
+static const KernelEntry kSignedGrouped[] = { { 16, 1, 1, 1, 1, kDecodeGroupedWaves, 3, &launch_decode_grouped<ABQ_Q, ABQ_P, true> } };
+static const KernelEntry kUnsignedGrouped[] = { { 16, 1, 1, 1, 1, kDecodeGroupedWaves, 3, &launch_decode_grouped<ABQ_Q, ABQ_P, false> } };
+
 // Native tile space of this kernel: waves per workgroup.  Entries reuse the MFMA tuple
 // (16-row tiles, K split over the waves) with nstage = 3 marking the LDS-staged activations.
 #define ABQ_DECODE_VARIANTS(V) V(4) V(8) V(16)
@@ -393,6 +611,12 @@ void ABQ_CAT(abq_decode_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)
 {
     out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSigned, (int)(sizeof(kSigned) / sizeof(kSigned[0])) };
     out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, kUnsigned, (int)(sizeof(kUnsigned) / sizeof(kUnsigned[0])) };
+}
+
+void ABQ_CAT(abq_decode_grouped_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)
+{
+    out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSignedGrouped, 1 };
+    out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, kUnsignedGrouped, 1 };
 }
 
 } // namespace abq

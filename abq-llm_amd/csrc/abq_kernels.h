@@ -50,6 +50,18 @@ const KernelTable *mfma_tables(int *count);
 const KernelTable *bcnt_tables(int *count);
 hipError_t launch_bcnt_generic(const GemmArgs &, int x_bits, int w_bits, int is_signed, hipStream_t);
 
+// Waves per workgroup of the decode kernel with group scales, and the LDS it needs (per-wave partial
+// tiles, the activation group sums, a page of zeros, the expanded activations); 0 if that exceeds a
+// compute unit's LDS.
+constexpr int kDecodeGroupedWaves = 16;
+inline size_t decode_grouped_lds(int M, int K, int group_size)
+{
+    const int mb = M < 16 ? M : 16;
+    const int row = (K + 511) / 512 * 512 + 16; // an expanded row, padded to whole 512-element steps
+    const size_t need = (size_t)kDecodeGroupedWaves * 256 * 4 + (size_t)16 * (K / group_size) * 4 + 128 + (size_t)mb * row;
+    return need <= 160 * 1024 ? need : 0;
+}
+
 // ---- output stage shared by all kernels ------------------------------------------------
 // out_kind values mirror abq_out_kind in include/abq_gemm.h.
 __device__ __forceinline__ void store_result(const GemmArgs &a, int m, int n, int acc)

@@ -110,19 +110,25 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     float *x_scale = reinterpret_cast<float *>(abq_gemm_workspace + planes_bytes);
     float *x_zero = x_scale + M;
     int32_t *sums = reinterpret_cast<int32_t *>(x_zero + M);
-    abq_status rc = abq_quant_pack_f16(A, M, K, x_bits_, x_symmetric ? 1 : 0, ABQ_LAYOUT_TILED, planes, x_scale, x_zero,
+    // at most 16 rows: decode kernel on plane operands; above: tiled kernel on the prefill layout
+    // (if the expanded activations fit the decode kernel's LDS: partial tiles, group sums, M padded rows)
+    const bool decode = M <= 16 && W.planes != nullptr &&
+                        16 * 1024 + (size_t)64 * (K / W.group_size) + 128 + (size_t)M * ((K + 511) / 512 * 512 + 16) <= 160 * 1024;
+    const int layout = decode ? ABQ_LAYOUT_PLANES : ABQ_LAYOUT_TILED;
+    abq_status rc = abq_quant_pack_f16(A, M, K, x_bits_, x_symmetric ? 1 : 0, layout, planes, x_scale, x_zero,
                                        sums, W.group_size, stream);
     if (rc != ABQ_OK) {
         printf("[ABQ][Error] pack failed: %s\n", abq_status_string(rc));
         return;
     }
     abq_gemm_state state;
-    rc = abq_gemm_init(nullptr, x_bits_, w_bits_, 1, planes, reinterpret_cast<const uint32_t *>(W.planes_tiled), M, N, K,
-                       D, nullptr, 0, ABQ_OUT_F16_SCALED, &state);
+    rc = abq_gemm_init(nullptr, x_bits_, w_bits_, 1, planes,
+                       reinterpret_cast<const uint32_t *>(decode ? W.planes : W.planes_tiled), M, N, K, D, nullptr, 0,
+                       ABQ_OUT_F16_SCALED, &state);
+    if (rc == ABQ_OK && !decode)
+        rc = abq_gemm_set_operand_layout(&state, ABQ_LAYOUT_TILED, ABQ_LAYOUT_TILED);
     if (rc == ABQ_OK)
         rc = abq_gemm_set_scales(&state, x_scale, W.scale, W.group_size);
-    if (rc == ABQ_OK)
-        rc = abq_gemm_set_operand_layout(&state, ABQ_LAYOUT_TILED, ABQ_LAYOUT_TILED);
     if (rc == ABQ_OK && (W.zero || !x_symmetric))
         rc = abq_gemm_set_zero_points(&state, x_symmetric ? nullptr : x_zero, W.zero, sums, W.zero_term);
     if (rc == ABQ_ERR_UNSUPPORTED) {

@@ -26,6 +26,8 @@ struct ABQGroupedWeight {
     const float *zero;        // [N][K/group_size] in units of (signed) weight codes, or nullptr
     const float *zero_term;   // [N] from abq_weight_zero_term; needed for asymmetric activations
     int group_size;           // 64 or 128
+    const int *planes;        // the same weights in the reference plane layout [w_bits][N][K/32], or nullptr;
+                              // with it, calls of at most 16 rows run the decode kernel
 };
 
 class ABQGEMMWrapper {

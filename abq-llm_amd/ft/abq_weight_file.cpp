@@ -193,5 +193,6 @@ bool ABQDeviceWeight::load(const ABQWeightBlob &blob, hipStream_t stream, std::s
 
 ABQGroupedWeight ABQDeviceWeight::grouped() const
 {
-    return ABQGroupedWeight{ reinterpret_cast<const int *>(tiled_), scale_, zero_, zero_term_, (int)info_.group_size };
+    return ABQGroupedWeight{ reinterpret_cast<const int *>(tiled_), scale_, zero_, zero_term_, (int)info_.group_size,
+                             reinterpret_cast<const int *>(planes_) };
 }

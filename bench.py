@@ -281,6 +281,47 @@ def main():
                 del gr, gs, out
             del Wr
         extra["decode_fused_linears"] = fused
+
+        # ------------------------------------------------------------ side measurement: decode with the dequantising epilogue
+        # group-128 weight scales and zero points, per-token scales, fp16 output (the decode kernel's
+        # group-scale variant); bytes add the scale and zero-point arrays to the packed weights
+        deq = []
+        for (N, K) in SHAPES:
+            G = K // 128
+            wbytes = P_BITS * N * K // 8
+            Wr = random_planes(torch, (max(2, math.ceil(ROTATE_BYTES / wbytes)), P_BITS, N, K // 32))
+            wsc = torch.rand((N, G), device="cuda") * 0.01 + 0.001
+            wz = torch.randint(-2, 2, (N, G), device="cuda").float()
+            for M in (1, 8):
+                xsc = torch.rand(M, device="cuda") * 0.05 + 0.01
+                sums = torch.randint(-1000, 1000, (M, G), dtype=torch.int32, device="cuda")
+                out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+                gs = [abq.Gemm(xs[(M, K)], Wr[r], SIGNED, out=out, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc,
+                               group_size=128, w_zero=wz, x_group_sums=sums) for r in range(Wr.shape[0])]
+                for r in range(4):
+                    gs[r % len(gs)].run()
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr):
+                    for r in range(100):
+                        gs[r % len(gs)].run()
+                gr.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                gr.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / 100
+                nbytes = algorithmic_bytes(M, N, K, Q_BITS, P_BITS, out_bytes=2) + 2 * N * G * 4
+                gbs = nbytes / (us * 1e-6) / 1e9
+                deq.append(dict(M=M, N=N, K=K, group_size=128, us=round(us, 3), hbm_gbs=round(gbs, 1),
+                                hbm_frac=round(gbs / HBM_PEAK_GBS, 4), kernel="%s:%s" % (gs[0].strategy, gs[0].config_name)))
+                log("dequant decode M=%d N=%d K=%d  %.2f us  %.0f GB/s (%.1f%% of HBM peak)  %s"
+                    % (M, N, K, us, gbs, 100 * gbs / HBM_PEAK_GBS, gs[0].strategy))
+                del gr, gs, out
+            del Wr
+        extra["decode_group_scales"] = deq
         for r in prefill:
             log("prefill W%dA%d %s M=%d N=%d K=%d  %.1f us  %.1f TOPS (%.1f%% of int8 MFMA peak)"
                 % (r["w_bits"], r["x_bits"], "int" if r["signed"] else "uint", r["M"], r["N"], r["K"], r["us"],

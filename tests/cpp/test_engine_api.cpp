@@ -213,7 +213,7 @@ static void gpu_paths()
         HIP_OK(hipMemcpy(d_wzero, wzero.data(), wzero.size() * 4, hipMemcpyHostToDevice));
         CHECK(abq_relayout_planes(d_wpl, d_wt, N, K, 2, stream) == ABQ_OK);
         CHECK(abq_weight_zero_term(d_wpl, N, K, 2, 1, d_wscale, d_wzero, G, d_term, stream) == ABQ_OK);
-        const ABQGroupedWeight weight = { reinterpret_cast<const int *>(d_wt), d_wscale, d_wzero, d_term, G };
+        const ABQGroupedWeight weight = { reinterpret_cast<const int *>(d_wt), d_wscale, d_wzero, d_term, G, nullptr };
         for (int symmetric = 1; symmetric >= 0; --symmetric) {
             wrap.gemm_dynamic(M, N, K, d_a, weight, d_d, symmetric != 0, d_ws, ws_bytes, stream);
             HIP_OK(hipStreamSynchronize(stream));

@@ -37,9 +37,9 @@ def assert_close_rel(got, want):
     assert np.linalg.norm(got - want) <= 2e-3 * np.linalg.norm(want)
 
 
-def run_grouped(abq, xp, wp, signed, **kw):
+def run_grouped(abq, xp, wp, signed, strategy="tiled", **kw):
     g = abq.Gemm(xp, wp, signed, out_kind=abq.OUT_F16_SCALED, **kw)
-    assert g.strategy == "tiled"
+    assert g.strategy == strategy
     if g.workspace_bytes:
         ws = torch.empty(g.workspace_bytes, dtype=torch.uint8, device="cuda")
         g = abq.Gemm(xp, wp, signed, out_kind=abq.OUT_F16_SCALED, workspace=ws, **kw)
@@ -119,6 +119,39 @@ def test_zero_point_corrections(abq, oracle, group_size, with_x_zero):
             kw.update(x_zero=fdev(xz), w_zero_term=term)
         got = run_grouped(abq, planes_dev(oracle.pack_i32(x, q)), wp, signed, **kw)
         assert_close_rel(got, want)
+
+
+@pytest.mark.parametrize("q,p,signed", [(8, 2, True), (4, 4, True), (8, 4, True), (4, 4, False), (6, 2, False)])
+@pytest.mark.parametrize("group_size", [128, 64])
+def test_decode_kernel_with_group_scales_and_zero_points(abq, oracle, q, p, signed, group_size):
+    """At most 16 activation rows on plane operands run the decode kernel's group-scale variant."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(q + 7 * p + group_size)
+    for (M, N, K, zeros) in [(1, 64, 128, 0), (5, 200, 384, 1), (16, 4096 + 8, 4096, 2), (8, 300, 11008, 2), (3, 4096, 1152, 1)]:
+        lo_x, hi_x = (-(1 << (q - 1)), 1 << (q - 1)) if signed else (0, 1 << q)
+        lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed else (0, 1 << p)
+        x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        G = K // group_size
+        xs = rng.uniform(0.01, 0.05, M)
+        wsc = rng.uniform(0.001, 0.02, (N, G))
+        wz = rng.integers(lo_w, hi_w, (N, G)).astype(np.float64) if zeros >= 1 else np.zeros((N, G))
+        xz = rng.integers(lo_x // 2, hi_x // 2, M).astype(np.float64) if zeros >= 2 else np.zeros(M)
+        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, group_size)
+        wp = planes_dev(oracle.pack_i32(w, p))
+        kw = dict(x_scale=fdev(xs), w_scale=fdev(wsc), group_size=group_size)
+        if zeros >= 1:
+            kw.update(w_zero=fdev(wz),
+                      x_group_sums=torch.from_numpy(x.reshape(M, G, group_size).sum(axis=2).astype(np.int32)).cuda())
+        if zeros >= 2:
+            kw.update(x_zero=fdev(xz), w_zero_term=abq.weight_zero_term(wp, signed, kw["w_scale"], kw["w_zero"], group_size))
+        out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        got = run_grouped(abq, planes_dev(oracle.pack_i32(x, q)), wp, signed, strategy="decode", out=out, **kw)
+        assert_close_rel(got, want)
+        # the same state moved to the tiled kernel by declaring prepared weights gives the same values
+        got2 = run_grouped(abq, planes_dev(oracle.pack_i32(x, q)), abq.relayout_planes(wp), signed, w_tiled=True, **kw)
+        assert_close_rel(got2, want)
+        assert np.abs(got.astype(np.float64) - got2.astype(np.float64)).max() <= 2e-3 * np.abs(want).max()
 
 
 def test_group_scale_argument_checks(abq, oracle):
