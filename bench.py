@@ -37,7 +37,7 @@ ROTATE_BYTES = 512 << 20
 
 # HBM bytes per launch of the dominant kernel, averaged over this workload's nine GEMMs, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled by a plain copy of known size
-# (summary with the commands: profiles/decode_w2a8_bench_hbm_traffic.md).  Reported only for the
+# (the summary with the commands is kept under profiles/, decode_w2a8_bench_hbm_traffic).  Reported only for the
 # kernel it was measured on.
 MEASURED_TRAFFIC_BYTES = {
     "decode:AqBMMA_8x2xtrue_16x16x8192_16x16x512_16x16x64_3": 9358234,
@@ -80,8 +80,8 @@ def main():
                          "calibrates FETCH_SIZE / WRITE_SIZE in a counter run)")
     args = ap.parse_args()
     if args.gpus != 1:
-        log("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "
-            "splitting N or K across GPUs, see DESIGN.md)." % args.gpus)
+        log("bench.py: this build measures one GPU; --gpus %d is not supported (the path would shard by "
+            "splitting N, or K with an integer all-reduce, across GPUs; nothing here uses a second GPU)." % args.gpus)
         sys.exit(2)
     K_STEPS, W_STEPS = args.steps, args.warmup
 
