@@ -22,6 +22,7 @@ OUT_I32, OUT_F16_TENSOR, OUT_F16_SCALED, OUT_F16_TENSOR_F32SCALE = 0, 1, 2, 3
 STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC, STRATEGY_DECODE, STRATEGY_TILED = range(7)
 STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic", "decode", "tiled"]
 LAYOUT_PLANES, LAYOUT_TILED = 0, 1
+ACT_NONE, ACT_SILU_GATE = 0, 1
 
 # every symbol include/abq_gemm.h declares
 EXPORTED = [
@@ -32,7 +33,7 @@ EXPORTED = [
     "abq_gemm_init", "abq_gemm_set_scales", "abq_gemm_exec", "abq_gemm_launch",
     "abq_planes_bytes", "abq_relayout_planes", "abq_gemm_set_operand_layout", "abq_gemm_workspace_bytes",
     "abq_gemm_set_workspace",
-    "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16",
+    "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16", "abq_gemm_set_activation",
 ]
 
 
@@ -69,6 +70,7 @@ class GemmState(ctypes.Structure):
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("x_zero", ctypes.c_void_p), ("w_zero", ctypes.c_void_p),
         ("x_group_sums", ctypes.c_void_p), ("w_zero_term", ctypes.c_void_p),
+        ("act", ctypes.c_int),
     ]
 
 
@@ -115,6 +117,7 @@ def lib():
         L.abq_gemm_workspace_bytes.restype = ctypes.c_size_t
         L.abq_gemm_set_workspace.argtypes = [ctypes.POINTER(GemmState), vp, ctypes.c_size_t]
         L.abq_gemm_set_zero_points.argtypes = [ctypes.POINTER(GemmState), vp, vp, vp, vp]
+        L.abq_gemm_set_activation.argtypes = [ctypes.POINTER(GemmState), ci]
         L.abq_weight_zero_term.argtypes = [vp, ci, ci, ci, ci, vp, vp, ci, vp, vp]
         L.abq_quant_pack_f16.argtypes = [vp, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, vp]
         _lib = L
@@ -248,7 +251,7 @@ class Gemm:
 
     def __init__(self, x_planes, w_planes, signed, out=None, cfg=None, out_kind=OUT_I32, c_scale=None,
                  x_scale=None, w_scale=None, group_size=0, x_tiled=False, w_tiled=False, workspace=None,
-                 x_zero=None, w_zero=None, x_group_sums=None, w_zero_term=None):
+                 x_zero=None, w_zero=None, x_group_sums=None, w_zero_term=None, act=ACT_NONE):
         import torch
         if x_tiled:
             kt, M, q, _ = x_planes.shape
@@ -264,8 +267,8 @@ class Gemm:
         assert x_planes.is_contiguous() and w_planes.is_contiguous()
         K = kw * 32
         if out is None:
-            out = torch.empty((M, N), dtype=torch.int32 if out_kind == OUT_I32 else torch.float16,
-                              device=x_planes.device)
+            out = torch.empty((M, N // 2 if act == ACT_SILU_GATE else N),
+                              dtype=torch.int32 if out_kind == OUT_I32 else torch.float16, device=x_planes.device)
         self.out, self.x_planes, self.w_planes = out, x_planes, w_planes
         self.c_scale, self.x_scale, self.w_scale = c_scale, x_scale, w_scale
         self.state = GemmState()
@@ -285,6 +288,8 @@ class Gemm:
         if x_tiled or w_tiled:
             _check(lib().abq_gemm_set_operand_layout(ctypes.byref(self.state), int(x_tiled), int(w_tiled)),
                    "abq_gemm_set_operand_layout")
+        if act != ACT_NONE:
+            _check(lib().abq_gemm_set_activation(ctypes.byref(self.state), act), "abq_gemm_set_activation")
         self.workspace = workspace
         if workspace is not None:
             _check(lib().abq_gemm_set_workspace(ctypes.byref(self.state), workspace.data_ptr(),

@@ -664,6 +664,29 @@ abq_status abq_gemm_set_zero_points(abq_gemm_state *state, const float *x_zero, 
     return ABQ_OK;
 }
 
+abq_status abq_gemm_set_activation(abq_gemm_state *state, int act)
+{
+    if (!state || !state->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    if (act != ABQ_ACT_NONE && act != ABQ_ACT_SILU_GATE)
+        return ABQ_ERR_INVALID_ARG;
+    if (act == ABQ_ACT_SILU_GATE) {
+        if (state->group_size == 0) // fused into the group-scale epilogues only
+            return ABQ_ERR_UNSUPPORTED;
+        if (state->N % 32 != 0)
+            return ABQ_ERR_INVALID_ARG;
+        // the decode kernel needs a gate tile and its up tile in one LDS pass
+        if (state->strategy == ABQ_STRATEGY_DECODE &&
+            decode_grouped_lds(state->M, state->K, state->group_size) + (size_t)kDecodeGroupedWaves * 1024 > 160 * 1024) {
+            const abq_status rc = pick_grouped_tiled(state);
+            if (rc != ABQ_OK)
+                return rc;
+        }
+    }
+    state->act = act;
+    return ABQ_OK;
+}
+
 abq_status abq_weight_zero_term(const uint32_t *w_planes, int n, int k, int bits, int is_signed,
                                 const float *w_scale, const float *w_zero, int group_size,
                                 float *w_zero_term, void *stream)
@@ -717,6 +740,7 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     a.out_kind = st->out_kind;
     a.group_size = st->group_size;
     a.lpr_log2 = st->reserved[0];
+    a.act = st->act;
     a.w_zero = st->w_zero;
     a.x_zero = st->x_zero;
     a.x_group_sums = st->x_group_sums;

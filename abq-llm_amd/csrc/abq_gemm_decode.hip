@@ -420,8 +420,12 @@ __global__ __launch_bounds__(64 * kDecodeGroupedWaves) void gemm_decode_grouped(
     const size_t xplane = (size_t)M * KW, wplane = (size_t)N * KW;
     const int ntiles = (N + 15) / 16;
     const int G = gridDim.x;
-    // tiles blockIdx.x, blockIdx.x + G, ... of this workgroup
-    const int TW = min(tiles_per_wg, (ntiles - (int)blockIdx.x + G - 1) / G);
+    // Tiles of this workgroup: blockIdx.x, blockIdx.x + G, ...; with the SiLU gate the unit is a pair of
+    // tiles (16 gate rows and their 16 up rows), so that both halves of an output meet in one workgroup.
+    const int unit = a.act ? 2 : 1;
+    const int nunits = ntiles / unit;
+    const int TW = min(tiles_per_wg, unit * ((nunits - (int)blockIdx.x + G - 1) / G));
+    auto tile_of = [&](int tl) { return unit == 2 ? 2 * ((int)blockIdx.x + (tl >> 1) * G) + (tl & 1) : (int)blockIdx.x + tl * G; };
 
     // Work items: (tile, step) pairs, step fastest; wave w takes items w, w + NW, ... of a pass.
     // The first item's weight words go in flight before the activation work.
@@ -429,7 +433,7 @@ __global__ __launch_bounds__(64 * kDecodeGroupedWaves) void gemm_decode_grouped(
     {
         const int tp0 = min(tiles_per_pass, TW);
         const int tl = wid / steps, st = wid - tl * steps;
-        load_weight_words<P>(wnext, a.W, wplane, KW, N, blockIdx.x + tl * G, r, st * 16 + 4 * g, KW, wid < tp0 * steps);
+        load_weight_words<P>(wnext, a.W, wplane, KW, N, tile_of(tl), r, st * 16 + 4 * g, KW, wid < tp0 * steps);
     }
 
     // activations -> int8 in LDS, one wave per 64 plane words of a row; the tail of a partial last
@@ -494,7 +498,7 @@ __global__ __launch_bounds__(64 * kDecodeGroupedWaves) void gemm_decode_grouped(
                 }
                 const int tpn = min(tiles_per_pass, TW - tbase);
                 const int tln = jn / steps, stn = jn - tln * steps;
-                load_weight_words<P>(wnext, a.W, wplane, KW, N, blockIdx.x + (tbase + tln) * G, r, stn * 16 + 4 * g, KW,
+                load_weight_words<P>(wnext, a.W, wplane, KW, N, tile_of(tbase + tln), r, stn * 16 + 4 * g, KW,
                                      tpn > 0 && jn < tpn * steps);
             }
             if (tl != cur_tl) {
@@ -509,7 +513,7 @@ __global__ __launch_bounds__(64 * kDecodeGroupedWaves) void gemm_decode_grouped(
             v4i bops[8];
             int unused_sum;
             expand_weight_words<P, WMODE, false>(wv, bops, unused_sum);
-            const int n = min(((int)blockIdx.x + (t0 + tl) * G) * 16 + r, N - 1);
+            const int n = min(tile_of(t0 + tl) * 16 + r, N - 1);
             const float *wsc = a.w_scale + (size_t)n * groups;
             const float *wzp = a.w_zero ? a.w_zero + (size_t)n * groups : nullptr;
 #pragma unroll
@@ -551,15 +555,27 @@ __global__ __launch_bounds__(64 * kDecodeGroupedWaves) void gemm_decode_grouped(
         // output: thread (tile, row i, column c) sums the waves' partial tiles in a fixed order
         for (int u = tid; u < tp * 256; u += NT) {
             const int tl = u >> 8, i = (u >> 4) & 15, c = u & 15;
-            const int nn = ((int)blockIdx.x + (t0 + tl) * G) * 16 + c;
-            if (i < Mb && nn < N) {
+            const int nn = tile_of(t0 + tl) * 16 + c;
+            if (i < Mb && nn < N && !(a.act && (tl & 1))) {
                 float v = 0.f;
 #pragma unroll
                 for (int w2 = 0; w2 < NW; ++w2)
                     v += part[(tl * NW + w2) * 256 + (u & 255)];
                 if (a.x_zero)
                     v -= a.x_zero[m0 + i] * a.w_zero_term[nn];
-                reinterpret_cast<_Float16 *>(a.D)[(size_t)(m0 + i) * N + nn] = (_Float16)(v * a.x_scale[m0 + i]);
+                v *= a.x_scale[m0 + i];
+                if (a.act) { // this tile holds gate rows, the next one their up rows
+                    float up = 0.f;
+#pragma unroll
+                    for (int w2 = 0; w2 < NW; ++w2)
+                        up += part[((tl + 1) * NW + w2) * 256 + (u & 255)];
+                    if (a.x_zero)
+                        up -= a.x_zero[m0 + i] * a.w_zero_term[nn + 16];
+                    up *= a.x_scale[m0 + i];
+                    reinterpret_cast<_Float16 *>(a.D)[(size_t)(m0 + i) * (N / 2) + (nn >> 5) * 16 + c] = (_Float16)(silu(v) * up);
+                } else {
+                    reinterpret_cast<_Float16 *>(a.D)[(size_t)(m0 + i) * N + nn] = (_Float16)v;
+                }
             }
         }
         __syncthreads();
@@ -574,13 +590,19 @@ static hipError_t launch_decode_grouped(const GemmArgs &a, hipStream_t stream)
     const size_t base = decode_grouped_lds(a.M, a.K, a.group_size); // with one tile per pass
     if (!base || (a.group_size != 64 && a.group_size != 128))
         return hipErrorInvalidValue;
-    const int tiles = (a.N + 15) / 16;
-    const int gx = tiles < 256 ? tiles : 256;
-    const int tpw = (tiles + gx - 1) / gx;
+    if (a.act && a.N % 32 != 0)
+        return hipErrorInvalidValue;
+    const int unit = a.act ? 2 : 1; // tiles that must stay together
+    const int units = (a.N + 15) / 16 / unit;
+    const int gx = units < 256 ? units : 256;
+    const int tpw = unit * ((units + gx - 1) / gx);
     // as many tiles per pass as the rest of the LDS holds (16 KiB of per-wave partial tiles each)
     int tpp = 1 + (int)((160 * 1024 - base) / ((size_t)kDecodeGroupedWaves * 1024));
     if (tpp > tpw)
         tpp = tpw;
+    tpp -= tpp % unit;
+    if (tpp == 0)
+        return hipErrorInvalidValue; // a gate / up pair does not fit beside the activations
     const size_t lds = base + (size_t)(tpp - 1) * kDecodeGroupedWaves * 1024;
     static const hipError_t attr = hipFuncSetAttribute(
         reinterpret_cast<const void *>(&gemm_decode_grouped<Q, P, SIGNED>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);

@@ -337,11 +337,20 @@ void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, i
                 const int ml = wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4);
                 const int m = m0 + ml;
                 if (GROUPED) {
-                    if (m < M && n < N) {
-                        float v = facc[i][j][e];
-                        if (a.x_zero) // activation zero points: a rank-one term
-                            v -= a.x_zero[m] * a.w_zero_term[n];
-                        reinterpret_cast<_Float16 *>(a.D)[(size_t)m * N + n] = (_Float16)(v * a.x_scale[m]);
+                    const int mc = min(m, M - 1), nc = min(n, N - 1);
+                    float v = facc[i][j][e];
+                    if (a.x_zero) // activation zero points: a rank-one term
+                        v -= a.x_zero[mc] * a.w_zero_term[nc];
+                    v *= a.x_scale[mc];
+                    if (a.act) {
+                        // SiLU gate: columns come in blocks of 16 gate rows followed by their 16 up rows, so
+                        // the partner of lane r is lane r ^ 16 of the same MFMA tile (N is a multiple of 32)
+                        const float up = __shfl_xor(v, 16);
+                        if (m < M && n < N && !(r & 16))
+                            reinterpret_cast<_Float16 *>(a.D)[(size_t)m * (N / 2) + (n >> 5) * 16 + (n & 15)] =
+                                (_Float16)(silu(v) * up);
+                    } else if (m < M && n < N) {
+                        reinterpret_cast<_Float16 *>(a.D)[(size_t)m * N + n] = (_Float16)v;
                     }
                     continue;
                 }

@@ -20,6 +20,8 @@ struct GemmArgs {
     int out_kind;
     int group_size;
     int lpr_log2;    // popcount kernels: log2(lanes that share one weight row)
+    int act;                 // 0: none; 1: SiLU gate (group-scale kernels): rows of W are gate / up blocks of 16,
+                             // D[m][16 b + c] = silu(out[m][32 b + c]) * out[m][32 b + 16 + c], D is [M][N / 2]
     // zero points of the group-scale path (all optional)
     const float *w_zero;       // [N][K/group_size], in units of weight codes
     const float *x_zero;       // [M], in units of activation codes
@@ -61,6 +63,8 @@ inline size_t decode_grouped_lds(int M, int K, int group_size)
     const size_t need = (size_t)kDecodeGroupedWaves * 256 * 4 + (size_t)16 * (K / group_size) * 4 + 128 + (size_t)mb * row;
     return need <= 160 * 1024 ? need : 0;
 }
+
+__device__ __forceinline__ float silu(float x) { return x / (1.0f + __expf(-x)); }
 
 // ---- output stage shared by all kernels ------------------------------------------------
 // out_kind values mirror abq_out_kind in include/abq_gemm.h.

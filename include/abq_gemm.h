@@ -172,6 +172,7 @@ typedef struct abq_gemm_state {
     const float *w_zero;
     const int32_t *x_group_sums;
     const float *w_zero_term;
+    int act;                 /* abq_activation fused into the epilogue */
 } abq_gemm_state;
 
 /* Replaces AqBMMAInitFn / AqBWMMAInitFn (engine/mma_any/aq_bmma_op.h:141-147,163 and
@@ -210,6 +211,19 @@ abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, cons
  *                              - x_zero[m] * w_zero_term[n] ). */
 abq_status abq_gemm_set_zero_points(abq_gemm_state *state, const float *x_zero, const float *w_zero,
                                     const int32_t *x_group_sums, const float *w_zero_term);
+
+/* Activation fused into the dequantising epilogue of a state with group scales.
+ * ABQ_ACT_SILU_GATE serves the gate / up pair of a LLaMA MLP (the reference runs them as two GEMMs
+ * followed by an elementwise kernel, FfnLayer.cc:341-374,575-577): W holds both matrices
+ * interleaved in blocks of 16 rows (gate rows 16b..16b+15, then up rows 16b..16b+15), N counts the
+ * rows of both and must be a multiple of 32, and D is [M][N/2]:
+ *     D[m][16 b + c] = silu(out[m][32 b + c]) * out[m][32 b + 16 + c],
+ * `out` being what the epilogue would have written without the activation. */
+typedef enum abq_activation {
+    ABQ_ACT_NONE = 0,
+    ABQ_ACT_SILU_GATE = 1
+} abq_activation;
+abq_status abq_gemm_set_activation(abq_gemm_state *state, int act);
 
 /* w_zero_term[n] = sum_g w_scale[n][g] * (sum_{k in g} w[n][k] - group_size * w_zero[n][g]),
  * from weight planes in the reference layout.  w_zero may be NULL (all zero). */

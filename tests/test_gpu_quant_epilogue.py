@@ -154,6 +154,48 @@ def test_decode_kernel_with_group_scales_and_zero_points(abq, oracle, q, p, sign
         assert np.abs(got.astype(np.float64) - got2.astype(np.float64)).max() <= 2e-3 * np.abs(want).max()
 
 
+def interleave16(gate, up):
+    """[I, ...] gate rows and [I, ...] up rows -> [2I, ...] in blocks of 16 gate rows followed by their 16 up rows."""
+    I = gate.shape[0]
+    assert I % 16 == 0
+    out = np.empty((2 * I,) + gate.shape[1:], dtype=gate.dtype)
+    blocks = out.reshape((I // 16, 2, 16) + gate.shape[1:])
+    blocks[:, 0] = gate.reshape((I // 16, 16) + gate.shape[1:])
+    blocks[:, 1] = up.reshape((I // 16, 16) + up.shape[1:])
+    return out
+
+
+@pytest.mark.parametrize("M,strategy", [(1, "decode"), (7, "decode"), (16, "decode"), (100, "tiled"), (300, "tiled")])
+@pytest.mark.parametrize("group_size", [128, 64])
+def test_silu_gate_epilogue(abq, oracle, M, strategy, group_size):
+    """gate / up pair fused into one GEMM: D = silu(x Wg^T) * (x Wu^T) on the dequantised values."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(M + group_size)
+    q, p, I, K = 8, 2, 11008 if M == 7 else 176, 4096 if M == 7 else 640
+    G = K // group_size
+    x = rng.integers(-128, 128, (M, K)).astype(np.int32)
+    xs, xz = rng.uniform(0.005, 0.02, M), rng.integers(-20, 20, M).astype(np.float64)
+    parts = []
+    for _ in range(2):  # gate, up
+        w = rng.integers(-2, 2, (I, K)).astype(np.int32)
+        parts.append((w, rng.uniform(0.002, 0.02, (I, G)), rng.integers(-2, 2, (I, G)).astype(np.float64)))
+    full = [Q.dequant_matmul(x, xs, xz, w, sc, z, group_size) for (w, sc, z) in parts]
+    want = full[0] / (1.0 + np.exp(-full[0])) * full[1]
+    w_cat, sc_cat, z_cat = (interleave16(parts[0][i], parts[1][i]) for i in range(3))
+    wp = planes_dev(oracle.pack_i32(w_cat, p))
+    kw = dict(x_scale=fdev(xs), w_scale=fdev(sc_cat), group_size=group_size, w_zero=fdev(z_cat), x_zero=fdev(xz),
+              x_group_sums=torch.from_numpy(x.reshape(M, G, group_size).sum(axis=2).astype(np.int32)).cuda(),
+              act=abq.ACT_SILU_GATE)
+    kw["w_zero_term"] = abq.weight_zero_term(wp, True, kw["w_scale"], kw["w_zero"], group_size)
+    out = torch.full((M, I), float("nan"), dtype=torch.float16, device="cuda")
+    if strategy == "tiled":
+        got = run_grouped(abq, planes_dev(oracle.pack_i32(x, q)), abq.relayout_planes(wp), True, w_tiled=True, out=out, **kw)
+    else:
+        got = run_grouped(abq, planes_dev(oracle.pack_i32(x, q)), wp, True, strategy="decode", out=out, **kw)
+    assert got.shape == (M, I)
+    assert_close_rel(got, want)
+
+
 def test_group_scale_argument_checks(abq, oracle):
     rng = np.random.default_rng(0)
     x = planes_dev(oracle.pack_i32(rng.integers(0, 256, (32, 256)).astype(np.int32), 8))
@@ -167,6 +209,9 @@ def test_group_scale_argument_checks(abq, oracle):
     assert e.value.status == abq.ABQ_ERR_UNSUPPORTED
     with pytest.raises(abq.AbqError) as e:  # zero points need group scales
         abq.Gemm(x, w, True, out_kind=abq.OUT_F16_SCALED, x_scale=s, w_scale=s, group_size=0, w_zero=s, x_group_sums=s)
+    assert e.value.status == abq.ABQ_ERR_UNSUPPORTED
+    with pytest.raises(abq.AbqError) as e:  # the fused activation lives in the group-scale epilogues
+        abq.Gemm(x, w, True, out_kind=abq.OUT_F16_SCALED, x_scale=s, w_scale=s, group_size=0, act=abq.ACT_SILU_GATE)
     assert e.value.status == abq.ABQ_ERR_UNSUPPORTED
     with pytest.raises(abq.AbqError) as e:  # w_zero without the activation group sums
         abq.Gemm(x, w, True, out_kind=abq.OUT_F16_SCALED, x_scale=s, w_scale=s, group_size=128, w_zero=s)
