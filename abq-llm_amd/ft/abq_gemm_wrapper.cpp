@@ -91,7 +91,7 @@ size_t ABQGEMMWrapper::dynamic_workspace_bytes(int M, int K, int group_size) con
 
 void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _Float16 *A, const ABQGroupedWeight &W,
                                   _Float16 *D, bool x_symmetric, char *abq_gemm_workspace, size_t abq_gemm_ws_bytes,
-                                  hipStream_t stream)
+                                  hipStream_t stream, bool silu_gate)
 {
     if (K < 128 || K % 128 != 0) {
         printf("[ABQ][Error] unsupport K = %d\n", K);
@@ -113,7 +113,7 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     // at most 16 rows: decode kernel on plane operands; above: tiled kernel on the prefill layout
     // (if the expanded activations fit the decode kernel's LDS: partial tiles, group sums, M padded rows)
     const bool decode = M <= 16 && W.planes != nullptr &&
-                        16 * 1024 + (size_t)64 * (K / W.group_size) + 128 + (size_t)M * ((K + 511) / 512 * 512 + 16) <= 160 * 1024;
+                        (silu_gate ? 32 : 16) * 1024 + (size_t)64 * (K / W.group_size) + 128 + (size_t)M * ((K + 511) / 512 * 512 + 16) <= 160 * 1024;
     const int layout = decode ? ABQ_LAYOUT_PLANES : ABQ_LAYOUT_TILED;
     abq_status rc = abq_quant_pack_f16(A, M, K, x_bits_, x_symmetric ? 1 : 0, layout, planes, x_scale, x_zero,
                                        sums, W.group_size, stream);
@@ -131,6 +131,8 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
         rc = abq_gemm_set_scales(&state, x_scale, W.scale, W.group_size);
     if (rc == ABQ_OK && (W.zero || !x_symmetric))
         rc = abq_gemm_set_zero_points(&state, x_symmetric ? nullptr : x_zero, W.zero, sums, W.zero_term);
+    if (rc == ABQ_OK && silu_gate)
+        rc = abq_gemm_set_activation(&state, ABQ_ACT_SILU_GATE);
     if (rc == ABQ_ERR_UNSUPPORTED) {
         printf("[ABQ][Error] unsupport w%da%d\n", w_bits_, x_bits_);
         return;

@@ -56,8 +56,11 @@ public:
     // A: fp16 activations [M][K], quantised per token to X_BITS signed codes inside the call
     // (symmetric, or asymmetric with a zero point); D: fp16 [M][N].  The wrapper must have been
     // constructed with SIGNED = true.  Workspace: dynamic_workspace_bytes(M, K, group_size).
+    // silu_gate: W holds a gate / up pair interleaved in blocks of 16 rows (abq_weight_blob_interleave_gate_up),
+    // N counts the rows of both and D is [M][N/2] = silu(gate) * up: the two GEMMs and the elementwise
+    // kernel of the reference's gated MLP (FfnLayer.cc:341-374,575-577) in one launch.
     void gemm_dynamic(const int M, const int N, const int K, const _Float16 *A, const ABQGroupedWeight &W,
                       _Float16 *D, bool x_symmetric, char *abq_gemm_workspace, size_t abq_gemm_ws_bytes,
-                      hipStream_t stream);
+                      hipStream_t stream, bool silu_gate = false);
     size_t dynamic_workspace_bytes(int M, int K, int group_size) const;
 };

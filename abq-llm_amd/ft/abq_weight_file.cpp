@@ -81,6 +81,34 @@ bool abq_quantize_weights(const float *w, uint32_t n, uint32_t k, uint32_t bits,
     return true;
 }
 
+bool abq_weight_blob_interleave_gate_up(const ABQWeightBlob &gate, const ABQWeightBlob &up, ABQWeightBlob *out,
+                                        std::string *error)
+{
+    const ABQWeightHeader &a = gate.info, &b = up.info;
+    if (!out || a.n != b.n || a.k != b.k || a.bits != b.bits || a.is_signed != b.is_signed || a.group_size != b.group_size ||
+        a.has_zero != b.has_zero)
+        return fail(error, "gate and up blobs do not have the same shape and quantisation");
+    if (a.n % 16 != 0)
+        return fail(error, "row count must be a multiple of 16");
+    const size_t kw = a.k / 32, groups = gate.groups(), n = a.n;
+    out->info = a;
+    out->info.n = 2 * a.n;
+    out->planes.resize(gate.planes.size() * 2);
+    out->scale.resize(gate.scale.size() * 2);
+    out->zero.resize(gate.zero.size() * 2);
+    for (size_t row = 0; row < 2 * n; ++row) {
+        const size_t blk = row / 32, within = row % 32;
+        const ABQWeightBlob &src = within < 16 ? gate : up;
+        const size_t srow = blk * 16 + within % 16;
+        for (uint32_t p = 0; p < a.bits; ++p)
+            memcpy(&out->planes[((size_t)p * 2 * n + row) * kw], &src.planes[((size_t)p * n + srow) * kw], kw * 4);
+        memcpy(&out->scale[row * groups], &src.scale[srow * groups], groups * 4);
+        if (a.has_zero)
+            memcpy(&out->zero[row * groups], &src.zero[srow * groups], groups * 4);
+    }
+    return true;
+}
+
 static bool check_header(const ABQWeightHeader &h, std::string *error)
 {
     if (memcmp(h.magic, kMagic, 8) != 0 || h.version != 1)

@@ -50,6 +50,13 @@ struct ABQWeightBlob {
 bool abq_quantize_weights(const float *w, uint32_t n, uint32_t k, uint32_t bits, bool symmetric, uint32_t group_size,
                           ABQWeightBlob *out, std::string *error);
 
+// The gate and up projections of one MLP as a single matrix for the fused SiLU-gate epilogue
+// (abq_gemm_set_activation): blocks of 16 gate rows followed by their 16 up rows; planes, scales
+// and zero points are interleaved alike.  Both blobs must agree in everything but their values,
+// and their row count must be a multiple of 16.
+bool abq_weight_blob_interleave_gate_up(const ABQWeightBlob &gate, const ABQWeightBlob &up, ABQWeightBlob *out,
+                                        std::string *error);
+
 bool abq_weight_file_write(const std::string &path, const ABQWeightBlob &blob, std::string *error);
 bool abq_weight_file_read(const std::string &path, ABQWeightBlob *blob, std::string *error);
 // headerless plane dump: what LlamaDecoderLayerWeight::loadModel reads for int8_mode 5

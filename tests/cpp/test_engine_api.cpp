@@ -333,6 +333,65 @@ static void gpu_paths()
         HIP_OK(hipFree(d_ws));
     }
 
+    {   // gate / up pair through the weight-blob interleave and the fused SiLU-gate epilogue, decode- and
+        // prefill-sized M, against silu(gate GEMM) * (up GEMM) run as two separate dynamic GEMMs
+        const int I = 96, K = 256, G = 128;
+        std::mt19937 r32(17);
+        std::normal_distribution<float> nd(0.f, 0.05f), xd_(0.f, 1.f);
+        std::vector<float> wg((size_t)I * K), wu((size_t)I * K);
+        for (auto &v : wg)
+            v = nd(r32);
+        for (auto &v : wu)
+            v = nd(r32);
+        ABQWeightBlob bg, bu, bcat;
+        std::string err;
+        CHECK(abq_quantize_weights(wg.data(), I, K, 2, false, G, &bg, &err));
+        CHECK(abq_quantize_weights(wu.data(), I, K, 2, false, G, &bu, &err));
+        CHECK(abq_weight_blob_interleave_gate_up(bg, bu, &bcat, &err));
+        CHECK(bcat.info.n == 2 * I && bcat.planes.size() == 2 * bg.planes.size());
+        ABQDeviceWeight dg, du, dcat;
+        CHECK(dg.load(bg, stream, &err) && du.load(bu, stream, &err) && dcat.load(bcat, stream, &err));
+        ABQGEMMWrapper wrap(8, 2, true);
+        for (int M : { 3, 70 }) {
+            std::vector<uint16_t> ha((size_t)M * K);
+            for (auto &h : ha)
+                h = abq_oracle_f32_to_f16(xd_(r32));
+            const size_t ws_bytes = wrap.dynamic_workspace_bytes(M, K, G);
+            _Float16 *d_a, *d_g, *d_u, *d_f;
+            char *d_ws;
+            HIP_OK(hipMalloc(&d_a, ha.size() * 2));
+            HIP_OK(hipMalloc(&d_g, (size_t)M * I * 2));
+            HIP_OK(hipMalloc(&d_u, (size_t)M * I * 2));
+            HIP_OK(hipMalloc(&d_f, (size_t)M * I * 2));
+            HIP_OK(hipMalloc(&d_ws, ws_bytes));
+            HIP_OK(hipMemcpy(d_a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
+            wrap.gemm_dynamic(M, I, K, d_a, dg.grouped(), d_g, false, d_ws, ws_bytes, stream);
+            wrap.gemm_dynamic(M, I, K, d_a, du.grouped(), d_u, false, d_ws, ws_bytes, stream);
+            wrap.gemm_dynamic(M, 2 * I, K, d_a, dcat.grouped(), d_f, false, d_ws, ws_bytes, stream, true);
+            HIP_OK(hipStreamSynchronize(stream));
+            std::vector<uint16_t> hg((size_t)M * I), hu((size_t)M * I), hf((size_t)M * I);
+            HIP_OK(hipMemcpy(hg.data(), d_g, hg.size() * 2, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(hu.data(), d_u, hu.size() * 2, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(hf.data(), d_f, hf.size() * 2, hipMemcpyDeviceToHost));
+            double worst = 0, rms = 0;
+            std::vector<double> want(hf.size());
+            for (size_t i = 0; i < hf.size(); ++i) {
+                const double gv = abq_oracle_f16_to_f32(hg[i]), uv = abq_oracle_f16_to_f32(hu[i]);
+                want[i] = gv / (1.0 + std::exp(-gv)) * uv;
+                rms += want[i] * want[i];
+            }
+            rms = std::sqrt(rms / want.size());
+            for (size_t i = 0; i < hf.size(); ++i)
+                worst = std::fmax(worst, std::fabs((double)abq_oracle_f16_to_f32(hf[i]) - want[i]) / (std::fabs(want[i]) + rms));
+            CHECK(worst <= 1e-2); // the separate GEMMs round gate and up to fp16 first: well inside the tolerance
+            HIP_OK(hipFree(d_a));
+            HIP_OK(hipFree(d_g));
+            HIP_OK(hipFree(d_u));
+            HIP_OK(hipFree(d_f));
+            HIP_OK(hipFree(d_ws));
+        }
+    }
+
     {   // timer interface
         CudaTimer t(stream);
         t.start();
