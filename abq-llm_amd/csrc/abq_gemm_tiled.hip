@@ -275,6 +275,10 @@ void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, i
                 if (GROUPED)
                     facc[i][j][e] = 0.f;
             }
+    v16i zero16;
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+        zero16[e] = 0;
     // GROUPED: this lane's output columns and where their scales live.  The signed route feeds
     // value * 2^(8-bits) to the MFMA: the exact power of two that undoes it rides on the scale.
     const float unshift = SIGNED ? 1.0f / (float)(1 << (16 - Q - P)) : 1.0f;
@@ -300,6 +304,12 @@ void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, i
         StageB::expand(RW, lds_b + (BUF) * BUF_BYTES, tid, sum_b, (LIVE));                            \
     }
 
+    float gsc[TN][2]; // GROUPED: scales of the stage being multiplied
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        gsc[j][0] = GROUPED ? wsc[j][0] : 0.f;
+        gsc[j][1] = (GROUPED && g64) ? wsc[j][1] : gsc[j][0];
+    }
     ABQ_LOAD_TILE(0, rx0, rw0)
     ABQ_LOAD_TILE(1, rx1, rw1)
     if (NEED_SX || NEED_SW)
@@ -315,15 +325,18 @@ void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, i
     // tile kt used, expansion of tile kt+1 (other register slot) into the other LDS buffer.
 #define ABQ_K_TILE(KT, BUF, RXC, RWC, RXN, RWN)                                                        \
     {                                                                                                  \
-        ABQ_LOAD_TILE((KT) + 2, RXC, RWC)                                                              \
-        float gsc[TN][2];                                                                              \
+        /* the next stage's scales are requested before the tile prefetch, so that waiting for this   \
+           stage's scales (requested one stage ago) never drains the prefetch behind them */          \
+        float gsn[TN][2];                                                                              \
         if (GROUPED) {                                                                                 \
+            const int kn = min((KT) + 1, ktiles - 1);                                                  \
             _Pragma("unroll") for (int j = 0; j < TN; ++j)                                             \
             {                                                                                          \
-                gsc[j][0] = (g64 ? wsc[j][2 * (KT)] : wsc[j][(KT)]) * unshift;                         \
-                gsc[j][1] = g64 ? wsc[j][2 * (KT) + 1] * unshift : gsc[j][0];                          \
+                gsn[j][0] = g64 ? wsc[j][2 * kn] : wsc[j][kn];                                         \
+                gsn[j][1] = g64 ? wsc[j][2 * kn + 1] : gsn[j][0];                                      \
             }                                                                                          \
         }                                                                                              \
+        ABQ_LOAD_TILE((KT) + 2, RXC, RWC)                                                              \
         const unsigned char *ab = a_lane + (BUF) * BUF_BYTES;                                          \
         const unsigned char *bb = b_lane + (BUF) * BUF_BYTES;                                          \
         _Pragma("unroll") for (int ks = 0; ks < WSETS; ++ks)                                           \
@@ -335,18 +348,27 @@ void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, i
                 bv[j] = *reinterpret_cast<const v4i *>(bb + j * 32 * LDS_ROW + ks * 32);               \
             _Pragma("unroll") for (int i = 0; i < TM; ++i)                                             \
                 _Pragma("unroll") for (int j = 0; j < TN; ++j)                                         \
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j], acc[i][j], 0, 0, 0); \
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j],                    \
+                                                                      (GROUPED && ks == 0) ? zero16 : acc[i][j], 0, 0, 0); \
             if (GROUPED && (ks == 3 || (ks == 1 && g64))) {                                            \
                 _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
                     _Pragma("unroll") for (int j = 0; j < TN; ++j)                                     \
                         _Pragma("unroll") for (int e = 0; e < 16; ++e)                                 \
                         {                                                                              \
-                            facc[i][j][e] += (float)acc[i][j][e] * gsc[j][ks >> 1];                    \
-                            acc[i][j][e] = 0;                                                          \
+                            facc[i][j][e] += (float)acc[i][j][e] * (gsc[j][ks >> 1] * unshift);        \
+                            if (ks != WSETS - 1) /* a new stage starts from the zero operand */       \
+                                acc[i][j][e] = 0;                                                      \
                         }                                                                              \
             }                                                                                          \
         }                                                                                              \
         ABQ_EXPAND_TILE(RXN, RWN, (BUF) ^ 1, (KT) + 1 < ktiles)                                        \
+        if (GROUPED) {                                                                                 \
+            _Pragma("unroll") for (int j = 0; j < TN; ++j)                                             \
+            {                                                                                          \
+                gsc[j][0] = gsn[j][0];                                                                 \
+                gsc[j][1] = gsn[j][1];                                                                 \
+            }                                                                                          \
+        }                                                                                              \
         __syncthreads();                                                                               \
     }
 

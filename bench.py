@@ -329,6 +329,51 @@ def main():
                 del gr, gs, out
             del Wr
         extra["decode_group_scales"] = deq
+
+        # ------------------------------------------------------------ side measurement: one decoder layer's linears
+        # BASELINE configs[4]: W2A8, 2-bit weights with group-128 scales and zero points (prepared layout),
+        # activations quantised per token on the device inside the timed call, fp16 output; gate and up run
+        # as one GEMM with the fused SiLU-gate epilogue.  Time = quantise+pack kernel + GEMM, graph replay.
+        layer = []
+        for tokens in (1024, 16384):
+            for name, N, K, act in (("qkv", 12288, 4096, 0), ("o", 4096, 4096, 0), ("gate_up_silu", 22016, 4096, 1),
+                                    ("down", 4096, 11008, 0)):
+                G = K // 128
+                wt = abq.relayout_planes(random_planes(torch, (P_BITS, N, K // 32)))
+                wsc = torch.rand((N, G), device="cuda") * 0.01 + 0.001
+                wz = torch.randint(-2, 2, (N, G), device="cuda").float()
+                x = torch.randn((tokens, K), device="cuda", dtype=torch.float16)
+                xt, xsc, _, sums = abq.quant_pack_f16(x, Q_BITS, symmetric=True, tiled=True, group_size=128)
+                out = torch.empty((tokens, N // 2 if act else N), dtype=torch.float16, device="cuda")
+                gm = abq.Gemm(xt, wt, SIGNED, out=out, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc, group_size=128,
+                              w_zero=wz, x_group_sums=sums, x_tiled=True, w_tiled=True, act=act)
+
+                def step():
+                    abq._check(abq.lib().abq_quant_pack_f16(x.data_ptr(), tokens, K, Q_BITS, 1, 1, xt.data_ptr(), xsc.data_ptr(),
+                                                            None, sums.data_ptr(), 128, abq._stream_ptr(None)), "quant_pack")
+                    gm.run()
+                step()
+                torch.cuda.synchronize()
+                reps = 3
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr):
+                    for _ in range(reps):
+                        step()
+                gr.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                gr.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / reps
+                tops = 2.0 * tokens * N * K / (us * 1e-6) / 1e12
+                layer.append(dict(linear=name, tokens=tokens, N=N, K=K, us=round(us, 1), tops=round(tops, 1),
+                                  mfma_frac=round(tops / INT8_MFMA_PEAK_TOPS, 4), kernel="%s:%s" % (gm.strategy, gm.config_name)))
+                log("layer %s tokens=%d N=%d K=%d  %.1f us  %.0f TOPS (%.1f%% of int8 MFMA peak)"
+                    % (name, tokens, N, K, us, tops, 100 * tops / INT8_MFMA_PEAK_TOPS))
+                del gr, gm, out, x, xt, wt
+        extra["decoder_layer_w2a8_group128"] = layer
         for r in prefill:
             log("prefill W%dA%d %s M=%d N=%d K=%d  %.1f us  %.1f TOPS (%.1f%% of int8 MFMA peak)"
                 % (r["w_bits"], r["x_bits"], "int" if r["signed"] else "uint", r["M"], r["N"], r["K"], r["us"],
