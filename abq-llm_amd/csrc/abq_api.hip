@@ -105,7 +105,9 @@ static void entry_to_config(const KernelEntry &e, int strategy, int x_bits, int 
         c->mma_k = 128;
         c->nstage = 1;
     } else {
-        const int stepk = e.nstage == 4 ? e.kb : (64 / e.mi) * 4 * 32; // NSTAGE 4: K-tiled layout, 128- or 64-element stages
+        // NSTAGE 4 (K-tiled layout, 128- or 64-element stages) and NSTAGE 3 (decode, 512- or 256-element steps)
+        // carry their K step; the direct kernels step 4 plane words per lane group
+        const int stepk = (e.nstage == 4 || e.nstage == 3) ? e.kb : (64 / e.mi) * 4 * 32;
         c->block_m = e.mi * e.tm * e.wm;
         c->block_n = e.mi * e.tn * e.wn;
         c->block_k = stepk * e.wk;
@@ -162,6 +164,9 @@ static int find_mfma_variant(const KernelTable &t, int mi, int tm, int tn, int w
 // Default choice when the caller names no native tile: the decode kernel (16-row MFMA tiles,
 // activations staged in LDS) up to 16 activation rows, 32-row MFMA tiles above.  The popcount
 // kernels stay reachable through their tile tuples (MMA 1x1x128).
+// K elements per work item of the default decode kernel (512 or 256, see abq_gemm_decode.hip)
+static const int kDefaultDecodeStep = 512;
+
 static void choose_default(int M, int N, int *strategy, int *mi, int *tm, int *tn, int *wm, int *wn,
                            int *wk)
 {
@@ -209,8 +214,10 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
 
     int mi = 0, tm = 0, tn = 0, wm = 0, wn = 0, wk = 0;
     int lpr_log2 = best_lpr_log2(K);
+    int decode_step = cfg ? cfg->warp_k : 0; // K elements per decode work item
     if (strategy == ABQ_STRATEGY_AUTO) {
         choose_default(M, N, &strategy, &mi, &tm, &tn, &wm, &wn, &wk);
+        decode_step = kDefaultDecodeStep;
     } else if (strategy == ABQ_STRATEGY_BCNT) {
         mi = 1; tm = cfg->block_m; tn = 1; wm = 1; wn = 4; wk = 1;
         // block_k = lanes per row * 128; accept 16, 32 or 64 lanes, else keep the best fit
@@ -219,7 +226,8 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
             lpr_log2 = lpr == 16 ? 4 : lpr == 32 ? 5 : 6;
     } else {
         mi = cfg->mma_m;
-        const int stepk = (strategy == ABQ_STRATEGY_MFMA32 && cfg->nstage == 4) ? cfg->warp_k : (64 / mi) * 4 * 32;
+        const int stepk = ((strategy == ABQ_STRATEGY_MFMA32 && cfg->nstage == 4) ||
+                           (strategy == ABQ_STRATEGY_MFMA16 && cfg->nstage == 3)) ? cfg->warp_k : (64 / mi) * 4 * 32;
         if (cfg->warp_m <= 0 || cfg->warp_n <= 0 || cfg->warp_m % mi || cfg->warp_n % mi ||
             cfg->block_m % cfg->warp_m || cfg->block_n % cfg->warp_n || cfg->warp_k != stepk ||
             cfg->block_k % stepk)
@@ -264,7 +272,7 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
             return ABQ_ERR_UNSUPPORTED;
         int v = -1;
         for (int i = 0; i < td_->count; ++i)
-            if (td_->entries[i].wk == wk)
+            if (td_->entries[i].wk == wk && td_->entries[i].kb == decode_step)
                 v = i;
         if (v < 0)
             return ABQ_ERR_UNSUPPORTED;

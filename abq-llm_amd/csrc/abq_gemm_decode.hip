@@ -38,9 +38,9 @@ __device__ __forceinline__ uint32_t comp4(const uint4 &v, int i)
     return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
 }
 
-// Loads the P plane words [word, word+4) of weight row (tile*16 + r); all-zero when the item or
-// the words are out of range (one predicated region for all planes).
-template <int P>
+// Loads the P x SW plane words [word, word+SW) of weight row (tile*16 + r), SW = 4 (16 bytes) or 2;
+// all-zero when the item or the words are out of range (one predicated region for all planes).
+template <int P, int SW = 4>
 __device__ __forceinline__ void load_weight_words(uint4 (&dst)[P], const uint32_t *W, size_t wplane, int KW,
                                                   int N, int tile, int r, int word, int word_end, bool item_valid)
 {
@@ -51,19 +51,25 @@ __device__ __forceinline__ void load_weight_words(uint4 (&dst)[P], const uint32_
         const uint32_t *p = W + (size_t)min(tile * 16 + r, N - 1) * KW + word;
 #pragma unroll
         for (int b = 0; b < P; ++b) {
-            dst[b] = *reinterpret_cast<const uint4 *>(p);
+            if (SW == 4) {
+                dst[b] = *reinterpret_cast<const uint4 *>(p);
+            } else {
+                const uint2 v = *reinterpret_cast<const uint2 *>(p);
+                dst[b].x = v.x;
+                dst[b].y = v.y;
+            }
             p += wplane;
         }
     }
 }
 
-// Expands the four plane words per plane held in wv into the eight B operands of one K step.
-template <int P, Int8Mode MODE, bool SUM>
-__device__ __forceinline__ void expand_weight_words(const uint4 (&wv)[P], v4i (&bops)[8], int &value_sum)
+// Expands the SW plane words per plane held in wv into the 2 * SW B operands of one K step.
+template <int P, Int8Mode MODE, bool SUM, int SW = 4>
+__device__ __forceinline__ void expand_weight_words(const uint4 (&wv)[P], v4i (&bops)[2 * SW], int &value_sum)
 {
     value_sum = 0;
 #pragma unroll
-    for (int ws = 0; ws < 4; ++ws) {
+    for (int ws = 0; ws < SW; ++ws) {
         uint32_t w[P], bop[8];
 #pragma unroll
         for (int b = 0; b < P; ++b)
@@ -76,11 +82,15 @@ __device__ __forceinline__ void expand_weight_words(const uint4 (&wv)[P], v4i (&
     }
 }
 
-template <int Q, int P, bool SIGNED, int NW>
+// SW: plane words per lane and item, 4 (a step is 16 words = 512 K elements, 16-byte loads) or 2
+// (steps of 256 elements: twice as many, half as long items, which spreads short K over all waves).
+template <int Q, int P, bool SIGNED, int NW, int SW>
 __global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, int chunk_words, int row_words,
                                                             int tw_base, int tw_rem)
 {
     constexpr int NT = 64 * NW;
+    constexpr int STEPW = 4 * SW;      // plane words per row and step
+    constexpr int STEPB = 32 * STEPW;  // bytes of expanded activations per row and step
     constexpr Int8Mode XMODE = Int8ModeOf<Q, SIGNED>::value;
     constexpr Int8Mode WMODE = Int8ModeOf<P, SIGNED>::value;
     constexpr bool NEED_SX = WMODE == kFlip; // see abq_gemm_mfma.hip: row-sum corrections for
@@ -111,7 +121,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, in
     // fastest.  (tl, st) is the item being computed, (tl1, st1) the next one.
     uint4 w1[P], w2[P];     // raw weight words of the next item and of the one after it
     uint32_t xcur[Q], xnext[Q];
-    v4i bops[8];            // expanded weights of the item being computed
+    v4i bops[2 * SW];       // expanded weights of the item being computed
     int bsum = 0;
     int tl = 0, st = wid, tl1, st1;
 
@@ -140,7 +150,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, in
                 xp += xplane;
             }
         }
-        const int csteps = (cw + 15) >> 4;
+        const int csteps = (cw + STEPW - 1) / STEPW;
         while (st >= csteps) {
             st -= csteps;
             ++tl;
@@ -152,8 +162,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, in
             ++tl1;
         }
         uint4 w0[P];
-        load_weight_words<P>(w0, a.W, wplane, KW, N, blockIdx.x + tl * G, r, st * 16 + 4 * g, cw, tl < TW);
-        load_weight_words<P>(w1, a.W, wplane, KW, N, blockIdx.x + tl1 * G, r, st1 * 16 + 4 * g, cw, tl1 < TW);
+        load_weight_words<P, SW>(w0, a.W, wplane, KW, N, blockIdx.x + tl * G, r, st * STEPW + SW * g, cw, tl < TW);
+        load_weight_words<P, SW>(w1, a.W, wplane, KW, N, blockIdx.x + tl1 * G, r, st1 * STEPW + SW * g, cw, tl1 < TW);
         __builtin_amdgcn_sched_barrier(0);
         for (int i = tid; i < kDecodeMaxTiles * (256 + 16) + 16; i += NT)
             tacc[i] = 0; // ordered before the first ds_add by the barrier that ends the expansion
@@ -161,7 +171,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, in
             __syncthreads(); // the activation row sums are accumulated during the expansion itself
         // The first item's weights are expanded while other waves expand activations.
         if (Mb * bpr <= wid)
-            expand_weight_words<P, WMODE, NEED_SW>(w0, bops, bsum);
+            expand_weight_words<P, WMODE, NEED_SW, SW>(w0, bops, bsum);
         else {
 #pragma unroll
             for (int b = 0; b < P; ++b)
@@ -172,10 +182,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, in
     int k_fed = 0;
     for (int c0 = 0; c0 < KW; c0 += chunk_words) {
         const int cw = min(chunk_words, KW - c0);
-        const int csteps = (cw + 15) >> 4;
+        const int csteps = (cw + STEPW - 1) / STEPW;
         const int bpr = (cw + 63) >> 6;
         const int wend = c0 + cw;
-        k_fed += csteps * 512;
+        k_fed += csteps * STEPW * 32;
         const bool has_x_work = wid < Mb * bpr;
 
         if (c0 != 0) { // later chunks (long K with many activation rows): same first loads, in place
@@ -200,11 +210,11 @@ __global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, in
                 st1 -= csteps;
                 ++tl1;
             }
-            load_weight_words<P>(w2, a.W, wplane, KW, N, blockIdx.x + tl * G, r, c0 + st * 16 + 4 * g, wend, tl < TW);
-            load_weight_words<P>(w1, a.W, wplane, KW, N, blockIdx.x + tl1 * G, r, c0 + st1 * 16 + 4 * g, wend, tl1 < TW);
+            load_weight_words<P, SW>(w2, a.W, wplane, KW, N, blockIdx.x + tl * G, r, c0 + st * STEPW + SW * g, wend, tl < TW);
+            load_weight_words<P, SW>(w1, a.W, wplane, KW, N, blockIdx.x + tl1 * G, r, c0 + st1 * STEPW + SW * g, wend, tl1 < TW);
             __syncthreads(); // previous chunk fully consumed before xs is overwritten
             if (!has_x_work)
-                expand_weight_words<P, WMODE, NEED_SW>(w2, bops, bsum);
+                expand_weight_words<P, WMODE, NEED_SW, SW>(w2, bops, bsum);
         }
 
         // Activation expansion: wave-sized blocks of 64 consecutive plane words of one row,
@@ -243,8 +253,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, in
         }
         // The tail of a partial last step must hold what all-zero planes expand to (weights
         // past K are fed as zero planes; the row-sum correction counts these elements).
-        if (cw & 15) {
-            const int pad = csteps * 16 - cw;
+        if (cw % STEPW) {
+            const int pad = csteps * STEPW - cw;
             const uint32_t fill = XMODE == kFlip ? 0x80808080u : 0u;
             for (int u = tid; u < Mb * pad * 2; u += NT) {
                 const int m = u / (pad * 2), q16 = u - m * (pad * 2);
@@ -252,21 +262,21 @@ __global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, in
             }
         }
         if (has_x_work)
-            expand_weight_words<P, WMODE, NEED_SW>(w2, bops, bsum);
+            expand_weight_words<P, WMODE, NEED_SW, SW>(w2, bops, bsum);
         __syncthreads();
 
         v4i acc = { 0, 0, 0, 0 };
         int sw_part = 0;
         int cur_tl = tl < TW ? tl : -1;
-        const unsigned char *xrow = xs + (size_t)min(r, Mb - 1) * RS + g * 128;
+        const unsigned char *xrow = xs + (size_t)min(r, Mb - 1) * RS + g * (32 * SW);
 
         while (tl < TW) {
-            // A operands of this step: 8 x 16 bytes per lane
-            v4i aop[8];
+            // A operands of this step: 2 * SW x 16 bytes per lane
+            v4i aop[2 * SW];
             {
-                const unsigned char *xw = xrow + st * 512;
+                const unsigned char *xw = xrow + st * STEPB;
 #pragma unroll
-                for (int i = 0; i < 8; ++i)
+                for (int i = 0; i < 2 * SW; ++i)
                     aop[i] = *reinterpret_cast<const v4i *>(xw + i * 16);
             }
             // weights of the item after next go in flight now
@@ -275,7 +285,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, in
                 st2 -= csteps;
                 ++tl2;
             }
-            load_weight_words<P>(w2, a.W, wplane, KW, N, blockIdx.x + tl2 * G, r, c0 + st2 * 16 + 4 * g, wend, tl2 < TW);
+            load_weight_words<P, SW>(w2, a.W, wplane, KW, N, blockIdx.x + tl2 * G, r, c0 + st2 * STEPW + SW * g, wend, tl2 < TW);
             if (tl != cur_tl) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
@@ -289,11 +299,11 @@ __global__ __launch_bounds__(64 * NW) void gemm_mfma_decode(const GemmArgs a, in
             }
             sw_part += bsum;
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
+            for (int i = 0; i < 2 * SW; ++i)
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[i], bops[i], acc, 0, 0, 0);
             // expand the next item's weights (loaded one iteration ago) for the next round
             if (tl1 < TW)
-                expand_weight_words<P, WMODE, NEED_SW>(w1, bops, bsum);
+                expand_weight_words<P, WMODE, NEED_SW, SW>(w1, bops, bsum);
 #pragma unroll
             for (int b = 0; b < P; ++b)
                 w1[b] = w2[b];
@@ -355,7 +365,7 @@ static void decode_chunking(int M, int KW, int *chunk_words, int *row_words)
     *row_words = cw;
 }
 
-template <int Q, int P, bool SIGNED, int NW>
+template <int Q, int P, bool SIGNED, int NW, int SW>
 static hipError_t launch_mfma_decode(const GemmArgs &a, hipStream_t stream)
 {
     const int tiles = (a.N + 15) / 16;
@@ -367,12 +377,12 @@ static hipError_t launch_mfma_decode(const GemmArgs &a, hipStream_t stream)
     const int mb = a.M < 16 ? a.M : 16;
     const size_t lds = kDecodeFixedLds + (size_t)mb * (rw * 32 + 16);
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&gemm_mfma_decode<Q, P, SIGNED, NW>),
+        reinterpret_cast<const void *>(&gemm_mfma_decode<Q, P, SIGNED, NW, SW>),
         hipFuncAttributeMaxDynamicSharedMemorySize, kDecodeFixedLds + kDecodeXBudget);
     if (attr != hipSuccess)
         return attr;
     const dim3 grid(gx, (a.M + 15) / 16);
-    hipLaunchKernelGGL((gemm_mfma_decode<Q, P, SIGNED, NW>), grid, dim3(64 * NW), lds, stream, a, cw, rw, tiles / gx, tiles % gx);
+    hipLaunchKernelGGL((gemm_mfma_decode<Q, P, SIGNED, NW, SW>), grid, dim3(64 * NW), lds, stream, a, cw, rw, tiles / gx, tiles % gx);
     return hipGetLastError();
 }
 
@@ -613,15 +623,16 @@ static hipError_t launch_decode_grouped(const GemmArgs &a, hipStream_t stream)
     return hipGetLastError();
 }
 
-static const KernelEntry kSignedGrouped[] = { { 16, 1, 1, 1, 1, kDecodeGroupedWaves, 3, &launch_decode_grouped<ABQ_Q, ABQ_P, true> } };
-static const KernelEntry kUnsignedGrouped[] = { { 16, 1, 1, 1, 1, kDecodeGroupedWaves, 3, &launch_decode_grouped<ABQ_Q, ABQ_P, false> } };
+static const KernelEntry kSignedGrouped[] = { { 16, 1, 1, 1, 1, kDecodeGroupedWaves, 3, &launch_decode_grouped<ABQ_Q, ABQ_P, true>, 512 } };
+static const KernelEntry kUnsignedGrouped[] = { { 16, 1, 1, 1, 1, kDecodeGroupedWaves, 3, &launch_decode_grouped<ABQ_Q, ABQ_P, false>, 512 } };
 
 // Native tile space of this kernel: waves per workgroup.  Entries reuse the MFMA tuple
 // (16-row tiles, K split over the waves) with nstage = 3 marking the LDS-staged activations.
-#define ABQ_DECODE_VARIANTS(V) V(4) V(8) V(16)
+// (waves, plane words per lane and item)
+#define ABQ_DECODE_VARIANTS(V) V(4, 4) V(8, 4) V(16, 4) V(16, 2)
 
-#define ABQ_ENTRY_T(NW) { 16, 1, 1, 1, 1, NW, 3, &launch_mfma_decode<ABQ_Q, ABQ_P, true, NW> },
-#define ABQ_ENTRY_F(NW) { 16, 1, 1, 1, 1, NW, 3, &launch_mfma_decode<ABQ_Q, ABQ_P, false, NW> },
+#define ABQ_ENTRY_T(NW, SW) { 16, 1, 1, 1, 1, NW, 3, &launch_mfma_decode<ABQ_Q, ABQ_P, true, NW, SW>, 128 * SW },
+#define ABQ_ENTRY_F(NW, SW) { 16, 1, 1, 1, 1, NW, 3, &launch_mfma_decode<ABQ_Q, ABQ_P, false, NW, SW>, 128 * SW },
 
 static const KernelEntry kSigned[] = { ABQ_DECODE_VARIANTS(ABQ_ENTRY_T) };
 static const KernelEntry kUnsigned[] = { ABQ_DECODE_VARIANTS(ABQ_ENTRY_F) };

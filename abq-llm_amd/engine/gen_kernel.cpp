@@ -172,6 +172,8 @@ std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits)
     // (NSTAGE = 3), NW waves per workgroup splitting K.
     for (int nw : { 4, 8, 16 })
         out.push_back(Tile{ 16, 16, 512 * nw, 16, 16, 512, 16, 16, 64, 1, nw, { 3 } });
+    // the same with steps of 256 K elements (short K spread over all waves)
+    out.push_back(Tile{ 16, 16, 256 * 16, 16, 16, 256, 16, 16, 64, 1, 16, { 3 } });
     for (const MfmaVariant &v : enumerate_mfma(x_bits, w_bits)) {
         const int stepk = (64 / v.mi) * 4 * 32;
         out.push_back(Tile{ v.mi * v.tm * v.wm, v.mi * v.tn * v.wn, stepk * v.wk, v.mi * v.tm, v.mi * v.tn,
