@@ -556,9 +556,14 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
     if (!tt)
         return ABQ_ERR_UNSUPPORTED;
     // candidates in order of preference: { TM, TN, waves along M, waves along N, workgroups needed }
-    static const int order[][5] = { { 2, 2, 4, 2, 250 }, { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 200 }, { 1, 1, 2, 2, 0 } };
+    // (the 256x256 tile of eight 64x128 waves halves the L2 -> L1 traffic again; it pays only for the widest
+    // operands, W8A8, and only on grids of several workgroups per compute unit)
+    static const int order[][5] = { { 2, 4, 4, 2, 600 }, { 2, 2, 4, 2, 250 }, { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 200 },
+                                    { 1, 1, 2, 2, 0 } };
     int pick = -1;
     for (const auto &o : order) {
+        if (o[1] == 4 && c.x_bits + c.w_bits < 16)
+            continue;
         const int bm = 32 * o[0] * o[2], bn = 32 * o[1] * o[3];
         const long tiles = (long)((st->M + bm - 1) / bm) * ((st->N + bn - 1) / bn);
         for (int i = 0; i < tt->count; ++i)

@@ -503,7 +503,7 @@ static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 // the default choice uses.
 #define ABQ_TILED_VARIANTS(V) V(4, 4) V(2, 4) V(2, 2) V(2, 1) V(1, 1)
 #define ABQ_TILED_HALF_VARIANTS(V) V(2, 4) V(2, 2)   // K stage of 64
-#define ABQ_TILED_WIDE_VARIANTS(V) V(2, 2, 4, 2) V(2, 2, 4, 4)   // TM, TN, waves along M, N
+#define ABQ_TILED_WIDE_VARIANTS(V) V(2, 2, 4, 2) V(2, 2, 4, 4) V(2, 4, 4, 2)   // TM, TN, waves along M, N
 #define ABQ_GROUPED_VARIANTS(V) V(2, 2) V(1, 1)
 
 #define ABQ_ENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, false, 128>, 128 },

@@ -193,6 +193,7 @@ std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits)
     // larger workgroups (4 x 2 and 4 x 4 waves of 64 x 64): less L2 -> L1 traffic per MFMA
     out.push_back(Tile{ 256, 128, 128, 64, 64, 128, 32, 32, 32, 4, 2, { 4 } });
     out.push_back(Tile{ 256, 256, 128, 64, 64, 128, 32, 32, 32, 4, 4, { 4 } });
+    out.push_back(Tile{ 256, 256, 128, 64, 128, 128, 32, 32, 32, 4, 2, { 4 } });
     const int half[][2] = { { 2, 4 }, { 2, 2 } };
     for (const auto &t : half)
         out.push_back(Tile{ 64 * t[0], 64 * t[1], 64, 32 * t[0], 32 * t[1], 64, 32, 32, 32, 2, 2, { 4 } });
