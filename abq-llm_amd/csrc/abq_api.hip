@@ -558,7 +558,7 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
     // candidates in order of preference: { TM, TN, waves along M, waves along N, workgroups needed }
     // (the 256x256 tile of eight 64x128 waves halves the L2 -> L1 traffic again; it pays only for the widest
     // operands, W8A8, and only on grids of several workgroups per compute unit)
-    static const int order[][5] = { { 2, 4, 4, 2, 600 }, { 2, 2, 4, 2, 250 }, { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 200 },
+    static const int order[][5] = { { 2, 4, 4, 2, 600 }, { 2, 2, 4, 2, 250 }, { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 400 },
                                     { 1, 1, 2, 2, 0 } };
     int pick = -1;
     for (const auto &o : order) {
