@@ -19,9 +19,9 @@ STATUS_NAMES = {
 }
 globals().update({name: code for code, name in STATUS_NAMES.items()})
 OUT_I32, OUT_F16_TENSOR, OUT_F16_SCALED, OUT_F16_TENSOR_F32SCALE = 0, 1, 2, 3
-STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC, STRATEGY_DECODE, STRATEGY_TILED = range(7)
-STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic", "decode", "tiled"]
-LAYOUT_PLANES, LAYOUT_TILED = 0, 1
+STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC, STRATEGY_DECODE, STRATEGY_TILED, STRATEGY_FP6 = range(8)
+STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic", "decode", "tiled", "fp6"]
+LAYOUT_PLANES, LAYOUT_TILED, LAYOUT_FP6 = 0, 1, 2
 ACT_NONE, ACT_SILU_GATE = 0, 1
 
 # every symbol include/abq_gemm.h declares
@@ -32,7 +32,7 @@ EXPORTED = [
     "abq_native_config_count", "abq_native_config_get",
     "abq_gemm_init", "abq_gemm_set_scales", "abq_gemm_exec", "abq_gemm_launch",
     "abq_planes_bytes", "abq_relayout_planes", "abq_gemm_set_operand_layout", "abq_gemm_workspace_bytes",
-    "abq_gemm_set_workspace",
+    "abq_gemm_set_workspace", "abq_fp6_bytes", "abq_fp6_eligible", "abq_relayout_planes_fp6",
     "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16", "abq_gemm_set_activation",
 ]
 
@@ -112,6 +112,10 @@ def lib():
         L.abq_planes_bytes.argtypes = [ci, ci, ci]
         L.abq_planes_bytes.restype = ctypes.c_size_t
         L.abq_relayout_planes.argtypes = [vp, vp, ci, ci, ci, vp]
+        L.abq_relayout_planes_fp6.argtypes = [vp, vp, ci, ci, ci, ci, vp]
+        L.abq_fp6_bytes.argtypes = [ci, ci]
+        L.abq_fp6_bytes.restype = ctypes.c_size_t
+        L.abq_fp6_eligible.argtypes = [ci, ci, ci, ci]
         L.abq_gemm_set_operand_layout.argtypes = [ctypes.POINTER(GemmState), ci, ci]
         L.abq_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GemmState)]
         L.abq_gemm_workspace_bytes.restype = ctypes.c_size_t
@@ -211,6 +215,23 @@ def relayout_planes(planes, out=None, stream=None):
     return out
 
 
+def fp6_eligible(x_bits, w_bits, signed, k):
+    """Whether the FP6 matrix-core route is exact for this bit pair and K (host-side check)."""
+    return bool(lib().abq_fp6_eligible(x_bits, w_bits, int(bool(signed)), k))
+
+
+def relayout_planes_fp6(planes, signed, out=None, stream=None):
+    """planes int32 tensor [bits, rows, k/32] -> FP6 records [k/128, rows, 24] (6-bit sign-magnitude codes)."""
+    import torch
+    bits, rows, kw = planes.shape
+    assert planes.is_cuda and planes.is_contiguous() and kw % 4 == 0
+    if out is None:
+        out = torch.empty((kw // 4, rows, 24), dtype=torch.int32, device=planes.device)
+    _check(lib().abq_relayout_planes_fp6(planes.data_ptr(), out.data_ptr(), rows, kw * 32, bits, int(bool(signed)),
+                                         _stream_ptr(stream)), "abq_relayout_planes_fp6")
+    return out
+
+
 def quant_pack_f16(x, bits, symmetric=True, tiled=False, group_size=0, stream=None):
     """Per-token dynamic quantisation + packing of fp16 activations [rows, k].
 
@@ -247,18 +268,26 @@ class Gemm:
     """One initialised GEMM (the role of AqBMMAOpState + InitFn/ExecFn in the reference).
 
     x_planes / w_planes are in the reference layout [bits, rows, k/32] unless x_tiled / w_tiled
-    say they were converted with relayout_planes ([k/128, rows, bits, 4])."""
+    say they were converted with relayout_planes ([k/128, rows, bits, 4]), or x_fp6 / w_fp6 give the
+    bit width of an operand converted with relayout_planes_fp6 ([k/128, rows, 24])."""
 
     def __init__(self, x_planes, w_planes, signed, out=None, cfg=None, out_kind=OUT_I32, c_scale=None,
                  x_scale=None, w_scale=None, group_size=0, x_tiled=False, w_tiled=False, workspace=None,
-                 x_zero=None, w_zero=None, x_group_sums=None, w_zero_term=None, act=ACT_NONE):
+                 x_zero=None, w_zero=None, x_group_sums=None, w_zero_term=None, act=ACT_NONE,
+                 x_fp6=0, w_fp6=0):
         import torch
-        if x_tiled:
+        if x_fp6:
+            kt, M, _ = x_planes.shape
+            q, kw = int(x_fp6), kt * 4
+        elif x_tiled:
             kt, M, q, _ = x_planes.shape
             kw = kt * 4
         else:
             q, M, kw = x_planes.shape
-        if w_tiled:
+        if w_fp6:
+            kt2, N, _ = w_planes.shape
+            p, kw2 = int(w_fp6), kt2 * 4
+        elif w_tiled:
             kt2, N, p, _ = w_planes.shape
             kw2 = kt2 * 4
         else:
@@ -285,9 +314,10 @@ class Gemm:
             _check(lib().abq_gemm_set_zero_points(ctypes.byref(self.state),
                                                   *[t.data_ptr() if t is not None else None
                                                     for t in self.zero_operands]), "abq_gemm_set_zero_points")
-        if x_tiled or w_tiled:
-            _check(lib().abq_gemm_set_operand_layout(ctypes.byref(self.state), int(x_tiled), int(w_tiled)),
-                   "abq_gemm_set_operand_layout")
+        if x_tiled or w_tiled or x_fp6 or w_fp6:
+            xl = LAYOUT_FP6 if x_fp6 else int(x_tiled)
+            wl = LAYOUT_FP6 if w_fp6 else int(w_tiled)
+            _check(lib().abq_gemm_set_operand_layout(ctypes.byref(self.state), xl, wl), "abq_gemm_set_operand_layout")
         if act != ACT_NONE:
             _check(lib().abq_gemm_set_activation(ctypes.byref(self.state), act), "abq_gemm_set_activation")
         self.workspace = workspace

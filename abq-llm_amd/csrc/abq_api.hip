@@ -15,6 +15,8 @@ hipError_t launch_pack_i32(const int32_t *, uint32_t *, int, int, int, hipStream
 hipError_t launch_pack_f16(const void *, const float *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
+hipError_t launch_relayout_planes_fp6(const uint32_t *, uint32_t *, int, int, int, int, hipStream_t);
+const KernelEntry *fp6_entries(int *count);
 hipError_t launch_quant_pack_rows(const void *, uint32_t *, float *, float *, int *, int, int, int, int, int, int,
                                   hipStream_t);
 hipError_t launch_weight_zero_term(const uint32_t *, int, int, int, int, const float *, const float *, int, float *,
@@ -107,7 +109,7 @@ static void entry_to_config(const KernelEntry &e, int strategy, int x_bits, int 
     } else {
         // NSTAGE 4 (K-tiled layout, 128- or 64-element stages) and NSTAGE 3 (decode, 512- or 256-element steps)
         // carry their K step; the direct kernels step 4 plane words per lane group
-        const int stepk = (e.nstage == 4 || e.nstage == 3) ? e.kb : (64 / e.mi) * 4 * 32;
+        const int stepk = (e.nstage >= 3) ? e.kb : (64 / e.mi) * 4 * 32;
         c->block_m = e.mi * e.tm * e.wm;
         c->block_n = e.mi * e.tn * e.wn;
         c->block_k = stepk * e.wk;
@@ -116,7 +118,7 @@ static void entry_to_config(const KernelEntry &e, int strategy, int x_bits, int 
         c->warp_k = stepk;
         c->mma_m = e.mi;
         c->mma_n = e.mi;
-        c->mma_k = 1024 / e.mi;
+        c->mma_k = e.nstage == 5 ? 64 : 1024 / e.mi; // NSTAGE 5: the FP6 MFMA, 32x32x64
         c->nstage = e.nstage;
     }
 }
@@ -129,8 +131,24 @@ static int strategy_of_mma(const abq_tile_config &c)
         return ABQ_STRATEGY_MFMA16;
     if (c.mma_m == 32 && c.mma_n == 32 && c.mma_k == 32)
         return ABQ_STRATEGY_MFMA32;
+    if (c.mma_m == 32 && c.mma_n == 32 && c.mma_k == 64)
+        return ABQ_STRATEGY_FP6;
     return ABQ_STRATEGY_AUTO;
 }
+
+// The FP6 route is exact when both operands are E2M3 numbers (magnitude <= 16 in units of 1/8:
+// unsigned up to 4 bits, signed up to 5) and no partial sum can reach 2^24.
+static bool fp6_eligible(int x_bits, int w_bits, int is_signed, int K)
+{
+    const int lim = is_signed ? 5 : 4;
+    if (x_bits < 1 || w_bits < 1 || x_bits > lim || w_bits > lim)
+        return false;
+    const long mx = is_signed ? (1L << (x_bits - 1)) : (1L << x_bits) - 1;
+    const long mw = is_signed ? (1L << (w_bits - 1)) : (1L << w_bits) - 1;
+    return mx * mw * (long)K < (1L << 24);
+}
+
+static size_t fp6_bytes(int rows, int k) { return (size_t)rows * (k / 128) * 96; }
 
 // Lanes per weight row for the popcount kernels: the power of two in [16, 64] that wastes
 // the fewest lanes for this K (a row has K/128 sixteen-byte units).
@@ -194,6 +212,32 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
 {
     const Registry &reg = registry();
     int strategy = cfg ? strategy_of_mma(*cfg) : ABQ_STRATEGY_AUTO;
+    if (strategy == ABQ_STRATEGY_FP6) {
+        if (cfg->nstage != 5 || cfg->warp_k != 128 || cfg->block_k != 128 || cfg->warp_m <= 0 || cfg->warp_n <= 0 ||
+            cfg->warp_m % 32 || cfg->warp_n % 32 || cfg->block_m % cfg->warp_m || cfg->block_n % cfg->warp_n)
+            return ABQ_ERR_UNSUPPORTED;
+        if (!fp6_eligible(x_bits, w_bits, is_signed, K))
+            return ABQ_ERR_UNSUPPORTED;
+        int count = 0;
+        const KernelEntry *es = fp6_entries(&count);
+        int v = -1;
+        for (int i = 0; i < count; ++i)
+            if (es[i].tm == cfg->warp_m / 32 && es[i].tn == cfg->warp_n / 32 && es[i].wm == cfg->block_m / cfg->warp_m &&
+                es[i].wn == cfg->block_n / cfg->warp_n)
+                v = i;
+        if (v < 0)
+            return ABQ_ERR_UNSUPPORTED;
+        const KernelEntry &e = es[v];
+        const int bm = 32 * e.tm * e.wm, bn = 32 * e.tn * e.wn;
+        const int mblocks = (M + bm - 1) / bm, npx = ((N + bn - 1) / bn + 7) / 8;
+        st->strategy = strategy;
+        st->variant = v;
+        entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
+        st->grid_dim = abq_dim3{ (unsigned)(8 * npx * mblocks), 1, 1 };
+        st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
+        st->shared_mem_size = 2 * (size_t)(bm + bn) * 112;
+        return ABQ_OK;
+    }
     const KernelTable *tm_ = find_table(reg.mfma, x_bits, w_bits, is_signed);
     const KernelTable *tb_ = find_table(reg.bcnt, x_bits, w_bits, is_signed);
     const KernelTable *td_ = find_table(reg.decode, x_bits, w_bits, is_signed);
@@ -457,7 +501,10 @@ int abq_native_config_count(int x_bits, int w_bits, int is_signed)
     const KernelTable *tt = find_table(reg.tiled, x_bits, w_bits, is_signed);
     if (!tb || !tm || !td || !tt)
         return 0;
-    return tb->count * 3 + td->count + tm->count + tt->count;
+    int nfp6 = 0;
+    if (fp6_eligible(x_bits, w_bits, is_signed, 128))
+        fp6_entries(&nfp6);
+    return tb->count * 3 + td->count + tm->count + tt->count + nfp6;
 }
 
 abq_status abq_native_config_get(int x_bits, int w_bits, int is_signed, int index, abq_tile_config *cfg)
@@ -484,8 +531,17 @@ abq_status abq_native_config_get(int x_bits, int w_bits, int is_signed, int inde
     if (index >= tm->count) {
         const KernelTable *tt = find_table(reg.tiled, x_bits, w_bits, is_signed);
         index -= tm->count;
-        if (!tt || index >= tt->count)
+        if (!tt)
             return ABQ_ERR_INVALID_ARG;
+        if (index >= tt->count) {
+            index -= tt->count;
+            int nfp6 = 0;
+            const KernelEntry *es = fp6_entries(&nfp6);
+            if (!fp6_eligible(x_bits, w_bits, is_signed, 128) || index >= nfp6)
+                return ABQ_ERR_INVALID_ARG;
+            entry_to_config(es[index], ABQ_STRATEGY_FP6, x_bits, w_bits, is_signed, 0, cfg);
+            return ABQ_OK;
+        }
         entry_to_config(tt->entries[index], ABQ_STRATEGY_TILED, x_bits, w_bits, is_signed, 0, cfg);
         return ABQ_OK;
     }
@@ -583,9 +639,41 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
     return ABQ_OK;
 }
 
+// Picks the FP6 kernel's tile for a shape: the largest tile that still yields enough workgroups.
+static abq_status switch_to_fp6(abq_gemm_state *st)
+{
+    const abq_tile_config &c = st->cfg;
+    if (!fp6_eligible(c.x_bits, c.w_bits, c.is_signed, st->K) || st->group_size)
+        return ABQ_ERR_UNSUPPORTED;
+    int count = 0;
+    const KernelEntry *es = fp6_entries(&count);
+    // { TM, TN, waves along M, waves along N, workgroups needed }
+    static const int order[][5] = { { 2, 2, 4, 2, 250 }, { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 400 }, { 1, 1, 2, 2, 0 } };
+    int pick = -1;
+    for (const auto &o : order) {
+        const int bm = 32 * o[0] * o[2], bn = 32 * o[1] * o[3];
+        const long tiles = (long)((st->M + bm - 1) / bm) * ((st->N + bn - 1) / bn);
+        for (int i = 0; i < count; ++i)
+            if (es[i].tm == o[0] && es[i].tn == o[1] && es[i].wm == o[2] && es[i].wn == o[3] && tiles >= o[4] && pick < 0)
+                pick = i;
+    }
+    if (pick < 0)
+        return ABQ_ERR_UNSUPPORTED;
+    abq_tile_config cfg;
+    entry_to_config(es[pick], ABQ_STRATEGY_FP6, c.x_bits, c.w_bits, c.is_signed, 0, &cfg);
+    abq_gemm_state tmp = *st;
+    const abq_status rc = resolve(&cfg, c.x_bits, c.w_bits, c.is_signed, st->M, st->N, st->K, &tmp);
+    if (rc != ABQ_OK)
+        return rc;
+    *st = tmp;
+    return ABQ_OK;
+}
+
 // Moves a state with group scales onto the tiled kernel's group-scale variants.
 static abq_status pick_grouped_tiled(abq_gemm_state *state)
 {
+    if (state->x_layout == ABQ_LAYOUT_FP6 || state->w_layout == ABQ_LAYOUT_FP6)
+        return ABQ_ERR_UNSUPPORTED; // group scales are folded by the int8 kernels only
     if (state->strategy != ABQ_STRATEGY_TILED) {
         if (!state->auto_chosen)
             return ABQ_ERR_UNSUPPORTED;
@@ -763,10 +851,40 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     hipError_t e;
     if (st->strategy == ABQ_STRATEGY_GENERIC) {
         e = launch_bcnt_generic(a, c.x_bits, c.w_bits, c.is_signed, (hipStream_t)stream);
+    } else if (st->strategy == ABQ_STRATEGY_FP6) {
+        // operands still in the reference layout are converted into the caller's workspace
+        const size_t xb = st->x_layout == ABQ_LAYOUT_FP6 ? 0 : fp6_bytes(st->M, st->K);
+        const size_t wb = st->w_layout == ABQ_LAYOUT_FP6 ? 0 : fp6_bytes(st->N, st->K);
+        if (st->group_size || st->x_layout == ABQ_LAYOUT_TILED || st->w_layout == ABQ_LAYOUT_TILED)
+            return ABQ_ERR_NOT_INITIALIZED;
+        if (xb + wb > st->workspace_bytes || ((xb + wb) && !st->workspace))
+            return ABQ_ERR_INVALID_ARG;
+        char *ws = static_cast<char *>(st->workspace);
+        if (xb) {
+            e = launch_relayout_planes_fp6(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, c.x_bits, c.is_signed,
+                                           (hipStream_t)stream);
+            if (e != hipSuccess)
+                return hip_status(e);
+            a.X = reinterpret_cast<const uint32_t *>(ws);
+        }
+        if (wb) {
+            e = launch_relayout_planes_fp6(st->W, reinterpret_cast<uint32_t *>(ws + xb), st->N, st->K, c.w_bits,
+                                           c.is_signed, (hipStream_t)stream);
+            if (e != hipSuccess)
+                return hip_status(e);
+            a.W = reinterpret_cast<const uint32_t *>(ws + xb);
+        }
+        int count = 0;
+        const KernelEntry *es = fp6_entries(&count);
+        if (st->variant < 0 || st->variant >= count)
+            return ABQ_ERR_NOT_INITIALIZED;
+        e = es[st->variant].launch(a, (hipStream_t)stream);
     } else if (st->strategy == ABQ_STRATEGY_TILED) {
         // operands still in the reference layout are converted into the caller's workspace
         const size_t xb = st->x_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->M, st->K, c.x_bits);
         const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, c.w_bits);
+        if (st->x_layout == ABQ_LAYOUT_FP6 || st->w_layout == ABQ_LAYOUT_FP6)
+            return ABQ_ERR_NOT_INITIALIZED;
         if (xb + wb > st->workspace_bytes || ((xb + wb) && !st->workspace))
             return ABQ_ERR_INVALID_ARG;
         char *ws = static_cast<char *>(st->workspace);
@@ -816,10 +934,34 @@ abq_status abq_relayout_planes(const uint32_t *planes, uint32_t *tiled, int rows
     return hip_status(launch_relayout_planes(planes, tiled, rows, k, bits, (hipStream_t)stream));
 }
 
+size_t abq_fp6_bytes(int rows, int k)
+{
+    if (rows <= 0 || k <= 0 || k % 128)
+        return 0;
+    return fp6_bytes(rows, k);
+}
+
+int abq_fp6_eligible(int x_bits, int w_bits, int is_signed, int k) { return fp6_eligible(x_bits, w_bits, is_signed, k) ? 1 : 0; }
+
+abq_status abq_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int rows, int k, int bits, int is_signed,
+                                   void *stream)
+{
+    if (!planes || !fp6 || rows <= 0 || bits < 1)
+        return ABQ_ERR_INVALID_ARG;
+    if (bits > (is_signed ? 5 : 4))
+        return ABQ_ERR_UNSUPPORTED;
+    if (k < 128 || k % 128 != 0)
+        return ABQ_ERR_BAD_K;
+    return hip_status(launch_relayout_planes_fp6(planes, fp6, rows, k, bits, is_signed ? 1 : 0, (hipStream_t)stream));
+}
+
 size_t abq_gemm_workspace_bytes(const abq_gemm_state *st)
 {
     if (!st || !st->init_success)
         return 0;
+    if (st->strategy == ABQ_STRATEGY_FP6)
+        return (st->x_layout == ABQ_LAYOUT_FP6 ? 0 : fp6_bytes(st->M, st->K)) +
+               (st->w_layout == ABQ_LAYOUT_FP6 ? 0 : fp6_bytes(st->N, st->K));
     const size_t xb = st->x_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->M, st->K, st->cfg.x_bits);
     const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, st->cfg.w_bits);
     return xb + wb;
@@ -829,10 +971,28 @@ abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_l
 {
     if (!st || !st->init_success)
         return ABQ_ERR_NOT_INITIALIZED;
-    if ((x_layout != ABQ_LAYOUT_PLANES && x_layout != ABQ_LAYOUT_TILED) ||
-        (w_layout != ABQ_LAYOUT_PLANES && w_layout != ABQ_LAYOUT_TILED))
+    if (x_layout < ABQ_LAYOUT_PLANES || x_layout > ABQ_LAYOUT_FP6 || w_layout < ABQ_LAYOUT_PLANES ||
+        w_layout > ABQ_LAYOUT_FP6)
         return ABQ_ERR_INVALID_ARG;
-    if ((x_layout == ABQ_LAYOUT_TILED || w_layout == ABQ_LAYOUT_TILED) && st->strategy != ABQ_STRATEGY_TILED) {
+    const bool any_fp6 = x_layout == ABQ_LAYOUT_FP6 || w_layout == ABQ_LAYOUT_FP6;
+    const bool any_tiled = x_layout == ABQ_LAYOUT_TILED || w_layout == ABQ_LAYOUT_TILED;
+    if (any_fp6 && any_tiled)
+        return ABQ_ERR_UNSUPPORTED;
+    if (any_fp6 && st->strategy != ABQ_STRATEGY_FP6) {
+        if (!st->auto_chosen || st->group_size)
+            return ABQ_ERR_UNSUPPORTED;
+        const abq_status rc = switch_to_fp6(st);
+        if (rc != ABQ_OK)
+            return rc;
+    }
+    if (st->strategy == ABQ_STRATEGY_FP6 && any_tiled) {
+        if (!st->auto_chosen)
+            return ABQ_ERR_UNSUPPORTED;
+        const abq_status rc = switch_to_tiled(st);
+        if (rc != ABQ_OK)
+            return rc;
+    }
+    if (any_tiled && st->strategy != ABQ_STRATEGY_TILED) {
         if (!st->auto_chosen)
             return ABQ_ERR_UNSUPPORTED;
         const abq_status rc = st->group_size ? pick_grouped_tiled(st) : switch_to_tiled(st);
@@ -852,8 +1012,8 @@ abq_status abq_gemm_set_workspace(abq_gemm_state *st, void *workspace, size_t by
         return ABQ_ERR_INVALID_ARG;
     st->workspace = workspace;
     st->workspace_bytes = bytes;
-    if (st->strategy != ABQ_STRATEGY_TILED && st->auto_chosen && st->M > 16 && workspace &&
-        bytes >= abq_gemm_workspace_bytes(st))
+    if (st->strategy != ABQ_STRATEGY_TILED && st->strategy != ABQ_STRATEGY_FP6 && st->auto_chosen && st->M > 16 &&
+        workspace && bytes >= abq_gemm_workspace_bytes(st))
         return switch_to_tiled(st);
     return ABQ_OK;
 }

@@ -198,6 +198,109 @@ hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int r
     return hipGetLastError();
 }
 
+// ---- FP6 records ---------------------------------------------------------------------------
+//
+// Operand format of the FP6 MFMA kernel (abq_gemm_fp6.hip).  An element becomes the 6-bit
+// sign-magnitude code (sign << 5) | |value|, which read as an E2M3 float is value / 8 for every
+// |value| <= 16.  A word-set (32 consecutive K elements, one plane word) becomes a string of
+// 192 bits: position p (bits [6p, 6p+6)) holds element 31 - 8 (p % 4) - p / 4, the order the
+// bit-matrix transpose leaves them in; both operands use it, and a dot product does not care.
+// A row's K tile of 128 elements is one record of 24 words, word-set ws at words
+// [12 (ws & 1) + 6 (ws >> 1), +6): the two word-sets that lanes 0-31 feed to the two MFMA
+// K steps come first, then the two of lanes 32-63.  Records are stored fp6[kt][row][24].
+
+// Bit-sliced |value| and sign of 32 elements: p[t] = plane t, planes at and above bits - 1 read
+// as the sign plane (two's complement sign extension) when the operand is signed.
+__device__ __forceinline__ void fp6_string(const uint32_t (&p)[5], int bits, bool is_signed, uint32_t (&out)[6])
+{
+    const uint32_t s = is_signed ? p[bits - 1] : 0u;
+    uint32_t r[8];
+    uint32_t carry = s; // |v| = (v ^ -sign) + sign, one ripple step per plane
+#pragma unroll
+    for (int t = 0; t < 5; ++t) {
+        const uint32_t x = ((t < bits - 1 || !is_signed) && t < bits ? p[t] : s) ^ s;
+        r[t] = x ^ carry;
+        carry &= x;
+    }
+    r[5] = s;
+    r[6] = 0u;
+    r[7] = 0u;
+    transpose8x8x4(r); // dword d, byte c: the code of the element at plane bit 8c + d
+    uint32_t y[8];
+#pragma unroll
+    for (int d = 0; d < 8; ++d)
+        y[d] = (r[d] & 0x3Fu) | ((r[d] >> 2) & 0xFC0u) | ((r[d] >> 4) & 0x3F000u) | ((r[d] >> 6) & 0xFC0000u);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        out[3 * h + 0] = y[4 * h] | (y[4 * h + 1] << 24);
+        out[3 * h + 1] = (y[4 * h + 1] >> 8) | (y[4 * h + 2] << 16);
+        out[3 * h + 2] = (y[4 * h + 2] >> 16) | (y[4 * h + 3] << 8);
+    }
+}
+
+// One thread per word-set; a workgroup covers 8 rows x 8 K tiles (32 consecutive plane words of a
+// row are one coalesced 128-byte read per plane) and writes each tile's 8 records (contiguous in
+// memory) with 16-byte stores out of LDS.
+template <int BITS>
+__global__ __launch_bounds__(256) void relayout_planes_fp6_kernel(const uint32_t *__restrict__ planes,
+                                                                  uint32_t *__restrict__ fp6, int rows, int KW,
+                                                                  int is_signed)
+{
+    constexpr int REC = 24;
+    constexpr int SLAB = 8 * REC + 4; // words per K tile in LDS (+16 bytes against bank conflicts)
+    __shared__ __align__(16) uint32_t buf[8 * SLAB];
+    const int tid = threadIdx.x;
+    const int kt_tiles = KW / 4;
+    const int row0 = blockIdx.x * 8, kt0 = blockIdx.y * 8;
+    const size_t plane_stride = (size_t)rows * KW;
+    {
+        const int i = tid >> 5, w = tid & 31; // row, word-set within the 8 tiles
+        const int row = row0 + i, kw = 4 * kt0 + w;
+        if (row < rows && kw < KW) {
+            uint32_t pw[5];
+            const uint32_t *p = planes + (size_t)row * KW + kw;
+#pragma unroll
+            for (int b = 0; b < 5; ++b)
+                pw[b] = b < BITS ? p[b * plane_stride] : 0u;
+            uint32_t o[6];
+            fp6_string(pw, BITS, is_signed != 0, o);
+            const int ws = w & 3;
+            uint32_t *rec = buf + (w >> 2) * SLAB + i * REC + 12 * (ws & 1) + 6 * (ws >> 1);
+            *reinterpret_cast<uint2 *>(rec) = make_uint2(o[0], o[1]);
+            *reinterpret_cast<uint2 *>(rec + 2) = make_uint2(o[2], o[3]);
+            *reinterpret_cast<uint2 *>(rec + 4) = make_uint2(o[4], o[5]);
+        }
+    }
+    __syncthreads();
+    const int nrow = min(8, rows - row0);
+    const int per_tile = nrow * (REC / 4); // 16-byte pieces per K tile
+    for (int u = tid; u < 8 * per_tile; u += 256) {
+        const int j = u / per_tile, q = u % per_tile;
+        const int kt = kt0 + j;
+        if (kt < kt_tiles)
+            reinterpret_cast<uint4 *>(fp6 + ((size_t)kt * rows + row0) * REC)[q] =
+                reinterpret_cast<const uint4 *>(buf + j * SLAB)[q];
+    }
+}
+
+hipError_t launch_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int rows, int k, int bits, int is_signed,
+                                      hipStream_t stream)
+{
+    const int KW = k / 32;
+    const dim3 grid((rows + 7) / 8, (KW / 4 + 7) / 8);
+    switch (bits) {
+#define ABQ_FP6_CASE(B)                                                                                                  \
+    case B:                                                                                                              \
+        hipLaunchKernelGGL(relayout_planes_fp6_kernel<B>, grid, dim3(256), 0, stream, planes, fp6, rows, KW, is_signed); \
+        break;
+        ABQ_FP6_CASE(1) ABQ_FP6_CASE(2) ABQ_FP6_CASE(3) ABQ_FP6_CASE(4) ABQ_FP6_CASE(5)
+#undef ABQ_FP6_CASE
+    default:
+        return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 // compress_fields + store_fields for a run-time bit width
 template <int BITS> __device__ __forceinline__ void store_fields_of(uint32_t *rec, int ws, const uint32_t (&e)[8])
 {

@@ -158,7 +158,7 @@ std::vector<MfmaVariant> enumerate_mfma(int x_bits, int w_bits)
     return out;
 }
 
-std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits)
+std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits, bool is_signed)
 {
     std::vector<Tile> out;
     // VALU popcount: MT activation rows per pass, LPR lanes per weight row (16, 32, 64).
@@ -197,6 +197,14 @@ std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits)
     const int half[][2] = { { 2, 4 }, { 2, 2 } };
     for (const auto &t : half)
         out.push_back(Tile{ 64 * t[0], 64 * t[1], 64, 32 * t[0], 32 * t[1], 64, 32, 32, 32, 2, 2, { 4 } });
+    // FP6 matrix-core kernel (NSTAGE = 5, MMA 32x32x64): operands that are E2M3 numbers, i.e. unsigned
+    // of at most 4 bits or signed of at most 5; { TM, TN, waves along M, waves along N }
+    const int lim = is_signed ? 5 : 4;
+    if (x_bits <= lim && w_bits <= lim) {
+        const int fp6[][4] = { { 2, 2, 4, 2 }, { 4, 2, 2, 2 }, { 2, 2, 2, 2 }, { 2, 1, 2, 2 }, { 1, 1, 2, 2 } };
+        for (const auto &t : fp6)
+            out.push_back(Tile{ 32 * t[0] * t[2], 32 * t[1] * t[3], 128, 32 * t[0], 32 * t[1], 128, 32, 32, 64, t[2], t[3], { 5 } });
+    }
     return out;
 }
 
@@ -226,7 +234,7 @@ int main(int argc, char **argv)
     }
     std::printf("////// W%dA%d %s\n", w_bits, x_bits, is_signed ? "int" : "uint");
     const std::vector<Tile> tiles = space == "sm80" ? enumerate_sm80(x_bits, w_bits, k_stages)
-                                                    : enumerate_gfx950(x_bits, w_bits);
+                                                    : enumerate_gfx950(x_bits, w_bits, is_signed);
     for (const Tile &t : tiles)
         print_tile(t, x_bits, w_bits, is_signed);
     return 0;

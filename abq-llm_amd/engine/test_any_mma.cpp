@@ -158,7 +158,8 @@ int main(int argc, char **argv)
     uint32_t *d_wt;
     char *d_ws;
     HIP_OK(hipMalloc(&d_wt, wp_bytes * nbuf));
-    HIP_OK(hipMalloc(&d_ws, xp_words * 4));
+    const size_t ws_bytes = std::max((size_t)xp_words * 4, abq_fp6_bytes(M, K));
+    HIP_OK(hipMalloc(&d_ws, ws_bytes));
     if (abq_relayout_planes(d_wp, d_wt, N, K, w_bits, stream) != ABQ_OK) {
         std::printf("abq_relayout_planes failed (hip error %d)\n", abq_last_hip_error());
         return -1;
@@ -167,6 +168,22 @@ int main(int argc, char **argv)
     for (size_t b = 1; b < nbuf; ++b)
         HIP_OK(hipMemcpyAsync((char *)d_wt + b * wp_bytes, d_wt, wp_bytes, hipMemcpyDeviceToDevice, stream));
     HIP_OK(hipStreamSynchronize(stream));
+
+    // The FP6 kernels (NSTAGE 5) read their own record format: 96 bytes per row and K tile.
+    const bool fp6_ok = abq_fp6_eligible(x_bits, w_bits, is_signed, K) != 0;
+    const size_t wf_bytes = abq_fp6_bytes(N, K);
+    uint32_t *d_wf = nullptr;
+    if (fp6_ok) {
+        HIP_OK(hipMalloc(&d_wf, wf_bytes * nbuf));
+        if (abq_relayout_planes_fp6(d_wp, d_wf, N, K, w_bits, is_signed, stream) != ABQ_OK) {
+            std::printf("abq_relayout_planes_fp6 failed (hip error %d)\n", abq_last_hip_error());
+            return -1;
+        }
+        HIP_OK(hipStreamSynchronize(stream));
+        for (size_t b = 1; b < nbuf; ++b)
+            HIP_OK(hipMemcpyAsync((char *)d_wf + b * wf_bytes, d_wf, wf_bytes, hipMemcpyDeviceToDevice, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+    }
 
     std::vector<uint32_t> h_xp(xp_words), h_wp(wp_words);
     HIP_OK(hipMemcpy(h_xp.data(), d_xp, xp_words * 4, hipMemcpyDeviceToHost));
@@ -202,14 +219,22 @@ int main(int argc, char **argv)
         std::vector<abq_gemm_state> states(nbuf);
         // tiled tiles (NSTAGE 4) and the library's own choice for M > 16 run on prepared weights
         const bool tiled = cfg ? cfg->nstage == 4 : M > 16;
+        const bool fp6 = cfg && cfg->nstage == 5;
+        if (fp6 && !fp6_ok) {
+            t.status = -1;
+            return;
+        }
         for (size_t b = 0; b < nbuf; ++b) {
-            const char *wbase = tiled ? (const char *)d_wt : (const char *)d_wp;
-            abq_status s = abq_gemm_init(cfg, x_bits, w_bits, is_signed, d_xp, (const uint32_t *)(wbase + b * wp_bytes),
+            const char *wbase = fp6 ? (const char *)d_wf + b * wf_bytes
+                                    : (tiled ? (const char *)d_wt : (const char *)d_wp) + b * wp_bytes;
+            abq_status s = abq_gemm_init(cfg, x_bits, w_bits, is_signed, d_xp, (const uint32_t *)wbase,
                                          M, N, K, d_out, nullptr, 0, ABQ_OUT_I32, &states[b]);
             if (s == ABQ_OK && tiled)
                 s = abq_gemm_set_operand_layout(&states[b], ABQ_LAYOUT_PLANES, ABQ_LAYOUT_TILED);
-            if (s == ABQ_OK && tiled)
-                s = abq_gemm_set_workspace(&states[b], d_ws, xp_words * 4);
+            if (s == ABQ_OK && fp6)
+                s = abq_gemm_set_operand_layout(&states[b], ABQ_LAYOUT_PLANES, ABQ_LAYOUT_FP6);
+            if (s == ABQ_OK && (tiled || fp6))
+                s = abq_gemm_set_workspace(&states[b], d_ws, ws_bytes);
             if (s != ABQ_OK || !states[b].init_success) {
                 t.status = -1;
                 return;
@@ -296,6 +321,8 @@ int main(int argc, char **argv)
     (void)hipFree(d_wp);
     (void)hipFree(d_out);
     (void)hipFree(d_wt);
+    if (d_wf)
+        (void)hipFree(d_wf);
     (void)hipFree(d_ws);
     (void)hipStreamDestroy(stream);
     return 0;

@@ -256,6 +256,33 @@ def main():
                 del wpl, wtl
         extra["prefill"] = prefill
 
+        # Yardstick for the prefill figures: the vendor library's plain int8 GEMM (torch._int_mm, operands
+        # already int8 and K-major, nothing to unpack) on the same shapes, timed the same way.
+        vendor = []
+        try:
+            for (N, K) in SHAPES:
+                for M in (512, 2048):
+                    a8 = torch.randint(-128, 128, (M, K), dtype=torch.int8, device="cuda")
+                    b8 = torch.randint(-128, 128, (N, K), dtype=torch.int8, device="cuda").t()
+                    for _ in range(3):
+                        torch._int_mm(a8, b8)
+                    torch.cuda.synchronize()
+                    reps = 10
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(reps):
+                        torch._int_mm(a8, b8)
+                    e1.record()
+                    torch.cuda.synchronize()
+                    us = e0.elapsed_time(e1) * 1e3 / reps
+                    tops = 2.0 * M * N * K / (us * 1e-6) / 1e12
+                    vendor.append(dict(M=M, N=N, K=K, us=round(us, 1), tops=round(tops, 2),
+                                       mfma_frac=round(tops / INT8_MFMA_PEAK_TOPS, 4)))
+                    del a8, b8
+        except Exception as exc:  # the yardstick is optional: a torch build without int8 matmul only loses this entry
+            vendor = {"unavailable": repr(exc)[:120]}
+        extra["library_int8_gemm"] = vendor
+
         # ------------------------------------------------------------ side measurement: several linears per launch
         # QKV (N = 3 * 4096) and gate + up (N = 2 * 11008) share their activations, so each is one GEMM
         # over concatenated weight planes: the launch + ramp cost is paid once for 12 or 22 MB.

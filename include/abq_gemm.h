@@ -101,8 +101,11 @@ typedef enum abq_strategy {
     ABQ_STRATEGY_GENERIC = 4, /* any 1..16 bit pair, runtime loops (slow, always available) */
     ABQ_STRATEGY_DECODE = 5,  /* int8 MFMA 16x16x64, activations expanded once per workgroup
                                  into LDS, persistent grid; tile tuples with NSTAGE = 3       */
-    ABQ_STRATEGY_TILED = 6    /* int8 MFMA 32x32x32, LDS-staged, operands in the K-tiled plane
+    ABQ_STRATEGY_TILED = 6,   /* int8 MFMA 32x32x32, LDS-staged, operands in the K-tiled plane
                                  layout (see abq_relayout_planes); tile tuples with NSTAGE = 4 */
+    ABQ_STRATEGY_FP6 = 7      /* FP6 (E2M3) MFMA 32x32x64 at twice the int8 rate, exact for operands
+                                 of at most 4 bits unsigned / 5 bits signed (see
+                                 abq_relayout_planes_fp6); tile tuples with NSTAGE = 5, MMA 32x32x64 */
 } abq_strategy;
 
 /* Parses "AqBMMA_8x2xtrue_1x48x512_8x24x128_8x8x128_4" (an optional _InitFn/_ExecFn suffix is
@@ -260,7 +263,8 @@ abq_status abq_quant_pack_f16(const void *x_f16, int rows, int k, int bits, int 
  * ------------------------------------------------------------------------------------- */
 typedef enum abq_layout {
     ABQ_LAYOUT_PLANES = 0, /* the reference's wire format */
-    ABQ_LAYOUT_TILED = 1
+    ABQ_LAYOUT_TILED = 1,
+    ABQ_LAYOUT_FP6 = 2     /* records of 6-bit sign-magnitude codes, see below */
 } abq_layout;
 
 /* bytes of a packed operand in either layout */
@@ -270,13 +274,29 @@ size_t abq_planes_bytes(int rows, int k, int bits);
 abq_status abq_relayout_planes(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits,
                                void *stream);
 
-/* Declares the layout of X and W of an initialised state.  A tiled operand moves a state whose
- * tile was the library's choice to ABQ_STRATEGY_TILED; a state initialised with an explicit
- * non-tiled tile tuple is refused (ABQ_ERR_UNSUPPORTED). */
+/* FP6 records (no counterpart in the reference): the operand format of ABQ_STRATEGY_FP6.
+ * CDNA4's matrix cores multiply 6-bit floats (E2M3) at twice their int8 rate, and an integer of
+ * magnitude <= 16 written as sign and magnitude is an E2M3 number (value / 8), so operands that
+ * are unsigned of at most 4 bits or signed of at most 5 bits run there with bit-exact int32
+ * results as long as max|x| * max|w| * K < 2^24 (fp32 accumulation of integers).  A record is
+ * 24 words per row and K tile of 128 elements: fp6[k/128][rows][24], 3/4 byte per element
+ * whatever the bit width.  abq_fp6_eligible tells whether a bit pair and K qualify. */
+size_t abq_fp6_bytes(int rows, int k);
+int abq_fp6_eligible(int x_bits, int w_bits, int is_signed, int k);
+/* planes [bits][rows][k/32] -> fp6 [k/128][rows][24]; bits <= 4, or <= 5 if is_signed. */
+abq_status abq_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int rows, int k, int bits,
+                                   int is_signed, void *stream);
+
+/* Declares the layout of X and W of an initialised state.  A tiled (FP6) operand moves a state
+ * whose tile was the library's choice to ABQ_STRATEGY_TILED (ABQ_STRATEGY_FP6); a state
+ * initialised with an explicit tile tuple of another strategy is refused (ABQ_ERR_UNSUPPORTED),
+ * and so are a tiled and an FP6 operand together, an FP6 operand with group scales, and an FP6
+ * operand of a bit pair or K that does not qualify. */
 abq_status abq_gemm_set_operand_layout(abq_gemm_state *state, int x_layout, int w_layout);
 
-/* Workspace needed by abq_gemm_exec if the state ran as ABQ_STRATEGY_TILED with its current
- * operand layouts (0 if both operands are tiled). */
+/* Workspace needed by abq_gemm_exec if the state ran as ABQ_STRATEGY_TILED (ABQ_STRATEGY_FP6)
+ * with its current operand layouts: the converted copies of the operands still in the reference
+ * layout (0 if neither is). */
 size_t abq_gemm_workspace_bytes(const abq_gemm_state *state);
 
 /* Hands a caller-owned device buffer to the state.  If the tile was the library's choice, M > 16

@@ -28,7 +28,7 @@ def planes_dev(planes):
 def run_cfg(abq, xd, wd, signed, cfg=None, **kw):
     """Runs one configuration; kernels on the K-tiled layout get the workspace they ask for."""
     g = abq.Gemm(xd, wd, signed, cfg=cfg, **kw)
-    if g.strategy == "tiled" and g.workspace_bytes and "workspace" not in kw:
+    if g.strategy in ("tiled", "fp6") and g.workspace_bytes and "workspace" not in kw:
         ws = torch.empty(g.workspace_bytes, dtype=torch.uint8, device="cuda")
         g = abq.Gemm(xd, wd, signed, cfg=cfg, workspace=ws, **kw)
     return g.run()
@@ -146,6 +146,160 @@ def test_tiled_kernels_with_prepared_operands(abq, oracle):
         cfg = [c for c in abq.native_configs(q, p, signed) if c.nstage == 4][0]
         with pytest.raises(abq.AbqError):
             abq.Gemm(xd, wd, signed, cfg=cfg).run()
+
+
+# ------------------------------------------------------------------ FP6 matrix-core route
+
+def fp6_records(values):
+    """FP6 records written out from their definition: values [rows, K] -> uint32 [K/128, rows, 24].
+    An element's code is (sign << 5) | |value|.  A word-set (32 consecutive K elements) is a string
+    of 192 bits, position p (bits [6p, 6p+6)) holding element 31 - 8*(p % 4) - p // 4; a record has
+    word-set ws at words [12*(ws & 1) + 6*(ws >> 1), +6)."""
+    rows, K = values.shape
+    kt = K // 128
+    v = values.astype(np.int64).reshape(rows, kt, 4, 32)
+    code = (np.where(v < 0, 32, 0) | np.abs(v)).astype(np.uint64)
+    pos = np.arange(32)
+    ordered = code[..., 31 - 8 * (pos % 4) - pos // 4]  # [rows, kt, ws, p]
+    rec = np.zeros((kt, rows, 24), dtype=np.uint32)
+    for ws in range(4):
+        words = np.zeros((rows, kt, 6), dtype=np.uint64)
+        for pp in range(32):
+            bit = 6 * pp
+            w0, sh = bit // 32, bit % 32
+            words[..., w0] |= (ordered[:, :, ws, pp] << np.uint64(sh)) & np.uint64(0xFFFFFFFF)
+            if sh > 26:
+                words[..., w0 + 1] |= ordered[:, :, ws, pp] >> np.uint64(32 - sh)
+        off = 12 * (ws & 1) + 6 * (ws >> 1)
+        rec[:, :, off:off + 6] = words.astype(np.uint32).transpose(1, 0, 2)
+    return rec
+
+
+FP6_OPERANDS = [(1, False), (2, False), (3, False), (4, False), (2, True), (3, True), (4, True), (5, True)]
+
+
+def test_relayout_planes_fp6_matches_closed_form(abq, oracle):
+    rng = np.random.default_rng(61)
+    for bits, signed in FP6_OPERANDS:
+        for rows, k in [(1, 128), (5, 256), (40, 1152), (67, 4096)]:
+            vals = rand_vals(rng, rows, k, bits, signed)
+            vals[0, :4] = [oracle.value_range(bits, signed)[0], oracle.value_range(bits, signed)[1], 0, vals[0, 3]]
+            got = abq.relayout_planes_fp6(planes_dev(oracle.pack_i32(vals, bits)), signed).cpu().numpy().view(np.uint32)
+            assert np.array_equal(got, fp6_records(vals)), (bits, signed, rows, k)
+    with pytest.raises(abq.AbqError):  # 5 bits unsigned / 6 bits signed have no exact FP6 form
+        abq.relayout_planes_fp6(planes_dev(oracle.pack_i32(rand_vals(rng, 4, 128, 5, False), 5)), False)
+    with pytest.raises(abq.AbqError):
+        abq.relayout_planes_fp6(planes_dev(oracle.pack_i32(rand_vals(rng, 4, 128, 6, True), 6)), True)
+
+
+def test_fp6_gemm_every_eligible_pair_and_tile(abq, oracle):
+    """FP6 route against the oracle: every eligible bit pair (also pairs without a popcount / int8
+    specialisation), every tile, ragged shapes, prepared and per-call converted operands."""
+    rng = np.random.default_rng(62)
+    shapes = [(33, 70, 128), (100, 200, 384), (300, 129, 640), (64, 257, 1152)]
+    cfg44 = [c for c in abq.native_configs(4, 4, True) if c.nstage == 5]
+    assert len(cfg44) >= 4 and all(c.mma_k == 64 for c in cfg44)
+    for signed in (True, False):
+        widths = [b for b, s in FP6_OPERANDS if s == signed]
+        for q in widths:
+            for p in widths:
+                M, N, K = shapes[(q + p) % len(shapes)]
+                assert abq.fp6_eligible(q, p, signed, K)
+                x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+                xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
+                xf, wf = abq.relayout_planes_fp6(xd, signed), abq.relayout_planes_fp6(wd, signed)
+                want = oracle.np_gemm(x, w)
+                for c in cfg44:
+                    cfg = abq.TileConfig(q, p, int(signed), c.block_m, c.block_n, c.block_k, c.warp_m, c.warp_n,
+                                         c.warp_k, c.mma_m, c.mma_n, c.mma_k, c.nstage)
+                    out = torch.full((M, N), -777, dtype=torch.int32, device="cuda")
+                    got = abq.gemm(xf, wf, signed, cfg=cfg, x_fp6=q, w_fp6=p, out=out).cpu().numpy()
+                    assert np.array_equal(got, want), (abq.format_kernel_name(cfg), M, N, K)
+                # activations converted inside the call, weights prepared; the library picks the tile
+                g = abq.Gemm(xd, wf, signed, w_fp6=p)
+                assert g.strategy == "fp6" and g.workspace_bytes == (K // 128) * M * 96
+                ws = torch.empty(g.workspace_bytes, dtype=torch.uint8, device="cuda")
+                got = abq.gemm(xd, wf, signed, w_fp6=p, workspace=ws).cpu().numpy()
+                assert np.array_equal(got, want), (q, p, signed)
+                with pytest.raises(abq.AbqError):  # no workspace for the activations
+                    g.run()
+
+
+def test_fp6_gemm_range_ends_and_limits(abq, oracle):
+    """Largest magnitudes over the longest K the route accepts: the fp32 accumulation stays exact."""
+    for q, p, signed, K in [(4, 4, False, 65536), (5, 5, True, 65536 - 128), (4, 4, True, 13824), (5, 2, True, 13824)]:
+        assert abq.fp6_eligible(q, p, signed, K)
+        xlo, xhi = oracle.value_range(q, signed)
+        wlo, whi = oracle.value_range(p, signed)
+        M, N = 40, 72
+        x = np.full((M, K), xlo if signed else xhi, dtype=np.int32)
+        w = np.full((N, K), wlo if signed else whi, dtype=np.int32)
+        x[1::2] = xhi
+        w[1::3] = whi
+        x[5, ::7] = 0
+        xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
+        got = abq.gemm(abq.relayout_planes_fp6(xd, signed), abq.relayout_planes_fp6(wd, signed), signed,
+                       x_fp6=q, w_fp6=p).cpu().numpy()
+        assert np.array_equal(got, oracle.np_gemm(x, w)), (q, p, signed, K)
+    rng = np.random.default_rng(63)
+    # beyond the exactness bound, wider operands, group scales and mixed layouts are refused
+    assert not abq.fp6_eligible(4, 4, False, 131072 - 128) and not abq.fp6_eligible(5, 5, True, 65536)
+    assert not abq.fp6_eligible(5, 4, False, 128) and not abq.fp6_eligible(6, 2, True, 128)
+    x, w = rand_vals(rng, 32, 256, 8, True), rand_vals(rng, 64, 256, 2, True)
+    xd, wd = planes_dev(oracle.pack_i32(x, 8)), planes_dev(oracle.pack_i32(w, 2))
+    wf = abq.relayout_planes_fp6(wd, True)
+    with pytest.raises(abq.AbqError):
+        abq.Gemm(xd, wf, True, w_fp6=2)  # 8-bit activations
+    x4 = rand_vals(rng, 32, 256, 4, True)
+    x4d = planes_dev(oracle.pack_i32(x4, 4))
+    with pytest.raises(abq.AbqError):
+        abq.Gemm(abq.relayout_planes(x4d), wf, True, x_tiled=True, w_fp6=2)  # tiled and FP6 together
+    sc = torch.ones(64 * 2, dtype=torch.float32, device="cuda")
+    with pytest.raises(abq.AbqError):
+        abq.Gemm(x4d, wf, True, w_fp6=2, out_kind=abq.OUT_F16_SCALED, x_scale=sc, w_scale=sc, group_size=128)
+
+
+def test_fp6_fp16_epilogues(abq, oracle):
+    rng = np.random.default_rng(64)
+    M, N, K, q, p = 130, 200, 512, 4, 4
+    x, w = rand_vals(rng, M, K, q, True), rand_vals(rng, N, K, p, True)
+    xf = abq.relayout_planes_fp6(planes_dev(oracle.pack_i32(x, q)), True)
+    wf = abq.relayout_planes_fp6(planes_dev(oracle.pack_i32(w, p)), True)
+    acc = oracle.np_gemm(x, w)
+    xs = torch.rand(M, device="cuda") * 0.01 + 0.001
+    ws = torch.rand(N, device="cuda") * 0.01 + 0.001
+    got = abq.gemm(xf, wf, True, x_fp6=q, w_fp6=p, out_kind=abq.OUT_F16_SCALED, x_scale=xs, w_scale=ws).float().cpu().numpy()
+    want = acc.astype(np.float64) * xs.cpu().numpy().astype(np.float64)[:, None] * ws.cpu().numpy().astype(np.float64)[None, :]
+    assert np.all(np.abs(got - want) <= 1e-2 * np.abs(want) + 1e-6)  # tolerance of the fp16 dequantised output: 1e-2 relative
+    c = torch.tensor([0.03125], dtype=torch.float16, device="cuda")
+    got = abq.gemm(xf, wf, True, x_fp6=q, w_fp6=p, out_kind=abq.OUT_F16_TENSOR, c_scale=c).cpu().numpy()
+    want16 = (acc.astype(np.float32).astype(np.float16) * np.float16(0.03125)).astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want16.view(np.uint16))
+
+
+@pytest.mark.parametrize("signed", [True, False])
+def test_config2_w4a4_prefill_full_size_fp6(abq, oracle, signed):
+    """W4A4 at M in {512, 2048} on the LLaMA-7B shapes through the FP6 route: exact against the fp64
+    closed form and the CPU oracle on sampled rows, and identical to the int8 tiled kernel."""
+    rng = np.random.default_rng(2000 + int(signed))
+    for (N, K) in [(4096, 4096), (11008, 4096), (4096, 11008)]:
+        w = rand_vals(rng, N, K, 4, signed)
+        wp = oracle.pack_i32(w, 4)
+        wd = planes_dev(wp)
+        wf6 = abq.relayout_planes_fp6(wd, signed)
+        wfd = torch.from_numpy(w).cuda().double()
+        for M in (512, 2048):
+            x = rand_vals(rng, M, K, 4, signed)
+            xp = oracle.pack_i32(x, 4)
+            xd = planes_dev(xp)
+            ws = torch.empty((K // 128) * M * 96, dtype=torch.uint8, device="cuda")
+            g = abq.Gemm(xd, wf6, signed, w_fp6=4, workspace=ws)
+            assert g.strategy == "fp6"
+            got_d = g.run()
+            ref = torch.from_numpy(x).cuda().double() @ wfd.T
+            assert torch.equal(got_d.double(), ref), (signed, M, N, K)
+            _sampled_oracle_check(oracle, xp, wp, signed, got_d.cpu().numpy(), rng, rows=2)
+            del ref
 
 
 # ------------------------------------------------------------------ GEMM: every native tile, every combination

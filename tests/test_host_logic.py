@@ -249,6 +249,33 @@ def test_native_configs_resolve_to_themselves(abq, q, p):
     assert abq.native_configs(9, 9, 1) == []
 
 
+def test_fp6_route_eligibility_and_tile_tuples(abq):
+    """The FP6 matrix-core route takes operands that are E2M3 numbers (unsigned <= 4 bits, signed
+    <= 5) while max|x| * max|w| * K stays below 2^24; its tiles are named MMA 32x32x64, NSTAGE 5."""
+    for q in range(1, 9):
+        for p in range(1, 9):
+            for signed in (0, 1):
+                lim = 5 if signed else 4
+                mx = (1 << (q - 1)) if signed else (1 << q) - 1
+                mw = (1 << (p - 1)) if signed else (1 << p) - 1
+                for K in (128, 4096, 13824, 65536, 1 << 20):
+                    want = q <= lim and p <= lim and mx * mw * K < (1 << 24)
+                    assert abq.fp6_eligible(q, p, signed, K) == want, (q, p, signed, K)
+    assert abq.lib().abq_fp6_bytes(10, 256) == 10 * 2 * 96 and abq.lib().abq_fp6_bytes(10, 200) == 0
+    cfg, _ = abq.parse_kernel_name("AqBMMA_4x4xtrue_256x128x128_64x64x128_32x32x64_5")
+    rc, st = _init(abq, cfg=cfg, M=2048, N=4096, K=4096)
+    assert rc == 0 and st.strategy == abq.STRATEGY_FP6
+    assert st.grid_dim.x == 8 * 4 * 8 and st.block_dim.x == 512 and st.shared_mem_size == 2 * 384 * 112
+    # not eligible: 8-bit activations; K beyond the exactness bound; unknown tile
+    cfg, _ = abq.parse_kernel_name("AqBMMA_8x2xtrue_256x128x128_64x64x128_32x32x64_5")
+    assert _init(abq, cfg=cfg, M=64, N=64, K=256)[0] == abq.ABQ_ERR_UNSUPPORTED
+    cfg, _ = abq.parse_kernel_name("AqBMMA_4x4xfalse_128x128x128_64x64x128_32x32x64_5")
+    assert _init(abq, cfg=cfg, M=64, N=64, K=65536)[0] == 0
+    assert _init(abq, cfg=cfg, M=64, N=64, K=131072)[0] == abq.ABQ_ERR_UNSUPPORTED
+    cfg, _ = abq.parse_kernel_name("AqBMMA_4x4xfalse_96x128x128_96x64x128_32x32x64_5")
+    assert _init(abq, cfg=cfg, M=64, N=64, K=256)[0] == abq.ABQ_ERR_UNSUPPORTED
+
+
 # ------------------------------------------------------------------ tile generator
 
 @pytest.fixture(scope="module")
