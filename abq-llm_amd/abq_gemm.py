@@ -232,20 +232,21 @@ def relayout_planes_fp6(planes, signed, out=None, stream=None):
     return out
 
 
-def quant_pack_f16(x, bits, symmetric=True, tiled=False, group_size=0, stream=None):
+def quant_pack_f16(x, bits, symmetric=True, tiled=False, group_size=0, stream=None, fp6=False):
     """Per-token dynamic quantisation + packing of fp16 activations [rows, k].
 
     Returns (planes, scale[rows], zero[rows] or None, group_sums[rows, k/group_size] or None);
-    planes hold signed codes, [bits, rows, k/32] or K-tiled [k/128, rows, bits, 4]."""
+    planes hold signed codes, [bits, rows, k/32], K-tiled [k/128, rows, bits, 4] or FP6 records
+    [k/128, rows, 24] (bits <= 5)."""
     import torch
-    assert x.dtype == torch.float16 and x.is_cuda and x.is_contiguous()
+    assert x.dtype == torch.float16 and x.is_cuda and x.is_contiguous() and not (tiled and fp6)
     rows, k = x.shape
-    shape = (k // 128, rows, bits, 4) if tiled else (bits, rows, k // 32)
+    shape = (k // 128, rows, 24) if fp6 else (k // 128, rows, bits, 4) if tiled else (bits, rows, k // 32)
     planes = torch.empty(shape, dtype=torch.int32, device=x.device)
     scale = torch.empty(rows, dtype=torch.float32, device=x.device)
     zero = None if symmetric else torch.empty(rows, dtype=torch.float32, device=x.device)
     sums = torch.empty((rows, k // group_size), dtype=torch.int32, device=x.device) if group_size else None
-    _check(lib().abq_quant_pack_f16(x.data_ptr(), rows, k, bits, int(bool(symmetric)), int(bool(tiled)),
+    _check(lib().abq_quant_pack_f16(x.data_ptr(), rows, k, bits, int(bool(symmetric)), LAYOUT_FP6 if fp6 else int(bool(tiled)),
                                     planes.data_ptr(), scale.data_ptr(),
                                     zero.data_ptr() if zero is not None else None,
                                     sums.data_ptr() if sums is not None else None, group_size,

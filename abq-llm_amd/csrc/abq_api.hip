@@ -810,15 +810,16 @@ abq_status abq_quant_pack_f16(const void *x_f16, int rows, int k, int bits, int 
         return ABQ_ERR_INVALID_ARG;
     if (!symmetric && !zero)
         return ABQ_ERR_INVALID_ARG;
-    if (layout != ABQ_LAYOUT_PLANES && layout != ABQ_LAYOUT_TILED)
+    if (layout < ABQ_LAYOUT_PLANES || layout > ABQ_LAYOUT_FP6)
         return ABQ_ERR_INVALID_ARG;
+    if (layout == ABQ_LAYOUT_FP6 && bits > 5) // the codes are signed: magnitude at most 16
+        return ABQ_ERR_UNSUPPORTED;
     if (k < 128 || k % 128 != 0)
         return ABQ_ERR_BAD_K;
     if (group_sums && group_size != 64 && group_size != 128)
         return ABQ_ERR_UNSUPPORTED;
     return hip_status(launch_quant_pack_rows(x_f16, planes, scale, zero, group_sums, rows, k, bits, symmetric ? 1 : 0,
-                                             group_sums ? group_size : 128, layout == ABQ_LAYOUT_TILED,
-                                             (hipStream_t)stream));
+                                             group_sums ? group_size : 128, layout, (hipStream_t)stream));
 }
 
 abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)

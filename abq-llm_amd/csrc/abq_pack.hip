@@ -344,7 +344,8 @@ __device__ __forceinline__ float wave_max(float v)
     return v;
 }
 
-template <bool TILED>
+// LAYOUT: 0 planes, 1 field-packed K tiles, 2 FP6 records (codes of at most 5 bits).
+template <int LAYOUT>
 __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__restrict__ x, uint32_t *__restrict__ planes,
                                                               float *__restrict__ scale_out, float *__restrict__ zero_out,
                                                               int *__restrict__ group_sums, int M, int K, int bits,
@@ -429,7 +430,31 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
                 group_sums[(size_t)row * (K / group_size) + u / lanes_per_group] = sum;
         }
         const int quad_lane = u & 3, w = u >> 2; // w: word-set (32 elements) within the row
-        if (TILED) {
+        if (LAYOUT == 2) {
+            // position p = 4 s + c of the word-set's 192-bit string holds element 31 - (8c + s): this lane's
+            // element j goes to position 4 (7 - j) + 3 - quad_lane as the code (sign << 5) | magnitude
+            uint32_t o[6] = { 0u, 0u, 0u, 0u, 0u, 0u };
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t code = v[j] < 0 ? (32u | (uint32_t)(-v[j])) : (uint32_t)v[j];
+                constexpr int kBase[8] = { 168, 144, 120, 96, 72, 48, 24, 0 }; // 24 (7 - j)
+                const int d0 = kBase[j] >> 5;                                   // first dword the code can touch
+                const uint64_t wide = (uint64_t)code << ((kBase[j] & 31) + 6 * (3 - quad_lane));
+                o[d0] |= (uint32_t)wide;
+                if (d0 + 1 < 6)
+                    o[d0 + 1] |= (uint32_t)(wide >> 32);
+            }
+#pragma unroll
+            for (int d = 0; d < 6; ++d)
+                o[d] = quad_or(o[d]);
+            if (active && quad_lane == 0) {
+                const int ws = w & 3;
+                uint32_t *rec = planes + ((size_t)(w >> 2) * M + row) * 24 + 12 * (ws & 1) + 6 * (ws >> 1);
+                *reinterpret_cast<uint2 *>(rec) = make_uint2(o[0], o[1]);
+                *reinterpret_cast<uint2 *>(rec + 2) = make_uint2(o[2], o[3]);
+                *reinterpret_cast<uint2 *>(rec + 4) = make_uint2(o[4], o[5]);
+            }
+        } else if (LAYOUT == 1) {
             // expanded dword s, byte c = element 31 - (8c + s) of the word-set: this lane's element
             // 7 - s goes to byte 3 - quad_lane
             const uint32_t pattern_mask = (1u << bits) - 1u;
@@ -452,15 +477,19 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
 }
 
 hipError_t launch_quant_pack_rows(const void *x, uint32_t *planes, float *scale, float *zero, int *group_sums,
-                                  int M, int K, int bits, int symmetric, int group_size, int tiled,
+                                  int M, int K, int bits, int symmetric, int group_size, int layout,
                                   hipStream_t stream)
 {
-    if (tiled)
-        hipLaunchKernelGGL(quant_pack_rows_kernel<true>, dim3(M), dim3(256), 0, stream,
+    if (layout == 2)
+        hipLaunchKernelGGL(quant_pack_rows_kernel<2>, dim3(M), dim3(256), 0, stream,
+                           reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits,
+                           symmetric, group_size);
+    else if (layout == 1)
+        hipLaunchKernelGGL(quant_pack_rows_kernel<1>, dim3(M), dim3(256), 0, stream,
                            reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits,
                            symmetric, group_size);
     else
-        hipLaunchKernelGGL(quant_pack_rows_kernel<false>, dim3(M), dim3(256), 0, stream,
+        hipLaunchKernelGGL(quant_pack_rows_kernel<0>, dim3(M), dim3(256), 0, stream,
                            reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits,
                            symmetric, group_size);
     return hipGetLastError();

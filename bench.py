@@ -256,6 +256,45 @@ def main():
                 del wpl, wtl
         extra["prefill"] = prefill
 
+        # The same W4A4 GEMMs on the FP6 matrix-core route (exact for operands of at most 4 bits unsigned /
+        # 5 bits signed): weights prepared once as FP6 records; activations either converted from planes inside
+        # the timed call, as above, or already FP6 (what the fused quantise-and-pack kernel hands over).
+        prefill_fp6 = []
+        for signed in (True, False):
+            for (N, K) in SHAPES:
+                wf6 = abq.relayout_planes_fp6(random_planes(torch, (4, N, K // 32)), signed)
+                for M in (512, 2048):
+                    xpl = random_planes(torch, (4, M, K // 32))
+                    xf6 = abq.relayout_planes_fp6(xpl, signed)
+                    ws = torch.empty((K // 128) * M * 96, dtype=torch.uint8, device="cuda")
+                    row = dict(w_bits=4, x_bits=4, signed=signed, M=M, N=N, K=K)
+                    for tag, gm in (("planes_in", abq.Gemm(xpl, wf6, signed, w_fp6=4, workspace=ws)),
+                                    ("fp6_in", abq.Gemm(xf6, wf6, signed, x_fp6=4, w_fp6=4))):
+                        gm.run()
+                        torch.cuda.synchronize()
+                        reps = 5
+                        gr = torch.cuda.CUDAGraph()
+                        with torch.cuda.graph(gr):
+                            for _ in range(reps):
+                                gm.run()
+                        gr.replay()
+                        torch.cuda.synchronize()
+                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        e0.record()
+                        gr.replay()
+                        e1.record()
+                        torch.cuda.synchronize()
+                        us = e0.elapsed_time(e1) * 1e3 / reps
+                        del gr
+                        tops = 2.0 * M * N * K / (us * 1e-6) / 1e12
+                        row[tag] = dict(us=round(us, 1), tops=round(tops, 2), mfma_int8_frac=round(tops / INT8_MFMA_PEAK_TOPS, 4))
+                        row["kernel"] = "%s:%s" % (gm.strategy, gm.config_name)
+                        del gm
+                    prefill_fp6.append(row)
+                    del xpl, xf6, ws
+                del wf6
+        extra["prefill_fp6"] = prefill_fp6
+
         # Yardstick for the prefill figures: the vendor library's plain int8 GEMM (torch._int_mm, operands
         # already int8 and K-major, nothing to unpack) on the same shapes, timed the same way.
         vendor = []

@@ -244,7 +244,7 @@ abq_status abq_weight_zero_term(const uint32_t *w_planes, int n, int k, int bits
  *   symmetric == 0: scale = clamp((max - min) / (2^bits - 1), 1e-5, 1e4),
  *                   zp = round(clamp(-min / scale, -1e4, 1e4)), stored code = u - 2^(bits-1),
  *                   zero = zp - 2^(bits-1)
- * fp32 arithmetic, round half to even.  2 <= bits <= 8, k % 128 == 0. */
+ * fp32 arithmetic, round half to even.  2 <= bits <= 8 (<= 5 for ABQ_LAYOUT_FP6), k % 128 == 0. */
 abq_status abq_quant_pack_f16(const void *x_f16, int rows, int k, int bits, int symmetric, int layout,
                               uint32_t *planes, float *scale, float *zero, int32_t *group_sums,
                               int group_size, void *stream);

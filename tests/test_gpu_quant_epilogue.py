@@ -52,7 +52,7 @@ def run_grouped(abq, xp, wp, signed, strategy="tiled", **kw):
 
 @pytest.mark.parametrize("rows,k,bits,symmetric", [(1, 128, 8, True), (5, 4096, 8, True), (33, 11008, 8, False),
                                                    (7, 256, 4, True), (16, 1152, 4, False), (3, 384, 2, True),
-                                                   (64, 4096, 6, False)])
+                                                   (64, 4096, 6, False), (9, 640, 5, False), (12, 512, 3, True)])
 def test_quant_pack_matches_the_restated_quantizer(abq, oracle, rows, k, bits, symmetric):
     from oracle import quantizer as Q
     rng = np.random.default_rng(rows + k + bits)
@@ -70,6 +70,13 @@ def test_quant_pack_matches_the_restated_quantizer(abq, oracle, rows, k, bits, s
     # K-tiled output equals the relayout of the plane output
     tiled, _, _, _ = abq.quant_pack_f16(torch.from_numpy(x).cuda(), bits, symmetric=symmetric, tiled=True)
     assert torch.equal(tiled, abq.relayout_planes(planes))
+    # FP6 records (codes of at most 5 bits) equal the FP6 relayout of the plane output
+    if bits <= 5:
+        rec, s6, _, _ = abq.quant_pack_f16(torch.from_numpy(x).cuda(), bits, symmetric=symmetric, fp6=True)
+        assert torch.equal(rec, abq.relayout_planes_fp6(planes, True)) and torch.equal(s6, s)
+    else:
+        with pytest.raises(abq.AbqError):
+            abq.quant_pack_f16(torch.from_numpy(x).cuda(), bits, symmetric=symmetric, fp6=True)
 
 
 # ------------------------------------------------------------------ group scales, zero points
