@@ -235,7 +235,7 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
         st->grid_dim = abq_dim3{ (unsigned)(8 * npx * mblocks), 1, 1 };
         st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
-        st->shared_mem_size = 2 * (size_t)(bm + bn) * 112;
+        st->shared_mem_size = 2 * (size_t)(bm + bn) * 96;
         return ABQ_OK;
     }
     const KernelTable *tm_ = find_table(reg.mfma, x_bits, w_bits, is_signed);

@@ -18,8 +18,8 @@
 // elements is one record of 96 bytes = four 192-bit strings of 32 six-bit codes; strings 0 and 1
 // feed lanes 0-31 of the two MFMA K steps of the tile, strings 2 and 3 lanes 32-63, so a lane
 // fetches both steps with three aligned ds_read_b128.  Records are stored tiled[kt][row][96 B].
-// Nothing is unpacked in this kernel: global -> registers -> LDS (rows 112 bytes apart, conflict
-// free for b128) -> MFMA.  LDS is double buffered, one barrier per K tile; workgroup -> tile
+// Nothing is unpacked in this kernel: global -> registers -> LDS (the records as they are, 16-byte
+// units swapped in pairs in every second 256-byte line: conflict free for b128 writes and reads) -> MFMA.  LDS is double buffered, one barrier per K tile; workgroup -> tile
 // mapping keeps a band of N per XCD as in the int8 tiled kernel.
 #include "abq_kernels.h"
 
@@ -31,14 +31,21 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4))); // a 16-byte piece (a native vector: copies stay in registers)
 
 constexpr int kFp6Units = 6;      // 16-byte units per record
-constexpr int kFp6LdsRow = 112;   // bytes per row in LDS (96 + 16 padding)
+constexpr int kFp6LdsRow = 96;    // bytes per row in LDS: the records as they are, no padding
+
+// LDS placement of 16-byte unit `pos` of an operand block (pos = row * 6 + unit): units are swapped
+// in pairs inside every second 256-byte line.  A wave's global load of 64 consecutive units then
+// lands as four conflict-free ds_write_b128 (each group of sixteen lanes fills one line), and the
+// fragment reads (sixteen lanes = sixteen consecutive rows, same unit: positions 6 apart, which
+// alone would meet in pairs eight rows = three lines apart) hit sixteen different bank groups.
+__device__ __forceinline__ int fp6_lds_offset(int pos) { return (pos ^ ((pos >> 4) & 1)) * 16; }
 
 // One lane's share of a 32-row fragment for both K steps of a tile: 48 bytes, three ds_read_b128.
-__device__ __forceinline__ void load_fragment(v8i (&f)[2], const unsigned char *p)
+__device__ __forceinline__ void load_fragment(v8i (&f)[2], const unsigned char *base, const int (&off)[3])
 {
-    const v4i q0 = *reinterpret_cast<const v4i *>(p);
-    const v4i q1 = *reinterpret_cast<const v4i *>(p + 16);
-    const v4i q2 = *reinterpret_cast<const v4i *>(p + 32);
+    const v4i q0 = *reinterpret_cast<const v4i *>(base + off[0]);
+    const v4i q1 = *reinterpret_cast<const v4i *>(base + off[1]);
+    const v4i q2 = *reinterpret_cast<const v4i *>(base + off[2]);
     const v8i lo = __builtin_shufflevector(q0, q1, 0, 1, 2, 3, 4, 5, 6, 7);
     const v8i hi = __builtin_shufflevector(q1, q2, 2, 3, 4, 5, 6, 7, -1, -1);
     f[0] = __builtin_shufflevector(lo, lo, 0, 1, 2, 3, 4, 5, -1, -1);
@@ -46,7 +53,7 @@ __device__ __forceinline__ void load_fragment(v8i (&f)[2], const unsigned char *
 }
 
 // This thread's share of one operand's tile: pieces of 16 bytes, piece p = tid + NT * i
-// (ROWS is a multiple of 16).
+// (ROWS is a multiple of 32).
 template <int ROWS, int NT> struct Fp6Stage {
     static constexpr int kPieces = ROWS * kFp6Units;
     static constexpr int NP = (kPieces + NT - 1) / NT;
@@ -58,13 +65,11 @@ template <int ROWS, int NT> struct Fp6Stage {
     {
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
-            // sixteen consecutive lanes take the same unit of sixteen consecutive rows: their LDS writes
-            // are 112 bytes apart and hit sixteen different groups of four banks
-            const int p = tid + NT * i;
-            const int rr = (p >> 4) / kFp6Units * 16 + (p & 15), u = (p >> 4) % kFp6Units;
+            const int p = tid + NT * i; // consecutive lanes, consecutive units: a wave loads 1 KiB in one piece
+            const int rr = p / kFp6Units, u = p % kFp6Units;
             const bool have = !kRagged || i + 1 < NP || p < kPieces;
             g[i] = (uint32_t)min(row0 + (have ? rr : 0), rows - 1) * kFp6Units + u;
-            l[i] = have ? rr * kFp6LdsRow + u * 16 : -1;
+            l[i] = have ? fp6_lds_offset(p) : -1;
         }
     }
     static __device__ __forceinline__ void load(v4u (&r)[NP], const v4u *tile, const uint32_t (&g)[NP])
@@ -92,7 +97,7 @@ void gemm_mfma_fp6(const GemmArgs a, const v4u *xt, const v4u *wt, int m_blocks,
     using StageA = Fp6Stage<BM, NT>;
     using StageB = Fp6Stage<BN, NT>;
 
-    extern __shared__ __align__(16) unsigned char smem[]; // [2][BM + BN][112]
+    extern __shared__ __align__(16) unsigned char smem[]; // [2][BM + BN][96]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -127,16 +132,24 @@ void gemm_mfma_fp6(const GemmArgs a, const v4u *xt, const v4u *wt, int m_blocks,
 
     unsigned char *lds_a = smem;
     unsigned char *lds_b = smem + BM * kFp6LdsRow;
-    // Software pipeline, two K tiles deep at every level.  While the MFMAs of tile t run out of one
-    // set of fragment registers, the ds_reads of tile t + 1 fill the other set, tile t + 2 waits in
-    // a register slot for its turn to be written to LDS (end of tile t, into the buffer tile t
-    // occupied) and the global loads of tile t + 3 are issued into the other slot.  Everything is
-    // unrolled by two with named arrays, so every register index is a constant.  Tiles past the end
+    // Software pipeline.  While the MFMAs of tile t run out of one set of fragment registers, the
+    // ds_reads of tile t + 1 fill the other set, tiles t + 2 .. t + D wait in register slots (tile
+    // t + 2 is written to LDS at the end of tile t, into the buffer tile t occupied) and the global
+    // loads of tile t + 1 + D are issued into the slot tile t + 1 left: D - 1 whole K tiles of MFMAs
+    // hide a load.  Everything is unrolled (by six for three slots) with named arrays, so every
+    // register index is a constant.  Tiles past the end
     // are clamped to the last one: their copies land in buffers and registers nobody uses again.
-    v4u ra0[StageA::NP], rb0[StageB::NP], ra1[StageA::NP], rb1[StageB::NP];
+    v4u ra0[StageA::NP], rb0[StageB::NP], ra1[StageA::NP], rb1[StageB::NP], ra2[StageA::NP], rb2[StageB::NP];
     v8i fa0[TM][2], fb0[TN][2], fa1[TM][2], fb1[TN][2];
-    const unsigned char *a_lane = lds_a + (wm * 32 * TM + r) * kFp6LdsRow + g * 48;
-    const unsigned char *b_lane = lds_b + (wn * 32 * TN + r) * kFp6LdsRow + g * 48;
+    // this lane's three units of a fragment row; 32 rows further on (192 units = 12 lines) and in the other
+    // buffer (a multiple of two lines) the placement repeats, so those offsets are plain constants
+    int a_off[3], b_off[3];
+#pragma unroll
+    for (int q = 0; q < 3; ++q) {
+        a_off[q] = fp6_lds_offset((wm * 32 * TM + r) * kFp6Units + 3 * g + q);
+        b_off[q] = fp6_lds_offset((wn * 32 * TN + r) * kFp6Units + 3 * g + q);
+    }
+    static_assert((32 * kFp6LdsRow) % 512 == 0, "fragment rows and buffers keep the line parity");
 #define ABQ_FP6_LOAD(KT, RA, RB)                               \
     {                                                          \
         const int kn_ = min((KT), ktiles - 1);                 \
@@ -148,15 +161,20 @@ void gemm_mfma_fp6(const GemmArgs a, const v4u *xt, const v4u *wt, int m_blocks,
 #define ABQ_FP6_READ(FA, FB, BUF)                                                   \
     {                                                                               \
         _Pragma("unroll") for (int i = 0; i < TM; ++i)                              \
-            load_fragment(FA[i], a_lane + (BUF) + i * 32 * kFp6LdsRow);             \
+            load_fragment(FA[i], lds_a + (BUF) + i * 32 * kFp6LdsRow, a_off);       \
         _Pragma("unroll") for (int j = 0; j < TN; ++j)                              \
-            load_fragment(FB[j], b_lane + (BUF) + j * 32 * kFp6LdsRow);             \
+            load_fragment(FB[j], lds_b + (BUF) + j * 32 * kFp6LdsRow, b_off);       \
     }
+    // D register slots: three where the registers allow it (eight waves share the tile: 20 registers a
+    // slot), two otherwise
+    constexpr int D = WM * WN > 4 ? 3 : 2;
     ABQ_FP6_LOAD(0, ra0, rb0)
     ABQ_FP6_LOAD(1, ra1, rb1)
+    if (D == 3)
+        ABQ_FP6_LOAD(2, ra2, rb2)
     StageA::store(ra0, lds_a, la);
     StageB::store(rb0, lds_b, lb);
-    ABQ_FP6_LOAD(2, ra0, rb0)
+    ABQ_FP6_LOAD(D, ra0, rb0) // tile D into slot D % D = 0
     StageA::store(ra1, lds_a + BUF_BYTES, la);
     StageB::store(rb1, lds_b + BUF_BYTES, lb);
     __syncthreads();
@@ -167,7 +185,7 @@ void gemm_mfma_fp6(const GemmArgs a, const v4u *xt, const v4u *wt, int m_blocks,
 #define ABQ_FP6_K_TILE(KT, FCA, FCB, FNA, FNB, RAL, RBL, RAS, RBS)                                              \
     {                                                                                                           \
         const int buf = ((KT) & 1) * BUF_BYTES;                                                                 \
-        ABQ_FP6_LOAD((KT) + 3, RAL, RBL)                                                                        \
+        ABQ_FP6_LOAD((KT) + 1 + D, RAL, RBL)                                                                    \
         __builtin_amdgcn_sched_barrier(0); /* the loads leave first: a whole tile of MFMAs hides them */        \
         ABQ_FP6_READ(FNA, FNB, BUF_BYTES - buf)                                                                 \
         _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                        \
@@ -180,13 +198,52 @@ void gemm_mfma_fp6(const GemmArgs a, const v4u *xt, const v4u *wt, int m_blocks,
         __syncthreads(); /* waits for this wave's ds_reads and ds_writes, then for the other waves */           \
     }
 
+    // fragment sets alternate (period 2), register slots rotate (period 3): six tiles per round
+#define ABQ_FP6_T0(KT) ABQ_FP6_K_TILE(KT, fa0, fb0, fa1, fb1, ra1, rb1, ra2, rb2)
+#define ABQ_FP6_T1(KT) ABQ_FP6_K_TILE(KT, fa1, fb1, fa0, fb0, ra2, rb2, ra0, rb0)
+#define ABQ_FP6_T2(KT) ABQ_FP6_K_TILE(KT, fa0, fb0, fa1, fb1, ra0, rb0, ra1, rb1)
+#define ABQ_FP6_T3(KT) ABQ_FP6_K_TILE(KT, fa1, fb1, fa0, fb0, ra1, rb1, ra2, rb2)
+#define ABQ_FP6_T4(KT) ABQ_FP6_K_TILE(KT, fa0, fb0, fa1, fb1, ra2, rb2, ra0, rb0)
+#define ABQ_FP6_T5(KT) ABQ_FP6_K_TILE(KT, fa1, fb1, fa0, fb0, ra0, rb0, ra1, rb1)
     int kt = 0;
-    for (; kt + 2 <= ktiles; kt += 2) {
-        ABQ_FP6_K_TILE(kt, fa0, fb0, fa1, fb1, ra1, rb1, ra0, rb0)
-        ABQ_FP6_K_TILE(kt + 1, fa1, fb1, fa0, fb0, ra0, rb0, ra1, rb1)
+    if (D == 3) {
+        for (; kt + 6 <= ktiles; kt += 6) {
+            ABQ_FP6_T0(kt)
+            ABQ_FP6_T1(kt + 1)
+            ABQ_FP6_T2(kt + 2)
+            ABQ_FP6_T3(kt + 3)
+            ABQ_FP6_T4(kt + 4)
+            ABQ_FP6_T5(kt + 5)
+        }
+        if (kt < ktiles) { // up to five tiles are left
+            ABQ_FP6_T0(kt)
+            if (kt + 1 < ktiles) {
+                ABQ_FP6_T1(kt + 1)
+                if (kt + 2 < ktiles) {
+                    ABQ_FP6_T2(kt + 2)
+                    if (kt + 3 < ktiles) {
+                        ABQ_FP6_T3(kt + 3)
+                        if (kt + 4 < ktiles)
+                            ABQ_FP6_T4(kt + 4)
+                    }
+                }
+            }
+        }
+    } else {
+        // two slots: tile t + 2 is written from slot t % 2 while tile t + 3 loads into slot (t + 1) % 2
+        for (; kt + 2 <= ktiles; kt += 2) {
+            ABQ_FP6_K_TILE(kt, fa0, fb0, fa1, fb1, ra1, rb1, ra0, rb0)
+            ABQ_FP6_K_TILE(kt + 1, fa1, fb1, fa0, fb0, ra0, rb0, ra1, rb1)
+        }
+        if (kt < ktiles)
+            ABQ_FP6_K_TILE(kt, fa0, fb0, fa1, fb1, ra1, rb1, ra0, rb0)
     }
-    if (kt < ktiles)
-        ABQ_FP6_K_TILE(kt, fa0, fb0, fa1, fb1, ra1, rb1, ra0, rb0)
+#undef ABQ_FP6_T0
+#undef ABQ_FP6_T1
+#undef ABQ_FP6_T2
+#undef ABQ_FP6_T3
+#undef ABQ_FP6_T4
+#undef ABQ_FP6_T5
 #undef ABQ_FP6_K_TILE
 #undef ABQ_FP6_READ
 #undef ABQ_FP6_LOAD
