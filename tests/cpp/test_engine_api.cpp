@@ -139,6 +139,50 @@ static void gpu_paths()
         CHECK(out == ref);
     }
 
+    {   // FP6 matrix-core tile by its name (W4A4 signed): weights prepared as FP6 records, activations converted
+        // per call into the workspace handed to the state
+        const Case c6{ 70, 200, 640, 4, 4, true };
+        std::vector<int> x6((size_t)c6.M * c6.K), w6((size_t)c6.N * c6.K);
+        fill(x6, c6.q, true, rng);
+        fill(w6, c6.p, true, rng);
+        const size_t kw6 = c6.K / 32, xw6 = (size_t)c6.q * c6.M * kw6, ww6 = (size_t)c6.p * c6.N * kw6;
+        std::vector<uint32_t> xp6(xw6), wp6(ww6);
+        abq_oracle_pack_i32(x6.data(), xp6.data(), c6.M, c6.K, c6.q);
+        abq_oracle_pack_i32(w6.data(), wp6.data(), c6.N, c6.K, c6.p);
+        std::vector<int> ref6((size_t)c6.M * c6.N);
+        abq_oracle_gemm_bitserial(wp6.data(), xp6.data(), ref6.data(), c6.M, c6.N, c6.K, c6.p, c6.q, true);
+        int *d_x6, *d_w6, *d_wf6, *d_o6;
+        char *d_ws6;
+        HIP_OK(hipMalloc(&d_x6, xw6 * 4));
+        HIP_OK(hipMalloc(&d_w6, ww6 * 4));
+        HIP_OK(hipMalloc(&d_wf6, abq_fp6_bytes(c6.N, c6.K)));
+        HIP_OK(hipMalloc(&d_ws6, abq_fp6_bytes(c6.M, c6.K)));
+        HIP_OK(hipMalloc(&d_o6, ref6.size() * 4));
+        HIP_OK(hipMemcpy(d_x6, xp6.data(), xw6 * 4, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(d_w6, wp6.data(), ww6 * 4, hipMemcpyHostToDevice));
+        CHECK(abq_fp6_eligible(4, 4, 1, c6.K) == 1 && abq_fp6_eligible(8, 2, 1, c6.K) == 0);
+        CHECK(abq_relayout_planes_fp6(reinterpret_cast<uint32_t *>(d_w6), reinterpret_cast<uint32_t *>(d_wf6), c6.N, c6.K,
+                                      c6.p, 1, stream) == ABQ_OK);
+        AqBMMAOpState st6 = (*AqBMMA_4x4xtrue_128x128x128_64x64x128_32x32x64_5_InitFn)(d_x6, d_wf6, c6.M, c6.N, c6.K, d_o6,
+                                                                                        nullptr, false);
+        CHECK(st6.initSuccess && st6.native.strategy == ABQ_STRATEGY_FP6);
+        CHECK(abq_gemm_set_operand_layout(&st6.native, ABQ_LAYOUT_PLANES, ABQ_LAYOUT_FP6) == ABQ_OK);
+        CHECK(abq_gemm_workspace_bytes(&st6.native) == abq_fp6_bytes(c6.M, c6.K));
+        CHECK(abq_gemm_exec(&st6.native, stream) == ABQ_ERR_INVALID_ARG); // no workspace yet
+        CHECK(abq_gemm_set_workspace(&st6.native, d_ws6, abq_fp6_bytes(c6.M, c6.K)) == ABQ_OK);
+        HIP_OK(hipMemsetAsync(d_o6, 0xff, ref6.size() * 4, stream));
+        (*AqBMMA_4x4xtrue_128x128x128_64x64x128_32x32x64_5_ExecFn)(st6, stream);
+        HIP_OK(hipStreamSynchronize(stream));
+        std::vector<int> out6(ref6.size());
+        HIP_OK(hipMemcpy(out6.data(), d_o6, out6.size() * 4, hipMemcpyDeviceToHost));
+        CHECK(out6 == ref6);
+        (void)hipFree(d_x6);
+        (void)hipFree(d_w6);
+        (void)hipFree(d_wf6);
+        (void)hipFree(d_ws6);
+        (void)hipFree(d_o6);
+    }
+
     {   // FT wrapper: fp16 activations, static scale, fp16 output scaled by scale_out
         const float in_scale = 21.0f, out_scale = 0.0123f;
         std::vector<uint16_t> ha((size_t)c.M * c.K);
