@@ -235,7 +235,8 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
         st->grid_dim = abq_dim3{ (unsigned)(8 * npx * mblocks), 1, 1 };
         st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
-        st->shared_mem_size = 2 * (size_t)(bm + bn) * 96;
+        const int stages = (e.tm == 2 && e.tn == 2 && e.wm == 2 && e.wn == 2) ? 3 : 4; // LDS stages, see abq_gemm_fp6.hip
+        st->shared_mem_size = (size_t)stages * (bm + bn) * 96;
         return ABQ_OK;
     }
     const KernelTable *tm_ = find_table(reg.mfma, x_bits, w_bits, is_signed);
@@ -648,7 +649,10 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
     int count = 0;
     const KernelEntry *es = fp6_entries(&count);
     // { TM, TN, waves along M, waves along N, workgroups needed }
-    static const int order[][5] = { { 2, 2, 4, 2, 250 }, { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 400 }, { 1, 1, 2, 2, 0 } };
+    // (the kernel runs at the rate L2 delivers its tiles, so the 256x128 tile wins as soon as it covers about
+    // two thirds of the compute units: M = 512, N = 11008 runs 1.4 times faster on its 172 tiles than on 344
+    // tiles of 128x128)
+    static const int order[][5] = { { 2, 2, 4, 2, 160 }, { 2, 2, 2, 2, 250 }, { 2, 1, 2, 2, 400 }, { 1, 1, 2, 2, 0 } };
     int pick = -1;
     for (const auto &o : order) {
         const int bm = 32 * o[0] * o[2], bn = 32 * o[1] * o[3];

@@ -265,7 +265,7 @@ def test_fp6_route_eligibility_and_tile_tuples(abq):
     cfg, _ = abq.parse_kernel_name("AqBMMA_4x4xtrue_256x128x128_64x64x128_32x32x64_5")
     rc, st = _init(abq, cfg=cfg, M=2048, N=4096, K=4096)
     assert rc == 0 and st.strategy == abq.STRATEGY_FP6
-    assert st.grid_dim.x == 8 * 4 * 8 and st.block_dim.x == 512 and st.shared_mem_size == 2 * 384 * 96
+    assert st.grid_dim.x == 8 * 4 * 8 and st.block_dim.x == 512 and st.shared_mem_size == 4 * 384 * 96
     # not eligible: 8-bit activations; K beyond the exactness bound; unknown tile
     cfg, _ = abq.parse_kernel_name("AqBMMA_8x2xtrue_256x128x128_64x64x128_32x32x64_5")
     assert _init(abq, cfg=cfg, M=64, N=64, K=256)[0] == abq.ABQ_ERR_UNSUPPORTED
