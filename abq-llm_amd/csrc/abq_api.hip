@@ -235,8 +235,7 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
         st->grid_dim = abq_dim3{ (unsigned)(8 * npx * mblocks), 1, 1 };
         st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
-        const int stages = (e.tm == 2 && e.tn == 2 && e.wm == 2 && e.wn == 2) ? 3 : 4; // LDS stages, see abq_gemm_fp6.hip
-        st->shared_mem_size = (size_t)stages * (bm + bn) * 96;
+        st->shared_mem_size = e.lds;
         return ABQ_OK;
     }
     const KernelTable *tm_ = find_table(reg.mfma, x_bits, w_bits, is_signed);
@@ -308,7 +307,7 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
         st->grid_dim = abq_dim3{ (unsigned)(8 * npx * mblocks), 1, 1 };
         st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
-        st->shared_mem_size = 2 * (size_t)(bm + bn) * (e.kb + 16) + (bm + bn) * 4;
+        st->shared_mem_size = e.lds ? e.lds : 2 * (size_t)(bm + bn) * (e.kb + 16) + (bm + bn) * 4;
         return ABQ_OK;
     }
 
@@ -617,15 +616,19 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
     // operands, W8A8, and only on grids of several workgroups per compute unit)
     static const int order[][5] = { { 2, 4, 4, 2, 600 }, { 2, 2, 4, 2, 250 }, { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 400 },
                                     { 1, 1, 2, 2, 0 } };
+    // signed 8-bit pairs run the 256x128 tile on the staged kernel, which is bound by the rate L2 delivers the
+    // tiles: the large tile pays as soon as it covers about two thirds of the compute units
+    const bool staged = c.x_bits == 8 && c.w_bits == 8 && c.is_signed;
     int pick = -1;
     for (const auto &o : order) {
         if (o[1] == 4 && c.x_bits + c.w_bits < 16)
             continue;
         const int bm = 32 * o[0] * o[2], bn = 32 * o[1] * o[3];
         const long tiles = (long)((st->M + bm - 1) / bm) * ((st->N + bn - 1) / bn);
+        const long need = (staged && o[0] == 2 && o[1] == 2 && o[2] == 4) ? 160 : o[4];
         for (int i = 0; i < tt->count; ++i)
             if (tt->entries[i].tm == o[0] && tt->entries[i].tn == o[1] && tt->entries[i].kb == 128 &&
-                tt->entries[i].wm == o[2] && tt->entries[i].wn == o[3] && tiles >= o[4] && pick < 0)
+                tt->entries[i].wm == o[2] && tt->entries[i].wn == o[3] && tiles >= need && pick < 0)
                 pick = i;
     }
     if (pick < 0)

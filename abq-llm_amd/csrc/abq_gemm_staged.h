@@ -1,0 +1,274 @@
+// LDS-staged GEMM core for operands that need no unpacking: the tiles go from global memory
+// straight into LDS, the waves feed the matrix cores out of LDS.
+//
+// Replaces AqBMMAKernel::mainLoop + ::epilogue of the reference
+// (engine/mma_any/aq_bmma_kernel.h:109-271, :485-580) for two operand formats:
+//
+//   kFmtFp6   FP6 records (abq_relayout_planes_fp6: 6-bit sign-magnitude codes, 96 bytes per row
+//             and K tile of 128), v_mfma_f32_32x32x64_f8f6f4 with E2M3 x E2M3 and fp32 accumulation;
+//             see abq_gemm_fp6.hip for why the result is the exact integer.
+//   kFmtI8    signed 8-bit x 8-bit operands in the K-tiled layout (abq_relayout_planes with 8 bits:
+//             the bytes themselves, 128 bytes per row and K tile), v_mfma_i32_32x32x32_i8.  (Unsigned
+//             bytes would have to be flipped to value - 128 and their row sums taken after every LDS
+//             read; measured, that costs more than the staging saves, so they stay on the kernel of
+//             abq_gemm_tiled.hip, which does both while it unpacks.)
+//
+// global_load_lds_dwordx4 writes a wave's 64 x 16 bytes straight into LDS (at M0 + 16 * lane): no
+// register staging, no ds_write instructions (LDS stores run at a third of the LDS read rate on
+// this chip), and the data never crosses the vector register file.  S LDS stages: tile t + S is
+// requested during tile t into the stage tile t has just left; the fragments of tile t + 1 are
+// read out of LDS while the MFMAs of tile t run.  The compiler would drain every outstanding load
+// of this kind before each ds_read, so they are issued from inline assembly and waited for by
+// hand: every wave issues the same number of loads per tile, which makes "all but the newest n
+// tiles have landed" one s_waitcnt vmcnt(n * loads per tile).  No other vector-memory instruction
+// may be in flight while that count is relied on: the kernel has none inside its K loop and
+// drains the counter before its epilogue.  One barrier per K tile.  Workgroups are numbered so
+// that the 8 XCDs (workgroup id modulo 8) each work on a contiguous band of N with M fastest.
+// What bounds the kernel on LLaMA-sized problems is the rate at which L2 delivers the tiles
+// (about 22 TB/s over the chip), not the matrix cores.
+#pragma once
+#include <type_traits>
+
+#include "abq_kernels.h"
+
+namespace abq {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4))); // a 16-byte unit
+
+enum StagedFormat { kFmtFp6 = 0, kFmtI8 = 1 };
+
+template <StagedFormat F> struct StagedTraits {
+    static constexpr bool kFp6 = F == kFmtFp6;
+    static constexpr int kUnits = kFp6 ? 6 : 8;   // 16-byte units per row and K tile
+    static constexpr int kRow = 16 * kUnits;      // bytes per row in LDS: the records as they are
+    static constexpr int kReads = kFp6 ? 3 : 4;   // ds_read_b128 per lane and 32-row fragment
+    static constexpr int kSteps = kFp6 ? 2 : 4;   // MFMA K steps per tile of 128
+
+    // LDS placement (in bytes) of 16-byte unit `pos` = row * kUnits + unit of an operand block.  The
+    // rows keep their place; units are permuted so that the fragment reads of sixteen consecutive rows
+    // (same unit) hit sixteen different bank groups, while 64 consecutive units still fill 64
+    // consecutive places (what one wave load delivers).  Both maps are their own inverse.
+    //   FP6: rows are 6 units apart; units swapped in pairs inside every second 256-byte line.
+    //   8 bit: rows are 8 units apart; the unit index is xor-ed with bits 1..3 of the row.
+    static __device__ __forceinline__ int lds_offset(int pos)
+    {
+        if (kFp6)
+            return (pos ^ ((pos >> 4) & 1)) * 16;
+        return (pos ^ ((pos >> 4) & 7)) * 16;
+    }
+    // unit of a row that lane group g reads as its c-th piece
+    static __device__ __forceinline__ int lane_unit(int g, int c) { return kFp6 ? 3 * g + c : 2 * c + g; }
+};
+
+template <int N> __device__ __forceinline__ void staged_wait_loads()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ void staged_load_to_lds(const v4u *src, unsigned lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "memory");
+}
+
+template <StagedFormat F, int TM, int TN, int WM, int WN, int S>
+__global__ __launch_bounds__(64 * WM * WN, (WM * WN > 4 || TM * TN > 4) ? 1 : 2)
+void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_blocks, int n_blocks_per_xcd)
+{
+    using T = StagedTraits<F>;
+    constexpr int NW = WM * WN;
+    constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
+    constexpr int BUF_BYTES = (BM + BN) * T::kRow;
+    constexpr int NIA = BM * T::kUnits / 64;             // wave loads of 1 KiB per tile: activations
+    constexpr int NI = (BM + BN) * T::kUnits / 64;       // ... and in all
+    constexpr int NPW = (NI + NW - 1) / NW;              // per wave
+    static_assert(S >= 3 && S <= 4, "three or four LDS stages");
+    static_assert(NPW * S < 64, "the load counter has six bits");
+    static_assert(BUF_BYTES % 512 == 0 && (32 * T::kRow) % 512 == 0, "stages and fragment rows keep the placement pattern");
+
+    extern __shared__ __align__(16) unsigned char smem[]; // [S][BM + BN][kRow]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wid / WN, wn = wid % WN;
+    const int r = lane & 31, g = lane >> 5;
+    const int M = __builtin_amdgcn_readfirstlane(a.M), N = __builtin_amdgcn_readfirstlane(a.N);
+    const int ktiles = __builtin_amdgcn_readfirstlane(a.K) / 128;
+
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int nb = xcd * n_blocks_per_xcd + slot / m_blocks;
+    const int mb = slot % m_blocks;
+    const int m0 = mb * BM, n0 = nb * BN;
+    if (n0 >= N)
+        return; // uniform over the workgroup, before any barrier
+
+    // Wave load q of a tile fills LDS units [64 q, 64 q + 64) of the stage, activations first; the unit
+    // at LDS place P is unit lds_offset(P) / 16 of the tile.  Loads past the last one repeat an earlier
+    // load of the wave (same data, same place), so that every wave issues NPW loads per tile.  Rows
+    // past the edge are clamped for loading and dropped at the store.
+    uint32_t goff[NPW]; // 16-byte units from the start of the operand's records of one K tile
+#pragma unroll
+    for (int i = 0; i < NPW; ++i) {
+        int q = wid + NW * i;
+        if (q >= NI)
+            q -= NW;
+        const bool is_a = q < NIA; // wave-uniform
+        const int P = 64 * q + lane - (is_a ? 0 : BM * T::kUnits);
+        const int v = T::lds_offset(P) >> 4;
+        const int row = v / T::kUnits, col = v % T::kUnits;
+        goff[i] = (uint32_t)(is_a ? min(m0 + row, M - 1) : min(n0 + row, N - 1)) * T::kUnits + col;
+    }
+    const size_t stride_a = (size_t)M * T::kUnits, stride_b = (size_t)N * T::kUnits;
+    const unsigned lds0 = (unsigned)(size_t)smem; // LDS byte address of the first stage
+
+    using Acc = typename std::conditional<T::kFp6, v16f, v16i>::type;
+    Acc acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                acc[i][j][e] = 0;
+
+    unsigned char *lds_a = smem;
+    unsigned char *lds_b = smem + BM * T::kRow;
+    int a_off[T::kReads], b_off[T::kReads];
+#pragma unroll
+    for (int c = 0; c < T::kReads; ++c) {
+        a_off[c] = T::lds_offset((wm * 32 * TM + r) * T::kUnits + T::lane_unit(g, c));
+        b_off[c] = T::lds_offset((wn * 32 * TN + r) * T::kUnits + T::lane_unit(g, c));
+    }
+    // Fragment sets as the raw 16-byte reads: piece kReads * f + c is read c of fragment f (activation
+    // fragments first); the MFMA operands are cut out of them when they are used.
+    constexpr int NF = TM + TN, NR = T::kReads * NF, NM = T::kSteps * TM * TN;
+    v4i q0[NR], q1[NR];
+    auto read_piece = [&](v4i(&q)[NR], int stage, int p) {
+        const int f = p / T::kReads, c = p % T::kReads;
+        q[p] = f < TM ? *reinterpret_cast<const v4i *>(lds_a + stage + f * 32 * T::kRow + a_off[c])
+                      : *reinterpret_cast<const v4i *>(lds_b + stage + (f - TM) * 32 * T::kRow + b_off[c]);
+    };
+    auto mfma = [&](Acc &c, const v4i(&q)[NR], int i, int j, int ks) {
+        if constexpr (T::kFp6) {
+            // dwords 0-5 of the 12 a lane holds are the first K step's operand, 6-11 the second's (the two
+            // upper dwords of the 8-dword operand are not read for 6-bit formats)
+            const int fa = 3 * i, fb = 3 * (TM + j);
+            const v8i av = ks == 0 ? __builtin_shufflevector(q[fa], q[fa + 1], 0, 1, 2, 3, 4, 5, -1, -1)
+                                   : __builtin_shufflevector(q[fa + 1], q[fa + 2], 2, 3, 4, 5, 6, 7, -1, -1);
+            const v8i bv = ks == 0 ? __builtin_shufflevector(q[fb], q[fb + 1], 0, 1, 2, 3, 4, 5, -1, -1)
+                                   : __builtin_shufflevector(q[fb + 1], q[fb + 2], 2, 3, 4, 5, 6, 7, -1, -1);
+            c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 2, 2, 0, 0, 0, 0);
+        } else {
+            c = __builtin_amdgcn_mfma_i32_32x32x32_i8(q[4 * i + ks], q[4 * (TM + j) + ks], c, 0, 0, 0);
+        }
+    };
+    auto request = [&](int kt_req, int stage, int i) {
+        const int kn = min(kt_req, ktiles - 1); // tiles past the end: copies of the last, into stages nobody reads
+        int q = wid + NW * i;
+        if (q >= NI)
+            q -= NW;
+        staged_load_to_lds((q < NIA ? xt + kn * stride_a : wt + kn * stride_b) + goff[i], lds0 + stage + q * 1024);
+    };
+
+    // Tile t lives in stage t % S from its request until its fragments have been read, which happens
+    // during tile t - 1; during tile t the stages therefore hold tiles t + 1 .. t + S, the last one
+    // requested right then into the stage tile t has just left.
+    // prologue: tiles 0 .. S-1 requested; tile 0 read into the first fragment set; tile 1 landed
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+#pragma unroll
+        for (int i = 0; i < NPW; ++i)
+            request(s, s * BUF_BYTES, i);
+    staged_wait_loads<NPW * (S - 1)>();
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < NR; ++p)
+        read_piece(q0, 0, p);
+    staged_wait_loads<NPW * (S - 2)>();
+    __syncthreads();
+
+    int st_req = 0;         // stage the next request goes to: the one tile t occupied
+    int st_rd = BUF_BYTES;  // stage of tile t + 1
+    // One K tile.  On entry every wave's share of tile KT + 1 has landed (wait + barrier at the end of
+    // the previous tile), and the fragment set QC holds tile KT.  The wave's load requests and LDS reads
+    // are dealt out between its MFMAs: a wave issues in order, and a burst of requests at the top of
+    // the tile would hold its MFMAs back until the load unit and the LDS have taken the whole burst.
+#define ABQ_STAGED_K_TILE(KT, QC, QN)                                                                           \
+    {                                                                                                           \
+        _Pragma("unroll") for (int k = 0; k < NM; ++k)                                                          \
+        {                                                                                                       \
+            mfma(acc[(k / TN) % TM][k % TN], QC, (k / TN) % TM, k % TN, k / (TM * TN));                         \
+            _Pragma("unroll") for (int d = k * NPW / NM; d < (k + 1) * NPW / NM; ++d)                           \
+                request((KT) + S, st_req, d);                                                                   \
+            _Pragma("unroll") for (int p = k * NR / NM; p < (k + 1) * NR / NM; ++p)                             \
+                read_piece(QN, st_rd, p);                                                                       \
+            __builtin_amdgcn_sched_barrier(0);                                                                  \
+        }                                                                                                       \
+        st_req = st_req + BUF_BYTES == S * BUF_BYTES ? 0 : st_req + BUF_BYTES;                                  \
+        st_rd = st_rd + BUF_BYTES == S * BUF_BYTES ? 0 : st_rd + BUF_BYTES;                                     \
+        staged_wait_loads<NPW * (S - 2)>(); /* tile KT + 2 has landed; the S - 2 younger ones may still fly */  \
+        __syncthreads();                                                                                        \
+    }
+
+    int kt = 0;
+    for (; kt + 2 <= ktiles; kt += 2) {
+        ABQ_STAGED_K_TILE(kt, q0, q1)
+        ABQ_STAGED_K_TILE(kt + 1, q1, q0)
+    }
+    if (kt < ktiles)
+        ABQ_STAGED_K_TILE(kt, q0, q1)
+#undef ABQ_STAGED_K_TILE
+    staged_wait_loads<0>(); // the clamped requests past the last tile: nothing of ours may be in flight below
+
+    const StoreOperands so = store_operands(a);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + wn * 32 * TN + j * 32 + r;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4);
+                int v;
+                if constexpr (T::kFp6)
+                    v = (int)(acc[i][j][e] * 64.0f); // both operands carry 1/8 as their unit: the sum is the result / 64, exactly
+                else
+                    v = acc[i][j][e];
+                if (m < M && n < N)
+                    store_result_compact(so, m, n, v);
+            }
+        }
+    }
+}
+
+// LDS stages of a tile: as many (up to four) as leave room for the workgroups that share a compute
+// unit: two for the four-wave tiles when three stages of theirs fit twice, else one.
+template <StagedFormat F, int TM, int TN, int WM, int WN> struct StagedStages {
+    static constexpr int kBuf = 32 * (TM * WM + TN * WN) * StagedTraits<F>::kRow;
+    static constexpr int value = (WM * WN <= 4 && TM * TN <= 4 && 2 * 4 * kBuf > 160 * 1024 && 2 * 3 * kBuf <= 160 * 1024) ? 3
+                                 : (4 * kBuf <= 160 * 1024 ? 4 : 3);
+    static_assert(3 * kBuf <= 160 * 1024, "three stages fit a compute unit's LDS");
+};
+
+template <StagedFormat F, int TM, int TN, int WM, int WN> static hipError_t launch_mfma_staged(const GemmArgs &a, hipStream_t stream)
+{
+    constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
+    constexpr int S = StagedStages<F, TM, TN, WM, WN>::value;
+    const int m_blocks = (a.M + BM - 1) / BM, n_blocks = (a.N + BN - 1) / BN;
+    const int npx = (n_blocks + 7) / 8;
+    const dim3 grid(8 * npx * m_blocks);
+    const size_t lds = S * (size_t)StagedStages<F, TM, TN, WM, WN>::kBuf;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_staged<F, TM, TN, WM, WN, S>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr != hipSuccess)
+        return attr;
+    hipLaunchKernelGGL((gemm_mfma_staged<F, TM, TN, WM, WN, S>), grid, dim3(64 * WM * WN), lds, stream, a,
+                       reinterpret_cast<const v4u *>(a.X), reinterpret_cast<const v4u *>(a.W), m_blocks, npx);
+    return hipGetLastError();
+}
+
+} // namespace abq

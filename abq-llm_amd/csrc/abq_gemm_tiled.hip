@@ -27,6 +27,7 @@
 // Workgroups are numbered so that the 8 XCDs (workgroup id modulo 8) each work on a
 // contiguous band of N with M fastest: a band's weight panels stay in that XCD's L2.
 #include "abq_kernels.h"
+#include "abq_gemm_staged.h"
 
 #ifndef ABQ_Q
 #error "compile with -DABQ_Q=<x_bits> -DABQ_P=<w_bits>"
@@ -34,8 +35,6 @@
 
 namespace abq {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kTileK = 128;        // K elements per tile
 constexpr int kLdsRow = 144;       // bytes per expanded row in LDS (128 + 16 padding)
@@ -515,10 +514,24 @@ static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 #define ABQ_GENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, true, 128>, 128 },
 #define ABQ_GENTRY_F(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN, true, 128>, 128 },
 
+#if ABQ_Q == 8 && ABQ_P == 8
+// Signed 8-bit x 8-bit needs no unpacking: the tiles that the staged kernel (abq_gemm_staged.h: tiles
+// loaded straight into LDS) is built for run on it, under the same tile tuples; the rest, and the
+// unsigned pair, keep the kernel above.
+#define ABQ_SENTRY(F, TM, TN, WM, WN)                                                        \
+    { 32, TM, TN, WM, WN, 1, 4, &launch_mfma_staged<F, TM, TN, WM, WN>, 128,                 \
+      (size_t)StagedStages<F, TM, TN, WM, WN>::value * StagedStages<F, TM, TN, WM, WN>::kBuf },
+static const KernelEntry kSigned[] = { ABQ_ENTRY_T(4, 4) ABQ_ENTRY_T(2, 4) ABQ_SENTRY(kFmtI8, 2, 2, 2, 2) ABQ_SENTRY(kFmtI8, 2, 1, 2, 2)
+                                       ABQ_SENTRY(kFmtI8, 1, 1, 2, 2) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_T)
+                                       ABQ_SENTRY(kFmtI8, 2, 2, 4, 2) ABQ_WENTRY_T(2, 2, 4, 4) ABQ_WENTRY_T(2, 4, 4, 2) };
+static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
+                                         ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_F) };
+#else
 static const KernelEntry kSigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_T) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_T)
                                        ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_T) };
 static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
                                          ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_F) };
+#endif
 static const KernelEntry kSignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_T) };
 static const KernelEntry kUnsignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_F) };
 

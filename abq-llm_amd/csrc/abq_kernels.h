@@ -39,6 +39,7 @@ struct KernelEntry {
     int nstage;
     GemmLauncher launch;
     int kb;                 // K elements per LDS stage (tiled kernel); 0 where it does not apply
+    size_t lds;             // dynamic LDS of the launch where the kernel fixes it itself; 0: derived from the tile
 };
 
 struct KernelTable {
