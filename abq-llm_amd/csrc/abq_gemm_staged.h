@@ -22,7 +22,9 @@
 // hand: every wave issues the same number of loads per tile, which makes "all but the newest n
 // tiles have landed" one s_waitcnt vmcnt(n * loads per tile).  No other vector-memory instruction
 // may be in flight while that count is relied on: the kernel has none inside its K loop and
-// drains the counter before its epilogue.  One barrier per K tile.  Workgroups are numbered so
+// drains the counter before its epilogue.  A register spill would be such an instruction: every
+// instantiation must compile with .vgpr_spill_count 0 and no private segment (hipcc -save-temps
+// shows both in the kernel's metadata), which is why the tile variants stop where they do.  One barrier per K tile.  Workgroups are numbered so
 // that the 8 XCDs (workgroup id modulo 8) each work on a contiguous band of N with M fastest.
 // What bounds the kernel on LLaMA-sized problems is the rate at which L2 delivers the tiles
 // (about 22 TB/s over the chip), not the matrix cores.
