@@ -28,8 +28,8 @@ namespace abq {
 // Tile space: MFMA tiles per wave (TM, TN) and waves along M, N; nstage 5 marks the FP6 records.
 #define ABQ_FP6_VARIANTS(V) V(2, 2, 4, 2) V(4, 2, 2, 2) V(2, 2, 2, 2) V(2, 1, 2, 2) V(1, 1, 2, 2)
 #define ABQ_FP6_ENTRY(TM, TN, WM, WN)                                                             \
-    { 32, TM, TN, WM, WN, 1, 5, &launch_mfma_staged<kFmtFp6, TM, TN, WM, WN>, 128,                \
-      (size_t)StagedStages<kFmtFp6, TM, TN, WM, WN>::value * StagedStages<kFmtFp6, TM, TN, WM, WN>::kBuf },
+    { 32, TM, TN, WM, WN, 1, 5, &launch_mfma_staged<6, 6, true, true, TM, TN, WM, WN>, 128,       \
+      StagedStages<6, 6, true, TM, TN, WM, WN>::kLds },
 static const KernelEntry kFp6Entries[] = { ABQ_FP6_VARIANTS(ABQ_FP6_ENTRY) };
 
 const KernelEntry *fp6_entries(int *count)

@@ -2,16 +2,20 @@
 // straight into LDS, the waves feed the matrix cores out of LDS.
 //
 // Replaces AqBMMAKernel::mainLoop + ::epilogue of the reference
-// (engine/mma_any/aq_bmma_kernel.h:109-271, :485-580) for two operand formats:
+// (engine/mma_any/aq_bmma_kernel.h:109-271, :485-580) for two families of operand formats:
 //
-//   kFmtFp6   FP6 records (abq_relayout_planes_fp6: 6-bit sign-magnitude codes, 96 bytes per row
-//             and K tile of 128), v_mfma_f32_32x32x64_f8f6f4 with E2M3 x E2M3 and fp32 accumulation;
-//             see abq_gemm_fp6.hip for why the result is the exact integer.
-//   kFmtI8    signed 8-bit x 8-bit operands in the K-tiled layout (abq_relayout_planes with 8 bits:
-//             the bytes themselves, 128 bytes per row and K tile), v_mfma_i32_32x32x32_i8.  (Unsigned
-//             bytes would have to be flipped to value - 128 and their row sums taken after every LDS
-//             read; measured, that costs more than the staging saves, so they stay on the kernel of
-//             abq_gemm_tiled.hip, which does both while it unpacks.)
+//   FP6       both operands as FP6 records (abq_relayout_planes_fp6: 6-bit sign-magnitude codes, 96 bytes
+//             per row and K tile of 128), v_mfma_f32_32x32x64_f8f6f4 with E2M3 x E2M3 and fp32
+//             accumulation; see abq_gemm_fp6.hip for why the result is the exact integer.
+//   integer   operands of 2, 4 or 8 bits in the K-tiled layout (abq_relayout_planes: one field per
+//             element, 32 / 64 / 128 bytes per row and K tile), v_mfma_i32_32x32x32_i8.  The records
+//             stay packed in LDS; a wave turns the field words of its own fragments into int8 with a
+//             shift and a mask per four elements right before the MFMA that uses them (8-bit
+//             operands need nothing).  Signed operands are placed at the top of the byte and the
+//             result shifted right by 16 - q - p, unsigned ones (at most 4 bits here) are fed as they
+//             are.  Pairs with an unsigned 8-bit operand (bit 7 to flip and row sums to take after
+//             every LDS read: measured slower than what the staging saves) and the widths made of
+//             several fields (3, 5, 6, 7 bits) stay on the kernel of abq_gemm_tiled.hip.
 //
 // global_load_lds_dwordx4 writes a wave's 64 x 16 bytes straight into LDS (at M0 + 16 * lane): no
 // register staging, no ds_write instructions (LDS stores run at a third of the LDS read rate on
@@ -41,30 +45,54 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4))); // a 16-byte unit
 
-enum StagedFormat { kFmtFp6 = 0, kFmtI8 = 1 };
-
-template <StagedFormat F> struct StagedTraits {
-    static constexpr bool kFp6 = F == kFmtFp6;
-    static constexpr int kUnits = kFp6 ? 6 : 8;   // 16-byte units per row and K tile
-    static constexpr int kRow = 16 * kUnits;      // bytes per row in LDS: the records as they are
-    static constexpr int kReads = kFp6 ? 3 : 4;   // ds_read_b128 per lane and 32-row fragment
-    static constexpr int kSteps = kFp6 ? 2 : 4;   // MFMA K steps per tile of 128
+// One operand's format: FP6 records, or BITS-wide integer fields (BITS in {2, 4, 8}).
+template <int BITS, bool FP6> struct StagedOperand {
+    static_assert(FP6 || BITS == 2 || BITS == 4 || BITS == 8, "single-field widths");
+    static constexpr int kUnits = FP6 ? 6 : BITS;     // 16-byte units per row and K tile
+    static constexpr int kRow = 16 * kUnits;          // bytes per row in LDS: the records as they are
+    static constexpr int kReads = FP6 ? 3 : BITS / 2; // ds_read_b128 per lane and 32-row fragment
 
     // LDS placement (in bytes) of 16-byte unit `pos` = row * kUnits + unit of an operand block.  The
     // rows keep their place; units are permuted so that the fragment reads of sixteen consecutive rows
     // (same unit) hit sixteen different bank groups, while 64 consecutive units still fill 64
-    // consecutive places (what one wave load delivers).  Both maps are their own inverse.
+    // consecutive places (what one wave load delivers).  Every map is its own inverse.
     //   FP6: rows are 6 units apart; units swapped in pairs inside every second 256-byte line.
-    //   8 bit: rows are 8 units apart; the unit index is xor-ed with bits 1..3 of the row.
+    //   integer: rows are 2, 4 or 8 units apart; the unit index is xor-ed with the number of the
+    //   256-byte line (which holds 8, 4 or 2 rows), modulo the units of a row.
     static __device__ __forceinline__ int lds_offset(int pos)
     {
-        if (kFp6)
-            return (pos ^ ((pos >> 4) & 1)) * 16;
-        return (pos ^ ((pos >> 4) & 7)) * 16;
+        return (pos ^ ((pos >> 4) & (FP6 ? 1 : kUnits - 1))) * 16;
     }
-    // unit of a row that lane group g reads as its c-th piece
-    static __device__ __forceinline__ int lane_unit(int g, int c) { return kFp6 ? 3 * g + c : 2 * c + g; }
+    // First unit of a row that lane half g reads as its c-th piece.  The two halves of the lanes split a
+    // row's K tile in the middle; any split works as long as both operands use the same one.
+    static __device__ __forceinline__ int lane_unit(int g, int c) { return kReads * g + c; }
 };
+
+// int8 MFMA operand of K step c (0..3) out of the pieces of one fragment (kReads 16-byte reads: this
+// lane half's 64 elements as field words; element order as abq_bits.h: field word j of a word-set
+// carries in byte c', at bits [f s, f s + f), the element at expanded dword (8 / f) j + s, byte c').
+template <int BITS, bool SIGNED> __device__ __forceinline__ v4i staged_int8_operand(const v4i *piece, int c)
+{
+    if constexpr (BITS == 8) {
+        return piece[c];
+    } else if constexpr (BITS == 4) {
+        // step c <- words 2c, 2c + 1 of the lane's eight; each word holds two expanded dwords
+        const uint32_t w0 = (uint32_t)piece[c / 2][2 * (c % 2)], w1 = (uint32_t)piece[c / 2][2 * (c % 2) + 1];
+        if (SIGNED) // value * 16: the sign bit lands on bit 7
+            return v4i{ (int)((w0 << 4) & 0xF0F0F0F0u), (int)(w0 & 0xF0F0F0F0u), (int)((w1 << 4) & 0xF0F0F0F0u),
+                        (int)(w1 & 0xF0F0F0F0u) };
+        return v4i{ (int)(w0 & 0x0F0F0F0Fu), (int)((w0 >> 4) & 0x0F0F0F0Fu), (int)(w1 & 0x0F0F0F0Fu),
+                    (int)((w1 >> 4) & 0x0F0F0F0Fu) };
+    } else {
+        // step c <- word c of the lane's four; it holds four expanded dwords
+        const uint32_t w = (uint32_t)piece[0][c];
+        if (SIGNED) // value * 64
+            return v4i{ (int)((w << 6) & 0xC0C0C0C0u), (int)((w << 4) & 0xC0C0C0C0u), (int)((w << 2) & 0xC0C0C0C0u),
+                        (int)(w & 0xC0C0C0C0u) };
+        return v4i{ (int)(w & 0x03030303u), (int)((w >> 2) & 0x03030303u), (int)((w >> 4) & 0x03030303u),
+                    (int)((w >> 6) & 0x03030303u) };
+    }
+}
 
 template <int N> __device__ __forceinline__ void staged_wait_loads()
 {
@@ -73,25 +101,32 @@ template <int N> __device__ __forceinline__ void staged_wait_loads()
 
 __device__ __forceinline__ void staged_load_to_lds(const v4u *src, unsigned lds_addr)
 {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "memory");
+    // the LDS address is the same in every lane; readfirstlane tells the compiler so
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)
+                 : "memory");
 }
 
-template <StagedFormat F, int TM, int TN, int WM, int WN, int S>
+// QB / PB: bits of the activation / weight fields (2, 4 or 8; ignored for FP6).
+template <int QB, int PB, bool SIGNED, bool FP6, int TM, int TN, int WM, int WN, int S>
 __global__ __launch_bounds__(64 * WM * WN, (WM * WN > 4 || TM * TN > 4) ? 1 : 2)
 void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_blocks, int n_blocks_per_xcd)
 {
-    using T = StagedTraits<F>;
+    using TA = StagedOperand<QB, FP6>;
+    using TB = StagedOperand<PB, FP6>;
     constexpr int NW = WM * WN;
     constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
-    constexpr int BUF_BYTES = (BM + BN) * T::kRow;
-    constexpr int NIA = BM * T::kUnits / 64;             // wave loads of 1 KiB per tile: activations
-    constexpr int NI = (BM + BN) * T::kUnits / 64;       // ... and in all
-    constexpr int NPW = (NI + NW - 1) / NW;              // per wave
+    constexpr int BUF_BYTES = BM * TA::kRow + BN * TB::kRow;
+    constexpr int NIA = BM * TA::kUnits / 64;                  // wave loads of 1 KiB per tile: activations
+    constexpr int NI = NIA + BN * TB::kUnits / 64;             // ... and in all
+    constexpr int NPW = (NI + NW - 1) / NW;                    // per wave
+    constexpr int kSteps = FP6 ? 2 : 4;                        // MFMA K steps per tile of 128
+    static_assert(FP6 || SIGNED || (QB < 8 && PB < 8), "unsigned 8-bit operands are not handled here");
     static_assert(S >= 3 && S <= 4, "three or four LDS stages");
     static_assert(NPW * S < 64, "the load counter has six bits");
-    static_assert(BUF_BYTES % 512 == 0 && (32 * T::kRow) % 512 == 0, "stages and fragment rows keep the placement pattern");
+    static_assert(BUF_BYTES % 512 == 0 && (BM * TA::kRow) % 512 == 0 && (32 * TA::kRow) % 256 == 0 && (32 * TB::kRow) % 256 == 0,
+                  "stages, operand blocks and fragment rows keep the placement pattern");
 
-    extern __shared__ __align__(16) unsigned char smem[]; // [S][BM + BN][kRow]
+    extern __shared__ __align__(16) unsigned char smem[]; // [S][BM rows of X | BN rows of W]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -109,25 +144,27 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         return; // uniform over the workgroup, before any barrier
 
     // Wave load q of a tile fills LDS units [64 q, 64 q + 64) of the stage, activations first; the unit
-    // at LDS place P is unit lds_offset(P) / 16 of the tile.  Loads past the last one repeat an earlier
-    // load of the wave (same data, same place), so that every wave issues NPW loads per tile.  Rows
-    // past the edge are clamped for loading and dropped at the store.
+    // at LDS place P of an operand block is unit lds_offset(P) / 16 of that operand's tile.  Loads past
+    // the last one repeat an earlier load of the wave (same data, same place), so that every wave
+    // issues NPW loads per tile.  Rows past the edge are clamped for loading and dropped at the store.
     uint32_t goff[NPW]; // 16-byte units from the start of the operand's records of one K tile
 #pragma unroll
     for (int i = 0; i < NPW; ++i) {
         int q = wid + NW * i;
         if (q >= NI)
             q -= NW;
-        const bool is_a = q < NIA; // wave-uniform
-        const int P = 64 * q + lane - (is_a ? 0 : BM * T::kUnits);
-        const int v = T::lds_offset(P) >> 4;
-        const int row = v / T::kUnits, col = v % T::kUnits;
-        goff[i] = (uint32_t)(is_a ? min(m0 + row, M - 1) : min(n0 + row, N - 1)) * T::kUnits + col;
+        if (q < NIA) { // wave-uniform
+            const int v = TA::lds_offset(64 * q + lane) >> 4;
+            goff[i] = (uint32_t)min(m0 + v / TA::kUnits, M - 1) * TA::kUnits + v % TA::kUnits;
+        } else {
+            const int v = TB::lds_offset(64 * (q - NIA) + lane) >> 4;
+            goff[i] = (uint32_t)min(n0 + v / TB::kUnits, N - 1) * TB::kUnits + v % TB::kUnits;
+        }
     }
-    const size_t stride_a = (size_t)M * T::kUnits, stride_b = (size_t)N * T::kUnits;
+    const size_t stride_a = (size_t)M * TA::kUnits, stride_b = (size_t)N * TB::kUnits;
     const unsigned lds0 = (unsigned)(size_t)smem; // LDS byte address of the first stage
 
-    using Acc = typename std::conditional<T::kFp6, v16f, v16i>::type;
+    using Acc = typename std::conditional<FP6, v16f, v16i>::type;
     Acc acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -138,34 +175,39 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
                 acc[i][j][e] = 0;
 
     unsigned char *lds_a = smem;
-    unsigned char *lds_b = smem + BM * T::kRow;
-    int a_off[T::kReads], b_off[T::kReads];
+    unsigned char *lds_b = smem + BM * TA::kRow;
+    int a_off[TA::kReads], b_off[TB::kReads];
 #pragma unroll
-    for (int c = 0; c < T::kReads; ++c) {
-        a_off[c] = T::lds_offset((wm * 32 * TM + r) * T::kUnits + T::lane_unit(g, c));
-        b_off[c] = T::lds_offset((wn * 32 * TN + r) * T::kUnits + T::lane_unit(g, c));
-    }
-    // Fragment sets as the raw 16-byte reads: piece kReads * f + c is read c of fragment f (activation
-    // fragments first); the MFMA operands are cut out of them when they are used.
-    constexpr int NF = TM + TN, NR = T::kReads * NF, NM = T::kSteps * TM * TN;
+    for (int c = 0; c < TA::kReads; ++c)
+        a_off[c] = TA::lds_offset((wm * 32 * TM + r) * TA::kUnits + TA::lane_unit(g, c));
+#pragma unroll
+    for (int c = 0; c < TB::kReads; ++c)
+        b_off[c] = TB::lds_offset((wn * 32 * TN + r) * TB::kUnits + TB::lane_unit(g, c));
+    // Fragment sets as the raw 16-byte reads: the kReads pieces of activation fragment i start at
+    // i * kReads, those of weight fragment j at NRA + j * kReads; the MFMA operands are cut (FP6) or
+    // unpacked (integer fields) out of them when they are used.
+    constexpr int NRA = TM * TA::kReads, NR = NRA + TN * TB::kReads, NM = kSteps * TM * TN;
     v4i q0[NR], q1[NR];
     auto read_piece = [&](v4i(&q)[NR], int stage, int p) {
-        const int f = p / T::kReads, c = p % T::kReads;
-        q[p] = f < TM ? *reinterpret_cast<const v4i *>(lds_a + stage + f * 32 * T::kRow + a_off[c])
-                      : *reinterpret_cast<const v4i *>(lds_b + stage + (f - TM) * 32 * T::kRow + b_off[c]);
+        if (p < NRA)
+            q[p] = *reinterpret_cast<const v4i *>(lds_a + stage + (p / TA::kReads) * 32 * TA::kRow + a_off[p % TA::kReads]);
+        else
+            q[p] = *reinterpret_cast<const v4i *>(lds_b + stage + ((p - NRA) / TB::kReads) * 32 * TB::kRow +
+                                                  b_off[(p - NRA) % TB::kReads]);
     };
     auto mfma = [&](Acc &c, const v4i(&q)[NR], int i, int j, int ks) {
-        if constexpr (T::kFp6) {
+        const v4i *pa = &q[i * TA::kReads], *pb = &q[NRA + j * TB::kReads];
+        if constexpr (FP6) {
             // dwords 0-5 of the 12 a lane holds are the first K step's operand, 6-11 the second's (the two
             // upper dwords of the 8-dword operand are not read for 6-bit formats)
-            const int fa = 3 * i, fb = 3 * (TM + j);
-            const v8i av = ks == 0 ? __builtin_shufflevector(q[fa], q[fa + 1], 0, 1, 2, 3, 4, 5, -1, -1)
-                                   : __builtin_shufflevector(q[fa + 1], q[fa + 2], 2, 3, 4, 5, 6, 7, -1, -1);
-            const v8i bv = ks == 0 ? __builtin_shufflevector(q[fb], q[fb + 1], 0, 1, 2, 3, 4, 5, -1, -1)
-                                   : __builtin_shufflevector(q[fb + 1], q[fb + 2], 2, 3, 4, 5, 6, 7, -1, -1);
+            const v8i av = ks == 0 ? __builtin_shufflevector(pa[0], pa[1], 0, 1, 2, 3, 4, 5, -1, -1)
+                                   : __builtin_shufflevector(pa[1], pa[2], 2, 3, 4, 5, 6, 7, -1, -1);
+            const v8i bv = ks == 0 ? __builtin_shufflevector(pb[0], pb[1], 0, 1, 2, 3, 4, 5, -1, -1)
+                                   : __builtin_shufflevector(pb[1], pb[2], 2, 3, 4, 5, 6, 7, -1, -1);
             c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 2, 2, 0, 0, 0, 0);
         } else {
-            c = __builtin_amdgcn_mfma_i32_32x32x32_i8(q[4 * i + ks], q[4 * (TM + j) + ks], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_i32_32x32x32_i8(staged_int8_operand<QB, SIGNED>(pa, ks),
+                                                      staged_int8_operand<PB, SIGNED>(pb, ks), c, 0, 0, 0);
         }
     };
     auto request = [&](int kt_req, int stage, int i) {
@@ -236,10 +278,10 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
             for (int e = 0; e < 16; ++e) {
                 const int m = m0 + wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4);
                 int v;
-                if constexpr (T::kFp6)
+                if constexpr (FP6)
                     v = (int)(acc[i][j][e] * 64.0f); // both operands carry 1/8 as their unit: the sum is the result / 64, exactly
                 else
-                    v = acc[i][j][e];
+                    v = SIGNED ? acc[i][j][e] >> (16 - QB - PB) : acc[i][j][e]; // signed fields sit at the top of their bytes
                 if (m < M && n < N)
                     store_result_compact(so, m, n, v);
             }
@@ -249,27 +291,30 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
 
 // LDS stages of a tile: as many (up to four) as leave room for the workgroups that share a compute
 // unit: two for the four-wave tiles when three stages of theirs fit twice, else one.
-template <StagedFormat F, int TM, int TN, int WM, int WN> struct StagedStages {
-    static constexpr int kBuf = 32 * (TM * WM + TN * WN) * StagedTraits<F>::kRow;
+template <int QB, int PB, bool FP6, int TM, int TN, int WM, int WN> struct StagedStages {
+    static constexpr int kBuf = 32 * (TM * WM * StagedOperand<QB, FP6>::kRow + TN * WN * StagedOperand<PB, FP6>::kRow);
     static constexpr int value = (WM * WN <= 4 && TM * TN <= 4 && 2 * 4 * kBuf > 160 * 1024 && 2 * 3 * kBuf <= 160 * 1024) ? 3
                                  : (4 * kBuf <= 160 * 1024 ? 4 : 3);
+    static constexpr size_t kLds = (size_t)value * kBuf;
     static_assert(3 * kBuf <= 160 * 1024, "three stages fit a compute unit's LDS");
 };
 
-template <StagedFormat F, int TM, int TN, int WM, int WN> static hipError_t launch_mfma_staged(const GemmArgs &a, hipStream_t stream)
+template <int QB, int PB, bool SIGNED, bool FP6, int TM, int TN, int WM, int WN>
+static hipError_t launch_mfma_staged(const GemmArgs &a, hipStream_t stream)
 {
     constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
-    constexpr int S = StagedStages<F, TM, TN, WM, WN>::value;
+    using Stages = StagedStages<QB, PB, FP6, TM, TN, WM, WN>;
+    constexpr int S = Stages::value;
     const int m_blocks = (a.M + BM - 1) / BM, n_blocks = (a.N + BN - 1) / BN;
     const int npx = (n_blocks + 7) / 8;
     const dim3 grid(8 * npx * m_blocks);
-    const size_t lds = S * (size_t)StagedStages<F, TM, TN, WM, WN>::kBuf;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_staged<F, TM, TN, WM, WN, S>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void *>(&gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess)
         return attr;
-    hipLaunchKernelGGL((gemm_mfma_staged<F, TM, TN, WM, WN, S>), grid, dim3(64 * WM * WN), lds, stream, a,
-                       reinterpret_cast<const v4u *>(a.X), reinterpret_cast<const v4u *>(a.W), m_blocks, npx);
+    hipLaunchKernelGGL((gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S>), grid, dim3(64 * WM * WN), Stages::kLds,
+                       stream, a, reinterpret_cast<const v4u *>(a.X), reinterpret_cast<const v4u *>(a.W), m_blocks, npx);
     return hipGetLastError();
 }
 

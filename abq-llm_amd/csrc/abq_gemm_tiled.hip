@@ -514,18 +514,25 @@ static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 #define ABQ_GENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, true, 128>, 128 },
 #define ABQ_GENTRY_F(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN, true, 128>, 128 },
 
-#if ABQ_Q == 8 && ABQ_P == 8
-// Signed 8-bit x 8-bit needs no unpacking: the tiles that the staged kernel (abq_gemm_staged.h: tiles
-// loaded straight into LDS) is built for run on it, under the same tile tuples; the rest, and the
-// unsigned pair, keep the kernel above.
-#define ABQ_SENTRY(F, TM, TN, WM, WN)                                                        \
-    { 32, TM, TN, WM, WN, 1, 4, &launch_mfma_staged<F, TM, TN, WM, WN>, 128,                 \
-      (size_t)StagedStages<F, TM, TN, WM, WN>::value * StagedStages<F, TM, TN, WM, WN>::kBuf },
-static const KernelEntry kSigned[] = { ABQ_ENTRY_T(4, 4) ABQ_ENTRY_T(2, 4) ABQ_SENTRY(kFmtI8, 2, 2, 2, 2) ABQ_SENTRY(kFmtI8, 2, 1, 2, 2)
-                                       ABQ_SENTRY(kFmtI8, 1, 1, 2, 2) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_T)
-                                       ABQ_SENTRY(kFmtI8, 2, 2, 4, 2) ABQ_WENTRY_T(2, 2, 4, 4) ABQ_WENTRY_T(2, 4, 4, 2) };
+// Pairs of single-field widths (2, 4, 8 bits; unsigned only up to 4) run the tiles that the staged kernel
+// (abq_gemm_staged.h: records loaded straight into LDS, unpacked by the waves after the LDS read) is built
+// for on that kernel, under the same tile tuples; the other tiles and pairs keep the kernel above.
+#define ABQ_FIELD1(B) ((B) == 2 || (B) == 4 || (B) == 8)
+#if ABQ_FIELD1(ABQ_Q) && ABQ_FIELD1(ABQ_P)
+#define ABQ_SENTRY(SG, TM, TN, WM, WN)                                                       \
+    { 32, TM, TN, WM, WN, 1, 4, &launch_mfma_staged<ABQ_Q, ABQ_P, SG, false, TM, TN, WM, WN>, 128, \
+      StagedStages<ABQ_Q, ABQ_P, false, TM, TN, WM, WN>::kLds },
+static const KernelEntry kSigned[] = { ABQ_ENTRY_T(4, 4) ABQ_ENTRY_T(2, 4) ABQ_SENTRY(true, 2, 2, 2, 2) ABQ_SENTRY(true, 2, 1, 2, 2)
+                                       ABQ_SENTRY(true, 1, 1, 2, 2) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_T)
+                                       ABQ_SENTRY(true, 2, 2, 4, 2) ABQ_WENTRY_T(2, 2, 4, 4) ABQ_WENTRY_T(2, 4, 4, 2) };
+#if ABQ_Q < 8 && ABQ_P < 8
+static const KernelEntry kUnsigned[] = { ABQ_ENTRY_F(4, 4) ABQ_ENTRY_F(2, 4) ABQ_SENTRY(false, 2, 2, 2, 2) ABQ_SENTRY(false, 2, 1, 2, 2)
+                                         ABQ_SENTRY(false, 1, 1, 2, 2) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
+                                         ABQ_SENTRY(false, 2, 2, 4, 2) ABQ_WENTRY_F(2, 2, 4, 4) ABQ_WENTRY_F(2, 4, 4, 2) };
+#else
 static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
                                          ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_F) };
+#endif
 #else
 static const KernelEntry kSigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_T) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_T)
                                        ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_T) };
