@@ -224,7 +224,7 @@ def main():
     # ---------------------------------------------------------------- side measurement: prefill shapes
     if not args.no_extra:
         prefill = []
-        for (q, p, signed) in [(4, 4, True), (4, 4, False), (8, 8, True), (8, 8, False)]:
+        for (q, p, signed) in [(8, 2, True), (4, 4, True), (4, 4, False), (8, 8, True), (8, 8, False)]:
             for (N, K) in SHAPES:
                 wpl = random_planes(torch, (p, N, K // 32))
                 wtl = abq.relayout_planes(wpl)  # weights prepared once in the K-tiled layout
