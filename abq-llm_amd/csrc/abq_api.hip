@@ -692,27 +692,52 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
     const KernelTable *tg = find_table(registry().tiled_grouped, c.x_bits, c.w_bits, c.is_signed);
     if (!tg)
         return ABQ_ERR_UNSUPPORTED;
+    // entries with a fixed LDS size are the staged kernel's: one scale per K tile, i.e. groups of 128 only;
+    // it is preferred where both kernels have the tile (they come later in the table)
+    auto usable = [&](const KernelEntry &e) { return e.lds == 0 || state->group_size == 128; };
+    auto block_m = [](const KernelEntry &e) { return e.mi * e.tm * e.wm; };
+    auto block_n = [](const KernelEntry &e) { return e.mi * e.tn * e.wn; };
     int pick = -1;
     for (int i = 0; i < tg->count; ++i)
-        if (tg->entries[i].mi * tg->entries[i].tm * tg->entries[i].wm == c.block_m &&
-            tg->entries[i].mi * tg->entries[i].tn * tg->entries[i].wn == c.block_n)
+        if (usable(tg->entries[i]) && block_m(tg->entries[i]) == c.block_m && block_n(tg->entries[i]) == c.block_n)
             pick = i;
     if (pick < 0) {
         // no group-scale build of this tile: when the library chose, take the largest group-scale
-        // tile that still yields a workgroup per compute unit
+        // tile that still yields a workgroup per compute unit, else the smallest
         if (!state->auto_chosen)
             return ABQ_ERR_UNSUPPORTED;
-        pick = tg->count - 1;
-        for (int i = tg->count - 1; i >= 0; --i) {
-            const int bm = tg->entries[i].mi * tg->entries[i].tm * tg->entries[i].wm;
-            const int bn = tg->entries[i].mi * tg->entries[i].tn * tg->entries[i].wn;
-            if ((long)((state->M + bm - 1) / bm) * ((state->N + bn - 1) / bn) >= 200)
+        long best_area = 0, least_area = 0;
+        int least = -1;
+        for (int i = 0; i < tg->count; ++i) {
+            const KernelEntry &e = tg->entries[i];
+            if (!usable(e))
+                continue;
+            const int bm = block_m(e), bn = block_n(e);
+            const long area = (long)bm * bn;
+            if (least < 0 || area <= least_area) {
+                least = i;
+                least_area = area;
+            }
+            if ((long)((state->M + bm - 1) / bm) * ((state->N + bn - 1) / bn) >= 200 && area >= best_area) {
                 pick = i;
+                best_area = area;
+            }
         }
+        if (pick < 0)
+            pick = least;
+        if (pick < 0)
+            return ABQ_ERR_UNSUPPORTED;
     }
     const int xb_ = c.x_bits, wb_ = c.w_bits, sg_ = c.is_signed;
     entry_to_config(tg->entries[pick], ABQ_STRATEGY_TILED, xb_, wb_, sg_, 0, &state->cfg);
     state->variant = pick;
+    {
+        const KernelEntry &e = tg->entries[pick];
+        const int bm = block_m(e), bn = block_n(e);
+        state->grid_dim = abq_dim3{ (unsigned)(8 * (((state->N + bn - 1) / bn + 7) / 8) * ((state->M + bm - 1) / bm)), 1, 1 };
+        state->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
+        state->shared_mem_size = e.lds ? e.lds : 2 * (size_t)(bm + bn) * (e.kb + 16) + (bm + bn) * 4;
+    }
     return ABQ_OK;
 }
 

@@ -35,6 +35,7 @@
 #pragma once
 #include <type_traits>
 
+#include "abq_group_epilogue.h"
 #include "abq_kernels.h"
 
 namespace abq {
@@ -106,8 +107,25 @@ __device__ __forceinline__ void staged_load_to_lds(const v4u *src, unsigned lds_
                  : "memory");
 }
 
+// The same with four bytes per lane (lane l lands at M0 + 4 * l): the group scales.
+__device__ __forceinline__ void staged_load_dword_to_lds(const float *src, unsigned lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)
+                 : "memory");
+}
+
 // QB / PB: bits of the activation / weight fields (2, 4 or 8; ignored for FP6).
-template <int QB, int PB, bool SIGNED, bool FP6, int TM, int TN, int WM, int WN, int S>
+//
+// GROUPED: group-wise weight scales (one per 128 elements along K, i.e. per K tile: w_scale[N][K / 128]),
+// per-token activation scales, optional zero points and SiLU gate, fp16 output (see abq_group_epilogue.h).
+// A tile's BN scales travel with its records: one more wave load or two of four bytes per lane into the
+// tile's LDS stage, so they are covered by the same load counter and barrier as the records.  The int32
+// accumulators cover one K tile; the MFMAs run tile by tile of the wave's TM x TN (four K steps in a
+// row into the same accumulator), and while the matrix core works on one MFMA tile the vector ALU folds
+// the one finished before it into the fp32 accumulators (a convert and a multiply-add per element: as
+// many cycles as the four MFMAs take).  The last MFMA tile of a K tile is folded during the first of the
+// next K tile.
+template <int QB, int PB, bool SIGNED, bool FP6, int TM, int TN, int WM, int WN, int S, bool GROUPED = false>
 __global__ __launch_bounds__(64 * WM * WN, (WM * WN > 4 || TM * TN > 4) ? 1 : 2)
 void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_blocks, int n_blocks_per_xcd)
 {
@@ -115,10 +133,13 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     using TB = StagedOperand<PB, FP6>;
     constexpr int NW = WM * WN;
     constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
-    constexpr int BUF_BYTES = BM * TA::kRow + BN * TB::kRow;
+    constexpr int SC_OFF = BM * TA::kRow + BN * TB::kRow;      // GROUPED: the tile's scales follow its records
+    constexpr int BUF_BYTES = SC_OFF + (GROUPED ? 512 : 0);
     constexpr int NIA = BM * TA::kUnits / 64;                  // wave loads of 1 KiB per tile: activations
     constexpr int NI = NIA + BN * TB::kUnits / 64;             // ... and in all
-    constexpr int NPW = (NI + NW - 1) / NW;                    // per wave
+    constexpr int NPR = (NI + NW - 1) / NW;                    // per wave
+    constexpr int NPW = NPR + (GROUPED ? 1 : 0);               // GROUPED: and one load of 64 scales (256 bytes)
+    static_assert(!GROUPED || (!FP6 && TM * TN >= 2 && BN <= 128), "group scales: integer fields, two MFMA tiles per wave or more");
     constexpr int kSteps = FP6 ? 2 : 4;                        // MFMA K steps per tile of 128
     static_assert(FP6 || SIGNED || (QB < 8 && PB < 8), "unsigned 8-bit operands are not handled here");
     static_assert(S >= 3 && S <= 4, "three or four LDS stages");
@@ -149,7 +170,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     // issues NPW loads per tile.  Rows past the edge are clamped for loading and dropped at the store.
     uint32_t goff[NPW]; // 16-byte units from the start of the operand's records of one K tile
 #pragma unroll
-    for (int i = 0; i < NPW; ++i) {
+    for (int i = 0; i < NPR; ++i) {
         int q = wid + NW * i;
         if (q >= NI)
             q -= NW;
@@ -161,6 +182,12 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
             goff[i] = (uint32_t)min(n0 + v / TB::kUnits, N - 1) * TB::kUnits + v % TB::kUnits;
         }
     }
+    // GROUPED: the wave's last load of a tile brings the scales of 64 weight rows (waves take the 64-row
+    // blocks of the tile in turn; several waves bring the same block, which costs 256 bytes each).  The
+    // offset counts floats from the start of w_scale to the row's scale of K tile 0.
+    const int sc_block = wid % (BN / 64 > 0 ? BN / 64 : 1);
+    if constexpr (GROUPED)
+        goff[NPR] = (uint32_t)min(n0 + 64 * sc_block + lane, N - 1) * (uint32_t)ktiles;
     const size_t stride_a = (size_t)M * TA::kUnits, stride_b = (size_t)N * TB::kUnits;
     const unsigned lds0 = (unsigned)(size_t)smem; // LDS byte address of the first stage
 
@@ -195,7 +222,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
             q[p] = *reinterpret_cast<const v4i *>(lds_b + stage + ((p - NRA) / TB::kReads) * 32 * TB::kRow +
                                                   b_off[(p - NRA) % TB::kReads]);
     };
-    auto mfma = [&](Acc &c, const v4i(&q)[NR], int i, int j, int ks) {
+    auto mfma = [&](Acc &c, const v4i(&q)[NR], int i, int j, int ks, bool fresh = false) {
         const v4i *pa = &q[i * TA::kReads], *pb = &q[NRA + j * TB::kReads];
         if constexpr (FP6) {
             // dwords 0-5 of the 12 a lane holds are the first K step's operand, 6-11 the second's (the two
@@ -206,12 +233,20 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
                                    : __builtin_shufflevector(pb[1], pb[2], 2, 3, 4, 5, 6, 7, -1, -1);
             c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 2, 2, 0, 0, 0, 0);
         } else {
+            Acc zero;
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                zero[e] = 0;
             c = __builtin_amdgcn_mfma_i32_32x32x32_i8(staged_int8_operand<QB, SIGNED>(pa, ks),
-                                                      staged_int8_operand<PB, SIGNED>(pb, ks), c, 0, 0, 0);
+                                                      staged_int8_operand<PB, SIGNED>(pb, ks), fresh ? zero : c, 0, 0, 0);
         }
     };
     auto request = [&](int kt_req, int stage, int i) {
         const int kn = min(kt_req, ktiles - 1); // tiles past the end: copies of the last, into stages nobody reads
+        if (GROUPED && i == NPR) {
+            staged_load_dword_to_lds(a.w_scale + goff[i] + kn, lds0 + stage + SC_OFF + sc_block * 256);
+            return;
+        }
         int q = wid + NW * i;
         if (q >= NI)
             q -= NW;
@@ -232,6 +267,27 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
 #pragma unroll
     for (int p = 0; p < NR; ++p)
         read_piece(q0, 0, p);
+    // GROUPED: fp32 accumulators; scales of the K tile being multiplied (sc_cur), of the next one (sc_next)
+    // and of the MFMA tile still to be folded from the previous K tile (sc_last).  The signed route feeds
+    // value * 2^(8-bits) to the MFMA: the exact power of two that undoes it rides on the scale.
+    v16f facc[GROUPED ? TM : 1][GROUPED ? TN : 1];
+    float sc_cur[TN], sc_next[TN], sc_last = 0.f;
+    const float unshift = SIGNED ? 1.0f / (float)(1 << (16 - QB - PB)) : 1.0f;
+    auto read_scales = [&](float(&sc)[TN], int stage) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            sc[j] = *reinterpret_cast<const float *>(smem + stage + SC_OFF + (wn * 32 * TN + j * 32 + r) * 4) * unshift;
+    };
+    if constexpr (GROUPED) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    facc[i][j][e] = 0.f;
+        read_scales(sc_cur, 0);
+    }
     staged_wait_loads<NPW * (S - 2)>();
     __syncthreads();
 
@@ -258,16 +314,96 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         __syncthreads();                                                                                        \
     }
 
-    int kt = 0;
-    for (; kt + 2 <= ktiles; kt += 2) {
-        ABQ_STAGED_K_TILE(kt, q0, q1)
-        ABQ_STAGED_K_TILE(kt + 1, q1, q0)
+    // The same with group scales.  MFMA step k works on MFMA tile u = k / 4 of the wave's TM x TN (K step
+    // k % 4, the first one starting from zero); beside it the vector ALU folds a quarter of the tile
+    // finished before u: tile u - 1 of this K tile, or for u = 0 the last tile of the previous K tile (all
+    // zeros, with a zero scale, when there is none).
+#define ABQ_STAGED_K_TILE_G(KT, QC, QN)                                                                         \
+    {                                                                                                           \
+        constexpr int NU = TM * TN;                                                                             \
+        read_scales(sc_next, st_rd);                                                                            \
+        _Pragma("unroll") for (int k = 0; k < NM; ++k)                                                          \
+        {                                                                                                       \
+            const int u = k / 4, ks = k % 4, uf = (u + NU - 1) % NU;                                            \
+            mfma(acc[u / TN][u % TN], QC, u / TN, u % TN, ks, ks == 0);                                         \
+            _Pragma("unroll") for (int d = k * NPW / NM; d < (k + 1) * NPW / NM; ++d)                           \
+                request((KT) + S, st_req, d);                                                                   \
+            _Pragma("unroll") for (int p = k * NR / NM; p < (k + 1) * NR / NM; ++p)                             \
+                read_piece(QN, st_rd, p);                                                                       \
+            const float scf = u == 0 ? sc_last : sc_cur[uf % TN];                                               \
+            _Pragma("unroll") for (int e = 4 * ks; e < 4 * ks + 4; ++e)                                         \
+                facc[uf / TN][uf % TN][e] += (float)acc[uf / TN][uf % TN][e] * scf;                             \
+            __builtin_amdgcn_sched_barrier(0);                                                                  \
+        }                                                                                                       \
+        sc_last = sc_cur[TN - 1];                                                                               \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                          \
+            sc_cur[j] = sc_next[j];                                                                             \
+        st_req = st_req + BUF_BYTES == S * BUF_BYTES ? 0 : st_req + BUF_BYTES;                                  \
+        st_rd = st_rd + BUF_BYTES == S * BUF_BYTES ? 0 : st_rd + BUF_BYTES;                                     \
+        staged_wait_loads<NPW * (S - 2)>();                                                                     \
+        __syncthreads();                                                                                        \
     }
-    if (kt < ktiles)
-        ABQ_STAGED_K_TILE(kt, q0, q1)
+
+    int kt = 0;
+    if constexpr (GROUPED) {
+        for (; kt + 2 <= ktiles; kt += 2) {
+            ABQ_STAGED_K_TILE_G(kt, q0, q1)
+            ABQ_STAGED_K_TILE_G(kt + 1, q1, q0)
+        }
+        if (kt < ktiles)
+            ABQ_STAGED_K_TILE_G(kt, q0, q1)
+    } else {
+        for (; kt + 2 <= ktiles; kt += 2) {
+            ABQ_STAGED_K_TILE(kt, q0, q1)
+            ABQ_STAGED_K_TILE(kt + 1, q1, q0)
+        }
+        if (kt < ktiles)
+            ABQ_STAGED_K_TILE(kt, q0, q1)
+    }
 #undef ABQ_STAGED_K_TILE
+#undef ABQ_STAGED_K_TILE_G
     staged_wait_loads<0>(); // the clamped requests past the last tile: nothing of ours may be in flight below
 
+    if constexpr (GROUPED) {
+        // the last MFMA tile of the last K tile is still to be folded
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            facc[TM - 1][TN - 1][e] += (float)acc[TM - 1][TN - 1][e] * sc_last;
+        static_assert(!GROUPED || zero_point_lds_bytes(BM, BN) <= S * BUF_BYTES, "the zero-point staging fits the tile buffers");
+        group_scale_epilogue<TM, TN, WM, WN>(a, facc, smem, M, N, m0, n0, wm, wn, r, g, tid);
+        return;
+    }
+
+    auto result = [&](int i, int j, int e) -> int {
+        if constexpr (FP6)
+            return (int)(acc[i][j][e] * 64.0f); // both operands carry 1/8 as their unit: the sum is the result / 64, exactly
+        else
+            return SIGNED ? acc[i][j][e] >> (16 - QB - PB) : acc[i][j][e]; // signed fields sit at the top of their bytes
+    };
+    if (a.out_kind == 2) {
+        // per-token x per-channel scales, fp16 out (same arithmetic as store_result): the lane's TN
+        // channel scales are loaded once, a row's token scale once per row
+        float wsv[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            wsv[j] = a.w_scale[min(n0 + wn * 32 * TN + j * 32 + r, N - 1)];
+        _Float16 *out = reinterpret_cast<_Float16 *>(a.D);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4);
+                const float xsv = a.x_scale[min(m, M - 1)];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const int n = n0 + wn * 32 * TN + j * 32 + r;
+                    if (m < M && n < N)
+                        out[(size_t)m * N + n] = (_Float16)((float)result(i, j, e) * xsv * wsv[j]);
+                }
+            }
+        }
+        return;
+    }
     const StoreOperands so = store_operands(a);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -277,13 +413,8 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int m = m0 + wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4);
-                int v;
-                if constexpr (FP6)
-                    v = (int)(acc[i][j][e] * 64.0f); // both operands carry 1/8 as their unit: the sum is the result / 64, exactly
-                else
-                    v = SIGNED ? acc[i][j][e] >> (16 - QB - PB) : acc[i][j][e]; // signed fields sit at the top of their bytes
                 if (m < M && n < N)
-                    store_result_compact(so, m, n, v);
+                    store_result_compact(so, m, n, result(i, j, e));
             }
         }
     }
@@ -291,29 +422,32 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
 
 // LDS stages of a tile: as many (up to four) as leave room for the workgroups that share a compute
 // unit: two for the four-wave tiles when three stages of theirs fit twice, else one.
-template <int QB, int PB, bool FP6, int TM, int TN, int WM, int WN> struct StagedStages {
-    static constexpr int kBuf = 32 * (TM * WM * StagedOperand<QB, FP6>::kRow + TN * WN * StagedOperand<PB, FP6>::kRow);
+template <int QB, int PB, bool FP6, int TM, int TN, int WM, int WN, bool GROUPED = false> struct StagedStages {
+    static constexpr int kBuf = 32 * (TM * WM * StagedOperand<QB, FP6>::kRow + TN * WN * StagedOperand<PB, FP6>::kRow) +
+                                (GROUPED ? 512 : 0);
     static constexpr int value = (WM * WN <= 4 && TM * TN <= 4 && 2 * 4 * kBuf > 160 * 1024 && 2 * 3 * kBuf <= 160 * 1024) ? 3
                                  : (4 * kBuf <= 160 * 1024 ? 4 : 3);
     static constexpr size_t kLds = (size_t)value * kBuf;
     static_assert(3 * kBuf <= 160 * 1024, "three stages fit a compute unit's LDS");
 };
 
-template <int QB, int PB, bool SIGNED, bool FP6, int TM, int TN, int WM, int WN>
+template <int QB, int PB, bool SIGNED, bool FP6, int TM, int TN, int WM, int WN, bool GROUPED = false>
 static hipError_t launch_mfma_staged(const GemmArgs &a, hipStream_t stream)
 {
     constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
-    using Stages = StagedStages<QB, PB, FP6, TM, TN, WM, WN>;
+    using Stages = StagedStages<QB, PB, FP6, TM, TN, WM, WN, GROUPED>;
     constexpr int S = Stages::value;
+    if (GROUPED && a.group_size != 128)
+        return hipErrorInvalidValue; // one scale per K tile
     const int m_blocks = (a.M + BM - 1) / BM, n_blocks = (a.N + BN - 1) / BN;
     const int npx = (n_blocks + 7) / 8;
     const dim3 grid(8 * npx * m_blocks);
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S>),
+        reinterpret_cast<const void *>(&gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S, GROUPED>),
         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess)
         return attr;
-    hipLaunchKernelGGL((gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S>), grid, dim3(64 * WM * WN), Stages::kLds,
+    hipLaunchKernelGGL((gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S, GROUPED>), grid, dim3(64 * WM * WN), Stages::kLds,
                        stream, a, reinterpret_cast<const v4u *>(a.X), reinterpret_cast<const v4u *>(a.W), m_blocks, npx);
     return hipGetLastError();
 }

@@ -263,7 +263,7 @@ void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, i
         sum_b[i] = 0;
 
     v16i acc[TM][TN];
-    float facc[GROUPED ? TM : 1][GROUPED ? TN : 1][16];
+    v16f facc[GROUPED ? TM : 1][GROUPED ? TN : 1];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -388,46 +388,10 @@ void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, i
         __syncthreads();
     }
 
-    if (GROUPED && a.w_zero) {
-        // Weight zero points: out -= sum_g w_scale[n][g] * w_zero[n][g] * (sum of the activation codes
-        // of row m in group g).  The two factors are staged through LDS 32 groups at a time.
-        constexpr int GC = 32;
-        float *zs_x = reinterpret_cast<float *>(smem); // [GC][BM]
-        float *zs_w = zs_x + GC * BM;                  // [GC][BN]
-        static_assert(GC * (BM + BN) * 4 <= 2 * BUF_BYTES, "staging fits the tile buffers");
-        for (int g0 = 0; g0 < groups; g0 += GC) {
-            __syncthreads();
-            for (int u = tid; u < GC * BM; u += NT) {
-                const int rr = u / GC, gl = u % GC;
-                const int m = min(m0 + rr, M - 1);
-                zs_x[gl * BM + rr] = g0 + gl < groups ? (float)a.x_group_sums[(size_t)m * groups + g0 + gl] : 0.f;
-            }
-            for (int u = tid; u < GC * BN; u += NT) {
-                const int rr = u / GC, gl = u % GC;
-                const size_t idx = (size_t)min(n0 + rr, N - 1) * groups + g0 + gl;
-                zs_w[gl * BN + rr] = g0 + gl < groups ? a.w_scale[idx] * a.w_zero[idx] : 0.f;
-            }
-            __syncthreads();
-            for (int gl = 0; gl < GC; ++gl) {
-                float wz[TN];
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    wz[j] = zs_w[gl * BN + wn * 32 * TN + j * 32 + r];
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int e4 = 0; e4 < 4; ++e4) {
-                        const float4 sx4 = *reinterpret_cast<const float4 *>(&zs_x[gl * BM + wm * 32 * TM + i * 32 + 8 * e4 + 4 * g]);
-#pragma unroll
-                        for (int j = 0; j < TN; ++j) {
-                            facc[i][j][4 * e4 + 0] -= wz[j] * sx4.x;
-                            facc[i][j][4 * e4 + 1] -= wz[j] * sx4.y;
-                            facc[i][j][4 * e4 + 2] -= wz[j] * sx4.z;
-                            facc[i][j][4 * e4 + 3] -= wz[j] * sx4.w;
-                        }
-                    }
-            }
-        }
+    if constexpr (GROUPED) {
+        static_assert(!GROUPED || zero_point_lds_bytes(BM, BN) <= 2 * BUF_BYTES, "the zero-point staging fits the tile buffers");
+        group_scale_epilogue<TM, TN, WM, WN>(a, facc, smem, M, N, m0, n0, wm, wn, r, g, tid);
+        return;
     }
 
     const int k_fed = ktiles * KB;
@@ -442,24 +406,6 @@ void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, i
             for (int e = 0; e < 16; ++e) {
                 const int ml = wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4);
                 const int m = m0 + ml;
-                if (GROUPED) {
-                    const int mc = min(m, M - 1), nc = min(n, N - 1);
-                    float v = facc[i][j][e];
-                    if (a.x_zero) // activation zero points: a rank-one term
-                        v -= a.x_zero[mc] * a.w_zero_term[nc];
-                    v *= a.x_scale[mc];
-                    if (a.act) {
-                        // SiLU gate: columns come in blocks of 16 gate rows followed by their 16 up rows, so
-                        // the partner of lane r is lane r ^ 16 of the same MFMA tile (N is a multiple of 32)
-                        const float up = __shfl_xor(v, 16);
-                        if (m < M && n < N && !(r & 16))
-                            reinterpret_cast<_Float16 *>(a.D)[(size_t)m * (N / 2) + (n >> 5) * 16 + (n & 15)] =
-                                (_Float16)(silu(v) * up);
-                    } else if (m < M && n < N) {
-                        reinterpret_cast<_Float16 *>(a.D)[(size_t)m * N + n] = (_Float16)v;
-                    }
-                    continue;
-                }
                 unsigned v = (unsigned)acc[i][j][e];
                 if (SIGNED) {
                     v = (unsigned)((int)v >> (16 - Q - P));
@@ -539,8 +485,28 @@ static const KernelEntry kSigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_T) ABQ_TILED
 static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
                                          ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_F) };
 #endif
+// Group scales: the kernel above for groups of 64 and 128; for groups of 128 and pairs of single-field
+// widths also the staged kernel (entries with a fixed LDS size), which the host prefers.
+#if ABQ_FIELD1(ABQ_Q) && ABQ_FIELD1(ABQ_P)
+#define ABQ_SGENTRY(SG, TM, TN, WM, WN)                                                                  \
+    { 32, TM, TN, WM, WN, 1, 4, &launch_mfma_staged<ABQ_Q, ABQ_P, SG, false, TM, TN, WM, WN, true>, 128, \
+      StagedStages<ABQ_Q, ABQ_P, false, TM, TN, WM, WN, true>::kLds },
+#if ABQ_Q == 8 && ABQ_P == 8
+// two fragment sets of 64x64 8-bit operands, the int32 and the fp32 accumulators do not fit 256 registers
+#define ABQ_STAGED_GROUPED(SG) ABQ_SGENTRY(SG, 2, 1, 2, 2)
+#else
+#define ABQ_STAGED_GROUPED(SG) ABQ_SGENTRY(SG, 2, 2, 4, 2) ABQ_SGENTRY(SG, 2, 2, 2, 2) ABQ_SGENTRY(SG, 2, 1, 2, 2)
+#endif
+static const KernelEntry kSignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_T) ABQ_STAGED_GROUPED(true) };
+#if ABQ_Q < 8 && ABQ_P < 8
+static const KernelEntry kUnsignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_F) ABQ_STAGED_GROUPED(false) };
+#else
+static const KernelEntry kUnsignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_F) };
+#endif
+#else
 static const KernelEntry kSignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_T) };
 static const KernelEntry kUnsignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_F) };
+#endif
 
 #define ABQ_CAT_(a, b, c, d) a##b##c##d
 #define ABQ_CAT(a, b, c, d) ABQ_CAT_(a, b, c, d)

@@ -224,6 +224,51 @@ def test_group_scale_argument_checks(abq, oracle):
         abq.Gemm(x, w, True, out_kind=abq.OUT_F16_SCALED, x_scale=s, w_scale=s, group_size=128, w_zero=s)
     assert e.value.status == abq.ABQ_ERR_INVALID_ARG
 
+def _staged_grouped_lds(cfg):
+    """LDS of the staged kernel's group-scale variant for a tile: 3 or 4 stages of the packed records
+    (16 bytes per bit of width per row and K tile) plus 512 bytes of scales each."""
+    buf = 16 * (cfg.block_m * cfg.x_bits + cfg.block_n * cfg.w_bits) + 512
+    two_per_cu = cfg.block_m * cfg.block_n <= 128 * 128 and 2 * 4 * buf > 160 * 1024 >= 2 * 3 * buf
+    return buf * (3 if two_per_cu or 4 * buf > 160 * 1024 else 4)
+
+
+@pytest.mark.parametrize("q,p,signed", [(8, 2, True), (4, 4, True), (4, 4, False), (8, 4, True), (2, 2, True),
+                                        (2, 2, False), (4, 2, True), (8, 8, True)])
+def test_group_scale_staged_kernel_every_tile(abq, oracle, q, p, signed):
+    """Groups of 128 on pairs of 2-, 4- and 8-bit fields run on the kernel that loads the records and
+    the scales straight into LDS; every tile it is built for, picked by its tuple, with zero points
+    on both sides, on shapes with ragged edges, fewer K tiles than LDS stages and an odd tile count."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(100 * q + 10 * p + signed)
+    tiles = [c for c in abq.native_configs(q, p, signed)
+             if c.nstage == 4 and c.warp_k == 128 and (c.block_m, c.block_n) in ((256, 128), (128, 128), (128, 64))]
+    if (q, p) == (8, 8):
+        tiles = [c for c in tiles if (c.block_m, c.block_n) == (128, 64)]
+    assert tiles
+    lo_x, hi_x = (-(1 << (q - 1)), 1 << (q - 1)) if signed else (0, 1 << q)
+    lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed else (0, 1 << p)
+    for (M, N, K) in [(300, 200, 640), (70, 330, 256), (129, 65, 128)]:
+        G = K // 128
+        x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        xs = rng.uniform(0.01, 0.05, M)
+        xz = rng.integers(lo_x // 2, hi_x // 2 + 1, M).astype(np.float64)
+        wsc = rng.uniform(0.001, 0.02, (N, G))
+        wz = rng.integers(lo_w, hi_w, (N, G)).astype(np.float64)
+        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, 128)
+        wp = planes_dev(oracle.pack_i32(w, p))
+        kw = dict(x_scale=fdev(xs), w_scale=fdev(wsc), group_size=128, w_zero=fdev(wz), x_zero=fdev(xz),
+                  x_group_sums=torch.from_numpy(x.reshape(M, G, 128).sum(axis=2).astype(np.int32)).cuda())
+        kw["w_zero_term"] = abq.weight_zero_term(wp, signed, kw["w_scale"], kw["w_zero"], 128)
+        xt, wt = abq.relayout_planes(planes_dev(oracle.pack_i32(x, q))), abq.relayout_planes(wp)
+        for cfg in tiles:
+            g = abq.Gemm(xt, wt, signed, cfg=cfg, out_kind=abq.OUT_F16_SCALED, x_tiled=True, w_tiled=True, **kw)
+            assert g.strategy == "tiled" and (g.state.cfg.block_m, g.state.cfg.block_n) == (cfg.block_m, cfg.block_n)
+            assert g.state.shared_mem_size == _staged_grouped_lds(cfg), (g.config_name, g.state.shared_mem_size)
+            got = g.run()
+            torch.cuda.synchronize()
+            assert_close_rel(got.cpu().numpy(), want)
+
 
 # ------------------------------------------------------------------ BASELINE.json configs[4]
 
