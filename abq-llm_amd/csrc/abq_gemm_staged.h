@@ -369,8 +369,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
 #pragma unroll
         for (int e = 0; e < 16; ++e)
             facc[TM - 1][TN - 1][e] += (float)acc[TM - 1][TN - 1][e] * sc_last;
-        static_assert(!GROUPED || zero_point_lds_bytes(BM, BN) <= S * BUF_BYTES, "the zero-point staging fits the tile buffers");
-        group_scale_epilogue<TM, TN, WM, WN>(a, facc, smem, M, N, m0, n0, wm, wn, r, g, tid);
+        group_scale_epilogue<TM, TN, WM, WN, S * BUF_BYTES>(a, facc, smem, M, N, m0, n0, wm, wn, r, g, tid);
         return;
     }
 
@@ -388,6 +387,21 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         for (int j = 0; j < TN; ++j)
             wsv[j] = a.w_scale[min(n0 + wn * 32 * TN + j * 32 + r, N - 1)];
         _Float16 *out = reinterpret_cast<_Float16 *>(a.D);
+        using WT = WaveTileF16<TM, TN>;
+        // (the narrowest operand pairs have stages smaller than the waves' output tiles: direct stores there)
+        if (WM * WN * WT::kBytes <= S * BUF_BYTES && store_wave_tile_f16_ok(out, N, N)) {
+            // whole 128-byte lines per store: the wave's tile goes through a region of LDS of its own
+            float xsv[TM][16];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    xsv[i][e] = a.x_scale[min(m0 + wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4), M - 1)];
+            __syncthreads(); // every wave's loads have landed and its fragment reads are done: the stages are free
+            store_wave_tile_f16<TM, TN>(out, N, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, smem + wid * WT::kBytes, lane,
+                                        [&](int i, int j, int e) { return (float)result(i, j, e) * xsv[i][e] * wsv[j]; });
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll

@@ -389,8 +389,7 @@ void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, i
     }
 
     if constexpr (GROUPED) {
-        static_assert(!GROUPED || zero_point_lds_bytes(BM, BN) <= 2 * BUF_BYTES, "the zero-point staging fits the tile buffers");
-        group_scale_epilogue<TM, TN, WM, WN>(a, facc, smem, M, N, m0, n0, wm, wn, r, g, tid);
+        group_scale_epilogue<TM, TN, WM, WN, 2 * BUF_BYTES>(a, facc, smem, M, N, m0, n0, wm, wn, r, g, tid);
         return;
     }
 

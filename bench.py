@@ -74,7 +74,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="plain stream launches instead of HIP graphs")
-    ap.add_argument("--no-extra", action="store_true", help="skip the prefill side measurements")
+    ap.add_argument("--no-extra", action="store_true", help="skip the side measurements")
+    ap.add_argument("--extras", default=None,
+                    help="comma-separated side measurements to run (default all): prefill, prefill_fp6, library_int8_gemm, "
+                         "decode_fused_linears, decode_group_scales, decoder_layer_w2a8_group128")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (the known-size kernel that "
                          "calibrates FETCH_SIZE / WRITE_SIZE in a counter run)")
@@ -222,7 +225,10 @@ def main():
                                      "sample": "M=1 N=4096 K=4096 once, engine/test_any_mma.cu compute_ref restated"}}
 
     # ---------------------------------------------------------------- side measurement: prefill shapes
-    if not args.no_extra:
+    def want(name):
+        return not args.no_extra and (args.extras is None or name in args.extras.split(","))
+
+    if want("prefill"):
         prefill = []
         for (q, p, signed) in [(8, 2, True), (4, 4, True), (4, 4, False), (8, 8, True), (8, 8, False)]:
             for (N, K) in SHAPES:
@@ -255,7 +261,12 @@ def main():
                     del gm, xpl, ws
                 del wpl, wtl
         extra["prefill"] = prefill
+        for r in prefill:
+            log("prefill W%dA%d %s M=%d N=%d K=%d  %.1f us  %.1f TOPS (%.1f%% of int8 MFMA peak)"
+                % (r["w_bits"], r["x_bits"], "int" if r["signed"] else "uint", r["M"], r["N"], r["K"], r["us"],
+                   r["tops"], 100 * r["mfma_frac"]))
 
+    if want("prefill_fp6"):
         # The same W4A4 GEMMs on the FP6 matrix-core route (exact for operands of at most 4 bits unsigned /
         # 5 bits signed): weights prepared once as FP6 records; activations either converted from planes inside
         # the timed call, as above, or already FP6 (what the fused quantise-and-pack kernel hands over).
@@ -268,8 +279,13 @@ def main():
                     xf6 = abq.relayout_planes_fp6(xpl, signed)
                     ws = torch.empty((K // 128) * M * 96, dtype=torch.uint8, device="cuda")
                     row = dict(w_bits=4, x_bits=4, signed=signed, M=M, N=N, K=K)
+                    xsc = torch.rand(M, device="cuda") * 0.01 + 0.001
+                    wsc = torch.rand(N, device="cuda") * 0.01 + 0.001
                     for tag, gm in (("planes_in", abq.Gemm(xpl, wf6, signed, w_fp6=4, workspace=ws)),
-                                    ("fp6_in", abq.Gemm(xf6, wf6, signed, x_fp6=4, w_fp6=4))):
+                                    ("fp6_in", abq.Gemm(xf6, wf6, signed, x_fp6=4, w_fp6=4)),
+                                    # per-token x per-channel scales, fp16 out: the epilogue the model's linears use
+                                    ("fp6_in_f16_scaled", abq.Gemm(xf6, wf6, signed, x_fp6=4, w_fp6=4, out_kind=abq.OUT_F16_SCALED,
+                                                                   x_scale=xsc, w_scale=wsc))):
                         gm.run()
                         torch.cuda.synchronize()
                         reps = 5
@@ -291,10 +307,14 @@ def main():
                         row["kernel"] = "%s:%s" % (gm.strategy, gm.config_name)
                         del gm
                     prefill_fp6.append(row)
-                    del xpl, xf6, ws
+                    log("prefill FP6 W4A4 %s M=%d N=%d K=%d  planes in %.0f  FP6 in %.0f  FP6 in, scaled fp16 out %.0f TOPS"
+                        % ("int" if signed else "uint", M, N, K, row["planes_in"]["tops"], row["fp6_in"]["tops"],
+                           row["fp6_in_f16_scaled"]["tops"]))
+                    del xpl, xf6, ws, xsc, wsc
                 del wf6
         extra["prefill_fp6"] = prefill_fp6
 
+    if want("library_int8_gemm"):
         # Yardstick for the prefill figures: the vendor library's plain int8 GEMM (torch._int_mm, operands
         # already int8 and K-major, nothing to unpack) on the same shapes, timed the same way.
         vendor = []
@@ -322,6 +342,7 @@ def main():
             vendor = {"unavailable": repr(exc)[:120]}
         extra["library_int8_gemm"] = vendor
 
+    if want("decode_fused_linears"):
         # ------------------------------------------------------------ side measurement: several linears per launch
         # QKV (N = 3 * 4096) and gate + up (N = 2 * 11008) share their activations, so each is one GEMM
         # over concatenated weight planes: the launch + ramp cost is paid once for 12 or 22 MB.
@@ -355,6 +376,7 @@ def main():
             del Wr
         extra["decode_fused_linears"] = fused
 
+    if want("decode_group_scales"):
         # ------------------------------------------------------------ side measurement: decode with the dequantising epilogue
         # group-128 weight scales and zero points, per-token scales, fp16 output (the decode kernel's
         # group-scale variant); bytes add the scale and zero-point arrays to the packed weights
@@ -396,6 +418,7 @@ def main():
             del Wr
         extra["decode_group_scales"] = deq
 
+    if want("decoder_layer_w2a8_group128"):
         # ------------------------------------------------------------ side measurement: one decoder layer's linears
         # BASELINE configs[4]: W2A8, 2-bit weights with group-128 scales and zero points (prepared layout),
         # activations quantised per token on the device inside the timed call, fp16 output; gate and up run
@@ -440,10 +463,7 @@ def main():
                     % (name, tokens, N, K, us, tops, 100 * tops / INT8_MFMA_PEAK_TOPS))
                 del gr, gm, out, x, xt, wt
         extra["decoder_layer_w2a8_group128"] = layer
-        for r in prefill:
-            log("prefill W%dA%d %s M=%d N=%d K=%d  %.1f us  %.1f TOPS (%.1f%% of int8 MFMA peak)"
-                % (r["w_bits"], r["x_bits"], "int" if r["signed"] else "uint", r["M"], r["N"], r["K"], r["us"],
-                   r["tops"], 100 * r["mfma_frac"]))
+
 
     result = {
         "metric": "effective int TOPS (2*M*N*K / t) over the LLaMA-7B W2A8 decode GEMMs, M in {1,4,8}",
