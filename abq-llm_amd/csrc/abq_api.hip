@@ -601,6 +601,83 @@ abq_status abq_gemm_init(const abq_tile_config *cfg, int x_bits, int w_bits, int
 
 static size_t planes_bytes(int rows, int k, int bits) { return (size_t)bits * rows * (k / 32) * 4; }
 
+// Large tiles against the 128x128 tile, from sweeps over M = 256 .. 16384 and the LLaMA widths on MI355X.
+// A large tile (one workgroup per compute unit) moves fewer bytes from L2 per MFMA and runs `gain` times
+// faster per output element once the chip is kept full over several rounds of workgroups (`gain1` while
+// the grid is a single round), but its grid is quantised: a last round that is partly empty costs up to
+// a full one.  Two 128x128 workgroups share a compute unit and one of them alone runs nearly twice as
+// fast, so that grid degrades smoothly with its tile count.
+struct LargeTile {
+    int tm, tn, wm, wn; // MFMA tiles per wave, waves along M and N
+    double gain1, gain;
+};
+
+// Cost of the shape on the 128x128 tile, in units of the time two co-resident 128x128 workgroups take.
+static double cost_128x128(int M, int N)
+{
+    const long t = (long)((M + 127) / 128) * ((N + 127) / 128);
+    return t <= 256 ? 0.6 : t <= 512 ? 1.0 : (double)t / 512.0;
+}
+
+static double cost_large(const LargeTile &c, int M, int N)
+{
+    const int bm = 32 * c.tm * c.wm, bn = 32 * c.tn * c.wn;
+    const long t = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+    const double area = (double)bm * bn / (2.0 * 128 * 128);
+    if (t <= 256)
+        return area / c.gain1;
+    // workgroups do not run in lockstep, so a short last round partly hides behind the others; not so for the
+    // 256x256 tiles, whose workgroups are few and long
+    const double frac = (double)(t % 256) / 256.0;
+    const double tail = area >= 2.0 ? (frac > 0 ? 1.0 : 0.0) : (1.5 * frac < 1.0 ? 1.5 * frac : 1.0);
+    return ((double)(t / 256) + tail) * area / c.gain;
+}
+
+// Index in `entries` of the best large tile that beats the 128x128 tile by a margin, or -1.
+static int pick_large_tile(const KernelEntry *entries, int count, const LargeTile *cands, int ncands, int M, int N)
+{
+    double best = 0.92 * cost_128x128(M, N);
+    int pick = -1;
+    for (int k = 0; k < ncands; ++k) {
+        const double cost = cost_large(cands[k], M, N);
+        if (cost >= best)
+            continue;
+        for (int i = 0; i < count; ++i)
+            if (entries[i].tm == cands[k].tm && entries[i].tn == cands[k].tn && entries[i].wm == cands[k].wm &&
+                entries[i].wn == cands[k].wn && entries[i].kb == 128) {
+                best = cost;
+                pick = i;
+            }
+    }
+    return pick;
+}
+
+// Large tiles of the int8 kernels per operand pair: activations wider than the weights (W2A8, W4A8, W2A4)
+// gain most from tiles that are wide in N, 128x256 on the staged kernel and 256x256 (sixteen waves); signed
+// W8A8 from 256x128 and 256x256 (eight waves of 64x128).  Pairs of widths made of several fields keep the
+// thresholds below.
+static int large_tiles_int8(int x_bits, int w_bits, int is_signed, const LargeTile **out)
+{
+    static const LargeTile wide_n[] = { { 2, 2, 4, 4, 1.22, 1.22 }, { 2, 2, 2, 4, 1.04, 1.15 } };
+    static const LargeTile w8a8[] = { { 2, 4, 4, 2, 1.45, 1.45 }, { 2, 2, 4, 2, 1.25, 1.30 } };
+    const bool field = (x_bits == 2 || x_bits == 4 || x_bits == 8) && (w_bits == 2 || w_bits == 4 || w_bits == 8);
+    if (field && x_bits > w_bits && (is_signed || x_bits < 8)) {
+        *out = wide_n;
+        return 2;
+    }
+    if (x_bits == 8 && w_bits == 8 && is_signed) {
+        *out = w8a8;
+        return 2;
+    }
+    // equal widths below 8 bits (W4A4, W2A2 on the int8 route): only 256x256 beats 128x128, and only just
+    static const LargeTile narrow[] = { { 2, 4, 4, 2, 1.10, 1.10 } };
+    if (field && x_bits == w_bits && x_bits < 8) {
+        *out = narrow;
+        return 1;
+    }
+    return 0;
+}
+
 // Picks the tiled-kernel tile for a shape.  Measured on MI355X (W4A4 / W8A8 / W2A8, LLaMA shapes):
 // the 256x128 tile of eight waves (least L2 -> L1 traffic per MFMA) is the fastest once it yields
 // one workgroup per compute unit, then 128x128; below that, smaller tiles win by filling the chip.
@@ -620,7 +697,14 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
     // tiles: the large tile pays as soon as it covers about two thirds of the compute units
     const bool staged = c.x_bits == 8 && c.w_bits == 8 && c.is_signed;
     int pick = -1;
+    const LargeTile *cands = nullptr;
+    const int ncands = large_tiles_int8(c.x_bits, c.w_bits, c.is_signed, &cands);
+    const bool modelled = ncands > 0 && (long)((st->M + 127) / 128) * ((st->N + 127) / 128) >= 200;
+    if (modelled)
+        pick = pick_large_tile(tt->entries, tt->count, cands, ncands, st->M, st->N);
     for (const auto &o : order) {
+        if (modelled && 32 * o[0] * o[2] * 32 * o[1] * o[3] > 128 * 128)
+            continue; // the large tiles have been weighed against 128x128 above
         if (o[1] == 4 && c.x_bits + c.w_bits < 16)
             continue;
         const int bm = 32 * o[0] * o[2], bn = 32 * o[1] * o[3];
@@ -651,12 +735,16 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
         return ABQ_ERR_UNSUPPORTED;
     int count = 0;
     const KernelEntry *es = fp6_entries(&count);
+    // The 256x128 tile of eight waves against 128x128 by the cost model above (it pays over several rounds
+    // of workgroups; alone on a compute unit, in a single round, it hides less latency than two 128x128
+    // workgroups do); below a chip's worth of 128x128 tiles the smaller ones:
     // { TM, TN, waves along M, waves along N, workgroups needed }
-    // (the kernel runs at the rate L2 delivers its tiles, so the 256x128 tile wins as soon as it covers about
-    // two thirds of the compute units: M = 512, N = 11008 runs 1.4 times faster on its 172 tiles than on 344
-    // tiles of 128x128)
-    static const int order[][5] = { { 2, 2, 4, 2, 160 }, { 2, 2, 2, 2, 250 }, { 2, 1, 2, 2, 400 }, { 1, 1, 2, 2, 0 } };
+    static const LargeTile large[] = { { 2, 2, 4, 2, 0.95, 1.18 } };
+    static const int order[][5] = { { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 400 }, { 1, 1, 2, 2, 0 } };
     int pick = -1;
+    // (beyond 8192 rows the 256x128 tile falls behind 128x128 again: 1620-2070 against 1820-2100 TOPS at 16384 rows)
+    if ((long)((st->M + 127) / 128) * ((st->N + 127) / 128) >= 200 && st->M <= 8192)
+        pick = pick_large_tile(es, count, large, 1, st->M, st->N);
     for (const auto &o : order) {
         const int bm = 32 * o[0] * o[2], bn = 32 * o[1] * o[3];
         const long tiles = (long)((st->M + bm - 1) / bm) * ((st->N + bn - 1) / bn);
@@ -698,36 +786,26 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
     auto block_m = [](const KernelEntry &e) { return e.mi * e.tm * e.wm; };
     auto block_n = [](const KernelEntry &e) { return e.mi * e.tn * e.wn; };
     int pick = -1;
-    for (int i = 0; i < tg->count; ++i)
-        if (usable(tg->entries[i]) && block_m(tg->entries[i]) == c.block_m && block_n(tg->entries[i]) == c.block_n)
-            pick = i;
-    if (pick < 0) {
-        // no group-scale build of this tile: when the library chose, take the largest group-scale
-        // tile that still yields a workgroup per compute unit, else the smallest
-        if (!state->auto_chosen)
-            return ABQ_ERR_UNSUPPORTED;
-        long best_area = 0, least_area = 0;
-        int least = -1;
-        for (int i = 0; i < tg->count; ++i) {
-            const KernelEntry &e = tg->entries[i];
-            if (!usable(e))
+    if (state->auto_chosen) {
+        // The fold of the int32 tiles into fp32 bounds these kernels more than the tile traffic does, so tile
+        // sizes from 128x128 up run within a few percent of each other (sweep over M = 256 .. 16384 and the
+        // LLaMA widths): 128x128 once it fills the chip, below that 128x64, then 64x64.
+        const long t128 = (long)((state->M + 127) / 128) * ((state->N + 127) / 128);
+        static const int order[][3] = { { 128, 128, 300 }, { 128, 64, 64 }, { 64, 64, 0 } };
+        for (const auto &o : order) {
+            if (pick >= 0 || t128 < o[2])
                 continue;
-            const int bm = block_m(e), bn = block_n(e);
-            const long area = (long)bm * bn;
-            if (least < 0 || area <= least_area) {
-                least = i;
-                least_area = area;
-            }
-            if ((long)((state->M + bm - 1) / bm) * ((state->N + bn - 1) / bn) >= 200 && area >= best_area) {
-                pick = i;
-                best_area = area;
-            }
+            for (int i = 0; i < tg->count; ++i) // the last match: the staged kernel's entry where there is one
+                if (usable(tg->entries[i]) && block_m(tg->entries[i]) == o[0] && block_n(tg->entries[i]) == o[1])
+                    pick = i;
         }
-        if (pick < 0)
-            pick = least;
-        if (pick < 0)
-            return ABQ_ERR_UNSUPPORTED;
+    } else {
+        for (int i = 0; i < tg->count; ++i)
+            if (usable(tg->entries[i]) && block_m(tg->entries[i]) == c.block_m && block_n(tg->entries[i]) == c.block_n)
+                pick = i;
     }
+    if (pick < 0)
+        return ABQ_ERR_UNSUPPORTED;
     const int xb_ = c.x_bits, wb_ = c.w_bits, sg_ = c.is_signed;
     entry_to_config(tg->entries[pick], ABQ_STRATEGY_TILED, xb_, wb_, sg_, 0, &state->cfg);
     state->variant = pick;

@@ -134,12 +134,12 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     constexpr int NW = WM * WN;
     constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
     constexpr int SC_OFF = BM * TA::kRow + BN * TB::kRow;      // GROUPED: the tile's scales follow its records
-    constexpr int BUF_BYTES = SC_OFF + (GROUPED ? 512 : 0);
+    constexpr int BUF_BYTES = SC_OFF + (GROUPED ? (BN > 128 ? 4 * BN : 512) : 0);
     constexpr int NIA = BM * TA::kUnits / 64;                  // wave loads of 1 KiB per tile: activations
     constexpr int NI = NIA + BN * TB::kUnits / 64;             // ... and in all
     constexpr int NPR = (NI + NW - 1) / NW;                    // per wave
     constexpr int NPW = NPR + (GROUPED ? 1 : 0);               // GROUPED: and one load of 64 scales (256 bytes)
-    static_assert(!GROUPED || (!FP6 && TM * TN >= 2 && BN <= 128), "group scales: integer fields, two MFMA tiles per wave or more");
+    static_assert(!GROUPED || (!FP6 && TM * TN >= 2 && BN / 64 <= WM * WN), "group scales: integer fields, two MFMA tiles per wave or more");
     constexpr int kSteps = FP6 ? 2 : 4;                        // MFMA K steps per tile of 128
     static_assert(FP6 || SIGNED || (QB < 8 && PB < 8), "unsigned 8-bit operands are not handled here");
     static_assert(S >= 3 && S <= 4, "three or four LDS stages");
@@ -438,7 +438,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
 // unit: two for the four-wave tiles when three stages of theirs fit twice, else one.
 template <int QB, int PB, bool FP6, int TM, int TN, int WM, int WN, bool GROUPED = false> struct StagedStages {
     static constexpr int kBuf = 32 * (TM * WM * StagedOperand<QB, FP6>::kRow + TN * WN * StagedOperand<PB, FP6>::kRow) +
-                                (GROUPED ? 512 : 0);
+                                (GROUPED ? (32 * TN * WN > 128 ? 128 * TN * WN : 512) : 0);
     static constexpr int value = (WM * WN <= 4 && TM * TN <= 4 && 2 * 4 * kBuf > 160 * 1024 && 2 * 3 * kBuf <= 160 * 1024) ? 3
                                  : (4 * kBuf <= 160 * 1024 ? 4 : 3);
     static constexpr size_t kLds = (size_t)value * kBuf;

@@ -467,13 +467,24 @@ static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 #define ABQ_SENTRY(SG, TM, TN, WM, WN)                                                       \
     { 32, TM, TN, WM, WN, 1, 4, &launch_mfma_staged<ABQ_Q, ABQ_P, SG, false, TM, TN, WM, WN>, 128, \
       StagedStages<ABQ_Q, ABQ_P, false, TM, TN, WM, WN>::kLds },
+// Activations wider than the weights: a 128 x 256 tile (eight waves of 64 x 64, 2 along M, 4 along N) moves fewer
+// bytes per MFMA than 256 x 128, since a row of activations is the longer record.
+#if ABQ_Q > ABQ_P
+#define ABQ_STAGED_WIDE_N(SG) ABQ_SENTRY(SG, 2, 2, 2, 4)
+#define ABQ_STAGED_WIDE_N_GROUPED(SG) ABQ_SGENTRY(SG, 2, 2, 2, 4)
+#else
+#define ABQ_STAGED_WIDE_N(SG)
+#define ABQ_STAGED_WIDE_N_GROUPED(SG)
+#endif
 static const KernelEntry kSigned[] = { ABQ_ENTRY_T(4, 4) ABQ_ENTRY_T(2, 4) ABQ_SENTRY(true, 2, 2, 2, 2) ABQ_SENTRY(true, 2, 1, 2, 2)
                                        ABQ_SENTRY(true, 1, 1, 2, 2) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_T)
-                                       ABQ_SENTRY(true, 2, 2, 4, 2) ABQ_WENTRY_T(2, 2, 4, 4) ABQ_WENTRY_T(2, 4, 4, 2) };
+                                       ABQ_SENTRY(true, 2, 2, 4, 2) ABQ_WENTRY_T(2, 2, 4, 4) ABQ_WENTRY_T(2, 4, 4, 2)
+                                       ABQ_STAGED_WIDE_N(true) };
 #if ABQ_Q < 8 && ABQ_P < 8
 static const KernelEntry kUnsigned[] = { ABQ_ENTRY_F(4, 4) ABQ_ENTRY_F(2, 4) ABQ_SENTRY(false, 2, 2, 2, 2) ABQ_SENTRY(false, 2, 1, 2, 2)
                                          ABQ_SENTRY(false, 1, 1, 2, 2) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
-                                         ABQ_SENTRY(false, 2, 2, 4, 2) ABQ_WENTRY_F(2, 2, 4, 4) ABQ_WENTRY_F(2, 4, 4, 2) };
+                                         ABQ_SENTRY(false, 2, 2, 4, 2) ABQ_WENTRY_F(2, 2, 4, 4) ABQ_WENTRY_F(2, 4, 4, 2)
+                                         ABQ_STAGED_WIDE_N(false) };
 #else
 static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
                                          ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_F) };
@@ -494,7 +505,7 @@ static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TIL
 // two fragment sets of 64x64 8-bit operands, the int32 and the fp32 accumulators do not fit 256 registers
 #define ABQ_STAGED_GROUPED(SG) ABQ_SGENTRY(SG, 2, 1, 2, 2)
 #else
-#define ABQ_STAGED_GROUPED(SG) ABQ_SGENTRY(SG, 2, 2, 4, 2) ABQ_SGENTRY(SG, 2, 2, 2, 2) ABQ_SGENTRY(SG, 2, 1, 2, 2)
+#define ABQ_STAGED_GROUPED(SG) ABQ_SGENTRY(SG, 2, 2, 4, 2) ABQ_SGENTRY(SG, 2, 2, 2, 2) ABQ_SGENTRY(SG, 2, 1, 2, 2) ABQ_STAGED_WIDE_N_GROUPED(SG)
 #endif
 static const KernelEntry kSignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_T) ABQ_STAGED_GROUPED(true) };
 #if ABQ_Q < 8 && ABQ_P < 8

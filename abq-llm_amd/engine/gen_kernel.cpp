@@ -194,6 +194,13 @@ std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits, bool is_signed)
     out.push_back(Tile{ 256, 128, 128, 64, 64, 128, 32, 32, 32, 4, 2, { 4 } });
     out.push_back(Tile{ 256, 256, 128, 64, 64, 128, 32, 32, 32, 4, 4, { 4 } });
     out.push_back(Tile{ 256, 256, 128, 64, 128, 128, 32, 32, 32, 4, 2, { 4 } });
+    // activations wider than the weights, both of a single field (2, 4, 8 bits): 128 x 256 on the staged
+    // kernel, eight waves of 64 x 64 (2 along M, 4 along N)
+    {
+        const bool field = (x_bits == 2 || x_bits == 4 || x_bits == 8) && (w_bits == 2 || w_bits == 4 || w_bits == 8);
+        if (field && x_bits > w_bits && (is_signed || x_bits < 8))
+            out.push_back(Tile{ 128, 256, 128, 64, 64, 128, 32, 32, 32, 2, 4, { 4 } });
+    }
     const int half[][2] = { { 2, 4 }, { 2, 2 } };
     for (const auto &t : half)
         out.push_back(Tile{ 64 * t[0], 64 * t[1], 64, 32 * t[0], 32 * t[1], 64, 32, 32, 32, 2, 2, { 4 } });

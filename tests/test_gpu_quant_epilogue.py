@@ -226,8 +226,8 @@ def test_group_scale_argument_checks(abq, oracle):
 
 def _staged_grouped_lds(cfg):
     """LDS of the staged kernel's group-scale variant for a tile: 3 or 4 stages of the packed records
-    (16 bytes per bit of width per row and K tile) plus 512 bytes of scales each."""
-    buf = 16 * (cfg.block_m * cfg.x_bits + cfg.block_n * cfg.w_bits) + 512
+    (16 bytes per bit of width per row and K tile) plus the tile's scales (at least 512 bytes) each."""
+    buf = 16 * (cfg.block_m * cfg.x_bits + cfg.block_n * cfg.w_bits) + max(512, 4 * cfg.block_n)
     two_per_cu = cfg.block_m * cfg.block_n <= 128 * 128 and 2 * 4 * buf > 160 * 1024 >= 2 * 3 * buf
     return buf * (3 if two_per_cu or 4 * buf > 160 * 1024 else 4)
 
@@ -241,7 +241,9 @@ def test_group_scale_staged_kernel_every_tile(abq, oracle, q, p, signed):
     from oracle import quantizer as Q
     rng = np.random.default_rng(100 * q + 10 * p + signed)
     tiles = [c for c in abq.native_configs(q, p, signed)
-             if c.nstage == 4 and c.warp_k == 128 and (c.block_m, c.block_n) in ((256, 128), (128, 128), (128, 64))]
+             if c.nstage == 4 and c.warp_k == 128 and (c.warp_m, c.warp_n) in ((64, 64), (64, 32)) and
+             (c.block_m, c.block_n) in ((256, 128), (128, 128), (128, 64), (128, 256))]
+    assert ((128, 256) in [(c.block_m, c.block_n) for c in tiles]) == (q > p)
     if (q, p) == (8, 8):
         tiles = [c for c in tiles if (c.block_m, c.block_n) == (128, 64)]
     assert tiles
