@@ -277,6 +277,31 @@ def test_fp6_fp16_epilogues(abq, oracle):
     assert np.array_equal(got.view(np.uint16), want16.view(np.uint16))
 
 
+@pytest.mark.parametrize("q,p,fp6", [(4, 4, True), (8, 2, False), (4, 4, False), (8, 8, False), (2, 2, False)])
+def test_scaled_fp16_epilogue_every_staged_tile(abq, oracle, q, p, fp6):
+    """Per-token x per-channel scales with fp16 output on every tile of the LDS-staged kernels: once with
+    an output width the whole-line store takes (multiple of 8) and once with one it does not, ragged M."""
+    rng = np.random.default_rng(900 + 10 * q + p + fp6)
+    tiles = [c for c in abq.native_configs(q, p, True) if c.nstage == (5 if fp6 else 4) and c.warp_k == 128]
+    assert tiles
+    for (M, N, K) in [(130, 328, 384), (70, 203, 256)]:
+        x, w = rand_vals(rng, M, K, q, True), rand_vals(rng, N, K, p, True)
+        xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
+        if fp6:
+            xo, wo, kw = abq.relayout_planes_fp6(xd, True), abq.relayout_planes_fp6(wd, True), dict(x_fp6=q, w_fp6=p)
+        else:
+            xo, wo, kw = abq.relayout_planes(xd), abq.relayout_planes(wd), dict(x_tiled=True, w_tiled=True)
+        xs = torch.rand(M, device="cuda") * 0.01 + 0.001
+        ws = torch.rand(N, device="cuda") * 0.01 + 0.001
+        want = (oracle.np_gemm(x, w).astype(np.float64) * xs.cpu().numpy().astype(np.float64)[:, None]
+                * ws.cpu().numpy().astype(np.float64)[None, :])
+        for cfg in tiles:
+            g = abq.Gemm(xo, wo, True, cfg=cfg, out_kind=abq.OUT_F16_SCALED, x_scale=xs, w_scale=ws, **kw)
+            got = g.run().float().cpu().numpy()
+            # tolerance of the fp16 dequantised output: 1e-2 relative
+            assert np.all(np.abs(got - want) <= 1e-2 * np.abs(want) + 1e-6), (g.config_name, M, N, K)
+
+
 @pytest.mark.parametrize("signed", [True, False])
 def test_config2_w4a4_prefill_full_size_fp6(abq, oracle, signed):
     """W4A4 at M in {512, 2048} on the LLaMA-7B shapes through the FP6 route: exact against the fp64

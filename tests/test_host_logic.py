@@ -328,3 +328,43 @@ def test_gen_kernel_native_space_is_what_the_library_instantiates(gen_kernel, ab
             gen = set(_tuples(text))
             native = set(c.as_tuple() for c in abq.native_configs(q, p, signed))
             assert gen == native, (q, p, signed)
+
+
+def test_prefill_tile_choice_on_the_baseline_shapes(abq):
+    """The tile the library picks for prepared operands, pinned on shapes of BASELINE.json configs[2] and
+    configs[4] and on a few where the sweep in profiles/prefill_tile_sweep.md separates the tiles clearly:
+    large tiles only where their quantised grids pay, 128x128 in between, small tiles for small grids."""
+    lib = abq.lib()
+
+    def picked(q, p, M, N, K, layout, group=0):
+        rc, st = _init(abq, q=q, p=p, M=M, N=N, K=K, out_kind=abq.OUT_F16_SCALED if group else abq.OUT_I32)
+        assert rc == 0
+        if group:
+            assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, group) == 0
+        assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), layout, layout) == 0
+        c = st.cfg
+        return (c.block_m, c.block_n, c.warp_m, c.warp_n, c.nstage)
+
+    T, F6 = abq.LAYOUT_TILED, abq.LAYOUT_FP6
+    # W4A4 on the FP6 route
+    assert picked(4, 4, 512, 4096, 4096, F6) == (64, 64, 32, 32, 5)
+    assert picked(4, 4, 512, 11008, 4096, F6) == (128, 128, 64, 64, 5)
+    assert picked(4, 4, 1024, 11008, 4096, F6) == (128, 128, 64, 64, 5)      # 344 tiles of 256x128: two rounds, one nearly empty
+    assert picked(4, 4, 2048, 12288, 4096, F6) == (256, 128, 64, 64, 5)      # 768 tiles: three full rounds
+    assert picked(4, 4, 16384, 4096, 4096, F6) == (128, 128, 64, 64, 5)
+    # W2A8: tiles that are wide in N
+    assert picked(8, 2, 2048, 4096, 4096, T) == (128, 128, 64, 64, 4)
+    assert picked(8, 2, 4096, 11008, 4096, T) == (128, 256, 64, 64, 4)
+    assert picked(8, 2, 1024, 12288, 4096, T) == (128, 128, 64, 64, 4)
+    assert picked(8, 2, 4096, 4096, 4096, T) == (256, 256, 64, 64, 4)
+    assert picked(8, 2, 512, 4096, 4096, T) == (64, 64, 32, 32, 4)
+    # signed W8A8
+    assert picked(8, 8, 2048, 4096, 4096, T) == (256, 128, 64, 64, 4)
+    assert picked(8, 8, 1024, 4096, 4096, T) == (128, 128, 64, 64, 4)
+    assert picked(8, 8, 4096, 4096, 4096, T) == (256, 256, 64, 128, 4)
+    assert picked(8, 8, 2048, 11008, 4096, T) == (256, 128, 64, 64, 4)       # 344 tiles of 256x256 would be two rounds
+    # group scales (the decoder-layer linears): 128x128 once it fills the chip, 128x64 below
+    assert picked(8, 2, 1024, 12288, 4096, T, group=128) == (128, 128, 64, 64, 4)
+    assert picked(8, 2, 1024, 4096, 4096, T, group=128) == (128, 64, 64, 32, 4)
+    assert picked(8, 2, 16384, 22016, 4096, T, group=128) == (128, 128, 64, 64, 4)
+    assert picked(8, 2, 128, 4096, 4096, T, group=64) == (64, 64, 32, 32, 4)
