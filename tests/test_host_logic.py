@@ -332,7 +332,7 @@ def test_gen_kernel_native_space_is_what_the_library_instantiates(gen_kernel, ab
 
 def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     """The tile the library picks for prepared operands, pinned on shapes of BASELINE.json configs[2] and
-    configs[4] and on a few where the sweep in profiles/prefill_tile_sweep.md separates the tiles clearly:
+    configs[4] and on a few where the measured sweep of all tiles separates them clearly:
     large tiles only where their quantised grids pay, 128x128 in between, small tiles for small grids."""
     lib = abq.lib()
 
