@@ -678,9 +678,9 @@ static int large_tiles_int8(int x_bits, int w_bits, int is_signed, const LargeTi
     return 0;
 }
 
-// Picks the tiled-kernel tile for a shape.  Measured on MI355X (W4A4 / W8A8 / W2A8, LLaMA shapes):
-// the 256x128 tile of eight waves (least L2 -> L1 traffic per MFMA) is the fastest once it yields
-// one workgroup per compute unit, then 128x128; below that, smaller tiles win by filling the chip.
+// Picks the tiled-kernel tile for a shape.  Pairs with a cost model (large_tiles_int8) weigh their large
+// tiles against 128x128 once the shape has 200 tiles of 128x128; everything else goes by the thresholds
+// below (measured on MI355X, LLaMA shapes): smaller tiles win by filling the chip.
 static abq_status switch_to_tiled(abq_gemm_state *st)
 {
     const Registry &reg = registry();
@@ -689,12 +689,12 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
     if (!tt)
         return ABQ_ERR_UNSUPPORTED;
     // candidates in order of preference: { TM, TN, waves along M, waves along N, workgroups needed }
-    // (the 256x256 tile of eight 64x128 waves halves the L2 -> L1 traffic again; it pays only for the widest
-    // operands, W8A8, and only on grids of several workgroups per compute unit)
+    // (pairs without a cost model: the 256x256 tile of eight 64x128 waves only for operands of 16 bits together,
+    // on grids of several workgroups per compute unit)
     static const int order[][5] = { { 2, 4, 4, 2, 600 }, { 2, 2, 4, 2, 250 }, { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 400 },
                                     { 1, 1, 2, 2, 0 } };
-    // signed 8-bit pairs run the 256x128 tile on the staged kernel, which is bound by the rate L2 delivers the
-    // tiles: the large tile pays as soon as it covers about two thirds of the compute units
+    // signed W8A8 below 200 tiles of 128x128: the staged kernel's 256x128 tile pays as soon as it covers about two
+    // thirds of the compute units
     const bool staged = c.x_bits == 8 && c.w_bits == 8 && c.is_signed;
     int pick = -1;
     const LargeTile *cands = nullptr;
