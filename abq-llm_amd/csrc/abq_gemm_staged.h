@@ -418,6 +418,21 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         }
         return;
     }
+    if (a.out_kind == 1 || a.out_kind == 3) {
+        // one fp16 scale for the whole output, half(acc) * scale with both steps rounding to fp16 (the arithmetic of
+        // store_result; fastertransformer/.../abqgemm/mma_any/aq_bmma_kernel.h:516-519 of the reference): through LDS
+        // as whole lines where the output allows it
+        _Float16 *out = reinterpret_cast<_Float16 *>(a.D);
+        using WT = WaveTileF16<TM, TN>;
+        if (WM * WN * WT::kBytes <= S * BUF_BYTES && store_wave_tile_f16_ok(out, N, N)) {
+            const _Float16 scale = a.out_kind == 1 ? *reinterpret_cast<const _Float16 *>(a.C)
+                                                   : (_Float16) * reinterpret_cast<const float *>(a.C);
+            __syncthreads(); // every wave's loads have landed and its fragment reads are done: the stages are free
+            store_wave_tile_f16<TM, TN>(out, N, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, smem + wid * WT::kBytes, lane,
+                                        [&](int i, int j, int e) { return (float)((_Float16)(float)result(i, j, e) * scale); });
+            return;
+        }
+    }
     const StoreOperands so = store_operands(a);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {

@@ -394,30 +394,60 @@ void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, i
     }
 
     const int k_fed = ktiles * KB;
+    auto result = [&](int i, int j, int e) -> int {
+        unsigned v = (unsigned)acc[i][j][e];
+        if (SIGNED) {
+            v = (unsigned)((int)v >> (16 - Q - P));
+        } else {
+            if (NEED_SX)
+                v += 128u * (unsigned)rowsum[wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4)];
+            if (NEED_SW)
+                v += 128u * (unsigned)rowsum[BM + wn * 32 * TN + j * 32 + r];
+            if (NEED_SX && NEED_SW)
+                v -= 16384u * (unsigned)k_fed;
+        }
+        return (int)v;
+    };
+    // fp16 outputs leave through LDS as whole lines where the output allows it (abq_group_epilogue.h); same
+    // arithmetic as store_result
+    using WT = WaveTileF16<TM, TN>;
+    if (a.out_kind != 0 && WM * WN * WT::kBytes <= 2 * BUF_BYTES &&
+        store_wave_tile_f16_ok(a.D, N, N)) {
+        _Float16 *out = reinterpret_cast<_Float16 *>(a.D);
+        unsigned char *region = smem + wid * WT::kBytes;
+        if (a.out_kind == 2) {
+            float wsv[TN], xsv[TM][16];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                wsv[j] = a.w_scale[min(n0 + wn * 32 * TN + j * 32 + r, N - 1)];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    xsv[i][e] = a.x_scale[min(m0 + wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4), M - 1)];
+            __syncthreads(); // the tile buffers are free: the last K tile is behind every wave
+            store_wave_tile_f16<TM, TN>(out, N, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, region, lane,
+                                        [&](int i, int j, int e) { return (float)result(i, j, e) * xsv[i][e] * wsv[j]; });
+        } else {
+            const _Float16 scale = a.out_kind == 1 ? *reinterpret_cast<const _Float16 *>(a.C)
+                                                   : (_Float16) * reinterpret_cast<const float *>(a.C);
+            __syncthreads();
+            store_wave_tile_f16<TM, TN>(out, N, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, region, lane,
+                                        [&](int i, int j, int e) { return (float)((_Float16)(float)result(i, j, e) * scale); });
+        }
+        return;
+    }
     const StoreOperands so = store_operands(a);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const int nl = wn * 32 * TN + j * 32 + r;
-            const int n = n0 + nl;
+            const int n = n0 + wn * 32 * TN + j * 32 + r;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int ml = wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4);
-                const int m = m0 + ml;
-                unsigned v = (unsigned)acc[i][j][e];
-                if (SIGNED) {
-                    v = (unsigned)((int)v >> (16 - Q - P));
-                } else {
-                    if (NEED_SX)
-                        v += 128u * (unsigned)rowsum[ml];
-                    if (NEED_SW)
-                        v += 128u * (unsigned)rowsum[BM + nl];
-                    if (NEED_SX && NEED_SW)
-                        v -= 16384u * (unsigned)k_fed;
-                }
+                const int m = m0 + wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4);
                 if (m < M && n < N)
-                    store_result_compact(so, m, n, (int)v);
+                    store_result_compact(so, m, n, result(i, j, e));
             }
         }
     }

@@ -277,29 +277,36 @@ def test_fp6_fp16_epilogues(abq, oracle):
     assert np.array_equal(got.view(np.uint16), want16.view(np.uint16))
 
 
-@pytest.mark.parametrize("q,p,fp6", [(4, 4, True), (8, 2, False), (4, 4, False), (8, 8, False), (2, 2, False)])
-def test_scaled_fp16_epilogue_every_staged_tile(abq, oracle, q, p, fp6):
+@pytest.mark.parametrize("q,p,fp6,signed", [(4, 4, True, True), (8, 2, False, True), (4, 4, False, True), (8, 8, False, True),
+                                             (2, 2, False, True), (6, 6, False, True), (8, 8, False, False), (4, 4, True, False)])
+def test_scaled_fp16_epilogue_every_staged_tile(abq, oracle, q, p, fp6, signed):
     """Per-token x per-channel scales with fp16 output on every tile of the LDS-staged kernels: once with
     an output width the whole-line store takes (multiple of 8) and once with one it does not, ragged M."""
-    rng = np.random.default_rng(900 + 10 * q + p + fp6)
-    tiles = [c for c in abq.native_configs(q, p, True) if c.nstage == (5 if fp6 else 4) and c.warp_k == 128]
+    rng = np.random.default_rng(900 + 10 * q + p + fp6 + 2 * signed)
+    tiles = [c for c in abq.native_configs(q, p, signed) if c.nstage == (5 if fp6 else 4) and c.warp_k == 128]
     assert tiles
     for (M, N, K) in [(130, 328, 384), (70, 203, 256)]:
-        x, w = rand_vals(rng, M, K, q, True), rand_vals(rng, N, K, p, True)
+        x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
         xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
         if fp6:
-            xo, wo, kw = abq.relayout_planes_fp6(xd, True), abq.relayout_planes_fp6(wd, True), dict(x_fp6=q, w_fp6=p)
+            xo, wo, kw = abq.relayout_planes_fp6(xd, signed), abq.relayout_planes_fp6(wd, signed), dict(x_fp6=q, w_fp6=p)
         else:
             xo, wo, kw = abq.relayout_planes(xd), abq.relayout_planes(wd), dict(x_tiled=True, w_tiled=True)
         xs = torch.rand(M, device="cuda") * 0.01 + 0.001
         ws = torch.rand(N, device="cuda") * 0.01 + 0.001
         want = (oracle.np_gemm(x, w).astype(np.float64) * xs.cpu().numpy().astype(np.float64)[:, None]
                 * ws.cpu().numpy().astype(np.float64)[None, :])
+        c16 = torch.tensor([0.03125], dtype=torch.float16, device="cuda")
+        with np.errstate(over="ignore"):  # beyond fp16's range both sides give infinity
+            want16 = (oracle.np_gemm(x, w).astype(np.float32).astype(np.float16) * np.float16(0.03125)).astype(np.float16)
         for cfg in tiles:
-            g = abq.Gemm(xo, wo, True, cfg=cfg, out_kind=abq.OUT_F16_SCALED, x_scale=xs, w_scale=ws, **kw)
+            g = abq.Gemm(xo, wo, signed, cfg=cfg, out_kind=abq.OUT_F16_SCALED, x_scale=xs, w_scale=ws, **kw)
             got = g.run().float().cpu().numpy()
             # tolerance of the fp16 dequantised output: 1e-2 relative
             assert np.all(np.abs(got - want) <= 1e-2 * np.abs(want) + 1e-6), (g.config_name, M, N, K)
+            # one fp16 scale for the whole output: half(acc) * scale, bit for bit
+            got16 = abq.Gemm(xo, wo, signed, cfg=cfg, out_kind=abq.OUT_F16_TENSOR, c_scale=c16, **kw).run().cpu().numpy()
+            assert np.array_equal(got16.view(np.uint16), want16.view(np.uint16)), (g.config_name, M, N, K)
 
 
 @pytest.mark.parametrize("signed", [True, False])
