@@ -17,6 +17,7 @@ hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream
 hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes_fp6(const uint32_t *, uint32_t *, int, int, int, int, hipStream_t);
 const KernelEntry *fp6_entries(int *count);
+const KernelEntry *fp6_grouped_entries(int *count);
 hipError_t launch_quant_pack_rows(const void *, uint32_t *, float *, float *, int *, int, int, int, int, int, int,
                                   hipStream_t);
 hipError_t launch_weight_zero_term(const uint32_t *, int, int, int, int, const float *, const float *, int, float *,
@@ -731,8 +732,36 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
 static abq_status switch_to_fp6(abq_gemm_state *st)
 {
     const abq_tile_config &c = st->cfg;
-    if (!fp6_eligible(c.x_bits, c.w_bits, c.is_signed, st->K) || st->group_size)
+    if (!fp6_eligible(c.x_bits, c.w_bits, c.is_signed, st->K))
         return ABQ_ERR_UNSUPPORTED;
+    if (st->group_size) {
+        // group scales: one scale per K tile, i.e. groups of 128; tiles as for the int8 group-scale kernels
+        // (128x128 once it fills the chip, else 128x64, the smallest tile with two MFMA tiles per wave)
+        if (st->group_size != 128)
+            return ABQ_ERR_UNSUPPORTED;
+        int gcount = 0;
+        const KernelEntry *ge = fp6_grouped_entries(&gcount);
+        const long t128 = (long)((st->M + 127) / 128) * ((st->N + 127) / 128);
+        int gpick = -1;
+        for (int i = 0; i < gcount; ++i) {
+            const int bm = 32 * ge[i].tm * ge[i].wm, bn = 32 * ge[i].tn * ge[i].wn;
+            if (!st->auto_chosen ? (bm == c.block_m && bn == c.block_n && 32 * ge[i].tm == c.warp_m)
+                                 : ((t128 >= 300 && bm == 128 && bn == 128) || (t128 < 300 && bm == 128 && bn == 64)))
+                gpick = i;
+        }
+        if (gpick < 0)
+            return ABQ_ERR_UNSUPPORTED;
+        const KernelEntry &e = ge[gpick];
+        const int bm = 32 * e.tm * e.wm, bn = 32 * e.tn * e.wn;
+        const int xb_ = c.x_bits, wb_ = c.w_bits, sg_ = c.is_signed;
+        entry_to_config(e, ABQ_STRATEGY_FP6, xb_, wb_, sg_, 0, &st->cfg);
+        st->strategy = ABQ_STRATEGY_FP6;
+        st->variant = gpick;
+        st->grid_dim = abq_dim3{ (unsigned)(8 * (((st->N + bn - 1) / bn + 7) / 8) * ((st->M + bm - 1) / bm)), 1, 1 };
+        st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
+        st->shared_mem_size = e.lds;
+        return ABQ_OK;
+    }
     int count = 0;
     const KernelEntry *es = fp6_entries(&count);
     // The 256x128 tile of eight waves against 128x128 by the cost model above (it pays over several rounds
@@ -767,8 +796,8 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
 // Moves a state with group scales onto the tiled kernel's group-scale variants.
 static abq_status pick_grouped_tiled(abq_gemm_state *state)
 {
-    if (state->x_layout == ABQ_LAYOUT_FP6 || state->w_layout == ABQ_LAYOUT_FP6)
-        return ABQ_ERR_UNSUPPORTED; // group scales are folded by the int8 kernels only
+    if (state->x_layout == ABQ_LAYOUT_FP6 || state->w_layout == ABQ_LAYOUT_FP6 || state->strategy == ABQ_STRATEGY_FP6)
+        return switch_to_fp6(state); // the FP6 kernel's group-scale variants
     if (state->strategy != ABQ_STRATEGY_TILED) {
         if (!state->auto_chosen)
             return ABQ_ERR_UNSUPPORTED;
@@ -966,7 +995,7 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
         // operands still in the reference layout are converted into the caller's workspace
         const size_t xb = st->x_layout == ABQ_LAYOUT_FP6 ? 0 : fp6_bytes(st->M, st->K);
         const size_t wb = st->w_layout == ABQ_LAYOUT_FP6 ? 0 : fp6_bytes(st->N, st->K);
-        if (st->group_size || st->x_layout == ABQ_LAYOUT_TILED || st->w_layout == ABQ_LAYOUT_TILED)
+        if (st->x_layout == ABQ_LAYOUT_TILED || st->w_layout == ABQ_LAYOUT_TILED)
             return ABQ_ERR_NOT_INITIALIZED;
         if (xb + wb > st->workspace_bytes || ((xb + wb) && !st->workspace))
             return ABQ_ERR_INVALID_ARG;
@@ -986,7 +1015,7 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
             a.W = reinterpret_cast<const uint32_t *>(ws + xb);
         }
         int count = 0;
-        const KernelEntry *es = fp6_entries(&count);
+        const KernelEntry *es = st->group_size ? fp6_grouped_entries(&count) : fp6_entries(&count);
         if (st->variant < 0 || st->variant >= count)
             return ABQ_ERR_NOT_INITIALIZED;
         e = es[st->variant].launch(a, (hipStream_t)stream);
@@ -1090,7 +1119,7 @@ abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_l
     if (any_fp6 && any_tiled)
         return ABQ_ERR_UNSUPPORTED;
     if (any_fp6 && st->strategy != ABQ_STRATEGY_FP6) {
-        if (!st->auto_chosen || st->group_size)
+        if (!st->auto_chosen)
             return ABQ_ERR_UNSUPPORTED;
         const abq_status rc = switch_to_fp6(st);
         if (rc != ABQ_OK)

@@ -38,4 +38,17 @@ const KernelEntry *fp6_entries(int *count)
     return kFp6Entries;
 }
 
+// The same tiles with group scales (groups of 128), where a wave has at least two MFMA tiles.
+#define ABQ_FP6_GROUPED_VARIANTS(V) V(2, 2, 4, 2) V(2, 2, 2, 2) V(2, 1, 2, 2)
+#define ABQ_FP6_GENTRY(TM, TN, WM, WN)                                                                   \
+    { 32, TM, TN, WM, WN, 1, 5, &launch_mfma_staged<6, 6, true, true, TM, TN, WM, WN, true>, 128,        \
+      StagedStages<6, 6, true, TM, TN, WM, WN, true>::kLds },
+static const KernelEntry kFp6GroupedEntries[] = { ABQ_FP6_GROUPED_VARIANTS(ABQ_FP6_GENTRY) };
+
+const KernelEntry *fp6_grouped_entries(int *count)
+{
+    *count = (int)(sizeof(kFp6GroupedEntries) / sizeof(kFp6GroupedEntries[0]));
+    return kFp6GroupedEntries;
+}
+
 } // namespace abq

@@ -117,7 +117,8 @@ __device__ __forceinline__ void staged_load_dword_to_lds(const float *src, unsig
 // QB / PB: bits of the activation / weight fields (2, 4 or 8; ignored for FP6).
 //
 // GROUPED: group-wise weight scales (one per 128 elements along K, i.e. per K tile: w_scale[N][K / 128]),
-// per-token activation scales, optional zero points and SiLU gate, fp16 output (see abq_group_epilogue.h).
+// per-token activation scales, optional zero points and SiLU gate, fp16 output (see abq_group_epilogue.h);
+// integer fields and FP6 records alike (an FP6 tile is already fp32, its fold is one multiply-add).
 // A tile's BN scales travel with its records: one more wave load or two of four bytes per lane into the
 // tile's LDS stage, so they are covered by the same load counter and barrier as the records.  The int32
 // accumulators cover one K tile; the MFMAs run tile by tile of the wave's TM x TN (four K steps in a
@@ -139,7 +140,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     constexpr int NI = NIA + BN * TB::kUnits / 64;             // ... and in all
     constexpr int NPR = (NI + NW - 1) / NW;                    // per wave
     constexpr int NPW = NPR + (GROUPED ? 1 : 0);               // GROUPED: and one load of 64 scales (256 bytes)
-    static_assert(!GROUPED || (!FP6 && TM * TN >= 2 && BN / 64 <= WM * WN), "group scales: integer fields, two MFMA tiles per wave or more");
+    static_assert(!GROUPED || (TM * TN >= 2 && BN / 64 <= WM * WN), "group scales: two MFMA tiles per wave or more");
     constexpr int kSteps = FP6 ? 2 : 4;                        // MFMA K steps per tile of 128
     static_assert(FP6 || SIGNED || (QB < 8 && PB < 8), "unsigned 8-bit operands are not handled here");
     static_assert(S >= 3 && S <= 4, "three or four LDS stages");
@@ -224,6 +225,10 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     };
     auto mfma = [&](Acc &c, const v4i(&q)[NR], int i, int j, int ks, bool fresh = false) {
         const v4i *pa = &q[i * TA::kReads], *pb = &q[NRA + j * TB::kReads];
+        Acc zero;
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            zero[e] = 0;
         if constexpr (FP6) {
             // dwords 0-5 of the 12 a lane holds are the first K step's operand, 6-11 the second's (the two
             // upper dwords of the 8-dword operand are not read for 6-bit formats)
@@ -231,12 +236,8 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
                                    : __builtin_shufflevector(pa[1], pa[2], 2, 3, 4, 5, 6, 7, -1, -1);
             const v8i bv = ks == 0 ? __builtin_shufflevector(pb[0], pb[1], 0, 1, 2, 3, 4, 5, -1, -1)
                                    : __builtin_shufflevector(pb[1], pb[2], 2, 3, 4, 5, 6, 7, -1, -1);
-            c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 2, 2, 0, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, fresh ? zero : c, 2, 2, 0, 0, 0, 0);
         } else {
-            Acc zero;
-#pragma unroll
-            for (int e = 0; e < 16; ++e)
-                zero[e] = 0;
             c = __builtin_amdgcn_mfma_i32_32x32x32_i8(staged_int8_operand<QB, SIGNED>(pa, ks),
                                                       staged_int8_operand<PB, SIGNED>(pb, ks), fresh ? zero : c, 0, 0, 0);
         }
@@ -272,7 +273,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     // value * 2^(8-bits) to the MFMA: the exact power of two that undoes it rides on the scale.
     v16f facc[GROUPED ? TM : 1][GROUPED ? TN : 1];
     float sc_cur[TN], sc_next[TN], sc_last = 0.f;
-    const float unshift = SIGNED ? 1.0f / (float)(1 << (16 - QB - PB)) : 1.0f;
+    const float unshift = FP6 ? 64.0f : SIGNED ? 1.0f / (float)(1 << (16 - QB - PB)) : 1.0f; // FP6: both operands carry 1/8 as their unit
     auto read_scales = [&](float(&sc)[TN], int stage) {
 #pragma unroll
         for (int j = 0; j < TN; ++j)
@@ -314,9 +315,9 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         __syncthreads();                                                                                        \
     }
 
-    // The same with group scales.  MFMA step k works on MFMA tile u = k / 4 of the wave's TM x TN (K step
-    // k % 4, the first one starting from zero); beside it the vector ALU folds a quarter of the tile
-    // finished before u: tile u - 1 of this K tile, or for u = 0 the last tile of the previous K tile (all
+    // The same with group scales.  MFMA step k works on MFMA tile u = k / kSteps of the wave's TM x TN (K
+    // step k % kSteps, the first one starting from zero); beside it the vector ALU folds its share (a
+    // quarter, or half for FP6) of the tile finished before u: tile u - 1 of this K tile, or for u = 0 the last tile of the previous K tile (all
     // zeros, with a zero scale, when there is none).
 #define ABQ_STAGED_K_TILE_G(KT, QC, QN)                                                                         \
     {                                                                                                           \
@@ -324,14 +325,14 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         read_scales(sc_next, st_rd);                                                                            \
         _Pragma("unroll") for (int k = 0; k < NM; ++k)                                                          \
         {                                                                                                       \
-            const int u = k / 4, ks = k % 4, uf = (u + NU - 1) % NU;                                            \
+            const int u = k / kSteps, ks = k % kSteps, uf = (u + NU - 1) % NU;                                  \
             mfma(acc[u / TN][u % TN], QC, u / TN, u % TN, ks, ks == 0);                                         \
             _Pragma("unroll") for (int d = k * NPW / NM; d < (k + 1) * NPW / NM; ++d)                           \
                 request((KT) + S, st_req, d);                                                                   \
             _Pragma("unroll") for (int p = k * NR / NM; p < (k + 1) * NR / NM; ++p)                             \
                 read_piece(QN, st_rd, p);                                                                       \
             const float scf = u == 0 ? sc_last : sc_cur[uf % TN];                                               \
-            _Pragma("unroll") for (int e = 4 * ks; e < 4 * ks + 4; ++e)                                         \
+            _Pragma("unroll") for (int e = (16 / kSteps) * ks; e < (16 / kSteps) * (ks + 1); ++e)               \
                 facc[uf / TN][uf % TN][e] += (float)acc[uf / TN][uf % TN][e] * scf;                             \
             __builtin_amdgcn_sched_barrier(0);                                                                  \
         }                                                                                                       \

@@ -290,8 +290,8 @@ abq_status abq_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int ro
 /* Declares the layout of X and W of an initialised state.  A tiled (FP6) operand moves a state
  * whose tile was the library's choice to ABQ_STRATEGY_TILED (ABQ_STRATEGY_FP6); a state
  * initialised with an explicit tile tuple of another strategy is refused (ABQ_ERR_UNSUPPORTED),
- * and so are a tiled and an FP6 operand together, an FP6 operand with group scales, and an FP6
- * operand of a bit pair or K that does not qualify. */
+ * and so are a tiled and an FP6 operand together, an FP6 operand with group scales of groups other
+ * than 128, and an FP6 operand of a bit pair or K that does not qualify. */
 abq_status abq_gemm_set_operand_layout(abq_gemm_state *state, int x_layout, int w_layout);
 
 /* Workspace needed by abq_gemm_exec if the state ran as ABQ_STRATEGY_TILED (ABQ_STRATEGY_FP6)

@@ -255,8 +255,8 @@ def test_fp6_gemm_range_ends_and_limits(abq, oracle):
     with pytest.raises(abq.AbqError):
         abq.Gemm(abq.relayout_planes(x4d), wf, True, x_tiled=True, w_fp6=2)  # tiled and FP6 together
     sc = torch.ones(64 * 2, dtype=torch.float32, device="cuda")
-    with pytest.raises(abq.AbqError):
-        abq.Gemm(x4d, wf, True, w_fp6=2, out_kind=abq.OUT_F16_SCALED, x_scale=sc, w_scale=sc, group_size=128)
+    with pytest.raises(abq.AbqError):  # group scales on the FP6 route: groups of 128 only
+        abq.Gemm(x4d, wf, True, w_fp6=2, out_kind=abq.OUT_F16_SCALED, x_scale=sc, w_scale=sc, group_size=64)
 
 
 def test_fp6_fp16_epilogues(abq, oracle):

@@ -271,6 +271,47 @@ def test_group_scale_staged_kernel_every_tile(abq, oracle, q, p, signed):
             torch.cuda.synchronize()
             assert_close_rel(got.cpu().numpy(), want)
 
+@pytest.mark.parametrize("q,p,signed", [(4, 4, True), (4, 4, False), (5, 5, True), (4, 2, True), (3, 3, False)])
+def test_group_scales_on_the_fp6_route(abq, oracle, q, p, signed):
+    """Groups of 128 with zero points on both sides through the FP6 matrix-core kernel: the library's own
+    tile choice and every tile it is built for, operands as FP6 records or converted from planes."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(300 + 10 * q + p + signed)
+    tiles = [None] + [c for c in abq.native_configs(q, p, signed)
+                      if c.nstage == 5 and (c.block_m, c.block_n, c.warp_m) in ((256, 128, 64), (128, 128, 64), (128, 64, 64))]
+    assert len(tiles) == 4
+    lo_x, hi_x = (-(1 << (q - 1)), 1 << (q - 1)) if signed else (0, 1 << q)
+    lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed else (0, 1 << p)
+    for (M, N, K) in [(300, 200, 640), (70, 330, 256), (129, 72, 128)]:
+        G = K // 128
+        x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        xs = rng.uniform(0.01, 0.05, M)
+        xz = rng.integers(lo_x // 2, hi_x // 2 + 1, M).astype(np.float64)
+        wsc = rng.uniform(0.001, 0.02, (N, G))
+        wz = rng.integers(lo_w, hi_w, (N, G)).astype(np.float64)
+        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, 128)
+        xp, wp = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
+        kw = dict(x_scale=fdev(xs), w_scale=fdev(wsc), group_size=128, w_zero=fdev(wz), x_zero=fdev(xz),
+                  x_group_sums=torch.from_numpy(x.reshape(M, G, 128).sum(axis=2).astype(np.int32)).cuda())
+        kw["w_zero_term"] = abq.weight_zero_term(wp, signed, kw["w_scale"], kw["w_zero"], 128)
+        xf, wf = abq.relayout_planes_fp6(xp, signed), abq.relayout_planes_fp6(wp, signed)
+        for cfg in tiles:
+            g = abq.Gemm(xf, wf, signed, cfg=cfg, out_kind=abq.OUT_F16_SCALED, x_fp6=q, w_fp6=p, **kw)
+            assert g.strategy == "fp6" and g.state.group_size == 128
+            got = g.run()
+            torch.cuda.synchronize()
+            assert_close_rel(got.cpu().numpy(), want)
+        # activations still as planes: converted into the caller's workspace inside the call
+        ws = torch.empty((K // 128) * M * 96, dtype=torch.uint8, device="cuda")
+        g = abq.Gemm(xp, wf, signed, out_kind=abq.OUT_F16_SCALED, w_fp6=p, workspace=ws, **kw)
+        assert g.strategy == "fp6"
+        assert_close_rel(g.run().cpu().numpy(), want)
+    # groups of 64 have no FP6 build
+    with pytest.raises(abq.AbqError):
+        abq.Gemm(xf, wf, signed, out_kind=abq.OUT_F16_SCALED, x_fp6=q, w_fp6=p, x_scale=kw["x_scale"],
+                 w_scale=fdev(rng.uniform(0.001, 0.02, (N, 2 * G))), group_size=64)
+
 
 # ------------------------------------------------------------------ BASELINE.json configs[4]
 
