@@ -85,8 +85,14 @@ void ABQGEMMWrapper::gemm_scaled(const int M, const int N, const int K, const in
 // workspace: activation planes | scale[M] | zero[M] | group sums [M][K/group_size]
 size_t ABQGEMMWrapper::dynamic_workspace_bytes(int M, int K, int group_size) const
 {
-    const size_t planes = ((size_t)x_bits_ * M * K / 8 + 255) / 256 * 256;
-    return planes + (size_t)M * 8 + (size_t)M * (K / group_size) * 4;
+    return activation_bytes(M, K) + (size_t)M * 8 + (size_t)M * (K / group_size) * 4;
+}
+
+// packed activations of a call: x_bits per element, or 6 where they may be written as FP6 records
+size_t ABQGEMMWrapper::activation_bytes(int M, int K) const
+{
+    const int bits = abq_fp6_eligible(x_bits_, w_bits_, signed_ ? 1 : 0, K) ? 6 : x_bits_;
+    return ((size_t)bits * M * K / 8 + 255) / 256 * 256;
 }
 
 void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _Float16 *A, const ABQGroupedWeight &W,
@@ -105,7 +111,7 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
         printf("[ABQ][Error] workspace too small: %zu bytes for M,K,bits = %d,%d,%d\n", abq_gemm_ws_bytes, M, K, x_bits_);
         return;
     }
-    const size_t planes_bytes = ((size_t)x_bits_ * M * K / 8 + 255) / 256 * 256;
+    const size_t planes_bytes = activation_bytes(M, K);
     uint32_t *planes = reinterpret_cast<uint32_t *>(abq_gemm_workspace);
     float *x_scale = reinterpret_cast<float *>(abq_gemm_workspace + planes_bytes);
     float *x_zero = x_scale + M;
@@ -114,7 +120,8 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     // (if the expanded activations fit the decode kernel's LDS: partial tiles, group sums, M padded rows)
     const bool decode = M <= 16 && W.planes != nullptr &&
                         (silu_gate ? 32 : 16) * 1024 + (size_t)64 * (K / W.group_size) + 128 + (size_t)M * ((K + 511) / 512 * 512 + 16) <= 160 * 1024;
-    const int layout = decode ? ABQ_LAYOUT_PLANES : ABQ_LAYOUT_TILED;
+    const bool fp6 = !decode && W.records_fp6 != nullptr && W.group_size == 128 && abq_fp6_eligible(x_bits_, w_bits_, 1, K);
+    const int layout = decode ? ABQ_LAYOUT_PLANES : fp6 ? ABQ_LAYOUT_FP6 : ABQ_LAYOUT_TILED;
     abq_status rc = abq_quant_pack_f16(A, M, K, x_bits_, x_symmetric ? 1 : 0, layout, planes, x_scale, x_zero,
                                        sums, W.group_size, stream);
     if (rc != ABQ_OK) {
@@ -123,10 +130,10 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     }
     abq_gemm_state state;
     rc = abq_gemm_init(nullptr, x_bits_, w_bits_, 1, planes,
-                       reinterpret_cast<const uint32_t *>(decode ? W.planes : W.planes_tiled), M, N, K, D, nullptr, 0,
-                       ABQ_OUT_F16_SCALED, &state);
+                       reinterpret_cast<const uint32_t *>(decode ? W.planes : fp6 ? W.records_fp6 : W.planes_tiled), M, N, K,
+                       D, nullptr, 0, ABQ_OUT_F16_SCALED, &state);
     if (rc == ABQ_OK && !decode)
-        rc = abq_gemm_set_operand_layout(&state, ABQ_LAYOUT_TILED, ABQ_LAYOUT_TILED);
+        rc = abq_gemm_set_operand_layout(&state, layout, layout);
     if (rc == ABQ_OK)
         rc = abq_gemm_set_scales(&state, x_scale, W.scale, W.group_size);
     if (rc == ABQ_OK && (W.zero || !x_symmetric))

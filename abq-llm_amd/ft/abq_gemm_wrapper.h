@@ -28,6 +28,9 @@ struct ABQGroupedWeight {
     int group_size;           // 64 or 128
     const int *planes;        // the same weights in the reference plane layout [w_bits][N][K/32], or nullptr;
                               // with it, calls of at most 16 rows run the decode kernel
+    const int *records_fp6;   // the same weights as FP6 records (abq_relayout_planes_fp6), or nullptr; with it,
+                              // groups of 128 and a bit pair that qualifies (abq_fp6_eligible, e.g. W4A4), calls of
+                              // more than 16 rows run on the FP6 matrix cores
 };
 
 class ABQGEMMWrapper {
@@ -63,4 +66,6 @@ public:
                       _Float16 *D, bool x_symmetric, char *abq_gemm_workspace, size_t abq_gemm_ws_bytes,
                       hipStream_t stream, bool silu_gate = false);
     size_t dynamic_workspace_bytes(int M, int K, int group_size) const;
+    // the packed activations' share of it (x_bits per element; 6 where the bit pair qualifies for FP6 records)
+    size_t activation_bytes(int M, int K) const;
 };

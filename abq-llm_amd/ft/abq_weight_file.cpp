@@ -180,10 +180,10 @@ ABQDeviceWeight::~ABQDeviceWeight() { release(); }
 
 void ABQDeviceWeight::release()
 {
-    for (void *p : { (void *)planes_, (void *)tiled_, (void *)scale_, (void *)zero_, (void *)zero_term_ })
+    for (void *p : { (void *)planes_, (void *)tiled_, (void *)fp6_, (void *)scale_, (void *)zero_, (void *)zero_term_ })
         if (p)
             (void)hipFree(p);
-    planes_ = tiled_ = nullptr;
+    planes_ = tiled_ = fp6_ = nullptr;
     scale_ = zero_ = zero_term_ = nullptr;
 }
 
@@ -214,6 +214,12 @@ bool ABQDeviceWeight::load(const ABQWeightBlob &blob, hipStream_t stream, std::s
     if (rc == ABQ_OK && (info_.group_size == 64 || info_.group_size == 128))
         rc = abq_weight_zero_term(planes_, (int)info_.n, (int)info_.k, (int)info_.bits, (int)info_.is_signed, scale_, zero_,
                                   (int)info_.group_size, zero_term_, stream);
+    // FP6 records for the FP6 matrix-core route (groups of 128; codes of magnitude at most 16)
+    if (rc == ABQ_OK && info_.group_size == 128 && info_.bits <= (info_.is_signed ? 5u : 4u)) {
+        if (!hip_ok(hipMalloc(&fp6_, abq_fp6_bytes((int)info_.n, (int)info_.k)), "hipMalloc fp6"))
+            return false;
+        rc = abq_relayout_planes_fp6(planes_, fp6_, (int)info_.n, (int)info_.k, (int)info_.bits, (int)info_.is_signed, stream);
+    }
     if (rc != ABQ_OK)
         return fail(error, std::string("weight preparation failed: ") + abq_status_string(rc));
     return hip_ok(hipStreamSynchronize(stream), "synchronise");
@@ -222,5 +228,5 @@ bool ABQDeviceWeight::load(const ABQWeightBlob &blob, hipStream_t stream, std::s
 ABQGroupedWeight ABQDeviceWeight::grouped() const
 {
     return ABQGroupedWeight{ reinterpret_cast<const int *>(tiled_), scale_, zero_, zero_term_, (int)info_.group_size,
-                             reinterpret_cast<const int *>(planes_) };
+                             reinterpret_cast<const int *>(planes_), reinterpret_cast<const int *>(fp6_) };
 }

@@ -83,6 +83,6 @@ public:
 
 private:
     ABQWeightHeader info_{};
-    uint32_t *planes_ = nullptr, *tiled_ = nullptr;
+    uint32_t *planes_ = nullptr, *tiled_ = nullptr, *fp6_ = nullptr; // fp6_: only for groups of 128 and at most 5 (4 unsigned) bits
     float *scale_ = nullptr, *zero_ = nullptr, *zero_term_ = nullptr;
 };

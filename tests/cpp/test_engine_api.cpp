@@ -377,6 +377,62 @@ static void gpu_paths()
         HIP_OK(hipFree(d_ws));
     }
 
+    {   // W4A4 with groups of 128: a loaded weight also carries FP6 records, and calls of more than 16 rows run
+        // on the FP6 matrix cores; same output as the int8 route (the integer tiles are exact on both and
+        // are folded in the same order)
+        const int M = 40, N = 192, K = 512, G = 128;
+        std::mt19937 r32(23);
+        std::normal_distribution<float> nd(0.f, 0.05f), xd_(0.f, 1.f);
+        std::vector<float> wf((size_t)N * K);
+        for (auto &v : wf)
+            v = nd(r32);
+        ABQWeightBlob blob;
+        std::string err;
+        CHECK(abq_quantize_weights(wf.data(), N, K, 4, false, G, &blob, &err));
+        ABQDeviceWeight dw;
+        CHECK(dw.load(blob, stream, &err));
+        ABQGroupedWeight with_fp6 = dw.grouped(), without = dw.grouped();
+        CHECK(with_fp6.records_fp6 != nullptr);
+        without.records_fp6 = nullptr;
+        std::vector<uint16_t> ha((size_t)M * K);
+        for (auto &h : ha)
+            h = abq_oracle_f32_to_f16(xd_(r32));
+        ABQGEMMWrapper wrap(4, 4, true);
+        const size_t ws_bytes = wrap.dynamic_workspace_bytes(M, K, G);
+        CHECK(wrap.activation_bytes(M, K) >= (size_t)M * K * 6 / 8);
+        _Float16 *d_a, *d_d;
+        char *d_ws;
+        HIP_OK(hipMalloc(&d_a, ha.size() * 2));
+        HIP_OK(hipMalloc(&d_d, (size_t)M * N * 2));
+        HIP_OK(hipMalloc(&d_ws, ws_bytes));
+        HIP_OK(hipMemcpy(d_a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
+        std::vector<uint16_t> got_fp6((size_t)M * N), got_int8((size_t)M * N);
+        for (int symmetric = 1; symmetric >= 0; --symmetric) {
+            HIP_OK(hipMemset(d_d, 0, (size_t)M * N * 2));
+            wrap.gemm_dynamic(M, N, K, d_a, with_fp6, d_d, symmetric != 0, d_ws, ws_bytes, stream);
+            HIP_OK(hipStreamSynchronize(stream));
+            HIP_OK(hipMemcpy(got_fp6.data(), d_d, got_fp6.size() * 2, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemset(d_d, 0, (size_t)M * N * 2));
+            wrap.gemm_dynamic(M, N, K, d_a, without, d_d, symmetric != 0, d_ws, ws_bytes, stream);
+            HIP_OK(hipStreamSynchronize(stream));
+            HIP_OK(hipMemcpy(got_int8.data(), d_d, got_int8.size() * 2, hipMemcpyDeviceToHost));
+            size_t nonzero = 0, differ = 0;
+            double worst = 0;
+            for (size_t i = 0; i < got_fp6.size(); ++i) {
+                nonzero += got_fp6[i] != 0;
+                differ += got_fp6[i] != got_int8[i];
+                const double a = abq_oracle_f16_to_f32(got_fp6[i]), b = abq_oracle_f16_to_f32(got_int8[i]);
+                worst = std::fmax(worst, std::fabs(a - b) / (std::fabs(b) + 1e-3));
+            }
+            CHECK(nonzero > got_fp6.size() / 2);
+            CHECK(worst <= 2e-3); // one fp16 unit at most: the zero-point terms are summed in a different association
+            (void)differ;
+        }
+        HIP_OK(hipFree(d_a));
+        HIP_OK(hipFree(d_d));
+        HIP_OK(hipFree(d_ws));
+    }
+
     {   // gate / up pair through the weight-blob interleave and the fused SiLU-gate epilogue, decode- and
         // prefill-sized M, against silu(gate GEMM) * (up GEMM) run as two separate dynamic GEMMs
         const int I = 96, K = 256, G = 128;
