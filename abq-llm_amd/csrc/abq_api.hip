@@ -654,12 +654,12 @@ static int pick_large_tile(const KernelEntry *entries, int count, const LargeTil
 }
 
 // Large tiles of the int8 kernels per operand pair: activations wider than the weights (W2A8, W4A8, W2A4)
-// gain most from tiles that are wide in N, 128x256 on the staged kernel and 256x256 (sixteen waves); signed
-// W8A8 from 256x128 and 256x256 (eight waves of 64x128).  Pairs of widths made of several fields keep the
+// gain most from tiles that are wide in N, 128x256 and 256x256 (eight waves of 64x128); signed W8A8 from 256x128
+// and 256x256.  Pairs of widths made of several fields keep the
 // thresholds below.
 static int large_tiles_int8(int x_bits, int w_bits, int is_signed, const LargeTile **out)
 {
-    static const LargeTile wide_n[] = { { 2, 2, 4, 4, 1.22, 1.22 }, { 2, 2, 2, 4, 1.04, 1.15 } };
+    static const LargeTile wide_n[] = { { 2, 4, 4, 2, 1.25, 1.25 }, { 2, 2, 2, 4, 1.04, 1.15 } };
     static const LargeTile w8a8[] = { { 2, 4, 4, 2, 1.45, 1.45 }, { 2, 2, 4, 2, 1.25, 1.30 } };
     const bool field = (x_bits == 2 || x_bits == 4 || x_bits == 8) && (w_bits == 2 || w_bits == 4 || w_bits == 8);
     if (field && x_bits > w_bits && (is_signed || x_bits < 8)) {

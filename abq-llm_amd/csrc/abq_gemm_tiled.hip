@@ -506,14 +506,22 @@ static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 #define ABQ_STAGED_WIDE_N(SG)
 #define ABQ_STAGED_WIDE_N_GROUPED(SG)
 #endif
+// The 256 x 256 tile of eight 64 x 128 waves: on the staged kernel where three LDS stages of it fit (not W8A8).
+#if ABQ_Q == 8 && ABQ_P == 8
+#define ABQ_STAGED_256(SG) ABQ_WENTRY_##SG(2, 4, 4, 2)
+#define ABQ_WENTRY_true(TM, TN, WM, WN) ABQ_WENTRY_T(TM, TN, WM, WN)
+#define ABQ_WENTRY_false(TM, TN, WM, WN) ABQ_WENTRY_F(TM, TN, WM, WN)
+#else
+#define ABQ_STAGED_256(SG) ABQ_SENTRY(SG, 2, 4, 4, 2)
+#endif
 static const KernelEntry kSigned[] = { ABQ_ENTRY_T(4, 4) ABQ_ENTRY_T(2, 4) ABQ_SENTRY(true, 2, 2, 2, 2) ABQ_SENTRY(true, 2, 1, 2, 2)
                                        ABQ_SENTRY(true, 1, 1, 2, 2) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_T)
-                                       ABQ_SENTRY(true, 2, 2, 4, 2) ABQ_WENTRY_T(2, 2, 4, 4) ABQ_WENTRY_T(2, 4, 4, 2)
+                                       ABQ_SENTRY(true, 2, 2, 4, 2) ABQ_WENTRY_T(2, 2, 4, 4) ABQ_STAGED_256(true)
                                        ABQ_STAGED_WIDE_N(true) };
 #if ABQ_Q < 8 && ABQ_P < 8
 static const KernelEntry kUnsigned[] = { ABQ_ENTRY_F(4, 4) ABQ_ENTRY_F(2, 4) ABQ_SENTRY(false, 2, 2, 2, 2) ABQ_SENTRY(false, 2, 1, 2, 2)
                                          ABQ_SENTRY(false, 1, 1, 2, 2) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
-                                         ABQ_SENTRY(false, 2, 2, 4, 2) ABQ_WENTRY_F(2, 2, 4, 4) ABQ_WENTRY_F(2, 4, 4, 2)
+                                         ABQ_SENTRY(false, 2, 2, 4, 2) ABQ_WENTRY_F(2, 2, 4, 4) ABQ_STAGED_256(false)
                                          ABQ_STAGED_WIDE_N(false) };
 #else
 static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)

@@ -354,9 +354,10 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(4, 4, 16384, 4096, 4096, F6) == (128, 128, 64, 64, 5)
     # W2A8: tiles that are wide in N
     assert picked(8, 2, 2048, 4096, 4096, T) == (128, 128, 64, 64, 4)
-    assert picked(8, 2, 4096, 11008, 4096, T) == (128, 256, 64, 64, 4)
+    assert picked(8, 2, 2048, 12288, 4096, T) == (128, 256, 64, 64, 4)
+    assert picked(8, 2, 4096, 11008, 4096, T) == (256, 256, 64, 128, 4)
     assert picked(8, 2, 1024, 12288, 4096, T) == (128, 128, 64, 64, 4)
-    assert picked(8, 2, 4096, 4096, 4096, T) == (256, 256, 64, 64, 4)
+    assert picked(8, 2, 4096, 4096, 4096, T) == (256, 256, 64, 128, 4)
     assert picked(8, 2, 512, 4096, 4096, T) == (64, 64, 32, 32, 4)
     # signed W8A8
     assert picked(8, 8, 2048, 4096, 4096, T) == (256, 128, 64, 64, 4)
