@@ -158,9 +158,8 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     const int M = __builtin_amdgcn_readfirstlane(a.M), N = __builtin_amdgcn_readfirstlane(a.N);
     const int ktiles = __builtin_amdgcn_readfirstlane(a.K) / 128;
 
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int nb = xcd * n_blocks_per_xcd + slot / m_blocks;
-    const int mb = slot % m_blocks;
+    int mb, nb;
+    tile_of_workgroup(blockIdx.x, m_blocks, n_blocks_per_xcd, &mb, &nb);
     const int m0 = mb * BM, n0 = nb * BN;
     if (n0 >= N)
         return; // uniform over the workgroup, before any barrier

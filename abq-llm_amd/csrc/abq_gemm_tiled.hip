@@ -239,9 +239,8 @@ void gemm_mfma_tiled(const GemmArgs a, const uint32_t *xt, const uint32_t *wt, i
     const int ktiles = __builtin_amdgcn_readfirstlane(a.K) / KB; // stages
 
     // workgroup -> tile: XCD x = id % 8 owns n blocks [x * npx, (x+1) * npx), M fastest
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int nb = xcd * n_blocks_per_xcd + slot / m_blocks;
-    const int mb = slot % m_blocks;
+    int mb, nb;
+    tile_of_workgroup(blockIdx.x, m_blocks, n_blocks_per_xcd, &mb, &nb);
     const int m0 = mb * BM, n0 = nb * BN;
     if (n0 >= N)
         return; // uniform over the workgroup, before any barrier

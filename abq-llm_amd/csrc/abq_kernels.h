@@ -65,6 +65,21 @@ inline size_t decode_grouped_lds(int M, int K, int group_size)
     return need <= 160 * 1024 ? need : 0;
 }
 
+// Workgroup id -> output tile.  XCD x = id % 8 owns n blocks [x * npx, (x + 1) * npx); inside an XCD the
+// workgroups run through groups of eight m blocks, M fastest inside a group, then N, then the next group:
+// the 32 or 64 workgroups an XCD runs at a time then cover a patch of 8 x 4 (or 8 x 8) tiles, so every
+// activation and weight block they load is shared in that XCD's L2, whatever M is.
+__device__ __forceinline__ void tile_of_workgroup(int id, int m_blocks, int n_blocks_per_xcd, int *mb, int *nb)
+{
+    constexpr int GM = 8;
+    const int xcd = id & 7, slot = id >> 3;
+    const int per_group = GM * n_blocks_per_xcd;
+    const int grp = slot / per_group, in = slot - grp * per_group;
+    const int gm = min(GM, m_blocks - grp * GM); // the last group may be short
+    *mb = grp * GM + in % gm;
+    *nb = xcd * n_blocks_per_xcd + in / gm;
+}
+
 __device__ __forceinline__ float silu(float x) { return x / (1.0f + __expf(-x)); }
 
 // ---- output stage shared by all kernels ------------------------------------------------
