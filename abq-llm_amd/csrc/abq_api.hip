@@ -637,7 +637,7 @@ static double cost_large(const LargeTile &c, int M, int N)
 // Index in `entries` of the best large tile that beats the 128x128 tile by a margin, or -1.
 static int pick_large_tile(const KernelEntry *entries, int count, const LargeTile *cands, int ncands, int M, int N)
 {
-    double best = 0.92 * cost_128x128(M, N);
+    double best = 0.97 * cost_128x128(M, N);
     int pick = -1;
     for (int k = 0; k < ncands; ++k) {
         const double cost = cost_large(cands[k], M, N);
@@ -653,27 +653,21 @@ static int pick_large_tile(const KernelEntry *entries, int count, const LargeTil
     return pick;
 }
 
-// Large tiles of the int8 kernels per operand pair: activations wider than the weights (W2A8, W4A8, W2A4)
-// gain most from tiles that are wide in N, 128x256 and 256x256 (eight waves of 64x128); signed W8A8 from 256x128
-// and 256x256.  Pairs of widths made of several fields keep the
-// thresholds below.
+// Large tiles of the int8 kernels per operand pair (sweep with the grouped tile mapping): for the pairs
+// below 16 bits together only 256x256 (eight waves of 64x128) beats 128x128, by 5-7 % once its grid
+// is a whole number of rounds; signed W8A8 gains 20 % from 256x128 as soon as that fills the chip.
+// Pairs of widths made of several fields keep the thresholds below.
 static int large_tiles_int8(int x_bits, int w_bits, int is_signed, const LargeTile **out)
 {
-    static const LargeTile wide_n[] = { { 2, 4, 4, 2, 1.25, 1.25 }, { 2, 2, 2, 4, 1.04, 1.15 } };
-    static const LargeTile w8a8[] = { { 2, 4, 4, 2, 1.45, 1.45 }, { 2, 2, 4, 2, 1.25, 1.30 } };
+    static const LargeTile wide_n[] = { { 2, 4, 4, 2, 1.06, 1.06 } };
+    static const LargeTile w8a8[] = { { 2, 2, 4, 2, 1.20, 1.20 } };
     const bool field = (x_bits == 2 || x_bits == 4 || x_bits == 8) && (w_bits == 2 || w_bits == 4 || w_bits == 8);
-    if (field && x_bits > w_bits && (is_signed || x_bits < 8)) {
-        *out = wide_n;
-        return 2;
-    }
-    if (x_bits == 8 && w_bits == 8 && is_signed) {
+    if (x_bits == 8 && w_bits == 8) {
         *out = w8a8;
-        return 2;
+        return is_signed ? 1 : 0;
     }
-    // equal widths below 8 bits (W4A4, W2A2 on the int8 route): only 256x256 beats 128x128, and only just
-    static const LargeTile narrow[] = { { 2, 4, 4, 2, 1.10, 1.10 } };
-    if (field && x_bits == w_bits && x_bits < 8) {
-        *out = narrow;
+    if (field && x_bits >= w_bits && (is_signed || x_bits < 8)) {
+        *out = wide_n;
         return 1;
     }
     return 0;
@@ -764,16 +758,11 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
     }
     int count = 0;
     const KernelEntry *es = fp6_entries(&count);
-    // The 256x128 tile of eight waves against 128x128 by the cost model above (it pays over several rounds
-    // of workgroups; alone on a compute unit, in a single round, it hides less latency than two 128x128
-    // workgroups do); below a chip's worth of 128x128 tiles the smaller ones:
-    // { TM, TN, waves along M, waves along N, workgroups needed }
-    static const LargeTile large[] = { { 2, 2, 4, 2, 0.95, 1.18 } };
+    // 128x128 (two workgroups per compute unit) is the fastest tile from 200 tiles up: with the grouped tile
+    // mapping it beats 256x128 at every M of the sweep but the very largest, by 3-10 %; below that the
+    // smaller ones: { TM, TN, waves along M, waves along N, workgroups needed }
     static const int order[][5] = { { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 400 }, { 1, 1, 2, 2, 0 } };
     int pick = -1;
-    // (beyond 8192 rows the 256x128 tile falls behind 128x128 again: 1620-2070 against 1820-2100 TOPS at 16384 rows)
-    if ((long)((st->M + 127) / 128) * ((st->N + 127) / 128) >= 200 && st->M <= 8192)
-        pick = pick_large_tile(es, count, large, 1, st->M, st->N);
     for (const auto &o : order) {
         const int bm = 32 * o[0] * o[2], bn = 32 * o[1] * o[3];
         const long tiles = (long)((st->M + bm - 1) / bm) * ((st->N + bn - 1) / bn);
