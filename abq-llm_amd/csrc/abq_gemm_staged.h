@@ -29,7 +29,8 @@
 // drains the counter before its epilogue.  A register spill would be such an instruction: every
 // instantiation must compile with .vgpr_spill_count 0 and no private segment (hipcc -save-temps
 // shows both in the kernel's metadata), which is why the tile variants stop where they do.  One barrier per K tile.  Workgroups are numbered so
-// that the 8 XCDs (workgroup id modulo 8) each work on a contiguous band of N with M fastest.
+// that the 8 XCDs (workgroup id modulo 8) each work on a contiguous band of N, in groups of four m blocks
+// (tile_of_workgroup).
 // What bounds the kernel on LLaMA-sized problems is the rate at which L2 delivers the tiles
 // (about 22 TB/s over the chip), not the matrix cores.
 #pragma once

@@ -25,7 +25,8 @@
 // and the plane words of the next two K tiles are in flight in registers, so the expansion
 // of tile i+1 and the loads of tile i+2 overlap the MFMAs of tile i; one barrier per K tile.
 // Workgroups are numbered so that the 8 XCDs (workgroup id modulo 8) each work on a
-// contiguous band of N with M fastest: a band's weight panels stay in that XCD's L2.
+// contiguous band of N, in groups of four m blocks (tile_of_workgroup): the workgroups an XCD
+// runs at a time share their activation and weight blocks in that XCD's L2.
 #include "abq_kernels.h"
 #include "abq_gemm_staged.h"
 

@@ -349,25 +349,39 @@ template <int LAYOUT>
 __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__restrict__ x, uint32_t *__restrict__ planes,
                                                               float *__restrict__ scale_out, float *__restrict__ zero_out,
                                                               int *__restrict__ group_sums, int M, int K, int bits,
-                                                              int symmetric, int group_size)
+                                                              int symmetric, int group_size, int keep_row)
 {
+    // keep_row: the row stays in LDS between the two passes (each lane re-reads the units it wrote itself),
+    // so that it comes from memory once; with rows of 22 KB the rows in flight no longer fit the L2
+    extern __shared__ uint4 row_lds[];
     __shared__ float red[2][4];
     const int row = blockIdx.x, tid = threadIdx.x;
     const int units = K / 8; // 8 halves per 16-byte load
     const uint4 *xr = x + (size_t)row * units;
 
     float mx = -INFINITY, mn = INFINITY;
-    for (int u = tid; u < units; u += 256) {
+    // four loads in flight per lane: with one, the pass is bound by the latency of memory, not its bandwidth
+    for (int u0 = tid; u0 < units; u0 += 1024) {
         union {
             uint4 q;
             _Float16 h[8];
-        } raw;
-        raw.q = xr[u];
+        } raw[4];
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            const float f = (float)raw.h[c];
-            mx = fmaxf(mx, f);
-            mn = fminf(mn, f);
+        for (int i = 0; i < 4; ++i) {
+            const int u = u0 + 256 * i;
+            raw[i].q = xr[u < units ? u : u0]; // past the end: the lane's first unit once more
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int u = u0 + 256 * i;
+            if (keep_row && u < units)
+                row_lds[u] = raw[i].q;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const float f = (float)raw[i].h[c];
+                mx = fmaxf(mx, f);
+                mn = fminf(mn, f);
+            }
         }
     }
     mx = wave_max(mx);
@@ -402,6 +416,20 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
             zero_out[row] = symmetric ? 0.f : zp - (float)half_range;
     }
 
+    // x / scale in three operations instead of the dozen of a full division, with the same bits: recip is the
+    // correctly rounded reciprocal (the fp64 quotient is never close enough to an fp32 midpoint for the second
+    // rounding to cross it), t = x recip is within an ulp of the quotient, the residual x - t scale is exact in
+    // an fma, and t + residual recip then rounds to the quotient itself (checked against the division on a CPU
+    // for every finite fp16 value and 600 000 scales of the forms above; a zero may come out with the other
+    // sign, which the rounding to an integer code forgets).  div_fixup restores what a division makes of an
+    // infinite x.
+    const float recip = (float)(1.0 / (double)scale);
+    // only a row that holds an infinity needs the fix-up (a NaN goes through the fmas as through a division)
+    const bool fix_up = __builtin_amdgcn_readfirstlane(!(fabsf(mx) <= 65504.f && fabsf(mn) <= 65504.f)) != 0;
+    // rint(q) + zp, clamped to [lo, hi], minus the offset of the stored code: the offset is taken off before the
+    // clamp instead (all three are small integers, so the sums are the same numbers)
+    const float code_offset = symmetric ? 0.f : (float)half_range;
+    const float zp_stored = zp - code_offset, lo_stored = (float)lo - code_offset, hi_stored = (float)hi - code_offset;
     const int KW = K / 32;
     const int rounded = (units + 255) / 256 * 256;
     const int lanes_per_group = group_size / 8;
@@ -414,12 +442,15 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
                 uint4 q;
                 _Float16 h[8];
             } raw;
-            raw.q = xr[u];
+            raw.q = keep_row ? row_lds[u] : xr[u];
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
-                float r = rintf((float)raw.h[c] / scale) + zp;
-                r = fminf(fmaxf(r, (float)lo), (float)hi);
-                v[c] = (int)r - (symmetric ? 0 : half_range);
+                const float xf = (float)raw.h[c];
+                const float t = xf * recip;
+                float quotient = __builtin_fmaf(__builtin_fmaf(-t, scale, xf), recip, t);
+                if (fix_up)
+                    quotient = __builtin_amdgcn_div_fixupf(quotient, scale, xf);
+                v[c] = (int)__builtin_amdgcn_fmed3f(rintf(quotient) + zp_stored, lo_stored, hi_stored);
                 sum += v[c];
             }
         }
@@ -480,18 +511,21 @@ hipError_t launch_quant_pack_rows(const void *x, uint32_t *planes, float *scale,
                                   int M, int K, int bits, int symmetric, int group_size, int layout,
                                   hipStream_t stream)
 {
+    // a row of up to 48 KiB is kept in LDS (within the default limit together with the static part)
+    const int keep_row = (size_t)K * 2 <= 48 * 1024;
+    const size_t lds = keep_row ? (size_t)K * 2 : 0;
     if (layout == 2)
-        hipLaunchKernelGGL(quant_pack_rows_kernel<2>, dim3(M), dim3(256), 0, stream,
+        hipLaunchKernelGGL(quant_pack_rows_kernel<2>, dim3(M), dim3(256), lds, stream,
                            reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits,
-                           symmetric, group_size);
+                           symmetric, group_size, keep_row);
     else if (layout == 1)
-        hipLaunchKernelGGL(quant_pack_rows_kernel<1>, dim3(M), dim3(256), 0, stream,
+        hipLaunchKernelGGL(quant_pack_rows_kernel<1>, dim3(M), dim3(256), lds, stream,
                            reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits,
-                           symmetric, group_size);
+                           symmetric, group_size, keep_row);
     else
-        hipLaunchKernelGGL(quant_pack_rows_kernel<0>, dim3(M), dim3(256), 0, stream,
+        hipLaunchKernelGGL(quant_pack_rows_kernel<0>, dim3(M), dim3(256), lds, stream,
                            reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits,
-                           symmetric, group_size);
+                           symmetric, group_size, keep_row);
     return hipGetLastError();
 }
 

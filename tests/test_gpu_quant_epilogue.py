@@ -79,6 +79,31 @@ def test_quant_pack_matches_the_restated_quantizer(abq, oracle, rows, k, bits, s
             abq.quant_pack_f16(torch.from_numpy(x).cuda(), bits, symmetric=symmetric, fp6=True)
 
 
+@pytest.mark.parametrize("absmax,bits", [(127.0, 8), (381.0, 8), (63.5, 8), (21.0, 4), (889.0, 8), (3.0, 2), (77.0, 4),
+                                         (35.0, 4), (91.0, 4)])
+def test_quant_pack_rounds_exact_ties_like_the_division(abq, oracle, absmax, bits):
+    """Rows whose scale is 1, 3, 0.5, 7 ... exactly and whose values are odd multiples of half a scale: every
+    quotient is a tie, so a quotient that is off by one ulp rounds to the other neighbour."""
+    from oracle import quantizer as Q
+    qmax = (1 << (bits - 1)) - 1
+    step = absmax / qmax
+    k = 256
+    x = np.zeros((4, k), dtype=np.float16)
+    odd = np.arange(k) * 2 + 1
+    x[0] = ((odd % (2 * qmax)) * step / 2)
+    x[1] = -x[0]
+    x[2] = (np.arange(k) % (qmax + 1)) * step
+    x[3] = x[0] * np.where(np.arange(k) % 3 == 0, -1, 1)
+    x[:, -1] = absmax
+    assert np.array_equal(x.astype(np.float64)[0, :-1], (odd % (2 * qmax))[:-1] * step / 2)  # exact in fp16
+    codes, scale, _ = Q.per_token_codes_f32(x, bits, True)
+    assert np.all(scale == np.float32(step))
+    planes, s, _, _ = abq.quant_pack_f16(torch.from_numpy(x).cuda(), bits, symmetric=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(s.cpu().numpy(), scale)
+    assert np.array_equal(planes.cpu().numpy().view(np.uint32), oracle.pack_i32(codes, bits))
+
+
 # ------------------------------------------------------------------ group scales, zero points
 
 @pytest.mark.parametrize("q,p,signed", [(8, 2, True), (4, 4, True), (8, 4, True), (4, 4, False), (6, 2, False),
