@@ -52,7 +52,8 @@ def run_grouped(abq, xp, wp, signed, strategy="tiled", **kw):
 
 @pytest.mark.parametrize("rows,k,bits,symmetric", [(1, 128, 8, True), (5, 4096, 8, True), (33, 11008, 8, False),
                                                    (7, 256, 4, True), (16, 1152, 4, False), (3, 384, 2, True),
-                                                   (64, 4096, 6, False), (9, 640, 5, False), (12, 512, 3, True)])
+                                                   (64, 4096, 6, False), (9, 640, 5, False), (12, 512, 3, True),
+                                                   (3, 24576, 8, True), (2, 24704, 8, False)])  # last row kept in LDS / first not
 def test_quant_pack_matches_the_restated_quantizer(abq, oracle, rows, k, bits, symmetric):
     from oracle import quantizer as Q
     rng = np.random.default_rng(rows + k + bits)
