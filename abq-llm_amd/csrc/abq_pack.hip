@@ -336,6 +336,33 @@ __device__ __forceinline__ void store_fields_any(uint32_t *rec, int ws, const ui
 // Optionally writes the sum of the codes over every group of group_size elements (the GEMM's
 // zero-point correction needs them).
 
+// The low bytes of four integers as one dword, a in byte 0.
+__device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d)
+{
+    const uint32_t ab = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
+    const uint32_t cd = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
+}
+
+// 4 x 4 byte transpose across a quad with the lane order reversed: lane s returns the dword whose byte c is
+// byte s of lane 3 - c's argument.  sel_pair / sel_half are the lane's byte selectors of the two exchange
+// steps (quad_transpose_selectors).
+__device__ __forceinline__ uint32_t quad_transpose_bytes(uint32_t v, uint32_t sel_pair, uint32_t sel_half)
+{
+    const uint32_t p = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true); // lane ^ 1
+    const uint32_t x = __builtin_amdgcn_perm(p, v, sel_pair);
+    const uint32_t q = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true); // lane ^ 2
+    return __builtin_amdgcn_perm(q, x, sel_half);
+}
+
+__device__ __forceinline__ void quad_transpose_selectors(int quad_lane, uint32_t &sel_pair, uint32_t &sel_half)
+{
+    // step 1: even lanes keep their bytes 0, 2 and take the partner's 0, 2; odd lanes the bytes 1, 3
+    sel_pair = (quad_lane & 1) ? 0x03070105u : 0x06020400u;
+    // step 2: lanes 0, 1 take the low halves, lanes 2, 3 the high halves, bytes in reversed order
+    sel_half = (quad_lane & 2) ? 0x06070203u : 0x00010405u;
+}
+
 __device__ __forceinline__ float wave_max(float v)
 {
 #pragma unroll
@@ -359,12 +386,14 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
     const int units = K / 8; // 8 halves per 16-byte load
     const uint4 *xr = x + (size_t)row * units;
 
-    float mx = -INFINITY, mn = INFINITY;
-    // four loads in flight per lane: with one, the pass is bound by the latency of memory, not its bandwidth
+    // four loads in flight per lane: with one, the pass is bound by the latency of memory, not its bandwidth.
+    // Minimum and maximum are taken on the fp16 pairs as they are (two elements per instruction).
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    half2_t mx2 = { (_Float16)-INFINITY, (_Float16)-INFINITY }, mn2 = { (_Float16)INFINITY, (_Float16)INFINITY };
     for (int u0 = tid; u0 < units; u0 += 1024) {
         union {
             uint4 q;
-            _Float16 h[8];
+            half2_t h2[4];
         } raw[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -377,13 +406,13 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
             if (keep_row && u < units)
                 row_lds[u] = raw[i].q;
 #pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                const float f = (float)raw[i].h[c];
-                mx = fmaxf(mx, f);
-                mn = fminf(mn, f);
+            for (int c = 0; c < 4; ++c) {
+                mx2 = __builtin_elementwise_max(mx2, raw[i].h2[c]);
+                mn2 = __builtin_elementwise_min(mn2, raw[i].h2[c]);
             }
         }
     }
+    float mx = fmaxf((float)mx2.x, (float)mx2.y), mn = fminf((float)mn2.x, (float)mn2.y);
     mx = wave_max(mx);
     mn = -wave_max(-mn);
     if ((tid & 63) == 0) {
@@ -433,6 +462,8 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
     const int KW = K / 32;
     const int rounded = (units + 255) / 256 * 256;
     const int lanes_per_group = group_size / 8;
+    uint32_t sel_pair, sel_half;
+    quad_transpose_selectors(tid & 3, sel_pair, sel_half);
     for (int u = tid; u < rounded; u += 256) {
         const bool active = u < units; // units is a multiple of 16: quads and groups are active as one
         int v[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
@@ -484,6 +515,17 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
                 *reinterpret_cast<uint2 *>(rec) = make_uint2(o[0], o[1]);
                 *reinterpret_cast<uint2 *>(rec + 2) = make_uint2(o[2], o[3]);
                 *reinterpret_cast<uint2 *>(rec + 4) = make_uint2(o[4], o[5]);
+            }
+        } else if (LAYOUT == 1 && bits == 8) {
+            // 8-bit codes are the record's bytes themselves: expanded dword s, byte c = element 31 - (8c + s) of
+            // the word-set = element 7 - s of lane 3 - c.  The quad transposes its bytes so that lane s ends
+            // with the dwords s and 4 + s, and every lane stores its two.
+            const uint32_t e_lo = quad_transpose_bytes(pack_low_bytes(v[7], v[6], v[5], v[4]), sel_pair, sel_half);
+            const uint32_t e_hi = quad_transpose_bytes(pack_low_bytes(v[3], v[2], v[1], v[0]), sel_pair, sel_half);
+            if (active) {
+                uint32_t *dst = planes + ((size_t)(w >> 2) * M + row) * 32 + 8 * (w & 3) + quad_lane;
+                dst[0] = e_lo;
+                dst[4] = e_hi;
             }
         } else if (LAYOUT == 1) {
             // expanded dword s, byte c = element 31 - (8c + s) of the word-set: this lane's element
