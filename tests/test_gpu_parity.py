@@ -309,6 +309,32 @@ def test_scaled_fp16_epilogue_every_staged_tile(abq, oracle, q, p, fp6, signed):
             assert np.array_equal(got16.view(np.uint16), want16.view(np.uint16)), (g.config_name, M, N, K)
 
 
+@pytest.mark.parametrize("q,p,fp6,signed", [(8, 2, False, True), (4, 4, True, True), (8, 8, False, True), (7, 7, False, False),
+                                             (4, 4, False, False)])
+def test_workgroup_numbering_covers_every_tile(abq, oracle, q, p, fp6, signed):
+    """Every tile of the LDS-staged kernels on grids whose number of m blocks is not a multiple of the four
+    the workgroup numbering groups them by (4 + 2, and 4 + 4 + 1), with n blocks that do not fill the eight
+    bands (18 blocks in bands of 3): every output element written once, with the right value."""
+    rng = np.random.default_rng(4100 + 10 * q + p + fp6)
+    tiles = [c for c in abq.native_configs(q, p, signed) if c.nstage == (5 if fp6 else 4) and c.warp_k == 128]
+    assert tiles
+    K = 256
+    for cfg in tiles:
+        for m_blocks, n_blocks in ((6, 18), (9, 5)):
+            M, N = (m_blocks - 1) * cfg.block_m + 9, (n_blocks - 1) * cfg.block_n + 40
+            x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+            xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
+            if fp6:
+                xo, wo, kw = abq.relayout_planes_fp6(xd, signed), abq.relayout_planes_fp6(wd, signed), dict(x_fp6=q, w_fp6=p)
+            else:
+                xo, wo, kw = abq.relayout_planes(xd), abq.relayout_planes(wd), dict(x_tiled=True, w_tiled=True)
+            want = (x.astype(np.float64) @ w.astype(np.float64).T).astype(np.int32)  # exact: |sums| < 2^53
+            out = torch.full((M, N), -12345, dtype=torch.int32, device="cuda")
+            g = abq.Gemm(xo, wo, signed, cfg=cfg, out=out, **kw)
+            got = g.run().cpu().numpy()
+            assert np.array_equal(got, want), (g.config_name, M, N, K)
+
+
 @pytest.mark.parametrize("signed", [True, False])
 def test_config2_w4a4_prefill_full_size_fp6(abq, oracle, signed):
     """W4A4 at M in {512, 2048} on the LLaMA-7B shapes through the FP6 route: exact against the fp64
