@@ -729,18 +729,23 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
     if (!fp6_eligible(c.x_bits, c.w_bits, c.is_signed, st->K))
         return ABQ_ERR_UNSUPPORTED;
     if (st->group_size) {
-        // group scales: one scale per K tile, i.e. groups of 128; tiles as for the int8 group-scale kernels
-        // (128x128 once it fills the chip, else 128x64, the smallest tile with two MFMA tiles per wave)
+        // group scales: one scale per K tile, i.e. groups of 128.  Below 300 tiles of 128x128: 128x64, the
+        // smallest tile with two MFMA tiles per wave; above, 256x128 runs 6 % faster than 128x128 where its
+        // rounds of workgroups come out even (sweep of the three tiles over M = 512 .. 16384 and the LLaMA
+        // widths: the choice is within 0.1 % of the best tile on average, 4 % at worst)
         if (st->group_size != 128)
             return ABQ_ERR_UNSUPPORTED;
         int gcount = 0;
         const KernelEntry *ge = fp6_grouped_entries(&gcount);
         const long t128 = (long)((st->M + 127) / 128) * ((st->N + 127) / 128);
+        static const LargeTile grouped_large[] = { { 2, 2, 4, 2, 1.06, 1.06 } };
+        const int large = st->auto_chosen && t128 >= 300 ? pick_large_tile(ge, gcount, grouped_large, 1, st->M, st->N) : -1;
         int gpick = -1;
         for (int i = 0; i < gcount; ++i) {
             const int bm = 32 * ge[i].tm * ge[i].wm, bn = 32 * ge[i].tn * ge[i].wn;
             if (!st->auto_chosen ? (bm == c.block_m && bn == c.block_n && 32 * ge[i].tm == c.warp_m)
-                                 : ((t128 >= 300 && bm == 128 && bn == 128) || (t128 < 300 && bm == 128 && bn == 64)))
+                                 : large >= 0 ? i == large
+                                              : ((t128 >= 300 && bm == 128 && bn == 128) || (t128 < 300 && bm == 128 && bn == 64)))
                 gpick = i;
         }
         if (gpick < 0)
@@ -807,9 +812,10 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
     if (state->auto_chosen) {
         // The fold of the int32 tiles into fp32 bounds these kernels more than the tile traffic does, so tile
         // sizes from 128x128 up run within a few percent of each other (sweep over M = 256 .. 16384 and the
-        // LLaMA widths): 128x128 once it fills the chip, below that 128x64, then 64x64.
+        // LLaMA widths): 128x128 once it fills the chip, below that 128x64, then 64x64.  With activations of
+        // at most 4 bits three workgroups of 128x64 fit a compute unit and stay ahead up to 400 tiles.
         const long t128 = (long)((state->M + 127) / 128) * ((state->N + 127) / 128);
-        static const int order[][3] = { { 128, 128, 300 }, { 128, 64, 64 }, { 64, 64, 0 } };
+        const int order[][3] = { { 128, 128, c.x_bits <= 4 ? 400 : 300 }, { 128, 64, 64 }, { 64, 64, 0 } };
         for (const auto &o : order) {
             if (pick >= 0 || t128 < o[2])
                 continue;

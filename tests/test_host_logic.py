@@ -367,3 +367,12 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(8, 2, 1024, 4096, 4096, T, group=128) == (128, 64, 64, 32, 4)
     assert picked(8, 2, 16384, 22016, 4096, T, group=128) == (128, 128, 64, 64, 4)
     assert picked(8, 2, 128, 4096, 4096, T, group=64) == (64, 64, 32, 32, 4)
+    # ... activations of at most 4 bits keep 128x64 up to 400 tiles
+    assert picked(4, 4, 512, 11008, 4096, T, group=128) == (128, 64, 64, 32, 4)
+    assert picked(8, 2, 512, 11008, 4096, T, group=128) == (128, 128, 64, 64, 4)
+    assert picked(4, 4, 2048, 4096, 4096, T, group=128) == (128, 128, 64, 64, 4)
+    # group scales on FP6 records: 256x128 where its rounds of workgroups come out even
+    assert picked(4, 4, 2048, 4096, 4096, F6, group=128) == (256, 128, 64, 64, 5)
+    assert picked(4, 4, 1024, 11008, 4096, F6, group=128) == (128, 128, 64, 64, 5)   # 344 tiles of 256x128: 1.3 rounds
+    assert picked(4, 4, 16384, 4096, 11008, F6, group=128) == (256, 128, 64, 64, 5)
+    assert picked(4, 4, 1024, 4096, 4096, F6, group=128) == (128, 64, 64, 32, 5)
