@@ -80,6 +80,26 @@ def test_quant_pack_matches_the_restated_quantizer(abq, oracle, rows, k, bits, s
             abq.quant_pack_f16(torch.from_numpy(x).cuda(), bits, symmetric=symmetric, fp6=True)
 
 
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_quant_pack_rows_with_infinities(abq, oracle, symmetric):
+    """A row that holds an infinity: the scale saturates at its upper clamp and the infinite elements take the
+    end codes, as a division would leave them (the kernel's quotient without a division needs its fix-up here)."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(77 + symmetric)
+    x = (rng.normal(0, 300, (4, 512))).astype(np.float16)
+    x[0, 3], x[0, 100] = np.inf, -np.inf
+    x[1, 511] = np.inf
+    x[2, 0] = -np.inf
+    with np.errstate(invalid="ignore", over="ignore"):
+        codes, scale, zero = Q.per_token_codes_f32(x, 8, symmetric)
+    planes, s, z, _ = abq.quant_pack_f16(torch.from_numpy(x).cuda(), 8, symmetric=symmetric)
+    torch.cuda.synchronize()
+    assert np.array_equal(s.cpu().numpy(), scale)
+    if not symmetric:
+        assert np.array_equal(z.cpu().numpy(), zero)
+    assert np.array_equal(planes.cpu().numpy().view(np.uint32), oracle.pack_i32(codes, 8))
+
+
 @pytest.mark.parametrize("absmax,bits", [(127.0, 8), (381.0, 8), (63.5, 8), (21.0, 4), (889.0, 8), (3.0, 2), (77.0, 4),
                                          (35.0, 4), (91.0, 4)])
 def test_quant_pack_rounds_exact_ties_like_the_division(abq, oracle, absmax, bits):
