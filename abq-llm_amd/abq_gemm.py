@@ -19,8 +19,9 @@ STATUS_NAMES = {
 }
 globals().update({name: code for code, name in STATUS_NAMES.items()})
 OUT_I32, OUT_F16_TENSOR, OUT_F16_SCALED, OUT_F16_TENSOR_F32SCALE = 0, 1, 2, 3
-STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC, STRATEGY_DECODE, STRATEGY_TILED, STRATEGY_FP6 = range(8)
-STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic", "decode", "tiled", "fp6"]
+(STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC, STRATEGY_DECODE, STRATEGY_TILED, STRATEGY_FP6,
+ STRATEGY_DECODE_TILED) = range(9)
+STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic", "decode", "tiled", "fp6", "decode_tiled"]
 LAYOUT_PLANES, LAYOUT_TILED, LAYOUT_FP6 = 0, 1, 2
 ACT_NONE, ACT_SILU_GATE = 0, 1
 

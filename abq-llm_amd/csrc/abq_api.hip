@@ -35,7 +35,8 @@ hipError_t launch_weight_zero_term(const uint32_t *, int, int, int, int, const f
     void abq_decode_register_##Q##_##P(KernelTable *); \
     void abq_decode_grouped_register_##Q##_##P(KernelTable *); \
     void abq_tiled_register_##Q##_##P(KernelTable *);  \
-    void abq_tiled_grouped_register_##Q##_##P(KernelTable *);
+    void abq_tiled_grouped_register_##Q##_##P(KernelTable *);  \
+    void abq_decode_tiled_register_##Q##_##P(KernelTable *);
 ABQ_FOR_EACH_COMBO(ABQ_DECL)
 #undef ABQ_DECL
 
@@ -46,6 +47,7 @@ struct Registry {
     KernelTable decode_grouped[2 * ABQ_NUM_COMBOS];
     KernelTable tiled[2 * ABQ_NUM_COMBOS];
     KernelTable tiled_grouped[2 * ABQ_NUM_COMBOS];
+    KernelTable decode_tiled[2 * ABQ_NUM_COMBOS];
     Registry()
     {
         int i = 0;
@@ -56,6 +58,7 @@ struct Registry {
     abq_decode_grouped_register_##Q##_##P(&decode_grouped[i]); \
     abq_tiled_register_##Q##_##P(&tiled[i]);           \
     abq_tiled_grouped_register_##Q##_##P(&tiled_grouped[i]); \
+    abq_decode_tiled_register_##Q##_##P(&decode_tiled[i]); \
     i += 2;
         ABQ_FOR_EACH_COMBO(ABQ_REG)
 #undef ABQ_REG
@@ -272,7 +275,7 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
     } else {
         mi = cfg->mma_m;
         const int stepk = ((strategy == ABQ_STRATEGY_MFMA32 && cfg->nstage == 4) ||
-                           (strategy == ABQ_STRATEGY_MFMA16 && cfg->nstage == 3)) ? cfg->warp_k : (64 / mi) * 4 * 32;
+                           (strategy == ABQ_STRATEGY_MFMA16 && (cfg->nstage == 3 || cfg->nstage == 6))) ? cfg->warp_k : (64 / mi) * 4 * 32;
         if (cfg->warp_m <= 0 || cfg->warp_n <= 0 || cfg->warp_m % mi || cfg->warp_n % mi ||
             cfg->block_m % cfg->warp_m || cfg->block_n % cfg->warp_n || cfg->warp_k != stepk ||
             cfg->block_k % stepk)
@@ -282,6 +285,8 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         wk = cfg->block_k / stepk;
         if (strategy == ABQ_STRATEGY_MFMA16 && cfg->nstage == 3)
             strategy = ABQ_STRATEGY_DECODE;
+        if (strategy == ABQ_STRATEGY_MFMA16 && cfg->nstage == 6)
+            strategy = ABQ_STRATEGY_DECODE_TILED;
         if (strategy == ABQ_STRATEGY_MFMA32 && cfg->nstage == 4)
             strategy = ABQ_STRATEGY_TILED;
     }
@@ -309,6 +314,31 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         st->grid_dim = abq_dim3{ (unsigned)(8 * npx * mblocks), 1, 1 };
         st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
         st->shared_mem_size = e.lds ? e.lds : 2 * (size_t)(bm + bn) * (e.kb + 16) + (bm + bn) * 4;
+        return ABQ_OK;
+    }
+
+    if (strategy == ABQ_STRATEGY_DECODE_TILED) {
+        const KernelTable *tdt = find_table(reg.decode_tiled, x_bits, w_bits, is_signed);
+        if (!tdt || mi != 16 || tm != 1 || wm != 1 || wn != 1)
+            return ABQ_ERR_UNSUPPORTED;
+        int v = -1;
+        for (int i = 0; i < tdt->count; ++i)
+            if (tdt->entries[i].tn == tn && tdt->entries[i].wk == wk && tdt->entries[i].kb == cfg->warp_k)
+                v = i;
+        if (v < 0)
+            return ABQ_ERR_UNSUPPORTED;
+        const KernelEntry &e = tdt->entries[v];
+        const int mrows = decode_tiled_rows(e.wk, e.tn, M, K, x_bits);
+        // byte offsets inside the kernel are 32 bits wide
+        if (mrows == 0 || K >= (1 << 17) || (size_t)N * K * w_bits / 8 >= (1ull << 32) || (size_t)M * K * x_bits / 8 >= (1ull << 32) ||
+            (M + mrows - 1) / mrows > 65535)
+            return ABQ_ERR_TOO_LARGE;
+        st->strategy = strategy;
+        st->variant = v;
+        entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
+        st->grid_dim = abq_dim3{ (unsigned)(((N + 15) / 16 + e.tn - 1) / e.tn), (unsigned)((M + mrows - 1) / mrows), 1 };
+        st->block_dim = abq_dim3{ (unsigned)(64 * e.wk), 1, 1 };
+        st->shared_mem_size = decode_tiled_lds(e.wk, e.tn, mrows, K, x_bits);
         return ABQ_OK;
     }
 
@@ -492,64 +522,60 @@ abq_status abq_format_kernel_name(const abq_tile_config *c, int is_wmma, char *b
     return (w < 0 || (size_t)w >= n) ? ABQ_ERR_TOO_LARGE : ABQ_OK;
 }
 
-// Native tile space: popcount entries for 16/32/64 lanes per row, then the MFMA entries.
-int abq_native_config_count(int x_bits, int w_bits, int is_signed)
+// Native tile space: popcount entries for 16/32/64 lanes per row, the decode kernel, the direct MFMA kernels,
+// the LDS-staged kernels, the FP6 kernel, the decode kernel on K-tiled operands.
+static int native_config(int x_bits, int w_bits, int is_signed, int index, abq_tile_config *cfg)
 {
     const Registry &reg = registry();
     const KernelTable *tb = find_table(reg.bcnt, x_bits, w_bits, is_signed);
     const KernelTable *tm = find_table(reg.mfma, x_bits, w_bits, is_signed);
     const KernelTable *td = find_table(reg.decode, x_bits, w_bits, is_signed);
     const KernelTable *tt = find_table(reg.tiled, x_bits, w_bits, is_signed);
+    const KernelTable *tdt = find_table(reg.decode_tiled, x_bits, w_bits, is_signed);
     if (!tb || !tm || !td || !tt)
         return 0;
-    int nfp6 = 0;
-    if (fp6_eligible(x_bits, w_bits, is_signed, 128))
-        fp6_entries(&nfp6);
-    return tb->count * 3 + td->count + tm->count + tt->count + nfp6;
+    int n = 0;
+    // returns true when `index` falls into the next `count` entries
+    auto in = [&](int count) {
+        const bool hit = cfg && index >= n && index < n + count;
+        n += count;
+        return hit;
+    };
+    if (in(tb->count * 3))
+        entry_to_config(tb->entries[(index - (n - tb->count * 3)) / 3], ABQ_STRATEGY_BCNT, x_bits, w_bits, is_signed,
+                        4 + (index - (n - tb->count * 3)) % 3, cfg);
+    if (in(td->count))
+        entry_to_config(td->entries[index - (n - td->count)], ABQ_STRATEGY_DECODE, x_bits, w_bits, is_signed, 0, cfg);
+    if (in(tm->count)) {
+        const KernelEntry &e = tm->entries[index - (n - tm->count)];
+        entry_to_config(e, e.mi == 16 ? ABQ_STRATEGY_MFMA16 : ABQ_STRATEGY_MFMA32, x_bits, w_bits, is_signed, 0, cfg);
+    }
+    if (in(tt->count))
+        entry_to_config(tt->entries[index - (n - tt->count)], ABQ_STRATEGY_TILED, x_bits, w_bits, is_signed, 0, cfg);
+    if (fp6_eligible(x_bits, w_bits, is_signed, 128)) {
+        int nfp6 = 0;
+        const KernelEntry *es = fp6_entries(&nfp6);
+        if (in(nfp6))
+            entry_to_config(es[index - (n - nfp6)], ABQ_STRATEGY_FP6, x_bits, w_bits, is_signed, 0, cfg);
+    }
+    if (tdt && in(tdt->count))
+        entry_to_config(tdt->entries[index - (n - tdt->count)], ABQ_STRATEGY_DECODE_TILED, x_bits, w_bits, is_signed, 0, cfg);
+    return n;
+}
+
+int abq_native_config_count(int x_bits, int w_bits, int is_signed)
+{
+    return native_config(x_bits, w_bits, is_signed, -1, nullptr);
 }
 
 abq_status abq_native_config_get(int x_bits, int w_bits, int is_signed, int index, abq_tile_config *cfg)
 {
     if (!cfg || index < 0)
         return ABQ_ERR_INVALID_ARG;
-    const Registry &reg = registry();
-    const KernelTable *tb = find_table(reg.bcnt, x_bits, w_bits, is_signed);
-    const KernelTable *tm = find_table(reg.mfma, x_bits, w_bits, is_signed);
-    const KernelTable *td = find_table(reg.decode, x_bits, w_bits, is_signed);
-    if (!tb || !tm || !td)
+    const int n = native_config(x_bits, w_bits, is_signed, index, cfg);
+    if (n == 0)
         return ABQ_ERR_UNSUPPORTED;
-    if (index < tb->count * 3) {
-        entry_to_config(tb->entries[index / 3], ABQ_STRATEGY_BCNT, x_bits, w_bits, is_signed,
-                        4 + index % 3, cfg);
-        return ABQ_OK;
-    }
-    index -= tb->count * 3;
-    if (index < td->count) {
-        entry_to_config(td->entries[index], ABQ_STRATEGY_DECODE, x_bits, w_bits, is_signed, 0, cfg);
-        return ABQ_OK;
-    }
-    index -= td->count;
-    if (index >= tm->count) {
-        const KernelTable *tt = find_table(reg.tiled, x_bits, w_bits, is_signed);
-        index -= tm->count;
-        if (!tt)
-            return ABQ_ERR_INVALID_ARG;
-        if (index >= tt->count) {
-            index -= tt->count;
-            int nfp6 = 0;
-            const KernelEntry *es = fp6_entries(&nfp6);
-            if (!fp6_eligible(x_bits, w_bits, is_signed, 128) || index >= nfp6)
-                return ABQ_ERR_INVALID_ARG;
-            entry_to_config(es[index], ABQ_STRATEGY_FP6, x_bits, w_bits, is_signed, 0, cfg);
-            return ABQ_OK;
-        }
-        entry_to_config(tt->entries[index], ABQ_STRATEGY_TILED, x_bits, w_bits, is_signed, 0, cfg);
-        return ABQ_OK;
-    }
-    const KernelEntry &e = tm->entries[index];
-    entry_to_config(e, e.mi == 16 ? ABQ_STRATEGY_MFMA16 : ABQ_STRATEGY_MFMA32, x_bits, w_bits,
-                    is_signed, 0, cfg);
-    return ABQ_OK;
+    return index < n ? ABQ_OK : ABQ_ERR_INVALID_ARG;
 }
 
 // ---- GEMM --------------------------------------------------------------------------------
@@ -787,6 +813,36 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
     return ABQ_OK;
 }
 
+// Decode-sized GEMM with both operands K-tiled: the decode kernel built for that layout, if it exists for the
+// pair.  Variant by shape (measured on MI355X, W2A8, LLaMA-7B widths): sixteen waves with one weight load each
+// in flight while a compute unit holds at most two workgroups; with more tiles than that, eight waves with two
+// loads each (twice the workgroups fit a compute unit).
+static abq_status switch_to_decode_tiled(abq_gemm_state *st)
+{
+    const abq_tile_config &c = st->cfg;
+    const KernelTable *tdt = find_table(registry().decode_tiled, c.x_bits, c.w_bits, c.is_signed);
+    if (!tdt || tdt->count == 0)
+        return ABQ_ERR_UNSUPPORTED;
+    const int tiles = (st->N + 15) / 16;
+    const int want_wk = tiles > 512 ? 8 : 16, want_d = tiles > 512 ? 2 : 1;
+    int pick = -1;
+    for (int i = 0; i < tdt->count; ++i) {
+        const KernelEntry &e = tdt->entries[i];
+        if (e.tn == 1 && e.wk == want_wk && e.kb == (512 / c.w_bits) * want_d)
+            pick = i;
+    }
+    if (pick < 0)
+        return ABQ_ERR_UNSUPPORTED;
+    abq_tile_config cfg;
+    entry_to_config(tdt->entries[pick], ABQ_STRATEGY_DECODE_TILED, c.x_bits, c.w_bits, c.is_signed, 0, &cfg);
+    abq_gemm_state tmp = *st;
+    const abq_status rc = resolve(&cfg, c.x_bits, c.w_bits, c.is_signed, st->M, st->N, st->K, &tmp);
+    if (rc != ABQ_OK)
+        return rc;
+    *st = tmp;
+    return ABQ_OK;
+}
+
 // Moves a state with group scales onto the tiled kernel's group-scale variants.
 static abq_status pick_grouped_tiled(abq_gemm_state *state)
 {
@@ -1014,7 +1070,7 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
         if (st->variant < 0 || st->variant >= count)
             return ABQ_ERR_NOT_INITIALIZED;
         e = es[st->variant].launch(a, (hipStream_t)stream);
-    } else if (st->strategy == ABQ_STRATEGY_TILED) {
+    } else if (st->strategy == ABQ_STRATEGY_TILED || st->strategy == ABQ_STRATEGY_DECODE_TILED) {
         // operands still in the reference layout are converted into the caller's workspace
         const size_t xb = st->x_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->M, st->K, c.x_bits);
         const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, c.w_bits);
@@ -1035,7 +1091,12 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
                 return hip_status(e);
             a.W = reinterpret_cast<const uint32_t *>(ws + xb);
         }
-        const KernelTable *t = find_table(st->group_size ? reg.tiled_grouped : reg.tiled, c.x_bits, c.w_bits, c.is_signed);
+        if (st->strategy == ABQ_STRATEGY_DECODE_TILED && (st->group_size || st->act))
+            return ABQ_ERR_NOT_INITIALIZED; // plain and per-channel epilogues only
+        const KernelTable *t = find_table(st->strategy == ABQ_STRATEGY_DECODE_TILED ? reg.decode_tiled
+                                          : st->group_size                          ? reg.tiled_grouped
+                                                                                    : reg.tiled,
+                                          c.x_bits, c.w_bits, c.is_signed);
         if (!t || st->variant < 0 || st->variant >= t->count)
             return ABQ_ERR_NOT_INITIALIZED;
         e = t->entries[st->variant].launch(a, (hipStream_t)stream);
@@ -1127,7 +1188,14 @@ abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_l
         if (rc != ABQ_OK)
             return rc;
     }
-    if (any_tiled && st->strategy != ABQ_STRATEGY_TILED) {
+    // decode-sized M with both operands prepared: the decode kernel of that layout (plain and per-channel epilogues)
+    if (x_layout == ABQ_LAYOUT_TILED && w_layout == ABQ_LAYOUT_TILED && st->auto_chosen && st->M <= 16 && !st->group_size &&
+        !st->act && st->strategy != ABQ_STRATEGY_DECODE_TILED && switch_to_decode_tiled(st) == ABQ_OK) {
+        st->x_layout = x_layout;
+        st->w_layout = w_layout;
+        return ABQ_OK;
+    }
+    if (any_tiled && st->strategy != ABQ_STRATEGY_TILED && st->strategy != ABQ_STRATEGY_DECODE_TILED) {
         if (!st->auto_chosen)
             return ABQ_ERR_UNSUPPORTED;
         const abq_status rc = st->group_size ? pick_grouped_tiled(st) : switch_to_tiled(st);

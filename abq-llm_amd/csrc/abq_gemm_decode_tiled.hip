@@ -1,0 +1,324 @@
+// GEMM core for decode-sized M on prepared operands: both operands in the K-tiled field-packed layout
+// (abq_bits.h), widths of a single field (2, 4 or 8 bits).
+//
+// Replaces AqBMMAKernel::mainLoop + ::epilogue of the reference
+// (engine/mma_any/aq_bmma_kernel.h:109-271, :485-580) for one (x_bits, w_bits) pair per
+// translation unit: compile with -DABQ_Q=<x_bits> -DABQ_P=<w_bits>.
+//
+// A decode GEMM streams 4 to 11 MB of weights once; at 8 TB/s that takes 0.5 to 1.4 us, the same order as
+// one memory round trip and as a kernel launch, and every kernel starts with cold caches.  What decides
+// the time is therefore the length of the dependent chain from the first instruction to the last store and
+// the number of vector instructions on it (with sixteen waves on a compute unit an instruction of every
+// wave costs sixteen issue cycles per SIMD quad), not the byte count.  Hence:
+//   * prepared operands: a lane's 16-byte weight load is what it feeds the matrix core after a shift and a
+//     mask per four elements (no bit-matrix transpose), activations are int8-ready records (nothing to
+//     expand, no bytes more than the planes have);
+//   * a workgroup is T tiles of 16 weight rows over the whole K; wave w takes K steps w, w + NW, ...
+//     (a step = one 16-byte load per lane = 512 / P elements of K over the four lane groups);
+//   * the activations of the workgroup's rows go from global memory straight into LDS
+//     (global_load_lds_dwordx4: no registers, nothing to wait for before the weight loads are issued);
+//     chunk c of a row lands at c ^ (row & (Q - 1)) so that the sixteen rows a lane group reads hit
+//     different banks (the permutation is applied to the source address, the destination is linear);
+//   * the first D steps' weight loads of every wave are issued right behind them, all before the first
+//     wait; one counted wait (the activation loads are older than the weight loads) and one barrier
+//     later every wave reads its A operands with ds_read_b128;
+//   * the loads are issued from inline assembly: the compiler would sink plain loads below the barrier,
+//     next to their first use.  Values loaded that way are consumed through `landed()` after a counted
+//     wait, in the loop iteration that issued them (no register of theirs lives across the back edge,
+//     where a compiler-inserted copy could read it before it has landed);
+//   * per-wave partial tiles meet in LDS and are summed by the threads that store them (integer adds:
+//     any order gives the same bits).
+// K longer than NW * D steps runs further rounds of the same loop (their latency is exposed).
+#include "abq_kernels.h"
+
+#ifndef ABQ_Q
+#error "compile with -DABQ_Q=<x_bits> -DABQ_P=<w_bits>"
+#endif
+
+namespace abq {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+constexpr bool decode_tiled_width(int b) { return b == 2 || b == 4 || b == 8; }
+// single-field widths; an unsigned 8-bit operand would need the row-sum corrections of the other kernels
+constexpr bool decode_tiled_built(int q, int p, bool is_signed)
+{
+    return decode_tiled_width(q) && decode_tiled_width(p) && q >= p && (is_signed || (q < 8 && p < 8));
+}
+
+__device__ __forceinline__ void dt_load_to_lds(const void *src, unsigned lds_addr)
+{
+    // lane l of the wave lands at lds_addr + 16 * l.  (M0 cannot be named as clobbered: the compiler reserves it and
+    // sets it up itself right before each of its own uses, it keeps no value there across other instructions.)
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)
+                 : "memory");
+}
+
+__device__ __forceinline__ v4u dt_load16(const char *base, uint32_t off)
+{
+    v4u v;
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(v) : "v"(off), "s"(base) : "memory");
+    return v;
+}
+
+template <int N> __device__ __forceinline__ void dt_wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// the same with a count that is constant only after unrolling
+__device__ __forceinline__ void dt_wait_loads_n(int n)
+{
+    switch (n) {
+    case 0: dt_wait_loads<0>(); break;
+    case 1: dt_wait_loads<1>(); break;
+    case 2: dt_wait_loads<2>(); break;
+    case 3: dt_wait_loads<3>(); break;
+    case 4: dt_wait_loads<4>(); break;
+    case 5: dt_wait_loads<5>(); break;
+    case 6: dt_wait_loads<6>(); break;
+    default: dt_wait_loads<0>(); break;
+    }
+}
+// ties a register filled by dt_load16 to the wait in front of it: every use comes after
+__device__ __forceinline__ void dt_landed(v4u &v) { asm volatile("" : "+v"(v)); }
+
+// One 16-byte unit of a BITS-wide single-field record -> 8 / BITS MFMA operands of four dwords.
+// Signed: value * 2^(8 - BITS) (the field at the top of the byte); unsigned: the value.
+template <int BITS, bool SIGNED> __device__ __forceinline__ void dt_unpack(const v4u &u, v4i (&out)[8 / BITS])
+{
+    if (BITS == 8) {
+        out[0] = v4i{ (int)u[0], (int)u[1], (int)u[2], (int)u[3] };
+    } else if (BITS == 4) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint32_t a = u[2 * i], b = u[2 * i + 1];
+            if (SIGNED)
+                out[i] = v4i{ (int)((a << 4) & 0xF0F0F0F0u), (int)(a & 0xF0F0F0F0u), (int)((b << 4) & 0xF0F0F0F0u), (int)(b & 0xF0F0F0F0u) };
+            else
+                out[i] = v4i{ (int)(a & 0x0F0F0F0Fu), (int)((a >> 4) & 0x0F0F0F0Fu), (int)(b & 0x0F0F0F0Fu), (int)((b >> 4) & 0x0F0F0F0Fu) };
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w = u[i];
+            if (SIGNED)
+                out[i] = v4i{ (int)((w << 6) & 0xC0C0C0C0u), (int)((w << 4) & 0xC0C0C0C0u), (int)((w << 2) & 0xC0C0C0C0u), (int)(w & 0xC0C0C0C0u) };
+            else
+                out[i] = v4i{ (int)(w & 0x03030303u), (int)((w >> 2) & 0x03030303u), (int)((w >> 4) & 0x03030303u), (int)((w >> 6) & 0x03030303u) };
+        }
+    }
+}
+
+template <int Q, int P, bool SIGNED, int NW, int D, int T>
+__global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, int mrows)
+{
+    constexpr int NXL = Q / P;   // activation chunks (16 bytes) per weight unit
+    constexpr int NM = 8 / P;    // MFMAs per weight unit
+    constexpr int MX = 8 / Q;    // MFMAs per activation chunk
+    constexpr int NT = 64 * NW;
+    constexpr int QLOG = Q == 8 ? 3 : Q == 4 ? 2 : 1;
+    constexpr int XC = 6;        // activation wave loads per wave that are unrolled
+    extern __shared__ __align__(16) unsigned char smem[];
+    int *red = reinterpret_cast<int *>(smem);   // [NW][T][16][16]
+    unsigned char *xs = smem + NW * T * 1024;   // [kt][row][Q chunks], chunks permuted within a row
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int M = a.M, N = a.N;
+    const int KT = a.K >> 7;
+    const int U = KT * P;            // 16-byte units per weight row
+    const int S = (U + 3) >> 2;      // steps
+    const int tile0 = blockIdx.x * T;
+    const int m0 = blockIdx.y * mrows;
+    const int Mb = min(mrows, M - m0);
+    const char *Xt = reinterpret_cast<const char *>(a.X);
+    const char *Wt = reinterpret_cast<const char *>(a.W);
+    const unsigned xs_addr = (unsigned)(size_t)xs;
+    const int xchunks = KT * Mb * Q;
+
+    // ---- activations: LDS chunk p <- chunk p ^ ((p / Q) & (Q - 1)) of the workgroup's rows -----------
+    if (Mb == M) { // the rows of all K tiles are one contiguous block
+#pragma unroll
+        for (int i = 0; i < XC; ++i) {
+            const int pb = wid * 64 + i * NT; // wave-uniform
+            if (pb < xchunks) {
+                const int p = pb + lane;
+                const int src = min(p ^ ((p >> QLOG) & (Q - 1)), xchunks - 1);
+                dt_load_to_lds(Xt + (uint32_t)src * 16u, xs_addr + (unsigned)pb * 16u);
+            }
+        }
+        for (int pb = wid * 64 + XC * NT; pb < xchunks; pb += NT) {
+            const int p = pb + lane;
+            const int src = min(p ^ ((p >> QLOG) & (Q - 1)), xchunks - 1);
+            dt_load_to_lds(Xt + (uint32_t)src * 16u, xs_addr + (unsigned)pb * 16u);
+        }
+    } else { // several blocks of rows: a K tile's rows are Mb * Q chunks out of M * Q
+        const int per = Mb * Q;
+        for (int pb = wid * 64; pb < xchunks; pb += NT) {
+            const int p = min(pb + lane, xchunks - 1);
+            const int q = p ^ ((p >> QLOG) & (Q - 1));
+            const int kt = q / per, rem = q - kt * per;
+            dt_load_to_lds(Xt + ((size_t)(kt * M + m0) * Q + rem) * 16u, xs_addr + (unsigned)pb * 16u);
+        }
+    }
+
+    // ---- weights: byte offset of (lane, step s, tile t) = step_w(s) + woff[t] ------------------------
+    uint32_t woff[T], back;
+    {
+        const int n = min(tile0 * 16 + r, N - 1);
+        const uint32_t lane_w = P == 2 ? ((uint32_t)(g >> 1) * N + n) * 32u + (g & 1) * 16u : (uint32_t)n * (P * 16u) + g * 16u;
+        back = lane_w - (uint32_t)n * (P * 16u); // distance to the first unit of the step in the same row
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+            woff[t] = lane_w + ((T > 1 && (tile0 + t) * 16 + r < N) ? t * (16u * P * 16u) : 0u);
+    }
+    const uint32_t step_bytes = (uint32_t)N * 64u; // a step covers 4 units of every row: 64 bytes times N rows
+    auto step_w = [&](int s) -> uint32_t {
+        return P == 8 ? (uint32_t)(s >> 1) * (2u * step_bytes) + (s & 1) * 64u : (uint32_t)s * step_bytes;
+    };
+    const bool ragged = (U & 3) != 0; // the last step has fewer than four units
+
+    v4i acc[T][2];
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+        acc[t][0] = acc[t][1] = v4i{ 0, 0, 0, 0 };
+    const int ml = min(r, Mb - 1);
+
+    int round = 0;
+    do {
+        // this round's steps of the wave: wid + (round * D + d) * NW.  Every wave issues D * T loads (steps past
+        // the end repeat the last one), so that the waits below can count.
+        v4u wb[D][T];
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int s = min(wid + (round * D + d) * NW, S - 1);
+            const char *wp = Wt + step_w(s);
+            // lanes past the end of K (last step only) read the step's first unit of their row instead
+            const uint32_t bk = (ragged && s == S - 1 && 4 * s + g >= U) ? back : 0u;
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+                wb[d][t] = dt_load16(wp, woff[t] - bk);
+        }
+        if (round == 0) {
+            dt_wait_loads<D * T>(); // the activation loads are older than these
+            __syncthreads();
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int cs = wid + (round * D + d) * NW;
+            const bool have = cs < S; // wave-uniform
+            v4i av[NM];
+            if (have) {
+                const int u0 = (4 * cs + g) * NXL;           // first activation chunk of lane group and step along K
+                const int rowi = (u0 >> QLOG) * Mb + ml;      // row index in LDS: K tile * rows + row
+#pragma unroll
+                for (int i = 0; i < NXL; ++i) {
+                    const int part = ((u0 + i) & (Q - 1)) ^ (rowi & (Q - 1));
+                    const v4u xv = *reinterpret_cast<const v4u *>(xs + ((uint32_t)rowi * Q + part) * 16u);
+                    v4i tt[MX];
+                    dt_unpack<Q, SIGNED>(xv, tt);
+#pragma unroll
+                    for (int k = 0; k < MX; ++k)
+                        av[i * MX + k] = tt[k];
+                }
+            }
+            // Waited for and marked as landed on every path: a register with a load still in flight must not
+            // look free to the compiler (it would reuse it, and the late data would land on the new value).
+            dt_wait_loads_n((D - 1 - d) * T);
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+                dt_landed(wb[d][t]);
+            if (have) {
+                const bool ok = 4 * cs + g < U;
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    const v4u wv = ok ? wb[d][t] : v4u{ 0u, 0u, 0u, 0u };
+                    v4i bv[NM];
+                    dt_unpack<P, SIGNED>(wv, bv);
+#pragma unroll
+                    for (int i = 0; i < NM; ++i)
+                        acc[t][i & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[i], bv[i], acc[t][i & 1], 0, 0, 0);
+                }
+            }
+        }
+        ++round;
+    } while (wid + round * D * NW < S);
+
+    // ---- the waves' partial tiles meet in LDS ----------------------------------------------------------
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (4 * g + e < Mb)
+                red[((wid * T + t) * 16 + 4 * g + e) * 16 + r] = acc[t][0][e] + acc[t][1][e];
+    __syncthreads();
+    for (int o = tid; o < T * 256; o += NT) {
+        const int t = o >> 8, rem = o & 255;
+        const int n = (tile0 + t) * 16 + (rem & 15);
+        if ((rem >> 4) < Mb && n < N) {
+            int part[NW];
+#pragma unroll
+            for (int w = 0; w < NW; ++w)
+                part[w] = red[(w * T + t) * 256 + rem];
+            int v = 0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w)
+                v += part[w];
+            if (SIGNED)
+                v >>= 16 - Q - P; // both operands were fed at the top of the byte
+            store_result(a, m0 + (rem >> 4), n, v);
+        }
+    }
+}
+
+template <int Q, int P, bool SIGNED, int NW, int D, int T>
+static hipError_t launch_decode_tiled(const GemmArgs &a, hipStream_t stream)
+{
+    const int mrows = decode_tiled_rows(NW, T, a.M, a.K, Q);
+    if (mrows == 0 || (size_t)a.N * a.K * P / 8 >= (1ull << 32) || (size_t)a.M * a.K * Q / 8 >= (1ull << 32))
+        return hipErrorInvalidValue;
+    const size_t lds = decode_tiled_lds(NW, T, mrows, a.K, Q);
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled<Q, P, SIGNED, NW, D, T>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr != hipSuccess)
+        return attr;
+    const int tiles = (a.N + 15) / 16;
+    const dim3 grid((tiles + T - 1) / T, (a.M + mrows - 1) / mrows);
+    hipLaunchKernelGGL((gemm_decode_tiled<Q, P, SIGNED, NW, D, T>), grid, dim3(64 * NW), lds, stream, a, mrows);
+    return hipGetLastError();
+}
+
+// Native tile space of this kernel: (waves, weight loads in flight per wave, tiles per workgroup).  Entries name
+// MFMA 16x16x64 with NSTAGE = 6; wk = waves, tn = tiles, kb = K elements a wave has in flight (D steps).
+#define ABQ_DT_VARIANTS(V) V(16, 1, 1) V(16, 3, 1) V(8, 2, 1) V(16, 1, 3) V(8, 1, 2)
+
+#define ABQ_DT_ENTRY_T(NW, D, T) { 16, 1, T, 1, 1, NW, 6, &launch_decode_tiled<ABQ_Q, ABQ_P, true, NW, D, T>, (512 / ABQ_P) * D },
+#define ABQ_DT_ENTRY_F(NW, D, T) { 16, 1, T, 1, 1, NW, 6, &launch_decode_tiled<ABQ_Q, ABQ_P, false, NW, D, T>, (512 / ABQ_P) * D },
+
+#if (ABQ_Q == 2 || ABQ_Q == 4 || ABQ_Q == 8) && (ABQ_P == 2 || ABQ_P == 4 || ABQ_P == 8)
+static const KernelEntry kSigned[] = { ABQ_DT_VARIANTS(ABQ_DT_ENTRY_T) };
+#if ABQ_Q < 8
+static const KernelEntry kUnsigned[] = { ABQ_DT_VARIANTS(ABQ_DT_ENTRY_F) };
+#define ABQ_DT_NUNSIGNED ((int)(sizeof(kUnsigned) / sizeof(kUnsigned[0])))
+#else
+static const KernelEntry *const kUnsigned = nullptr;
+#define ABQ_DT_NUNSIGNED 0
+#endif
+#define ABQ_DT_NSIGNED ((int)(sizeof(kSigned) / sizeof(kSigned[0])))
+#else
+static const KernelEntry *const kSigned = nullptr;
+static const KernelEntry *const kUnsigned = nullptr;
+#define ABQ_DT_NSIGNED 0
+#define ABQ_DT_NUNSIGNED 0
+#endif
+
+#define ABQ_CAT_(a, b, c, d) a##b##c##d
+#define ABQ_CAT(a, b, c, d) ABQ_CAT_(a, b, c, d)
+
+void ABQ_CAT(abq_decode_tiled_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)
+{
+    out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSigned, ABQ_DT_NSIGNED };
+    out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, kUnsigned, ABQ_DT_NUNSIGNED };
+}
+
+} // namespace abq

@@ -65,6 +65,21 @@ inline size_t decode_grouped_lds(int M, int K, int group_size)
     return need <= 160 * 1024 ? need : 0;
 }
 
+// Decode kernel on K-tiled operands (abq_gemm_decode_tiled.hip): LDS of one workgroup = per-wave partial tiles,
+// then the activations of its rows (one K tile of slack for the ragged last step, whole wave loads), and the
+// rows per workgroup (up to 16) that keep it within a compute unit's LDS; 0 if not even one row fits.
+inline size_t decode_tiled_lds(int nw, int t, int mrows, int K, int q)
+{
+    return (size_t)nw * t * 1024 + (size_t)mrows * (K / 128 + 1) * q * 16 + 1024;
+}
+inline int decode_tiled_rows(int nw, int t, int M, int K, int q)
+{
+    int mrows = M < 16 ? M : 16;
+    while (mrows > 1 && decode_tiled_lds(nw, t, mrows, K, q) > 150 * 1024)
+        mrows = (mrows + 1) / 2;
+    return decode_tiled_lds(nw, t, mrows, K, q) <= 160 * 1024 ? mrows : 0;
+}
+
 // Workgroup id -> output tile.  XCD x = id % 8 owns n blocks [x * npx, (x + 1) * npx); inside an XCD the
 // workgroups run through groups of four m blocks, M fastest inside a group, then N, then the next group:
 // the 32 or 64 workgroups an XCD runs at a time then cover a patch of 4 x 8 (or 4 x 16) tiles, so every

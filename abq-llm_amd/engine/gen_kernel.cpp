@@ -5,8 +5,8 @@
 // prints one "AQ_INSTANTIATE_FUN(AqBMMA, ...);" line per tile configuration, preceded by a
 // comment line per tile shape.
 //
-//   --space gfx950 (default)  the native MI355X space: VALU-popcount tiles (MMA 1x1x128) and
-//                             int8-MFMA tiles (MMA 16x16x64 and 32x32x32), bounded by what one
+//   --space gfx950 (default)  the native MI355X space: VALU-popcount tiles (MMA 1x1x128), int8-MFMA
+//                             tiles (MMA 16x16x64 and 32x32x32) and FP6-MFMA tiles, bounded by what one
 //                             CDNA4 compute unit offers (wave64, 512 VGPRs per lane at one wave
 //                             per SIMD, 160 KiB LDS, 1024 threads per workgroup).
 //   --space sm80              the reference's own rules, restated; its output is compared with
@@ -211,6 +211,17 @@ std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits, bool is_signed)
         const int fp6[][4] = { { 2, 2, 4, 2 }, { 4, 2, 2, 2 }, { 2, 2, 2, 2 }, { 2, 1, 2, 2 }, { 1, 1, 2, 2 } };
         for (const auto &t : fp6)
             out.push_back(Tile{ 32 * t[0] * t[2], 32 * t[1] * t[3], 128, 32 * t[0], 32 * t[1], 128, 32, 32, 64, t[2], t[3], { 5 } });
+    }
+    // Decode kernel on K-tiled operands (NSTAGE = 6): single-field widths, no unsigned 8-bit operand;
+    // { waves, weight loads in flight per wave, 16-row tiles per workgroup }; a load covers 512 / W_BITS elements of K
+    {
+        const bool field = (x_bits == 2 || x_bits == 4 || x_bits == 8) && (w_bits == 2 || w_bits == 4 || w_bits == 8);
+        if (field && x_bits >= w_bits && (is_signed || x_bits < 8)) {
+            const int dt[][3] = { { 16, 1, 1 }, { 16, 3, 1 }, { 8, 2, 1 }, { 16, 1, 3 }, { 8, 1, 2 } };
+            const int stepk = 512 / w_bits;
+            for (const auto &v : dt)
+                out.push_back(Tile{ 16, 16 * v[2], stepk * v[1] * v[0], 16, 16 * v[2], stepk * v[1], 16, 16, 64, 1, v[0], { 6 } });
+        }
     }
     return out;
 }

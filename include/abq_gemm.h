@@ -80,7 +80,8 @@ abq_status abq_pack_f16(const void *in_f16, const float *scale_dev, uint32_t *pl
  *   1 x 1 x 128   VALU AND + popcount, K along the lanes, wavefront reduction
  *   16 x 16 x 64  planes re-assembled to int8 in registers, v_mfma_i32_16x16x64_i8
  *                 (NSTAGE = 3: decode kernel, activations staged in LDS; NSTAGE = 2: every wave
- *                 expands its own activations)
+ *                 expands its own activations; NSTAGE = 6: decode kernel on K-tiled operands,
+ *                 BN / 16 weight tiles per workgroup, WK = K elements a wave keeps in flight)
  *   32 x 32 x 32  the same feeding v_mfma_i32_32x32x32_i8
  * Any other triple (the reference's 8x8x128, 16x8x128, 16x8x256 tensor-core shapes) asks the
  * library to choose strategy and tile itself from (bits, M, N, K).
@@ -103,9 +104,14 @@ typedef enum abq_strategy {
                                  into LDS, persistent grid; tile tuples with NSTAGE = 3       */
     ABQ_STRATEGY_TILED = 6,   /* int8 MFMA 32x32x32, LDS-staged, operands in the K-tiled plane
                                  layout (see abq_relayout_planes); tile tuples with NSTAGE = 4 */
-    ABQ_STRATEGY_FP6 = 7      /* FP6 (E2M3) MFMA 32x32x64 at twice the int8 rate, exact for operands
+    ABQ_STRATEGY_FP6 = 7,     /* FP6 (E2M3) MFMA 32x32x64 at twice the int8 rate, exact for operands
                                  of at most 4 bits unsigned / 5 bits signed (see
                                  abq_relayout_planes_fp6); tile tuples with NSTAGE = 5, MMA 32x32x64 */
+    ABQ_STRATEGY_DECODE_TILED = 8 /* int8 MFMA 16x16x64 for decode-sized M on operands that are both in the
+                                 K-tiled layout (widths 2, 4 or 8 bits; no unsigned 8-bit operand):
+                                 nothing is expanded or transposed inside the kernel; tile tuples with
+                                 NSTAGE = 6.  A state with M <= 16 whose operands are both declared
+                                 ABQ_LAYOUT_TILED moves here by itself */
 } abq_strategy;
 
 /* Parses "AqBMMA_8x2xtrue_1x48x512_8x24x128_8x8x128_4" (an optional _InitFn/_ExecFn suffix is

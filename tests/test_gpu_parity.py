@@ -28,7 +28,7 @@ def planes_dev(planes):
 def run_cfg(abq, xd, wd, signed, cfg=None, **kw):
     """Runs one configuration; kernels on the K-tiled layout get the workspace they ask for."""
     g = abq.Gemm(xd, wd, signed, cfg=cfg, **kw)
-    if g.strategy in ("tiled", "fp6") and g.workspace_bytes and "workspace" not in kw:
+    if g.strategy in ("tiled", "fp6", "decode_tiled") and g.workspace_bytes and "workspace" not in kw:
         ws = torch.empty(g.workspace_bytes, dtype=torch.uint8, device="cuda")
         g = abq.Gemm(xd, wd, signed, cfg=cfg, workspace=ws, **kw)
     return g.run()
@@ -416,6 +416,61 @@ def test_decode_kernel_k_chunking_and_many_tiles(abq, oracle):
             assert np.array_equal(got, want), (abq.format_kernel_name(cfg), M, N, K)
 
 
+DECODE_TILED_PAIRS = [(2, 2), (4, 2), (8, 2), (4, 4), (8, 4), (8, 8)]
+
+
+@pytest.mark.parametrize("q,p", DECODE_TILED_PAIRS)
+@pytest.mark.parametrize("signed", [True, False])
+def test_decode_on_prepared_operands(abq, oracle, q, p, signed):
+    """Decode-sized GEMM with both operands K-tiled: the library moves to the decode kernel of that layout by
+    itself (no workspace, one launch); every tile tuple of that kernel on ragged shapes: partial tiles of N, an odd
+    number of K tiles (half-filled last step), M past 16 (several row blocks), long K (rows per workgroup limited
+    by the LDS), more steps than the waves hold in flight."""
+    built = signed or q < 8
+    rng = np.random.default_rng(500 + 10 * q + p + int(signed))
+    shapes = [(1, 64, 128), (1, 4096, 4096), (3, 37, 384), (4, 200, 1408), (8, 130, 1152), (8, 64, 11008), (13, 72, 4096),
+              (16, 100, 13824), (16, 48, 2048), (17, 64, 512), (40, 96, 640), (2, 300, 24576)]
+    for (M, N, K) in shapes:
+        x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+        xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
+        xt, wt = abq.relayout_planes(xd), abq.relayout_planes(wd)
+        want = oracle.np_gemm(x, w)
+        g = abq.Gemm(xt, wt, signed, x_tiled=True, w_tiled=True)
+        assert g.strategy == ("decode_tiled" if built and M <= 16 else "tiled"), (g.strategy, M, N, K)
+        assert g.workspace_bytes == 0
+        assert np.array_equal(g.run().cpu().numpy(), want), (g.config_name, M, N, K)
+        for cfg in abq.native_configs(q, p, signed):
+            if cfg.nstage != 6:
+                continue
+            out = torch.full((M, N), -12345, dtype=torch.int32, device="cuda")
+            got = abq.Gemm(xt, wt, signed, cfg=cfg, out=out, x_tiled=True, w_tiled=True).run().cpu().numpy()
+            assert np.array_equal(got, want), (abq.format_kernel_name(cfg), M, N, K)
+    assert built == any(c.nstage == 6 for c in abq.native_configs(q, p, signed))
+
+
+def test_decode_on_prepared_operands_epilogues(abq, oracle):
+    """The fp16 epilogues of the decode kernel on K-tiled operands: the reference's per-tensor formula bit for bit,
+    per-token x per-channel scales within 1e-2 relative."""
+    rng = np.random.default_rng(77)
+    M, N, K = 8, 200, 1152
+    x, w = rand_vals(rng, M, K, 8, True), rand_vals(rng, N, K, 2, True)
+    xp, wp = oracle.pack_i32(x, 8), oracle.pack_i32(w, 2)
+    xt, wt = abq.relayout_planes(planes_dev(xp)), abq.relayout_planes(planes_dev(wp))
+    acc = oracle.np_gemm(x, w)
+    scale = torch.tensor([0.0123], dtype=torch.float16, device="cuda")
+    g = abq.Gemm(xt, wt, True, out_kind=abq.OUT_F16_TENSOR, c_scale=scale, x_tiled=True, w_tiled=True)
+    assert g.strategy == "decode_tiled"
+    got = g.run().cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), oracle.epilogue_f16(acc, np.float16(0.0123)).view(np.uint16))
+    xs = (rng.random(M) * 0.05 + 0.01).astype(np.float32)
+    ws = (rng.random(N) * 0.01 + 0.001).astype(np.float32)
+    g = abq.Gemm(xt, wt, True, out_kind=abq.OUT_F16_SCALED, x_scale=dev(xs), w_scale=dev(ws), x_tiled=True, w_tiled=True)
+    assert g.strategy == "decode_tiled"
+    got = g.run().cpu().numpy().astype(np.float64)
+    want = acc.astype(np.float64) * xs[:, None].astype(np.float64) * ws[None, :].astype(np.float64)
+    assert np.all(np.abs(got - want) <= 1e-2 * np.abs(want) + 1e-6)  # 1e-2 relative (fp16 rounding is 2^-11)
+
+
 def test_gemm_generic_bit_widths(abq, oracle):
     """Bit pairs without a specialised kernel (the W1A1 / W1A4 / W1A8 / W1A16 / W2A16 samples)."""
     rng = np.random.default_rng(5)
@@ -507,6 +562,10 @@ def test_config1_w2a8_decode_full_size(abq, oracle, N, K):
                 continue
             got = run_cfg(abq, xd, wd, True, cfg=cfg).cpu().numpy()
             assert np.array_equal(got, want), (M, cfg)
+        # prepared operands (weights converted once, activations as the quantising kernel hands them over)
+        g = abq.Gemm(abq.relayout_planes(xd), abq.relayout_planes(wd), True, x_tiled=True, w_tiled=True)
+        assert g.strategy == "decode_tiled"
+        assert np.array_equal(g.run().cpu().numpy(), want), (M, g.config_name)
 
 
 @pytest.mark.parametrize("q,p,signed", [(4, 4, True), (4, 4, False), (8, 8, True), (8, 8, False)])
