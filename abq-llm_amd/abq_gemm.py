@@ -35,6 +35,7 @@ EXPORTED = [
     "abq_planes_bytes", "abq_relayout_planes", "abq_gemm_set_operand_layout", "abq_gemm_workspace_bytes",
     "abq_gemm_set_workspace", "abq_fp6_bytes", "abq_fp6_eligible", "abq_relayout_planes_fp6",
     "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16", "abq_gemm_set_activation",
+    "abq_probe_launch",
 ]
 
 
@@ -125,6 +126,7 @@ def lib():
         L.abq_gemm_set_activation.argtypes = [ctypes.POINTER(GemmState), ci]
         L.abq_weight_zero_term.argtypes = [vp, ci, ci, ci, ci, vp, vp, ci, vp, vp]
         L.abq_quant_pack_f16.argtypes = [vp, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, vp]
+        L.abq_probe_launch.argtypes = [ci, vp, ctypes.c_size_t, vp]
         _lib = L
     return _lib
 

@@ -3,7 +3,7 @@
 // :21-160).
 //
 //     test_any_mma M N K X_BITS W_BITS SIGNED [--repeat R] [--warmup W] [--rotate-mib MiB]
-//                  [--stream] [--only SUBSTR] [--seed S]
+//                  [--stream] [--only SUBSTR] [--seed S] [--read-floor]
 //
 // Like the reference it builds random operands, packs them on the GPU, computes the expected
 // result on the CPU, then runs EVERY tile configuration of the bit combination, checks each
@@ -24,6 +24,12 @@
 //    (HBM 8 TB/s on the packed bytes, int8 MFMA 5 POP/s on 2*M*N*K);
 //  * kernels on the K-tiled layout (NSTAGE 4) get weights converted once before the timed loop
 //    (part of weight preparation, like packing) and convert the activations inside every call;
+//    the decode kernel of that layout (NSTAGE 6) gets the activations K-tiled as well, which is how
+//    the quantising kernel hands them over, and for M <= 16 a last line times the library's own
+//    choice on such operands;
+//  * --read-floor adds two lines timed the same way (same rotation, same graph replay): a kernel
+//    that does nothing, and one that reads the packed weights once with 16-byte loads and computes
+//    nothing: the floor of one launch over that many bytes;
 //  * inputs come from std::mt19937_64 with a fixed seed instead of unseeded rand().
 #include <hip/hip_runtime.h>
 
@@ -91,12 +97,14 @@ int main(int argc, char **argv)
     const int x_bits = std::atoi(argv[4]), w_bits = std::atoi(argv[5]);
     const bool is_signed = std::atoi(argv[6]) == 1;
     int repeat = 1000, warmup = 10, rotate_mib = 512;
-    bool use_graph = true;
+    bool use_graph = true, read_floor = false;
     unsigned long seed = 0;
     std::string only;
     for (int i = 7; i < argc; ++i) {
         if (!std::strcmp(argv[i], "--stream"))
             use_graph = false;
+        else if (!std::strcmp(argv[i], "--read-floor"))
+            read_floor = true;
         else if (i + 1 < argc && !std::strcmp(argv[i], "--repeat"))
             repeat = std::atoi(argv[++i]);
         else if (i + 1 < argc && !std::strcmp(argv[i], "--warmup"))
@@ -169,6 +177,15 @@ int main(int argc, char **argv)
         HIP_OK(hipMemcpyAsync((char *)d_wt + b * wp_bytes, d_wt, wp_bytes, hipMemcpyDeviceToDevice, stream));
     HIP_OK(hipStreamSynchronize(stream));
 
+    // the decode kernel on K-tiled operands takes the activations in that layout too
+    uint32_t *d_xt;
+    HIP_OK(hipMalloc(&d_xt, xp_words * 4));
+    if (abq_relayout_planes(d_xp, d_xt, M, K, x_bits, stream) != ABQ_OK) {
+        std::printf("abq_relayout_planes failed (hip error %d)\n", abq_last_hip_error());
+        return -1;
+    }
+    HIP_OK(hipStreamSynchronize(stream));
+
     // The FP6 kernels (NSTAGE 5) read their own record format: 96 bytes per row and K tile.
     const bool fp6_ok = abq_fp6_eligible(x_bits, w_bits, is_signed, K) != 0;
     const size_t wf_bytes = abq_fp6_bytes(N, K);
@@ -215,10 +232,12 @@ int main(int argc, char **argv)
     char config_str[32];
     std::snprintf(config_str, sizeof config_str, "W%dA%d %s", w_bits, x_bits, is_signed ? "int" : "uint");
 
-    auto run_one = [&](const abq_tile_config *cfg, Timing &t, abq_gemm_state &st0) {
+    auto run_one = [&](const abq_tile_config *cfg, Timing &t, abq_gemm_state &st0, bool prepared = false) {
         std::vector<abq_gemm_state> states(nbuf);
-        // tiled tiles (NSTAGE 4) and the library's own choice for M > 16 run on prepared weights
-        const bool tiled = cfg ? cfg->nstage == 4 : M > 16;
+        // tiled tiles (NSTAGE 4) and the library's own choice for M > 16 run on prepared weights;
+        // NSTAGE 6 and the `prepared` default on prepared weights and activations
+        const bool both = prepared || (cfg && cfg->nstage == 6);
+        const bool tiled = both || (cfg ? cfg->nstage == 4 : M > 16);
         const bool fp6 = cfg && cfg->nstage == 5;
         if (fp6 && !fp6_ok) {
             t.status = -1;
@@ -227,10 +246,10 @@ int main(int argc, char **argv)
         for (size_t b = 0; b < nbuf; ++b) {
             const char *wbase = fp6 ? (const char *)d_wf + b * wf_bytes
                                     : (tiled ? (const char *)d_wt : (const char *)d_wp) + b * wp_bytes;
-            abq_status s = abq_gemm_init(cfg, x_bits, w_bits, is_signed, d_xp, (const uint32_t *)wbase,
+            abq_status s = abq_gemm_init(cfg, x_bits, w_bits, is_signed, both ? d_xt : d_xp, (const uint32_t *)wbase,
                                          M, N, K, d_out, nullptr, 0, ABQ_OUT_I32, &states[b]);
             if (s == ABQ_OK && tiled)
-                s = abq_gemm_set_operand_layout(&states[b], ABQ_LAYOUT_PLANES, ABQ_LAYOUT_TILED);
+                s = abq_gemm_set_operand_layout(&states[b], both ? ABQ_LAYOUT_TILED : ABQ_LAYOUT_PLANES, ABQ_LAYOUT_TILED);
             if (s == ABQ_OK && fp6)
                 s = abq_gemm_set_operand_layout(&states[b], ABQ_LAYOUT_PLANES, ABQ_LAYOUT_FP6);
             if (s == ABQ_OK && (tiled || fp6))
@@ -282,12 +301,16 @@ int main(int argc, char **argv)
     double best_tops = 0;
     std::string best;
     const int ncfg = abq_native_config_count(x_bits, w_bits, is_signed);
-    for (int i = 0; i <= ncfg; ++i) {
+    const int nlines = ncfg + (M <= 16 ? 2 : 1); // + the library's choice (+ its choice on prepared operands)
+    for (int i = 0; i < nlines; ++i) {
         abq_tile_config cfg;
-        const bool library_default = i == ncfg;
+        const bool library_default = i >= ncfg;
+        const bool prepared = i == ncfg + 1;
         if (!library_default && abq_native_config_get(x_bits, w_bits, is_signed, i, &cfg) != ABQ_OK)
             continue;
         char name[160] = "library default";
+        if (prepared)
+            std::snprintf(name, sizeof name, "library default, prepared operands");
         if (!library_default)
             abq_format_kernel_name(&cfg, 0, name, sizeof name);
         if (!only.empty() && std::string(name).find(only) == std::string::npos)
@@ -295,7 +318,7 @@ int main(int argc, char **argv)
         Timing t;
         abq_gemm_state st;
         std::memset(&st, 0, sizeof st);
-        run_one(library_default ? nullptr : &cfg, t, st);
+        run_one(library_default ? nullptr : &cfg, t, st, prepared);
         const abq_tile_config &c = st.cfg;
         const double tops = t.status == 0 ? ops / (t.exec_us * 1e-6) / 1e12 : 0;
         std::printf("gfx950 %s %d %d %d %d %d %d %d %d %d %d ", config_str, c.block_m, c.block_n, c.block_k, c.warp_m,
@@ -303,7 +326,7 @@ int main(int argc, char **argv)
         std::printf("packing %f (us) exec %f (us) %f TOPS | %f B-TOPS | %s | %.1f%% HBM %.1f%% MFMA%s\n", t.pack_us,
                     t.exec_us, tops, tops * x_bits * w_bits, t.status == 0 ? "PASSED" : t.status == -1 ? "ERROR" : "FAILED",
                     t.status == 0 ? 100.0 * alg_bytes / (t.exec_us * 1e-6) / 8e12 : 0.0, 100.0 * tops / 5000.0,
-                    library_default ? " | library default" : "");
+                    prepared ? " | library default, prepared operands" : library_default ? " | library default" : "");
         if (t.status == 0 && !library_default && tops > best_tops) {
             best_tops = tops;
             char buf[128];
@@ -315,12 +338,51 @@ int main(int argc, char **argv)
     }
     std::printf("The best kernel config is %s with %f TOPS\n", best.c_str(), best_tops);
 
+    if (read_floor) {
+        auto time_probe = [&](int kind) {
+            auto body = [&](int count) {
+                for (int i = 0; i < count; ++i)
+                    abq_probe_launch(kind, (const char *)d_wp + (size_t)(i % nbuf) * wp_bytes, wp_bytes, stream);
+            };
+            body(warmup);
+            HIP_OK(hipStreamSynchronize(stream));
+            float ms = 0;
+            hipGraph_t g;
+            hipGraphExec_t ge;
+            if (use_graph) {
+                HIP_OK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+                body(repeat);
+                HIP_OK(hipStreamEndCapture(stream, &g));
+                HIP_OK(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0));
+                HIP_OK(hipGraphLaunch(ge, stream));
+                HIP_OK(hipStreamSynchronize(stream));
+            }
+            HIP_OK(hipEventRecord(e0, stream));
+            if (use_graph)
+                HIP_OK(hipGraphLaunch(ge, stream));
+            else
+                body(repeat);
+            HIP_OK(hipEventRecord(e1, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+            if (use_graph) {
+                HIP_OK(hipGraphExecDestroy(ge));
+                HIP_OK(hipGraphDestroy(g));
+            }
+            return ms * 1e3f / repeat;
+        };
+        const float empty_us = time_probe(ABQ_PROBE_EMPTY), read_us = time_probe(ABQ_PROBE_READ);
+        std::printf("floor: empty kernel %f (us) | read of the %zu packed weight bytes, 16-byte loads, no compute %f (us) = %.1f%% HBM\n",
+                    empty_us, wp_bytes, read_us, 100.0 * (double)wp_bytes / (read_us * 1e-6) / 8e12);
+    }
+
     (void)hipFree(d_x);
     (void)hipFree(d_w);
     (void)hipFree(d_xp);
     (void)hipFree(d_wp);
     (void)hipFree(d_out);
     (void)hipFree(d_wt);
+    (void)hipFree(d_xt);
     if (d_wf)
         (void)hipFree(d_wf);
     (void)hipFree(d_ws);

@@ -319,6 +319,16 @@ abq_status abq_gemm_exec(const abq_gemm_state *state, void *stream);
 abq_status abq_gemm_launch(const abq_tile_config *cfg, const uint32_t *X, const uint32_t *W,
                            const void *C, int32_t *D, int bias, int M, int N, int K, void *stream);
 
+/* Measurement aid (no counterpart in the reference): launches a kernel that does nothing
+ * (ABQ_PROBE_EMPTY; buf and bytes ignored) or one that reads `bytes` of `buf` once with 16-byte loads and
+ * computes nothing (ABQ_PROBE_READ).  The harness times them the way it times the GEMMs: the floor a
+ * decode GEMM, which is one launch over a few MB of weights, can be compared with. */
+typedef enum abq_probe_kind {
+    ABQ_PROBE_EMPTY = 0,
+    ABQ_PROBE_READ = 1
+} abq_probe_kind;
+abq_status abq_probe_launch(int kind, const void *buf, size_t bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
