@@ -824,7 +824,10 @@ static abq_status switch_to_decode_tiled(abq_gemm_state *st)
     if (!tdt || tdt->count == 0)
         return ABQ_ERR_UNSUPPORTED;
     const int tiles = (st->N + 15) / 16;
-    const int want_wk = tiles > 512 ? 8 : 16, want_d = tiles > 512 ? 2 : 1;
+    const int steps = (st->K / 128 * c.w_bits + 3) / 4;
+    // long K with one or two rows: three loads per wave in flight instead of three rounds of one (4.4 against 4.8 us
+    // at K = 11008); with more rows the activation traffic comes first and one load at a time is as fast
+    const int want_wk = tiles > 512 ? 8 : 16, want_d = tiles > 512 ? 2 : (steps > 32 && st->M <= 2) ? 3 : 1;
     int pick = -1;
     for (int i = 0; i < tdt->count; ++i) {
         const KernelEntry &e = tdt->entries[i];
