@@ -35,7 +35,7 @@ EXPORTED = [
     "abq_planes_bytes", "abq_relayout_planes", "abq_gemm_set_operand_layout", "abq_gemm_workspace_bytes",
     "abq_gemm_set_workspace", "abq_fp6_bytes", "abq_fp6_eligible", "abq_relayout_planes_fp6",
     "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16", "abq_gemm_set_activation",
-    "abq_probe_launch",
+    "abq_probe_launch", "abq_gemm_exec_static",
 ]
 
 
@@ -110,6 +110,7 @@ def lib():
                                     ctypes.POINTER(GemmState)]
         L.abq_gemm_set_scales.argtypes = [ctypes.POINTER(GemmState), vp, vp, ci]
         L.abq_gemm_exec.argtypes = [ctypes.POINTER(GemmState), vp]
+        L.abq_gemm_exec_static.argtypes = [ctypes.POINTER(GemmState), vp]
         L.abq_gemm_launch.argtypes = [ctypes.POINTER(TileConfig), vp, vp, vp, vp, ci, ci, ci, ci, vp]
         L.abq_planes_bytes.argtypes = [ci, ci, ci]
         L.abq_planes_bytes.restype = ctypes.c_size_t
@@ -343,6 +344,11 @@ class Gemm:
 
     def run(self, stream=None):
         _check(lib().abq_gemm_exec(ctypes.byref(self.state), _stream_ptr(stream)), "abq_gemm_exec")
+        return self.out
+
+    def run_static(self, stream=None):
+        """The same through the entry point that allocates nothing (conversions into the library's static array)."""
+        _check(lib().abq_gemm_exec_static(ctypes.byref(self.state), _stream_ptr(stream)), "abq_gemm_exec_static")
         return self.out
 
 

@@ -7,6 +7,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "abq_kernels.h"
 
 namespace abq {
@@ -1013,6 +1015,65 @@ abq_status abq_quant_pack_f16(const void *x_f16, int rows, int k, int bits, int 
         return ABQ_ERR_UNSUPPORTED;
     return hip_status(launch_quant_pack_rows(x_f16, planes, scale, zero, group_sums, rows, k, bits, symmetric ? 1 : 0,
                                              group_sums ? group_size : 128, layout, (hipStream_t)stream));
+}
+
+// ---- entry point that allocates nothing ----------------------------------------------------
+//
+// The layout conversions of abq_gemm_exec write into a workspace the caller brings.  Callers that cannot
+// allocate one (code under HIP graph capture, serving loops, harnesses that forbid it) use
+// abq_gemm_exec_static instead: the same launches with the workspace in a file-scope device array.  Every
+// device the library runs on holds its own copy of the array, at its own address, until the process ends.
+static __device__ __align__(256) unsigned char g_static_scratch[ABQ_STATIC_WORKSPACE_BYTES];
+
+static const int kMaxDevices = 64;
+static void *g_static_scratch_ptr[kMaxDevices]; // device address of the array, per device; null until asked for
+static std::mutex g_static_scratch_mutex;
+
+// Device address of the current device's copy of the array (the array's name is only a host-side handle).
+static abq_status static_scratch_address(void **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return hip_status(e);
+    if (dev < 0 || dev >= kMaxDevices)
+        return ABQ_ERR_TOO_LARGE;
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (!g_static_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch));
+        if (e != hipSuccess)
+            return hip_status(e);
+        if (!ptr)
+            return ABQ_ERR_LAUNCH;
+        g_static_scratch_ptr[dev] = ptr;
+    }
+    *out = g_static_scratch_ptr[dev];
+    return ABQ_OK;
+}
+
+abq_status abq_gemm_exec_static(const abq_gemm_state *st, void *stream)
+{
+    if (!st || !st->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    // only the strategies on prepared layouts convert anything
+    const bool converts = st->strategy == ABQ_STRATEGY_TILED || st->strategy == ABQ_STRATEGY_FP6 || st->strategy == ABQ_STRATEGY_DECODE_TILED;
+    const size_t need = converts ? abq_gemm_workspace_bytes(st) : 0;
+    if (need > (size_t)ABQ_STATIC_WORKSPACE_BYTES) {
+        fprintf(stderr, "[ABQ][Error] abq_gemm_exec_static: this GEMM converts %zu bytes of operands, the static workspace holds %zu\n",
+                need, (size_t)ABQ_STATIC_WORKSPACE_BYTES);
+        return ABQ_ERR_TOO_LARGE;
+    }
+    abq_gemm_state local = *st;
+    if (need) {
+        void *ptr = nullptr;
+        const abq_status rc = static_scratch_address(&ptr);
+        if (rc != ABQ_OK)
+            return rc;
+        local.workspace = ptr;
+        local.workspace_bytes = ABQ_STATIC_WORKSPACE_BYTES;
+    }
+    return abq_gemm_exec(&local, stream);
 }
 
 abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)

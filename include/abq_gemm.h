@@ -314,6 +314,17 @@ abq_status abq_gemm_set_workspace(abq_gemm_state *state, void *workspace, size_t
  * asynchronous launch on `stream`. */
 abq_status abq_gemm_exec(const abq_gemm_state *state, void *stream);
 
+/* No counterpart in the reference.  abq_gemm_exec for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the same launches, with
+ * the layout conversions writing into a static device array inside the library instead of a workspace the
+ * caller brings (a workspace attached to the state is ignored).  Allocates nothing.  A state whose
+ * conversions need more than ABQ_STATIC_WORKSPACE_BYTES is refused with ABQ_ERR_TOO_LARGE and a message
+ * on stderr.  All calls on one device share that device's array: calls that may run concurrently on one
+ * device (different streams) race on it; order them or use abq_gemm_exec with separate workspaces.  The
+ * first call on a device looks the array's address up (hipGetSymbolAddress): make it before a capture. */
+#define ABQ_STATIC_WORKSPACE_BYTES (32u << 20)
+abq_status abq_gemm_exec_static(const abq_gemm_state *state, void *stream);
+
 /* Replaces launchWmmaAnyKernel (engine/wmma_any/wmma_any.h:18-38, wmma_any.cu:28-87): the
  * first-generation entry point, init + exec in one call, int32 D. */
 abq_status abq_gemm_launch(const abq_tile_config *cfg, const uint32_t *X, const uint32_t *W,
