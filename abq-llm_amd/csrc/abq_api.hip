@@ -103,7 +103,7 @@ static void entry_to_config(const KernelEntry &e, int strategy, int x_bits, int 
     if (strategy == ABQ_STRATEGY_BCNT) {
         const int lpr = 1 << lpr_log2;
         c->block_m = e.tm;
-        c->block_n = 4 * (64 / lpr);
+        c->block_n = e.wn * (64 / lpr);
         c->block_k = lpr * 128;
         c->warp_m = e.tm;
         c->warp_n = 64 / lpr;
@@ -111,7 +111,7 @@ static void entry_to_config(const KernelEntry &e, int strategy, int x_bits, int 
         c->mma_m = 1;
         c->mma_n = 1;
         c->mma_k = 128;
-        c->nstage = 1;
+        c->nstage = e.nstage; // passes whose loads a lane keeps in flight
     } else {
         // NSTAGE 4 (K-tiled layout, 128- or 64-element stages) and NSTAGE 3 (decode, 512- or 256-element steps)
         // carry their K step; the direct kernels step 4 plane words per lane group
@@ -185,18 +185,31 @@ static int find_mfma_variant(const KernelTable &t, int mi, int tm, int tn, int w
     return -1;
 }
 
-// Default choice when the caller names no native tile: the decode kernel (16-row MFMA tiles,
-// activations staged in LDS) up to 16 activation rows, 32-row MFMA tiles above.  The popcount
-// kernels stay reachable through their tile tuples (MMA 1x1x128).
+// Default choice when the caller names no native tile (operands in the reference's plane layout).
+//
+// Decode-sized M (at most 16 rows): the VALU popcount kernel or the matrix-core decode kernel.  The popcount
+// kernel works on the planes as they are and costs x_bits * w_bits * M AND + popcount pairs per 128 weights; the
+// matrix-core kernel pays a bit-matrix transpose per 32 weights that grows with w_bits (steeply from 6 planes
+// up) and nothing per row.  Measured on MI355X over the twelve bit pairs, M = 1, 2, 4, 8 and the LLaMA-7B
+// shapes, the popcount kernel is the faster one while x_bits * w_bits * M stays at or below a bound that
+// depends on w_bits: it wins every pair at M = 1 (by 2 to 52 %), the low products and the 6- to 8-bit weights at
+// M = 2, and almost nothing from M = 4 up.  Above 16 rows: 32-row MFMA tiles.
 // K elements per work item of the default decode kernel (512 or 256, see abq_gemm_decode.hip)
 static const int kDefaultDecodeStep = 512;
 
-static void choose_default(int M, int N, int *strategy, int *mi, int *tm, int *tn, int *wm, int *wn,
-                           int *wk)
+static bool popcount_is_faster(int x_bits, int w_bits, int M)
 {
-    if (M <= 16) {
-        // Measured on MI355X (W2A8, LLaMA-7B shapes, M = 1, 4, 8): the decode kernel with 16
-        // waves beats the popcount kernel at every M including M = 1, and the other MFMA tiles.
+    static const int bound[9] = { 0, 16, 16, 27, 32, 40, 100, 150, 200 }; // by w_bits
+    return w_bits >= 1 && w_bits <= 8 && x_bits * w_bits * M <= bound[w_bits];
+}
+
+static void choose_default(int M, int N, int x_bits, int w_bits, int *strategy, int *mi, int *tm, int *tn, int *wm,
+                           int *wn, int *wk)
+{
+    if (M <= 16 && popcount_is_faster(x_bits, w_bits, M)) {
+        *strategy = ABQ_STRATEGY_BCNT;
+        *mi = 1; *tm = M <= 1 ? 1 : M <= 2 ? 2 : 4; *tn = 1; *wm = 1; *wn = 8; *wk = 1;
+    } else if (M <= 16) {
         *strategy = ABQ_STRATEGY_DECODE;
         *mi = 16; *tm = 1; *tn = 1; *wm = 1; *wn = 1; *wk = 16;
     } else {
@@ -266,10 +279,10 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
     int lpr_log2 = best_lpr_log2(K);
     int decode_step = cfg ? cfg->warp_k : 0; // K elements per decode work item
     if (strategy == ABQ_STRATEGY_AUTO) {
-        choose_default(M, N, &strategy, &mi, &tm, &tn, &wm, &wn, &wk);
+        choose_default(M, N, x_bits, w_bits, &strategy, &mi, &tm, &tn, &wm, &wn, &wk);
         decode_step = kDefaultDecodeStep;
     } else if (strategy == ABQ_STRATEGY_BCNT) {
-        mi = 1; tm = cfg->block_m; tn = 1; wm = 1; wn = 4; wk = 1;
+        mi = 1; tm = cfg->block_m; tn = 1; wm = 1; wn = 8; wk = 1;
         // block_k = lanes per row * 128; accept 16, 32 or 64 lanes, else keep the best fit
         const int lpr = cfg->block_k / 128;
         if (cfg->block_k % 128 == 0 && (lpr == 16 || lpr == 32 || lpr == 64))
@@ -371,23 +384,25 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
 
     if (strategy == ABQ_STRATEGY_BCNT) {
         int v = -1;
+        // passes in flight: the tuple's NSTAGE; a library choice takes one pass per lane when that covers K, else three
+        const int want_d = cfg && strategy_of_mma(*cfg) == ABQ_STRATEGY_BCNT ? cfg->nstage : (K / 128 <= (1 << lpr_log2) ? 1 : 3);
         for (int i = 0; i < tb_->count; ++i)
-            if (tb_->entries[i].tm == tm)
+            if (tb_->entries[i].tm == tm && tb_->entries[i].nstage == want_d)
                 v = i;
         if (v < 0)
             return ABQ_ERR_UNSUPPORTED;
         const KernelEntry &e = tb_->entries[v];
-        const int rpp = 64 >> lpr_log2;
-        const int npass = (N + rpp - 1) / rpp;
-        if ((M + e.tm - 1) / e.tm > 65535)
+        const int rows_per_wg = e.wn * (64 >> lpr_log2);
+        const int mb = M < e.tm ? M : e.tm;
+        const size_t lds = (size_t)x_bits * mb * (K / 32) * 4 + 1024;
+        if ((M + e.tm - 1) / e.tm > 65535 || lds > 160 * 1024 || (size_t)N * (K / 32) * 4 >= (1ull << 32))
             return ABQ_ERR_TOO_LARGE;
         st->strategy = strategy;
         st->variant = v;
         entry_to_config(e, strategy, x_bits, w_bits, is_signed, lpr_log2, &st->cfg);
-        st->grid_dim = abq_dim3{ (unsigned)((npass + 3) / 4 > 65536 ? 65536 : (npass + 3) / 4),
-                                 (unsigned)((M + e.tm - 1) / e.tm), 1 };
-        st->block_dim = abq_dim3{ 256, 1, 1 };
-        st->shared_mem_size = 0;
+        st->grid_dim = abq_dim3{ (unsigned)((N + rows_per_wg - 1) / rows_per_wg), (unsigned)((M + e.tm - 1) / e.tm), 1 };
+        st->block_dim = abq_dim3{ (unsigned)(64 * e.wn), 1, 1 };
+        st->shared_mem_size = lds;
         st->reserved[0] = lpr_log2;
         return ABQ_OK;
     }
@@ -815,6 +830,27 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
     return ABQ_OK;
 }
 
+// Moves a state whose tile was the library's choice onto the matrix-core decode kernel for plane operands.
+static abq_status switch_to_decode(abq_gemm_state *st)
+{
+    const abq_tile_config &c = st->cfg;
+    const KernelTable *td = find_table(registry().decode, c.x_bits, c.w_bits, c.is_signed);
+    if (!td)
+        return ABQ_ERR_UNSUPPORTED;
+    for (int i = 0; i < td->count; ++i) {
+        if (td->entries[i].wk != 16 || td->entries[i].kb != kDefaultDecodeStep)
+            continue;
+        abq_tile_config cfg;
+        entry_to_config(td->entries[i], ABQ_STRATEGY_DECODE, c.x_bits, c.w_bits, c.is_signed, 0, &cfg);
+        abq_gemm_state tmp = *st;
+        const abq_status rc = resolve(&cfg, c.x_bits, c.w_bits, c.is_signed, st->M, st->N, st->K, &tmp);
+        if (rc == ABQ_OK)
+            *st = tmp;
+        return rc;
+    }
+    return ABQ_ERR_UNSUPPORTED;
+}
+
 // Decode-sized GEMM with both operands K-tiled: the decode kernel built for that layout, if it exists for the
 // pair.  Variant by shape (measured on MI355X, W2A8, LLaMA-7B widths): sixteen waves with one weight load each
 // in flight while a compute unit holds at most two workgroups; with more tiles than that, eight waves with two
@@ -922,6 +958,8 @@ abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, cons
         if (!c.is_signed && (c.x_bits == 8 || c.w_bits == 8))
             return ABQ_ERR_UNSUPPORTED;
         state->group_size = group_size;
+        if (state->strategy == ABQ_STRATEGY_BCNT && state->auto_chosen && state->M <= 16)
+            switch_to_decode(state); // the popcount kernel has no group-scale epilogue
         const bool decode_ok = state->strategy == ABQ_STRATEGY_DECODE && state->auto_chosen && state->M <= 16 &&
                                state->x_layout == ABQ_LAYOUT_PLANES && state->w_layout == ABQ_LAYOUT_PLANES &&
                                decode_grouped_lds(state->M, state->K, group_size) != 0 &&

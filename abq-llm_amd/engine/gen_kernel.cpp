@@ -161,11 +161,14 @@ std::vector<MfmaVariant> enumerate_mfma(int x_bits, int w_bits)
 std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits, bool is_signed)
 {
     std::vector<Tile> out;
-    // VALU popcount: MT activation rows per pass, LPR lanes per weight row (16, 32, 64).
-    for (int mt : { 1, 2, 4 }) {
-        for (int lpr : { 16, 32, 64 }) {
-            const int rows = 64 / lpr;
-            out.push_back(Tile{ mt, 4 * rows, lpr * 128, mt, rows, lpr * 128, 1, 1, 128, 1, 4, { 1 } });
+    // VALU popcount: MT activation rows per workgroup, LPR lanes per weight row (16, 32, 64), eight waves;
+    // NSTAGE = passes of a lane whose loads are in flight together (1 or 3).
+    for (int d : { 1, 3 }) {
+        for (int mt : { 1, 2, 4 }) {
+            for (int lpr : { 16, 32, 64 }) {
+                const int rows = 64 / lpr;
+                out.push_back(Tile{ mt, 8 * rows, lpr * 128, mt, rows, lpr * 128, 1, 1, 128, 1, 8, { d } });
+            }
         }
     }
     // Decode kernel: 16-row MFMA tiles, activations expanded once per workgroup into LDS

@@ -119,7 +119,7 @@ static void gpu_paths()
 #define RUN(type, ...)                                                                                        \
     CHECK((run_config<AQ_INIT_FUN(type), AQ_EXEC_FUN(type), AQ_OP_STATE(type)>(                               \
         AQ_NAME_FUN(type, Init, __VA_ARGS__), AQ_NAME_FUN(type, Exec, __VA_ARGS__), c, d_xp, d_wp, d_out, ref, stream)))
-    RUN(AqBMMA, 8, 2, true, 1, 8, 4096, 1, 2, 4096, 1, 1, 128, 1);          // VALU popcount
+    RUN(AqBMMA, 8, 2, true, 1, 16, 4096, 1, 2, 4096, 1, 1, 128, 1);          // VALU popcount
     RUN(AqBMMA, 8, 2, true, 16, 16, 4096, 16, 16, 512, 16, 16, 64, 3);      // decode kernel
     RUN(AqBMMA, 8, 2, true, 16, 16, 4096, 16, 16, 512, 16, 16, 64, 2);      // int8 MFMA 16x16x64
     RUN(AqBMMA, 8, 2, true, 128, 128, 256, 64, 64, 256, 32, 32, 32, 2);     // int8 MFMA 32x32x32

@@ -222,11 +222,22 @@ def test_init_error_paths(abq):
 
 
 def test_default_strategy_choice_and_reference_tuples(abq):
-    for M, want in ((1, abq.STRATEGY_DECODE), (2, abq.STRATEGY_DECODE), (4, abq.STRATEGY_DECODE),
+    # W2A8 on plane operands: the popcount kernel for one row, the matrix-core decode kernel up to 16, MFMA 32x32 above
+    for M, want in ((1, abq.STRATEGY_BCNT), (2, abq.STRATEGY_DECODE), (4, abq.STRATEGY_DECODE),
                     (8, abq.STRATEGY_DECODE), (16, abq.STRATEGY_DECODE), (128, abq.STRATEGY_MFMA32),
                     (2048, abq.STRATEGY_MFMA32)):
         rc, st = _init(abq, M=M, N=4096)
         assert rc == 0 and st.strategy == want, M
+    # the choice follows x_bits * w_bits * M against a bound by w_bits (popcount work against the cost of the weight transposes)
+    for q, p, M, want in ((2, 2, 4, abq.STRATEGY_BCNT), (2, 2, 8, abq.STRATEGY_DECODE), (4, 4, 2, abq.STRATEGY_BCNT),
+                          (4, 4, 4, abq.STRATEGY_DECODE), (8, 8, 2, abq.STRATEGY_BCNT), (8, 8, 4, abq.STRATEGY_DECODE),
+                          (5, 5, 1, abq.STRATEGY_BCNT), (5, 5, 2, abq.STRATEGY_DECODE), (8, 4, 1, abq.STRATEGY_BCNT)):
+        rc, st = _init(abq, q=q, p=p, M=M, N=4096)
+        assert rc == 0 and st.strategy == want, (q, p, M)
+    rc, st = _init(abq, M=1, N=4096)   # K = 4096: 32 lanes per row, one pass per lane in flight, eight waves of two rows
+    assert st.cfg.as_tuple()[3:] == (1, 16, 4096, 1, 2, 4096, 1, 1, 128, 1) and st.block_dim.x == 512 and st.grid_dim.x == 256
+    rc, st = _init(abq, M=1, N=4096, K=11008)  # three passes of 32 lanes
+    assert st.cfg.nstage == 3 and st.cfg.block_k == 4096
     # a reference (tensor-core) tuple is accepted and resolved to a native tile
     cfg, _ = abq.parse_kernel_name("AqBMMA_8x2xtrue_8x48x256_32x48x128_8x8x128_5")
     rc, st = _init(abq, cfg=cfg, M=8)
