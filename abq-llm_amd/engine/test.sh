@@ -9,7 +9,7 @@ rm -rf results
 mkdir -p results
 # "x_bits w_bits" pairs: the symmetric widths, then the mixed ones
 COMBOS="2:2 3:3 4:4 5:5 6:6 7:7 8:8 4:2 6:2 8:2 8:3 8:4"
-for shape in "4096 4096" "8192 1024" "11008 4096" "5120 5120"; do
+for shape in "4096 4096" "8192 1024" "11008 4096" "5120 5120" "4096 11008"; do
     set -- $shape
     N=$1
     K=$2
