@@ -2,7 +2,7 @@
 // file (abq_weight_file.h), optionally also as the headerless plane dump the reference's
 // FasterTransformer loader reads.
 //
-//   abq_convert_weights IN.bin N K BITS GROUP_SIZE {sym|asym} OUT.abqw [--fp16] [--ft-bin OUT.bin]
+//   abq_convert_weights IN.bin N K BITS GROUP_SIZE {sym|asym} OUT.abqw [--fp16] [--ft-bin OUT.bin] [--bit-balance]
 //
 // IN.bin: row-major [N][K] float32 (or fp16 with --fp16), the layout of torch's linear.weight.
 #include <stdio.h>
@@ -42,19 +42,21 @@ static float half_to_float(uint16_t h)
 int main(int argc, char **argv)
 {
     if (argc < 8) {
-        printf("Usage: ./abq_convert_weights IN.bin N K BITS GROUP_SIZE {sym|asym} OUT.abqw [--fp16] [--ft-bin OUT.bin]\n");
+        printf("Usage: ./abq_convert_weights IN.bin N K BITS GROUP_SIZE {sym|asym} OUT.abqw [--fp16] [--ft-bin OUT.bin] [--bit-balance]\n");
         return 2;
     }
     const std::string in = argv[1], mode = argv[6], out = argv[7];
     const uint32_t n = (uint32_t)atoi(argv[2]), k = (uint32_t)atoi(argv[3]), bits = (uint32_t)atoi(argv[4]),
                    group = (uint32_t)atoi(argv[5]);
-    bool fp16 = false;
+    bool fp16 = false, bit_balance = false;
     std::string ft_bin;
     for (int i = 8; i < argc; ++i) {
         if (!strcmp(argv[i], "--fp16"))
             fp16 = true;
         else if (!strcmp(argv[i], "--ft-bin") && i + 1 < argc)
             ft_bin = argv[++i];
+        else if (!strcmp(argv[i], "--bit-balance"))
+            bit_balance = true; // the reference's default for asymmetric 1- and 2-bit weights: 2^BITS + 1 levels, BITS + 1 planes
     }
     if (mode != "sym" && mode != "asym") {
         printf("[ABQ][Error] mode must be sym or asym\n");
@@ -84,11 +86,12 @@ int main(int argc, char **argv)
     }
     ABQWeightBlob blob;
     std::string err;
-    if (!abq_quantize_weights(w.data(), n, k, bits, mode == "sym", group, &blob, &err) ||
+    if (!abq_quantize_weights(w.data(), n, k, bits, mode == "sym", group, &blob, &err, bit_balance) ||
         !abq_weight_file_write(out, blob, &err) || (!ft_bin.empty() && !abq_weight_file_write_ft_bin(ft_bin, blob, &err))) {
         printf("[ABQ][Error] %s\n", err.c_str());
         return 1;
     }
-    printf("wrote %s: W%u %s, %u x %u, group %u, %zu plane bytes\n", out.c_str(), bits, mode.c_str(), n, k, group, blob.planes.size() * 4);
+    printf("wrote %s: W%u %s%s, %u x %u, group %u, %u planes, %zu plane bytes\n", out.c_str(), bits, mode.c_str(),
+           bit_balance ? " (bit balance)" : "", n, k, group, blob.info.bits, blob.planes.size() * 4);
     return 0;
 }

@@ -18,11 +18,16 @@ static bool fail(std::string *error, const std::string &what)
     return false;
 }
 
-bool abq_quantize_weights(const float *w, uint32_t n, uint32_t k, uint32_t bits, bool symmetric, uint32_t group_size,
-                          ABQWeightBlob *out, std::string *error)
+bool abq_quantize_weights(const float *w, uint32_t n, uint32_t k, uint32_t nominal_bits, bool symmetric, uint32_t group_size,
+                          ABQWeightBlob *out, std::string *error, bool bit_balance)
 {
-    if (!w || !out || n == 0 || bits < 2 || bits > 8)
+    if (!w || !out || n == 0 || nominal_bits < (bit_balance ? 1u : 2u) || nominal_bits > 8)
         return fail(error, "bad arguments");
+    if (bit_balance && (symmetric || nominal_bits > 2))
+        return fail(error, "bit balance applies to asymmetric 1- and 2-bit weights only");
+    // with bit balance the unsigned codes run from 0 to 2^bits inclusive: one more plane
+    const uint32_t bits = bit_balance ? nominal_bits + 1 : nominal_bits;
+    const int levels = bit_balance ? (1 << nominal_bits) : (1 << nominal_bits) - 1; // qmax of the unsigned code
     if (k < 128 || k % 128 != 0)
         return fail(error, "K must be >= 128 and a multiple of 128");
     const uint32_t g = group_size ? group_size : k;
@@ -31,6 +36,7 @@ bool abq_quantize_weights(const float *w, uint32_t n, uint32_t k, uint32_t bits,
     const uint32_t groups = k / g;
     const int half = 1 << (bits - 1);
     memset(&out->info, 0, sizeof(out->info));
+    out->info.reserved[0] = bit_balance ? 1u : 0u;
     memcpy(out->info.magic, kMagic, 8);
     out->info.version = 1;
     out->info.n = n;
@@ -56,7 +62,7 @@ bool abq_quantize_weights(const float *w, uint32_t n, uint32_t k, uint32_t bits,
                 scale = std::max(fabs(mn), fabs(mx)) / (half - 1);
                 scale = std::min(std::max(scale, 1e-5), 1e4);
             } else {
-                scale = (mx - mn) / (2 * half - 1);
+                scale = (mx - mn) / levels;
                 scale = std::min(std::max(scale, 1e-5), 1e4);
                 zp = nearbyint(std::min(std::max(-mn / scale, -1e4), 1e4));
             }
@@ -69,7 +75,7 @@ bool abq_quantize_weights(const float *w, uint32_t n, uint32_t k, uint32_t bits,
                 if (symmetric)
                     code = (int)std::min(std::max(q, (double)-half), (double)(half - 1));
                 else
-                    code = (int)std::min(std::max(q + zp, 0.0), (double)(2 * half - 1)) - half;
+                    code = (int)std::min(std::max(q + zp, 0.0), (double)levels) - half;
                 const uint32_t e = gi * g + i; // element within the row
                 const uint32_t pattern = (uint32_t)code & ((1u << bits) - 1u);
                 for (uint32_t b = 0; b < bits; ++b)

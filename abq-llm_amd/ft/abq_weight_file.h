@@ -47,8 +47,13 @@ struct ABQWeightBlob {
 // 2^bits - 1 level range): asymmetric codes u in [0, 2^bits) with zero point zp per (row, group),
 // stored as signed codes u - 2^(bits-1) with zero = zp - 2^(bits-1); symmetric: signed codes in
 // [-2^(bits-1), 2^(bits-1)-1], no zero points.  group_size 0 = one group per row.
+// bit_balance (asymmetric 1- and 2-bit weights only): the reference's default at those widths
+// (quantizer.py:66-68,169-171): the range is widened by one level, qmax = 2^bits and scale = range / 2^bits, so a
+// 2-bit weight takes the five values u in [0, 4].  Five levels do not fit two planes: the codes are stored with
+// bits + 1 planes (info.bits = bits + 1, info.reserved[0] = 1) as u - 2^bits with zero = zp - 2^bits, and the GEMM
+// runs as a (bits + 1)-bit weight.
 bool abq_quantize_weights(const float *w, uint32_t n, uint32_t k, uint32_t bits, bool symmetric, uint32_t group_size,
-                          ABQWeightBlob *out, std::string *error);
+                          ABQWeightBlob *out, std::string *error, bool bit_balance = false);
 
 // The gate and up projections of one MLP as a single matrix for the fused SiLU-gate epilogue
 // (abq_gemm_set_activation): blocks of 16 gate rows followed by their 16 up rows; planes, scales

@@ -9,7 +9,8 @@ Learnable clipping (lwc) and the "fix0to1" metric are training-only and not rest
 Pinned by: closed-form cases in tests/test_oracle.py (a row that is exactly representable
 quantizes to itself; the max-abs element of a symmetric row maps to +/-(2^(n-1)-1); the
 min / max of an asymmetric row map to qmin / qmax; the dequantization error of every
-in-range element is at most scale/2).
+in-range element is at most scale/2; bit balance: five levels at 2 bits, a row spanning [0, 4 s] maps to
+0..4 exactly; rows padded to whole groups: the padded group's scale is that of its real elements).
 """
 import numpy as np
 
@@ -32,13 +33,23 @@ class QuantParams:
                 self.qmax += 1
 
 
+def _into_groups(x, qp):
+    """quantizer.py:151-156 / :112-118: rows reshaped into groups; a row whose length is not a multiple of the
+    group size is padded with zeros first (the "deficiency", :82-91; the reference allows it for symmetric
+    quantisation only)."""
+    deficiency = (-x.shape[-1]) % qp.group_size
+    if deficiency:
+        assert qp.symmetric, "the reference pads rows to whole groups only for symmetric quantisation"
+        x = np.concatenate([x, np.zeros((x.shape[0], deficiency), dtype=x.dtype)], axis=1)
+    return x.reshape(-1, qp.group_size), deficiency
+
+
 def calibrate(x, qp):
     """quantizer.py:149-179.  x: float [rows, cols].  Returns (scale, round_zero_point|None),
-    each of shape [rows * cols/group, 1] (or [rows, 1] without groups)."""
+    each of shape [rows * ceil(cols/group), 1] (or [rows, 1] without groups)."""
     x = np.asarray(x, dtype=np.float64)
     if qp.group_size:
-        assert x.shape[-1] % qp.group_size == 0, "deficiency padding is not restated"
-        x = x.reshape(-1, qp.group_size)
+        x, _ = _into_groups(x, qp)
     xmin = x.min(axis=-1, keepdims=True)
     xmax = x.max(axis=-1, keepdims=True)
     n = qp.n_bits
@@ -60,12 +71,15 @@ def quantize(x, qp, scale, zp):
     """Integer codes of fake_quant (quantizer.py:120-123): clamp(round(x/scale) + zp)."""
     x = np.asarray(x, dtype=np.float64)
     shape = x.shape
+    deficiency = 0
     if qp.group_size:
-        x = x.reshape(-1, qp.group_size)
+        x, deficiency = _into_groups(x, qp)
     xi = np.round(x / scale)
     if zp is not None:
         xi = xi + zp
     xi = np.clip(xi, qp.qmin, qp.qmax)
+    if deficiency:  # the padding is cut off again (quantizer.py:130-131)
+        return xi.reshape(shape[0], -1)[:, :shape[1]]
     return xi.reshape(shape)
 
 
@@ -73,10 +87,13 @@ def dequantize(xi, qp, scale, zp):
     """quantizer.py:124-128."""
     shape = xi.shape
     xi = np.asarray(xi, dtype=np.float64)
+    deficiency = 0
     if qp.group_size:
-        xi = xi.reshape(-1, qp.group_size)
+        xi, deficiency = _into_groups(xi, qp)
     if zp is not None:
         xi = xi - zp
+    if deficiency:
+        return (xi * scale).reshape(shape[0], -1)[:, :shape[1]]
     return (xi * scale).reshape(shape)
 
 
@@ -111,6 +128,22 @@ def per_token_codes_f32(x, n_bits, symmetric):
         codes = np.clip(np.rint(x / scale) + zp, 0, 2 * half - 1) - half
         zero = zp - f(half)
     return codes.astype(np.int32), scale[:, 0].astype(f), zero[:, 0].astype(f)
+
+
+def group_affine_codes_bit_balance(w, n_bits, group_size):
+    """The reference's default weight quantiser at 1 and 2 bits ("bit balance", quantizer.py:66-68,169-171): the
+    asymmetric range is widened by one level, qmax = 2^n and scale = range / 2^n, so a 2-bit weight takes five
+    values u in [0, 4].  Goes through calibrate / quantize above (QuantParams applies the widening).  The codes need
+    n + 1 bits; they are returned in the signed representation of that width: code = u - 2^n, zero = zp - 2^n.
+    Returns (codes int32 [N, K], scale float64 [N, K/g], zero float64 [N, K/g], storage bits n + 1)."""
+    assert n_bits in (1, 2)
+    w = np.asarray(w, dtype=np.float64)
+    n, k = w.shape
+    qp = QuantParams(n_bits, symmetric=False, group_size=group_size)
+    scale, zp = calibrate(w, qp)
+    u = quantize(w, qp, scale, zp)
+    half = 1 << n_bits
+    return ((u - half).astype(np.int32), scale.reshape(n, k // group_size), zp.reshape(n, k // group_size) - half, n_bits + 1)
 
 
 def group_affine_codes(w, n_bits, group_size):

@@ -27,13 +27,16 @@ def fdev(a):
 
 
 def assert_close_rel(got, want):
-    """|got - want| <= REL_TOL * |want| elementwise, with an absolute floor of REL_TOL times the
-    matrix's RMS for entries that cancel to nearly zero; plus a much tighter norm-wise bound."""
+    """|got - want| <= REL_TOL * |want| elementwise (BASELINE: 1e-2 relative), plus a much tighter norm-wise bound.
+    The only slack is an absolute 1e-3 of the matrix's RMS for entries that cancel to nearly zero: the fp32 epilogue
+    adds group terms and zero-point corrections that are each up to a few hundred times the matrix's RMS (asymmetric
+    activations, K = 11008), so their rounding (6e-8 relative each) leaves about 1e-4 of the RMS as absolute noise,
+    which no relative bound on a vanishing entry can absorb (measured worst case: 1.5e-4 of the RMS)."""
     got = got.astype(np.float64)
     rms = np.sqrt(np.mean(want ** 2))
     err = np.abs(got - want)
     assert np.all(np.isfinite(got))
-    assert np.all(err <= REL_TOL * np.abs(want) + REL_TOL * rms), float((err / (np.abs(want) + rms)).max())
+    assert np.all(err <= REL_TOL * np.abs(want) + 1e-3 * rms), float((err / (np.abs(want) + 1e-1 * rms)).max())
     assert np.linalg.norm(got - want) <= 2e-3 * np.linalg.norm(want)
 
 
@@ -364,14 +367,19 @@ def test_group_scales_on_the_fp6_route(abq, oracle, q, p, signed):
 LAYER_LINEARS = [("qkv", 12288, 4096), ("o", 4096, 4096), ("gate_up", 2 * 11008, 4096), ("down", 4096, 11008)]
 
 
-def _layer_linear(abq, oracle, name, N, K, tokens, x_symmetric, seed, sample_rows):
+def _layer_linear(abq, oracle, name, N, K, tokens, x_symmetric, seed, sample_rows, bit_balance=False):
     """One W2A8 linear: fp16 weights N(0, 0.02) quantised to 2 bits per (channel, group of 128),
-    fp16 activations quantised per token on the device; checks `sample_rows` output rows."""
+    fp16 activations quantised per token on the device; checks `sample_rows` output rows.
+    bit_balance: the reference's default 2-bit weight quantiser (five levels, quantizer.py:66-68,169-171),
+    whose codes take three planes."""
     from oracle import quantizer as Q
     rng = np.random.default_rng(seed)
     w = rng.normal(0, 0.02, (N, K)).astype(np.float16)
-    w_codes, w_scale, w_zero = Q.group_affine_codes(w, 2, 128)
-    wp = planes_dev(oracle.pack_i32(w_codes, 2))
+    if bit_balance:
+        w_codes, w_scale, w_zero, w_planes = Q.group_affine_codes_bit_balance(w, 2, 128)
+    else:
+        (w_codes, w_scale, w_zero), w_planes = Q.group_affine_codes(w, 2, 128), 2
+    wp = planes_dev(oracle.pack_i32(w_codes, w_planes))
     wt = abq.relayout_planes(wp)
     ws_d, wz_d = fdev(w_scale), fdev(w_zero)
 
@@ -384,6 +392,13 @@ def _layer_linear(abq, oracle, name, N, K, tokens, x_symmetric, seed, sample_row
     if not x_symmetric:
         kw.update(x_zero=xz, w_zero_term=abq.weight_zero_term(wp, True, ws_d, wz_d, 128))
     got = run_grouped(abq, xt, wt, True, **kw)
+    got2 = None
+    if tokens <= 16:  # decode-sized: also the decode kernel's group-scale variant on plane operands
+        xp, xs2, xz2, sums2 = abq.quant_pack_f16(x, 8, symmetric=x_symmetric, tiled=False, group_size=128)
+        kw2 = dict(kw, x_scale=xs2, x_group_sums=sums2, x_tiled=False, w_tiled=False)
+        if not x_symmetric:
+            kw2.update(x_zero=xz2)
+        got2 = run_grouped(abq, xp, wp, True, strategy="decode", **kw2)
 
     rows = np.sort(rng.choice(tokens, size=min(sample_rows, tokens), replace=False))
     x_rows = x[torch.from_numpy(rows).cuda()].cpu().numpy()
@@ -391,6 +406,8 @@ def _layer_linear(abq, oracle, name, N, K, tokens, x_symmetric, seed, sample_row
     assert np.array_equal(xs.cpu().numpy()[rows], scale)
     want = Q.dequant_matmul(codes, scale, zero, w_codes, w_scale, w_zero, 128)
     assert_close_rel(got[rows], want)
+    if got2 is not None:
+        assert_close_rel(got2[rows], want)
     # and the quantised result tracks the unquantised fp16 linear as 2-bit weights allow: the
     # dequantised weights are within scale/2 of the originals, so this is only a sanity bound
     full = x_rows.astype(np.float64) @ w.astype(np.float64).T
@@ -401,6 +418,14 @@ def _layer_linear(abq, oracle, name, N, K, tokens, x_symmetric, seed, sample_row
 @pytest.mark.parametrize("x_symmetric", [True, False])
 def test_config4_decoder_layer_linears_batch1(abq, oracle, name, N, K, x_symmetric):
     _layer_linear(abq, oracle, name, N, K, 1024, x_symmetric, seed=len(name) + N % 97, sample_rows=48)
+
+
+@pytest.mark.parametrize("tokens", [8, 1024])
+@pytest.mark.parametrize("x_symmetric", [True, False])
+def test_config4_linear_with_bit_balanced_2bit_weights(abq, oracle, tokens, x_symmetric):
+    """The O projection with the reference's default 2-bit weight quantiser (bit balance: five levels, three planes):
+    W3A8 with group-128 scales and zero points against the fp64 matmul of the dequantised operands."""
+    _layer_linear(abq, oracle, "o", 4096, 4096, tokens, x_symmetric, seed=91 + tokens, sample_rows=48, bit_balance=True)
 
 
 @pytest.mark.parametrize("name,N,K", LAYER_LINEARS)

@@ -274,3 +274,46 @@ def test_group_affine_codes_and_dequant_matmul():
             for k in range(256):
                 want[m, n] += (xc[m, k] - xz[m]) * xs[m] * (codes[n, k] - zero[n, k // 128]) * scale[n, k // 128]
     assert np.allclose(got, want, rtol=1e-12, atol=1e-12)
+
+
+def test_quantizer_bit_balance_closed_forms():
+    """quantizer.py:66-68,169-171: asymmetric 1- and 2-bit ranges are widened by one level.  A row holding the
+    exact multiples 0, s, 2s, 3s, 4s of a step s is quantised to 0..4 with scale s and dequantises to itself; with
+    the plain range (3 bits) the same row would use scale 4s/7."""
+    from oracle import quantizer as Q
+    s = 0.125
+    x = np.array([[0.0, s, 2 * s, 3 * s, 4 * s, 2 * s, s, 4 * s]])
+    qp = Q.QuantParams(2)
+    assert (qp.qmin, qp.qmax) == (0, 4)
+    scale, zp = Q.calibrate(x, qp)
+    assert scale[0, 0] == s and zp[0, 0] == 0
+    assert np.array_equal(Q.quantize(x, qp, scale, zp), np.array([[0, 1, 2, 3, 4, 2, 1, 4]], dtype=np.float64))
+    assert np.array_equal(Q.fake_quant(x, qp), x)
+    assert Q.QuantParams(1).qmax == 2 and Q.QuantParams(3).qmax == 7 and Q.QuantParams(2, disable_zero_point=True).qmax == 1
+    # shifted row: the zero point takes the offset, the codes stay
+    scale, zp = Q.calibrate(x - 2 * s, qp)
+    assert scale[0, 0] == s and zp[0, 0] == 2
+    assert np.array_equal(Q.quantize(x - 2 * s, qp, scale, zp), np.array([[0, 1, 2, 3, 4, 2, 1, 4]], dtype=np.float64))
+    codes, sc, zero, bits = Q.group_affine_codes_bit_balance(np.tile(x - 2 * s, (2, 16)), 2, 64)
+    assert bits == 3 and codes.min() == -4 and codes.max() == 0 and np.all(sc == s) and np.all(zero == 2 - 4)
+    # x ~ scale * (code - zero) reproduces the row
+    assert np.array_equal((codes - np.repeat(zero, 64, axis=1)) * np.repeat(sc, 64, axis=1), np.tile(x - 2 * s, (2, 16)))
+
+
+def test_quantizer_pads_rows_to_whole_groups():
+    """quantizer.py:82-91,112-118,151-156: a row whose length is no multiple of the group size is padded with zeros
+    (symmetric quantisation only); the padded group's scale comes from its real elements and the padding is cut off."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(3)
+    x = rng.normal(0, 1, (3, 100))
+    qp = Q.QuantParams(4, symmetric=True, disable_zero_point=True, group_size=64)
+    scale, zp = Q.calibrate(x, qp)
+    assert zp is None and scale.shape == (6, 1)
+    want = np.stack([np.abs(x[:, :64]).max(axis=1), np.abs(x[:, 64:]).max(axis=1)], axis=1).reshape(-1, 1) / 7
+    assert np.allclose(scale, want, rtol=0, atol=0)
+    q = Q.quantize(x, qp, scale, zp)
+    assert q.shape == x.shape and np.array_equal(q[:, :64], np.clip(np.round(x[:, :64] / scale[0::2]), -8, 7))
+    assert np.array_equal(q[:, 64:], np.clip(np.round(x[:, 64:] / scale[1::2]), -8, 7))
+    assert Q.fake_quant(x, qp).shape == x.shape
+    with pytest.raises(AssertionError):
+        Q.calibrate(x, Q.QuantParams(4, symmetric=False, group_size=64))

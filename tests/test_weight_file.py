@@ -60,6 +60,33 @@ def test_converter_asymmetric_matches_the_restated_quantizer(tmp_path, oracle, b
     assert raw == f["planes"].tobytes() and len(raw) == bits * k * n // 16 * 2
 
 
+@pytest.mark.parametrize("bits", [2, 1])
+def test_converter_bit_balance_matches_the_restated_quantizer(tmp_path, oracle, bits):
+    """--bit-balance: the reference's default for asymmetric 1- and 2-bit weights (quantizer.py:66-68,169-171):
+    2^bits + 1 levels, scale = range / 2^bits, stored with one more plane."""
+    from oracle import quantizer as Q
+    _need_tool()
+    rng = np.random.default_rng(40 + bits)
+    n, k, group = 48, 384, 128
+    w = rng.normal(0, 0.02, (n, k)).astype(np.float32)
+    src, dst = tmp_path / "w.bin", tmp_path / "w.abqw"
+    w.tofile(src)
+    out = subprocess.run([TOOL, str(src), str(n), str(k), str(bits), str(group), "asym", str(dst), "--bit-balance"],
+                         capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, out.stdout + out.stderr
+    f = read_abqw(dst)
+    codes, scale, zero, store_bits = Q.group_affine_codes_bit_balance(w, bits, group)
+    assert store_bits == bits + 1 and (f["n"], f["k"], f["bits"], f["signed"], f["group"]) == (n, k, bits + 1, 1, group)
+    assert set(np.unique(codes + (1 << bits))) == set(range((1 << bits) + 1))  # all 2^bits + 1 levels occur
+    assert np.array_equal(f["planes"], oracle.pack_i32(codes, bits + 1))
+    assert np.array_equal(f["scale"], scale.astype(np.float32))
+    assert np.array_equal(f["zero"], zero.astype(np.float32))
+    # refused where the reference has no such mode
+    for extra in (["3", str(group), "asym"], ["2", str(group), "sym"]):
+        out = subprocess.run([TOOL, str(src), str(n), str(k)] + extra + [str(dst), "--bit-balance"], capture_output=True, text=True)
+        assert out.returncode == 1 and "bit balance" in out.stdout
+
+
 def test_converter_symmetric_per_channel(tmp_path, oracle):
     from oracle import quantizer as Q
     _need_tool()
