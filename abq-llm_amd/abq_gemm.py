@@ -28,7 +28,7 @@ ACT_NONE, ACT_SILU_GATE = 0, 1
 # every symbol include/abq_gemm.h declares
 EXPORTED = [
     "abq_status_string", "abq_last_hip_error", "abq_version",
-    "abq_pack_i32", "abq_pack_u4", "abq_pack_f16",
+    "abq_pack_i32", "abq_pack_u4", "abq_pack_f16", "abq_pack_f16_tiled",
     "abq_parse_kernel_name", "abq_format_kernel_name",
     "abq_native_config_count", "abq_native_config_get",
     "abq_gemm_init", "abq_gemm_set_scales", "abq_gemm_exec", "abq_gemm_launch",
@@ -101,6 +101,7 @@ def lib():
         L.abq_pack_i32.argtypes = [vp, vp, ci, ci, ci, vp]
         L.abq_pack_u4.argtypes = [vp, vp, ci, ci, ci, vp]
         L.abq_pack_f16.argtypes = [vp, vp, vp, ci, ci, ci, vp]
+        L.abq_pack_f16_tiled.argtypes = [vp, vp, vp, ci, ci, ci, vp]
         L.abq_parse_kernel_name.argtypes = [ctypes.c_char_p, ctypes.POINTER(TileConfig), ctypes.POINTER(ci)]
         L.abq_format_kernel_name.argtypes = [ctypes.POINTER(TileConfig), ci, ctypes.c_char_p, ctypes.c_size_t]
         L.abq_native_config_count.argtypes = [ci, ci, ci]
@@ -194,16 +195,17 @@ def pack_u4(words, rows, k, bits=4, out=None, stream=None):
     return out
 
 
-def pack_f16(values, scale, bits, out=None, stream=None):
-    """values: fp16 device tensor [rows, k]; scale: float32 device tensor with one element."""
+def pack_f16(values, scale, bits, out=None, stream=None, tiled=False):
+    """values: fp16 device tensor [rows, k]; scale: float32 device tensor with one element.
+    tiled: write the K-tiled layout (what relayout_planes makes of the planes) directly."""
     import torch
     assert values.dtype == torch.float16 and values.is_cuda and values.is_contiguous()
     assert scale.dtype == torch.float32 and scale.is_cuda
     rows, k = values.shape
     if out is None:
         out = planes_empty(bits, rows, k, values.device)
-    _check(lib().abq_pack_f16(values.data_ptr(), scale.data_ptr(), out.data_ptr(), rows, k, bits,
-                              _stream_ptr(stream)), "abq_pack_f16")
+    fn, name = (lib().abq_pack_f16_tiled, "abq_pack_f16_tiled") if tiled else (lib().abq_pack_f16, "abq_pack_f16")
+    _check(fn(values.data_ptr(), scale.data_ptr(), out.data_ptr(), rows, k, bits, _stream_ptr(stream)), name)
     return out
 
 

@@ -15,6 +15,7 @@ namespace abq {
 
 hipError_t launch_pack_i32(const int32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_pack_f16(const void *, const float *, uint32_t *, int, int, int, hipStream_t);
+hipError_t launch_pack_f16_tiled(const void *, const float *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes_fp6(const uint32_t *, uint32_t *, int, int, int, int, hipStream_t);
@@ -487,6 +488,17 @@ abq_status abq_pack_f16(const void *in_f16, const float *scale_dev, uint32_t *pl
     if (!scale_dev)
         return ABQ_ERR_INVALID_ARG;
     return hip_status(launch_pack_f16(in_f16, scale_dev, planes, rows, k, bits, (hipStream_t)stream));
+}
+
+abq_status abq_pack_f16_tiled(const void *in_f16, const float *scale_dev, uint32_t *tiled, int rows, int k, int bits,
+                              void *stream)
+{
+    abq_status s = check_pack(in_f16, tiled, rows, k, bits);
+    if (s != ABQ_OK)
+        return s;
+    if (!scale_dev || bits > 8)
+        return ABQ_ERR_INVALID_ARG;
+    return hip_status(launch_pack_f16_tiled(in_f16, scale_dev, tiled, rows, k, bits, (hipStream_t)stream));
 }
 
 // ---- names -------------------------------------------------------------------------------

@@ -363,6 +363,66 @@ __device__ __forceinline__ void quad_transpose_selectors(int quad_lane, uint32_t
     sel_half = (quad_lane & 2) ? 0x06070203u : 0x00010405u;
 }
 
+// Writes the word-set w (32 elements) of `row` into the field-packed K-tiled records tiled[kt][row][bits * 4];
+// the quad's lane q holds the elements 8q..8q+7 of the word-set, of which the low `bits` bits are kept.
+__device__ __forceinline__ void emit_tiled(const int (&v)[8], uint32_t *tiled, int rows, int row, int w, int quad_lane,
+                                           int bits, bool active, uint32_t sel_pair, uint32_t sel_half)
+{
+    if (bits == 8) {
+        // 8-bit codes are the record's bytes themselves: expanded dword s, byte c = element 31 - (8c + s) of
+        // the word-set = element 7 - s of lane 3 - c.  The quad transposes its bytes so that lane s ends
+        // with the dwords s and 4 + s, and every lane stores its two.
+        const uint32_t e_lo = quad_transpose_bytes(pack_low_bytes(v[7], v[6], v[5], v[4]), sel_pair, sel_half);
+        const uint32_t e_hi = quad_transpose_bytes(pack_low_bytes(v[3], v[2], v[1], v[0]), sel_pair, sel_half);
+        if (active) {
+            uint32_t *dst = tiled + ((size_t)(w >> 2) * rows + row) * 32 + 8 * (w & 3) + quad_lane;
+            dst[0] = e_lo;
+            dst[4] = e_hi;
+        }
+        return;
+    }
+    // expanded dword s, byte c = element 31 - (8c + s) of the word-set: this lane's element
+    // 7 - s goes to byte 3 - quad_lane
+    const uint32_t pattern_mask = (1u << bits) - 1u;
+    uint32_t e[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+        e[s] = quad_or(((uint32_t)v[7 - s] & pattern_mask) << (24 - 8 * quad_lane));
+    if (active && quad_lane == 0)
+        store_fields_any(tiled + ((size_t)(w >> 2) * rows + row) * (bits * 4), w & 3, e, bits);
+}
+
+// pack_f16_kernel's values (fp16 product with the scale, truncated, no clamp: abq_gemm_wrapper.cu:29-54 of the
+// reference), written as field-packed K-tiled records instead of planes: what relayout_planes_kernel makes of
+// pack_f16_kernel's output, in one pass.
+__global__ __launch_bounds__(256) void pack_f16_tiled_kernel(const uint4 *__restrict__ in, const float *__restrict__ scale,
+                                                             uint32_t *__restrict__ tiled, int rows, int units, int bits)
+{
+    const _Float16 hs = (_Float16)scale[0];
+    const size_t n_units = (size_t)rows * units; // units per row: a multiple of 16, so a quad is active as one
+    const size_t rounded = (n_units + 255) / 256 * 256;
+    uint32_t sel_pair, sel_half;
+    quad_transpose_selectors(threadIdx.x & 3, sel_pair, sel_half);
+    for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < rounded; t += (size_t)gridDim.x * 256) {
+        const bool active = t < n_units;
+        int v[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
+        if (active) {
+            union {
+                uint4 u;
+                _Float16 h[8];
+            } raw;
+            raw.u = in[t];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const _Float16 p = raw.h[c] * hs; // fp16 product, rounded to nearest even
+                v[c] = (int)p;                    // truncation
+            }
+        }
+        const int row = (int)(t / units), u = (int)(t % units);
+        emit_tiled(v, tiled, rows, active ? row : 0, u >> 2, u & 3, bits, active, sel_pair, sel_half);
+    }
+}
+
 __device__ __forceinline__ float wave_max(float v)
 {
 #pragma unroll
@@ -516,27 +576,8 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
                 *reinterpret_cast<uint2 *>(rec + 2) = make_uint2(o[2], o[3]);
                 *reinterpret_cast<uint2 *>(rec + 4) = make_uint2(o[4], o[5]);
             }
-        } else if (LAYOUT == 1 && bits == 8) {
-            // 8-bit codes are the record's bytes themselves: expanded dword s, byte c = element 31 - (8c + s) of
-            // the word-set = element 7 - s of lane 3 - c.  The quad transposes its bytes so that lane s ends
-            // with the dwords s and 4 + s, and every lane stores its two.
-            const uint32_t e_lo = quad_transpose_bytes(pack_low_bytes(v[7], v[6], v[5], v[4]), sel_pair, sel_half);
-            const uint32_t e_hi = quad_transpose_bytes(pack_low_bytes(v[3], v[2], v[1], v[0]), sel_pair, sel_half);
-            if (active) {
-                uint32_t *dst = planes + ((size_t)(w >> 2) * M + row) * 32 + 8 * (w & 3) + quad_lane;
-                dst[0] = e_lo;
-                dst[4] = e_hi;
-            }
         } else if (LAYOUT == 1) {
-            // expanded dword s, byte c = element 31 - (8c + s) of the word-set: this lane's element
-            // 7 - s goes to byte 3 - quad_lane
-            const uint32_t pattern_mask = (1u << bits) - 1u;
-            uint32_t e[8];
-#pragma unroll
-            for (int s = 0; s < 8; ++s)
-                e[s] = quad_or(((uint32_t)v[7 - s] & pattern_mask) << (24 - 8 * quad_lane));
-            if (active && quad_lane == 0)
-                store_fields_any(planes + ((size_t)(w >> 2) * M + row) * (bits * 4), w & 3, e, bits);
+            emit_tiled(v, planes, M, row, w, quad_lane, bits, active, sel_pair, sel_half);
         } else {
             const uint64_t bytes = eight_values_to_plane_bytes(v);
             for (int b = 0; b < bits; ++b) {
@@ -626,6 +667,15 @@ hipError_t launch_pack_i32(const int32_t *in, uint32_t *planes, int rows, int k,
     const size_t n_units = (size_t)rows * k / 8;
     hipLaunchKernelGGL(pack_i32_kernel, dim3(grid_for(n_units)), dim3(256), 0, stream,
                        reinterpret_cast<const int4 *>(in), planes, n_units, bits);
+    return hipGetLastError();
+}
+
+hipError_t launch_pack_f16_tiled(const void *in, const float *scale, uint32_t *tiled, int rows, int k, int bits,
+                                 hipStream_t stream)
+{
+    const size_t n_units = (size_t)rows * k / 8;
+    hipLaunchKernelGGL(pack_f16_tiled_kernel, dim3(grid_for(n_units)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint4 *>(in), scale, tiled, rows, k / 8, bits);
     return hipGetLastError();
 }
 

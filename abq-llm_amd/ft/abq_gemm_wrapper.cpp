@@ -6,7 +6,77 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <mutex>
+#include <unordered_map>
+
 #include "abq_gemm.h"
+
+namespace {
+
+struct PreparedWeight {
+    int N, K, bits;
+};
+
+std::mutex g_prepared_mutex;
+
+std::unordered_map<const void *, PreparedWeight> &prepared_table()
+{
+    static std::unordered_map<const void *, PreparedWeight> table;
+    return table;
+}
+
+bool find_prepared(const void *B, PreparedWeight *out)
+{
+    std::lock_guard<std::mutex> lock(g_prepared_mutex);
+    const auto it = prepared_table().find(B);
+    if (it == prepared_table().end())
+        return false;
+    *out = it->second;
+    return true;
+}
+
+} // namespace
+
+size_t ABQGEMMWrapper::prepared_weight_bytes(int N, int K, int W_BITS) { return abq_planes_bytes(N, K, W_BITS); }
+
+bool ABQGEMMWrapper::prepare_weight(int *B, int N, int K, int W_BITS, int *scratch, hipStream_t stream)
+{
+    if (!B || !scratch || N <= 0 || K < 128 || K % 128 != 0 || W_BITS < 1 || W_BITS > 8) {
+        printf("[ABQ][Error] prepare_weight: bad argument (N, K, bits = %d, %d, %d)\n", N, K, W_BITS);
+        return false;
+    }
+    PreparedWeight seen;
+    if (find_prepared(B, &seen)) {
+        printf("[ABQ][Error] prepare_weight: %p is prepared already\n", (void *)B);
+        return false;
+    }
+    const abq_status rc = abq_relayout_planes(reinterpret_cast<const uint32_t *>(B), reinterpret_cast<uint32_t *>(scratch),
+                                              N, K, W_BITS, stream);
+    if (rc != ABQ_OK) {
+        printf("[ABQ][Error] prepare_weight failed: %s\n", abq_status_string(rc));
+        return false;
+    }
+    const hipError_t e = hipMemcpyAsync(B, scratch, abq_planes_bytes(N, K, W_BITS), hipMemcpyDeviceToDevice, stream);
+    if (e != hipSuccess) {
+        printf("[ABQ][Error] prepare_weight failed: %s\n", hipGetErrorString(e));
+        return false;
+    }
+    std::lock_guard<std::mutex> lock(g_prepared_mutex);
+    prepared_table()[B] = PreparedWeight{ N, K, W_BITS };
+    return true;
+}
+
+void ABQGEMMWrapper::release_weight(const int *B)
+{
+    std::lock_guard<std::mutex> lock(g_prepared_mutex);
+    prepared_table().erase(B);
+}
+
+bool ABQGEMMWrapper::is_prepared(const int *B)
+{
+    PreparedWeight w;
+    return find_prepared(B, &w);
+}
 
 ABQGEMMWrapper::ABQGEMMWrapper(int X_BITS, int W_BITS, bool SIGNED) : x_bits_(X_BITS), w_bits_(W_BITS), signed_(SIGNED) {}
 
@@ -41,17 +111,34 @@ void ABQGEMMWrapper::gemm(const int M, const int N, const int K, const _Float16 
         printf("[ABQ][Error] workspace too small: %zu bytes for M,K,bits = %d,%d,%d\n", abq_gemm_ws_bytes, M, K, x_bits_);
         return;
     }
-    // quant + packing
-    pack(A, scale, reinterpret_cast<int *>(abq_gemm_workspace), M, K, x_bits_, stream);
+    PreparedWeight prepared;
+    const bool tiled = find_prepared(B, &prepared);
+    if (tiled && (prepared.N != N || prepared.K != K || prepared.bits != w_bits_)) {
+        printf("[ABQ][Error] weight prepared as N, K, bits = %d, %d, %d, called with %d, %d, %d\n", prepared.N, prepared.K,
+               prepared.bits, N, K, w_bits_);
+        return;
+    }
+    // quant + packing; for a prepared weight straight into the layout its kernels read
+    if (tiled) {
+        const abq_status prc = abq_pack_f16_tiled(A, scale, reinterpret_cast<uint32_t *>(abq_gemm_workspace), M, K, x_bits_, stream);
+        if (prc != ABQ_OK) {
+            printf("[ABQ][Error] pack failed: %s\n", abq_status_string(prc));
+            return;
+        }
+    } else {
+        pack(A, scale, reinterpret_cast<int *>(abq_gemm_workspace), M, K, x_bits_, stream);
+    }
     abq_gemm_state state;
-    const abq_status rc = abq_gemm_init(nullptr, x_bits_, w_bits_, signed_ ? 1 : 0,
-                                        reinterpret_cast<const uint32_t *>(abq_gemm_workspace),
-                                        reinterpret_cast<const uint32_t *>(B), M, N, K, D, scale_out, bias ? 1 : 0,
-                                        ABQ_OUT_F16_TENSOR_F32SCALE, &state);
+    abq_status rc = abq_gemm_init(nullptr, x_bits_, w_bits_, signed_ ? 1 : 0,
+                                  reinterpret_cast<const uint32_t *>(abq_gemm_workspace),
+                                  reinterpret_cast<const uint32_t *>(B), M, N, K, D, scale_out, bias ? 1 : 0,
+                                  ABQ_OUT_F16_TENSOR_F32SCALE, &state);
     if (rc == ABQ_ERR_UNSUPPORTED) {
         printf("[ABQ][Error] unsupport w%da%d\n", w_bits_, x_bits_);
         return;
     }
+    if (rc == ABQ_OK && tiled)
+        rc = abq_gemm_set_operand_layout(&state, ABQ_LAYOUT_TILED, ABQ_LAYOUT_TILED);
     if (rc != ABQ_OK || !state.init_success) {
         printf("[ABQ][Error] return due to unsuccessful initialization.\n");
         return;

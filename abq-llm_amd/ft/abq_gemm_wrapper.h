@@ -12,6 +12,8 @@
 //  * scale_out[0] is read as the float it is (the reference reinterprets the pointer as half*
 //    and reads the low 16 bits of the float, abq_gemm_wrapper.cu:126);
 //  * the workspace size is checked.
+// prepare_weight() is new: a loader calls it once per weight matrix; gemm() then runs the kernels built for
+// the prepared (K-tiled) layout, for prefill and decode, with unchanged call sites.
 // gemm_scaled() is new: per-token activation scales and per-channel weight scales.
 // gemm_dynamic() is new: per-token dynamic activation quantisation on the device, group-wise
 // weight scales and zero points (the quantiser semantics of algorithm/quantize/quantizer.py).
@@ -46,6 +48,21 @@ public:
     void pack(const int *in_data, int *packed_data, int M, int K, int BIT, hipStream_t stream);
     void pack(const _Float16 *in_data, const float *scale, int *packed_data, int M, int K, int BIT,
               hipStream_t stream);
+    // One-time weight preparation for gemm() (no counterpart in the reference, whose kernels stop at M = 8; belongs
+    // after the loader's reads of the plane files, LlamaDecoderLayerWeight.cc:377-400).  Rewrites the W_BITS planes at
+    // B, [W_BITS][N][K/32] device words, in place as K-tiled records (same size) through `scratch`, device memory
+    // of prepared_weight_bytes(N, K, W_BITS) that may be freed or reused once `stream` has passed this call, and
+    // enters B into a process-wide table.  Every later gemm() of any wrapper whose B is this pointer packs its
+    // activations into the same layout and runs the LDS-staged prefill kernel (M > 16) or the decode kernel on
+    // prepared operands (M <= 16) with no conversion inside the call; a B that was never prepared keeps the plane
+    // kernels.  B must not be handed to gemm_scaled() or to ABQGroupedWeight::planes afterwards.  Returns false
+    // (after "[ABQ][Error] ...") on a bad argument or a failed launch.  release_weight() takes B out of the table
+    // (before its memory is freed or refilled).  The table is guarded by a mutex.
+    static size_t prepared_weight_bytes(int N, int K, int W_BITS);
+    static bool prepare_weight(int *B, int N, int K, int W_BITS, int *scratch, hipStream_t stream);
+    static void release_weight(const int *B);
+    static bool is_prepared(const int *B);
+
     // A: fp16 activations [M][K]; B: packed weight planes [w_bits][N][K/32]; C unused;
     // D: fp16 [M][N]; scale: activation quantisation scale (1 float, device);
     // scale_inter unused; scale_out: output scale (1 float, device);

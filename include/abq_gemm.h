@@ -280,6 +280,12 @@ size_t abq_planes_bytes(int rows, int k, int bits);
 abq_status abq_relayout_planes(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits,
                                void *stream);
 
+/* abq_pack_f16 (pack_half of the reference, abq_gemm_wrapper.cu:29-69: same values, same scale) writing the
+ * K-tiled layout directly: bit for bit what abq_relayout_planes makes of abq_pack_f16's planes, without the
+ * second pass.  bits <= 8, k % 128 == 0. */
+abq_status abq_pack_f16_tiled(const void *in_f16, const float *scale_dev, uint32_t *tiled, int rows, int k, int bits,
+                              void *stream);
+
 /* FP6 records (no counterpart in the reference): the operand format of ABQ_STRATEGY_FP6.
  * CDNA4's matrix cores multiply 6-bit floats (E2M3) at twice their int8 rate, and an integer of
  * magnitude <= 16 written as sign and magnitude is an E2M3 number (value / 8), so operands that

@@ -218,6 +218,91 @@ static void gpu_paths()
         HIP_OK(hipFree(d_ws));
     }
 
+    {   // FT wrapper on a prepared weight: gemm() with unchanged arguments, prefill- and decode-sized, bit-equal
+        // to the same call on the plane weight; timed beside it
+        const int N = 4096, K = 4096, Mmax = 1024;
+        std::mt19937 r32(11);
+        std::normal_distribution<float> nd(0.f, 2.f);
+        std::vector<uint16_t> ha((size_t)Mmax * K);
+        for (auto &h : ha)
+            h = abq_oracle_f32_to_f16(nd(r32));
+        std::vector<uint32_t> wpl((size_t)2 * N * K / 32);
+        for (auto &v : wpl)
+            v = r32();
+        _Float16 *d_a, *d_d0, *d_d1;
+        int *d_b0, *d_b1, *d_scratch;
+        float *d_scales;
+        char *d_ws;
+        const size_t ws_bytes = (size_t)8 * Mmax * K / 8, wbytes = wpl.size() * 4;
+        CHECK(ABQGEMMWrapper::prepared_weight_bytes(N, K, 2) == wbytes);
+        HIP_OK(hipMalloc(&d_a, ha.size() * 2));
+        HIP_OK(hipMalloc(&d_d0, (size_t)Mmax * N * 2));
+        HIP_OK(hipMalloc(&d_d1, (size_t)Mmax * N * 2));
+        HIP_OK(hipMalloc(&d_b0, wbytes));
+        HIP_OK(hipMalloc(&d_b1, wbytes));
+        HIP_OK(hipMalloc(&d_scratch, wbytes));
+        HIP_OK(hipMalloc(&d_scales, 8));
+        HIP_OK(hipMalloc(&d_ws, ws_bytes));
+        HIP_OK(hipMemcpy(d_a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(d_b0, wpl.data(), wbytes, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(d_b1, wpl.data(), wbytes, hipMemcpyHostToDevice));
+        const float scales[2] = { 21.0f, 0.0123f };
+        HIP_OK(hipMemcpy(d_scales, scales, 8, hipMemcpyHostToDevice));
+        CHECK(!ABQGEMMWrapper::is_prepared(d_b1));
+        CHECK(!ABQGEMMWrapper::prepare_weight(d_b1, N, 100, 2, d_scratch, stream)); // K not a multiple of 128
+        CHECK(ABQGEMMWrapper::prepare_weight(d_b1, N, K, 2, d_scratch, stream));
+        CHECK(ABQGEMMWrapper::is_prepared(d_b1) && !ABQGEMMWrapper::is_prepared(d_b0));
+        CHECK(!ABQGEMMWrapper::prepare_weight(d_b1, N, K, 2, d_scratch, stream)); // twice
+        ABQGEMMWrapper wrap(8, 2, true);
+        hipEvent_t e0, e1;
+        HIP_OK(hipEventCreate(&e0));
+        HIP_OK(hipEventCreate(&e1));
+        for (int M : { 1024, 300, 16, 1 }) {
+            float us[2] = { 0.f, 0.f };
+            for (int prepared = 0; prepared < 2; ++prepared) {
+                _Float16 *d_d = prepared ? d_d1 : d_d0;
+                const int *d_b = prepared ? d_b1 : d_b0;
+                HIP_OK(hipMemsetAsync(d_d, 0xff, (size_t)M * N * 2, stream));
+                const int reps = 20;
+                for (int it = 0; it < reps + 2; ++it) {
+                    if (it == 2)
+                        HIP_OK(hipEventRecord(e0, stream));
+                    wrap.gemm(M, N, K, d_a, d_b, nullptr, d_d, d_scales, nullptr, d_scales + 1, false, d_ws, ws_bytes, stream);
+                }
+                HIP_OK(hipEventRecord(e1, stream));
+                HIP_OK(hipStreamSynchronize(stream));
+                float ms = 0.f;
+                HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+                us[prepared] = ms * 1000.f / reps;
+            }
+            std::vector<uint16_t> got0((size_t)M * N), got1((size_t)M * N);
+            HIP_OK(hipMemcpy(got0.data(), d_d0, got0.size() * 2, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(got1.data(), d_d1, got1.size() * 2, hipMemcpyDeviceToHost));
+            CHECK(got0 == got1);
+            printf("  gemm() W2A8 M = %4d, N = K = 4096 (pack + GEMM per call): plane weight %.1f us, prepared weight %.1f us\n", M,
+                   us[0], us[1]);
+        }
+        // a prepared weight is checked against the shape it was prepared for: D stays as it was
+        HIP_OK(hipMemset(d_d1, 0xff, 64));
+        wrap.gemm(1, N / 2, K, d_a, d_b1, nullptr, d_d1, d_scales, nullptr, d_scales + 1, false, d_ws, ws_bytes, stream);
+        HIP_OK(hipStreamSynchronize(stream));
+        uint16_t first = 0;
+        HIP_OK(hipMemcpy(&first, d_d1, 2, hipMemcpyDeviceToHost));
+        CHECK(first == 0xffff);
+        ABQGEMMWrapper::release_weight(d_b1);
+        CHECK(!ABQGEMMWrapper::is_prepared(d_b1));
+        HIP_OK(hipEventDestroy(e0));
+        HIP_OK(hipEventDestroy(e1));
+        HIP_OK(hipFree(d_a));
+        HIP_OK(hipFree(d_d0));
+        HIP_OK(hipFree(d_d1));
+        HIP_OK(hipFree(d_b0));
+        HIP_OK(hipFree(d_b1));
+        HIP_OK(hipFree(d_scratch));
+        HIP_OK(hipFree(d_scales));
+        HIP_OK(hipFree(d_ws));
+    }
+
     {   // FT wrapper, dynamic path: per-token int8 activations, 2-bit weights with group scales and
         // zero points; expected values from a double-precision loop over the dequantised operands
         const int M = 40, N = 192, K = 512, G = 128, groups = K / G;

@@ -82,6 +82,19 @@ def test_pack_f16_all_finite_bit_patterns(abq, oracle, scale):
         assert np.array_equal(got & mask, want & mask)
 
 
+@pytest.mark.parametrize("rows,k", [(1, 128), (5, 4096), (16, 11008), (300, 512), (1024, 4096)])
+def test_pack_f16_tiled_equals_the_relayout_of_the_planes(abq, rows, k):
+    """abq_pack_f16_tiled writes in one pass what abq_relayout_planes makes of abq_pack_f16's planes."""
+    g = torch.Generator(device="cuda").manual_seed(rows + k)
+    x = (torch.randn((rows, k), generator=g, device="cuda") * 3).to(torch.float16)
+    s = torch.tensor([127.0 / 6.0], dtype=torch.float32, device="cuda")
+    for bits in range(1, 9):
+        want = abq.relayout_planes(abq.pack_f16(x, s, bits))
+        got = abq.pack_f16(x, s, bits, tiled=True)
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(-1), want.view(-1)), bits
+
+
 def field_packed(patterns, bits):
     """The K-tiled, field-packed layout written out from its definition: patterns [rows, K] are the
     elements' bit patterns (low `bits` bits).  A row's K tile of 128 elements is one record of
