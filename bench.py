@@ -40,13 +40,13 @@ ROTATE_BYTES = 512 << 20
 
 # HBM bytes per launch of the dominant kernel, averaged over this workload's nine GEMMs, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled by a plain copy of known size
-# (the summary with the commands is kept under profiles/, decode_w2a8_bench_hbm_traffic).  Reported only for the
+# (the summary with the commands is kept under profiles/, decode_w2a8_prepared_bench_hbm_traffic).  Reported only for the
 # kernel it was measured on.
 MEASURED_TRAFFIC_BYTES = {
     "decode:AqBMMA_8x2xtrue_16x16x8192_16x16x512_16x16x64_3": 9358234,
 }
 # one figure for the whole headline workload when its GEMMs run on several tile tuples of one kernel family
-MEASURED_TRAFFIC_BYTES_DECODE_TILED = None
+MEASURED_TRAFFIC_BYTES_DECODE_TILED = 9306992
 
 
 def log(*a):
