@@ -39,7 +39,8 @@ hipError_t launch_weight_zero_term(const uint32_t *, int, int, int, int, const f
     void abq_decode_grouped_register_##Q##_##P(KernelTable *); \
     void abq_tiled_register_##Q##_##P(KernelTable *);  \
     void abq_tiled_grouped_register_##Q##_##P(KernelTable *);  \
-    void abq_decode_tiled_register_##Q##_##P(KernelTable *);
+    void abq_decode_tiled_register_##Q##_##P(KernelTable *); \
+    void abq_decode_tiled_grouped_register_##Q##_##P(KernelTable *);
 ABQ_FOR_EACH_COMBO(ABQ_DECL)
 #undef ABQ_DECL
 
@@ -51,6 +52,7 @@ struct Registry {
     KernelTable tiled[2 * ABQ_NUM_COMBOS];
     KernelTable tiled_grouped[2 * ABQ_NUM_COMBOS];
     KernelTable decode_tiled[2 * ABQ_NUM_COMBOS];
+    KernelTable decode_tiled_grouped[2 * ABQ_NUM_COMBOS];
     Registry()
     {
         int i = 0;
@@ -62,6 +64,7 @@ struct Registry {
     abq_tiled_register_##Q##_##P(&tiled[i]);           \
     abq_tiled_grouped_register_##Q##_##P(&tiled_grouped[i]); \
     abq_decode_tiled_register_##Q##_##P(&decode_tiled[i]); \
+    abq_decode_tiled_grouped_register_##Q##_##P(&decode_tiled_grouped[i]); \
     i += 2;
         ABQ_FOR_EACH_COMBO(ABQ_REG)
 #undef ABQ_REG
@@ -896,6 +899,16 @@ static abq_status switch_to_decode_tiled(abq_gemm_state *st)
     return ABQ_OK;
 }
 
+// Group scales on a decode-sized GEMM whose operands are (or are about to be declared) both prepared: whether the
+// decode kernel of that layout has a group-scale variant for the pair that fits this shape.
+static bool decode_tiled_grouped_fits(const abq_gemm_state *st, int group_size, int act)
+{
+    const abq_tile_config &c = st->cfg;
+    const KernelTable *t = find_table(registry().decode_tiled_grouped, c.x_bits, c.w_bits, c.is_signed);
+    return t && t->count > 0 && st->auto_chosen && st->M <= 16 && group_size == 128 && (!act || st->N % 32 == 0) &&
+           decode_tiled_grouped_rows(16, act ? 2 : 1, st->M, st->K, c.x_bits) != 0;
+}
+
 // Moves a state with group scales onto the tiled kernel's group-scale variants.
 static abq_status pick_grouped_tiled(abq_gemm_state *state)
 {
@@ -969,19 +982,22 @@ abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, cons
             return ABQ_ERR_INVALID_ARG;
         if (!c.is_signed && (c.x_bits == 8 || c.w_bits == 8))
             return ABQ_ERR_UNSUPPORTED;
+        const abq_gemm_state before = *state; // a failed call leaves the state as it was
         state->group_size = group_size;
         if (state->strategy == ABQ_STRATEGY_BCNT && state->auto_chosen && state->M <= 16)
             switch_to_decode(state); // the popcount kernel has no group-scale epilogue
+        // both operands prepared: the decode kernel of that layout has its own group-scale variant
+        const bool decode_tiled_ok = state->strategy == ABQ_STRATEGY_DECODE_TILED && decode_tiled_grouped_fits(state, group_size, state->act);
         const bool decode_ok = state->strategy == ABQ_STRATEGY_DECODE && state->auto_chosen && state->M <= 16 &&
                                state->x_layout == ABQ_LAYOUT_PLANES && state->w_layout == ABQ_LAYOUT_PLANES &&
                                decode_grouped_lds(state->M, state->K, group_size) != 0 &&
                                find_table(registry().decode_grouped, c.x_bits, c.w_bits, c.is_signed);
-        if (decode_ok) {
+        if (decode_ok || decode_tiled_ok) {
             state->variant = 0;
         } else {
             const abq_status rc = pick_grouped_tiled(state);
             if (rc != ABQ_OK) {
-                state->group_size = 0;
+                *state = before;
                 return rc;
             }
         }
@@ -1022,8 +1038,9 @@ abq_status abq_gemm_set_activation(abq_gemm_state *state, int act)
         if (state->N % 32 != 0)
             return ABQ_ERR_INVALID_ARG;
         // the decode kernel needs a gate tile and its up tile in one LDS pass
-        if (state->strategy == ABQ_STRATEGY_DECODE &&
-            decode_grouped_lds(state->M, state->K, state->group_size) + (size_t)kDecodeGroupedWaves * 1024 > 160 * 1024) {
+        if ((state->strategy == ABQ_STRATEGY_DECODE &&
+             decode_grouped_lds(state->M, state->K, state->group_size) + (size_t)kDecodeGroupedWaves * 1024 > 160 * 1024) ||
+            (state->strategy == ABQ_STRATEGY_DECODE_TILED && !decode_tiled_grouped_fits(state, state->group_size, act))) {
             const abq_status rc = pick_grouped_tiled(state);
             if (rc != ABQ_OK)
                 return rc;
@@ -1205,11 +1222,10 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
                 return hip_status(e);
             a.W = reinterpret_cast<const uint32_t *>(ws + xb);
         }
-        if (st->strategy == ABQ_STRATEGY_DECODE_TILED && (st->group_size || st->act))
-            return ABQ_ERR_NOT_INITIALIZED; // plain and per-channel epilogues only
-        const KernelTable *t = find_table(st->strategy == ABQ_STRATEGY_DECODE_TILED ? reg.decode_tiled
-                                          : st->group_size                          ? reg.tiled_grouped
-                                                                                    : reg.tiled,
+        const KernelTable *t = find_table(st->strategy == ABQ_STRATEGY_DECODE_TILED
+                                              ? (st->group_size ? reg.decode_tiled_grouped : reg.decode_tiled)
+                                          : st->group_size ? reg.tiled_grouped
+                                                           : reg.tiled,
                                           c.x_bits, c.w_bits, c.is_signed);
         if (!t || st->variant < 0 || st->variant >= t->count)
             return ABQ_ERR_NOT_INITIALIZED;
@@ -1305,6 +1321,14 @@ abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_l
     // decode-sized M with both operands prepared: the decode kernel of that layout (plain and per-channel epilogues)
     if (x_layout == ABQ_LAYOUT_TILED && w_layout == ABQ_LAYOUT_TILED && st->auto_chosen && st->M <= 16 && !st->group_size &&
         !st->act && st->strategy != ABQ_STRATEGY_DECODE_TILED && switch_to_decode_tiled(st) == ABQ_OK) {
+        st->x_layout = x_layout;
+        st->w_layout = w_layout;
+        return ABQ_OK;
+    }
+    // the same with group scales attached before the layouts were declared
+    if (x_layout == ABQ_LAYOUT_TILED && w_layout == ABQ_LAYOUT_TILED && st->group_size && st->strategy != ABQ_STRATEGY_DECODE_TILED &&
+        decode_tiled_grouped_fits(st, st->group_size, st->act) && switch_to_decode_tiled(st) == ABQ_OK) {
+        st->variant = 0;
         st->x_layout = x_layout;
         st->w_layout = w_layout;
         return ABQ_OK;

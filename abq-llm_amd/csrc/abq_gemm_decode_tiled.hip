@@ -74,6 +74,11 @@ __device__ __forceinline__ void dt_wait_loads_n(int n)
     case 4: dt_wait_loads<4>(); break;
     case 5: dt_wait_loads<5>(); break;
     case 6: dt_wait_loads<6>(); break;
+    case 8: dt_wait_loads<8>(); break;
+    case 10: dt_wait_loads<10>(); break;
+    case 12: dt_wait_loads<12>(); break;
+    case 16: dt_wait_loads<16>(); break;
+    case 20: dt_wait_loads<20>(); break;
     default: dt_wait_loads<0>(); break;
     }
 }
@@ -288,6 +293,320 @@ static hipError_t launch_decode_tiled(const GemmArgs &a, hipStream_t stream)
     return hipGetLastError();
 }
 
+// ---- the same plan with group-wise weight scales -------------------------------------------------
+//
+// D[m][n] = x_scale[m] * ( sum_g w_scale[n][g] * (acc_g - w_zero[n][g] * Sx[m][g]) - x_zero[m] * T[n] ),
+// acc_g the integer dot product over scale group g; semantics of algorithm/quantize/quantizer.py:111-179 of the
+// reference, groups of 128, fp16 output, optionally the fused SiLU gate (tile pairs: 16 gate rows, their 16 up rows).
+//
+// A matrix-core instruction sums over its four lane groups, so all four must hold elements of the same scale
+// group: a step is ONE K tile (= one group of 128) here, lane group g holds 32 of its elements (4 P bytes of the
+// weight record: an 8-, 16- or 32-byte load; the two 16-byte pieces 2g, 2g + 1 of an 8-bit activation record), and
+// the step's two instructions leave acc_g itself, which is folded into fp32 with the group's scale right away.  For
+// 2-bit weights the sixteen records of a tile's K tile are 512 contiguous bytes: one wave load covers them exactly.
+// The scales, zero points and activation group sums of the workgroup's rows are staged in LDS as [group][16 rows]
+// by four-byte DMA loads issued with the activations (no register, no wait before the weight loads; issuing them
+// behind the weight loads and waiting for everything was 0.2 to 0.5 us slower), so the fold reads them with
+// conflict-free ds_reads instead of a gather per step.  All the waves of a
+// compute unit share one LDS pipeline, so bank conflicts on these reads cost real time here: with the rows stored
+// as they lie in memory ([16 rows][groups], a column read is 8-way conflicted at 32 groups) the zero-point variant
+// took 0.5 to 1 us longer.
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void dt_dma_dword(const void *src, unsigned lds_addr)
+{
+    // lane l of the wave lands at lds_addr + 4 * l
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)
+                 : "memory");
+}
+
+// a lane's share of one weight record (32 elements): P dwords
+template <int P> struct DtgShare {
+    v4u v[P / 4];
+    static constexpr int kLoads = P / 4;
+    __device__ __forceinline__ void issue(const char *base, uint32_t off)
+    {
+#pragma unroll
+        for (int i = 0; i < P / 4; ++i)
+            v[i] = dt_load16(base, off + 16u * i);
+    }
+    __device__ __forceinline__ void landed()
+    {
+#pragma unroll
+        for (int i = 0; i < P / 4; ++i)
+            dt_landed(v[i]);
+    }
+};
+template <> struct DtgShare<2> {
+    v2u v;
+    static constexpr int kLoads = 1;
+    __device__ __forceinline__ void issue(const char *base, uint32_t off)
+    {
+        asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(v) : "v"(off), "s"(base) : "memory");
+    }
+    __device__ __forceinline__ void landed() { asm volatile("" : "+v"(v)); }
+};
+
+// one dword of a 2-bit record -> one MFMA operand
+template <bool SIGNED> __device__ __forceinline__ v4i dtg_unpack2(uint32_t w)
+{
+    if (SIGNED)
+        return v4i{ (int)((w << 6) & 0xC0C0C0C0u), (int)((w << 4) & 0xC0C0C0C0u), (int)((w << 2) & 0xC0C0C0C0u), (int)(w & 0xC0C0C0C0u) };
+    return v4i{ (int)(w & 0x03030303u), (int)((w >> 2) & 0x03030303u), (int)((w >> 4) & 0x03030303u), (int)((w >> 6) & 0x03030303u) };
+}
+
+template <int P, bool SIGNED> __device__ __forceinline__ void dtg_operands(const DtgShare<P> &w, v4i (&bv)[2])
+{
+    if constexpr (P == 2) {
+        bv[0] = dtg_unpack2<SIGNED>(w.v[0]);
+        bv[1] = dtg_unpack2<SIGNED>(w.v[1]);
+    } else if constexpr (P == 4) {
+        dt_unpack<4, SIGNED>(w.v[0], bv);
+    } else {
+        bv[0] = v4i{ (int)w.v[0][0], (int)w.v[0][1], (int)w.v[0][2], (int)w.v[0][3] };
+        bv[1] = v4i{ (int)w.v[1][0], (int)w.v[1][1], (int)w.v[1][2], (int)w.v[1][3] };
+    }
+}
+
+template <int Q, int P, bool SIGNED, int NW, int D, int T>
+__global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmArgs a, int mrows)
+{
+    constexpr int NT = 64 * NW;
+    constexpr int QLOG = Q == 8 ? 3 : Q == 4 ? 2 : 1;
+    constexpr int LPS = DtgShare<P>::kLoads; // loads per step and tile
+    extern __shared__ __align__(16) unsigned char smem[];
+    float *red = reinterpret_cast<float *>(smem); // [NW][T][16][16]
+    unsigned char *xs = smem + NW * T * 1024;     // [kt][row][Q chunks], chunks permuted within a row
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int M = a.M, N = a.N;
+    const int KT = a.K >> 7; // K tiles = scale groups = steps
+    const int tile0 = blockIdx.x * T;
+    const int m0 = blockIdx.y * mrows;
+    const int Mb = min(mrows, M - m0);
+    const char *Xt = reinterpret_cast<const char *>(a.X);
+    const char *Wt = reinterpret_cast<const char *>(a.W);
+    const unsigned xs_addr = (unsigned)(size_t)xs;
+    const int xchunks = KT * Mb * Q;
+    const int per_arr = (KT * 16 + 63) & ~63; // floats of one [group][16] array, in whole wave loads
+    float *sws = reinterpret_cast<float *>(xs + (size_t)mrows * (KT + 1) * Q * 16 + 1024); // [T][group][16]
+    float *zws = sws + T * per_arr;                                                       // [T][group][16]
+    int *sxs = reinterpret_cast<int *>(zws + T * per_arr);                                // [group][16]
+    const bool zp = a.w_zero != nullptr;
+
+    // ---- activations: LDS chunk p <- chunk p ^ ((p / Q) & (Q - 1)) of the workgroup's rows -----------
+    {
+        const int per = Mb * Q;
+        for (int pb = wid * 64; pb < xchunks; pb += NT) {
+            const int p = min(pb + lane, xchunks - 1);
+            const int q = p ^ ((p >> QLOG) & (Q - 1));
+            size_t src = (size_t)q;
+            if (Mb != M) { // several blocks of rows: a K tile's rows are Mb * Q chunks out of M * Q
+                const int kt = q / per, rem = q - kt * per;
+                src = (size_t)(kt * M + m0) * Q + rem;
+            }
+            dt_load_to_lds(Xt + src * 16u, xs_addr + (unsigned)pb * 16u);
+        }
+    }
+    // ---- scales, zero points of the tiles' rows and group sums of the activation rows: [group][16] ----
+    {
+        const int nfl = KT * 16;
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            for (int pb = wid * 64; pb < nfl; pb += NT) {
+                const int p = min(pb + lane, nfl - 1);
+                const int n = min((tile0 + t) * 16 + (p & 15), N - 1);
+                const size_t src = (size_t)n * KT + (p >> 4);
+                dt_dma_dword(a.w_scale + src, (unsigned)(size_t)(sws + t * per_arr + pb));
+                if (zp)
+                    dt_dma_dword(a.w_zero + src, (unsigned)(size_t)(zws + t * per_arr + pb));
+            }
+        }
+        if (zp) {
+            for (int pb = wid * 64; pb < nfl; pb += NT) {
+                const int p = min(pb + lane, nfl - 1);
+                const int m = m0 + min(p & 15, Mb - 1);
+                dt_dma_dword(a.x_group_sums + (size_t)m * KT + (p >> 4), (unsigned)(size_t)(sxs + pb));
+            }
+        }
+    }
+
+    // ---- weights: byte offset of (lane, step s, tile t) = s * N * 16 P + woff[t] ----------------------
+    uint32_t woff[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        const int n = min((tile0 + t) * 16 + r, N - 1);
+        woff[t] = (uint32_t)n * (P * 16u) + (uint32_t)g * (4u * P);
+    }
+    const uint32_t step_bytes = (uint32_t)N * (P * 16u);
+
+    float facc[T][4];
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            facc[t][e] = 0.f;
+    const int ml = min(r, Mb - 1);
+    // the signed route feeds value * 2^(8 - bits): the exact power of two that undoes it rides on the scale
+    const float unshift = SIGNED ? 1.0f / (float)(1 << (16 - Q - P)) : 1.0f;
+
+    int round = 0;
+    do {
+        DtgShare<P> wb[D][T];
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int s = min(wid + (round * D + d) * NW, KT - 1); // steps past the end repeat the last one
+            const char *wp = Wt + (size_t)s * step_bytes;
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+                wb[d][t].issue(wp, woff[t]);
+        }
+        if (round == 0) {
+            dt_wait_loads<D * T * LPS>(); // the DMA loads are older than these
+            __syncthreads();
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int cs = wid + (round * D + d) * NW;
+            const bool have = cs < KT; // wave-uniform
+            v4i av[2];
+            float sw[T], zs[T], sxf[4];
+            if (have) {
+                const int rowi = cs * Mb + ml; // row index in LDS: K tile * rows + row
+                const unsigned char *xrow = xs + (uint32_t)rowi * (Q * 16u);
+                if (Q == 8) {
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        const v4u xv = *reinterpret_cast<const v4u *>(xrow + (((2 * g + i) ^ (rowi & 7)) * 16u));
+                        av[i] = v4i{ (int)xv[0], (int)xv[1], (int)xv[2], (int)xv[3] };
+                    }
+                } else if (Q == 4) {
+                    const v4u xv = *reinterpret_cast<const v4u *>(xrow + ((g ^ (rowi & 3)) * 16u));
+                    dt_unpack<4, SIGNED>(xv, av);
+                } else {
+                    const v4u xv = *reinterpret_cast<const v4u *>(xrow + (((g >> 1) ^ (rowi & 1)) * 16u));
+                    av[0] = dtg_unpack2<SIGNED>((g & 1) ? xv[2] : xv[0]);
+                    av[1] = dtg_unpack2<SIGNED>((g & 1) ? xv[3] : xv[1]);
+                }
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    sw[t] = sws[t * per_arr + cs * 16 + r];
+                    zs[t] = zp ? sw[t] * zws[t * per_arr + cs * 16 + r] : 0.f;
+                    sw[t] *= unshift;
+                }
+                if (zp) {
+                    const v4i sx = *reinterpret_cast<const v4i *>(sxs + cs * 16 + 4 * g);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        sxf[e] = (float)sx[e];
+                } else {
+                    sxf[0] = sxf[1] = sxf[2] = sxf[3] = 0.f;
+                }
+            }
+            // Waited for and marked as landed on every path: a register with a load still in flight must not
+            // look free to the compiler.
+            dt_wait_loads_n((D - 1 - d) * T * LPS);
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+                wb[d][t].landed();
+            if (have) {
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    v4i bv[2];
+                    dtg_operands<P, SIGNED>(wb[d][t], bv);
+                    v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[0], bv[0], v4i{ 0, 0, 0, 0 }, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[1], bv[1], acc, 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        facc[t][e] += sw[t] * (float)acc[e] - zs[t] * sxf[e];
+                }
+            }
+        }
+        ++round;
+    } while (wid + round * D * NW < KT);
+
+    // ---- the waves' partial tiles meet in LDS, summed in a fixed order ---------------------------------
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            red[((wid * T + t) * 16 + 4 * g + e) * 16 + r] = facc[t][e];
+    __syncthreads();
+    for (int o = tid; o < T * 256; o += NT) {
+        const int t = o >> 8, rem = o & 255, i = rem >> 4, c = rem & 15;
+        const int n = (tile0 + t) * 16 + c;
+        if (i < Mb && n < N && !(a.act && (t & 1))) {
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w)
+                v += red[(w * T + t) * 256 + rem];
+            if (a.x_zero)
+                v -= a.x_zero[m0 + i] * a.w_zero_term[n];
+            v *= a.x_scale[m0 + i];
+            if (T > 1 && a.act) { // this tile holds gate rows, the next one their up rows
+                float up = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w)
+                    up += red[(w * T + (T > 1 ? t + 1 : t)) * 256 + rem];
+                if (a.x_zero)
+                    up -= a.x_zero[m0 + i] * a.w_zero_term[n + 16];
+                up *= a.x_scale[m0 + i];
+                reinterpret_cast<_Float16 *>(a.D)[(size_t)(m0 + i) * (N / 2) + (n >> 5) * 16 + c] = (_Float16)(silu(v) * up);
+            } else {
+                reinterpret_cast<_Float16 *>(a.D)[(size_t)(m0 + i) * N + n] = (_Float16)v;
+            }
+        }
+    }
+}
+
+// (waves, loads in flight per wave, tiles) by shape; the fused gate needs a tile pair per workgroup.
+template <int Q, int P, bool SIGNED, int NW, int D, int T>
+static hipError_t launch_decode_tiled_grouped_as(const GemmArgs &a, hipStream_t stream)
+{
+    const int mrows = decode_tiled_grouped_rows(NW, T, a.M, a.K, Q);
+    if (mrows == 0)
+        return hipErrorInvalidValue;
+    const size_t lds = decode_tiled_grouped_lds(NW, T, mrows, a.K, Q);
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr != hipSuccess)
+        return attr;
+    const int tiles = (a.N + 15) / 16;
+    const dim3 grid((tiles + T - 1) / T, (a.M + mrows - 1) / mrows);
+    hipLaunchKernelGGL((gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T>), grid, dim3(64 * NW), lds, stream, a, mrows);
+    return hipGetLastError();
+}
+
+template <int Q, int P, bool SIGNED, int T>
+static hipError_t launch_decode_tiled_grouped_t(const GemmArgs &a, hipStream_t stream)
+{
+    // loads in flight per wave, in units of 8 bytes per lane: 2 or 6 (1 or 3 steps of 8-bit weights)
+    constexpr int DS = P == 8 ? 1 : 2, DL = P == 8 ? 3 : 6, DM = P == 8 ? 2 : 4;
+    const int KT = a.K / 128;
+    const int wgs = ((a.N + 15) / 16 + T - 1) / T;
+    if (wgs > 512) // twice the workgroups fit a compute unit with eight waves
+        return (KT + 7) / 8 > DM ? launch_decode_tiled_grouped_as<Q, P, SIGNED, 8, DL, T>(a, stream)
+                                 : launch_decode_tiled_grouped_as<Q, P, SIGNED, 8, DM, T>(a, stream);
+    return (KT + 15) / 16 > DS ? launch_decode_tiled_grouped_as<Q, P, SIGNED, 16, DL, T>(a, stream)
+                               : launch_decode_tiled_grouped_as<Q, P, SIGNED, 16, DS, T>(a, stream);
+}
+
+template <int Q, int P, bool SIGNED> static hipError_t launch_decode_tiled_grouped(const GemmArgs &a, hipStream_t stream)
+{
+    if (a.group_size != 128 || !a.w_scale || !a.x_scale || (size_t)a.N * a.K * P / 8 >= (1ull << 32) ||
+        (size_t)a.M * a.K * Q / 8 >= (1ull << 32))
+        return hipErrorInvalidValue;
+    if (a.act) {
+        if (a.N % 32 != 0)
+            return hipErrorInvalidValue;
+        return launch_decode_tiled_grouped_t<Q, P, SIGNED, 2>(a, stream);
+    }
+    return launch_decode_tiled_grouped_t<Q, P, SIGNED, 1>(a, stream);
+}
+
 // Native tile space of this kernel: (waves, weight loads in flight per wave, tiles per workgroup).  Entries name
 // MFMA 16x16x64 with NSTAGE = 6; wk = waves, tn = tiles, kb = K elements a wave has in flight (D steps).
 #define ABQ_DT_VARIANTS(V) V(16, 1, 1) V(16, 3, 1) V(8, 2, 1) V(16, 1, 3) V(8, 1, 2)
@@ -297,6 +616,13 @@ static hipError_t launch_decode_tiled(const GemmArgs &a, hipStream_t stream)
 
 #if (ABQ_Q == 2 || ABQ_Q == 4 || ABQ_Q == 8) && (ABQ_P == 2 || ABQ_P == 4 || ABQ_P == 8)
 static const KernelEntry kSigned[] = { ABQ_DT_VARIANTS(ABQ_DT_ENTRY_T) };
+// one entry: the launcher picks waves, loads in flight and tiles by shape
+static const KernelEntry kSignedGrouped[] = { { 16, 1, 1, 1, 1, 16, 6, &launch_decode_tiled_grouped<ABQ_Q, ABQ_P, true>, 128 } };
+#if ABQ_Q < 8
+static const KernelEntry kUnsignedGrouped[] = { { 16, 1, 1, 1, 1, 16, 6, &launch_decode_tiled_grouped<ABQ_Q, ABQ_P, false>, 128 } };
+#else
+static const KernelEntry *const kUnsignedGrouped = nullptr;
+#endif
 #if ABQ_Q < 8
 static const KernelEntry kUnsigned[] = { ABQ_DT_VARIANTS(ABQ_DT_ENTRY_F) };
 #define ABQ_DT_NUNSIGNED ((int)(sizeof(kUnsigned) / sizeof(kUnsigned[0])))
@@ -308,6 +634,8 @@ static const KernelEntry *const kUnsigned = nullptr;
 #else
 static const KernelEntry *const kSigned = nullptr;
 static const KernelEntry *const kUnsigned = nullptr;
+static const KernelEntry *const kSignedGrouped = nullptr;
+static const KernelEntry *const kUnsignedGrouped = nullptr;
 #define ABQ_DT_NSIGNED 0
 #define ABQ_DT_NUNSIGNED 0
 #endif
@@ -319,6 +647,12 @@ void ABQ_CAT(abq_decode_tiled_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)
 {
     out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSigned, ABQ_DT_NSIGNED };
     out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, kUnsigned, ABQ_DT_NUNSIGNED };
+}
+
+void ABQ_CAT(abq_decode_tiled_grouped_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)
+{
+    out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSignedGrouped, kSignedGrouped ? 1 : 0 };
+    out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, kUnsignedGrouped, kUnsignedGrouped ? 1 : 0 };
 }
 
 } // namespace abq

@@ -29,7 +29,9 @@ struct ABQGroupedWeight {
     const float *zero_term;   // [N] from abq_weight_zero_term; needed for asymmetric activations
     int group_size;           // 64 or 128
     const int *planes;        // the same weights in the reference plane layout [w_bits][N][K/32], or nullptr;
-                              // with it, calls of at most 16 rows run the decode kernel
+                              // with it, calls of at most 16 rows run the decode kernel on plane operands where
+                              // the one on prepared operands does not exist (widths other than 2, 4, 8 bits, groups
+                              // of 64); for those that have it, planes_tiled serves every M
     const int *records_fp6;   // the same weights as FP6 records (abq_relayout_planes_fp6), or nullptr; with it,
                               // groups of 128 and a bit pair that qualifies (abq_fp6_eligible, e.g. W4A4), calls of
                               // more than 16 rows run on the FP6 matrix cores

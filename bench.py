@@ -412,6 +412,30 @@ def main():
             vendor = {"unavailable": repr(exc)[:120]}
         extra["library_int8_gemm"] = vendor
 
+    def time_rotating(gs, reps=100):
+        """us per launch of the GEMMs in gs run round robin, HIP-graph replay"""
+        for r in range(4):
+            gs[r % len(gs)].run()
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            for r in range(reps):
+                gs[r % len(gs)].run()
+        gr.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
+
+    def tiled_copies(Wr):
+        wt = torch.empty((Wr.shape[0], Wr.shape[3] // 4, Wr.shape[2], Wr.shape[1], 4), dtype=torch.int32, device="cuda")
+        for r in range(Wr.shape[0]):
+            abq.relayout_planes(Wr[r], out=wt[r])
+        return wt
+
     if want("decode_fused_linears"):
         # ------------------------------------------------------------ side measurement: several linears per launch
         # QKV (N = 3 * 4096) and gate + up (N = 2 * 11008) share their activations, so each is one GEMM
@@ -420,72 +444,51 @@ def main():
         for name, N, K in (("qkv", 3 * 4096, 4096), ("gate_up", 2 * 11008, 4096)):
             wbytes = P_BITS * N * K // 8
             Wr = random_planes(torch, (max(2, math.ceil(ROTATE_BYTES / wbytes)), P_BITS, N, K // 32))
+            Wt = tiled_copies(Wr)
             for M in MS:
                 out = torch.empty((M, N), dtype=torch.int32, device="cuda")
-                gs = [abq.Gemm(xs[(M, K)], Wr[r], SIGNED, out=out) for r in range(Wr.shape[0])]
-                for r in range(4):
-                    gs[r % len(gs)].run()
-                torch.cuda.synchronize()
-                gr = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(gr):
-                    for r in range(100):
-                        gs[r % len(gs)].run()
-                gr.replay()
-                torch.cuda.synchronize()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                gr.replay()
-                e1.record()
-                torch.cuda.synchronize()
-                us = e0.elapsed_time(e1) * 1e3 / 100
+                gs = [abq.Gemm(xs_tiled[(M, K)], Wt[r], SIGNED, out=out, x_tiled=True, w_tiled=True) for r in range(Wt.shape[0])]
+                us = time_rotating(gs)
+                us_planes = time_rotating([abq.Gemm(xs[(M, K)], Wr[r], SIGNED, out=out) for r in range(Wr.shape[0])])
                 gbs = algorithmic_bytes(M, N, K, Q_BITS, P_BITS) / (us * 1e-6) / 1e9
                 fused.append(dict(linears=name, M=M, N=N, K=K, us=round(us, 3), hbm_gbs=round(gbs, 1),
-                                  hbm_frac=round(gbs / HBM_PEAK_GBS, 4), kernel="%s:%s" % (gs[0].strategy, gs[0].config_name)))
-                log("fused %s M=%d N=%d K=%d  %.2f us  %.0f GB/s (%.1f%% of HBM peak)" % (name, M, N, K, us, gbs, 100 * gbs / HBM_PEAK_GBS))
-                del gr, gs, out
-            del Wr
+                                  hbm_frac=round(gbs / HBM_PEAK_GBS, 4), kernel="%s:%s" % (gs[0].strategy, gs[0].config_name),
+                                  plane_operands_us=round(us_planes, 3)))
+                log("fused %s M=%d N=%d K=%d  %.2f us  %.0f GB/s (%.1f%% of HBM peak); plane operands %.2f us"
+                    % (name, M, N, K, us, gbs, 100 * gbs / HBM_PEAK_GBS, us_planes))
+                del gs, out
+            del Wr, Wt
         extra["decode_fused_linears"] = fused
 
     if want("decode_group_scales"):
         # ------------------------------------------------------------ side measurement: decode with the dequantising epilogue
-        # group-128 weight scales and zero points, per-token scales, fp16 output (the decode kernel's
-        # group-scale variant); bytes add the scale and zero-point arrays to the packed weights
+        # group-128 weight scales and zero points, per-token scales, fp16 output, on prepared operands (the
+        # group-scale variant of the decode kernel on K-tiled operands) and on plane operands beside it; bytes add
+        # the scale and zero-point arrays to the packed weights
         deq = []
         for (N, K) in SHAPES:
             G = K // 128
             wbytes = P_BITS * N * K // 8
-            Wr = random_planes(torch, (max(2, math.ceil(ROTATE_BYTES / wbytes)), P_BITS, N, K // 32))
+            Wr = weights[(N, K)]
             wsc = torch.rand((N, G), device="cuda") * 0.01 + 0.001
             wz = torch.randint(-2, 2, (N, G), device="cuda").float()
             for M in (1, 8):
                 xsc = torch.rand(M, device="cuda") * 0.05 + 0.01
                 sums = torch.randint(-1000, 1000, (M, G), dtype=torch.int32, device="cuda")
                 out = torch.empty((M, N), dtype=torch.float16, device="cuda")
-                gs = [abq.Gemm(xs[(M, K)], Wr[r], SIGNED, out=out, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc,
-                               group_size=128, w_zero=wz, x_group_sums=sums) for r in range(Wr.shape[0])]
-                for r in range(4):
-                    gs[r % len(gs)].run()
-                torch.cuda.synchronize()
-                gr = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(gr):
-                    for r in range(100):
-                        gs[r % len(gs)].run()
-                gr.replay()
-                torch.cuda.synchronize()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                gr.replay()
-                e1.record()
-                torch.cuda.synchronize()
-                us = e0.elapsed_time(e1) * 1e3 / 100
+                kw = dict(out=out, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc, group_size=128, w_zero=wz, x_group_sums=sums)
+                Wt = weights_tiled[(N, K)]
+                gs = [abq.Gemm(xs_tiled[(M, K)], Wt[r], SIGNED, x_tiled=True, w_tiled=True, **kw) for r in range(Wt.shape[0])]
+                us = time_rotating(gs)
+                us_planes = time_rotating([abq.Gemm(xs[(M, K)], Wr[r], SIGNED, **kw) for r in range(Wr.shape[0])])
                 nbytes = algorithmic_bytes(M, N, K, Q_BITS, P_BITS, out_bytes=2) + 2 * N * G * 4
                 gbs = nbytes / (us * 1e-6) / 1e9
                 deq.append(dict(M=M, N=N, K=K, group_size=128, us=round(us, 3), hbm_gbs=round(gbs, 1),
-                                hbm_frac=round(gbs / HBM_PEAK_GBS, 4), kernel="%s:%s" % (gs[0].strategy, gs[0].config_name)))
-                log("dequant decode M=%d N=%d K=%d  %.2f us  %.0f GB/s (%.1f%% of HBM peak)  %s"
-                    % (M, N, K, us, gbs, 100 * gbs / HBM_PEAK_GBS, gs[0].strategy))
-                del gr, gs, out
-            del Wr
+                                hbm_frac=round(gbs / HBM_PEAK_GBS, 4), kernel="%s:%s" % (gs[0].strategy, gs[0].config_name),
+                                plane_operands_us=round(us_planes, 3)))
+                log("dequant decode M=%d N=%d K=%d  %.2f us  %.0f GB/s (%.1f%% of HBM peak)  %s; plane operands %.2f us"
+                    % (M, N, K, us, gbs, 100 * gbs / HBM_PEAK_GBS, gs[0].strategy, us_planes))
+                del gs, out
         extra["decode_group_scales"] = deq
 
     if want("decoder_layer_w2a8_group128"):

@@ -111,7 +111,8 @@ typedef enum abq_strategy {
                                  K-tiled layout (widths 2, 4 or 8 bits; no unsigned 8-bit operand):
                                  nothing is expanded or transposed inside the kernel; tile tuples with
                                  NSTAGE = 6.  A state with M <= 16 whose operands are both declared
-                                 ABQ_LAYOUT_TILED moves here by itself */
+                                 ABQ_LAYOUT_TILED moves here by itself; with group scales of 128 it runs
+                                 this strategy's group-scale variant (zero points, fused SiLU gate) */
 } abq_strategy;
 
 /* Parses "AqBMMA_8x2xtrue_1x48x512_8x24x128_8x8x128_4" (an optional _InitFn/_ExecFn suffix is
@@ -202,9 +203,13 @@ abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, cons
  * group_size 64 or 128: w_scale is [N][K/group_size] (the reference reshapes W to
  * [-1, group_size] before calibrating, quantizer.py:151-156) and
  *     D[m][n] = x_scale[m] * sum_g w_scale[n][g] * (sum_{k in g} x[m][k] * w[n][k]).
- * Group scales run on ABQ_STRATEGY_TILED only: a state whose tile was the library's choice is
- * moved there (and needs the workspace / layouts of that strategy); a state pinned to another
- * tile tuple, or 8-bit unsigned operands, return ABQ_ERR_UNSUPPORTED. */
+ * Four kernels carry group scales, and a state whose tile was the library's choice is moved to the one that
+ * fits: M <= 16 on plane operands -> the group-scale variant of ABQ_STRATEGY_DECODE (64 or 128); M <= 16 with both
+ * operands ABQ_LAYOUT_TILED, groups of 128 and widths of 2, 4 or 8 bits -> that of ABQ_STRATEGY_DECODE_TILED (whichever
+ * of abq_gemm_set_scales and abq_gemm_set_operand_layout comes first); FP6 operands -> ABQ_STRATEGY_FP6 (128
+ * only); everything else -> ABQ_STRATEGY_TILED (and needs the workspace / layouts of that strategy).  A state
+ * pinned to a tile tuple of another strategy, or 8-bit unsigned operands, return ABQ_ERR_UNSUPPORTED.  If the call
+ * fails the state is left as it was. */
 
 /* Zero points for a state with group scales (asymmetric quantisation, quantizer.py:120-128:
  * x ~ scale * (code - zero)).  Codes are the integers in the bit planes, read with the
@@ -300,7 +305,8 @@ abq_status abq_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int ro
                                    int is_signed, void *stream);
 
 /* Declares the layout of X and W of an initialised state.  A tiled (FP6) operand moves a state
- * whose tile was the library's choice to ABQ_STRATEGY_TILED (ABQ_STRATEGY_FP6); a state
+ * whose tile was the library's choice to ABQ_STRATEGY_TILED (ABQ_STRATEGY_FP6), or, with M <= 16 and both operands
+ * tiled, to ABQ_STRATEGY_DECODE_TILED where that kernel exists for the pair and epilogue; a state
  * initialised with an explicit tile tuple of another strategy is refused (ABQ_ERR_UNSUPPORTED),
  * and so are a tiled and an FP6 operand together, an FP6 operand with group scales of groups other
  * than 128, and an FP6 operand of a bit pair or K that does not qualify. */

@@ -210,6 +210,62 @@ def test_decode_kernel_with_group_scales_and_zero_points(abq, oracle, q, p, sign
         assert np.abs(got.astype(np.float64) - got2.astype(np.float64)).max() <= 2e-3 * np.abs(want).max()
 
 
+@pytest.mark.parametrize("q,p,signed", [(8, 2, True), (8, 4, True), (8, 8, True), (4, 4, True), (4, 2, True), (2, 2, True),
+                                        (4, 4, False), (4, 2, False), (2, 2, False)])
+def test_decode_on_prepared_operands_with_group_scales(abq, oracle, q, p, signed):
+    """At most 16 activation rows with both operands K-tiled and groups of 128: the prepared-operand decode
+    kernel's group-scale variant (one K tile = one scale group per step), with zero points on both sides."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(3 * q + 11 * p + signed)
+    for (M, N, K, zeros) in [(1, 64, 128, 0), (5, 200, 384, 1), (16, 4096 + 8, 4096, 2), (8, 300, 11008, 2), (3, 4096, 1152, 1),
+                             (1, 11008, 4096, 2), (16, 48, 11008, 2), (2, 16, 2176, 1), (13, 20, 256, 2)]:
+        lo_x, hi_x = (-(1 << (q - 1)), 1 << (q - 1)) if signed else (0, 1 << q)
+        lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed else (0, 1 << p)
+        x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        G = K // 128
+        xs = rng.uniform(0.01, 0.05, M)
+        wsc = rng.uniform(0.001, 0.02, (N, G))
+        wz = rng.integers(lo_w, hi_w, (N, G)).astype(np.float64) if zeros >= 1 else np.zeros((N, G))
+        xz = rng.integers(lo_x // 2, hi_x // 2, M).astype(np.float64) if zeros >= 2 else np.zeros(M)
+        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, 128)
+        wp = planes_dev(oracle.pack_i32(w, p))
+        kw = dict(x_scale=fdev(xs), w_scale=fdev(wsc), group_size=128, x_tiled=True, w_tiled=True)
+        if zeros >= 1:
+            kw.update(w_zero=fdev(wz), x_group_sums=torch.from_numpy(x.reshape(M, G, 128).sum(axis=2).astype(np.int32)).cuda())
+        if zeros >= 2:
+            kw.update(x_zero=fdev(xz), w_zero_term=abq.weight_zero_term(wp, signed, kw["w_scale"], kw["w_zero"], 128))
+        out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        xt, wt = abq.relayout_planes(planes_dev(oracle.pack_i32(x, q))), abq.relayout_planes(wp)
+        got = run_grouped(abq, xt, wt, signed, strategy="decode_tiled", out=out, **kw)
+        assert_close_rel(got, want)
+
+
+def test_decode_on_prepared_operands_group_scales_either_call_order(abq, oracle):
+    """Layouts declared before the scales are attached (the C ABI allows both orders) lands on the same kernel."""
+    import ctypes
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(5)
+    M, N, K = 4, 96, 512
+    x = rng.integers(-128, 128, (M, K)).astype(np.int32)
+    w = rng.integers(-2, 2, (N, K)).astype(np.int32)
+    xs, wsc = rng.uniform(0.01, 0.05, M), rng.uniform(0.001, 0.02, (N, K // 128))
+    xt = abq.relayout_planes(planes_dev(oracle.pack_i32(x, 8)))
+    wt = abq.relayout_planes(planes_dev(oracle.pack_i32(w, 2)))
+    g = abq.Gemm(xt, wt, True, out_kind=abq.OUT_F16_SCALED, x_scale=fdev(xs), w_scale=fdev(wsc), x_tiled=True, w_tiled=True)
+    assert g.strategy == "decode_tiled"  # per-channel state on prepared operands
+    wsc_d = fdev(wsc)
+    st = abq.lib().abq_gemm_set_scales(ctypes.byref(g.state), g.x_scale.data_ptr(), wsc_d.data_ptr(), 128)
+    assert st == 0 and g.strategy == "decode_tiled"
+    out = g.run()
+    torch.cuda.synchronize()
+    assert_close_rel(out.cpu().numpy(), Q.dequant_matmul(x, xs, np.zeros(M), w, wsc, np.zeros_like(wsc), 128))
+    # groups of 64 have no variant there: the state moves to the tiled kernel
+    g2 = abq.Gemm(xt, wt, True, out_kind=abq.OUT_F16_SCALED, x_scale=fdev(xs), w_scale=fdev(np.repeat(wsc, 2, axis=1)),
+                  group_size=64, x_tiled=True, w_tiled=True)
+    assert g2.strategy == "tiled"
+
+
 def interleave16(gate, up):
     """[I, ...] gate rows and [I, ...] up rows -> [2I, ...] in blocks of 16 gate rows followed by their 16 up rows."""
     I = gate.shape[0]
@@ -221,7 +277,8 @@ def interleave16(gate, up):
     return out
 
 
-@pytest.mark.parametrize("M,strategy", [(1, "decode"), (7, "decode"), (16, "decode"), (100, "tiled"), (300, "tiled")])
+@pytest.mark.parametrize("M,strategy", [(1, "decode"), (7, "decode"), (16, "decode"), (100, "tiled"), (300, "tiled"),
+                                        (1, "decode_tiled"), (7, "decode_tiled"), (16, "decode_tiled")])
 @pytest.mark.parametrize("group_size", [128, 64])
 def test_silu_gate_epilogue(abq, oracle, M, strategy, group_size):
     """gate / up pair fused into one GEMM: D = silu(x Wg^T) * (x Wu^T) on the dequantised values."""
@@ -246,6 +303,11 @@ def test_silu_gate_epilogue(abq, oracle, M, strategy, group_size):
     out = torch.full((M, I), float("nan"), dtype=torch.float16, device="cuda")
     if strategy == "tiled":
         got = run_grouped(abq, planes_dev(oracle.pack_i32(x, q)), abq.relayout_planes(wp), True, w_tiled=True, out=out, **kw)
+    elif strategy == "decode_tiled":
+        if group_size == 64:
+            pytest.skip("the prepared-operand decode kernel has groups of 128 only")
+        got = run_grouped(abq, abq.relayout_planes(planes_dev(oracle.pack_i32(x, q))), abq.relayout_planes(wp), True,
+                          strategy="decode_tiled", x_tiled=True, w_tiled=True, out=out, **kw)
     else:
         got = run_grouped(abq, planes_dev(oracle.pack_i32(x, q)), wp, True, strategy="decode", out=out, **kw)
     assert got.shape == (M, I)

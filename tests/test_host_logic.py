@@ -341,6 +341,57 @@ def test_gen_kernel_native_space_is_what_the_library_instantiates(gen_kernel, ab
             assert gen == native, (q, p, signed)
 
 
+def test_group_scales_move_a_state_to_the_kernel_that_carries_them(abq):
+    """Which strategy a state ends on once group scales are attached, for both orders of the two calls, and that
+    a refused call leaves the state untouched (host logic only: nothing is launched)."""
+    lib = abq.lib()
+    T = abq.LAYOUT_TILED
+
+    def state(q=8, p=2, M=1, signed=1, **kw):
+        rc, st = _init(abq, q=q, p=p, M=M, signed=signed, N=4096, K=4096, out_kind=abq.OUT_F16_SCALED, **kw)
+        assert rc == 0
+        return st
+
+    names = abq.STRATEGY_NAMES
+    # plane operands, at most 16 rows: popcount by default, the decode kernel once it has to carry group scales
+    st = state()
+    assert names[st.strategy] == "bcnt"
+    assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 128) == 0
+    assert names[st.strategy] == "decode" and st.group_size == 128
+    # ... and the prepared-operand decode kernel when the layouts are declared afterwards
+    assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0
+    assert names[st.strategy] == "decode_tiled" and st.group_size == 128 and st.variant == 0
+    # layouts first, scales second: the same place
+    st = state(M=8)
+    assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0 and names[st.strategy] == "decode_tiled"
+    assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 128) == 0
+    assert names[st.strategy] == "decode_tiled" and st.variant == 0
+    assert lib.abq_gemm_set_activation(ctypes.byref(st), abq.ACT_SILU_GATE) == 0 and names[st.strategy] == "decode_tiled"
+    # groups of 64, or widths of several fields, have no variant there: the tiled kernel
+    st = state(M=8)
+    assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0
+    assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 64) == 0 and names[st.strategy] == "tiled"
+    st = state(q=6, p=2, M=8)
+    assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 128) == 0
+    assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0 and names[st.strategy] == "tiled"
+    # more than 16 rows: tiled
+    st = state(M=64)
+    assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 128) == 0 and names[st.strategy] == "tiled"
+    # a refused call (unsigned 8-bit operands have no group-scale kernel) changes nothing, not even the strategy the
+    # call had moved the state to on its way
+    st = state(q=8, p=8, signed=0)
+    before = bytes(st)
+    assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 128) == abq.ABQ_ERR_UNSUPPORTED
+    assert bytes(st) == before
+    cfg = abq.native_configs(8, 2, 1)
+    pinned = [c for c in cfg if c.mma_k == 128][0]  # a popcount tile named by the caller stays where it is
+    rc, st = _init(abq, cfg=pinned, q=8, p=2, M=1, N=4096, K=4096, out_kind=abq.OUT_F16_SCALED)
+    assert rc == 0
+    before = bytes(st)
+    assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 128) == abq.ABQ_ERR_UNSUPPORTED
+    assert bytes(st) == before
+
+
 def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     """The tile the library picks for prepared operands, pinned on shapes of BASELINE.json configs[2] and
     configs[4] and on a few where the measured sweep of all tiles separates them clearly:
