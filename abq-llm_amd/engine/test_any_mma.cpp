@@ -34,6 +34,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -85,19 +86,214 @@ struct Timing {
     int status = -1; // 0 PASSED, -1 ERROR, -2 FAILED (test_mma.h:114-159)
 };
 
+double half_bits_to_double(uint16_t h)
+{
+    const int e = (h >> 10) & 31, f = h & 1023;
+    const double v = e == 0 ? std::ldexp((double)f, -24) : e == 31 ? (f ? NAN : INFINITY) : std::ldexp((double)(f | 1024), e - 25);
+    return (h & 0x8000) ? -v : v;
+}
+
+// --group G [--fp6]: every tile of the kernels that carry group scales (the dequantising epilogue: weight scales
+// and zero points per G elements of K, per-token activation scales, fp16 out), on prepared operands (K-tiled, or
+// FP6 records with --fp6), plus the library's own choice.  Results are checked on up to eight rows against a
+// double-precision loop over the dequantised operands (1e-2 relative, with 1e-3 of the rows' RMS as the floor
+// for entries that cancel).  One line per tile in the format of the int32 sweep.
+int sweep_group_scales(int M, int N, int K, int x_bits, int w_bits, bool is_signed, int group, bool fp6, const std::vector<int> &h_x,
+                       const std::vector<int> &h_w, const uint32_t *d_xp, const uint32_t *d_xt, const uint32_t *d_wt,
+                       const uint32_t *d_wf, size_t wp_bytes, size_t wf_bytes, size_t nbuf, int repeat, int warmup,
+                       const std::string &only, hipStream_t stream)
+{
+    if ((group != 64 && group != 128) || K % group) {
+        std::printf("Error, --group takes 64 or 128\n");
+        return -1;
+    }
+    if (fp6 && (!d_wf || group != 128)) {
+        std::printf("Error, --fp6 needs a bit pair that qualifies for FP6 records and groups of 128\n");
+        return -1;
+    }
+    const int G = K / group;
+    std::mt19937 rng(7);
+    std::uniform_real_distribution<float> sd(0.001f, 0.011f);
+    std::vector<float> h_ws((size_t)N * G), h_wz((size_t)N * G), h_xs(M);
+    const int wlo = is_signed ? -(1 << (w_bits - 1)) : 0;
+    for (auto &v : h_ws)
+        v = sd(rng);
+    for (auto &v : h_wz)
+        v = (float)(wlo + (int)(rng() % (1u << w_bits)));
+    for (auto &v : h_xs)
+        v = sd(rng);
+    std::vector<int> h_sums((size_t)M * G);
+    for (int m = 0; m < M; ++m)
+        for (int g = 0; g < G; ++g) {
+            int sum = 0;
+            for (int k = 0; k < group; ++k)
+                sum += h_x[(size_t)m * K + (size_t)g * group + k];
+            h_sums[(size_t)m * G + g] = sum;
+        }
+    // expected values of the sampled rows
+    const int nrows = std::min(M, 8);
+    std::vector<int> rows(nrows);
+    for (int i = 0; i < nrows; ++i)
+        rows[i] = (int)((long)i * (M - 1) / std::max(1, nrows - 1));
+    std::vector<double> want((size_t)nrows * N);
+    double sq = 0;
+#pragma omp parallel for collapse(2) schedule(static) reduction(+ : sq)
+    for (int i = 0; i < nrows; ++i)
+        for (int n = 0; n < N; ++n) {
+            const int *xr = &h_x[(size_t)rows[i] * K], *wr = &h_w[(size_t)n * K];
+            double v = 0;
+            for (int g = 0; g < G; ++g) {
+                long acc = 0;
+                for (int k = g * group; k < (g + 1) * group; ++k)
+                    acc += (long)xr[k] * wr[k];
+                v += (double)h_ws[(size_t)n * G + g] * ((double)acc - (double)h_wz[(size_t)n * G + g] * h_sums[(size_t)rows[i] * G + g]);
+            }
+            v *= h_xs[rows[i]];
+            want[(size_t)i * N + n] = v;
+            sq += v * v;
+        }
+    const double rms = std::sqrt(sq / ((double)nrows * N));
+
+    float *d_ws_, *d_wz_, *d_xs_;
+    int *d_sums;
+    uint16_t *d_out; // fp16
+    uint32_t *d_xf = nullptr;
+    HIP_OK(hipMalloc(&d_ws_, h_ws.size() * 4));
+    HIP_OK(hipMalloc(&d_wz_, h_wz.size() * 4));
+    HIP_OK(hipMalloc(&d_xs_, h_xs.size() * 4));
+    HIP_OK(hipMalloc(&d_sums, h_sums.size() * 4));
+    HIP_OK(hipMalloc(&d_out, (size_t)M * N * 2));
+    HIP_OK(hipMemcpy(d_ws_, h_ws.data(), h_ws.size() * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d_wz_, h_wz.data(), h_wz.size() * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d_xs_, h_xs.data(), h_xs.size() * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d_sums, h_sums.data(), h_sums.size() * 4, hipMemcpyHostToDevice));
+    if (fp6) {
+        HIP_OK(hipMalloc(&d_xf, abq_fp6_bytes(M, K)));
+        if (abq_relayout_planes_fp6(d_xp, d_xf, M, K, x_bits, is_signed, stream) != ABQ_OK) {
+            std::printf("abq_relayout_planes_fp6 failed (hip error %d)\n", abq_last_hip_error());
+            return -1;
+        }
+    }
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    const int layout = fp6 ? ABQ_LAYOUT_FP6 : ABQ_LAYOUT_TILED;
+    const double ops = 2.0 * M * N * K;
+    std::vector<uint16_t> h_out((size_t)M * N);
+    std::vector<std::string> seen;
+    double best_tops = 0;
+    std::string best;
+    const int ncfg = abq_native_config_count(x_bits, w_bits, is_signed);
+    for (int i = 0; i <= ncfg; ++i) {
+        abq_tile_config cfg;
+        const bool library_default = i == ncfg;
+        if (!library_default) {
+            if (abq_native_config_get(x_bits, w_bits, is_signed, i, &cfg) != ABQ_OK || cfg.nstage != (fp6 ? 5 : 4) || cfg.warp_k != 128)
+                continue;
+            char name[160];
+            abq_format_kernel_name(&cfg, 0, name, sizeof name);
+            if (!only.empty() && std::string(name).find(only) == std::string::npos)
+                continue;
+        }
+        std::vector<abq_gemm_state> states(nbuf);
+        bool ok = true;
+        for (size_t b = 0; b < nbuf && ok; ++b) {
+            const char *wbase = fp6 ? (const char *)d_wf + b * wf_bytes : (const char *)d_wt + b * wp_bytes;
+            abq_status s = abq_gemm_init(library_default ? nullptr : &cfg, x_bits, w_bits, is_signed, fp6 ? d_xf : d_xt,
+                                         (const uint32_t *)wbase, M, N, K, d_out, nullptr, 0, ABQ_OUT_F16_SCALED, &states[b]);
+            if (s == ABQ_OK)
+                s = abq_gemm_set_operand_layout(&states[b], layout, layout);
+            if (s == ABQ_OK)
+                s = abq_gemm_set_scales(&states[b], d_xs_, d_ws_, group);
+            if (s == ABQ_OK)
+                s = abq_gemm_set_zero_points(&states[b], nullptr, d_wz_, d_sums, nullptr);
+            ok = s == ABQ_OK && states[b].init_success;
+        }
+        if (!ok)
+            continue; // no group-scale build of this tile
+        const abq_tile_config &c = states[0].cfg;
+        char key[96];
+        std::snprintf(key, sizeof key, "%d %d %d %d %d %zu", c.block_m, c.block_n, c.warp_m, c.warp_n, c.nstage, states[0].shared_mem_size);
+        if (!library_default) {
+            if (std::find(seen.begin(), seen.end(), key) != seen.end())
+                continue; // tuples that resolve to the same group-scale kernel
+            seen.push_back(key);
+        }
+        HIP_OK(hipMemsetAsync(d_out, 0xff, (size_t)M * N * 2, stream));
+        int status = 0;
+        if (abq_gemm_exec(&states[0], stream) != ABQ_OK || hipStreamSynchronize(stream) != hipSuccess)
+            status = -1;
+        if (status == 0) {
+            HIP_OK(hipMemcpy(h_out.data(), d_out, (size_t)M * N * 2, hipMemcpyDeviceToHost));
+            for (int r = 0; r < nrows && status == 0; ++r)
+                for (int n = 0; n < N; ++n) {
+                    const double got = half_bits_to_double(h_out[(size_t)rows[r] * N + n]), w = want[(size_t)r * N + n];
+                    if (!(std::fabs(got - w) <= 1e-2 * std::fabs(w) + 1e-3 * rms)) {
+                        status = -2;
+                        break;
+                    }
+                }
+        }
+        float ms = 0;
+        if (status == 0) {
+            for (int j = 0; j < warmup; ++j)
+                abq_gemm_exec(&states[j % nbuf], stream);
+            hipGraph_t g;
+            hipGraphExec_t ge;
+            HIP_OK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+            for (int j = 0; j < repeat; ++j)
+                abq_gemm_exec(&states[j % nbuf], stream);
+            HIP_OK(hipStreamEndCapture(stream, &g));
+            HIP_OK(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0));
+            HIP_OK(hipEventRecord(e0, stream));
+            HIP_OK(hipGraphLaunch(ge, stream));
+            HIP_OK(hipEventRecord(e1, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+            HIP_OK(hipGraphExecDestroy(ge));
+            HIP_OK(hipGraphDestroy(g));
+        }
+        const float us = ms * 1e3f / repeat;
+        const double tops = status == 0 ? ops / (us * 1e-6) / 1e12 : 0;
+        std::printf("gfx950 W%dA%d %s group %d%s %d %d %d %d %d %d %d %d %d %d lds %zu exec %f (us) %f TOPS | %s | %.1f%% MFMA%s\n", w_bits,
+                    x_bits, is_signed ? "int" : "uint", group, fp6 ? " FP6" : "", c.block_m, c.block_n, c.block_k, c.warp_m, c.warp_n,
+                    c.warp_k, c.mma_m, c.mma_n, c.mma_k, c.nstage, states[0].shared_mem_size, us, tops,
+                    status == 0 ? "PASSED" : status == -1 ? "ERROR" : "FAILED", 100.0 * tops / 5000.0,
+                    library_default ? " | library default" : "");
+        if (status == 0 && !library_default && tops > best_tops) {
+            best_tops = tops;
+            char buf[128];
+            std::snprintf(buf, sizeof buf, "%d, %d, %d, %d, %d, %d, %d, %d, %d, %d", c.block_m, c.block_n, c.block_k, c.warp_m, c.warp_n,
+                          c.warp_k, c.mma_m, c.mma_n, c.mma_k, c.nstage);
+            best = buf;
+        }
+        std::fflush(stdout);
+    }
+    std::printf("The best kernel config is %s with %f TOPS\n", best.c_str(), best_tops);
+    (void)hipFree(d_ws_);
+    (void)hipFree(d_wz_);
+    (void)hipFree(d_xs_);
+    (void)hipFree(d_sums);
+    (void)hipFree(d_out);
+    if (d_xf)
+        (void)hipFree(d_xf);
+    return 0;
+}
+
 } // namespace
 
 int main(int argc, char **argv)
 {
     if (argc < 7) {
-        std::printf("Usage: ./test_any_mma M N K X_BITS W_BITS SIGNED [--repeat R] [--warmup W] [--rotate-mib MiB] [--stream] [--only SUBSTR] [--seed S]\n");
+        std::printf("Usage: ./test_any_mma M N K X_BITS W_BITS SIGNED [--repeat R] [--warmup W] [--rotate-mib MiB] [--stream] [--only SUBSTR] [--seed S] [--read-floor] [--group 64|128 [--fp6]]\n");
         return -1;
     }
     const int M = std::atoi(argv[1]), N = std::atoi(argv[2]), K = std::atoi(argv[3]);
     const int x_bits = std::atoi(argv[4]), w_bits = std::atoi(argv[5]);
     const bool is_signed = std::atoi(argv[6]) == 1;
     int repeat = 1000, warmup = 10, rotate_mib = 512;
-    bool use_graph = true, read_floor = false;
+    bool use_graph = true, read_floor = false, group_fp6 = false;
+    int group = 0; // --group: sweep the tiles of the kernels with group scales and zero points (fp16 out) instead
     unsigned long seed = 0;
     std::string only;
     for (int i = 7; i < argc; ++i) {
@@ -105,6 +301,10 @@ int main(int argc, char **argv)
             use_graph = false;
         else if (!std::strcmp(argv[i], "--read-floor"))
             read_floor = true;
+        else if (!std::strcmp(argv[i], "--fp6"))
+            group_fp6 = true;
+        else if (i + 1 < argc && !std::strcmp(argv[i], "--group"))
+            group = std::atoi(argv[++i]);
         else if (i + 1 < argc && !std::strcmp(argv[i], "--repeat"))
             repeat = std::atoi(argv[++i]);
         else if (i + 1 < argc && !std::strcmp(argv[i], "--warmup"))
@@ -201,6 +401,10 @@ int main(int argc, char **argv)
             HIP_OK(hipMemcpyAsync((char *)d_wf + b * wf_bytes, d_wf, wf_bytes, hipMemcpyDeviceToDevice, stream));
         HIP_OK(hipStreamSynchronize(stream));
     }
+
+    if (group)
+        return sweep_group_scales(M, N, K, x_bits, w_bits, is_signed, group, group_fp6, h_x, h_w, d_xp, d_xt, d_wt, d_wf, wp_bytes,
+                                  wf_bytes, nbuf, repeat, warmup, only, stream);
 
     std::vector<uint32_t> h_xp(xp_words), h_wp(wp_words);
     HIP_OK(hipMemcpy(h_xp.data(), d_xp, xp_words * 4, hipMemcpyDeviceToHost));
