@@ -114,70 +114,96 @@ ABQ_HD uint64_t transpose8x8(uint64_t x)
 ABQ_HD constexpr uint32_t field_mask(int f) { return 0x01010101u * ((1u << f) - 1u); }
 ABQ_HD constexpr int field_base(int bits, int f) { return bits & (f - 1); }             // lowest value bit of the field
 ABQ_HD constexpr int field_word_offset(int bits, int f) { return 4 * (bits & ~(2 * f - 1)); }
+// words of the wider fields in front of field f in a per-word-set list [4-bit: 4][2-bit: 2][1-bit: 1]
+ABQ_HD constexpr int field_list_index(int bits, int f) { return bits & ~(2 * f - 1); }
+// The routines below treat one field width at a time, as a template parameter: every trip count and register
+// index is then a constant of the instantiation.  (Written as one loop over f = 4, 2, 1 with the inner trip
+// count f, the compiler left the 6- and 7-bit cases rolled and indexed the register arrays at run time: the
+// prefill kernel for those widths ran ten times slower than for 5 bits.)
 
 // Expanded bytes (bit pattern in the low BITS bits of each byte) of one word-set -> its BITS
 // field words, ordered [4-bit field: 4 words][2-bit field: 2 words][1-bit field: 1 word].
-template <int BITS> ABQ_HD void compress_fields(const uint32_t (&e)[8], uint32_t (&out)[BITS])
+template <int BITS, int F> ABQ_HD void compress_one_field(const uint32_t (&e)[8], uint32_t (&out)[BITS])
 {
-    static_assert(BITS >= 1 && BITS <= 8, "1..8 bits");
-    if (BITS == 8) {
+    if constexpr ((BITS & F) != 0) {
+        constexpr int per = 8 / F, idx = field_list_index(BITS, F);
 #pragma unroll
-        for (int d = 0; d < 8; ++d)
-            out[d % BITS] = e[d];
-        return;
-    }
-    int idx = 0;
-#pragma unroll
-    for (int f = 4; f >= 1; f >>= 1) {
-        if (!(BITS & f))
-            continue;
-        const int per = 8 / f;
-#pragma unroll
-        for (int j = 0; j < f; ++j) {
+        for (int j = 0; j < F; ++j) {
             uint32_t v = 0;
 #pragma unroll
             for (int s = 0; s < per; ++s)
-                v |= ((e[per * j + s] >> field_base(BITS, f)) & field_mask(f)) << (f * s);
-            out[(idx + j) % BITS] = v;
+                v |= ((e[per * j + s] >> field_base(BITS, F)) & field_mask(F)) << (F * s);
+            out[idx + j] = v;
         }
-        idx += f;
+    }
+}
+
+template <int BITS> ABQ_HD void compress_fields(const uint32_t (&e)[8], uint32_t (&out)[BITS])
+{
+    static_assert(BITS >= 1 && BITS <= 8, "1..8 bits");
+    if constexpr (BITS == 8) {
+#pragma unroll
+        for (int d = 0; d < 8; ++d)
+            out[d] = e[d];
+    } else {
+        compress_one_field<BITS, 4>(e, out);
+        compress_one_field<BITS, 2>(e, out);
+        compress_one_field<BITS, 1>(e, out);
     }
 }
 
 // The reverse, fused with the placement in the int8 lane (MODE as for planes_to_int8).  `raw`
 // holds the fields of WPT consecutive word-sets of one row, [4-bit field: 4*WPT words][2-bit:
 // 2*WPT][1-bit: WPT] (or 8*WPT bytes-as-words for 8 bits); `ws` selects the word-set.
+template <int BITS, int WPT, Int8Mode MODE, int F, int WS>
+ABQ_HD void expand_one_field(const uint32_t (&raw)[BITS * WPT], uint32_t (&e)[8])
+{
+    if constexpr ((BITS & F) != 0) {
+        constexpr int per = 8 / F, idx = field_list_index(BITS, F) * WPT;
+        constexpr int t = field_base(BITS, F) + (MODE == kTop ? 8 - BITS : 0); // where the field lands in the byte
+#pragma unroll
+        for (int j = 0; j < F; ++j) {
+            const uint32_t w = raw[idx + F * WS + j];
+#pragma unroll
+            for (int s = 0; s < per; ++s) {
+                const int net = t - F * s;
+                const uint32_t y = net >= 0 ? (w << (net & 31)) : (w >> ((-net) & 31));
+                e[per * j + s] |= y & (field_mask(F) << t);
+            }
+        }
+    }
+}
+
+template <int BITS, int WPT, Int8Mode MODE, int WS> ABQ_HD void expand_fields_of(const uint32_t (&raw)[BITS * WPT], uint32_t (&e)[8])
+{
+    static_assert(WS >= 0 && WS < WPT, "word-set of the list");
+    if constexpr (BITS == 8) {
+#pragma unroll
+        for (int d = 0; d < 8; ++d)
+            e[d] = raw[8 * WS + d] ^ (MODE == kFlip ? 0x80808080u : 0u);
+    } else {
+#pragma unroll
+        for (int d = 0; d < 8; ++d)
+            e[d] = 0u;
+        expand_one_field<BITS, WPT, MODE, 4, WS>(raw, e);
+        expand_one_field<BITS, WPT, MODE, 2, WS>(raw, e);
+        expand_one_field<BITS, WPT, MODE, 1, WS>(raw, e);
+    }
+}
+
+// the same with the word-set as an argument (0 <= ws < WPT <= 4)
 template <int BITS, int WPT, Int8Mode MODE>
 ABQ_HD void expand_fields(const uint32_t (&raw)[BITS * WPT], int ws, uint32_t (&e)[8])
 {
-    if (BITS == 8) {
-#pragma unroll
-        for (int d = 0; d < 8; ++d)
-            e[d] = raw[(8 * ws + d) % (BITS * WPT)] ^ (MODE == kFlip ? 0x80808080u : 0u);
-        return;
-    }
-#pragma unroll
-    for (int d = 0; d < 8; ++d)
-        e[d] = 0u;
-    int idx = 0;
-#pragma unroll
-    for (int f = 4; f >= 1; f >>= 1) {
-        if (!(BITS & f))
-            continue;
-        const int per = 8 / f;
-        const int t = field_base(BITS, f) + (MODE == kTop ? 8 - BITS : 0); // where the field lands in the byte
-#pragma unroll
-        for (int j = 0; j < f; ++j) {
-            const uint32_t w = raw[(idx + f * ws + j) % (BITS * WPT)];
-#pragma unroll
-            for (int s = 0; s < per; ++s) {
-                const int net = t - f * s;
-                const uint32_t y = net >= 0 ? (w << (net & 31)) : (w >> ((-net) & 31));
-                e[per * j + s] |= y & (field_mask(f) << t);
-            }
-        }
-        idx += f * WPT;
-    }
+    static_assert(WPT >= 1 && WPT <= 4, "at most four word-sets in a list");
+    if (WPT == 1 || ws == 0)
+        expand_fields_of<BITS, WPT, MODE, 0>(raw, e);
+    else if (WPT == 2 || ws == 1)
+        expand_fields_of<BITS, WPT, MODE, (WPT > 1 ? 1 : 0)>(raw, e);
+    else if (WPT == 3 || ws == 2)
+        expand_fields_of<BITS, WPT, MODE, (WPT > 2 ? 2 : 0)>(raw, e);
+    else
+        expand_fields_of<BITS, WPT, MODE, (WPT > 3 ? 3 : 0)>(raw, e);
 }
 
 // Sum of the four bytes of every dword of an expanded word-set (values fed unsigned, before

@@ -63,23 +63,16 @@ __device__ __forceinline__ void load_tile_words(uint32_t (&dst)[BITS * WPT], con
                                                 int kt, int first_ws)
 {
     const uint32_t *rec = tiled + ((size_t)kt * rows + row) * (BITS * 4);
-    if (BITS == 8) {
+    if constexpr (BITS == 8) {
         load_words<8 * WPT>(dst, rec + 8 * first_ws);
         return;
     }
-    int idx = 0;
-#pragma unroll
-    for (int f = 4; f >= 1; f >>= 1) {
-        if (!(BITS & f))
-            continue;
-        if (f == 4)
-            load_words<4 * WPT>(dst + idx, rec + field_word_offset(BITS, 4) + 4 * first_ws);
-        else if (f == 2)
-            load_words<2 * WPT>(dst + idx, rec + field_word_offset(BITS, 2) + 2 * first_ws);
-        else
-            load_words<WPT>(dst + idx, rec + field_word_offset(BITS, 1) + first_ws);
-        idx += f * WPT;
-    }
+    if constexpr ((BITS & 4) != 0)
+        load_words<4 * WPT>(dst + field_list_index(BITS, 4) * WPT, rec + field_word_offset(BITS, 4) + 4 * first_ws);
+    if constexpr ((BITS & 2) != 0)
+        load_words<2 * WPT>(dst + field_list_index(BITS, 2) * WPT, rec + field_word_offset(BITS, 2) + 2 * first_ws);
+    if constexpr ((BITS & 1) != 0)
+        load_words<WPT>(dst + field_list_index(BITS, 1) * WPT, rec + field_word_offset(BITS, 1) + first_ws);
 }
 
 // Expands WPT word-sets (32 K elements each) of one row and writes the int8 values to LDS.

@@ -108,26 +108,22 @@ __global__ __launch_bounds__(256) void pack_u4_kernel(const uint4 *__restrict__ 
 template <int BITS>
 __device__ __forceinline__ void store_fields(uint32_t *rec, int ws, const uint32_t (&f)[BITS])
 {
-    if (BITS == 8) {
+    if constexpr (BITS == 8) {
         uint4 *dst = reinterpret_cast<uint4 *>(rec + 8 * ws);
-        dst[0] = make_uint4(f[0], f[1 % BITS], f[2 % BITS], f[3 % BITS]);
-        dst[1] = make_uint4(f[4 % BITS], f[5 % BITS], f[6 % BITS], f[7 % BITS]);
+        dst[0] = make_uint4(f[0], f[1], f[2], f[3]);
+        dst[1] = make_uint4(f[4], f[5], f[6], f[7]);
         return;
     }
-    int idx = 0;
-#pragma unroll
-    for (int w = 4; w >= 1; w >>= 1) {
-        if (!(BITS & w))
-            continue;
-        uint32_t *dst = rec + field_word_offset(BITS, w) + w * ws;
-        if (w == 4)
-            *reinterpret_cast<uint4 *>(dst) = make_uint4(f[idx % BITS], f[(idx + 1) % BITS], f[(idx + 2) % BITS], f[(idx + 3) % BITS]);
-        else if (w == 2)
-            *reinterpret_cast<uint2 *>(dst) = make_uint2(f[idx % BITS], f[(idx + 1) % BITS]);
-        else
-            dst[0] = f[idx % BITS];
-        idx += w;
+    if constexpr ((BITS & 4) != 0) {
+        constexpr int i = field_list_index(BITS, 4);
+        *reinterpret_cast<uint4 *>(rec + field_word_offset(BITS, 4) + 4 * ws) = make_uint4(f[i], f[i + 1], f[i + 2], f[i + 3]);
     }
+    if constexpr ((BITS & 2) != 0) {
+        constexpr int i = field_list_index(BITS, 2);
+        *reinterpret_cast<uint2 *>(rec + field_word_offset(BITS, 2) + 2 * ws) = make_uint2(f[i], f[i + 1]);
+    }
+    if constexpr ((BITS & 1) != 0)
+        rec[field_word_offset(BITS, 1) + ws] = f[field_list_index(BITS, 1)];
 }
 
 // One workgroup converts 32 rows x 8 K tiles.  A thread owns one record (one row, one K tile): it

@@ -1,6 +1,9 @@
 """GPU parity tests: every kernel is called through the C ABI (libabq_gemm.so) and compared
 bit for bit with the CPU oracle on the same seeded inputs.  Inputs are packed by the oracle on
 the host, so the GEMM tests do not depend on the pack kernels."""
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -610,16 +613,32 @@ def test_config2_prefill_full_size(abq, oracle, q, p, signed):
             del ref
 
 
+def _config3_best_tiles():
+    """(x_bits, w_bits, signed, N, K) -> the tile tuple the autotune harness measured as fastest on MI355X (the
+    'fastest tile' column of the kept sweep), from tests/golden/config3_best_tiles.json."""
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "config3_best_tiles.json")) as f:
+        return {(e["x_bits"], e["w_bits"], e["signed"], e["N"], e["K"]): tuple(e["tile"]) for e in json.load(f)["best"]}
+
+
 @pytest.mark.parametrize("q,p", BASELINE_COMBOS)
 def test_config3_bit_combo_sweep_m128(abq, oracle, q, p):
+    """BASELINE configs[3]: every combination at M = 128 on the LLaMA-13B shapes, signed and unsigned, bit exact on
+    the library's own choice and on the autotuned tile (the fastest one of the harness sweep for that case)."""
     rng = np.random.default_rng(3000 + 10 * q + p)
+    best = _config3_best_tiles()
     M = 128
     for (N, K) in [(5120, 5120), (13824, 5120), (5120, 13824)]:
         for signed in (True, False):
             x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
             xp, wp = oracle.pack_i32(x, q), oracle.pack_i32(w, p)
-            got_d = run_cfg(abq, planes_dev(xp), planes_dev(wp), signed,
+            xd, wd = planes_dev(xp), planes_dev(wp)
+            got_d = run_cfg(abq, xd, wd, signed,
                             workspace=torch.empty((xp.size + wp.size) * 4, dtype=torch.uint8, device="cuda"))
             ref = torch.from_numpy(x).cuda().double() @ torch.from_numpy(w).cuda().double().T
             assert torch.equal(got_d.double(), ref), (q, p, signed, N, K)
             _sampled_oracle_check(oracle, xp, wp, signed, got_d.cpu().numpy(), rng, rows=2)
+            tile = best[(q, p, signed, N, K)]
+            cfg = [c for c in abq.native_configs(q, p, signed) if c.as_tuple()[3:] == tile]
+            assert len(cfg) == 1, tile  # the autotuned tile is one the library builds
+            got_t = run_cfg(abq, xd, wd, signed, cfg=cfg[0])
+            assert torch.equal(got_t.double(), ref), (q, p, signed, N, K, tile)
