@@ -86,6 +86,48 @@ struct Timing {
     int status = -1; // 0 PASSED, -1 ERROR, -2 FAILED (test_mma.h:114-159)
 };
 
+// --mfma-ceiling: what the matrix cores sustain in a register-only loop (abq_probe_launch), on constant operand
+// bits and on random ones, int8 and FP6: launches of about 30 ms so that clocks settle, the best of three.
+int matrix_core_ceiling(hipStream_t stream)
+{
+    int dev = 0, cus = 0;
+    HIP_OK(hipGetDevice(&dev));
+    HIP_OK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    std::mt19937 rng(1);
+    std::vector<uint32_t> h(2048);
+    uint32_t *d;
+    HIP_OK(hipMalloc(&d, h.size() * 4));
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    const size_t n = 1u << 19;
+    for (int kind : { ABQ_PROBE_MFMA_I8, ABQ_PROBE_MFMA_FP6 })
+        for (int random = 0; random < 2; ++random) {
+            // FP6: six dwords of a lane's eight hold 32 codes; constant = every code 0b001000 (1.0), i8: every byte 1
+            for (auto &v : h)
+                v = random ? (uint32_t)rng() : (kind == ABQ_PROBE_MFMA_FP6 ? 0x20820820u : 0x01010101u);
+            HIP_OK(hipMemcpy(d, h.data(), h.size() * 4, hipMemcpyHostToDevice));
+            float best = 1e30f;
+            for (int rep = 0; rep < 4; ++rep) {
+                HIP_OK(hipEventRecord(e0, stream));
+                if (abq_probe_launch(kind, d, n, stream) != ABQ_OK)
+                    return -1;
+                HIP_OK(hipEventRecord(e1, stream));
+                HIP_OK(hipStreamSynchronize(stream));
+                float ms;
+                HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+                if (rep)
+                    best = std::min(best, ms);
+            }
+            const double ops = 2.0 * cus * 4 * (double)n * (kind == ABQ_PROBE_MFMA_FP6 ? 131072.0 : 65536.0);
+            std::printf("matrix-core ceiling: %s, %s operand bits: %.1f ms per launch, %.2f P%s/s on %d compute units\n",
+                        kind == ABQ_PROBE_MFMA_FP6 ? "v_mfma_f32_32x32x64_f8f6f4 (E2M3)" : "v_mfma_i32_32x32x32_i8",
+                        random ? "random" : "constant", best, ops / (best * 1e-3) / 1e15, kind == ABQ_PROBE_MFMA_FP6 ? "FLOP" : "OP", cus);
+        }
+    (void)hipFree(d);
+    return 0;
+}
+
 double half_bits_to_double(uint16_t h)
 {
     const int e = (h >> 10) & 31, f = h & 1023;
@@ -285,14 +327,14 @@ int sweep_group_scales(int M, int N, int K, int x_bits, int w_bits, bool is_sign
 int main(int argc, char **argv)
 {
     if (argc < 7) {
-        std::printf("Usage: ./test_any_mma M N K X_BITS W_BITS SIGNED [--repeat R] [--warmup W] [--rotate-mib MiB] [--stream] [--only SUBSTR] [--seed S] [--read-floor] [--group 64|128 [--fp6]]\n");
+        std::printf("Usage: ./test_any_mma M N K X_BITS W_BITS SIGNED [--repeat R] [--warmup W] [--rotate-mib MiB] [--stream] [--only SUBSTR] [--seed S] [--read-floor] [--mfma-ceiling] [--group 64|128 [--fp6]]\n");
         return -1;
     }
     const int M = std::atoi(argv[1]), N = std::atoi(argv[2]), K = std::atoi(argv[3]);
     const int x_bits = std::atoi(argv[4]), w_bits = std::atoi(argv[5]);
     const bool is_signed = std::atoi(argv[6]) == 1;
     int repeat = 1000, warmup = 10, rotate_mib = 512;
-    bool use_graph = true, read_floor = false, group_fp6 = false;
+    bool use_graph = true, read_floor = false, group_fp6 = false, mfma_ceiling = false;
     int group = 0; // --group: sweep the tiles of the kernels with group scales and zero points (fp16 out) instead
     unsigned long seed = 0;
     std::string only;
@@ -303,6 +345,8 @@ int main(int argc, char **argv)
             read_floor = true;
         else if (!std::strcmp(argv[i], "--fp6"))
             group_fp6 = true;
+        else if (!std::strcmp(argv[i], "--mfma-ceiling"))
+            mfma_ceiling = true;
         else if (i + 1 < argc && !std::strcmp(argv[i], "--group"))
             group = std::atoi(argv[++i]);
         else if (i + 1 < argc && !std::strcmp(argv[i], "--repeat"))
@@ -323,6 +367,8 @@ int main(int argc, char **argv)
 
     hipStream_t stream;
     HIP_OK(hipStreamCreate(&stream));
+    if (mfma_ceiling)
+        return matrix_core_ceiling(stream);
 
     // ---- host operands: uniform over the full range of the bit width
     std::mt19937_64 rng(seed);
