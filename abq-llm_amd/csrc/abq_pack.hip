@@ -367,13 +367,13 @@ __device__ __forceinline__ void emit_tiled(const int (&v)[8], uint32_t *tiled, i
     if (bits == 8) {
         // 8-bit codes are the record's bytes themselves: expanded dword s, byte c = element 31 - (8c + s) of
         // the word-set = element 7 - s of lane 3 - c.  The quad transposes its bytes so that lane s ends
-        // with the dwords s and 4 + s, and every lane stores its two.
-        const uint32_t e_lo = quad_transpose_bytes(pack_low_bytes(v[7], v[6], v[5], v[4]), sel_pair, sel_half);
-        const uint32_t e_hi = quad_transpose_bytes(pack_low_bytes(v[3], v[2], v[1], v[0]), sel_pair, sel_half);
+        // with the dwords 2 s and 2 s + 1, which it stores as one piece of 8 bytes: sixteen lanes cover a
+        // record's 128 bytes with one store instruction.
+        const uint32_t e_even = quad_transpose_bytes(pack_low_bytes(v[7], v[5], v[3], v[1]), sel_pair, sel_half);
+        const uint32_t e_odd = quad_transpose_bytes(pack_low_bytes(v[6], v[4], v[2], v[0]), sel_pair, sel_half);
         if (active) {
-            uint32_t *dst = tiled + ((size_t)(w >> 2) * rows + row) * 32 + 8 * (w & 3) + quad_lane;
-            dst[0] = e_lo;
-            dst[4] = e_hi;
+            uint32_t *dst = tiled + ((size_t)(w >> 2) * rows + row) * 32 + 8 * (w & 3) + 2 * quad_lane;
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(e_even, e_odd);
         }
         return;
     }
@@ -427,6 +427,240 @@ __device__ __forceinline__ float wave_max(float v)
     return v;
 }
 
+// What a row's quantisation needs once its minimum and maximum are known.
+struct QuantRow {
+    float scale, recip, zp_stored, lo_stored, hi_stored, zero_out;
+};
+
+// scale, zero point and code range of a row from its extrema (formulas in the comment above)
+__device__ __forceinline__ QuantRow quant_row_params(float mx, float mn, int bits, int symmetric)
+{
+    const int half_range = 1 << (bits - 1);
+    float scale, zp;
+    int lo, hi;
+    if (symmetric) {
+        scale = fmaxf(fabsf(mx), fabsf(mn)) / (float)(half_range - 1);
+        scale = fminf(fmaxf(scale, 1e-5f), 1e4f);
+        zp = 0.f;
+        lo = -half_range;
+        hi = half_range - 1;
+    } else {
+        scale = (mx - mn) / (float)(2 * half_range - 1);
+        scale = fminf(fmaxf(scale, 1e-5f), 1e4f);
+        zp = rintf(fminf(fmaxf(-mn / scale, -1e4f), 1e4f));
+        lo = 0;
+        hi = 2 * half_range - 1;
+    }
+    QuantRow q;
+    q.scale = scale;
+    // x / scale in three operations instead of the dozen of a full division, with the same bits: recip is the
+    // correctly rounded reciprocal (the fp64 quotient is never close enough to an fp32 midpoint for the second
+    // rounding to cross it), t = x recip is within an ulp of the quotient, the residual x - t scale is exact in
+    // an fma, and t + residual recip then rounds to the quotient itself (checked against the division on a CPU
+    // for every finite fp16 value and 600 000 scales of the forms above; a zero may come out with the other
+    // sign, which the rounding to an integer code forgets).  div_fixup restores what a division makes of an
+    // infinite x.
+    q.recip = (float)(1.0 / (double)scale);
+    // rint(q) + zp, clamped to [lo, hi], minus the offset of the stored code: the offset is taken off before the
+    // clamp instead (all three are small integers, so the sums are the same numbers)
+    const float code_offset = symmetric ? 0.f : (float)half_range;
+    q.zp_stored = zp - code_offset;
+    q.lo_stored = (float)lo - code_offset;
+    q.hi_stored = (float)hi - code_offset;
+    q.zero_out = symmetric ? 0.f : zp - (float)half_range;
+    return q;
+}
+
+// Quantises the eight fp16 values of unit u (elements 8u .. 8u + 7) of `row` and writes their share of the
+// packed row; the lanes of a quad hold consecutive units (quad_lane = u & 3), a scale group's lanes are
+// consecutive too.  Inactive lanes (units past the row) take part in the cross-lane steps with zeros.
+// BITS: the code width where the instantiation fixes it (8), 0 where it is the run-time argument.
+template <int LAYOUT, int BITS = 0>
+__device__ __forceinline__ void quant_emit_unit(const uint4 &rawq, bool active, int u, int row, int M, int K, int bits_arg,
+                                                const QuantRow &q, uint32_t *planes, int *group_sums, int group_size,
+                                                uint32_t sel_pair, uint32_t sel_half)
+{
+    const int bits = BITS ? BITS : bits_arg;
+    const int KW = K / 32;
+    const int lanes_per_group = group_size / 8;
+    int v[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
+    int sum = 0;
+    if (active) {
+        union {
+            uint4 q;
+            _Float16 h[8];
+        } raw;
+        raw.q = rawq;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const float xf = (float)raw.h[c];
+            const float t = xf * q.recip;
+            // the fix-up only matters for an infinite x, but one more instruction per element is cheaper than a
+            // branch around it per element
+            const float quotient = __builtin_amdgcn_div_fixupf(__builtin_fmaf(__builtin_fmaf(-t, q.scale, xf), q.recip, t), q.scale, xf);
+            v[c] = (int)__builtin_amdgcn_fmed3f(rintf(quotient) + q.zp_stored, q.lo_stored, q.hi_stored);
+            sum += v[c];
+        }
+    }
+    if (group_sums) {
+        const int glog = group_size == 64 ? 3 : 4; // lanes of a scale group: 8 or 16
+        for (int o = 1; o < lanes_per_group; o <<= 1)
+            sum += __shfl_xor(sum, o);
+        if (active && (u & (lanes_per_group - 1)) == 0)
+            group_sums[(size_t)row * (K >> (glog + 3)) + (u >> glog)] = sum;
+    }
+    const int quad_lane = u & 3, w = u >> 2; // w: word-set (32 elements) within the row
+    if (LAYOUT == 2) {
+        // position p = 4 s + c of the word-set's 192-bit string holds element 31 - (8c + s): this lane's
+        // element j goes to position 4 (7 - j) + 3 - quad_lane as the code (sign << 5) | magnitude
+        uint32_t o[6] = { 0u, 0u, 0u, 0u, 0u, 0u };
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t code = v[j] < 0 ? (32u | (uint32_t)(-v[j])) : (uint32_t)v[j];
+            constexpr int kBase[8] = { 168, 144, 120, 96, 72, 48, 24, 0 }; // 24 (7 - j)
+            const int d0 = kBase[j] >> 5;                                   // first dword the code can touch
+            const uint64_t wide = (uint64_t)code << ((kBase[j] & 31) + 6 * (3 - quad_lane));
+            o[d0] |= (uint32_t)wide;
+            if (d0 + 1 < 6)
+                o[d0 + 1] |= (uint32_t)(wide >> 32);
+        }
+#pragma unroll
+        for (int d = 0; d < 6; ++d)
+            o[d] = quad_or(o[d]);
+        if (active && quad_lane == 0) {
+            const int ws = w & 3;
+            uint32_t *rec = planes + ((size_t)(w >> 2) * M + row) * 24 + 12 * (ws & 1) + 6 * (ws >> 1);
+            *reinterpret_cast<uint2 *>(rec) = make_uint2(o[0], o[1]);
+            *reinterpret_cast<uint2 *>(rec + 2) = make_uint2(o[2], o[3]);
+            *reinterpret_cast<uint2 *>(rec + 4) = make_uint2(o[4], o[5]);
+        }
+    } else if (LAYOUT == 1) {
+        emit_tiled(v, planes, M, row, w, quad_lane, bits, active, sel_pair, sel_half);
+    } else {
+        const uint64_t bytes = eight_values_to_plane_bytes(v);
+        for (int b = 0; b < bits; ++b) {
+            uint32_t word = (uint32_t)((bytes >> (8 * b)) & 0xFFu) << (24 - 8 * quad_lane);
+            word = quad_or(word);
+            if (active && quad_lane == 0)
+                planes[((size_t)b * M + row) * KW + w] = word;
+        }
+    }
+}
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+// One WAVE per token row, the row held in registers between the two passes: NU 16-byte units per lane are all in
+// flight at once, there is no barrier and no LDS round trip, and the waves of a compute unit are each at their
+// own point of their rows, so loads, arithmetic and stores of different rows overlap.  (With one workgroup per
+// row, a row's loads were in flight only during the first third of the workgroup's life: 3.2 TB/s where a plain
+// copy of the same buffers reaches 5.5.)  Rows of up to NU * 512 elements, NU <= 24 (beyond, the row spills).
+template <int LAYOUT, int NU, int BITS>
+__global__ __launch_bounds__(256) void quant_pack_wave_rows_kernel(const uint4 *__restrict__ x, uint32_t *__restrict__ planes,
+                                                                   float *__restrict__ scale_out, float *__restrict__ zero_out,
+                                                                   int *__restrict__ group_sums, int M, int K, int bits,
+                                                                   int symmetric, int group_size)
+{
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M)
+        return; // whole waves leave: nothing below synchronises across waves
+    const int units = K / 8;
+    const uint4 *xr = x + (size_t)row * units;
+    uint4 raw[NU];
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+        const int u = lane + 64 * i;
+        raw[i] = xr[u < units ? u : 0]; // past the end: the row's first unit once more (it changes no extremum)
+    }
+    half2_t mx2 = { (_Float16)-INFINITY, (_Float16)-INFINITY }, mn2 = { (_Float16)INFINITY, (_Float16)INFINITY };
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+        union {
+            uint4 q;
+            half2_t h2[4];
+        } r;
+        r.q = raw[i];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            mx2 = __builtin_elementwise_max(mx2, r.h2[c]);
+            mn2 = __builtin_elementwise_min(mn2, r.h2[c]);
+        }
+    }
+    float mx = fmaxf((float)mx2.x, (float)mx2.y), mn = fminf((float)mn2.x, (float)mn2.y);
+    mx = wave_max(mx);
+    mn = -wave_max(-mn);
+    const QuantRow q = quant_row_params(mx, mn, bits, symmetric);
+    if (lane == 0) {
+        scale_out[row] = q.scale;
+        if (zero_out)
+            zero_out[row] = q.zero_out;
+    }
+    uint32_t sel_pair, sel_half;
+    quad_transpose_selectors(lane & 3, sel_pair, sel_half);
+    // a row that holds an infinity (or a NaN) takes the general path, whose quotients get the division's fix-up
+    const bool finite_row = __builtin_amdgcn_readfirstlane(fabsf(mx) <= 65504.f && fabsf(mn) <= 65504.f) != 0;
+    if (LAYOUT == 1 && BITS == 8 && finite_row) {
+        // The common case written out: 8-bit codes into K-tiled records.  Per unit: eight quotients, two byte
+        // packs, the group sum as two dot products with ones and a butterfly of row operations over the
+        // group's 8 or 16 lanes, two 4 x 4 byte transposes across the quad, one 8-byte store.  Unit
+        // u = lane + 64 i lies in K tile (lane >> 4) + 4 i: a fixed stride between a lane's records.
+        // clamp(rint(q) + zp, lo, hi) = rint(clamp(q, lo - zp, hi - zp)) + zp (the bounds are integers), and
+        // adding 1.5 * 2^23 to a float of magnitude below 2^22 rounds it to an integer, to nearest even like rint,
+        // and leaves that integer in the low mantissa bits: clamp, add, integer subtract.
+        const float q_lo = q.lo_stored - q.zp_stored, q_hi = q.hi_stored - q.zp_stored;
+        const float magic = 12582912.0f; // 1.5 * 2^23
+        const int unmagic = 0x4B400000 - (int)q.zp_stored;
+        uint32_t *rec = planes + ((size_t)(lane >> 4) * M + row) * 32 + 8 * ((lane >> 2) & 3) + 2 * (lane & 3);
+        const size_t rec_stride = (size_t)4 * M * 32;
+        const int glog = group_size == 64 ? 3 : 4; // lanes of a scale group
+        int *gs = group_sums ? group_sums + (size_t)row * (K / group_size) + (lane >> glog) : nullptr;
+        const int gs_stride = 64 >> glog;
+        const bool gs_lane = (lane & ((1 << glog) - 1)) == 0;
+#pragma unroll
+        for (int i = 0; i < NU; ++i) {
+            if (64 * (i + 1) <= units) { // wave-uniform: every lane has a unit
+                union {
+                    uint4 q;
+                    _Float16 h[8];
+                } r;
+                r.q = raw[i];
+                int v[8];
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    const float xf = (float)r.h[c];
+                    const float t = xf * q.recip;
+                    const float quotient = __builtin_fmaf(__builtin_fmaf(-t, q.scale, xf), q.recip, t);
+                    v[c] = __builtin_bit_cast(int, __builtin_amdgcn_fmed3f(quotient, q_lo, q_hi) + magic) - unmagic;
+                }
+                const uint32_t pa = pack_low_bytes(v[7], v[5], v[3], v[1]), pb = pack_low_bytes(v[6], v[4], v[2], v[0]);
+                if (gs) {
+                    int sum = __builtin_amdgcn_sdot4((int)pa, 0x01010101, __builtin_amdgcn_sdot4((int)pb, 0x01010101, 0, false), false);
+                    sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+                    sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+                    sum += __builtin_amdgcn_update_dpp(0, sum, 0x141, 0xF, 0xF, true); // row_half_mirror
+                    if (glog == 4)
+                        sum += __builtin_amdgcn_update_dpp(0, sum, 0x140, 0xF, 0xF, true); // row_mirror
+                    if (gs_lane)
+                        gs[i * gs_stride] = sum;
+                }
+                const uint32_t e_even = quad_transpose_bytes(pa, sel_pair, sel_half);
+                const uint32_t e_odd = quad_transpose_bytes(pb, sel_pair, sel_half);
+                *reinterpret_cast<uint2 *>(rec + i * rec_stride) = make_uint2(e_even, e_odd);
+            } else if (64 * i < units) { // the row's last, partly filled round
+                const int u = lane + 64 * i;
+                quant_emit_unit<LAYOUT, BITS>(raw[i], u < units, u, row, M, K, bits, q, planes, group_sums, group_size, sel_pair, sel_half);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < NU; ++i) {
+            const int u = lane + 64 * i;
+            if (64 * i < units) // wave-uniform: units is a multiple of 16, so quads and groups are active as one
+                quant_emit_unit<LAYOUT, BITS>(raw[i], u < units, u, row, M, K, bits, q, planes, group_sums, group_size, sel_pair, sel_half);
+        }
+    }
+}
+
 // LAYOUT: 0 planes, 1 field-packed K tiles, 2 FP6 records (codes of at most 5 bits).
 template <int LAYOUT>
 __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__restrict__ x, uint32_t *__restrict__ planes,
@@ -444,7 +678,6 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
 
     // four loads in flight per lane: with one, the pass is bound by the latency of memory, not its bandwidth.
     // Minimum and maximum are taken on the fp16 pairs as they are (two elements per instruction).
-    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
     half2_t mx2 = { (_Float16)-INFINITY, (_Float16)-INFINITY }, mn2 = { (_Float16)INFINITY, (_Float16)INFINITY };
     for (int u0 = tid; u0 < units; u0 += 1024) {
         union {
@@ -479,110 +712,21 @@ __global__ __launch_bounds__(256) void quant_pack_rows_kernel(const uint4 *__res
     mx = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
     mn = fminf(fminf(red[1][0], red[1][1]), fminf(red[1][2], red[1][3]));
 
-    const int half_range = 1 << (bits - 1);
-    float scale, zp;
-    int lo, hi;
-    if (symmetric) {
-        scale = fmaxf(fabsf(mx), fabsf(mn)) / (float)(half_range - 1);
-        scale = fminf(fmaxf(scale, 1e-5f), 1e4f);
-        zp = 0.f;
-        lo = -half_range;
-        hi = half_range - 1;
-    } else {
-        scale = (mx - mn) / (float)(2 * half_range - 1);
-        scale = fminf(fmaxf(scale, 1e-5f), 1e4f);
-        zp = rintf(fminf(fmaxf(-mn / scale, -1e4f), 1e4f));
-        lo = 0;
-        hi = 2 * half_range - 1;
-    }
+    const QuantRow q = quant_row_params(mx, mn, bits, symmetric);
     if (tid == 0) {
-        scale_out[row] = scale;
+        scale_out[row] = q.scale;
         if (zero_out)
-            zero_out[row] = symmetric ? 0.f : zp - (float)half_range;
+            zero_out[row] = q.zero_out;
     }
-
-    // x / scale in three operations instead of the dozen of a full division, with the same bits: recip is the
-    // correctly rounded reciprocal (the fp64 quotient is never close enough to an fp32 midpoint for the second
-    // rounding to cross it), t = x recip is within an ulp of the quotient, the residual x - t scale is exact in
-    // an fma, and t + residual recip then rounds to the quotient itself (checked against the division on a CPU
-    // for every finite fp16 value and 600 000 scales of the forms above; a zero may come out with the other
-    // sign, which the rounding to an integer code forgets).  div_fixup restores what a division makes of an
-    // infinite x.
-    const float recip = (float)(1.0 / (double)scale);
-    // only a row that holds an infinity needs the fix-up (a NaN goes through the fmas as through a division)
-    const bool fix_up = __builtin_amdgcn_readfirstlane(!(fabsf(mx) <= 65504.f && fabsf(mn) <= 65504.f)) != 0;
-    // rint(q) + zp, clamped to [lo, hi], minus the offset of the stored code: the offset is taken off before the
-    // clamp instead (all three are small integers, so the sums are the same numbers)
-    const float code_offset = symmetric ? 0.f : (float)half_range;
-    const float zp_stored = zp - code_offset, lo_stored = (float)lo - code_offset, hi_stored = (float)hi - code_offset;
-    const int KW = K / 32;
     const int rounded = (units + 255) / 256 * 256;
-    const int lanes_per_group = group_size / 8;
     uint32_t sel_pair, sel_half;
     quad_transpose_selectors(tid & 3, sel_pair, sel_half);
     for (int u = tid; u < rounded; u += 256) {
         const bool active = u < units; // units is a multiple of 16: quads and groups are active as one
-        int v[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
-        int sum = 0;
-        if (active) {
-            union {
-                uint4 q;
-                _Float16 h[8];
-            } raw;
-            raw.q = keep_row ? row_lds[u] : xr[u];
-#pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                const float xf = (float)raw.h[c];
-                const float t = xf * recip;
-                float quotient = __builtin_fmaf(__builtin_fmaf(-t, scale, xf), recip, t);
-                if (fix_up)
-                    quotient = __builtin_amdgcn_div_fixupf(quotient, scale, xf);
-                v[c] = (int)__builtin_amdgcn_fmed3f(rintf(quotient) + zp_stored, lo_stored, hi_stored);
-                sum += v[c];
-            }
-        }
-        if (group_sums) {
-            for (int o = 1; o < lanes_per_group; o <<= 1)
-                sum += __shfl_xor(sum, o);
-            if (active && (u % lanes_per_group) == 0)
-                group_sums[(size_t)row * (K / group_size) + u / lanes_per_group] = sum;
-        }
-        const int quad_lane = u & 3, w = u >> 2; // w: word-set (32 elements) within the row
-        if (LAYOUT == 2) {
-            // position p = 4 s + c of the word-set's 192-bit string holds element 31 - (8c + s): this lane's
-            // element j goes to position 4 (7 - j) + 3 - quad_lane as the code (sign << 5) | magnitude
-            uint32_t o[6] = { 0u, 0u, 0u, 0u, 0u, 0u };
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint32_t code = v[j] < 0 ? (32u | (uint32_t)(-v[j])) : (uint32_t)v[j];
-                constexpr int kBase[8] = { 168, 144, 120, 96, 72, 48, 24, 0 }; // 24 (7 - j)
-                const int d0 = kBase[j] >> 5;                                   // first dword the code can touch
-                const uint64_t wide = (uint64_t)code << ((kBase[j] & 31) + 6 * (3 - quad_lane));
-                o[d0] |= (uint32_t)wide;
-                if (d0 + 1 < 6)
-                    o[d0 + 1] |= (uint32_t)(wide >> 32);
-            }
-#pragma unroll
-            for (int d = 0; d < 6; ++d)
-                o[d] = quad_or(o[d]);
-            if (active && quad_lane == 0) {
-                const int ws = w & 3;
-                uint32_t *rec = planes + ((size_t)(w >> 2) * M + row) * 24 + 12 * (ws & 1) + 6 * (ws >> 1);
-                *reinterpret_cast<uint2 *>(rec) = make_uint2(o[0], o[1]);
-                *reinterpret_cast<uint2 *>(rec + 2) = make_uint2(o[2], o[3]);
-                *reinterpret_cast<uint2 *>(rec + 4) = make_uint2(o[4], o[5]);
-            }
-        } else if (LAYOUT == 1) {
-            emit_tiled(v, planes, M, row, w, quad_lane, bits, active, sel_pair, sel_half);
-        } else {
-            const uint64_t bytes = eight_values_to_plane_bytes(v);
-            for (int b = 0; b < bits; ++b) {
-                uint32_t word = (uint32_t)((bytes >> (8 * b)) & 0xFFu) << (24 - 8 * quad_lane);
-                word = quad_or(word);
-                if (active && quad_lane == 0)
-                    planes[((size_t)b * M + row) * KW + w] = word;
-            }
-        }
+        uint4 rawq = make_uint4(0u, 0u, 0u, 0u);
+        if (active)
+            rawq = keep_row ? row_lds[u] : xr[u];
+        quant_emit_unit<LAYOUT>(rawq, active, u, row, M, K, bits, q, planes, group_sums, group_size, sel_pair, sel_half);
     }
 }
 
@@ -590,6 +734,46 @@ hipError_t launch_quant_pack_rows(const void *x, uint32_t *planes, float *scale,
                                   int M, int K, int bits, int symmetric, int group_size, int layout,
                                   hipStream_t stream)
 {
+    // Many rows, or rows of at most 4096 elements: one wave per row, the row in registers (up to 12288 elements).
+    // (Measured on MI355X, 8-bit codes into K-tiled records: ahead of the kernel below from 16 rows up at K = 4096,
+    // from 1024 rows at K = 11008, where a lone wave's 22 units in a row cost more than four waves' barrier.)
+    const int nu = (K + 511) / 512;
+    if (nu <= 24 && (M >= 1024 || nu <= 8)) {
+        const dim3 grid((M + 3) / 4), block(256);
+#define ABQ_QP_WAVE(L, NU)                                                                                                  \
+    do {                                                                                                                    \
+        if (L == 1 && bits == 8)                                                                                            \
+            hipLaunchKernelGGL((quant_pack_wave_rows_kernel<L, NU, (L == 1 ? 8 : 0)>), grid, block, 0, stream,                 \
+                               reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits, symmetric,  \
+                               group_size);                                                                                 \
+        else                                                                                                                \
+            hipLaunchKernelGGL((quant_pack_wave_rows_kernel<L, NU, 0>), grid, block, 0, stream,                               \
+                               reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits, symmetric,  \
+                               group_size);                                                                                 \
+    } while (0)
+#define ABQ_QP_WAVE_NU(L)       \
+    do {                        \
+        if (nu <= 2)            \
+            ABQ_QP_WAVE(L, 2);  \
+        else if (nu <= 4)       \
+            ABQ_QP_WAVE(L, 4);  \
+        else if (nu <= 8)       \
+            ABQ_QP_WAVE(L, 8);  \
+        else if (nu <= 16)      \
+            ABQ_QP_WAVE(L, 16); \
+        else                    \
+            ABQ_QP_WAVE(L, 24); \
+    } while (0)
+        if (layout == 2)
+            ABQ_QP_WAVE_NU(2);
+        else if (layout == 1)
+            ABQ_QP_WAVE_NU(1);
+        else
+            ABQ_QP_WAVE_NU(0);
+#undef ABQ_QP_WAVE_NU
+#undef ABQ_QP_WAVE
+        return hipGetLastError();
+    }
     // a row of up to 48 KiB is kept in LDS (within the default limit together with the static part)
     const int keep_row = (size_t)K * 2 <= 48 * 1024;
     const size_t lds = keep_row ? (size_t)K * 2 : 0;
