@@ -22,7 +22,7 @@ OUT_I32, OUT_F16_TENSOR, OUT_F16_SCALED, OUT_F16_TENSOR_F32SCALE = 0, 1, 2, 3
 (STRATEGY_AUTO, STRATEGY_BCNT, STRATEGY_MFMA16, STRATEGY_MFMA32, STRATEGY_GENERIC, STRATEGY_DECODE, STRATEGY_TILED, STRATEGY_FP6,
  STRATEGY_DECODE_TILED) = range(9)
 STRATEGY_NAMES = ["auto", "bcnt", "mfma16", "mfma32", "generic", "decode", "tiled", "fp6", "decode_tiled"]
-LAYOUT_PLANES, LAYOUT_TILED, LAYOUT_FP6 = 0, 1, 2
+LAYOUT_PLANES, LAYOUT_TILED, LAYOUT_FP6, LAYOUT_F16 = 0, 1, 2, 3
 ACT_NONE, ACT_SILU_GATE = 0, 1
 
 # every symbol include/abq_gemm.h declares
@@ -35,7 +35,7 @@ EXPORTED = [
     "abq_planes_bytes", "abq_relayout_planes", "abq_gemm_set_operand_layout", "abq_gemm_workspace_bytes",
     "abq_gemm_set_workspace", "abq_fp6_bytes", "abq_fp6_eligible", "abq_relayout_planes_fp6",
     "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16", "abq_gemm_set_activation",
-    "abq_probe_launch", "abq_gemm_exec_static",
+    "abq_probe_launch", "abq_gemm_exec_static", "abq_gemm_set_f16_activations",
 ]
 
 
@@ -73,6 +73,7 @@ class GemmState(ctypes.Structure):
         ("x_zero", ctypes.c_void_p), ("w_zero", ctypes.c_void_p),
         ("x_group_sums", ctypes.c_void_p), ("w_zero_term", ctypes.c_void_p),
         ("act", ctypes.c_int),
+        ("x_pack_scale", ctypes.c_void_p),
     ]
 
 
@@ -112,6 +113,7 @@ def lib():
         L.abq_gemm_set_scales.argtypes = [ctypes.POINTER(GemmState), vp, vp, ci]
         L.abq_gemm_exec.argtypes = [ctypes.POINTER(GemmState), vp]
         L.abq_gemm_exec_static.argtypes = [ctypes.POINTER(GemmState), vp]
+        L.abq_gemm_set_f16_activations.argtypes = [ctypes.POINTER(GemmState), vp, vp]
         L.abq_gemm_launch.argtypes = [ctypes.POINTER(TileConfig), vp, vp, vp, vp, ci, ci, ci, ci, vp]
         L.abq_planes_bytes.argtypes = [ci, ci, ci]
         L.abq_planes_bytes.restype = ctypes.c_size_t
@@ -203,7 +205,8 @@ def pack_f16(values, scale, bits, out=None, stream=None, tiled=False):
     assert scale.dtype == torch.float32 and scale.is_cuda
     rows, k = values.shape
     if out is None:
-        out = planes_empty(bits, rows, k, values.device)
+        out = (torch.empty((k // 128, rows, bits, 4), dtype=torch.int32, device=values.device) if tiled
+               else planes_empty(bits, rows, k, values.device))
     fn, name = (lib().abq_pack_f16_tiled, "abq_pack_f16_tiled") if tiled else (lib().abq_pack_f16, "abq_pack_f16")
     _check(fn(values.data_ptr(), scale.data_ptr(), out.data_ptr(), rows, k, bits, _stream_ptr(stream)), name)
     return out
@@ -347,6 +350,16 @@ class Gemm:
     def run(self, stream=None):
         _check(lib().abq_gemm_exec(ctypes.byref(self.state), _stream_ptr(stream)), "abq_gemm_exec")
         return self.out
+
+    def set_f16_activations(self, x_f16, scale):
+        """Decode on prepared weights without a packing launch: the kernel quantises the fp16 activations [M, K]
+        itself with the static scale (one float on the device).  Raises ABQ_ERR_UNSUPPORTED where that kernel does
+        not apply."""
+        import torch
+        assert x_f16.dtype == torch.float16 and x_f16.is_cuda and x_f16.is_contiguous() and scale.dtype == torch.float32
+        _check(lib().abq_gemm_set_f16_activations(ctypes.byref(self.state), x_f16.data_ptr(), scale.data_ptr()),
+               "abq_gemm_set_f16_activations")
+        self.x_f16, self.x_pack_scale = x_f16, scale
 
     def run_static(self, stream=None):
         """The same through the entry point that allocates nothing (conversions into the library's static array)."""

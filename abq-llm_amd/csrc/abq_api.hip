@@ -40,7 +40,8 @@ hipError_t launch_weight_zero_term(const uint32_t *, int, int, int, int, const f
     void abq_tiled_register_##Q##_##P(KernelTable *);  \
     void abq_tiled_grouped_register_##Q##_##P(KernelTable *);  \
     void abq_decode_tiled_register_##Q##_##P(KernelTable *); \
-    void abq_decode_tiled_grouped_register_##Q##_##P(KernelTable *);
+    void abq_decode_tiled_grouped_register_##Q##_##P(KernelTable *); \
+    void abq_decode_tiled_f16_register_##Q##_##P(KernelTable *);
 ABQ_FOR_EACH_COMBO(ABQ_DECL)
 #undef ABQ_DECL
 
@@ -53,6 +54,7 @@ struct Registry {
     KernelTable tiled_grouped[2 * ABQ_NUM_COMBOS];
     KernelTable decode_tiled[2 * ABQ_NUM_COMBOS];
     KernelTable decode_tiled_grouped[2 * ABQ_NUM_COMBOS];
+    KernelTable decode_tiled_f16[2 * ABQ_NUM_COMBOS];
     Registry()
     {
         int i = 0;
@@ -65,6 +67,7 @@ struct Registry {
     abq_tiled_grouped_register_##Q##_##P(&tiled_grouped[i]); \
     abq_decode_tiled_register_##Q##_##P(&decode_tiled[i]); \
     abq_decode_tiled_grouped_register_##Q##_##P(&decode_tiled_grouped[i]); \
+    abq_decode_tiled_f16_register_##Q##_##P(&decode_tiled_f16[i]); \
     i += 2;
         ABQ_FOR_EACH_COMBO(ABQ_REG)
 #undef ABQ_REG
@@ -1168,6 +1171,7 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     a.x_zero = st->x_zero;
     a.x_group_sums = st->x_group_sums;
     a.w_zero_term = st->w_zero_term;
+    a.x_pack_scale = st->x_pack_scale;
     const Registry &reg = registry();
     const abq_tile_config &c = st->cfg;
     hipError_t e;
@@ -1203,9 +1207,12 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
         e = es[st->variant].launch(a, (hipStream_t)stream);
     } else if (st->strategy == ABQ_STRATEGY_TILED || st->strategy == ABQ_STRATEGY_DECODE_TILED) {
         // operands still in the reference layout are converted into the caller's workspace
-        const size_t xb = st->x_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->M, st->K, c.x_bits);
+        const bool x_f16 = st->x_layout == ABQ_LAYOUT_F16; // quantised inside the decode kernel
+        const size_t xb = (st->x_layout == ABQ_LAYOUT_TILED || x_f16) ? 0 : planes_bytes(st->M, st->K, c.x_bits);
         const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, c.w_bits);
         if (st->x_layout == ABQ_LAYOUT_FP6 || st->w_layout == ABQ_LAYOUT_FP6)
+            return ABQ_ERR_NOT_INITIALIZED;
+        if (x_f16 && (st->strategy != ABQ_STRATEGY_DECODE_TILED || st->group_size || !st->x_pack_scale))
             return ABQ_ERR_NOT_INITIALIZED;
         if (xb + wb > st->workspace_bytes || ((xb + wb) && !st->workspace))
             return ABQ_ERR_INVALID_ARG;
@@ -1223,7 +1230,7 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
             a.W = reinterpret_cast<const uint32_t *>(ws + xb);
         }
         const KernelTable *t = find_table(st->strategy == ABQ_STRATEGY_DECODE_TILED
-                                              ? (st->group_size ? reg.decode_tiled_grouped : reg.decode_tiled)
+                                              ? (st->group_size ? reg.decode_tiled_grouped : x_f16 ? reg.decode_tiled_f16 : reg.decode_tiled)
                                           : st->group_size ? reg.tiled_grouped
                                                            : reg.tiled,
                                           c.x_bits, c.w_bits, c.is_signed);
@@ -1342,6 +1349,24 @@ abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_l
     }
     st->x_layout = x_layout;
     st->w_layout = w_layout;
+    return ABQ_OK;
+}
+
+abq_status abq_gemm_set_f16_activations(abq_gemm_state *st, const void *x_f16, const float *scale_dev)
+{
+    if (!st || !st->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    if (!x_f16 || !scale_dev)
+        return ABQ_ERR_INVALID_ARG;
+    const abq_tile_config &c = st->cfg;
+    const KernelTable *t = find_table(registry().decode_tiled_f16, c.x_bits, c.w_bits, c.is_signed);
+    // the quantising instances mirror the first entries of the kernel's table
+    if (st->strategy != ABQ_STRATEGY_DECODE_TILED || st->group_size || st->act || st->w_layout != ABQ_LAYOUT_TILED || !t ||
+        st->variant < 0 || st->variant >= t->count || (size_t)st->M * st->K * 2 >= (1ull << 32))
+        return ABQ_ERR_UNSUPPORTED;
+    st->X = static_cast<const uint32_t *>(x_f16);
+    st->x_layout = ABQ_LAYOUT_F16;
+    st->x_pack_scale = scale_dev;
     return ABQ_OK;
 }
 

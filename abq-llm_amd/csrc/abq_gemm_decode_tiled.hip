@@ -112,9 +112,15 @@ template <int BITS, bool SIGNED> __device__ __forceinline__ void dt_unpack(const
     }
 }
 
-template <int Q, int P, bool SIGNED, int NW, int D, int T>
+// XF16: the activations arrive as fp16 [M][K] and are quantised here with one static scale, value =
+// (int)(half(x) * half(scale)) as pack_half of the reference does (abq_gemm_wrapper.cu:29-54), straight into the
+// int8 records in LDS: the pack kernel and its launch in front of every decode GEMM of the FT wrapper fall away.
+// Every workgroup converts the rows it multiplies (M x K halves, from L2 after the first).  8-bit activations.
+template <int Q, int P, bool SIGNED, int NW, int D, int T, bool XF16 = false>
 __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, int mrows)
 {
+    static_assert(!XF16 || Q == 8, "in-kernel quantisation writes 8-bit records");
+    constexpr int XP = 4;        // XF16: 16-byte units of eight halves per thread and pass (eight rows of 4096 in one pass; more spills)
     constexpr int NXL = Q / P;   // activation chunks (16 bytes) per weight unit
     constexpr int NM = 8 / P;    // MFMAs per weight unit
     constexpr int MX = 8 / Q;    // MFMAs per activation chunk
@@ -142,7 +148,37 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
     const int xchunks = KT * Mb * Q;
 
     // ---- activations: LDS chunk p <- chunk p ^ ((p / Q) & (Q - 1)) of the workgroup's rows -----------
-    if (Mb == M) { // the rows of all K tiles are one contiguous block
+    // (XF16: loaded, quantised and written inside the first round below)
+    const int upr = a.K >> 3;     // XF16: units of eight halves per row
+    const int nunits = Mb * upr;
+    const char *Xh = Xt + (size_t)m0 * a.K * 2;
+    uint32_t sel_pair = 0, sel_half = 0;
+    if constexpr (XF16)
+        quad_transpose_selectors(tid & 3, sel_pair, sel_half);
+    // eight halves of unit p (row p / upr, elements 8 u .. 8 u + 7) -> their bytes of the row's int8 record: the
+    // quad's four units are one word-set, whose expanded dword s, byte c is element 7 - s of lane 3 - c
+    auto quantise_unit = [&](const v4u &raw, int p, _Float16 hs) {
+        union {
+            v4u q;
+            _Float16 h[8];
+        } r;
+        r.q = raw;
+        int v[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            v[c] = (int)(_Float16)(r.h[c] * hs); // fp16 product rounded to nearest even, conversion truncating
+        const uint32_t e_even = quad_transpose_bytes(pack_low_bytes(v[7], v[5], v[3], v[1]), sel_pair, sel_half);
+        const uint32_t e_odd = quad_transpose_bytes(pack_low_bytes(v[6], v[4], v[2], v[0]), sel_pair, sel_half);
+        if (p < nunits) {
+            const int row = p / upr, u = p - row * upr;
+            const int rowi = (u >> 4) * Mb + row;                        // K tile * rows + row
+            const int dw = 8 * ((u >> 2) & 3) + 2 * (u & 3);             // first of the lane's two dwords in the record
+            const int chunk = (dw >> 2) ^ (rowi & 7);
+            *reinterpret_cast<uint2 *>(xs + ((uint32_t)rowi * 8 + chunk) * 16u + (dw & 3) * 4u) = make_uint2(e_even, e_odd);
+        }
+    };
+    if constexpr (XF16) {
+    } else if (Mb == M) { // the rows of all K tiles are one contiguous block
 #pragma unroll
         for (int i = 0; i < XC; ++i) {
             const int pb = wid * 64 + i * NT; // wave-uniform
@@ -194,6 +230,13 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
         // this round's steps of the wave: wid + (round * D + d) * NW.  Every wave issues D * T loads (steps past
         // the end repeat the last one), so that the waits below can count.
         v4u wb[D][T];
+        v4u xr[XF16 ? XP : 1];
+        if (XF16 && round == 0) {
+#pragma unroll
+            for (int i = 0; i < XP; ++i)
+                if (i * NT < nunits) // the same for every wave: the counted waits below do not depend on it
+                    xr[i] = dt_load16(Xh, (uint32_t)min(tid + i * NT, nunits - 1) * 16u);
+        }
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             const int s = min(wid + (round * D + d) * NW, S - 1);
@@ -206,6 +249,30 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
         }
         if (round == 0) {
             dt_wait_loads<D * T>(); // the activation loads are older than these
+            if constexpr (XF16) {
+                const _Float16 hs = (_Float16)a.x_pack_scale[0];
+#pragma unroll
+                for (int i = 0; i < XP; ++i) {
+                    if (i * NT < nunits) { // the quads of a wave are whole
+                        dt_landed(xr[i]);
+                        quantise_unit(xr[i], tid + i * NT, hs);
+                    }
+                }
+                // rows too long for one pass: further passes, their latency exposed
+                for (int base = XP * NT; base < nunits; base += XP * NT) {
+                    v4u more[XP];
+#pragma unroll
+                    for (int i = 0; i < XP; ++i)
+                        more[i] = dt_load16(Xh, (uint32_t)min(base + tid + i * NT, nunits - 1) * 16u);
+                    dt_wait_loads<0>(); // these are the youngest loads
+#pragma unroll
+                    for (int i = 0; i < XP; ++i) {
+                        dt_landed(more[i]);
+                        if (base + i * NT < nunits)
+                            quantise_unit(more[i], base + tid + i * NT, hs);
+                    }
+                }
+            }
             __syncthreads();
         }
 #pragma unroll
@@ -276,20 +343,22 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
     }
 }
 
-template <int Q, int P, bool SIGNED, int NW, int D, int T>
+template <int Q, int P, bool SIGNED, int NW, int D, int T, bool XF16 = false>
 static hipError_t launch_decode_tiled(const GemmArgs &a, hipStream_t stream)
 {
     const int mrows = decode_tiled_rows(NW, T, a.M, a.K, Q);
-    if (mrows == 0 || (size_t)a.N * a.K * P / 8 >= (1ull << 32) || (size_t)a.M * a.K * Q / 8 >= (1ull << 32))
+    if (mrows == 0 || (size_t)a.N * a.K * P / 8 >= (1ull << 32) || (size_t)a.M * a.K * (XF16 ? 16 : Q) / 8 >= (1ull << 32))
+        return hipErrorInvalidValue;
+    if (XF16 && !a.x_pack_scale)
         return hipErrorInvalidValue;
     const size_t lds = decode_tiled_lds(NW, T, mrows, a.K, Q);
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled<Q, P, SIGNED, NW, D, T>),
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled<Q, P, SIGNED, NW, D, T, XF16>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess)
         return attr;
     const int tiles = (a.N + 15) / 16;
     const dim3 grid((tiles + T - 1) / T, (a.M + mrows - 1) / mrows);
-    hipLaunchKernelGGL((gemm_decode_tiled<Q, P, SIGNED, NW, D, T>), grid, dim3(64 * NW), lds, stream, a, mrows);
+    hipLaunchKernelGGL((gemm_decode_tiled<Q, P, SIGNED, NW, D, T, XF16>), grid, dim3(64 * NW), lds, stream, a, mrows);
     return hipGetLastError();
 }
 
@@ -616,6 +685,15 @@ template <int Q, int P, bool SIGNED> static hipError_t launch_decode_tiled_group
 
 #if (ABQ_Q == 2 || ABQ_Q == 4 || ABQ_Q == 8) && (ABQ_P == 2 || ABQ_P == 4 || ABQ_P == 8)
 static const KernelEntry kSigned[] = { ABQ_DT_VARIANTS(ABQ_DT_ENTRY_T) };
+// the single-tile instances with in-kernel quantisation of fp16 activations (8-bit activations, signed), same order
+#if ABQ_Q == 8
+#define ABQ_DT_ENTRY_X(NW, D, T) { 16, 1, T, 1, 1, NW, 6, &launch_decode_tiled<ABQ_Q, ABQ_P, true, NW, D, T, true>, (512 / ABQ_P) * D },
+static const KernelEntry kSignedF16[] = { ABQ_DT_ENTRY_X(16, 1, 1) ABQ_DT_ENTRY_X(16, 3, 1) ABQ_DT_ENTRY_X(8, 2, 1) };
+#define ABQ_DT_NF16 3
+#else
+static const KernelEntry *const kSignedF16 = nullptr;
+#define ABQ_DT_NF16 0
+#endif
 // one entry: the launcher picks waves, loads in flight and tiles by shape
 static const KernelEntry kSignedGrouped[] = { { 16, 1, 1, 1, 1, 16, 6, &launch_decode_tiled_grouped<ABQ_Q, ABQ_P, true>, 128 } };
 #if ABQ_Q < 8
@@ -636,6 +714,8 @@ static const KernelEntry *const kSigned = nullptr;
 static const KernelEntry *const kUnsigned = nullptr;
 static const KernelEntry *const kSignedGrouped = nullptr;
 static const KernelEntry *const kUnsignedGrouped = nullptr;
+static const KernelEntry *const kSignedF16 = nullptr;
+#define ABQ_DT_NF16 0
 #define ABQ_DT_NSIGNED 0
 #define ABQ_DT_NUNSIGNED 0
 #endif
@@ -647,6 +727,12 @@ void ABQ_CAT(abq_decode_tiled_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)
 {
     out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSigned, ABQ_DT_NSIGNED };
     out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, kUnsigned, ABQ_DT_NUNSIGNED };
+}
+
+void ABQ_CAT(abq_decode_tiled_f16_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)
+{
+    out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSignedF16, ABQ_DT_NF16 };
+    out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, nullptr, 0 };
 }
 
 void ABQ_CAT(abq_decode_tiled_grouped_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)

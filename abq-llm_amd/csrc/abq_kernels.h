@@ -27,6 +27,7 @@ struct GemmArgs {
     const float *x_zero;       // [M], in units of activation codes
     const int *x_group_sums;   // [M][K/group_size] sums of activation codes (needed with w_zero)
     const float *w_zero_term;  // [N] sum_g w_scale * (sum of weight codes - group_size * w_zero) (needed with x_zero)
+    const float *x_pack_scale; // kernels that quantise fp16 activations themselves: X is fp16 [M][K], this the static scale
 };
 
 typedef hipError_t (*GemmLauncher)(const GemmArgs &, hipStream_t);
@@ -112,6 +113,36 @@ __device__ __forceinline__ void tile_of_workgroup(int id, int m_blocks, int n_bl
     const int gm = min(GM, m_blocks - grp * GM); // the last group may be short
     *mb = grp * GM + in % gm;
     *nb = xcd * n_blocks_per_xcd + in / gm;
+}
+
+// ---- byte shuffles inside a quad of lanes (the packing kernels and the decode kernel that quantises its own
+// activations assemble K-tiled 8-bit records with them) ------------------------------------------------
+
+// The low bytes of four integers as one dword, a in byte 0.
+__device__ __forceinline__ uint32_t pack_low_bytes(int a, int b, int c, int d)
+{
+    const uint32_t ab = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
+    const uint32_t cd = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
+}
+
+// 4 x 4 byte transpose across a quad with the lane order reversed: lane s returns the dword whose byte c is
+// byte s of lane 3 - c's argument.  sel_pair / sel_half are the lane's byte selectors of the two exchange
+// steps (quad_transpose_selectors).
+__device__ __forceinline__ uint32_t quad_transpose_bytes(uint32_t v, uint32_t sel_pair, uint32_t sel_half)
+{
+    const uint32_t p = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true); // lane ^ 1
+    const uint32_t x = __builtin_amdgcn_perm(p, v, sel_pair);
+    const uint32_t q = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true); // lane ^ 2
+    return __builtin_amdgcn_perm(q, x, sel_half);
+}
+
+__device__ __forceinline__ void quad_transpose_selectors(int quad_lane, uint32_t &sel_pair, uint32_t &sel_half)
+{
+    // step 1: even lanes keep their bytes 0, 2 and take the partner's 0, 2; odd lanes the bytes 1, 3
+    sel_pair = (quad_lane & 1) ? 0x03070105u : 0x06020400u;
+    // step 2: lanes 0, 1 take the low halves, lanes 2, 3 the high halves, bytes in reversed order
+    sel_half = (quad_lane & 2) ? 0x06070203u : 0x00010405u;
 }
 
 __device__ __forceinline__ float silu(float x) { return x / (1.0f + __expf(-x)); }

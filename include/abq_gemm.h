@@ -183,6 +183,7 @@ typedef struct abq_gemm_state {
     const int32_t *x_group_sums;
     const float *w_zero_term;
     int act;                 /* abq_activation fused into the epilogue */
+    const float *x_pack_scale; /* x_layout == ABQ_LAYOUT_F16: the static quantisation scale, see abq_gemm_set_f16_activations */
 } abq_gemm_state;
 
 /* Replaces AqBMMAInitFn / AqBWMMAInitFn (engine/mma_any/aq_bmma_op.h:141-147,163 and
@@ -275,7 +276,8 @@ abq_status abq_quant_pack_f16(const void *x_f16, int rows, int k, int bits, int 
 typedef enum abq_layout {
     ABQ_LAYOUT_PLANES = 0, /* the reference's wire format */
     ABQ_LAYOUT_TILED = 1,
-    ABQ_LAYOUT_FP6 = 2     /* records of 6-bit sign-magnitude codes, see below */
+    ABQ_LAYOUT_FP6 = 2,    /* records of 6-bit sign-magnitude codes, see below */
+    ABQ_LAYOUT_F16 = 3     /* activations only, set by abq_gemm_set_f16_activations: X is the fp16 matrix itself */
 } abq_layout;
 
 /* bytes of a packed operand in either layout */
@@ -311,6 +313,15 @@ abq_status abq_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int ro
  * and so are a tiled and an FP6 operand together, an FP6 operand with group scales of groups other
  * than 128, and an FP6 operand of a bit pair or K that does not qualify. */
 abq_status abq_gemm_set_operand_layout(abq_gemm_state *state, int x_layout, int w_layout);
+
+/* Decode without a packing launch (ABQGEMMWrapper::gemm of the reference packs A and runs the GEMM, two launches,
+ * fastertransformer/src/fastertransformer/kernels/abqgemm/abq_gemm_wrapper.cu:79-138; at M = 1 the second costs as
+ * much as the first).  On a state that runs ABQ_STRATEGY_DECODE_TILED (M <= 16, prepared weights) with signed
+ * 8-bit activations and no group scales, X becomes the fp16 activations [M][K] themselves: every workgroup
+ * quantises the rows it multiplies, value = (int)(half(x) * half(scale_dev[0])) as abq_pack_f16 does, into its
+ * LDS.  Results are bit for bit those of abq_pack_f16_tiled followed by the same GEMM.  Any other state:
+ * ABQ_ERR_UNSUPPORTED, and the caller packs as before. */
+abq_status abq_gemm_set_f16_activations(abq_gemm_state *state, const void *x_f16, const float *scale_dev);
 
 /* Workspace needed by abq_gemm_exec if the state ran as ABQ_STRATEGY_TILED (ABQ_STRATEGY_FP6)
  * with its current operand layouts: the converted copies of the operands still in the reference

@@ -257,13 +257,13 @@ static void gpu_paths()
         hipEvent_t e0, e1;
         HIP_OK(hipEventCreate(&e0));
         HIP_OK(hipEventCreate(&e1));
-        for (int M : { 1024, 300, 16, 1 }) {
+        for (int M : { 1024, 300, 16, 8, 4, 2, 1 }) {
             float us[2] = { 0.f, 0.f };
             for (int prepared = 0; prepared < 2; ++prepared) {
                 _Float16 *d_d = prepared ? d_d1 : d_d0;
                 const int *d_b = prepared ? d_b1 : d_b0;
                 HIP_OK(hipMemsetAsync(d_d, 0xff, (size_t)M * N * 2, stream));
-                const int reps = 20;
+                const int reps = 200;
                 for (int it = 0; it < reps + 2; ++it) {
                     if (it == 2)
                         HIP_OK(hipEventRecord(e0, stream));

@@ -98,6 +98,40 @@ def test_pack_f16_tiled_equals_the_relayout_of_the_planes(abq, rows, k):
         assert torch.equal(got.view(-1), want.view(-1)), bits
 
 
+@pytest.mark.parametrize("p", [2, 4, 8])
+def test_decode_quantises_fp16_activations_itself(abq, oracle, p):
+    """abq_gemm_set_f16_activations: the decode kernel on prepared weights reads fp16 activations and quantises them
+    with the static scale inside the kernel; bit for bit abq_pack_f16 followed by the GEMM, on every shape class
+    (several passes over long rows, row blocks, ragged N, every instance the default picks)."""
+    rng = np.random.default_rng(70 + p)
+    scale = torch.tensor([127.0 / 6.0], dtype=torch.float32, device="cuda")
+    for (M, N, K) in [(1, 4096, 4096), (4, 11008, 4096), (8, 4096, 11008), (16, 200, 384), (3, 16, 128), (16, 1040, 11008),
+                      (2, 4096, 11008), (13, 4100, 2176)]:
+        x = (torch.randn((M, K), device="cuda") * 3).to(torch.float16)
+        x[0, :4] = torch.tensor([0.0, -0.0, 6.0, -6.0], dtype=torch.float16)
+        w = rand_vals(rng, N, K, p, True)
+        wt = abq.relayout_planes(planes_dev(oracle.pack_i32(w, p)))
+        xt = abq.pack_f16(x, scale, 8, tiled=True)
+        for kw in (dict(), dict(out_kind=abq.OUT_F16_TENSOR_F32SCALE, c_scale=torch.tensor([0.0123], dtype=torch.float32, device="cuda"))):
+            want = abq.Gemm(xt, wt, True, x_tiled=True, w_tiled=True, **kw)
+            assert want.strategy == "decode_tiled"
+            want_out = want.run().clone()
+            g = abq.Gemm(xt, wt, True, x_tiled=True, w_tiled=True, **kw)
+            g.set_f16_activations(x, scale)
+            got = g.run()
+            torch.cuda.synchronize()
+            assert torch.equal(got, want_out), (M, N, K, p, kw.keys())
+    # states the kernel does not serve are refused and stay usable
+    x = (torch.randn((64, 256), device="cuda")).to(torch.float16)
+    xt = abq.pack_f16(x, scale, 8, tiled=True)
+    wt = abq.relayout_planes(planes_dev(oracle.pack_i32(rand_vals(rng, 32, 256, p, True), p)))
+    g = abq.Gemm(xt, wt, True, x_tiled=True, w_tiled=True)  # 64 rows: the prefill kernel
+    with pytest.raises(abq.AbqError) as e:
+        g.set_f16_activations(x, scale)
+    assert e.value.status == abq.ABQ_ERR_UNSUPPORTED
+    g.run()
+
+
 def field_packed(patterns, bits):
     """The K-tiled, field-packed layout written out from its definition: patterns [rows, K] are the
     elements' bit patterns (low `bits` bits).  A row's K tile of 128 elements is one record of
