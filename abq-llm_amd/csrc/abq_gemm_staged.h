@@ -104,6 +104,8 @@ template <int N> __device__ __forceinline__ void staged_wait_loads()
 __device__ __forceinline__ void staged_load_to_lds(const v4u *src, unsigned lds_addr)
 {
     // the LDS address is the same in every lane; readfirstlane tells the compiler so
+    // (M0 cannot be named as clobbered: the compiler reserves it, rejects it in a clobber list, and sets it up itself
+    // right before each of its own uses; it keeps no value there across other instructions.)
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)
                  : "memory");
 }
