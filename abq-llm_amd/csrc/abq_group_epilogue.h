@@ -66,89 +66,138 @@ __device__ __forceinline__ void store_wave_tile_f16(_Float16 *out, int row_len, 
     }
 }
 
-constexpr int kZeroPointChunk = 32;                      // groups staged through LDS at a time
-constexpr int kZeroPointRow = kZeroPointChunk + 1;       // floats per staged row: odd, so that 32 rows hit 32 banks
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 
-// LDS the zero-point staging needs for a BM x BN tile.
-constexpr int zero_point_lds_bytes(int bm, int bn) { return (bm + bn) * kZeroPointRow * 4; }
+// Eight consecutive per-group values of one row, groups [gb, gb + 8) of `groups`, zeros past the end.  `whole`:
+// the eight exist and rows start on 16-byte boundaries (wave-uniform), so two 16-byte loads do.
+template <typename T> __device__ __forceinline__ void load_groups8(const T *row, int gb, int groups, bool whole, T (&v)[8])
+{
+    if (whole) {
+        struct alignas(16) Q { T q[4]; };
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const Q t = *reinterpret_cast<const Q *>(row + gb + 4 * c);
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                v[4 * c + d] = t.q[d];
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            v[t] = gb + t < groups ? row[gb + t] : T(0);
+    }
+}
 
 // facc[i][j][e]: MFMA tile (i, j) of this wave, element e in the 32x32 accumulator layout (row
 // 8 * (e / 4) + 4 * g + e % 4, column r).  smem: the workgroup's LDS, free for reuse once a barrier has
-// been passed; zero_point_lds_bytes(BM, BN) of it are used when w_zero is set.
+// been passed (only the fp16 store uses it).
 //
 // The weight zero points are a small matrix product of their own, out -= Sx (M x groups) times
-// (w_scale * w_zero)^T (groups x N).  Both factors are staged through LDS 32 groups at a time (coalesced
-// loads along the groups) and multiplied on the fp32 matrix cores: v_mfma_f32_32x32x2_f32, lane (r, g)
-// supplies row r of the activation block and column r of the weight block for the g-th of the
-// instruction's two K indices.
+// (w_scale * w_zero)^T (groups x N), done on the bf16 matrix cores (v_mfma_f32_32x32x16_bf16, an eighth of the
+// time of the fp32 instruction per product) without loss: a group sum of at most 128 8-bit codes splits exactly
+// into two bf16 numbers (its multiple of 128 and the remainder below 128), c = -w_scale * w_zero into bf16(c) and
+// bf16(c - bf16(c)), both rounded to nearest, which carries c to 2^-18 relative; the four products of the pieces
+// take four of the instruction's sixteen K slots, so one instruction covers four groups and a chunk of 32 groups
+// takes eight per MFMA tile.  Lane (r, g) supplies row r of the activation block and column r of the weight block
+// for the K slots 8 g .. 8 g + 7, i.e. for two groups; which two is free as long as both operands agree, and the
+// choice here, groups 16 g + 2 q and 16 g + 2 q + 1 for instruction q of the chunk, lets every lane read its
+// sixteen groups of a row as 64 contiguous bytes straight from global memory: no staging, no barrier.
 // LDS_BYTES: size of the workgroup's LDS at smem.
 template <int TM, int TN, int WM, int WN, int LDS_BYTES>
 __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&facc)[TM][TN], unsigned char *smem, int M,
                                                      int N, int m0, int n0, int wm, int wn, int r, int g, int tid)
 {
-    static_assert(zero_point_lds_bytes(32 * TM * WM, 32 * TN * WN) <= LDS_BYTES, "the zero-point staging fits");
-    constexpr int NT = 64 * WM * WN;
-    constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
-    constexpr int GC = kZeroPointChunk, GP = kZeroPointRow;
+    // The rows' scales: element e of a lane sits in row 8 (e / 4) + 4 g + e % 4 of its MFMA tile, four consecutive
+    // rows per e / 4.  Requested before the zero-point product, used after it.
+    auto row_values = [&](const float *src, float (&v)[TM][16]) {
+        const bool whole = (M & 3) == 0 && (reinterpret_cast<size_t>(src) & 15) == 0; // wave-uniform
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int mr = m0 + wm * 32 * TM + i * 32 + 8 * q + 4 * g;
+                float4 s4;
+                if (whole)
+                    s4 = *reinterpret_cast<const float4 *>(src + min(mr, M - 4));
+                else
+                    s4 = make_float4(src[min(mr, M - 1)], src[min(mr + 1, M - 1)], src[min(mr + 2, M - 1)], src[min(mr + 3, M - 1)]);
+                v[i][4 * q] = s4.x, v[i][4 * q + 1] = s4.y, v[i][4 * q + 2] = s4.z, v[i][4 * q + 3] = s4.w;
+            }
+    };
+    float xs[TM][16];
+    row_values(a.x_scale, xs);
+
     if (a.w_zero) {
         const int groups = a.K / a.group_size;
-        float *zs_x = reinterpret_cast<float *>(smem); // [BM][GP]
-        float *zs_w = zs_x + BM * GP;                  // [BN][GP], negated
-        for (int g0 = 0; g0 < groups; g0 += GC) {
-            __syncthreads();
-            // every thread's loads of a chunk are issued back to back (trip counts are compile-time)
-            static_assert((GC * BM) % NT == 0 && (GC * BN) % NT == 0, "whole passes of the workgroup");
-            float vx[GC * BM / NT], vw[GC * BN / NT];
+        const bool rows16 = (groups & 3) == 0 && ((reinterpret_cast<size_t>(a.x_group_sums) | reinterpret_cast<size_t>(a.w_scale) |
+                                                   reinterpret_cast<size_t>(a.w_zero)) & 15) == 0;
+        for (int g0 = 0; g0 < groups; g0 += 32) {
+            const bool whole = rows16 && g0 + 32 <= groups; // wave-uniform
 #pragma unroll
-            for (int it = 0; it < GC * BM / NT; ++it) {
-                const int u = tid + it * NT, rr = u / GC, gl = u % GC;
-                const int m = min(m0 + rr, M - 1);
-                vx[it] = g0 + gl < groups ? (float)a.x_group_sums[(size_t)m * groups + g0 + gl] : 0.f;
-            }
+            for (int h = 0; h < 2; ++h) { // half of the lane's sixteen groups at a time: four instructions per MFMA tile
+                const int gb = g0 + 16 * g + 8 * h;
+                unsigned ap[TM][8][2], bp[TN][8];
 #pragma unroll
-            for (int it = 0; it < GC * BN / NT; ++it) {
-                const int u = tid + it * NT, rr = u / GC, gl = u % GC;
-                const size_t idx = (size_t)min(n0 + rr, N - 1) * groups + g0 + gl;
-                vw[it] = g0 + gl < groups ? -(a.w_scale[idx] * a.w_zero[idx]) : 0.f;
-            }
+                for (int i = 0; i < TM; ++i) {
+                    int sx[8];
+                    load_groups8(a.x_group_sums + (size_t)min(m0 + wm * 32 * TM + i * 32 + r, M - 1) * groups, gb, groups, whole, sx);
 #pragma unroll
-            for (int it = 0; it < GC * BM / NT; ++it) {
-                const int u = tid + it * NT;
-                zs_x[(u / GC) * GP + u % GC] = vx[it];
-            }
+                    for (int t = 0; t < 8; ++t) {
+                        const int low = sx[t] & 127;
+                        const unsigned hi = __builtin_bit_cast(unsigned, (float)(sx[t] - low)), lo = __builtin_bit_cast(unsigned, (float)low);
+                        ap[i][t][0] = __builtin_amdgcn_perm(hi, hi, 0x07060706u); // (hi, hi) as two bf16: the upper halves, exact
+                        ap[i][t][1] = __builtin_amdgcn_perm(lo, lo, 0x07060706u);
+                    }
+                }
 #pragma unroll
-            for (int it = 0; it < GC * BN / NT; ++it) {
-                const int u = tid + it * NT;
-                zs_w[(u / GC) * GP + u % GC] = vw[it];
-            }
-            __syncthreads();
-            const float *xa = zs_x + (wm * 32 * TM + r) * GP + g;
-            const float *wb = zs_w + (wn * 32 * TN + r) * GP + g;
-#pragma unroll 4
-            for (int t = 0; t < GC / 2; ++t) {
-                float av[TM], bv[TN];
+                for (int j = 0; j < TN; ++j) {
+                    float ws[8], wz[8];
+                    const size_t row = (size_t)min(n0 + wn * 32 * TN + j * 32 + r, N - 1) * groups;
+                    load_groups8(a.w_scale + row, gb, groups, whole, ws);
+                    load_groups8(a.w_zero + row, gb, groups, whole, wz);
 #pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    av[i] = xa[i * 32 * GP + 2 * t];
+                    for (int t = 0; t < 8; ++t) {
+                        const float c = -(ws[t] * wz[t]);
+                        v2bf p;
+                        p[0] = (__bf16)c;
+                        p[1] = (__bf16)(c - (float)p[0]);
+                        bp[j][t] = __builtin_bit_cast(unsigned, p);
+                    }
+                }
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    bv[j] = wb[j * 32 * GP + 2 * t];
+                for (int q = 0; q < 4; ++q)
 #pragma unroll
-                for (int i = 0; i < TM; ++i)
+                    for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        facc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], facc[i][j], 0, 0, 0);
+                        for (int j = 0; j < TN; ++j) {
+                            // K slots of a group: (hi, hi, lo, lo) against (c1, c2, c1, c2)
+                            const v4u av = {ap[i][2 * q][0], ap[i][2 * q][1], ap[i][2 * q + 1][0], ap[i][2 * q + 1][1]};
+                            const v4u bv = {bp[j][2 * q], bp[j][2 * q], bp[j][2 * q + 1], bp[j][2 * q + 1]};
+                            facc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, av),
+                                                                                 __builtin_bit_cast(v8bf, bv), facc[i][j], 0, 0, 0);
+                        }
             }
         }
     }
-    // what is left per element: the activation zero points (a rank-one term), the token scale, the gate
+    if (a.x_zero) {
+        // the activation zero points: a rank-one term
+        float xz[TM][16], wzt[TN];
+        row_values(a.x_zero, xz);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            wzt[j] = a.w_zero_term[min(n0 + wn * 32 * TN + j * 32 + r, N - 1)];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    facc[i][j][e] -= xz[i][e] * wzt[j];
+    }
     auto finish = [&](int i, int j, int e) -> float {
-        const int mc = min(m0 + wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4), M - 1);
-        const int nc = min(n0 + wn * 32 * TN + j * 32 + r, N - 1);
-        float v = facc[i][j][e];
-        if (a.x_zero)
-            v -= a.x_zero[mc] * a.w_zero_term[nc];
-        v *= a.x_scale[mc];
+        float v = facc[i][j][e] * xs[i][e];
         if (a.act) {
             // SiLU gate: columns come in blocks of 16 gate rows followed by their 16 up rows, so the
             // partner of lane r is lane r ^ 16 of the same MFMA tile (N is a multiple of 32); lanes
@@ -163,7 +212,7 @@ __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&f
     const int cols = a.act ? N / 2 : N;
     // whole lines per store where the output allows it: the wave's tile goes through a region of LDS of its own
     if (WM * WN * WaveTileF16<TM, TN, 32>::kBytes <= LDS_BYTES && store_wave_tile_f16_ok(out, cols, cols)) {
-        __syncthreads(); // the LDS is free: K loop and zero-point staging are behind every wave
+        __syncthreads(); // the LDS is free: the K loop is behind every wave
         if (a.act)
             store_wave_tile_f16<TM, TN, 16>(out, cols, M, cols, m0 + wm * 32 * TM, (n0 + wn * 32 * TN) / 2,
                                             smem + wave * WaveTileF16<TM, TN, 16>::kBytes, lane, finish);
