@@ -117,6 +117,14 @@ __device__ __forceinline__ void staged_load_dword_to_lds(const float *src, unsig
                  : "memory");
 }
 
+// LDS of a launch that writes fp16: the stages, or the waves' output tiles if those are larger and still fit beside
+// the other workgroup of the compute unit (two for the four-wave tiles with at most four MFMA tiles a wave).
+template <int TM, int TN, int WM, int WN, int STAGE_BYTES> struct StagedOutputLds {
+    static constexpr int kTiles = WM * WN * WaveTileF16<TM, TN>::kBytes;
+    static constexpr int kCap = ((WM * WN > 4 || TM * TN > 4) ? 160 : 80) * 1024;
+    static constexpr int value = (kTiles > STAGE_BYTES && kTiles <= kCap) ? kTiles : STAGE_BYTES;
+};
+
 // QB / PB: bits of the activation / weight fields (2, 4 or 8; ignored for FP6).
 //
 // GROUPED: group-wise weight scales (one per 128 elements along K, i.e. per K tile: w_scale[N][K / 128]),
@@ -150,6 +158,13 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     static_assert(NPW * S < 64, "the load counter has six bits");
     static_assert(BUF_BYTES % 512 == 0 && (BM * TA::kRow) % 512 == 0 && (32 * TA::kRow) % 256 == 0 && (32 * TB::kRow) % 256 == 0,
                   "stages, operand blocks and fragment rows keep the placement pattern");
+
+    // fp16 outputs leave through LDS as whole lines, each wave's tile in a region of its own; where the stages are
+    // smaller than that (the narrowest operand pairs), the launch asks for the larger of the two, as long as the
+    // workgroups that share a compute unit still fit
+    constexpr int F16_LDS = WM * WN * WaveTileF16<TM, TN>::kBytes;
+    constexpr int LDS_BYTES = StagedOutputLds<TM, TN, WM, WN, S * BUF_BYTES>::value;
+    constexpr bool F16_VIA_LDS = F16_LDS <= LDS_BYTES;
 
     extern __shared__ __align__(16) unsigned char smem[]; // [S][BM rows of X | BN rows of W]
 
@@ -372,7 +387,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
 #pragma unroll
         for (int e = 0; e < 16; ++e)
             facc[TM - 1][TN - 1][e] += (float)acc[TM - 1][TN - 1][e] * sc_last;
-        group_scale_epilogue<TM, TN, WM, WN, S * BUF_BYTES>(a, facc, smem, M, N, m0, n0, wm, wn, r, g, tid);
+        group_scale_epilogue<TM, TN, WM, WN, LDS_BYTES>(a, facc, smem, M, N, m0, n0, wm, wn, r, g, tid);
         return;
     }
 
@@ -391,8 +406,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
             wsv[j] = a.w_scale[min(n0 + wn * 32 * TN + j * 32 + r, N - 1)];
         _Float16 *out = reinterpret_cast<_Float16 *>(a.D);
         using WT = WaveTileF16<TM, TN>;
-        // (the narrowest operand pairs have stages smaller than the waves' output tiles: direct stores there)
-        if (WM * WN * WT::kBytes <= S * BUF_BYTES && store_wave_tile_f16_ok(out, N, N)) {
+        if (F16_VIA_LDS && store_wave_tile_f16_ok(out, N, N)) {
             // whole 128-byte lines per store: the wave's tile goes through a region of LDS of its own
             float xsv[TM][16];
 #pragma unroll
@@ -427,7 +441,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         // as whole lines where the output allows it
         _Float16 *out = reinterpret_cast<_Float16 *>(a.D);
         using WT = WaveTileF16<TM, TN>;
-        if (WM * WN * WT::kBytes <= S * BUF_BYTES && store_wave_tile_f16_ok(out, N, N)) {
+        if (F16_VIA_LDS && store_wave_tile_f16_ok(out, N, N)) {
             const _Float16 scale = a.out_kind == 1 ? *reinterpret_cast<const _Float16 *>(a.C)
                                                    : (_Float16) * reinterpret_cast<const float *>(a.C);
             __syncthreads(); // every wave's loads have landed and its fragment reads are done: the stages are free
@@ -479,7 +493,9 @@ static hipError_t launch_mfma_staged(const GemmArgs &a, hipStream_t stream)
         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess)
         return attr;
-    hipLaunchKernelGGL((gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S, GROUPED>), grid, dim3(64 * WM * WN), Stages::kLds,
+    // int32 results are stored from the registers; every other kind goes through LDS
+    const size_t lds = a.out_kind == 0 ? Stages::kLds : (size_t)StagedOutputLds<TM, TN, WM, WN, (int)Stages::kLds>::value;
+    hipLaunchKernelGGL((gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S, GROUPED>), grid, dim3(64 * WM * WN), lds,
                        stream, a, reinterpret_cast<const v4u *>(a.X), reinterpret_cast<const v4u *>(a.W), m_blocks, npx);
     return hipGetLastError();
 }

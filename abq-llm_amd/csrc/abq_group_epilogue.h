@@ -20,8 +20,9 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 // 128-byte lines.  Each wave uses a region of its own (wave_tile_f16_lds_bytes), so only the wave's own
 // LDS traffic has to be ordered.  Needs an output row length and column count that are multiples
 // of 8 and a 16-byte aligned output (store_wave_tile_f16_ok).
-// CW: output columns per 32-column MFMA tile: 32, or 16 when only lanes r < 16 hold an output (the SiLU
-// gate folds each tile's two halves into one).
+// CW: output columns per 32-column MFMA tile: 32, or 16 for the SiLU gate, which folds each tile's two halves
+// into one: lanes r < 16 then hold the outputs of the elements e < 8 of column r, lanes r >= 16 those of the
+// elements e >= 8 of column r - 16 (value(i, j, e) is only used where the lane holds an output).
 template <int TM, int TN, int CW = 32> struct WaveTileF16 {
     static constexpr int kStride = 2 * CW * TN + 16;    // bytes per tile row in LDS
     static constexpr int kBytes = 32 * TM * kStride;    // per wave
@@ -48,9 +49,10 @@ __device__ __forceinline__ void store_wave_tile_f16(_Float16 *out, int row_len, 
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const _Float16 h = (_Float16)value(i, j, e); // every lane evaluates it (it may exchange data between lanes)
-                if (CW == 32 || r < CW)
-                    *reinterpret_cast<_Float16 *>(wave_lds + (i * 32 + 8 * (e / 4) + 4 * g + (e % 4)) * T::kStride + (j * CW + r) * 2) = h;
+                const _Float16 h = (_Float16)value(i, j, e);
+                if (CW == 32 || (e >> 3) == (r >> 4))
+                    *reinterpret_cast<_Float16 *>(wave_lds + (i * 32 + 8 * (e / 4) + 4 * g + (e % 4)) * T::kStride +
+                                                  (j * CW + (r & (CW - 1))) * 2) = h;
             }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -213,10 +215,25 @@ __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&f
     // whole lines per store where the output allows it: the wave's tile goes through a region of LDS of its own
     if (WM * WN * WaveTileF16<TM, TN, 32>::kBytes <= LDS_BYTES && store_wave_tile_f16_ok(out, cols, cols)) {
         __syncthreads(); // the LDS is free: the K loop is behind every wave
-        if (a.act)
+        if (a.act) {
+            // SiLU gate: columns come in blocks of 16 gate rows followed by their 16 up rows, so lane r < 16 holds the
+            // gate values of its 16 elements and lane r + 16 the up values of the same outputs.  The pair splits
+            // the 16 outputs: one exchange of eight values each way, and either lane evaluates eight gates.
+            float res[TM][TN][8];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        const float lo = facc[i][j][k] * xs[i][k], hi = facc[i][j][k + 8] * xs[i][k + 8];
+                        const float got = __shfl_xor(r < 16 ? hi : lo, 16);
+                        res[i][j][k] = r < 16 ? silu(lo) * got : silu(got) * hi;
+                    }
             store_wave_tile_f16<TM, TN, 16>(out, cols, M, cols, m0 + wm * 32 * TM, (n0 + wn * 32 * TN) / 2,
-                                            smem + wave * WaveTileF16<TM, TN, 16>::kBytes, lane, finish);
-        else
+                                            smem + wave * WaveTileF16<TM, TN, 16>::kBytes, lane,
+                                            [&](int i, int j, int e) { return res[i][j][e & 7]; });
+        } else
             store_wave_tile_f16<TM, TN, 32>(out, cols, M, cols, m0 + wm * 32 * TM, n0 + wn * 32 * TN,
                                             smem + wave * WaveTileF16<TM, TN, 32>::kBytes, lane, finish);
         return;

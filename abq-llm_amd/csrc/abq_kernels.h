@@ -145,7 +145,8 @@ __device__ __forceinline__ void quad_transpose_selectors(int quad_lane, uint32_t
     sel_half = (quad_lane & 2) ? 0x06070203u : 0x00010405u;
 }
 
-__device__ __forceinline__ float silu(float x) { return x / (1.0f + __expf(-x)); }
+// x * sigmoid(x), the reciprocal by the hardware instruction (1 ulp) instead of the division sequence
+__device__ __forceinline__ float silu(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
 // ---- output stage shared by all kernels ------------------------------------------------
 // out_kind values mirror abq_out_kind in include/abq_gemm.h.
