@@ -101,19 +101,22 @@ template <int N> __device__ __forceinline__ void staged_wait_loads()
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-__device__ __forceinline__ void staged_load_to_lds(const v4u *src, unsigned lds_addr)
+// `base` is the same in every lane (a scalar register pair), `offset` the lane's byte offset from it.
+__device__ __forceinline__ void staged_load_to_lds(const void *base, uint32_t offset, unsigned lds_addr)
 {
     // the LDS address is the same in every lane; readfirstlane tells the compiler so
     // (M0 cannot be named as clobbered: the compiler reserves it, rejects it in a clobber list, and sets it up itself
     // right before each of its own uses; it keeps no value there across other instructions.)
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(offset),
+                 "s"(base)
                  : "memory");
 }
 
 // The same with four bytes per lane (lane l lands at M0 + 4 * l): the group scales.
-__device__ __forceinline__ void staged_load_dword_to_lds(const float *src, unsigned lds_addr)
+__device__ __forceinline__ void staged_load_dword_to_lds(const void *base, uint32_t offset, unsigned lds_addr)
 {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(offset),
+                 "s"(base)
                  : "memory");
 }
 
@@ -186,7 +189,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     // at LDS place P of an operand block is unit lds_offset(P) / 16 of that operand's tile.  Loads past
     // the last one repeat an earlier load of the wave (same data, same place), so that every wave
     // issues NPW loads per tile.  Rows past the edge are clamped for loading and dropped at the store.
-    uint32_t goff[NPW]; // 16-byte units from the start of the operand's records of one K tile
+    uint32_t goff[NPW]; // bytes from the start of the operand's records of one K tile
 #pragma unroll
     for (int i = 0; i < NPR; ++i) {
         int q = wid + NW * i;
@@ -194,18 +197,18 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
             q -= NW;
         if (q < NIA) { // wave-uniform
             const int v = TA::lds_offset(64 * q + lane) >> 4;
-            goff[i] = (uint32_t)min(m0 + v / TA::kUnits, M - 1) * TA::kUnits + v % TA::kUnits;
+            goff[i] = 16u * ((uint32_t)min(m0 + v / TA::kUnits, M - 1) * TA::kUnits + v % TA::kUnits);
         } else {
             const int v = TB::lds_offset(64 * (q - NIA) + lane) >> 4;
-            goff[i] = (uint32_t)min(n0 + v / TB::kUnits, N - 1) * TB::kUnits + v % TB::kUnits;
+            goff[i] = 16u * ((uint32_t)min(n0 + v / TB::kUnits, N - 1) * TB::kUnits + v % TB::kUnits);
         }
     }
     // GROUPED: the wave's last load of a tile brings the scales of 64 weight rows (waves take the 64-row
     // blocks of the tile in turn; several waves bring the same block, which costs 256 bytes each).  The
-    // offset counts floats from the start of w_scale to the row's scale of K tile 0.
+    // offset counts bytes from the start of w_scale to the row's scale of K tile 0.
     const int sc_block = wid % (BN / 64 > 0 ? BN / 64 : 1);
     if constexpr (GROUPED)
-        goff[NPR] = (uint32_t)min(n0 + 64 * sc_block + lane, N - 1) * (uint32_t)ktiles;
+        goff[NPR] = 4u * ((uint32_t)min(n0 + 64 * sc_block + lane, N - 1) * (uint32_t)ktiles);
     const size_t stride_a = (size_t)M * TA::kUnits, stride_b = (size_t)N * TB::kUnits;
     const unsigned lds0 = (unsigned)(size_t)smem; // LDS byte address of the first stage
 
@@ -259,16 +262,32 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
                                                       staged_int8_operand<PB, SIGNED>(pb, ks), fresh ? zero : c, 0, 0, 0);
         }
     };
-    auto request = [&](int kt_req, int stage, int i) {
-        const int kn = min(kt_req, ktiles - 1); // tiles past the end: copies of the last, into stages nobody reads
+    // The tile the next requests are for: its operands' records and its scales, all wave-uniform (scalar
+    // registers), the lanes adding their 32-bit offsets.  Tiles past the end are copies of the last, into stages
+    // nobody reads.
+    const v4u *xq = xt, *wq = wt;
+    const float *sq = a.w_scale;
+    const unsigned lds_wave = lds0 + wid * 1024;
+    int kq = 0;
+    auto request = [&](int stage, int i) {
         if (GROUPED && i == NPR) {
-            staged_load_dword_to_lds(a.w_scale + goff[i] + kn, lds0 + stage + SC_OFF + sc_block * 256);
+            staged_load_dword_to_lds(sq, goff[i], lds0 + stage + SC_OFF + sc_block * 256);
             return;
         }
         int q = wid + NW * i;
-        if (q >= NI)
+        if (NI % NW != 0 && q >= NI)
             q -= NW;
-        staged_load_to_lds((q < NIA ? xt + kn * stride_a : wt + kn * stride_b) + goff[i], lds0 + stage + q * 1024);
+        // (which operand request i is for does not depend on the wave when the waves divide both operands' loads)
+        const bool activations = (NIA % NW == 0 && NI % NW == 0) ? NW * i < NIA : q < NIA;
+        staged_load_to_lds(activations ? (const void *)xq : (const void *)wq, goff[i], lds_wave + stage + (q - wid) * 1024);
+    };
+    auto next_tile = [&]() {
+        if (kq < ktiles - 1) {
+            xq += stride_a;
+            wq += stride_b;
+            sq += 1;
+        }
+        ++kq;
     };
 
     // Tile t lives in stage t % S from its request until its fragments have been read, which happens
@@ -276,10 +295,12 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     // requested right then into the stage tile t has just left.
     // prologue: tiles 0 .. S-1 requested; tile 0 read into the first fragment set; tile 1 landed
 #pragma unroll
-    for (int s = 0; s < S; ++s)
+    for (int s = 0; s < S; ++s) {
 #pragma unroll
         for (int i = 0; i < NPW; ++i)
-            request(s, s * BUF_BYTES, i);
+            request(s * BUF_BYTES, i);
+        next_tile();
+    }
     staged_wait_loads<NPW * (S - 1)>();
     __syncthreads();
 #pragma unroll
@@ -321,11 +342,12 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         {                                                                                                       \
             mfma(acc[(k / TN) % TM][k % TN], QC, (k / TN) % TM, k % TN, k / (TM * TN));                         \
             _Pragma("unroll") for (int d = k * NPW / NM; d < (k + 1) * NPW / NM; ++d)                           \
-                request((KT) + S, st_req, d);                                                                   \
+                request(st_req, d);                                                                             \
             _Pragma("unroll") for (int p = k * NR / NM; p < (k + 1) * NR / NM; ++p)                             \
                 read_piece(QN, st_rd, p);                                                                       \
             __builtin_amdgcn_sched_barrier(0);                                                                  \
         }                                                                                                       \
+        next_tile();                                                                                            \
         st_req = st_req + BUF_BYTES == S * BUF_BYTES ? 0 : st_req + BUF_BYTES;                                  \
         st_rd = st_rd + BUF_BYTES == S * BUF_BYTES ? 0 : st_rd + BUF_BYTES;                                     \
         staged_wait_loads<NPW * (S - 2)>(); /* tile KT + 2 has landed; the S - 2 younger ones may still fly */  \
@@ -345,7 +367,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
             const int u = k / kSteps, ks = k % kSteps, uf = (u + NU - 1) % NU;                                  \
             mfma(acc[u / TN][u % TN], QC, u / TN, u % TN, ks, ks == 0);                                         \
             _Pragma("unroll") for (int d = k * NPW / NM; d < (k + 1) * NPW / NM; ++d)                           \
-                request((KT) + S, st_req, d);                                                                   \
+                request(st_req, d);                                                                             \
             _Pragma("unroll") for (int p = k * NR / NM; p < (k + 1) * NR / NM; ++p)                             \
                 read_piece(QN, st_rd, p);                                                                       \
             const float scf = u == 0 ? sc_last : sc_cur[uf % TN];                                               \
@@ -356,6 +378,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         sc_last = sc_cur[TN - 1];                                                                               \
         _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                          \
             sc_cur[j] = sc_next[j];                                                                             \
+        next_tile();                                                                                            \
         st_req = st_req + BUF_BYTES == S * BUF_BYTES ? 0 : st_req + BUF_BYTES;                                  \
         st_rd = st_rd + BUF_BYTES == S * BUF_BYTES ? 0 : st_rd + BUF_BYTES;                                     \
         staged_wait_loads<NPW * (S - 2)>();                                                                     \
