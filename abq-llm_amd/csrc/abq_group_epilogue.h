@@ -92,6 +92,60 @@ template <typename T> __device__ __forceinline__ void load_groups8(const T *row,
     }
 }
 
+// Eight groups (from gb on) of the lane's TM activation rows and TN weight rows: group sums, scales, zero points.
+template <int TM, int TN>
+__device__ __forceinline__ void zero_point_loads(const GemmArgs &a, const uint32_t (&arow)[TM], const uint32_t (&brow)[TN], int gb,
+                                                 int groups, bool whole, int (&sx)[TM][8], float (&ws)[TN][8], float (&wz)[TN][8])
+{
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+        load_groups8(a.x_group_sums + arow[i], gb, groups, whole, sx[i]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        load_groups8(a.w_scale + brow[j], gb, groups, whole, ws[j]);
+        load_groups8(a.w_zero + brow[j], gb, groups, whole, wz[j]);
+    }
+}
+
+// facc -= (the eight groups' sums) x (their w_scale * w_zero)^T: four bf16 MFMAs per MFMA tile, see below.
+template <int TM, int TN>
+__device__ __forceinline__ void zero_point_product(const int (&sx)[TM][8], const float (&ws)[TN][8], const float (&wz)[TN][8],
+                                                   v16f (&facc)[TM][TN])
+{
+    unsigned ap[TM][8][2], bp[TN][8];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int low = sx[i][t] & 127;
+            const unsigned hi = __builtin_bit_cast(unsigned, (float)(sx[i][t] - low)), lo = __builtin_bit_cast(unsigned, (float)low);
+            ap[i][t][0] = __builtin_amdgcn_perm(hi, hi, 0x07060706u); // (hi, hi) as two bf16: the upper halves, exact
+            ap[i][t][1] = __builtin_amdgcn_perm(lo, lo, 0x07060706u);
+        }
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const float c = -(ws[j][t] * wz[j][t]);
+            v2bf p;
+            p[0] = (__bf16)c;
+            p[1] = (__bf16)(c - (float)p[0]);
+            bp[j][t] = __builtin_bit_cast(unsigned, p);
+        }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                // K slots of a group: (hi, hi, lo, lo) against (c1, c2, c1, c2)
+                const v4u av = {ap[i][2 * q][0], ap[i][2 * q][1], ap[i][2 * q + 1][0], ap[i][2 * q + 1][1]};
+                const v4u bv = {bp[j][2 * q], bp[j][2 * q], bp[j][2 * q + 1], bp[j][2 * q + 1]};
+                facc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, av), __builtin_bit_cast(v8bf, bv),
+                                                                     facc[i][j], 0, 0, 0);
+            }
+}
+
 // facc[i][j][e]: MFMA tile (i, j) of this wave, element e in the 32x32 accumulator layout (row
 // 8 * (e / 4) + 4 * g + e % 4, column r).  smem: the workgroup's LDS, free for reuse once a barrier has
 // been passed (only the fp16 store uses it).
@@ -106,8 +160,9 @@ template <typename T> __device__ __forceinline__ void load_groups8(const T *row,
 // for the K slots 8 g .. 8 g + 7, i.e. for two groups; which two is free as long as both operands agree, and the
 // choice here, groups 16 g + 2 q and 16 g + 2 q + 1 for instruction q of the chunk, lets every lane read its
 // sixteen groups of a row as 64 contiguous bytes straight from global memory: no staging, no barrier.
-// LDS_BYTES: size of the workgroup's LDS at smem.
-template <int TM, int TN, int WM, int WN, int LDS_BYTES>
+// LDS_BYTES: size of the workgroup's LDS at smem.  LOADS_FIRST: a chunk's loads are all requested before any is
+// used (one memory latency per chunk instead of two, 48 more registers).
+template <int TM, int TN, int WM, int WN, int LDS_BYTES, bool LOADS_FIRST = false>
 __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&facc)[TM][TN], unsigned char *smem, int M,
                                                      int N, int m0, int n0, int wm, int wn, int r, int g, int tid)
 {
@@ -135,52 +190,27 @@ __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&f
         const int groups = a.K / a.group_size;
         const bool rows16 = (groups & 3) == 0 && ((reinterpret_cast<size_t>(a.x_group_sums) | reinterpret_cast<size_t>(a.w_scale) |
                                                    reinterpret_cast<size_t>(a.w_zero)) & 15) == 0;
+        // rows of this lane in the three arrays (32-bit element offsets: the arrays hold fewer than 2^32 elements)
+        uint32_t arow[TM], brow[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            arow[i] = (uint32_t)min(m0 + wm * 32 * TM + i * 32 + r, M - 1) * (uint32_t)groups;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            brow[j] = (uint32_t)min(n0 + wn * 32 * TN + j * 32 + r, N - 1) * (uint32_t)groups;
         for (int g0 = 0; g0 < groups; g0 += 32) {
             const bool whole = rows16 && g0 + 32 <= groups; // wave-uniform
-#pragma unroll
-            for (int h = 0; h < 2; ++h) { // half of the lane's sixteen groups at a time: four instructions per MFMA tile
-                const int gb = g0 + 16 * g + 8 * h;
-                unsigned ap[TM][8][2], bp[TN][8];
-#pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    int sx[8];
-                    load_groups8(a.x_group_sums + (size_t)min(m0 + wm * 32 * TM + i * 32 + r, M - 1) * groups, gb, groups, whole, sx);
-#pragma unroll
-                    for (int t = 0; t < 8; ++t) {
-                        const int low = sx[t] & 127;
-                        const unsigned hi = __builtin_bit_cast(unsigned, (float)(sx[t] - low)), lo = __builtin_bit_cast(unsigned, (float)low);
-                        ap[i][t][0] = __builtin_amdgcn_perm(hi, hi, 0x07060706u); // (hi, hi) as two bf16: the upper halves, exact
-                        ap[i][t][1] = __builtin_amdgcn_perm(lo, lo, 0x07060706u);
-                    }
-                }
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    float ws[8], wz[8];
-                    const size_t row = (size_t)min(n0 + wn * 32 * TN + j * 32 + r, N - 1) * groups;
-                    load_groups8(a.w_scale + row, gb, groups, whole, ws);
-                    load_groups8(a.w_zero + row, gb, groups, whole, wz);
-#pragma unroll
-                    for (int t = 0; t < 8; ++t) {
-                        const float c = -(ws[t] * wz[t]);
-                        v2bf p;
-                        p[0] = (__bf16)c;
-                        p[1] = (__bf16)(c - (float)p[0]);
-                        bp[j][t] = __builtin_bit_cast(unsigned, p);
-                    }
-                }
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-#pragma unroll
-                    for (int i = 0; i < TM; ++i)
-#pragma unroll
-                        for (int j = 0; j < TN; ++j) {
-                            // K slots of a group: (hi, hi, lo, lo) against (c1, c2, c1, c2)
-                            const v4u av = {ap[i][2 * q][0], ap[i][2 * q][1], ap[i][2 * q + 1][0], ap[i][2 * q + 1][1]};
-                            const v4u bv = {bp[j][2 * q], bp[j][2 * q], bp[j][2 * q + 1], bp[j][2 * q + 1]};
-                            facc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, av),
-                                                                                 __builtin_bit_cast(v8bf, bv), facc[i][j], 0, 0, 0);
-                        }
-            }
+            // half of the lane's sixteen groups at a time
+            const int gb = g0 + 16 * g;
+            int sx0[TM][8], sx1[TM][8];
+            float ws0[TN][8], wz0[TN][8], ws1[TN][8], wz1[TN][8];
+            zero_point_loads<TM, TN>(a, arow, brow, gb, groups, whole, sx0, ws0, wz0);
+            if constexpr (LOADS_FIRST)
+                zero_point_loads<TM, TN>(a, arow, brow, gb + 8, groups, whole, sx1, ws1, wz1);
+            zero_point_product<TM, TN>(sx0, ws0, wz0, facc);
+            if constexpr (!LOADS_FIRST)
+                zero_point_loads<TM, TN>(a, arow, brow, gb + 8, groups, whole, sx1, ws1, wz1);
+            zero_point_product<TM, TN>(sx1, ws1, wz1, facc);
         }
     }
     if (a.x_zero) {
