@@ -3,7 +3,7 @@
 // :21-160).
 //
 //     test_any_mma M N K X_BITS W_BITS SIGNED [--repeat R] [--warmup W] [--rotate-mib MiB]
-//                  [--stream] [--only SUBSTR] [--seed S] [--read-floor]
+//                  [--stream] [--only SUBSTR] [--seed S] [--read-floor] [--zero-operands]
 //
 // Like the reference it builds random operands, packs them on the GPU, computes the expected
 // result on the CPU, then runs EVERY tile configuration of the bit combination, checks each
@@ -30,7 +30,9 @@
 //  * --read-floor adds two lines timed the same way (same rotation, same graph replay): a kernel
 //    that does nothing, and one that reads the packed weights once with 16-byte loads and computes
 //    nothing: the floor of one launch over that many bytes;
-//  * inputs come from std::mt19937_64 with a fixed seed instead of unseeded rand().
+//  * inputs come from std::mt19937_64 with a fixed seed instead of unseeded rand(); --zero-operands makes every
+//    code zero instead: the same instructions on operands that toggle no bits, i.e. what the kernels' time owes
+//    to the clock the chip sustains on real data.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -327,14 +329,14 @@ int sweep_group_scales(int M, int N, int K, int x_bits, int w_bits, bool is_sign
 int main(int argc, char **argv)
 {
     if (argc < 7) {
-        std::printf("Usage: ./test_any_mma M N K X_BITS W_BITS SIGNED [--repeat R] [--warmup W] [--rotate-mib MiB] [--stream] [--only SUBSTR] [--seed S] [--read-floor] [--mfma-ceiling] [--group 64|128 [--fp6]]\n");
+        std::printf("Usage: ./test_any_mma M N K X_BITS W_BITS SIGNED [--repeat R] [--warmup W] [--rotate-mib MiB] [--stream] [--only SUBSTR] [--seed S] [--read-floor] [--zero-operands] [--mfma-ceiling] [--group 64|128 [--fp6]]\n");
         return -1;
     }
     const int M = std::atoi(argv[1]), N = std::atoi(argv[2]), K = std::atoi(argv[3]);
     const int x_bits = std::atoi(argv[4]), w_bits = std::atoi(argv[5]);
     const bool is_signed = std::atoi(argv[6]) == 1;
     int repeat = 1000, warmup = 10, rotate_mib = 512;
-    bool use_graph = true, read_floor = false, group_fp6 = false, mfma_ceiling = false;
+    bool use_graph = true, read_floor = false, group_fp6 = false, mfma_ceiling = false, zero_operands = false;
     int group = 0; // --group: sweep the tiles of the kernels with group scales and zero points (fp16 out) instead
     unsigned long seed = 0;
     std::string only;
@@ -345,6 +347,8 @@ int main(int argc, char **argv)
             read_floor = true;
         else if (!std::strcmp(argv[i], "--fp6"))
             group_fp6 = true;
+        else if (!std::strcmp(argv[i], "--zero-operands"))
+            zero_operands = true;
         else if (!std::strcmp(argv[i], "--mfma-ceiling"))
             mfma_ceiling = true;
         else if (i + 1 < argc && !std::strcmp(argv[i], "--group"))
@@ -376,7 +380,7 @@ int main(int argc, char **argv)
         const int lo = is_signed ? -(1 << (bits - 1)) : 0;
         const int span = 1 << bits;
         for (auto &e : v)
-            e = lo + (int)(rng() % (unsigned long)span);
+            e = zero_operands ? 0 : lo + (int)(rng() % (unsigned long)span);
     };
     std::vector<int> h_x((size_t)M * K), h_w((size_t)N * K);
     fill(h_x, x_bits);

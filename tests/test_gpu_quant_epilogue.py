@@ -382,6 +382,40 @@ def test_group_scale_staged_kernel_every_tile(abq, oracle, q, p, signed):
             torch.cuda.synchronize()
             assert_close_rel(got.cpu().numpy(), want)
 
+@pytest.mark.parametrize("M,K", [(200, 4096), (130, 4608), (64, 8192)])
+@pytest.mark.parametrize("q,p,fp6", [(8, 2, False), (4, 4, False), (4, 4, True)])
+def test_zero_points_over_whole_chunks_of_groups(abq, oracle, M, K, q, p, fp6):
+    """The weight zero points on the prefill kernels when the groups of a row come in whole chunks of 32 that start
+    on 16-byte boundaries (32, 36 = 32 + 4 and 64 groups; token counts that are and are not multiples of 4):
+    the 16-byte loads of the group sums, scales and zero points, and the row scales as 16-byte loads."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(M + K + q)
+    N, G = 264, K // 128
+    lo_x, hi_x, lo_w, hi_w = -(1 << (q - 1)), 1 << (q - 1), -(1 << (p - 1)), 1 << (p - 1)
+    x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32) + (rng.integers(0, hi_x // 2, (M, 1)) if q == 8 else 0)
+    x = np.clip(x, lo_x, hi_x - 1).astype(np.int32)  # rows with a mean: group sums of several thousand
+    w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+    xs = rng.uniform(0.01, 0.05, M)
+    xz = rng.integers(lo_x // 2, hi_x // 2 + 1, M).astype(np.float64)
+    wsc = rng.uniform(0.001, 0.02, (N, G))
+    wz = rng.integers(lo_w, hi_w, (N, G)).astype(np.float64) + rng.uniform(-0.5, 0.5, (N, G))  # not whole numbers
+    want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, 128)
+    wp, xp = planes_dev(oracle.pack_i32(w, p)), planes_dev(oracle.pack_i32(x, q))
+    kw = dict(x_scale=fdev(xs), w_scale=fdev(wsc), group_size=128, w_zero=fdev(wz), x_zero=fdev(xz),
+              x_group_sums=torch.from_numpy(x.reshape(M, G, 128).sum(axis=2).astype(np.int32)).cuda())
+    kw["w_zero_term"] = abq.weight_zero_term(wp, True, kw["w_scale"], kw["w_zero"], 128)
+    if fp6:
+        g = abq.Gemm(abq.relayout_planes_fp6(xp, True), abq.relayout_planes_fp6(wp, True), True, out_kind=abq.OUT_F16_SCALED,
+                     x_fp6=q, w_fp6=p, **kw)
+    else:
+        g = abq.Gemm(abq.relayout_planes(xp), abq.relayout_planes(wp), True, out_kind=abq.OUT_F16_SCALED, x_tiled=True,
+                     w_tiled=True, **kw)
+    got = g.run()
+    torch.cuda.synchronize()
+    assert g.strategy in ("tiled", "fp6"), g.strategy
+    assert_close_rel(got.cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("q,p,signed", [(4, 4, True), (4, 4, False), (5, 5, True), (4, 2, True), (3, 3, False)])
 def test_group_scales_on_the_fp6_route(abq, oracle, q, p, signed):
     """Groups of 128 with zero points on both sides through the FP6 matrix-core kernel: the library's own
