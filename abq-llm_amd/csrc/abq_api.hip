@@ -869,6 +869,34 @@ static abq_status switch_to_decode(abq_gemm_state *st)
     return ABQ_ERR_UNSUPPORTED;
 }
 
+// Between 17 and 128 rows on prepared operands the decode kernel, run over blocks of 16 rows that each stream the
+// weights again (from L2 after the first), is weighed against the 64 x 64 tile of the prefill kernel, whose time
+// does not depend on M there but is a whole K loop of 0.23 us per K tile on a quarter of the compute units.  Both
+// estimates are fits to a sweep of W2A8, W4A8, W8A8, W4A4 and W2A2 over M = 24 ... 128 and the LLaMA-7B widths on
+// MI355X (microseconds; MB = 10^6 bytes of weights plus of the activations all workgroups of a block stage); the
+// decode kernel is taken when it is estimated at least 10 % ahead, which on the sweep never picks the slower kernel
+// by more than 5 % and gains up to 2.7 x (W4A4 64 x 4096 x 4096: 5.7 against 9.5 us).
+constexpr int kDecodeTiledBlocksWaves = 8, kDecodeTiledBlocksTiles = 2;
+static bool decode_tiled_pays(const abq_gemm_state *st)
+{
+    if (st->M <= 16)
+        return true;
+    if (st->M > 128)
+        return false;
+    const abq_tile_config &c = st->cfg;
+    const int mrows = decode_tiled_rows(kDecodeTiledBlocksWaves, kDecodeTiledBlocksTiles, st->M, st->K, c.x_bits);
+    if (mrows == 0)
+        return false;
+    const double blocks = (st->M + mrows - 1) / mrows;
+    const double w_mb = (double)st->N * st->K * c.w_bits / 8e6;
+    const double x_mb = (double)((st->N + 16 * kDecodeTiledBlocksTiles - 1) / (16 * kDecodeTiledBlocksTiles)) * mrows * st->K * c.x_bits / 8e6;
+    const double per_block = c.x_bits == 8 ? 0.11 * (w_mb + x_mb) + 0.5 : 0.07 * (w_mb + x_mb) + 0.9;
+    const double decode_us = 0.8 + blocks * per_block;
+    const long tiles64 = (long)((st->M + 63) / 64) * ((st->N + 63) / 64);
+    const double tiled_us = (2.3 + 0.23 * (st->K / 128)) * (tiles64 > 256 ? 1.35 : 1.0);
+    return decode_us < 0.9 * tiled_us;
+}
+
 // Decode-sized GEMM with both operands K-tiled: the decode kernel built for that layout, if it exists for the
 // pair.  Variant by shape (measured on MI355X, W2A8, LLaMA-7B widths): sixteen waves with one weight load each
 // in flight while a compute unit holds at most two workgroups; with more tiles than that, eight waves with two
@@ -882,12 +910,16 @@ static abq_status switch_to_decode_tiled(abq_gemm_state *st)
     const int tiles = (st->N + 15) / 16;
     const int steps = (st->K / 128 * c.w_bits + 3) / 4;
     // long K with one or two rows: three loads per wave in flight instead of three rounds of one (4.4 against 4.8 us
-    // at K = 11008); with more rows the activation traffic comes first and one load at a time is as fast
-    const int want_wk = tiles > 512 ? 8 : 16, want_d = tiles > 512 ? 2 : (steps > 32 && st->M <= 2) ? 3 : 1;
+    // at K = 11008); with more rows the activation traffic comes first and one load at a time is as fast.  Several
+    // blocks of 16 rows (M > 16): eight waves on two tiles, so that a workgroup's activations serve twice the weights.
+    const bool row_blocks = st->M > 16;
+    const int want_t = row_blocks ? kDecodeTiledBlocksTiles : 1;
+    const int want_wk = row_blocks ? kDecodeTiledBlocksWaves : tiles > 512 ? 8 : 16;
+    const int want_d = row_blocks ? 1 : tiles > 512 ? 2 : (steps > 32 && st->M <= 2) ? 3 : 1;
     int pick = -1;
     for (int i = 0; i < tdt->count; ++i) {
         const KernelEntry &e = tdt->entries[i];
-        if (e.tn == 1 && e.wk == want_wk && e.kb == (512 / c.w_bits) * want_d)
+        if (e.tn == want_t && e.wk == want_wk && e.kb == (512 / c.w_bits) * want_d)
             pick = i;
     }
     if (pick < 0)
@@ -1325,8 +1357,9 @@ abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_l
         if (rc != ABQ_OK)
             return rc;
     }
-    // decode-sized M with both operands prepared: the decode kernel of that layout (plain and per-channel epilogues)
-    if (x_layout == ABQ_LAYOUT_TILED && w_layout == ABQ_LAYOUT_TILED && st->auto_chosen && st->M <= 16 && !st->group_size &&
+    // decode-sized M (and up to 128 rows where it pays) with both operands prepared: the decode kernel of that layout
+    // (plain and per-channel epilogues)
+    if (x_layout == ABQ_LAYOUT_TILED && w_layout == ABQ_LAYOUT_TILED && st->auto_chosen && decode_tiled_pays(st) && !st->group_size &&
         !st->act && st->strategy != ABQ_STRATEGY_DECODE_TILED && switch_to_decode_tiled(st) == ABQ_OK) {
         st->x_layout = x_layout;
         st->w_layout = w_layout;

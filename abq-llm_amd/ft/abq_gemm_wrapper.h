@@ -56,7 +56,8 @@ public:
     // of prepared_weight_bytes(N, K, W_BITS) that may be freed or reused once `stream` has passed this call, and
     // enters B into a process-wide table.  Every later gemm() of any wrapper whose B is this pointer packs its
     // activations into the same layout and runs the LDS-staged prefill kernel (M > 16) or the decode kernel on
-    // prepared operands (M <= 16) with no conversion inside the call; a B that was never prepared keeps the plane
+    // prepared operands (M <= 16, and small batches above that where the library estimates it ahead) with no
+    // conversion inside the call; a B that was never prepared keeps the plane
     // kernels.  B must not be handed to gemm_scaled() or to ABQGroupedWeight::planes afterwards.  Returns false
     // (after "[ABQ][Error] ...") on a bad argument or a failed launch.  release_weight() takes B out of the table
     // (before its memory is freed or refilled).  The table is guarded by a mutex.

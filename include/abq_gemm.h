@@ -111,8 +111,11 @@ typedef enum abq_strategy {
                                  K-tiled layout (widths 2, 4 or 8 bits; no unsigned 8-bit operand):
                                  nothing is expanded or transposed inside the kernel; tile tuples with
                                  NSTAGE = 6.  A state with M <= 16 whose operands are both declared
-                                 ABQ_LAYOUT_TILED moves here by itself; with group scales of 128 it runs
-                                 this strategy's group-scale variant (zero points, fused SiLU gate) */
+                                 ABQ_LAYOUT_TILED moves here by itself, and so does one of up to 128 rows
+                                 where the library estimates this kernel, run over blocks of 16 rows, ahead
+                                 of the prefill kernel's smallest tile (narrow pairs, few blocks); with
+                                 group scales of 128 and M <= 16 it runs this strategy's group-scale variant
+                                 (zero points, fused SiLU gate) */
 } abq_strategy;
 
 /* Parses "AqBMMA_8x2xtrue_1x48x512_8x24x128_8x8x128_4" (an optional _InitFn/_ExecFn suffix is
@@ -307,8 +310,9 @@ abq_status abq_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int ro
                                    int is_signed, void *stream);
 
 /* Declares the layout of X and W of an initialised state.  A tiled (FP6) operand moves a state
- * whose tile was the library's choice to ABQ_STRATEGY_TILED (ABQ_STRATEGY_FP6), or, with M <= 16 and both operands
- * tiled, to ABQ_STRATEGY_DECODE_TILED where that kernel exists for the pair and epilogue; a state
+ * whose tile was the library's choice to ABQ_STRATEGY_TILED (ABQ_STRATEGY_FP6), or, with both operands tiled and
+ * M <= 16 (or M <= 128 where the decode kernel over blocks of 16 rows is estimated ahead), to
+ * ABQ_STRATEGY_DECODE_TILED where that kernel exists for the pair and epilogue; a state
  * initialised with an explicit tile tuple of another strategy is refused (ABQ_ERR_UNSUPPORTED),
  * and so are a tiled and an FP6 operand together, an FP6 operand with group scales of groups other
  * than 128, and an FP6 operand of a bit pair or K that does not qualify. */

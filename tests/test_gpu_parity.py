@@ -486,7 +486,9 @@ def test_decode_on_prepared_operands(abq, oracle, q, p, signed):
         xt, wt = abq.relayout_planes(xd), abq.relayout_planes(wd)
         want = oracle.np_gemm(x, w)
         g = abq.Gemm(xt, wt, signed, x_tiled=True, w_tiled=True)
-        assert g.strategy == ("decode_tiled" if built and M <= 16 else "tiled"), (g.strategy, M, N, K)
+        # up to 16 rows always; up to 128 rows where the library estimates the decode kernel ahead (several blocks of rows)
+        assert g.strategy == "decode_tiled" if built and M <= 16 else g.strategy in ("decode_tiled", "tiled"), (g.strategy, M, N, K)
+        assert built or g.strategy == "tiled"
         assert g.workspace_bytes == 0
         assert np.array_equal(g.run().cpu().numpy(), want), (g.config_name, M, N, K)
         for cfg in abq.native_configs(q, p, signed):
@@ -496,6 +498,33 @@ def test_decode_on_prepared_operands(abq, oracle, q, p, signed):
             got = abq.Gemm(xt, wt, signed, cfg=cfg, out=out, x_tiled=True, w_tiled=True).run().cpu().numpy()
             assert np.array_equal(got, want), (abq.format_kernel_name(cfg), M, N, K)
     assert built == any(c.nstage == 6 for c in abq.native_configs(q, p, signed))
+
+
+def test_decode_kernel_over_row_blocks_is_the_default_where_it_pays(abq, oracle):
+    """Between 17 and 128 rows on prepared operands the library weighs the decode kernel over blocks of 16 rows
+    against the prefill kernel's 64 x 64 tile: the choices its fit makes on the LLaMA-7B width, the result either
+    way, and the per-token x per-channel epilogue over several row blocks."""
+    rng = np.random.default_rng(640)
+    N = K = 4096
+    for q, p, M, want in [(4, 4, 64, "decode_tiled"), (8, 2, 32, "decode_tiled"), (8, 2, 128, "tiled"), (8, 8, 64, "tiled"),
+                          (4, 4, 200, "tiled"), (2, 2, 48, "decode_tiled")]:
+        x, w = rand_vals(rng, M, K, q, True), rand_vals(rng, N, K, p, True)
+        xt = abq.relayout_planes(planes_dev(oracle.pack_i32(x, q)))
+        wt = abq.relayout_planes(planes_dev(oracle.pack_i32(w, p)))
+        g = abq.Gemm(xt, wt, True, x_tiled=True, w_tiled=True)
+        assert g.strategy == want, (q, p, M, g.strategy, g.config_name)
+        assert np.array_equal(g.run().cpu().numpy(), oracle.np_gemm(x, w)), (q, p, M)
+    M, N, K = 40, 200, 1152
+    x, w = rand_vals(rng, M, K, 8, True), rand_vals(rng, N, K, 2, True)
+    xt = abq.relayout_planes(planes_dev(oracle.pack_i32(x, 8)))
+    wt = abq.relayout_planes(planes_dev(oracle.pack_i32(w, 2)))
+    xs = (rng.random(M) * 0.05 + 0.01).astype(np.float32)
+    ws = (rng.random(N) * 0.01 + 0.001).astype(np.float32)
+    g = abq.Gemm(xt, wt, True, out_kind=abq.OUT_F16_SCALED, x_scale=dev(xs), w_scale=dev(ws), x_tiled=True, w_tiled=True)
+    assert g.strategy == "decode_tiled" and g.state.grid_dim.y == 3
+    got = g.run().cpu().numpy().astype(np.float64)
+    want = oracle.np_gemm(x, w).astype(np.float64) * xs[:, None].astype(np.float64) * ws[None, :].astype(np.float64)
+    assert np.all(np.abs(got - want) <= 1e-2 * np.abs(want) + 1e-6)  # 1e-2 relative (fp16 rounding is 2^-11)
 
 
 def test_decode_on_prepared_operands_epilogues(abq, oracle):
