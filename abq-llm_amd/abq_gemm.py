@@ -33,7 +33,7 @@ EXPORTED = [
     "abq_native_config_count", "abq_native_config_get",
     "abq_gemm_init", "abq_gemm_set_scales", "abq_gemm_exec", "abq_gemm_launch",
     "abq_planes_bytes", "abq_relayout_planes", "abq_gemm_set_operand_layout", "abq_gemm_workspace_bytes",
-    "abq_gemm_set_workspace", "abq_fp6_bytes", "abq_fp6_eligible", "abq_relayout_planes_fp6",
+    "abq_gemm_set_workspace", "abq_fp6_bytes", "abq_fp6_eligible", "abq_prepared_decode_pays", "abq_relayout_planes_fp6",
     "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16", "abq_gemm_set_activation",
     "abq_probe_launch", "abq_gemm_exec_static", "abq_gemm_set_f16_activations",
 ]
@@ -122,6 +122,8 @@ def lib():
         L.abq_fp6_bytes.argtypes = [ci, ci]
         L.abq_fp6_bytes.restype = ctypes.c_size_t
         L.abq_fp6_eligible.argtypes = [ci, ci, ci, ci]
+        L.abq_prepared_decode_pays.argtypes = [ci] * 8
+        L.abq_prepared_decode_pays.restype = ci
         L.abq_gemm_set_operand_layout.argtypes = [ctypes.POINTER(GemmState), ci, ci]
         L.abq_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GemmState)]
         L.abq_gemm_workspace_bytes.restype = ctypes.c_size_t
@@ -227,6 +229,11 @@ def relayout_planes(planes, out=None, stream=None):
 def fp6_eligible(x_bits, w_bits, signed, k):
     """Whether the FP6 matrix-core route is exact for this bit pair and K (host-side check)."""
     return bool(lib().abq_fp6_eligible(x_bits, w_bits, int(bool(signed)), k))
+
+
+def prepared_decode_pays(x_bits, w_bits, signed, m, n, k, group_size=0, act=ACT_NONE):
+    """Whether a GEMM of this shape on operands that are both K-tiled runs the decode kernel of that layout."""
+    return bool(lib().abq_prepared_decode_pays(x_bits, w_bits, int(bool(signed)), m, n, k, group_size, act))
 
 
 def relayout_planes_fp6(planes, signed, out=None, stream=None):

@@ -877,23 +877,22 @@ static abq_status switch_to_decode(abq_gemm_state *st)
 // decode kernel is taken when it is estimated at least 10 % ahead, which on the sweep never picks the slower kernel
 // by more than 5 % and gains up to 2.7 x (W4A4 64 x 4096 x 4096: 5.7 against 9.5 us).
 constexpr int kDecodeTiledBlocksWaves = 8, kDecodeTiledBlocksTiles = 2;
-static bool decode_tiled_pays(const abq_gemm_state *st)
+static bool decode_tiled_pays(int x_bits, int w_bits, int M, int N, int K)
 {
-    if (st->M <= 16)
+    if (M <= 16)
         return true;
-    if (st->M > 128)
+    if (M > 128)
         return false;
-    const abq_tile_config &c = st->cfg;
-    const int mrows = decode_tiled_rows(kDecodeTiledBlocksWaves, kDecodeTiledBlocksTiles, st->M, st->K, c.x_bits);
+    const int mrows = decode_tiled_rows(kDecodeTiledBlocksWaves, kDecodeTiledBlocksTiles, M, K, x_bits);
     if (mrows == 0)
         return false;
-    const double blocks = (st->M + mrows - 1) / mrows;
-    const double w_mb = (double)st->N * st->K * c.w_bits / 8e6;
-    const double x_mb = (double)((st->N + 16 * kDecodeTiledBlocksTiles - 1) / (16 * kDecodeTiledBlocksTiles)) * mrows * st->K * c.x_bits / 8e6;
-    const double per_block = c.x_bits == 8 ? 0.11 * (w_mb + x_mb) + 0.5 : 0.07 * (w_mb + x_mb) + 0.9;
+    const double blocks = (M + mrows - 1) / mrows;
+    const double w_mb = (double)N * K * w_bits / 8e6;
+    const double x_mb = (double)((N + 16 * kDecodeTiledBlocksTiles - 1) / (16 * kDecodeTiledBlocksTiles)) * mrows * K * x_bits / 8e6;
+    const double per_block = x_bits == 8 ? 0.11 * (w_mb + x_mb) + 0.5 : 0.07 * (w_mb + x_mb) + 0.9;
     const double decode_us = 0.8 + blocks * per_block;
-    const long tiles64 = (long)((st->M + 63) / 64) * ((st->N + 63) / 64);
-    const double tiled_us = (2.3 + 0.23 * (st->K / 128)) * (tiles64 > 256 ? 1.35 : 1.0);
+    const long tiles64 = (long)((M + 63) / 64) * ((N + 63) / 64);
+    const double tiled_us = (2.3 + 0.23 * (K / 128)) * (tiles64 > 256 ? 1.35 : 1.0);
     return decode_us < 0.9 * tiled_us;
 }
 
@@ -936,12 +935,39 @@ static abq_status switch_to_decode_tiled(abq_gemm_state *st)
 
 // Group scales on a decode-sized GEMM whose operands are (or are about to be declared) both prepared: whether the
 // decode kernel of that layout has a group-scale variant for the pair that fits this shape.
+// The same weighing for the group-scale variant (one tile per workgroup, two with the SiLU gate), against the
+// group-scale prefill kernel, whose smallest grids (64 x 64 or 128 x 64 tiles) take 0.6 us per K tile whatever M is
+// and 1.45 times that once they exceed one workgroup per compute unit.  Fits to a sweep of W2A8, W4A8 and W4A4 with
+// zero points over M = 24 ... 128 on the LLaMA-7B linears (4096 x 4096, QKV, gate + up with the gate fused, down);
+// taken when estimated 15 % ahead: W2A8 32 x 4096 x 4096 8.3 against 20.1 us, 32 x 4096 x 11008 23.2 against 48.8,
+// W4A4 32 x 12288 x 4096 13.2 against 20.6; the wide outputs of the 8-bit activations stay on the prefill kernel.
+static bool decode_tiled_grouped_pays(int x_bits, int w_bits, int M, int N, int K, int act)
+{
+    if (M <= 16)
+        return true;
+    if (M > 128)
+        return false;
+    const int t = act ? 2 : 1;
+    const int mrows = decode_tiled_grouped_rows(16, t, M, K, x_bits);
+    if (mrows == 0)
+        return false;
+    const double blocks = (M + mrows - 1) / mrows;
+    const double w_mb = (double)N * K * w_bits / 8e6;
+    const double x_mb = (double)((N + 16 * t - 1) / (16 * t)) * mrows * K * x_bits / 8e6;
+    const double per_block = x_bits == 8 ? 0.165 * (w_mb + x_mb) : 0.11 * (w_mb + x_mb) + 0.7;
+    const double decode_us = 1.0 + blocks * per_block;
+    const long wgs = (long)((N + 63) / 64) * ((M + 127) / 128);
+    const double tiled_us = 1.0 + 0.6 * (K / 128) * (wgs > 256 ? 1.45 : 1.0);
+    return decode_us < 0.85 * tiled_us;
+}
+
 static bool decode_tiled_grouped_fits(const abq_gemm_state *st, int group_size, int act)
 {
     const abq_tile_config &c = st->cfg;
     const KernelTable *t = find_table(registry().decode_tiled_grouped, c.x_bits, c.w_bits, c.is_signed);
-    return t && t->count > 0 && st->auto_chosen && st->M <= 16 && group_size == 128 && (!act || st->N % 32 == 0) &&
-           decode_tiled_grouped_rows(16, act ? 2 : 1, st->M, st->K, c.x_bits) != 0;
+    return t && t->count > 0 && st->auto_chosen && group_size == 128 && (!act || st->N % 32 == 0) &&
+           decode_tiled_grouped_rows(16, act ? 2 : 1, st->M, st->K, c.x_bits) != 0 &&
+           decode_tiled_grouped_pays(c.x_bits, c.w_bits, st->M, st->N, st->K, act);
 }
 
 // Moves a state with group scales onto the tiled kernel's group-scale variants.
@@ -1022,7 +1048,13 @@ abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, cons
         if (state->strategy == ABQ_STRATEGY_BCNT && state->auto_chosen && state->M <= 16)
             switch_to_decode(state); // the popcount kernel has no group-scale epilogue
         // both operands prepared: the decode kernel of that layout has its own group-scale variant
-        const bool decode_tiled_ok = state->strategy == ABQ_STRATEGY_DECODE_TILED && decode_tiled_grouped_fits(state, group_size, state->act);
+        // (a state of 17 to 128 rows may sit on the prefill kernel because the plain decode kernel did not pay there)
+        const bool both_tiled = state->x_layout == ABQ_LAYOUT_TILED && state->w_layout == ABQ_LAYOUT_TILED;
+        bool decode_tiled_ok = (state->strategy == ABQ_STRATEGY_DECODE_TILED ||
+                                (state->strategy == ABQ_STRATEGY_TILED && both_tiled && state->auto_chosen)) &&
+                               decode_tiled_grouped_fits(state, group_size, state->act);
+        if (decode_tiled_ok && state->strategy != ABQ_STRATEGY_DECODE_TILED)
+            decode_tiled_ok = switch_to_decode_tiled(state) == ABQ_OK;
         const bool decode_ok = state->strategy == ABQ_STRATEGY_DECODE && state->auto_chosen && state->M <= 16 &&
                                state->x_layout == ABQ_LAYOUT_PLANES && state->w_layout == ABQ_LAYOUT_PLANES &&
                                decode_grouped_lds(state->M, state->K, group_size) != 0 &&
@@ -1308,6 +1340,23 @@ size_t abq_fp6_bytes(int rows, int k)
 
 int abq_fp6_eligible(int x_bits, int w_bits, int is_signed, int k) { return fp6_eligible(x_bits, w_bits, is_signed, k) ? 1 : 0; }
 
+int abq_prepared_decode_pays(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size, int act)
+{
+    if (M <= 0 || N <= 0 || K < 128 || K % 128 != 0)
+        return 0;
+    const Registry &reg = registry();
+    if (group_size) {
+        const KernelTable *t = find_table(reg.decode_tiled_grouped, x_bits, w_bits, is_signed);
+        return t && t->count > 0 && group_size == 128 && (!act || N % 32 == 0) &&
+                       decode_tiled_grouped_rows(16, act ? 2 : 1, M, K, x_bits) != 0 &&
+                       decode_tiled_grouped_pays(x_bits, w_bits, M, N, K, act)
+                   ? 1
+                   : 0;
+    }
+    const KernelTable *t = find_table(reg.decode_tiled, x_bits, w_bits, is_signed);
+    return t && t->count > 0 && !act && decode_tiled_pays(x_bits, w_bits, M, N, K) ? 1 : 0;
+}
+
 abq_status abq_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int rows, int k, int bits, int is_signed,
                                    void *stream)
 {
@@ -1359,7 +1408,8 @@ abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_l
     }
     // decode-sized M (and up to 128 rows where it pays) with both operands prepared: the decode kernel of that layout
     // (plain and per-channel epilogues)
-    if (x_layout == ABQ_LAYOUT_TILED && w_layout == ABQ_LAYOUT_TILED && st->auto_chosen && decode_tiled_pays(st) && !st->group_size &&
+    if (x_layout == ABQ_LAYOUT_TILED && w_layout == ABQ_LAYOUT_TILED && st->auto_chosen &&
+        decode_tiled_pays(st->cfg.x_bits, st->cfg.w_bits, st->M, st->N, st->K) && !st->group_size &&
         !st->act && st->strategy != ABQ_STRATEGY_DECODE_TILED && switch_to_decode_tiled(st) == ABQ_OK) {
         st->x_layout = x_layout;
         st->w_layout = w_layout;

@@ -208,16 +208,16 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     float *x_scale = reinterpret_cast<float *>(abq_gemm_workspace + planes_bytes);
     float *x_zero = x_scale + M;
     int32_t *sums = reinterpret_cast<int32_t *>(x_zero + M);
-    // at most 16 rows: the decode kernel on prepared operands where it is built for the pair (widths of 2, 4 or 8
-    // bits, groups of 128; the library moves the state there once both layouts are declared), else the decode
-    // kernel on plane operands if the caller kept the planes; above 16 rows the tiled kernel on the prefill layout
-    auto single_field = [](int b) { return b == 2 || b == 4 || b == 8; };
-    const bool decode_prepared = M <= 16 && W.planes_tiled != nullptr && W.group_size == 128 && single_field(x_bits_) &&
-                                 single_field(w_bits_) && x_bits_ >= w_bits_;
+    // at most 16 rows (and small batches above that where the library estimates it ahead): the decode kernel on
+    // prepared operands where it is built for the pair (widths of 2, 4 or 8 bits, groups of 128; the library moves
+    // the state there once both layouts are declared), else the decode kernel on plane operands if the caller kept
+    // the planes; otherwise the tiled kernel on the prefill layout
+    const bool decode_prepared = W.planes_tiled != nullptr &&
+                                 abq_prepared_decode_pays(x_bits_, w_bits_, 1, M, N, K, W.group_size, silu_gate ? 1 : 0) != 0;
     // (if the expanded activations fit the decode kernel's LDS: partial tiles, group sums, M padded rows)
     const bool decode = !decode_prepared && M <= 16 && W.planes != nullptr &&
                         (silu_gate ? 32 : 16) * 1024 + (size_t)64 * (K / W.group_size) + 128 + (size_t)M * ((K + 511) / 512 * 512 + 16) <= 160 * 1024;
-    const bool fp6 = !decode && W.records_fp6 != nullptr && W.group_size == 128 && abq_fp6_eligible(x_bits_, w_bits_, 1, K);
+    const bool fp6 = !decode && !decode_prepared && W.records_fp6 != nullptr && W.group_size == 128 && abq_fp6_eligible(x_bits_, w_bits_, 1, K);
     const int layout = decode ? ABQ_LAYOUT_PLANES : fp6 ? ABQ_LAYOUT_FP6 : ABQ_LAYOUT_TILED;
     abq_status rc = abq_quant_pack_f16(A, M, K, x_bits_, x_symmetric ? 1 : 0, layout, planes, x_scale, x_zero,
                                        sums, W.group_size, stream);

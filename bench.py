@@ -82,7 +82,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the side measurements")
     ap.add_argument("--extras", default=None,
                     help="comma-separated side measurements to run (default all): decode_plane_operands, prefill, prefill_fp6, library_int8_gemm, "
-                         "decode_fused_linears, decode_group_scales, decoder_layer_w2a8_group128")
+                         "decode_fused_linears, decode_group_scales, small_batch, decoder_layer_w2a8_group128")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (the known-size kernel that "
                          "calibrates FETCH_SIZE / WRITE_SIZE in a counter run)")
@@ -490,6 +490,33 @@ def main():
                     % (M, N, K, us, gbs, 100 * gbs / HBM_PEAK_GBS, gs[0].strategy, us_planes))
                 del gs, out
         extra["decode_group_scales"] = deq
+
+    if want("small_batch"):
+        # ------------------------------------------------------------ side measurement: 32 and 64 rows on prepared operands
+        # Between 17 and 128 rows the library weighs the decode kernel over blocks of 16 rows against the prefill
+        # kernel's smallest tile; the kernel it picks and its time, int32 output and the group-128 dequantising epilogue.
+        small = []
+        for (N, K) in SHAPES:
+            G = K // 128
+            Wt = weights_tiled[(N, K)]
+            wsc = torch.rand((N, G), device="cuda") * 0.01 + 0.001
+            wz = torch.randint(-2, 2, (N, G), device="cuda").float()
+            for M in (32, 64):
+                xt = abq.relayout_planes(random_planes(torch, (Q_BITS, M, K // 32)))
+                gs = [abq.Gemm(xt, Wt[r], SIGNED, x_tiled=True, w_tiled=True) for r in range(Wt.shape[0])]
+                us = time_rotating(gs)
+                xsc = torch.rand(M, device="cuda") * 0.05 + 0.01
+                sums = torch.randint(-1000, 1000, (M, G), dtype=torch.int32, device="cuda")
+                out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+                gg = [abq.Gemm(xt, Wt[r], SIGNED, x_tiled=True, w_tiled=True, out=out, out_kind=abq.OUT_F16_SCALED, x_scale=xsc,
+                               w_scale=wsc, group_size=128, w_zero=wz, x_group_sums=sums) for r in range(Wt.shape[0])]
+                us_g = time_rotating(gg)
+                small.append(dict(M=M, N=N, K=K, us=round(us, 2), kernel="%s:%s" % (gs[0].strategy, gs[0].config_name),
+                                  group128=dict(us=round(us_g, 2), kernel=gg[0].strategy)))
+                log("small batch M=%d N=%d K=%d  int32 %.2f us (%s)  group scales %.2f us (%s)"
+                    % (M, N, K, us, gs[0].strategy, us_g, gg[0].strategy))
+                del gs, gg, out, xt
+        extra["small_batch"] = small
 
     if want("decoder_layer_w2a8_group128"):
         # ------------------------------------------------------------ side measurement: one decoder layer's linears

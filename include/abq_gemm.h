@@ -305,6 +305,13 @@ abq_status abq_pack_f16_tiled(const void *in_f16, const float *scale_dev, uint32
  * whatever the bit width.  abq_fp6_eligible tells whether a bit pair and K qualify. */
 size_t abq_fp6_bytes(int rows, int k);
 int abq_fp6_eligible(int x_bits, int w_bits, int is_signed, int k);
+
+/* Whether a GEMM of this shape whose operands are both K-tiled runs ABQ_STRATEGY_DECODE_TILED when the tile is the
+ * library's choice: always up to 16 rows where that kernel is built for the pair (and, with group scales, for
+ * groups of 128), and up to 128 rows where the library estimates the kernel, run over blocks of 16 rows, ahead of
+ * the prefill kernel.  For callers that hold their weights in several prepared forms and have to pick one before
+ * they quantise the activations (ABQGEMMWrapper::gemm_dynamic).  No counterpart in the reference. */
+int abq_prepared_decode_pays(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size, int act);
 /* planes [bits][rows][k/32] -> fp6 [k/128][rows][24]; bits <= 4, or <= 5 if is_signed. */
 abq_status abq_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int rows, int k, int bits,
                                    int is_signed, void *stream);

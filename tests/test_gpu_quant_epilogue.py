@@ -241,6 +241,51 @@ def test_decode_on_prepared_operands_with_group_scales(abq, oracle, q, p, signed
         assert_close_rel(got, want)
 
 
+@pytest.mark.parametrize("q,p,signed", [(8, 2, True), (4, 4, True), (8, 4, True), (4, 4, False)])
+def test_group_scale_decode_kernel_over_row_blocks(abq, oracle, q, p, signed):
+    """17 to 128 rows on prepared operands with groups of 128: where the library estimates it ahead of the prefill
+    kernel, the decode kernel's group-scale variant runs over blocks of 16 rows (8 where a block's activations would
+    not fit the LDS); zero points on both sides, ragged last block, the fused SiLU gate, either order of the calls."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(900 + 10 * q + p + signed)
+    lo_x, hi_x = (-(1 << (q - 1)), 1 << (q - 1)) if signed else (0, 1 << q)
+    lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed else (0, 1 << p)
+    for (M, N, K, act) in [(24, 192, 1152, False), (40, 330, 640, False), (33, 192, 1152, True), (17, 64, 11008, False),
+                           (32, 4096, 4096, False)]:
+        G = K // 128
+        x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        xs = rng.uniform(0.01, 0.05, M)
+        xz = rng.integers(lo_x // 2, hi_x // 2 + 1, M).astype(np.float64)
+        wsc = rng.uniform(0.001, 0.02, (N, G))
+        wz = rng.integers(lo_w, hi_w, (N, G)).astype(np.float64)
+        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, 128)
+        if act:  # rows of W come in blocks of 16 gate rows followed by their 16 up rows
+            blocks = want.reshape(M, N // 32, 2, 16)
+            gate, up = blocks[:, :, 0, :], blocks[:, :, 1, :]
+            want = (gate / (1.0 + np.exp(-gate)) * up).reshape(M, N // 2)
+        wp = planes_dev(oracle.pack_i32(w, p))
+        kw = dict(x_scale=fdev(xs), w_scale=fdev(wsc), group_size=128, w_zero=fdev(wz), x_zero=fdev(xz), x_tiled=True, w_tiled=True,
+                  x_group_sums=torch.from_numpy(x.reshape(M, G, 128).sum(axis=2).astype(np.int32)).cuda())
+        kw["w_zero_term"] = abq.weight_zero_term(wp, signed, kw["w_scale"], kw["w_zero"], 128)
+        if act:
+            kw["act"] = abq.ACT_SILU_GATE
+        xt, wt = abq.relayout_planes(planes_dev(oracle.pack_i32(x, q))), abq.relayout_planes(wp)
+        assert abq.prepared_decode_pays(q, p, signed, M, N, K, 128, abq.ACT_SILU_GATE if act else abq.ACT_NONE)
+        g = abq.Gemm(xt, wt, signed, out_kind=abq.OUT_F16_SCALED, **kw)
+        assert g.strategy == "decode_tiled", (g.strategy, M, N, K)
+        got = g.run()
+        torch.cuda.synchronize()
+        assert_close_rel(got.cpu().numpy(), want)
+    # what the estimate decides on the decoder-layer linears (W2A8: the narrow outputs only)
+    if (q, p, signed) == (8, 2, True):
+        assert abq.prepared_decode_pays(8, 2, True, 32, 4096, 4096, 128) and abq.prepared_decode_pays(8, 2, True, 32, 4096, 11008, 128)
+        assert not abq.prepared_decode_pays(8, 2, True, 32, 12288, 4096, 128)
+        assert not abq.prepared_decode_pays(8, 2, True, 96, 4096, 4096, 128)
+        assert not abq.prepared_decode_pays(8, 2, True, 200, 4096, 4096, 128)
+        assert not abq.prepared_decode_pays(8, 2, True, 32, 4096, 4096, 64)
+
+
 def test_decode_on_prepared_operands_group_scales_either_call_order(abq, oracle):
     """Layouts declared before the scales are attached (the C ABI allows both orders) lands on the same kernel."""
     import ctypes
@@ -382,7 +427,7 @@ def test_group_scale_staged_kernel_every_tile(abq, oracle, q, p, signed):
             torch.cuda.synchronize()
             assert_close_rel(got.cpu().numpy(), want)
 
-@pytest.mark.parametrize("M,K", [(200, 4096), (130, 4608), (64, 8192)])
+@pytest.mark.parametrize("M,K", [(200, 4096), (130, 4608), (136, 8192)])
 @pytest.mark.parametrize("q,p,fp6", [(8, 2, False), (4, 4, False), (4, 4, True)])
 def test_zero_points_over_whole_chunks_of_groups(abq, oracle, M, K, q, p, fp6):
     """The weight zero points on the prefill kernels when the groups of a row come in whole chunks of 32 that start
