@@ -210,7 +210,7 @@ static bool popcount_is_faster(int x_bits, int w_bits, int M)
     return w_bits >= 1 && w_bits <= 8 && x_bits * w_bits * M <= bound[w_bits];
 }
 
-static void choose_default(int M, int N, int x_bits, int w_bits, int *strategy, int *mi, int *tm, int *tn, int *wm,
+static void choose_default(int M, int N, int K, int x_bits, int w_bits, int *strategy, int *mi, int *tm, int *tn, int *wm,
                            int *wn, int *wk)
 {
     if (M <= 16 && popcount_is_faster(x_bits, w_bits, M)) {
@@ -219,6 +219,19 @@ static void choose_default(int M, int N, int x_bits, int w_bits, int *strategy, 
     } else if (M <= 16) {
         *strategy = ABQ_STRATEGY_DECODE;
         *mi = 16; *tm = 1; *tn = 1; *wm = 1; *wn = 1; *wk = 16;
+    } else if (M <= 64 || ((M <= 128 || (M <= 256 && K >= 8192)) && N < 8192)) {
+        // 17 to 128 rows: blocks of 16 rows whose waves split K (16-row MFMA tiles, two per wave), which fill the chip
+        // where the 32-row tiles below leave most of it idle (W2A8 32 x 4096 x 4096: 8.7 against 22.4 us, W4A4
+        // 64 x 4096 x 4096, the reference's own test shape: 12.9 against 32.7 us).  Up to 64 rows the workgroup is one
+        // column of four waves (eight for long K) on 32 weight rows, above that two columns of two on 64 (up to 256
+        // rows when K is long: 256 x 4096 x 11008 53.7 against 74.9 us).
+        *strategy = ABQ_STRATEGY_MFMA16;
+        *mi = 16; *tm = 1; *tn = 2; *wm = 1;
+        if (M <= 64) {
+            *wn = 1; *wk = K >= 8192 ? 8 : 4;
+        } else {
+            *wn = 2; *wk = 2;
+        }
     } else {
         *strategy = ABQ_STRATEGY_MFMA32;
         *mi = 32; *wm = 2; *wn = 2; *wk = 1;
@@ -286,7 +299,7 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
     int lpr_log2 = best_lpr_log2(K);
     int decode_step = cfg ? cfg->warp_k : 0; // K elements per decode work item
     if (strategy == ABQ_STRATEGY_AUTO) {
-        choose_default(M, N, x_bits, w_bits, &strategy, &mi, &tm, &tn, &wm, &wn, &wk);
+        choose_default(M, N, K, x_bits, w_bits, &strategy, &mi, &tm, &tn, &wm, &wn, &wk);
         decode_step = kDefaultDecodeStep;
     } else if (strategy == ABQ_STRATEGY_BCNT) {
         mi = 1; tm = cfg->block_m; tn = 1; wm = 1; wn = 8; wk = 1;
@@ -1461,7 +1474,10 @@ abq_status abq_gemm_set_workspace(abq_gemm_state *st, void *workspace, size_t by
         return ABQ_ERR_INVALID_ARG;
     st->workspace = workspace;
     st->workspace_bytes = bytes;
-    if (st->strategy != ABQ_STRATEGY_TILED && st->strategy != ABQ_STRATEGY_FP6 && st->auto_chosen && st->M > 16 &&
+    // (up to 64 rows, 32 on wide outputs, the conversion launch costs more than the LDS-staged kernel gains over the
+    // 16-row tiles on plane operands: W2A8 32 x 4096 x 4096 12.6 against 8.7 us)
+    const bool pays = st->group_size != 0 || st->M > 64 || (st->M > 32 && st->N >= 8192);
+    if (st->strategy != ABQ_STRATEGY_TILED && st->strategy != ABQ_STRATEGY_FP6 && st->auto_chosen && st->M > 16 && pays &&
         workspace && bytes >= abq_gemm_workspace_bytes(st))
         return switch_to_tiled(st);
     return ABQ_OK;

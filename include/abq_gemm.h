@@ -339,9 +339,10 @@ abq_status abq_gemm_set_f16_activations(abq_gemm_state *state, const void *x_f16
  * layout (0 if neither is). */
 size_t abq_gemm_workspace_bytes(const abq_gemm_state *state);
 
-/* Hands a caller-owned device buffer to the state.  If the tile was the library's choice, M > 16
- * and the buffer is large enough, the state moves to ABQ_STRATEGY_TILED; otherwise it keeps
- * its kernel (which needs no workspace). */
+/* Hands a caller-owned device buffer to the state.  If the tile was the library's choice, M > 64
+ * (32 for outputs of 8192 columns or more; 16 with group scales) and the buffer is large enough, the
+ * state moves to ABQ_STRATEGY_TILED; otherwise it keeps its kernel (which needs no workspace:
+ * below those sizes the conversion launch costs more than the LDS-staged kernel gains). */
 abq_status abq_gemm_set_workspace(abq_gemm_state *state, void *workspace, size_t bytes);
 
 /* Replaces AqBMMAExecFn / AqBWMMAExecFn (engine/mma_any/aq_bmma_op.h:155-161,164): one

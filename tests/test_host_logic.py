@@ -222,12 +222,21 @@ def test_init_error_paths(abq):
 
 
 def test_default_strategy_choice_and_reference_tuples(abq):
-    # W2A8 on plane operands: the popcount kernel for one row, the matrix-core decode kernel up to 16, MFMA 32x32 above
+    # W2A8 on plane operands: the popcount kernel for one row, the matrix-core decode kernel up to 16, blocks of 16 rows
+    # whose waves split K up to 128 (64 on wide outputs), MFMA 32x32 above
     for M, want in ((1, abq.STRATEGY_BCNT), (2, abq.STRATEGY_DECODE), (4, abq.STRATEGY_DECODE),
-                    (8, abq.STRATEGY_DECODE), (16, abq.STRATEGY_DECODE), (128, abq.STRATEGY_MFMA32),
-                    (2048, abq.STRATEGY_MFMA32)):
+                    (8, abq.STRATEGY_DECODE), (16, abq.STRATEGY_DECODE), (17, abq.STRATEGY_MFMA16), (64, abq.STRATEGY_MFMA16),
+                    (128, abq.STRATEGY_MFMA16), (129, abq.STRATEGY_MFMA32), (2048, abq.STRATEGY_MFMA32)):
         rc, st = _init(abq, M=M, N=4096)
         assert rc == 0 and st.strategy == want, M
+    rc, st = _init(abq, M=64, N=4096)
+    assert st.cfg.as_tuple()[3:] == (16, 32, 2048, 16, 32, 512, 16, 16, 64, 2) and st.grid_dim.y == 4
+    rc, st = _init(abq, M=64, N=4096, K=11008)
+    assert st.cfg.block_k == 4096
+    rc, st = _init(abq, M=100, N=4096)
+    assert st.cfg.as_tuple()[3:] == (16, 64, 1024, 16, 32, 512, 16, 16, 64, 2)
+    rc, st = _init(abq, M=100, N=11008)
+    assert st.strategy == abq.STRATEGY_MFMA32
     # the choice follows x_bits * w_bits * M against a bound by w_bits (popcount work against the cost of the weight transposes)
     for q, p, M, want in ((2, 2, 4, abq.STRATEGY_BCNT), (2, 2, 8, abq.STRATEGY_DECODE), (4, 4, 2, abq.STRATEGY_BCNT),
                           (4, 4, 4, abq.STRATEGY_DECODE), (8, 8, 2, abq.STRATEGY_BCNT), (8, 8, 4, abq.STRATEGY_DECODE),
