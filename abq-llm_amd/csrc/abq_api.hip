@@ -219,12 +219,15 @@ static void choose_default(int M, int N, int K, int x_bits, int w_bits, int *str
     } else if (M <= 16) {
         *strategy = ABQ_STRATEGY_DECODE;
         *mi = 16; *tm = 1; *tn = 1; *wm = 1; *wn = 1; *wk = 16;
-    } else if (M <= 64 || ((M <= 128 || (M <= 256 && K >= 8192)) && N < 8192)) {
+    } else if (M <= 64 ? (N < 8192 || w_bits <= 4 || M <= 32)
+                       : (w_bits < 8 && (M <= 128 || (M <= 256 && K >= 8192)) && N < 8192)) {
         // 17 to 128 rows: blocks of 16 rows whose waves split K (16-row MFMA tiles, two per wave), which fill the chip
         // where the 32-row tiles below leave most of it idle (W2A8 32 x 4096 x 4096: 8.7 against 22.4 us, W4A4
         // 64 x 4096 x 4096, the reference's own test shape: 12.9 against 32.7 us).  Up to 64 rows the workgroup is one
         // column of four waves (eight for long K) on 32 weight rows, above that two columns of two on 64 (up to 256
-        // rows when K is long: 256 x 4096 x 11008 53.7 against 74.9 us).
+        // rows when K is long: 256 x 4096 x 11008 53.7 against 74.9 us).  Every block of rows transposes the weight
+        // planes again, which costs by the plane: wide outputs of weights of five bits or more keep the 32-row tiles from
+        // 33 rows on, 8-bit weights from 65 (W8A8 64 x 13824 x 5120: 55 against 101 us).
         *strategy = ABQ_STRATEGY_MFMA16;
         *mi = 16; *tm = 1; *tn = 2; *wm = 1;
         if (M <= 64) {
@@ -238,7 +241,7 @@ static void choose_default(int M, int N, int K, int x_bits, int w_bits, int *str
         const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
         if (M > 64 && tiles128 >= 256) {
             *tm = 2; *tn = 2;
-        } else if (M > 32) {
+        } else if (M > 64 && w_bits < 8) {
             *tm = 1; *tn = 2;
         } else {
             *tm = 1; *tn = 1;
