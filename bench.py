@@ -516,6 +516,14 @@ def main():
                 log("small batch M=%d N=%d K=%d  int32 %.2f us (%s)  group scales %.2f us (%s)"
                     % (M, N, K, us, gs[0].strategy, us_g, gg[0].strategy))
                 del gs, gg, out, xt
+        # the reference's own test shape (BASELINE configs[0]): W4A4 unsigned, 64 x 4096 x 4096, plane operands through
+        # init + exec, nothing prepared
+        x4, w4 = random_planes(torch, (4, 64, 4096 // 32)), random_planes(torch, (4, 4096, 4096 // 32))
+        g4 = abq.Gemm(x4, w4, False)
+        us4 = time_rotating([g4])
+        small.append(dict(M=64, N=4096, K=4096, x_bits=4, w_bits=4, signed=False, operands="planes", us=round(us4, 2),
+                          tops=round(2.0 * 64 * 4096 * 4096 / (us4 * 1e-6) / 1e12, 2), kernel="%s:%s" % (g4.strategy, g4.config_name)))
+        log("reference test shape W4A4 uint 64x4096x4096 on plane operands  %.2f us (%s)" % (us4, g4.config_name))
         extra["small_batch"] = small
 
     if want("decoder_layer_w2a8_group128"):
