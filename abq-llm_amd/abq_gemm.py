@@ -33,7 +33,7 @@ EXPORTED = [
     "abq_native_config_count", "abq_native_config_get",
     "abq_gemm_init", "abq_gemm_set_scales", "abq_gemm_exec", "abq_gemm_launch",
     "abq_planes_bytes", "abq_relayout_planes", "abq_gemm_set_operand_layout", "abq_gemm_workspace_bytes",
-    "abq_gemm_set_workspace", "abq_fp6_bytes", "abq_fp6_eligible", "abq_prepared_decode_pays", "abq_relayout_planes_fp6",
+    "abq_gemm_set_workspace", "abq_fp6_bytes", "abq_fp6_eligible", "abq_prepared_decode_pays", "abq_gemm_set_dynamic_f16_activations", "abq_relayout_planes_fp6",
     "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16", "abq_gemm_set_activation",
     "abq_probe_launch", "abq_gemm_exec_static", "abq_gemm_set_f16_activations",
 ]
@@ -114,6 +114,7 @@ def lib():
         L.abq_gemm_exec.argtypes = [ctypes.POINTER(GemmState), vp]
         L.abq_gemm_exec_static.argtypes = [ctypes.POINTER(GemmState), vp]
         L.abq_gemm_set_f16_activations.argtypes = [ctypes.POINTER(GemmState), vp, vp]
+        L.abq_gemm_set_dynamic_f16_activations.argtypes = [ctypes.POINTER(GemmState), vp, ci]
         L.abq_gemm_launch.argtypes = [ctypes.POINTER(TileConfig), vp, vp, vp, vp, ci, ci, ci, ci, vp]
         L.abq_planes_bytes.argtypes = [ci, ci, ci]
         L.abq_planes_bytes.restype = ctypes.c_size_t
@@ -367,6 +368,22 @@ class Gemm:
         _check(lib().abq_gemm_set_f16_activations(ctypes.byref(self.state), x_f16.data_ptr(), scale.data_ptr()),
                "abq_gemm_set_f16_activations")
         self.x_f16, self.x_pack_scale = x_f16, scale
+
+    def set_dynamic_f16_activations(self, x_f16, symmetric, w_zero=None, w_zero_term=None):
+        """Group-scale decode on prepared weights without a quantising launch: the kernel quantises the fp16
+        activations [M, K] per token itself (symmetric, or with a zero point, which needs w_zero_term).  w_zero: the
+        weight zero points, if any (group sums are made inside the kernel).  Raises ABQ_ERR_UNSUPPORTED where that
+        kernel does not apply."""
+        import torch
+        assert x_f16.dtype == torch.float16 and x_f16.is_cuda and x_f16.is_contiguous()
+        _check(lib().abq_gemm_set_dynamic_f16_activations(ctypes.byref(self.state), x_f16.data_ptr(), int(bool(symmetric))),
+               "abq_gemm_set_dynamic_f16_activations")
+        self.x_f16 = x_f16
+        if w_zero is not None or w_zero_term is not None:
+            self.zero_operands = (None, w_zero, None, w_zero_term)
+            _check(lib().abq_gemm_set_zero_points(ctypes.byref(self.state), None, w_zero.data_ptr() if w_zero is not None else None,
+                                                  None, w_zero_term.data_ptr() if w_zero_term is not None else None),
+                   "abq_gemm_set_zero_points")
 
     def run_static(self, stream=None):
         """The same through the entry point that allocates nothing (conversions into the library's static array)."""

@@ -41,7 +41,8 @@ hipError_t launch_weight_zero_term(const uint32_t *, int, int, int, int, const f
     void abq_tiled_grouped_register_##Q##_##P(KernelTable *);  \
     void abq_decode_tiled_register_##Q##_##P(KernelTable *); \
     void abq_decode_tiled_grouped_register_##Q##_##P(KernelTable *); \
-    void abq_decode_tiled_f16_register_##Q##_##P(KernelTable *);
+    void abq_decode_tiled_f16_register_##Q##_##P(KernelTable *); \
+    void abq_decode_tiled_grouped_dyn_register_##Q##_##P(KernelTable *);
 ABQ_FOR_EACH_COMBO(ABQ_DECL)
 #undef ABQ_DECL
 
@@ -55,6 +56,7 @@ struct Registry {
     KernelTable decode_tiled[2 * ABQ_NUM_COMBOS];
     KernelTable decode_tiled_grouped[2 * ABQ_NUM_COMBOS];
     KernelTable decode_tiled_f16[2 * ABQ_NUM_COMBOS];
+    KernelTable decode_tiled_grouped_dyn[2 * ABQ_NUM_COMBOS];
     Registry()
     {
         int i = 0;
@@ -68,6 +70,7 @@ struct Registry {
     abq_decode_tiled_register_##Q##_##P(&decode_tiled[i]); \
     abq_decode_tiled_grouped_register_##Q##_##P(&decode_tiled_grouped[i]); \
     abq_decode_tiled_f16_register_##Q##_##P(&decode_tiled_f16[i]); \
+    abq_decode_tiled_grouped_dyn_register_##Q##_##P(&decode_tiled_grouped_dyn[i]); \
     i += 2;
         ABQ_FOR_EACH_COMBO(ABQ_REG)
 #undef ABQ_REG
@@ -1100,7 +1103,8 @@ abq_status abq_gemm_set_zero_points(abq_gemm_state *state, const float *x_zero, 
         return ABQ_ERR_NOT_INITIALIZED;
     if (state->group_size == 0) // only the group-scale kernel carries the correction terms
         return ABQ_ERR_UNSUPPORTED;
-    if ((w_zero && !x_group_sums) || (x_zero && !w_zero_term))
+    const bool x_dynamic = state->x_layout == ABQ_LAYOUT_F16 && state->reserved[1] != 0; // sums and zero points made in the kernel
+    if ((w_zero && !x_group_sums && !x_dynamic) || (x_zero && !w_zero_term) || (x_dynamic && state->reserved[1] == 2 && !w_zero_term))
         return ABQ_ERR_INVALID_ARG;
     state->x_zero = x_zero;
     state->w_zero = w_zero;
@@ -1230,7 +1234,8 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
 {
     if (!st || !st->init_success)
         return ABQ_ERR_NOT_INITIALIZED;
-    if (st->out_kind == ABQ_OUT_F16_SCALED && (!st->x_scale || !st->w_scale))
+    const bool x_dynamic = st->x_layout == ABQ_LAYOUT_F16 && st->reserved[1] != 0; // the kernel takes the token scales itself
+    if (st->out_kind == ABQ_OUT_F16_SCALED && ((!st->x_scale && !x_dynamic) || !st->w_scale))
         return ABQ_ERR_INVALID_ARG;
     GemmArgs a;
     a.X = st->X;
@@ -1252,6 +1257,7 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     a.x_group_sums = st->x_group_sums;
     a.w_zero_term = st->w_zero_term;
     a.x_pack_scale = st->x_pack_scale;
+    a.x_dynamic = st->x_layout == ABQ_LAYOUT_F16 ? st->reserved[1] : 0;
     const Registry &reg = registry();
     const abq_tile_config &c = st->cfg;
     hipError_t e;
@@ -1292,7 +1298,9 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
         const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, c.w_bits);
         if (st->x_layout == ABQ_LAYOUT_FP6 || st->w_layout == ABQ_LAYOUT_FP6)
             return ABQ_ERR_NOT_INITIALIZED;
-        if (x_f16 && (st->strategy != ABQ_STRATEGY_DECODE_TILED || st->group_size || !st->x_pack_scale))
+        if (x_f16 && (st->strategy != ABQ_STRATEGY_DECODE_TILED ||
+                      (x_dynamic ? st->group_size != 128 || (st->reserved[1] == 2 && !st->w_zero_term)
+                                 : st->group_size != 0 || !st->x_pack_scale)))
             return ABQ_ERR_NOT_INITIALIZED;
         if (xb + wb > st->workspace_bytes || ((xb + wb) && !st->workspace))
             return ABQ_ERR_INVALID_ARG;
@@ -1310,7 +1318,10 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
             a.W = reinterpret_cast<const uint32_t *>(ws + xb);
         }
         const KernelTable *t = find_table(st->strategy == ABQ_STRATEGY_DECODE_TILED
-                                              ? (st->group_size ? reg.decode_tiled_grouped : x_f16 ? reg.decode_tiled_f16 : reg.decode_tiled)
+                                              ? (x_dynamic         ? reg.decode_tiled_grouped_dyn
+                                                 : st->group_size ? reg.decode_tiled_grouped
+                                                 : x_f16          ? reg.decode_tiled_f16
+                                                                  : reg.decode_tiled)
                                           : st->group_size ? reg.tiled_grouped
                                                            : reg.tiled,
                                           c.x_bits, c.w_bits, c.is_signed);
@@ -1466,6 +1477,27 @@ abq_status abq_gemm_set_f16_activations(abq_gemm_state *st, const void *x_f16, c
     st->X = static_cast<const uint32_t *>(x_f16);
     st->x_layout = ABQ_LAYOUT_F16;
     st->x_pack_scale = scale_dev;
+    return ABQ_OK;
+}
+
+abq_status abq_gemm_set_dynamic_f16_activations(abq_gemm_state *st, const void *x_f16, int symmetric)
+{
+    if (!st || !st->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    if (!x_f16)
+        return ABQ_ERR_INVALID_ARG;
+    const abq_tile_config &c = st->cfg;
+    const KernelTable *t = find_table(registry().decode_tiled_grouped_dyn, c.x_bits, c.w_bits, c.is_signed);
+    // a workgroup quantises all of its rows in registers: 16384 elements (the instance of eight waves; all rows of a
+    // call at most 16, which is what the decode kernel takes per workgroup without splitting M)
+    if (st->strategy != ABQ_STRATEGY_DECODE_TILED || st->group_size != 128 || st->w_layout != ABQ_LAYOUT_TILED || !t || t->count == 0 ||
+        st->variant != 0 || st->M > 16 || (size_t)st->M * st->K > 16384 || (st->x_zero && symmetric))
+        return ABQ_ERR_UNSUPPORTED;
+    if (!symmetric && !st->w_zero_term && st->x_zero)
+        return ABQ_ERR_INVALID_ARG;
+    st->X = static_cast<const uint32_t *>(x_f16);
+    st->x_layout = ABQ_LAYOUT_F16;
+    st->reserved[1] = symmetric ? 1 : 2;
     return ABQ_OK;
 }
 

@@ -30,6 +30,7 @@
 //     any order gives the same bits).
 // K longer than NW * D steps runs further rounds of the same loop (their latency is exposed).
 #include "abq_kernels.h"
+#include "abq_quant.h"
 
 #ifndef ABQ_Q
 #error "compile with -DABQ_Q=<x_bits> -DABQ_P=<w_bits>"
@@ -232,10 +233,11 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
         v4u wb[D][T];
         v4u xr[XF16 ? XP : 1];
         if (XF16 && round == 0) {
+            // every pass is loaded, past the rows' end the last unit once more: a load under a condition would leave the
+            // compiler a register to merge with an undefined one, and a copy it inserts for that reads before the data lands
 #pragma unroll
             for (int i = 0; i < XP; ++i)
-                if (i * NT < nunits) // the same for every wave: the counted waits below do not depend on it
-                    xr[i] = dt_load16(Xh, (uint32_t)min(tid + i * NT, nunits - 1) * 16u);
+                xr[i] = dt_load16(Xh, (uint32_t)min(tid + i * NT, nunits - 1) * 16u);
         }
 #pragma unroll
         for (int d = 0; d < D; ++d) {
@@ -252,11 +254,12 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
             if constexpr (XF16) {
                 const _Float16 hs = (_Float16)a.x_pack_scale[0];
 #pragma unroll
+                for (int i = 0; i < XP; ++i)
+                    dt_landed(xr[i]);
+#pragma unroll
                 for (int i = 0; i < XP; ++i) {
-                    if (i * NT < nunits) { // the quads of a wave are whole
-                        dt_landed(xr[i]);
+                    if (i * NT < nunits) // the quads of a wave are whole
                         quantise_unit(xr[i], tid + i * NT, hs);
-                    }
                 }
                 // rows too long for one pass: further passes, their latency exposed
                 for (int base = XP * NT; base < nunits; base += XP * NT) {
@@ -437,9 +440,16 @@ template <int P, bool SIGNED> __device__ __forceinline__ void dtg_operands(const
     }
 }
 
-template <int Q, int P, bool SIGNED, int NW, int D, int T>
+// XDYN: the activations arrive as fp16 [M][K] and are quantised here per token, symmetric or with a zero point
+// (a.x_dynamic = 1 or 2), exactly as the quantise-and-pack kernel does it (abq_quant.h): every workgroup loads the
+// rows it multiplies (at most XP * 64 NW units of eight halves), takes their extrema through LDS, writes the int8
+// records and the group sums into LDS and keeps the rows' scales and zero points there for the epilogue.  The
+// quantising launch in front of every decode GEMM, and the memory round trip between the two, fall away.
+template <int Q, int P, bool SIGNED, int NW, int D, int T, bool XDYN = false>
 __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmArgs a, int mrows)
 {
+    static_assert(!XDYN || (Q == 8 && SIGNED), "in-kernel quantisation writes signed 8-bit records");
+    constexpr int XP = NW == 16 ? 2 : 4; // XDYN: units per thread (16384 elements per workgroup either way)
     constexpr int NT = 64 * NW;
     constexpr int QLOG = Q == 8 ? 3 : Q == 4 ? 2 : 1;
     constexpr int LPS = DtgShare<P>::kLoads; // loads per step and tile
@@ -464,10 +474,23 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
     float *sws = reinterpret_cast<float *>(xs + (size_t)mrows * (KT + 1) * Q * 16 + 1024); // [T][group][16]
     float *zws = sws + T * per_arr;                                                       // [T][group][16]
     int *sxs = reinterpret_cast<int *>(zws + T * per_arr);                                // [group][16]
+    // XDYN: the rows' extrema (as integers that order like the floats), then their scales and zero points
+    int *row_ext = sxs + per_arr;                                                         // [2][16]
+    float *row_par = reinterpret_cast<float *>(row_ext + 32);                             // [2][16]
     const bool zp = a.w_zero != nullptr;
+    const int upr = a.K >> 3; // XDYN: units of eight halves per row
+    const int nunits = Mb * upr;
+    const char *Xh = Xt + (size_t)m0 * a.K * 2;
+    if constexpr (XDYN) {
+        if (tid < 16) {
+            row_ext[tid] = INT_MIN;      // maxima
+            row_ext[16 + tid] = INT_MAX; // minima
+        }
+        __syncthreads(); // the extrema are initialised before any wave updates them
+    }
 
     // ---- activations: LDS chunk p <- chunk p ^ ((p / Q) & (Q - 1)) of the workgroup's rows -----------
-    {
+    if constexpr (!XDYN) {
         const int per = Mb * Q;
         for (int pb = wid * 64; pb < xchunks; pb += NT) {
             const int p = min(pb + lane, xchunks - 1);
@@ -494,7 +517,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
                     dt_dma_dword(a.w_zero + src, (unsigned)(size_t)(zws + t * per_arr + pb));
             }
         }
-        if (zp) {
+        if (zp && !XDYN) {
             for (int pb = wid * 64; pb < nfl; pb += NT) {
                 const int p = min(pb + lane, nfl - 1);
                 const int m = m0 + min(p & 15, Mb - 1);
@@ -525,6 +548,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
     int round = 0;
     do {
         DtgShare<P> wb[D][T];
+        v4u xr[XDYN ? XP : 1]; // (declared and loaded inside the round that uses them, like the weight registers)
+        if (XDYN && round == 0) {
+            // every pass is loaded, past the rows' end the last unit once more: a load under a condition would leave the
+            // compiler a register to merge with an undefined one, and a copy it inserts for that reads before the data lands
+#pragma unroll
+            for (int i = 0; i < XP; ++i)
+                xr[i] = dt_load16(Xh, (uint32_t)min(tid + i * NT, nunits - 1) * 16u);
+        }
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             const int s = min(wid + (round * D + d) * NW, KT - 1); // steps past the end repeat the last one
@@ -534,7 +565,91 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
                 wb[d][t].issue(wp, woff[t]);
         }
         if (round == 0) {
-            dt_wait_loads<D * T * LPS>(); // the DMA loads are older than these
+            dt_wait_loads<D * T * LPS>(); // the DMA loads (and the rows' fp16 units) are older than these
+            if constexpr (XDYN) {
+                // extrema of the rows: per unit on the fp16 pairs, per wave across the lanes where the wave's units
+                // of this pass belong to one row, then one LDS update per wave (per lane where rows meet in a wave)
+                typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+                for (int i = 0; i < XP; ++i)
+                    dt_landed(xr[i]);
+#pragma unroll
+                for (int i = 0; i < XP; ++i) {
+                    if (i * NT < nunits) {
+                        const int p = tid + i * NT;
+                        union {
+                            v4u q;
+                            h2 h[4];
+                        } raw;
+                        raw.q = xr[i];
+                        h2 mx2 = __builtin_elementwise_max(__builtin_elementwise_max(raw.h[0], raw.h[1]), __builtin_elementwise_max(raw.h[2], raw.h[3]));
+                        h2 mn2 = __builtin_elementwise_min(__builtin_elementwise_min(raw.h[0], raw.h[1]), __builtin_elementwise_min(raw.h[2], raw.h[3]));
+                        float mx = fmaxf((float)mx2.x, (float)mx2.y), mn = fminf((float)mn2.x, (float)mn2.y);
+                        const int pc = min(p, nunits - 1);
+                        const int row = pc / upr;
+                        const int first = __builtin_amdgcn_readfirstlane(min(p - lane, nunits - 1) / upr);
+                        const int last = __builtin_amdgcn_readfirstlane(min(p - lane + 63, nunits - 1) / upr);
+                        auto ordered = [](float f) { const int k = __builtin_bit_cast(int, f); return k ^ ((k >> 31) & 0x7FFFFFFF); };
+                        if (first == last) {
+#pragma unroll
+                            for (int o = 32; o > 0; o >>= 1) {
+                                mx = fmaxf(mx, __shfl_xor(mx, o));
+                                mn = fminf(mn, __shfl_xor(mn, o));
+                            }
+                            if (lane == 0) {
+                                atomicMax(&row_ext[row], ordered(mx));
+                                atomicMin(&row_ext[16 + row], ordered(mn));
+                            }
+                        } else if (p < nunits) {
+                            atomicMax(&row_ext[row], ordered(mx));
+                            atomicMin(&row_ext[16 + row], ordered(mn));
+                        }
+                    }
+                }
+                __syncthreads();
+                uint32_t sel_pair, sel_half;
+                quad_transpose_selectors(tid & 3, sel_pair, sel_half);
+                auto unordered = [](int k) { return __builtin_bit_cast(float, k ^ ((k >> 31) & 0x7FFFFFFF)); };
+#pragma unroll
+                for (int i = 0; i < XP; ++i) {
+                    if (i * NT < nunits) { // quads and scale groups of a wave are whole: K is a multiple of 128
+                        const int p = tid + i * NT;
+                        const int pc = min(p, nunits - 1);
+                        const int row = pc / upr, u = pc - row * upr;
+                        const QuantRow qr = quant_row_params(unordered(row_ext[row]), unordered(row_ext[16 + row]), 8, a.x_dynamic == 1);
+                        union {
+                            v4u q;
+                            _Float16 h[8];
+                        } raw;
+                        raw.q = xr[i];
+                        int v[8], sum = 0;
+#pragma unroll
+                        for (int c = 0; c < 8; ++c) {
+                            v[c] = quant_code((float)raw.h[c], qr);
+                            sum += v[c];
+                        }
+                        // the sixteen units of a scale group sit in sixteen consecutive lanes
+                        sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+                        sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+                        sum += __builtin_amdgcn_update_dpp(0, sum, 0x141, 0xF, 0xF, true); // row_half_mirror
+                        sum += __builtin_amdgcn_update_dpp(0, sum, 0x140, 0xF, 0xF, true); // row_mirror
+                        const uint32_t e_even = quad_transpose_bytes(pack_low_bytes(v[7], v[5], v[3], v[1]), sel_pair, sel_half);
+                        const uint32_t e_odd = quad_transpose_bytes(pack_low_bytes(v[6], v[4], v[2], v[0]), sel_pair, sel_half);
+                        if (p < nunits) {
+                            const int rowi = (u >> 4) * Mb + row;            // K tile * rows + row
+                            const int dw = 8 * ((u >> 2) & 3) + 2 * (u & 3); // first of the lane's two dwords in the record
+                            const int chunk = (dw >> 2) ^ (rowi & 7);
+                            *reinterpret_cast<uint2 *>(xs + ((uint32_t)rowi * 8 + chunk) * 16u + (dw & 3) * 4u) = make_uint2(e_even, e_odd);
+                            if ((u & 15) == 0)
+                                sxs[(u >> 4) * 16 + row] = sum;
+                            if (u == 0) {
+                                row_par[row] = qr.scale;
+                                row_par[16 + row] = qr.zero_out;
+                            }
+                        }
+                    }
+                }
+            }
             __syncthreads();
         }
 #pragma unroll
@@ -612,17 +727,20 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
 #pragma unroll
             for (int w = 0; w < NW; ++w)
                 v += red[(w * T + t) * 256 + rem];
-            if (a.x_zero)
-                v -= a.x_zero[m0 + i] * a.w_zero_term[n];
-            v *= a.x_scale[m0 + i];
+            const bool row_zero = XDYN ? a.x_dynamic == 2 : a.x_zero != nullptr;
+            const float xz = !row_zero ? 0.f : XDYN ? row_par[16 + i] : a.x_zero[m0 + i];
+            const float xsc = XDYN ? row_par[i] : a.x_scale[m0 + i];
+            if (row_zero)
+                v -= xz * a.w_zero_term[n];
+            v *= xsc;
             if (T > 1 && a.act) { // this tile holds gate rows, the next one their up rows
                 float up = 0.f;
 #pragma unroll
                 for (int w = 0; w < NW; ++w)
                     up += red[(w * T + (T > 1 ? t + 1 : t)) * 256 + rem];
-                if (a.x_zero)
-                    up -= a.x_zero[m0 + i] * a.w_zero_term[n + 16];
-                up *= a.x_scale[m0 + i];
+                if (row_zero)
+                    up -= xz * a.w_zero_term[n + 16];
+                up *= xsc;
                 reinterpret_cast<_Float16 *>(a.D)[(size_t)(m0 + i) * (N / 2) + (n >> 5) * 16 + c] = (_Float16)(silu(v) * up);
             } else {
                 reinterpret_cast<_Float16 *>(a.D)[(size_t)(m0 + i) * N + n] = (_Float16)v;
@@ -632,48 +750,53 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
 }
 
 // (waves, loads in flight per wave, tiles) by shape; the fused gate needs a tile pair per workgroup.
-template <int Q, int P, bool SIGNED, int NW, int D, int T>
+template <int Q, int P, bool SIGNED, int NW, int D, int T, bool XDYN = false>
 static hipError_t launch_decode_tiled_grouped_as(const GemmArgs &a, hipStream_t stream)
 {
     const int mrows = decode_tiled_grouped_rows(NW, T, a.M, a.K, Q);
     if (mrows == 0)
         return hipErrorInvalidValue;
+    // in-kernel quantisation: a workgroup's rows fit its threads' registers (two or four units of eight halves each)
+    if (XDYN && (size_t)mrows * a.K > 16384)
+        return hipErrorInvalidValue;
     const size_t lds = decode_tiled_grouped_lds(NW, T, mrows, a.K, Q);
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T>),
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T, XDYN>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess)
         return attr;
     const int tiles = (a.N + 15) / 16;
     const dim3 grid((tiles + T - 1) / T, (a.M + mrows - 1) / mrows);
-    hipLaunchKernelGGL((gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T>), grid, dim3(64 * NW), lds, stream, a, mrows);
+    hipLaunchKernelGGL((gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T, XDYN>), grid, dim3(64 * NW), lds, stream, a, mrows);
     return hipGetLastError();
 }
 
-template <int Q, int P, bool SIGNED, int T>
+template <int Q, int P, bool SIGNED, int T, bool XDYN = false>
 static hipError_t launch_decode_tiled_grouped_t(const GemmArgs &a, hipStream_t stream)
 {
     // loads in flight per wave, in units of 8 bytes per lane: 2 or 6 (1 or 3 steps of 8-bit weights)
     constexpr int DS = P == 8 ? 1 : 2, DL = P == 8 ? 3 : 6, DM = P == 8 ? 2 : 4;
     const int KT = a.K / 128;
     const int wgs = ((a.N + 15) / 16 + T - 1) / T;
+    // (the quantising variant on tile pairs has no registers left for the long instances: more rounds instead)
+    constexpr bool kLong = !(XDYN && T == 2);
     if (wgs > 512) // twice the workgroups fit a compute unit with eight waves
-        return (KT + 7) / 8 > DM ? launch_decode_tiled_grouped_as<Q, P, SIGNED, 8, DL, T>(a, stream)
-                                 : launch_decode_tiled_grouped_as<Q, P, SIGNED, 8, DM, T>(a, stream);
-    return (KT + 15) / 16 > DS ? launch_decode_tiled_grouped_as<Q, P, SIGNED, 16, DL, T>(a, stream)
-                               : launch_decode_tiled_grouped_as<Q, P, SIGNED, 16, DS, T>(a, stream);
+        return kLong && (KT + 7) / 8 > DM ? launch_decode_tiled_grouped_as<Q, P, SIGNED, 8, kLong ? DL : DM, T, XDYN>(a, stream)
+                                          : launch_decode_tiled_grouped_as<Q, P, SIGNED, 8, DM, T, XDYN>(a, stream);
+    return kLong && (KT + 15) / 16 > DS ? launch_decode_tiled_grouped_as<Q, P, SIGNED, 16, kLong ? DL : DS, T, XDYN>(a, stream)
+                                        : launch_decode_tiled_grouped_as<Q, P, SIGNED, 16, DS, T, XDYN>(a, stream);
 }
 
-template <int Q, int P, bool SIGNED> static hipError_t launch_decode_tiled_grouped(const GemmArgs &a, hipStream_t stream)
+template <int Q, int P, bool SIGNED, bool XDYN = false> static hipError_t launch_decode_tiled_grouped(const GemmArgs &a, hipStream_t stream)
 {
-    if (a.group_size != 128 || !a.w_scale || !a.x_scale || (size_t)a.N * a.K * P / 8 >= (1ull << 32) ||
-        (size_t)a.M * a.K * Q / 8 >= (1ull << 32))
+    if (a.group_size != 128 || !a.w_scale || (!XDYN && !a.x_scale) || (size_t)a.N * a.K * P / 8 >= (1ull << 32) ||
+        (size_t)a.M * a.K * Q / 8 >= (1ull << 32) || (XDYN && (a.x_dynamic < 1 || a.x_dynamic > 2 || (a.x_dynamic == 2 && !a.w_zero_term))))
         return hipErrorInvalidValue;
     if (a.act) {
         if (a.N % 32 != 0)
             return hipErrorInvalidValue;
-        return launch_decode_tiled_grouped_t<Q, P, SIGNED, 2>(a, stream);
+        return launch_decode_tiled_grouped_t<Q, P, SIGNED, 2, XDYN>(a, stream);
     }
-    return launch_decode_tiled_grouped_t<Q, P, SIGNED, 1>(a, stream);
+    return launch_decode_tiled_grouped_t<Q, P, SIGNED, 1, XDYN>(a, stream);
 }
 
 // Native tile space of this kernel: (waves, weight loads in flight per wave, tiles per workgroup).  Entries name
@@ -696,6 +819,14 @@ static const KernelEntry *const kSignedF16 = nullptr;
 #endif
 // one entry: the launcher picks waves, loads in flight and tiles by shape
 static const KernelEntry kSignedGrouped[] = { { 16, 1, 1, 1, 1, 16, 6, &launch_decode_tiled_grouped<ABQ_Q, ABQ_P, true>, 128 } };
+// ... and the same quantising fp16 activations per token itself (8-bit activations)
+#if ABQ_Q == 8
+static const KernelEntry kSignedGroupedDyn[] = { { 16, 1, 1, 1, 1, 16, 6, &launch_decode_tiled_grouped<ABQ_Q, ABQ_P, true, true>, 128 } };
+#define ABQ_DT_NDYN 1
+#else
+static const KernelEntry *const kSignedGroupedDyn = nullptr;
+#define ABQ_DT_NDYN 0
+#endif
 #if ABQ_Q < 8
 static const KernelEntry kUnsignedGrouped[] = { { 16, 1, 1, 1, 1, 16, 6, &launch_decode_tiled_grouped<ABQ_Q, ABQ_P, false>, 128 } };
 #else
@@ -714,6 +845,8 @@ static const KernelEntry *const kSigned = nullptr;
 static const KernelEntry *const kUnsigned = nullptr;
 static const KernelEntry *const kSignedGrouped = nullptr;
 static const KernelEntry *const kUnsignedGrouped = nullptr;
+static const KernelEntry *const kSignedGroupedDyn = nullptr;
+#define ABQ_DT_NDYN 0
 static const KernelEntry *const kSignedF16 = nullptr;
 #define ABQ_DT_NF16 0
 #define ABQ_DT_NSIGNED 0
@@ -739,6 +872,12 @@ void ABQ_CAT(abq_decode_tiled_grouped_register_, ABQ_Q, _, ABQ_P)(KernelTable *o
 {
     out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSignedGrouped, kSignedGrouped ? 1 : 0 };
     out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, kUnsignedGrouped, kUnsignedGrouped ? 1 : 0 };
+}
+
+void ABQ_CAT(abq_decode_tiled_grouped_dyn_register_, ABQ_Q, _, ABQ_P)(KernelTable *out)
+{
+    out[0] = KernelTable{ ABQ_Q, ABQ_P, 1, kSignedGroupedDyn, ABQ_DT_NDYN };
+    out[1] = KernelTable{ ABQ_Q, ABQ_P, 0, nullptr, 0 };
 }
 
 } // namespace abq

@@ -28,6 +28,7 @@ struct GemmArgs {
     const int *x_group_sums;   // [M][K/group_size] sums of activation codes (needed with w_zero)
     const float *w_zero_term;  // [N] sum_g w_scale * (sum of weight codes - group_size * w_zero) (needed with x_zero)
     const float *x_pack_scale; // kernels that quantise fp16 activations themselves: X is fp16 [M][K], this the static scale
+    int x_dynamic;             // ... or, per token from the rows' own extrema: 1 symmetric, 2 with a zero point; 0: not
 };
 
 typedef hipError_t (*GemmLauncher)(const GemmArgs &, hipStream_t);

@@ -10,6 +10,7 @@
 // a quad assemble the bytes into one word per plane with DPP moves.  Input bytes are read
 // once, every load is 16 bytes wide and consecutive lanes touch consecutive memory.
 #include "abq_kernels.h"
+#include "abq_quant.h"
 
 namespace abq {
 
@@ -400,50 +401,6 @@ __device__ __forceinline__ float wave_max(float v)
     return v;
 }
 
-// What a row's quantisation needs once its minimum and maximum are known.
-struct QuantRow {
-    float scale, recip, zp_stored, lo_stored, hi_stored, zero_out;
-};
-
-// scale, zero point and code range of a row from its extrema (formulas in the comment above)
-__device__ __forceinline__ QuantRow quant_row_params(float mx, float mn, int bits, int symmetric)
-{
-    const int half_range = 1 << (bits - 1);
-    float scale, zp;
-    int lo, hi;
-    if (symmetric) {
-        scale = fmaxf(fabsf(mx), fabsf(mn)) / (float)(half_range - 1);
-        scale = fminf(fmaxf(scale, 1e-5f), 1e4f);
-        zp = 0.f;
-        lo = -half_range;
-        hi = half_range - 1;
-    } else {
-        scale = (mx - mn) / (float)(2 * half_range - 1);
-        scale = fminf(fmaxf(scale, 1e-5f), 1e4f);
-        zp = rintf(fminf(fmaxf(-mn / scale, -1e4f), 1e4f));
-        lo = 0;
-        hi = 2 * half_range - 1;
-    }
-    QuantRow q;
-    q.scale = scale;
-    // x / scale in three operations instead of the dozen of a full division, with the same bits: recip is the
-    // correctly rounded reciprocal (the fp64 quotient is never close enough to an fp32 midpoint for the second
-    // rounding to cross it), t = x recip is within an ulp of the quotient, the residual x - t scale is exact in
-    // an fma, and t + residual recip then rounds to the quotient itself (checked against the division on a CPU
-    // for every finite fp16 value and 600 000 scales of the forms above; a zero may come out with the other
-    // sign, which the rounding to an integer code forgets).  div_fixup restores what a division makes of an
-    // infinite x.
-    q.recip = (float)(1.0 / (double)scale);
-    // rint(q) + zp, clamped to [lo, hi], minus the offset of the stored code: the offset is taken off before the
-    // clamp instead (all three are small integers, so the sums are the same numbers)
-    const float code_offset = symmetric ? 0.f : (float)half_range;
-    q.zp_stored = zp - code_offset;
-    q.lo_stored = (float)lo - code_offset;
-    q.hi_stored = (float)hi - code_offset;
-    q.zero_out = symmetric ? 0.f : zp - (float)half_range;
-    return q;
-}
-
 // Quantises the eight fp16 values of unit u (elements 8u .. 8u + 7) of `row` and writes their share of the
 // packed row; the lanes of a quad hold consecutive units (quad_lane = u & 3), a scale group's lanes are
 // consecutive too.  Inactive lanes (units past the row) take part in the cross-lane steps with zeros.
@@ -466,12 +423,7 @@ __device__ __forceinline__ void quant_emit_unit(const uint4 &rawq, bool active, 
         raw.q = rawq;
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
-            const float xf = (float)raw.h[c];
-            const float t = xf * q.recip;
-            // the fix-up only matters for an infinite x, but one more instruction per element is cheaper than a
-            // branch around it per element
-            const float quotient = __builtin_amdgcn_div_fixupf(__builtin_fmaf(__builtin_fmaf(-t, q.scale, xf), q.recip, t), q.scale, xf);
-            v[c] = (int)__builtin_amdgcn_fmed3f(rintf(quotient) + q.zp_stored, q.lo_stored, q.hi_stored);
+            v[c] = quant_code((float)raw.h[c], q);
             sum += v[c];
         }
     }

@@ -532,7 +532,7 @@ def main():
         # activations quantised per token on the device inside the timed call, fp16 output; gate and up run
         # as one GEMM with the fused SiLU-gate epilogue.  Time = quantise+pack kernel + GEMM, graph replay.
         layer = []
-        for tokens in (1024, 16384):
+        for tokens in (1, 16, 1024, 16384):  # a decode step of batch 1 and 16 (weights stay in the Infinity Cache), two prefills
             for name, N, K, act in (("qkv", 12288, 4096, 0), ("o", 4096, 4096, 0), ("gate_up_silu", 22016, 4096, 1),
                                     ("down", 4096, 11008, 0)):
                 G = K // 128

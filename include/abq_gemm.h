@@ -334,6 +334,18 @@ abq_status abq_gemm_set_operand_layout(abq_gemm_state *state, int x_layout, int 
  * ABQ_ERR_UNSUPPORTED, and the caller packs as before. */
 abq_status abq_gemm_set_f16_activations(abq_gemm_state *state, const void *x_f16, const float *scale_dev);
 
+/* The group-scale variant of the same: a state that runs ABQ_STRATEGY_DECODE_TILED with group scales of 128 (at most
+ * 16 rows, M * K <= 16384, 8-bit signed activations, prepared weights) takes its activations as fp16 [M][K] and
+ * quantises them per token inside the kernel, symmetric (symmetric != 0) or with a zero point, with the formulas
+ * and the rounding of abq_quant_pack_f16 (bit for bit: the output equals that of the two launches).  The token
+ * scales, zero points and group sums never leave the kernel: x_scale given to abq_gemm_set_scales is not read, and
+ * abq_gemm_set_zero_points, called after this, takes w_zero (x_group_sums may be NULL) and, for activations with a
+ * zero point, w_zero_term (x_zero may be NULL).  One launch instead of two and no memory round trip between them:
+ * the quantising launch costs as much as the GEMM at these sizes.  ABQ_ERR_UNSUPPORTED where the kernel or the
+ * shape does not qualify (the caller then quantises with abq_quant_pack_f16 as before).  No counterpart in the
+ * reference, whose activations are quantised by a kernel of their own (abq_gemm_wrapper.cu:29-69). */
+abq_status abq_gemm_set_dynamic_f16_activations(abq_gemm_state *state, const void *x_f16, int symmetric);
+
 /* Workspace needed by abq_gemm_exec if the state ran as ABQ_STRATEGY_TILED (ABQ_STRATEGY_FP6)
  * with its current operand layouts: the converted copies of the operands still in the reference
  * layout (0 if neither is). */

@@ -286,6 +286,68 @@ def test_group_scale_decode_kernel_over_row_blocks(abq, oracle, q, p, signed):
         assert not abq.prepared_decode_pays(8, 2, True, 32, 4096, 4096, 64)
 
 
+def test_decode_kernel_quantises_fp16_activations_per_token_itself(abq, oracle):
+    """abq_gemm_set_dynamic_f16_activations: the group-scale decode kernel on prepared weights takes fp16 activations and
+    quantises them per token in the kernel, symmetric or with a zero point.  Same formulas and rounding as the
+    quantise-and-pack kernel, so the output equals that of the two launches bit for bit (and through it the oracle,
+    which the two-launch path is checked against); rows with outliers, a constant row, ragged N, the fused gate."""
+    rng = np.random.default_rng(4242)
+    for (M, N, K, p, symmetric, with_wz, act) in [(1, 4096, 4096, 2, True, True, False), (1, 4096, 4096, 2, False, True, False),
+                                                  (4, 200, 4096, 2, False, True, False), (3, 330, 1152, 4, True, False, False),
+                                                  (1, 192, 11008, 2, False, True, True), (2, 12288, 4096, 2, False, True, False),
+                                                  (1, 22016, 4096, 2, True, True, True), (4, 64, 128, 8, False, True, False),
+                                                  (16, 96, 1024, 2, False, True, False)]:
+        G = K // 128
+        lo_w, hi_w = -(1 << (p - 1)), 1 << (p - 1)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        wp = planes_dev(oracle.pack_i32(w, p))
+        wt = abq.relayout_planes(wp)
+        wsc = fdev(rng.uniform(0.001, 0.02, (N, G)))
+        wz = fdev(rng.integers(lo_w, hi_w, (N, G)).astype(np.float64)) if with_wz else None
+        xg = torch.Generator(device="cuda").manual_seed(M + N + K)
+        x = torch.randn((M, K), generator=xg, device="cuda", dtype=torch.float32)
+        x[:, ::97] *= 8.0
+        if M > 1:
+            x[M - 1] = 0.25  # a constant row: the scale clamps, the codes saturate
+        x = x.to(torch.float16)
+        xt, xs, xz, sums = abq.quant_pack_f16(x, 8, symmetric=symmetric, tiled=True, group_size=128)
+        term = abq.weight_zero_term(wp, True, wsc, wz, 128) if (with_wz and not symmetric) else None
+        kw = dict(x_scale=xs, w_scale=wsc, group_size=128, x_tiled=True, w_tiled=True, out_kind=abq.OUT_F16_SCALED,
+                  act=abq.ACT_SILU_GATE if act else abq.ACT_NONE)
+        if with_wz:
+            kw.update(w_zero=wz, x_group_sums=sums)
+        if not symmetric:
+            if term is None:
+                term = abq.weight_zero_term(wp, True, wsc, torch.zeros_like(wsc), 128)
+                kw.update(w_zero=torch.zeros_like(wsc), x_group_sums=sums)
+            kw.update(x_zero=xz, w_zero_term=term)
+        ref = abq.Gemm(xt, wt, True, **kw)
+        assert ref.strategy == "decode_tiled"
+        want = ref.run().clone()
+        # the same state, fed the fp16 rows
+        kw2 = {k: v for k, v in kw.items() if k not in ("x_zero", "w_zero_term", "w_zero", "x_group_sums")}
+        out = torch.full_like(want, float("nan"))
+        g = abq.Gemm(xt, wt, True, out=out, **kw2)
+        g.set_dynamic_f16_activations(x, symmetric, w_zero=kw.get("w_zero"), w_zero_term=kw.get("w_zero_term"))
+        got = g.run()
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (M, N, K, p, symmetric, with_wz, act)
+    # shapes and states the kernel does not take: 8 x 4096 elements are too many for one workgroup's registers,
+    # and a state without group scales has no such variant
+    K, N = 4096, 64
+    wt = abq.relayout_planes(planes_dev(oracle.pack_i32(rng.integers(-2, 2, (N, K)).astype(np.int32), 2)))
+    wsc = fdev(rng.uniform(0.001, 0.02, (N, K // 128)))
+    x = torch.randn((8, K), device="cuda", dtype=torch.float16)
+    xt, xs, _, _ = abq.quant_pack_f16(x, 8, symmetric=True, tiled=True, group_size=128)
+    g = abq.Gemm(xt, wt, True, x_scale=xs, w_scale=wsc, group_size=128, x_tiled=True, w_tiled=True, out_kind=abq.OUT_F16_SCALED)
+    with pytest.raises(abq.AbqError):
+        g.set_dynamic_f16_activations(x, True)
+    g = abq.Gemm(xt[:, :4].contiguous(), wt, True, x_scale=xs[:4].contiguous(), w_scale=fdev(rng.uniform(0.001, 0.02, N)),
+                 x_tiled=True, w_tiled=True, out_kind=abq.OUT_F16_SCALED)
+    with pytest.raises(abq.AbqError):
+        g.set_dynamic_f16_activations(x[:4].contiguous(), True)
+
+
 def test_decode_on_prepared_operands_group_scales_either_call_order(abq, oracle):
     """Layouts declared before the scales are attached (the C ABI allows both orders) lands on the same kernel."""
     import ctypes

@@ -162,6 +162,10 @@ def test_library_exports_every_declared_symbol(abq):
     L = abq.lib()
     for name in declared:
         assert hasattr(L, name), name
+        # every entry point that takes arguments has its ctypes signature declared: without one a 64-bit device pointer
+        # is passed as a C int and arrives truncated
+        takes_args = not re.search(r"\b%s\s*\(\s*void\s*\)" % name, header)
+        assert getattr(L, name).argtypes is not None or not takes_args, name
     assert L.abq_version() == 1
     assert L.abq_status_string(2).decode().startswith("K must")
 
