@@ -219,13 +219,37 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
                         (silu_gate ? 32 : 16) * 1024 + (size_t)64 * (K / W.group_size) + 128 + (size_t)M * ((K + 511) / 512 * 512 + 16) <= 160 * 1024;
     const bool fp6 = !decode && !decode_prepared && W.records_fp6 != nullptr && W.group_size == 128 && abq_fp6_eligible(x_bits_, w_bits_, 1, K);
     const int layout = decode ? ABQ_LAYOUT_PLANES : fp6 ? ABQ_LAYOUT_FP6 : ABQ_LAYOUT_TILED;
-    abq_status rc = abq_quant_pack_f16(A, M, K, x_bits_, x_symmetric ? 1 : 0, layout, planes, x_scale, x_zero,
-                                       sums, W.group_size, stream);
+    abq_status rc;
+    abq_gemm_state state;
+    // the smallest calls on the prepared-operand decode kernel: the kernel quantises the rows itself (one launch
+    // instead of two; the quantising launch costs as much as the GEMM at these sizes), same result bit for bit
+    if (decode_prepared && M <= 16 && (size_t)M * K <= 16384) {
+        rc = abq_gemm_init(nullptr, x_bits_, w_bits_, 1, planes, reinterpret_cast<const uint32_t *>(W.planes_tiled), M, N, K, D,
+                           nullptr, 0, ABQ_OUT_F16_SCALED, &state);
+        if (rc == ABQ_OK)
+            rc = abq_gemm_set_operand_layout(&state, ABQ_LAYOUT_TILED, ABQ_LAYOUT_TILED);
+        if (rc == ABQ_OK)
+            rc = abq_gemm_set_scales(&state, x_scale /* not read */, W.scale, W.group_size);
+        if (rc == ABQ_OK && silu_gate)
+            rc = abq_gemm_set_activation(&state, ABQ_ACT_SILU_GATE);
+        if (rc == ABQ_OK)
+            rc = abq_gemm_set_dynamic_f16_activations(&state, A, x_symmetric ? 1 : 0);
+        if (rc == ABQ_OK && (W.zero || !x_symmetric))
+            rc = abq_gemm_set_zero_points(&state, nullptr, W.zero, nullptr, x_symmetric ? nullptr : W.zero_term);
+        if (rc == ABQ_OK && state.init_success) {
+            const abq_status ex = abq_gemm_exec(&state, stream);
+            if (ex != ABQ_OK)
+                printf("[ABQ][Error] launch failed: %s\n", abq_status_string(ex));
+            return;
+        }
+        // (a pair or shape that kernel does not take: the two launches below)
+    }
+    rc = abq_quant_pack_f16(A, M, K, x_bits_, x_symmetric ? 1 : 0, layout, planes, x_scale, x_zero,
+                            sums, W.group_size, stream);
     if (rc != ABQ_OK) {
         printf("[ABQ][Error] pack failed: %s\n", abq_status_string(rc));
         return;
     }
-    abq_gemm_state state;
     rc = abq_gemm_init(nullptr, x_bits_, w_bits_, 1, planes,
                        reinterpret_cast<const uint32_t *>(decode ? W.planes : fp6 ? W.records_fp6 : W.planes_tiled), M, N, K,
                        D, nullptr, 0, ABQ_OUT_F16_SCALED, &state);

@@ -565,10 +565,25 @@ def main():
                 torch.cuda.synchronize()
                 us = e0.elapsed_time(e1) * 1e3 / reps
                 tops = 2.0 * tokens * N * K / (us * 1e-6) / 1e12
-                layer.append(dict(linear=name, tokens=tokens, N=N, K=K, us=round(us, 1), tops=round(tops, 1),
-                                  mfma_frac=round(tops / INT8_MFMA_PEAK_TOPS, 4), kernel="%s:%s" % (gm.strategy, gm.config_name)))
+                entry = dict(linear=name, tokens=tokens, N=N, K=K, us=round(us, 1), tops=round(tops, 1),
+                             mfma_frac=round(tops / INT8_MFMA_PEAK_TOPS, 4), kernel="%s:%s" % (gm.strategy, gm.config_name))
                 log("layer %s tokens=%d N=%d K=%d  %.1f us  %.0f TOPS (%.1f%% of int8 MFMA peak)"
                     % (name, tokens, N, K, us, tops, 100 * tops / INT8_MFMA_PEAK_TOPS))
+                if tokens <= 16 and tokens * K <= 16384 and gm.strategy == "decode_tiled":
+                    # the smallest calls: the decode kernel quantises the rows itself, one launch, same output bit for bit
+                    out1 = torch.empty_like(out)
+                    g1 = abq.Gemm(xt, wt, SIGNED, out=out1, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc, group_size=128,
+                                  x_tiled=True, w_tiled=True, act=act)
+                    g1.set_dynamic_f16_activations(x, True, w_zero=wz)
+                    g1.run()
+                    torch.cuda.synchronize()
+                    if not torch.equal(out1, out):
+                        raise RuntimeError("one-launch dynamic GEMM differs from quantise + GEMM (%s, tokens=%d)" % (name, tokens))
+                    us1 = time_rotating([g1], reps=20)
+                    entry["one_launch_us"] = round(us1, 1)
+                    log("layer %s tokens=%d: one launch (kernel quantises the rows) %.1f us" % (name, tokens, us1))
+                    del g1, out1
+                layer.append(entry)
                 del gr, gm, out, x, xt, wt
         extra["decoder_layer_w2a8_group128"] = layer
 

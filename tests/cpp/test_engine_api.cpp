@@ -577,6 +577,81 @@ static void gpu_paths()
         }
     }
 
+    {   // the smallest dynamic calls on prepared weights with groups of 128: one launch that quantises the rows
+        // itself; the workspace stays untouched and the output equals, bit for bit, quantise + GEMM called
+        // through the C interface
+        const int N = 320, K = 1024, G = 128;
+        std::mt19937 r32(29);
+        std::normal_distribution<float> nd(0.f, 0.05f), xd_(0.3f, 1.f);
+        std::vector<float> wf((size_t)N * K);
+        for (auto &v : wf)
+            v = nd(r32);
+        ABQWeightBlob blob;
+        std::string err;
+        CHECK(abq_quantize_weights(wf.data(), N, K, 2, false, G, &blob, &err));
+        ABQDeviceWeight dw;
+        CHECK(dw.load(blob, stream, &err));
+        const ABQGroupedWeight W = dw.grouped();
+        ABQGEMMWrapper wrap(8, 2, true);
+        for (int M : { 1, 5, 16 })
+            for (int symmetric = 0; symmetric < 2; ++symmetric) {
+                std::vector<uint16_t> ha((size_t)M * K);
+                for (auto &h : ha)
+                    h = abq_oracle_f32_to_f16(xd_(r32));
+                const size_t ws_bytes = wrap.dynamic_workspace_bytes(M, K, G);
+                _Float16 *d_a, *d_d, *d_e;
+                char *d_ws, *d_ws2;
+                HIP_OK(hipMalloc(&d_a, ha.size() * 2));
+                HIP_OK(hipMalloc(&d_d, (size_t)M * N * 2));
+                HIP_OK(hipMalloc(&d_e, (size_t)M * N * 2));
+                HIP_OK(hipMalloc(&d_ws, ws_bytes));
+                HIP_OK(hipMalloc(&d_ws2, ws_bytes));
+                HIP_OK(hipMemcpy(d_a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
+                HIP_OK(hipMemset(d_ws, 0xAB, ws_bytes));
+                HIP_OK(hipMemset(d_d, 0, (size_t)M * N * 2));
+                CHECK(abq_prepared_decode_pays(8, 2, 1, M, N, K, G, ABQ_ACT_NONE) == 1);
+                wrap.gemm_dynamic(M, N, K, d_a, W, d_d, symmetric != 0, d_ws, ws_bytes, stream);
+                HIP_OK(hipStreamSynchronize(stream));
+                std::vector<unsigned char> hws(ws_bytes);
+                HIP_OK(hipMemcpy(hws.data(), d_ws, ws_bytes, hipMemcpyDeviceToHost));
+                bool untouched = true;
+                for (unsigned char b : hws)
+                    untouched = untouched && b == 0xAB;
+                CHECK(untouched);
+                // the same call as two launches
+                const size_t planes_bytes = ((size_t)M * K + 255) / 256 * 256;
+                uint32_t *planes = reinterpret_cast<uint32_t *>(d_ws2);
+                float *x_scale = reinterpret_cast<float *>(d_ws2 + planes_bytes);
+                float *x_zero = x_scale + M;
+                int32_t *sums = reinterpret_cast<int32_t *>(x_zero + M);
+                CHECK(planes_bytes + (size_t)M * 8 + (size_t)M * (K / G) * 4 <= ws_bytes);
+                CHECK(abq_quant_pack_f16(d_a, M, K, 8, symmetric, ABQ_LAYOUT_TILED, planes, x_scale, x_zero, sums, G,
+                                         stream) == ABQ_OK);
+                abq_gemm_state st;
+                CHECK(abq_gemm_init(nullptr, 8, 2, 1, planes, reinterpret_cast<const uint32_t *>(W.planes_tiled), M, N,
+                                    K, d_e, nullptr, 0, ABQ_OUT_F16_SCALED, &st) == ABQ_OK);
+                CHECK(abq_gemm_set_operand_layout(&st, ABQ_LAYOUT_TILED, ABQ_LAYOUT_TILED) == ABQ_OK);
+                CHECK(abq_gemm_set_scales(&st, x_scale, W.scale, G) == ABQ_OK);
+                CHECK(abq_gemm_set_zero_points(&st, symmetric ? nullptr : x_zero, W.zero, sums,
+                                               symmetric ? nullptr : W.zero_term) == ABQ_OK);
+                CHECK(abq_gemm_exec(&st, stream) == ABQ_OK);
+                HIP_OK(hipStreamSynchronize(stream));
+                std::vector<uint16_t> got((size_t)M * N), want((size_t)M * N);
+                HIP_OK(hipMemcpy(got.data(), d_d, got.size() * 2, hipMemcpyDeviceToHost));
+                HIP_OK(hipMemcpy(want.data(), d_e, want.size() * 2, hipMemcpyDeviceToHost));
+                bool nonzero = false;
+                for (uint16_t h : want)
+                    nonzero = nonzero || (h & 0x7fff);
+                CHECK(nonzero);
+                CHECK(got == want);
+                HIP_OK(hipFree(d_a));
+                HIP_OK(hipFree(d_d));
+                HIP_OK(hipFree(d_e));
+                HIP_OK(hipFree(d_ws));
+                HIP_OK(hipFree(d_ws2));
+            }
+    }
+
     {   // timer interface
         CudaTimer t(stream);
         t.start();
