@@ -279,7 +279,7 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         st->variant = v;
         entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
         st->grid_dim = abq_dim3{ (unsigned)(8 * npx * mblocks), 1, 1 };
-        st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
+        st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn * e.wk), 1, 1 };
         st->shared_mem_size = e.lds;
         return ABQ_OK;
     }
@@ -334,12 +334,12 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
 
     if (strategy == ABQ_STRATEGY_TILED) {
         const KernelTable *tt_ = find_table(reg.tiled, x_bits, w_bits, is_signed);
-        if (!tt_ || mi != 32 || wk != 1)
+        if (!tt_ || mi != 32)
             return ABQ_ERR_UNSUPPORTED;
         int v = -1;
         for (int i = 0; i < tt_->count; ++i) {
             const KernelEntry &t = tt_->entries[i];
-            if (t.tm == tm && t.tn == tn && t.wm == wm && t.wn == wn && t.kb == cfg->warp_k)
+            if (t.tm == tm && t.tn == tn && t.wm == wm && t.wn == wn && t.wk == wk && t.kb == cfg->warp_k)
                 v = i;
         }
         if (v < 0)
@@ -353,7 +353,7 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         st->variant = v;
         entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
         st->grid_dim = abq_dim3{ (unsigned)(8 * npx * mblocks), 1, 1 };
-        st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
+        st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn * e.wk), 1, 1 };
         st->shared_mem_size = e.lds ? e.lds : 2 * (size_t)(bm + bn) * (e.kb + 16) + (bm + bn) * 4;
         return ABQ_OK;
     }
@@ -725,7 +725,7 @@ static int pick_large_tile(const KernelEntry *entries, int count, const LargeTil
             continue;
         for (int i = 0; i < count; ++i)
             if (entries[i].tm == cands[k].tm && entries[i].tn == cands[k].tn && entries[i].wm == cands[k].wm &&
-                entries[i].wn == cands[k].wn && entries[i].kb == 128) {
+                entries[i].wn == cands[k].wn && entries[i].wk == 1 && entries[i].kb == 128) {
                 best = cost;
                 pick = i;
             }
@@ -786,12 +786,40 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
         const long tiles = (long)((st->M + bm - 1) / bm) * ((st->N + bn - 1) / bn);
         const long need = (staged && o[0] == 2 && o[1] == 2 && o[2] == 4) ? 160 : o[4];
         for (int i = 0; i < tt->count; ++i)
-            if (tt->entries[i].tm == o[0] && tt->entries[i].tn == o[1] && tt->entries[i].kb == 128 &&
+            if (tt->entries[i].tm == o[0] && tt->entries[i].tn == o[1] && tt->entries[i].kb == 128 && tt->entries[i].wk == 1 &&
                 tt->entries[i].wm == o[2] && tt->entries[i].wn == o[3] && tiles >= need && pick < 0)
                 pick = i;
     }
     if (pick < 0)
         return ABQ_ERR_UNSUPPORTED;
+    {
+        // Small grids on the staged kernel.  What bounds them is the LDS traffic per MFMA (every byte of a tile is
+        // written into LDS once and read by two waves) and the chain of latencies per K tile, not the matrix cores:
+        // below 200 tiles of 128x128, two groups of waves per workgroup split K (half the K loop's trips for the same
+        // tile), and where an activation row is the longer record the tile is laid along N (64x128: 12 instead of
+        // 18 KB per K tile for W2A8), also up to 400 tiles, where 128x128 leaves part of the chip idle.  Sweep over
+        // W2A8 and W4A4, M = 256 .. 2048 on the LLaMA-7B widths: 5-12 % below 200 tiles, 2-9 % on 64x128 up to 400
+        // (W2A2 7-12 %, W4A8 1-5 %; W8A8, whose tiles are all LDS traffic, -5 .. +4 %: left as it was).
+        const long t128 = (long)((st->M + 127) / 128) * ((st->N + 127) / 128);
+        const long n128x64 = (long)((st->M + 127) / 128) * ((st->N + 63) / 64);
+        const bool along_n = c.x_bits > c.w_bits;
+        int want[5] = { 0, 0, 2, 2, 0 }; // TM, TN, waves along M and N, K groups
+        if (tt->entries[pick].lds != 0 && t128 < 200 && c.x_bits + c.w_bits < 16) {
+            want[4] = 2;
+            want[0] = n128x64 < 256 ? 1 : along_n ? 1 : 2;
+            want[1] = n128x64 < 256 ? 1 : along_n ? 2 : 1;
+        } else if (tt->entries[pick].lds != 0 && along_n && t128 < 400 && tt->entries[pick].tm * tt->entries[pick].wm <= 4 &&
+                   tt->entries[pick].tn * tt->entries[pick].wn <= 4) {
+            want[4] = 1;
+            want[0] = 1;
+            want[1] = 2;
+        }
+        for (int i = 0; want[4] && i < tt->count; ++i) {
+            const KernelEntry &e = tt->entries[i];
+            if (e.lds != 0 && e.tm == want[0] && e.tn == want[1] && e.wm == want[2] && e.wn == want[3] && e.wk == want[4] && e.kb == 128)
+                pick = i;
+        }
+    }
     abq_tile_config cfg;
     entry_to_config(tt->entries[pick], ABQ_STRATEGY_TILED, c.x_bits, c.w_bits, c.is_signed, 0, &cfg);
     abq_gemm_state tmp = *st;
@@ -837,7 +865,7 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
         st->strategy = ABQ_STRATEGY_FP6;
         st->variant = gpick;
         st->grid_dim = abq_dim3{ (unsigned)(8 * (((st->N + bn - 1) / bn + 7) / 8) * ((st->M + bm - 1) / bm)), 1, 1 };
-        st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
+        st->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn * e.wk), 1, 1 };
         st->shared_mem_size = e.lds;
         return ABQ_OK;
     }
@@ -1021,13 +1049,19 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
         for (const auto &o : order) {
             if (pick >= 0 || t128 < o[2])
                 continue;
+            // below 200 tiles two groups of waves split K inside the workgroup where that is built (8-13 % on
+            // 256 and 512 rows of the LLaMA-7B widths, nothing from 1024 on)
+            const bool split = t128 < 200;
             for (int i = 0; i < tg->count; ++i) // the last match: the staged kernel's entry where there is one
-                if (usable(tg->entries[i]) && block_m(tg->entries[i]) == o[0] && block_n(tg->entries[i]) == o[1])
+                if (usable(tg->entries[i]) && block_m(tg->entries[i]) == o[0] && block_n(tg->entries[i]) == o[1] &&
+                    (tg->entries[i].wk == 1 || (split && tg->entries[i].wk == 2)))
                     pick = i;
         }
     } else {
+        const int wk = c.warp_k > 0 ? c.block_k / c.warp_k : 1;
         for (int i = 0; i < tg->count; ++i)
-            if (usable(tg->entries[i]) && block_m(tg->entries[i]) == c.block_m && block_n(tg->entries[i]) == c.block_n)
+            if (usable(tg->entries[i]) && block_m(tg->entries[i]) == c.block_m && block_n(tg->entries[i]) == c.block_n &&
+                tg->entries[i].wk == wk)
                 pick = i;
     }
     if (pick < 0)
@@ -1039,7 +1073,7 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
         const KernelEntry &e = tg->entries[pick];
         const int bm = block_m(e), bn = block_n(e);
         state->grid_dim = abq_dim3{ (unsigned)(8 * (((state->N + bn - 1) / bn + 7) / 8) * ((state->M + bm - 1) / bm)), 1, 1 };
-        state->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn), 1, 1 };
+        state->block_dim = abq_dim3{ (unsigned)(64 * e.wm * e.wn * e.wk), 1, 1 };
         state->shared_mem_size = e.lds ? e.lds : 2 * (size_t)(bm + bn) * (e.kb + 16) + (bm + bn) * 4;
     }
     return ABQ_OK;

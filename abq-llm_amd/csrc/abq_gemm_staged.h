@@ -24,7 +24,8 @@
 // read out of LDS while the MFMAs of tile t run.  The compiler would drain every outstanding load
 // of this kind before each ds_read, so they are issued from inline assembly and waited for by
 // hand: every wave issues the same number of loads per tile, which makes "all but the newest n
-// tiles have landed" one s_waitcnt vmcnt(n * loads per tile).  No other vector-memory instruction
+// tiles have landed" one s_waitcnt vmcnt(n * loads per tile).  (WK > 1: a "tile" here is the K tiles of
+// one trip of the K loop, one per group of waves; see the kernel's comment.)  No other vector-memory instruction
 // may be in flight while that count is relied on: the kernel has none inside its K loop and
 // drains the counter before its epilogue.  A register spill would be such an instruction: every
 // instantiation must compile with .vgpr_spill_count 0 and no private segment (hipcc -save-temps
@@ -140,13 +141,22 @@ template <int TM, int TN, int WM, int WN, int STAGE_BYTES> struct StagedOutputLd
 // the one finished before it into the fp32 accumulators (a convert and a multiply-add per element: as
 // many cycles as the four MFMAs take).  The last MFMA tile of a K tile is folded during the first of the
 // next K tile.
-template <int QB, int PB, bool SIGNED, bool FP6, int TM, int TN, int WM, int WN, int S, bool GROUPED = false>
-__global__ __launch_bounds__(64 * WM * WN, (WM * WN > 4 || TM * TN > 4) ? 1 : 2)
+//
+// WK > 1: WK groups of WM x WN waves share the workgroup's output tile and split K between them: a stage holds WK
+// consecutive K tiles, group wk loads and multiplies the wk-th of them, and the groups' partial tiles meet in LDS
+// after the K loop (added in a fixed order; int32 sums are exact whatever the order).  A K loop on a grid that
+// leaves a compute unit one or two workgroups is a chain of latencies per K tile (wait, barrier, LDS read, four
+// dependent MFMAs) that does not shrink with the tile; WK groups walk through it side by side and pay it K / (128 WK)
+// times.  With a number of K tiles that is no multiple of WK the last trip finds some groups without a tile: they
+// request their last tile once more, like every wave past the end, and leave its MFMAs out (with group scales: run
+// them under a scale of zero).
+template <int QB, int PB, bool SIGNED, bool FP6, int TM, int TN, int WM, int WN, int S, bool GROUPED = false, int WK = 1>
+__global__ __launch_bounds__(64 * WM * WN * WK, (WM * WN * WK > 4 || TM * TN > 4) ? 1 : 2)
 void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_blocks, int n_blocks_per_xcd)
 {
     using TA = StagedOperand<QB, FP6>;
     using TB = StagedOperand<PB, FP6>;
-    constexpr int NW = WM * WN;
+    constexpr int NW = WM * WN;                                // waves of one K group
     constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
     constexpr int SC_OFF = BM * TA::kRow + BN * TB::kRow;      // GROUPED: the tile's scales follow its records
     constexpr int BUF_BYTES = SC_OFF + (GROUPED ? (BN > 128 ? 4 * BN : 512) : 0);
@@ -165,19 +175,24 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     // fp16 outputs leave through LDS as whole lines, each wave's tile in a region of its own; where the stages are
     // smaller than that (the narrowest operand pairs), the launch asks for the larger of the two, as long as the
     // workgroups that share a compute unit still fit
+    constexpr int SBUF = WK * BUF_BYTES;                       // a stage: the K tiles of all K groups
     constexpr int F16_LDS = WM * WN * WaveTileF16<TM, TN>::kBytes;
-    constexpr int LDS_BYTES = StagedOutputLds<TM, TN, WM, WN, S * BUF_BYTES>::value;
+    constexpr int LDS_BYTES = StagedOutputLds<TM, TN, WM, WN, S * SBUF>::value;
+    static_assert(WK == 1 || NW * TM * TN * 4096 <= S * SBUF, "the K groups' partial tiles meet in the stages");
     constexpr bool F16_VIA_LDS = F16_LDS <= LDS_BYTES;
 
     extern __shared__ __align__(16) unsigned char smem[]; // [S][BM rows of X | BN rows of W]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wk = WK > 1 ? wave / NW : 0;   // K group
+    const int wid = WK > 1 ? wave % NW : wave; // wave within its K group
     const int wm = wid / WN, wn = wid % WN;
     const int r = lane & 31, g = lane >> 5;
     const int M = __builtin_amdgcn_readfirstlane(a.M), N = __builtin_amdgcn_readfirstlane(a.N);
-    const int ktiles = __builtin_amdgcn_readfirstlane(a.K) / 128;
+    const int ktot = __builtin_amdgcn_readfirstlane(a.K) / 128;         // K tiles
+    const int ktiles = (ktot + WK - 1) / WK;                            // trips of the K loop: a K tile per group
 
     int mb, nb;
     tile_of_workgroup(blockIdx.x, m_blocks, n_blocks_per_xcd, &mb, &nb);
@@ -208,7 +223,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     // offset counts bytes from the start of w_scale to the row's scale of K tile 0.
     const int sc_block = wid % (BN / 64 > 0 ? BN / 64 : 1);
     if constexpr (GROUPED)
-        goff[NPR] = 4u * ((uint32_t)min(n0 + 64 * sc_block + lane, N - 1) * (uint32_t)ktiles);
+        goff[NPR] = 4u * ((uint32_t)min(n0 + 64 * sc_block + lane, N - 1) * (uint32_t)ktot);
     const size_t stride_a = (size_t)M * TA::kUnits, stride_b = (size_t)N * TB::kUnits;
     const unsigned lds0 = (unsigned)(size_t)smem; // LDS byte address of the first stage
 
@@ -222,8 +237,8 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
             for (int e = 0; e < 16; ++e)
                 acc[i][j][e] = 0;
 
-    unsigned char *lds_a = smem;
-    unsigned char *lds_b = smem + BM * TA::kRow;
+    unsigned char *lds_a = smem + wk * BUF_BYTES; // the K group's tile within a stage
+    unsigned char *lds_b = lds_a + BM * TA::kRow;
     int a_off[TA::kReads], b_off[TB::kReads];
 #pragma unroll
     for (int c = 0; c < TA::kReads; ++c)
@@ -265,13 +280,14 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     // The tile the next requests are for: its operands' records and its scales, all wave-uniform (scalar
     // registers), the lanes adding their 32-bit offsets.  Tiles past the end are copies of the last, into stages
     // nobody reads.
-    const v4u *xq = xt, *wq = wt;
-    const float *sq = a.w_scale;
-    const unsigned lds_wave = lds0 + wid * 1024;
+    const int first = min(wk, ktot - 1); // (a group beyond the last K tile never has one of its own)
+    const v4u *xq = xt + first * stride_a, *wq = wt + first * stride_b;
+    const float *sq = a.w_scale + first;
+    const unsigned lds_wave = lds0 + wk * BUF_BYTES + wid * 1024;
     int kq = 0;
     auto request = [&](int stage, int i) {
         if (GROUPED && i == NPR) {
-            staged_load_dword_to_lds(sq, goff[i], lds0 + stage + SC_OFF + sc_block * 256);
+            staged_load_dword_to_lds(sq, goff[i], lds0 + wk * BUF_BYTES + stage + SC_OFF + sc_block * 256);
             return;
         }
         int q = wid + NW * i;
@@ -282,10 +298,10 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         staged_load_to_lds(activations ? (const void *)xq : (const void *)wq, goff[i], lds_wave + stage + (q - wid) * 1024);
     };
     auto next_tile = [&]() {
-        if (kq < ktiles - 1) {
-            xq += stride_a;
-            wq += stride_b;
-            sq += 1;
+        if ((kq + 1) * WK + wk < ktot) {
+            xq += WK * stride_a;
+            wq += WK * stride_b;
+            sq += WK;
         }
         ++kq;
     };
@@ -298,7 +314,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     for (int s = 0; s < S; ++s) {
 #pragma unroll
         for (int i = 0; i < NPW; ++i)
-            request(s * BUF_BYTES, i);
+            request(s * SBUF, i);
         next_tile();
     }
     staged_wait_loads<NPW * (S - 1)>();
@@ -312,10 +328,13 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     v16f facc[GROUPED ? TM : 1][GROUPED ? TN : 1];
     float sc_cur[TN], sc_next[TN], sc_last = 0.f;
     const float unshift = FP6 ? 64.0f : SIGNED ? 1.0f / (float)(1 << (16 - QB - PB)) : 1.0f; // FP6: both operands carry 1/8 as their unit
+    int kr = 0; // trip whose scales are read next
     auto read_scales = [&](float(&sc)[TN], int stage) {
+        const float f = (WK == 1 || kr * WK + wk < ktot) ? unshift : 0.f; // a trip in which the group has no K tile
+        ++kr;
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-            sc[j] = *reinterpret_cast<const float *>(smem + stage + SC_OFF + (wn * 32 * TN + j * 32 + r) * 4) * unshift;
+            sc[j] = *reinterpret_cast<const float *>(lds_a + stage + SC_OFF + (wn * 32 * TN + j * 32 + r) * 4) * f;
     };
     if constexpr (GROUPED) {
 #pragma unroll
@@ -331,16 +350,17 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     __syncthreads();
 
     int st_req = 0;         // stage the next request goes to: the one tile t occupied
-    int st_rd = BUF_BYTES;  // stage of tile t + 1
+    int st_rd = SBUF;       // stage of tile t + 1
     // One K tile.  On entry every wave's share of tile KT + 1 has landed (wait + barrier at the end of
     // the previous tile), and the fragment set QC holds tile KT.  The wave's load requests and LDS reads
     // are dealt out between its MFMAs: a wave issues in order, and a burst of requests at the top of
     // the tile would hold its MFMAs back until the load unit and the LDS have taken the whole burst.
-#define ABQ_STAGED_K_TILE(KT, QC, QN)                                                                           \
+#define ABQ_STAGED_K_TILE(KT, QC, QN, LIVE)                                                                     \
     {                                                                                                           \
         _Pragma("unroll") for (int k = 0; k < NM; ++k)                                                          \
         {                                                                                                       \
-            mfma(acc[(k / TN) % TM][k % TN], QC, (k / TN) % TM, k % TN, k / (TM * TN));                         \
+            if (LIVE)                                                                                           \
+                mfma(acc[(k / TN) % TM][k % TN], QC, (k / TN) % TM, k % TN, k / (TM * TN));                     \
             _Pragma("unroll") for (int d = k * NPW / NM; d < (k + 1) * NPW / NM; ++d)                           \
                 request(st_req, d);                                                                             \
             _Pragma("unroll") for (int p = k * NR / NM; p < (k + 1) * NR / NM; ++p)                             \
@@ -348,8 +368,8 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
             __builtin_amdgcn_sched_barrier(0);                                                                  \
         }                                                                                                       \
         next_tile();                                                                                            \
-        st_req = st_req + BUF_BYTES == S * BUF_BYTES ? 0 : st_req + BUF_BYTES;                                  \
-        st_rd = st_rd + BUF_BYTES == S * BUF_BYTES ? 0 : st_rd + BUF_BYTES;                                     \
+        st_req = st_req + SBUF == S * SBUF ? 0 : st_req + SBUF;                                                 \
+        st_rd = st_rd + SBUF == S * SBUF ? 0 : st_rd + SBUF;                                                    \
         staged_wait_loads<NPW * (S - 2)>(); /* tile KT + 2 has landed; the S - 2 younger ones may still fly */  \
         __syncthreads();                                                                                        \
     }
@@ -379,8 +399,8 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                          \
             sc_cur[j] = sc_next[j];                                                                             \
         next_tile();                                                                                            \
-        st_req = st_req + BUF_BYTES == S * BUF_BYTES ? 0 : st_req + BUF_BYTES;                                  \
-        st_rd = st_rd + BUF_BYTES == S * BUF_BYTES ? 0 : st_rd + BUF_BYTES;                                     \
+        st_req = st_req + SBUF == S * SBUF ? 0 : st_req + SBUF;                                                 \
+        st_rd = st_rd + SBUF == S * SBUF ? 0 : st_rd + SBUF;                                                    \
         staged_wait_loads<NPW * (S - 2)>();                                                                     \
         __syncthreads();                                                                                        \
     }
@@ -393,13 +413,28 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         }
         if (kt < ktiles)
             ABQ_STAGED_K_TILE_G(kt, q0, q1)
-    } else {
+    } else if constexpr (WK == 1) {
         for (; kt + 2 <= ktiles; kt += 2) {
-            ABQ_STAGED_K_TILE(kt, q0, q1)
-            ABQ_STAGED_K_TILE(kt + 1, q1, q0)
+            ABQ_STAGED_K_TILE(kt, q0, q1, true)
+            ABQ_STAGED_K_TILE(kt + 1, q1, q0, true)
         }
         if (kt < ktiles)
-            ABQ_STAGED_K_TILE(kt, q0, q1)
+            ABQ_STAGED_K_TILE(kt, q0, q1, true)
+    } else {
+        // the trips in which every group has a K tile, then the one in which only the first ktot % WK groups do
+        const int full = ktot / WK;
+        const bool live = full * WK + wk < ktot; // wave-uniform
+        for (; kt + 2 <= full; kt += 2) {
+            ABQ_STAGED_K_TILE(kt, q0, q1, true)
+            ABQ_STAGED_K_TILE(kt + 1, q1, q0, true)
+        }
+        if (kt < full) {
+            ABQ_STAGED_K_TILE(kt, q0, q1, true)
+            if (full < ktiles)
+                ABQ_STAGED_K_TILE(kt + 1, q1, q0, live)
+        } else if (full < ktiles) {
+            ABQ_STAGED_K_TILE(kt, q0, q1, live)
+        }
     }
 #undef ABQ_STAGED_K_TILE
 #undef ABQ_STAGED_K_TILE_G
@@ -410,6 +445,54 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
 #pragma unroll
         for (int e = 0; e < 16; ++e)
             facc[TM - 1][TN - 1][e] += (float)acc[TM - 1][TN - 1][e] * sc_last;
+    }
+    if constexpr (WK > 1) {
+        // The K groups' partial tiles: group 1, 2, .. in turn leave theirs in LDS (lane-contiguous 16-byte pieces,
+        // the place of the stages, which nobody reads any more) and group 0 adds them; the other groups are done
+        // then (a barrier waits for the waves of a workgroup that have not ended).
+        v4u *red = reinterpret_cast<v4u *>(smem) + (wid * TM * TN * 4) * 64 + lane;
+        for (int kg = 1; kg < WK; ++kg) {
+            __syncthreads();
+            if (wk == kg) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            v4u v;
+#pragma unroll
+                            for (int c = 0; c < 4; ++c)
+                                v[c] = GROUPED ? __float_as_uint(facc[GROUPED ? i : 0][GROUPED ? j : 0][4 * e + c])
+                                               : (FP6 ? __float_as_uint((float)acc[i][j][4 * e + c]) : (uint32_t)acc[i][j][4 * e + c]);
+                            red[((i * TN + j) * 4 + e) * 64] = v;
+                        }
+            }
+            __syncthreads();
+            if (wk == 0) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const v4u v = red[((i * TN + j) * 4 + e) * 64];
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) {
+                                if constexpr (GROUPED)
+                                    facc[GROUPED ? i : 0][GROUPED ? j : 0][4 * e + c] += __uint_as_float(v[c]);
+                                else if constexpr (FP6)
+                                    acc[i][j][4 * e + c] += __uint_as_float(v[c]);
+                                else
+                                    acc[i][j][4 * e + c] += (int)v[c];
+                            }
+                        }
+            }
+        }
+        if (wk != 0)
+            return;
+    }
+    if constexpr (GROUPED) {
         group_scale_epilogue<TM, TN, WM, WN, LDS_BYTES>(a, facc, smem, M, N, m0, n0, wm, wn, r, g, tid);
         return;
     }
@@ -491,20 +574,20 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
 
 // LDS stages of a tile: as many (up to four) as leave room for the workgroups that share a compute
 // unit: two for the four-wave tiles when three stages of theirs fit twice, else one.
-template <int QB, int PB, bool FP6, int TM, int TN, int WM, int WN, bool GROUPED = false> struct StagedStages {
-    static constexpr int kBuf = 32 * (TM * WM * StagedOperand<QB, FP6>::kRow + TN * WN * StagedOperand<PB, FP6>::kRow) +
-                                (GROUPED ? (32 * TN * WN > 128 ? 128 * TN * WN : 512) : 0);
+template <int QB, int PB, bool FP6, int TM, int TN, int WM, int WN, bool GROUPED = false, int WK = 1> struct StagedStages {
+    static constexpr int kBuf = WK * (32 * (TM * WM * StagedOperand<QB, FP6>::kRow + TN * WN * StagedOperand<PB, FP6>::kRow) +
+                                      (GROUPED ? (32 * TN * WN > 128 ? 128 * TN * WN : 512) : 0));
     static constexpr int value = (WM * WN <= 4 && TM * TN <= 4 && 2 * 4 * kBuf > 160 * 1024 && 2 * 3 * kBuf <= 160 * 1024) ? 3
                                  : (4 * kBuf <= 160 * 1024 ? 4 : 3);
     static constexpr size_t kLds = (size_t)value * kBuf;
     static_assert(3 * kBuf <= 160 * 1024, "three stages fit a compute unit's LDS");
 };
 
-template <int QB, int PB, bool SIGNED, bool FP6, int TM, int TN, int WM, int WN, bool GROUPED = false>
+template <int QB, int PB, bool SIGNED, bool FP6, int TM, int TN, int WM, int WN, bool GROUPED = false, int WK = 1>
 static hipError_t launch_mfma_staged(const GemmArgs &a, hipStream_t stream)
 {
     constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
-    using Stages = StagedStages<QB, PB, FP6, TM, TN, WM, WN, GROUPED>;
+    using Stages = StagedStages<QB, PB, FP6, TM, TN, WM, WN, GROUPED, WK>;
     constexpr int S = Stages::value;
     if (GROUPED && a.group_size != 128)
         return hipErrorInvalidValue; // one scale per K tile
@@ -512,13 +595,13 @@ static hipError_t launch_mfma_staged(const GemmArgs &a, hipStream_t stream)
     const int npx = (n_blocks + 7) / 8;
     const dim3 grid(8 * npx * m_blocks);
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S, GROUPED>),
+        reinterpret_cast<const void *>(&gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S, GROUPED, WK>),
         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess)
         return attr;
     // int32 results are stored from the registers; every other kind goes through LDS
     const size_t lds = a.out_kind == 0 ? Stages::kLds : (size_t)StagedOutputLds<TM, TN, WM, WN, (int)Stages::kLds>::value;
-    hipLaunchKernelGGL((gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S, GROUPED>), grid, dim3(64 * WM * WN), lds,
+    hipLaunchKernelGGL((gemm_mfma_staged<QB, PB, SIGNED, FP6, TM, TN, WM, WN, S, GROUPED, WK>), grid, dim3(64 * WM * WN * WK), lds,
                        stream, a, reinterpret_cast<const v4u *>(a.X), reinterpret_cast<const v4u *>(a.W), m_blocks, npx);
     return hipGetLastError();
 }

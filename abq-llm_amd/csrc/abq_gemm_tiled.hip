@@ -490,10 +490,16 @@ static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 #define ABQ_SENTRY(SG, TM, TN, WM, WN)                                                       \
     { 32, TM, TN, WM, WN, 1, 4, &launch_mfma_staged<ABQ_Q, ABQ_P, SG, false, TM, TN, WM, WN>, 128, \
       StagedStages<ABQ_Q, ABQ_P, false, TM, TN, WM, WN>::kLds },
+// The small tiles with two groups of waves that split K inside the workgroup (small grids).
+#define ABQ_SENTRY_K(SG, TM, TN, WM, WN, WK)                                                            \
+    { 32, TM, TN, WM, WN, WK, 4, &launch_mfma_staged<ABQ_Q, ABQ_P, SG, false, TM, TN, WM, WN, false, WK>, 128, \
+      StagedStages<ABQ_Q, ABQ_P, false, TM, TN, WM, WN, false, WK>::kLds },
+#define ABQ_STAGED_KSPLIT(SG) ABQ_SENTRY_K(SG, 1, 1, 2, 2, 2) ABQ_SENTRY_K(SG, 2, 1, 2, 2, 2)
 // Activations wider than the weights: a 128 x 256 tile (eight waves of 64 x 64, 2 along M, 4 along N) moves fewer
 // bytes per MFMA than 256 x 128, since a row of activations is the longer record.
 #if ABQ_Q > ABQ_P
-#define ABQ_STAGED_WIDE_N(SG) ABQ_SENTRY(SG, 2, 2, 2, 4)
+// ... and for small grids a 64 x 128 tile (four waves of 32 x 64), plain and with two groups of waves that split K.
+#define ABQ_STAGED_WIDE_N(SG) ABQ_SENTRY(SG, 2, 2, 2, 4) ABQ_SENTRY(SG, 1, 2, 2, 2) ABQ_SENTRY_K(SG, 1, 2, 2, 2, 2)
 #define ABQ_STAGED_WIDE_N_GROUPED(SG) ABQ_SGENTRY(SG, 2, 2, 2, 4)
 #else
 #define ABQ_STAGED_WIDE_N(SG)
@@ -510,12 +516,12 @@ static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 static const KernelEntry kSigned[] = { ABQ_ENTRY_T(4, 4) ABQ_ENTRY_T(2, 4) ABQ_SENTRY(true, 2, 2, 2, 2) ABQ_SENTRY(true, 2, 1, 2, 2)
                                        ABQ_SENTRY(true, 1, 1, 2, 2) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_T)
                                        ABQ_SENTRY(true, 2, 2, 4, 2) ABQ_WENTRY_T(2, 2, 4, 4) ABQ_STAGED_256(true)
-                                       ABQ_STAGED_WIDE_N(true) };
+                                       ABQ_STAGED_WIDE_N(true) ABQ_STAGED_KSPLIT(true) };
 #if ABQ_Q < 8 && ABQ_P < 8
 static const KernelEntry kUnsigned[] = { ABQ_ENTRY_F(4, 4) ABQ_ENTRY_F(2, 4) ABQ_SENTRY(false, 2, 2, 2, 2) ABQ_SENTRY(false, 2, 1, 2, 2)
                                          ABQ_SENTRY(false, 1, 1, 2, 2) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
                                          ABQ_SENTRY(false, 2, 2, 4, 2) ABQ_WENTRY_F(2, 2, 4, 4) ABQ_STAGED_256(false)
-                                         ABQ_STAGED_WIDE_N(false) };
+                                         ABQ_STAGED_WIDE_N(false) ABQ_STAGED_KSPLIT(false) };
 #else
 static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
                                          ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_F) };
@@ -532,11 +538,17 @@ static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TIL
 #define ABQ_SGENTRY(SG, TM, TN, WM, WN)                                                                  \
     { 32, TM, TN, WM, WN, 1, 4, &launch_mfma_staged<ABQ_Q, ABQ_P, SG, false, TM, TN, WM, WN, true>, 128, \
       StagedStages<ABQ_Q, ABQ_P, false, TM, TN, WM, WN, true>::kLds },
+// (the 128 x 64 tile also with two groups of waves that split K, for small grids)
+#define ABQ_SGENTRY_K(SG, TM, TN, WM, WN, WK)                                                                  \
+    { 32, TM, TN, WM, WN, WK, 4, &launch_mfma_staged<ABQ_Q, ABQ_P, SG, false, TM, TN, WM, WN, true, WK>, 128, \
+      StagedStages<ABQ_Q, ABQ_P, false, TM, TN, WM, WN, true, WK>::kLds },
 #if ABQ_Q == 8 && ABQ_P == 8
 // two fragment sets of 64x64 8-bit operands, the int32 and the fp32 accumulators do not fit 256 registers
-#define ABQ_STAGED_GROUPED(SG) ABQ_SGENTRY(SG, 2, 1, 2, 2)
+#define ABQ_STAGED_GROUPED(SG) ABQ_SGENTRY(SG, 2, 1, 2, 2) ABQ_SGENTRY_K(SG, 2, 1, 2, 2, 2)
 #else
-#define ABQ_STAGED_GROUPED(SG) ABQ_SGENTRY(SG, 2, 2, 4, 2) ABQ_SGENTRY(SG, 2, 2, 2, 2) ABQ_SGENTRY(SG, 2, 1, 2, 2) ABQ_STAGED_WIDE_N_GROUPED(SG)
+#define ABQ_STAGED_GROUPED(SG)                                                                                          \
+    ABQ_SGENTRY(SG, 2, 2, 4, 2) ABQ_SGENTRY(SG, 2, 2, 2, 2) ABQ_SGENTRY(SG, 2, 1, 2, 2) ABQ_STAGED_WIDE_N_GROUPED(SG) \
+    ABQ_SGENTRY_K(SG, 2, 1, 2, 2, 2)
 #endif
 static const KernelEntry kSignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_T) ABQ_STAGED_GROUPED(true) };
 #if ABQ_Q < 8 && ABQ_P < 8

@@ -203,6 +203,16 @@ std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits, bool is_signed)
         const bool field = (x_bits == 2 || x_bits == 4 || x_bits == 8) && (w_bits == 2 || w_bits == 4 || w_bits == 8);
         if (field && x_bits > w_bits && (is_signed || x_bits < 8))
             out.push_back(Tile{ 128, 256, 128, 64, 64, 128, 32, 32, 32, 2, 4, { 4 } });
+        // small grids on the staged kernel: two groups of waves that split K inside the workgroup (64 x 64 and
+        // 128 x 64), and a 64 x 128 tile, plain and split, where an activation row is the longer record
+        if (field && (is_signed || (x_bits < 8 && w_bits < 8))) {
+            out.push_back(Tile{ 64, 64, 256, 32, 32, 128, 32, 32, 32, 2, 4, { 4 } });
+            out.push_back(Tile{ 128, 64, 256, 64, 32, 128, 32, 32, 32, 2, 4, { 4 } });
+        }
+        if (field && x_bits > w_bits && (is_signed || x_bits < 8)) {
+            out.push_back(Tile{ 64, 128, 128, 32, 64, 128, 32, 32, 32, 2, 2, { 4 } });
+            out.push_back(Tile{ 64, 128, 256, 32, 64, 128, 32, 32, 32, 2, 4, { 4 } });
+        }
     }
     const int half[][2] = { { 2, 4 }, { 2, 2 } };
     for (const auto &t : half)

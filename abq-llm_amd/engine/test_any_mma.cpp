@@ -257,7 +257,7 @@ int sweep_group_scales(int M, int N, int K, int x_bits, int w_bits, bool is_sign
             continue; // no group-scale build of this tile
         const abq_tile_config &c = states[0].cfg;
         char key[96];
-        std::snprintf(key, sizeof key, "%d %d %d %d %d %zu", c.block_m, c.block_n, c.warp_m, c.warp_n, c.nstage, states[0].shared_mem_size);
+        std::snprintf(key, sizeof key, "%d %d %d %d %d %d %zu", c.block_m, c.block_n, c.block_k, c.warp_m, c.warp_n, c.nstage, states[0].shared_mem_size);
         if (!library_default) {
             if (std::find(seen.begin(), seen.end(), key) != seen.end())
                 continue; // tuples that resolve to the same group-scale kernel

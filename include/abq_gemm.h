@@ -82,7 +82,9 @@ abq_status abq_pack_f16(const void *in_f16, const float *scale_dev, uint32_t *pl
  *                 (NSTAGE = 3: decode kernel, activations staged in LDS; NSTAGE = 2: every wave
  *                 expands its own activations; NSTAGE = 6: decode kernel on K-tiled operands,
  *                 BN / 16 weight tiles per workgroup, WK = K elements a wave keeps in flight)
- *   32 x 32 x 32  the same feeding v_mfma_i32_32x32x32_i8
+ *   32 x 32 x 32  the same feeding v_mfma_i32_32x32x32_i8 (NSTAGE = 4: LDS-staged kernels on K-tiled
+ *                 operands, WK = 128 (or 64) = K elements per LDS stage and group of waves; BK = 2 WK:
+ *                 two groups of waves share the tile and split K between them, for small grids)
  * Any other triple (the reference's 8x8x128, 16x8x128, 16x8x256 tensor-core shapes) asks the
  * library to choose strategy and tile itself from (bits, M, N, K).
  * ------------------------------------------------------------------------------------- */

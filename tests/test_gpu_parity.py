@@ -178,7 +178,8 @@ def test_relayout_planes_matches_closed_form(abq, oracle):
 def test_tiled_kernels_with_prepared_operands(abq, oracle):
     """K-tiled kernels fed tiled activations and/or tiled weights directly, ragged shapes."""
     rng = np.random.default_rng(13)
-    for q, p, signed, M, N, K in [(8, 2, True, 300, 200, 640), (4, 4, False, 70, 513, 1152), (8, 8, False, 257, 129, 384)]:
+    for q, p, signed, M, N, K in [(8, 2, True, 300, 200, 640), (4, 4, False, 70, 513, 1152), (8, 8, False, 257, 129, 384),
+                                  (8, 4, True, 130, 200, 768), (8, 8, True, 70, 129, 128)]:
         x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
         xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
         xt, wt = abq.relayout_planes(xd), abq.relayout_planes(wd)

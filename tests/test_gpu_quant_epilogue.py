@@ -446,6 +446,7 @@ def _staged_grouped_lds(cfg):
     """LDS of the staged kernel's group-scale variant for a tile: 3 or 4 stages of the packed records
     (16 bytes per bit of width per row and K tile) plus the tile's scales (at least 512 bytes) each."""
     buf = 16 * (cfg.block_m * cfg.x_bits + cfg.block_n * cfg.w_bits) + max(512, 4 * cfg.block_n)
+    buf *= cfg.block_k // cfg.warp_k  # groups of waves that split K: a stage holds a K tile for each
     two_per_cu = cfg.block_m * cfg.block_n <= 128 * 128 and 2 * 4 * buf > 160 * 1024 >= 2 * 3 * buf
     return buf * (3 if two_per_cu or 4 * buf > 160 * 1024 else 4)
 
@@ -465,9 +466,10 @@ def test_group_scale_staged_kernel_every_tile(abq, oracle, q, p, signed):
     if (q, p) == (8, 8):
         tiles = [c for c in tiles if (c.block_m, c.block_n) == (128, 64)]
     assert tiles
+    assert [c.block_k for c in tiles if (c.block_m, c.block_n) == (128, 64)] == [128, 256]  # plain, and waves that split K
     lo_x, hi_x = (-(1 << (q - 1)), 1 << (q - 1)) if signed else (0, 1 << q)
     lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed else (0, 1 << p)
-    for (M, N, K) in [(300, 200, 640), (70, 330, 256), (129, 65, 128)]:
+    for (M, N, K) in [(300, 200, 640), (70, 330, 256), (129, 65, 128), (200, 136, 1536)]:
         G = K // 128
         x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
         w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
@@ -483,7 +485,8 @@ def test_group_scale_staged_kernel_every_tile(abq, oracle, q, p, signed):
         xt, wt = abq.relayout_planes(planes_dev(oracle.pack_i32(x, q))), abq.relayout_planes(wp)
         for cfg in tiles:
             g = abq.Gemm(xt, wt, signed, cfg=cfg, out_kind=abq.OUT_F16_SCALED, x_tiled=True, w_tiled=True, **kw)
-            assert g.strategy == "tiled" and (g.state.cfg.block_m, g.state.cfg.block_n) == (cfg.block_m, cfg.block_n)
+            assert g.strategy == "tiled" and (g.state.cfg.block_m, g.state.cfg.block_n, g.state.cfg.block_k) == (
+                cfg.block_m, cfg.block_n, cfg.block_k)
             assert g.state.shared_mem_size == _staged_grouped_lds(cfg), (g.config_name, g.state.shared_mem_size)
             got = g.run()
             torch.cuda.synchronize()

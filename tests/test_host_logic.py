@@ -418,36 +418,44 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
             assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, group) == 0
         assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), layout, layout) == 0
         c = st.cfg
-        return (c.block_m, c.block_n, c.warp_m, c.warp_n, c.nstage)
+        return (c.block_m, c.block_n, c.block_k, c.warp_m, c.warp_n, c.nstage)
 
     T, F6 = abq.LAYOUT_TILED, abq.LAYOUT_FP6
     # W4A4 on the FP6 route: 128x128 from a chip's worth of tiles up
-    assert picked(4, 4, 512, 4096, 4096, F6) == (64, 64, 32, 32, 5)
-    assert picked(4, 4, 512, 11008, 4096, F6) == (128, 128, 64, 64, 5)
-    assert picked(4, 4, 2048, 12288, 4096, F6) == (128, 128, 64, 64, 5)
-    assert picked(4, 4, 16384, 4096, 4096, F6) == (128, 128, 64, 64, 5)
+    assert picked(4, 4, 512, 4096, 4096, F6) == (64, 64, 128, 32, 32, 5)
+    assert picked(4, 4, 512, 11008, 4096, F6) == (128, 128, 128, 64, 64, 5)
+    assert picked(4, 4, 2048, 12288, 4096, F6) == (128, 128, 128, 64, 64, 5)
+    assert picked(4, 4, 16384, 4096, 4096, F6) == (128, 128, 128, 64, 64, 5)
     # W2A8: 256x256 only where its grid is whole rounds of the chip
-    assert picked(8, 2, 2048, 4096, 4096, T) == (128, 128, 64, 64, 4)
-    assert picked(8, 2, 4096, 11008, 4096, T) == (128, 128, 64, 64, 4)       # 688 tiles of 256x256: a third round mostly empty
-    assert picked(8, 2, 4096, 4096, 4096, T) == (256, 256, 64, 128, 4)
-    assert picked(8, 2, 8192, 4096, 4096, T) == (256, 256, 64, 128, 4)
-    assert picked(8, 2, 512, 4096, 4096, T) == (64, 64, 32, 32, 4)
+    assert picked(8, 2, 2048, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)
+    assert picked(8, 2, 4096, 11008, 4096, T) == (128, 128, 128, 64, 64, 4)       # 688 tiles of 256x256: a third round mostly empty
+    assert picked(8, 2, 4096, 4096, 4096, T) == (256, 256, 128, 64, 128, 4)
+    assert picked(8, 2, 8192, 4096, 4096, T) == (256, 256, 128, 64, 128, 4)
+    # small grids: two groups of waves split K inside the workgroup, and the tile lies along N where an activation
+    # row is the longer record (also up to 400 tiles of 128x128, without the split)
+    assert picked(8, 2, 512, 4096, 4096, T) == (64, 128, 256, 32, 64, 4)
+    assert picked(8, 2, 256, 4096, 4096, T) == (64, 64, 256, 32, 32, 4)
+    assert picked(4, 4, 512, 4096, 4096, T) == (128, 64, 256, 64, 32, 4)
+    assert picked(8, 2, 512, 11008, 4096, T) == (64, 128, 128, 32, 64, 4)
+    assert picked(8, 2, 1024, 4096, 4096, T) == (64, 128, 128, 32, 64, 4)
+    assert picked(4, 4, 1024, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)
     # signed W8A8: 256x128 as soon as it fills the chip
-    assert picked(8, 8, 2048, 4096, 4096, T) == (256, 128, 64, 64, 4)
-    assert picked(8, 8, 1024, 4096, 4096, T) == (128, 128, 64, 64, 4)
-    assert picked(8, 8, 512, 11008, 4096, T) == (256, 128, 64, 64, 4)
-    assert picked(8, 8, 4096, 4096, 4096, T) == (256, 128, 64, 64, 4)
+    assert picked(8, 8, 2048, 4096, 4096, T) == (256, 128, 128, 64, 64, 4)
+    assert picked(8, 8, 1024, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)
+    assert picked(8, 8, 512, 11008, 4096, T) == (256, 128, 128, 64, 64, 4)
+    assert picked(8, 8, 4096, 4096, 4096, T) == (256, 128, 128, 64, 64, 4)
     # group scales (the decoder-layer linears): 128x128 once it fills the chip, 128x64 below
-    assert picked(8, 2, 1024, 12288, 4096, T, group=128) == (128, 128, 64, 64, 4)
-    assert picked(8, 2, 1024, 4096, 4096, T, group=128) == (128, 64, 64, 32, 4)
-    assert picked(8, 2, 16384, 22016, 4096, T, group=128) == (128, 128, 64, 64, 4)
-    assert picked(8, 2, 128, 4096, 4096, T, group=64) == (64, 64, 32, 32, 4)
+    assert picked(8, 2, 1024, 12288, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
+    assert picked(8, 2, 1024, 4096, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
+    assert picked(8, 2, 16384, 22016, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
+    assert picked(8, 2, 128, 4096, 4096, T, group=64) == (64, 64, 128, 32, 32, 4)
+    assert picked(8, 2, 512, 4096, 4096, T, group=128) == (128, 64, 256, 64, 32, 4)   # small grid: waves split K
     # ... activations of at most 4 bits keep 128x64 up to 400 tiles
-    assert picked(4, 4, 512, 11008, 4096, T, group=128) == (128, 64, 64, 32, 4)
-    assert picked(8, 2, 512, 11008, 4096, T, group=128) == (128, 128, 64, 64, 4)
-    assert picked(4, 4, 2048, 4096, 4096, T, group=128) == (128, 128, 64, 64, 4)
+    assert picked(4, 4, 512, 11008, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
+    assert picked(8, 2, 512, 11008, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
+    assert picked(4, 4, 2048, 4096, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
     # group scales on FP6 records: 256x128 where its rounds of workgroups come out even
-    assert picked(4, 4, 2048, 4096, 4096, F6, group=128) == (256, 128, 64, 64, 5)
-    assert picked(4, 4, 1024, 11008, 4096, F6, group=128) == (128, 128, 64, 64, 5)   # 344 tiles of 256x128: 1.3 rounds
-    assert picked(4, 4, 16384, 4096, 11008, F6, group=128) == (256, 128, 64, 64, 5)
-    assert picked(4, 4, 1024, 4096, 4096, F6, group=128) == (128, 64, 64, 32, 5)
+    assert picked(4, 4, 2048, 4096, 4096, F6, group=128) == (256, 128, 128, 64, 64, 5)
+    assert picked(4, 4, 1024, 11008, 4096, F6, group=128) == (128, 128, 128, 64, 64, 5)   # 344 tiles of 256x128: 1.3 rounds
+    assert picked(4, 4, 16384, 4096, 11008, F6, group=128) == (256, 128, 128, 64, 64, 5)
+    assert picked(4, 4, 1024, 4096, 4096, F6, group=128) == (128, 64, 128, 64, 32, 5)
