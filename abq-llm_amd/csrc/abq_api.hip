@@ -801,13 +801,13 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
         // W2A8 and W4A4, M = 256 .. 2048 on the LLaMA-7B widths: 5-12 % below 200 tiles, 2-9 % on 64x128 up to 400
         // (W2A2 7-12 %, W4A8 1-5 %; W8A8, whose tiles are all LDS traffic, -5 .. +4 %: left as it was).
         const long t128 = (long)((st->M + 127) / 128) * ((st->N + 127) / 128);
-        const long n128x64 = (long)((st->M + 127) / 128) * ((st->N + 63) / 64);
+        const long n64x64 = (long)((st->M + 63) / 64) * ((st->N + 63) / 64);
         const bool along_n = c.x_bits > c.w_bits;
         int want[5] = { 0, 0, 2, 2, 0 }; // TM, TN, waves along M and N, K groups
         if (tt->entries[pick].lds != 0 && t128 < 200 && c.x_bits + c.w_bits < 16) {
             want[4] = 2;
-            want[0] = n128x64 < 256 ? 1 : along_n ? 1 : 2;
-            want[1] = n128x64 < 256 ? 1 : along_n ? 2 : 1;
+            want[0] = n64x64 <= 256 ? 1 : along_n ? 1 : 2; // 64x64 up to one workgroup per compute unit
+            want[1] = n64x64 <= 256 ? 1 : along_n ? 2 : 1;
         } else if (tt->entries[pick].lds != 0 && along_n && t128 < 400 && tt->entries[pick].tm * tt->entries[pick].wm <= 4 &&
                    tt->entries[pick].tn * tt->entries[pick].wn <= 4) {
             want[4] = 1;
@@ -936,10 +936,17 @@ static bool decode_tiled_pays(int x_bits, int w_bits, int M, int N, int K)
     const double blocks = (M + mrows - 1) / mrows;
     const double w_mb = (double)N * K * w_bits / 8e6;
     const double x_mb = (double)((N + 16 * kDecodeTiledBlocksTiles - 1) / (16 * kDecodeTiledBlocksTiles)) * mrows * K * x_bits / 8e6;
-    const double per_block = x_bits == 8 ? 0.11 * (w_mb + x_mb) + 0.5 : 0.07 * (w_mb + x_mb) + 0.9;
-    const double decode_us = 0.8 + blocks * per_block;
+    // 8-bit activations: a block costs by the bytes it moves; narrower ones by the elements it multiplies (0.037 us per
+    // 10^6 for 16 rows: W4A4 64 x 4096 x 4096 5.7, 128 x 11008 x 4096 18.0; W2A2 128 x 4096 x 4096 7.5), half as much
+    // again for weights of 4 bits on long K
+    const double melems = (double)N * K / 1e6 * mrows / 16.0;
+    const double per_block = x_bits == 8 ? 0.11 * (w_mb + x_mb) + 0.5 : 0.037 * melems * (w_bits >= 4 && K > 8192 ? 1.5 : 1.0);
+    const double decode_us = (x_bits == 8 ? 0.8 : 2.7) + blocks * per_block;
+    // (all pairs but W8A8 run that tile with two groups of waves that split K: 4.5 + 0.13 us per K tile, e.g. W2A8
+    // 128 x 4096 x 11008 15.5 against 20.9 us)
     const long tiles64 = (long)((M + 63) / 64) * ((N + 63) / 64);
-    const double tiled_us = (2.3 + 0.23 * (K / 128)) * (tiles64 > 256 ? 1.35 : 1.0);
+    const int kt = K / 128;
+    const double tiled_us = (x_bits + w_bits < 16 ? 4.5 + 0.13 * kt : 2.3 + 0.23 * kt) * (tiles64 > 256 ? 1.35 : 1.0);
     return decode_us < 0.9 * tiled_us;
 }
 
@@ -983,8 +990,8 @@ static abq_status switch_to_decode_tiled(abq_gemm_state *st)
 // Group scales on a decode-sized GEMM whose operands are (or are about to be declared) both prepared: whether the
 // decode kernel of that layout has a group-scale variant for the pair that fits this shape.
 // The same weighing for the group-scale variant (one tile per workgroup, two with the SiLU gate), against the
-// group-scale prefill kernel, whose smallest grids (64 x 64 or 128 x 64 tiles) take 0.6 us per K tile whatever M is
-// and 1.45 times that once they exceed one workgroup per compute unit.  Fits to a sweep of W2A8, W4A8 and W4A4 with
+// group-scale prefill kernel, whose smallest grids (128 x 64 tiles) take 0.48 us per K tile whatever M is
+// and 0.6 x 1.45 once they exceed one workgroup per compute unit.  Fits to a sweep of W2A8, W4A8 and W4A4 with
 // zero points over M = 24 ... 128 on the LLaMA-7B linears (4096 x 4096, QKV, gate + up with the gate fused, down);
 // taken when estimated 15 % ahead: W2A8 32 x 4096 x 4096 8.3 against 20.1 us, 32 x 4096 x 11008 23.2 against 48.8,
 // W4A4 32 x 12288 x 4096 13.2 against 20.6; the wide outputs of the 8-bit activations stay on the prefill kernel.
@@ -1003,8 +1010,9 @@ static bool decode_tiled_grouped_pays(int x_bits, int w_bits, int M, int N, int 
     const double x_mb = (double)((N + 16 * t - 1) / (16 * t)) * mrows * K * x_bits / 8e6;
     const double per_block = x_bits == 8 ? 0.165 * (w_mb + x_mb) : 0.11 * (w_mb + x_mb) + 0.7;
     const double decode_us = 1.0 + blocks * per_block;
+    // (up to one workgroup per compute unit the prefill kernel's waves split K: 0.48 us per K tile)
     const long wgs = (long)((N + 63) / 64) * ((M + 127) / 128);
-    const double tiled_us = 1.0 + 0.6 * (K / 128) * (wgs > 256 ? 1.45 : 1.0);
+    const double tiled_us = 1.0 + (wgs > 256 ? 0.6 * 1.45 : 0.48) * (K / 128);
     return decode_us < 0.85 * tiled_us;
 }
 
@@ -1049,14 +1057,20 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
         for (const auto &o : order) {
             if (pick >= 0 || t128 < o[2])
                 continue;
-            // below 200 tiles two groups of waves split K inside the workgroup where that is built (8-13 % on
-            // 256 and 512 rows of the LLaMA-7B widths, nothing from 1024 on)
-            const bool split = t128 < 200;
             for (int i = 0; i < tg->count; ++i) // the last match: the staged kernel's entry where there is one
                 if (usable(tg->entries[i]) && block_m(tg->entries[i]) == o[0] && block_n(tg->entries[i]) == o[1] &&
-                    (tg->entries[i].wk == 1 || (split && tg->entries[i].wk == 2)))
+                    tg->entries[i].wk == 1)
                     pick = i;
         }
+        // Grids of at most one 128x64 workgroup per compute unit: the tile whose two groups of waves split K (its
+        // stages fill a compute unit's LDS, so beyond 256 workgroups it would run in two rounds).  W2A8 with zero
+        // points: 4096 x 4096 64-512 rows 16-19 us against 19-21, 4096 x 11008 37-45 against 47-53, QKV up to 128
+        // rows 17.5 against 20.3; QKV at 192 rows (384 workgroups) 33 against 29: not taken there.
+        if ((long)((state->M + 127) / 128) * ((state->N + 63) / 64) <= 256)
+            for (int i = 0; i < tg->count; ++i)
+                if (usable(tg->entries[i]) && tg->entries[i].lds != 0 && block_m(tg->entries[i]) == 128 &&
+                    block_n(tg->entries[i]) == 64 && tg->entries[i].wk == 2)
+                    pick = i;
     } else {
         const int wk = c.warp_k > 0 ? c.block_k / c.warp_k : 1;
         for (int i = 0; i < tg->count; ++i)

@@ -449,7 +449,12 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(8, 2, 1024, 4096, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
     assert picked(8, 2, 16384, 22016, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
     assert picked(8, 2, 128, 4096, 4096, T, group=64) == (64, 64, 128, 32, 32, 4)
-    assert picked(8, 2, 512, 4096, 4096, T, group=128) == (128, 64, 256, 64, 32, 4)   # small grid: waves split K
+    # up to one 128x64 workgroup per compute unit: the tile whose waves split K (its stages fill a compute unit's LDS)
+    assert picked(8, 2, 512, 4096, 4096, T, group=128) == (128, 64, 256, 64, 32, 4)
+    assert picked(8, 2, 128, 4096, 11008, T, group=128) == (128, 64, 256, 64, 32, 4)
+    assert picked(8, 2, 128, 12288, 4096, T, group=128) == (128, 64, 256, 64, 32, 4)
+    assert picked(8, 2, 192, 12288, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)   # 384 workgroups: two rounds of it
+    assert picked(8, 2, 128, 22016, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
     # ... activations of at most 4 bits keep 128x64 up to 400 tiles
     assert picked(4, 4, 512, 11008, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
     assert picked(8, 2, 512, 11008, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
