@@ -1066,10 +1066,14 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
         // stages fill a compute unit's LDS, so beyond 256 workgroups it would run in two rounds).  W2A8 with zero
         // points: 4096 x 4096 64-512 rows 16-19 us against 19-21, 4096 x 11008 37-45 against 47-53, QKV up to 128
         // rows 17.5 against 20.3; QKV at 192 rows (384 workgroups) 33 against 29: not taken there.
-        if ((long)((state->M + 127) / 128) * ((state->N + 63) / 64) <= 256)
+        // Wider outputs of at most 64 rows, activations wider than the weights: the same along N (64x128: gate + up of
+        // LLaMA-7B, 22016 wide, at 32-64 rows 19.4 against 28.7 us).
+        const bool one_round = (long)((state->M + 127) / 128) * ((state->N + 63) / 64) <= 256;
+        const bool along_n = !one_round && state->M <= 64 && (state->N + 127) / 128 <= 256;
+        if (one_round || along_n)
             for (int i = 0; i < tg->count; ++i)
-                if (usable(tg->entries[i]) && tg->entries[i].lds != 0 && block_m(tg->entries[i]) == 128 &&
-                    block_n(tg->entries[i]) == 64 && tg->entries[i].wk == 2)
+                if (usable(tg->entries[i]) && tg->entries[i].lds != 0 && block_m(tg->entries[i]) == (one_round ? 128 : 64) &&
+                    block_n(tg->entries[i]) == (one_round ? 64 : 128) && tg->entries[i].wk == 2)
                     pick = i;
     } else {
         const int wk = c.warp_k > 0 ? c.block_k / c.warp_k : 1;

@@ -500,7 +500,7 @@ static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 #if ABQ_Q > ABQ_P
 // ... and for small grids a 64 x 128 tile (four waves of 32 x 64), plain and with two groups of waves that split K.
 #define ABQ_STAGED_WIDE_N(SG) ABQ_SENTRY(SG, 2, 2, 2, 4) ABQ_SENTRY(SG, 1, 2, 2, 2) ABQ_SENTRY_K(SG, 1, 2, 2, 2, 2)
-#define ABQ_STAGED_WIDE_N_GROUPED(SG) ABQ_SGENTRY(SG, 2, 2, 2, 4)
+#define ABQ_STAGED_WIDE_N_GROUPED(SG) ABQ_SGENTRY(SG, 2, 2, 2, 4) ABQ_SGENTRY(SG, 1, 2, 2, 2) ABQ_SGENTRY_K(SG, 1, 2, 2, 2, 2)
 #else
 #define ABQ_STAGED_WIDE_N(SG)
 #define ABQ_STAGED_WIDE_N_GROUPED(SG)

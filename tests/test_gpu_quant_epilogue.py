@@ -460,9 +460,10 @@ def test_group_scale_staged_kernel_every_tile(abq, oracle, q, p, signed):
     from oracle import quantizer as Q
     rng = np.random.default_rng(100 * q + 10 * p + signed)
     tiles = [c for c in abq.native_configs(q, p, signed)
-             if c.nstage == 4 and c.warp_k == 128 and (c.warp_m, c.warp_n) in ((64, 64), (64, 32)) and
-             (c.block_m, c.block_n) in ((256, 128), (128, 128), (128, 64), (128, 256))]
+             if c.nstage == 4 and c.warp_k == 128 and (c.warp_m, c.warp_n) in ((64, 64), (64, 32), (32, 64)) and
+             (c.block_m, c.block_n) in ((256, 128), (128, 128), (128, 64), (128, 256), (64, 128))]
     assert ((128, 256) in [(c.block_m, c.block_n) for c in tiles]) == (q > p)
+    assert [c.block_k for c in tiles if (c.block_m, c.block_n) == (64, 128)] == ([128, 256] if q > p else [])
     if (q, p) == (8, 8):
         tiles = [c for c in tiles if (c.block_m, c.block_n) == (128, 64)]
     assert tiles

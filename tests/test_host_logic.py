@@ -455,6 +455,8 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(8, 2, 128, 12288, 4096, T, group=128) == (128, 64, 256, 64, 32, 4)
     assert picked(8, 2, 192, 12288, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)   # 384 workgroups: two rounds of it
     assert picked(8, 2, 128, 22016, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
+    assert picked(8, 2, 64, 22016, 4096, T, group=128) == (64, 128, 256, 32, 64, 4)    # ... one round of the 64x128 one
+    assert picked(4, 4, 64, 22016, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)    # (built for activations wider than weights)
     # ... activations of at most 4 bits keep 128x64 up to 400 tiles
     assert picked(4, 4, 512, 11008, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
     assert picked(8, 2, 512, 11008, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
