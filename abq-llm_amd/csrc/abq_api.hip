@@ -1069,11 +1069,15 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
         // Wider outputs of at most 64 rows, activations wider than the weights: the same along N (64x128: gate + up of
         // LLaMA-7B, 22016 wide, at 32-64 rows 19.4 against 28.7 us).
         const bool one_round = (long)((state->M + 127) / 128) * ((state->N + 63) / 64) <= 256;
-        const bool along_n = !one_round && state->M <= 64 && (state->N + 127) / 128 <= 256;
-        if (one_round || along_n)
+        const bool along_n = !one_round && c.x_bits > c.w_bits && state->M <= 64 && (state->N + 127) / 128 <= 256;
+        // Otherwise, up to one round of 128x128 tiles, that tile with the split (1024 x 4096 x 11008: 73 against 85 us,
+        // 768 x 4096 x 4096 27.3 against 29.3; 320 workgroups, 1024 x 5120 x 5120: 68 against 57, not taken).
+        const bool one_round_128 = !one_round && !along_n && (long)((state->M + 127) / 128) * ((state->N + 127) / 128) <= 256;
+        if (one_round || along_n || one_round_128)
             for (int i = 0; i < tg->count; ++i)
-                if (usable(tg->entries[i]) && tg->entries[i].lds != 0 && block_m(tg->entries[i]) == (one_round ? 128 : 64) &&
-                    block_n(tg->entries[i]) == (one_round ? 64 : 128) && tg->entries[i].wk == 2)
+                if (usable(tg->entries[i]) && tg->entries[i].lds != 0 && block_m(tg->entries[i]) == (along_n ? 64 : 128) &&
+                    block_n(tg->entries[i]) == (one_round ? 64 : 128) && tg->entries[i].wk == 2 &&
+                    tg->entries[i].wm * tg->entries[i].wn == 4)
                     pick = i;
     } else {
         const int wk = c.warp_k > 0 ? c.block_k / c.warp_k : 1;

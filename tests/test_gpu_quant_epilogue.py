@@ -493,6 +493,46 @@ def test_group_scale_staged_kernel_every_tile(abq, oracle, q, p, signed):
             torch.cuda.synchronize()
             assert_close_rel(got.cpu().numpy(), want)
 
+@pytest.mark.parametrize("q,p,act", [(8, 2, False), (4, 4, False), (8, 2, True)])
+def test_group_scale_tiles_whose_waves_split_k_are_the_default_on_grids_of_one_round(abq, oracle, q, p, act):
+    """Grids of at most one workgroup per compute unit run the tile with two groups of waves that split K inside the
+    workgroup: 128x64 while that makes at most 256 workgroups, 128x128 beyond while that does, 64x128 for wide outputs
+    of at most 64 rows (activations wider than the weights); an odd number of K tiles (the last trip has one group
+    without a tile), zero points on both sides, ragged edges, the fused SiLU gate."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(7100 + 10 * q + p + act)
+    lo_x, hi_x, lo_w, hi_w = -(1 << (q - 1)), 1 << (q - 1), -(1 << (p - 1)), 1 << (p - 1)
+    cases = [(300, 192, 640, (128, 64, 256)), (1040, 2144, 384, (128, 128, 256)), (130, 16000, 256, (128, 128, 256))]
+    if q > p:
+        cases.append((40, 16640, 384, (64, 128, 256)))
+    for (M, N, K, tile) in cases:
+        G = K // 128
+        x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        xs = rng.uniform(0.01, 0.05, M)
+        xz = rng.integers(lo_x // 2, hi_x // 2 + 1, M).astype(np.float64)
+        wsc = rng.uniform(0.001, 0.02, (N, G))
+        wz = rng.integers(lo_w, hi_w, (N, G)).astype(np.float64)
+        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, 128)
+        if act:  # rows of W come in blocks of 16 gate rows followed by their 16 up rows
+            blocks = want.reshape(M, N // 32, 2, 16)
+            gate, up = blocks[:, :, 0, :], blocks[:, :, 1, :]
+            want = (gate / (1.0 + np.exp(-gate)) * up).reshape(M, N // 2)
+        wp = planes_dev(oracle.pack_i32(w, p))
+        kw = dict(x_scale=fdev(xs), w_scale=fdev(wsc), group_size=128, w_zero=fdev(wz), x_zero=fdev(xz), x_tiled=True, w_tiled=True,
+                  x_group_sums=torch.from_numpy(x.reshape(M, G, 128).sum(axis=2).astype(np.int32)).cuda())
+        kw["w_zero_term"] = abq.weight_zero_term(wp, True, kw["w_scale"], kw["w_zero"], 128)
+        if act:
+            kw["act"] = abq.ACT_SILU_GATE
+        xt, wt = abq.relayout_planes(planes_dev(oracle.pack_i32(x, q))), abq.relayout_planes(wp)
+        g = abq.Gemm(xt, wt, True, out_kind=abq.OUT_F16_SCALED, **kw)
+        c = g.state.cfg
+        assert g.strategy == "tiled" and (c.block_m, c.block_n, c.block_k) == tile, (M, N, K, g.config_name)
+        got = g.run()
+        torch.cuda.synchronize()
+        assert_close_rel(got.float().cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("M,K", [(200, 4096), (130, 4608), (136, 8192)])
 @pytest.mark.parametrize("q,p,fp6", [(8, 2, False), (4, 4, False), (4, 4, True)])
 def test_zero_points_over_whole_chunks_of_groups(abq, oracle, M, K, q, p, fp6):

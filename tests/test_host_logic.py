@@ -446,17 +446,20 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(8, 8, 4096, 4096, 4096, T) == (256, 128, 128, 64, 64, 4)
     # group scales (the decoder-layer linears): 128x128 once it fills the chip, 128x64 below
     assert picked(8, 2, 1024, 12288, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
-    assert picked(8, 2, 1024, 4096, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
+    assert picked(8, 2, 1024, 4096, 4096, T, group=128) == (128, 128, 256, 64, 64, 4)  # one round of 128x128: waves split K
+    assert picked(8, 2, 1024, 5120, 5120, T, group=128) == (128, 128, 128, 64, 64, 4)  # 320 workgroups: not
     assert picked(8, 2, 16384, 22016, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
     assert picked(8, 2, 128, 4096, 4096, T, group=64) == (64, 64, 128, 32, 32, 4)
     # up to one 128x64 workgroup per compute unit: the tile whose waves split K (its stages fill a compute unit's LDS)
     assert picked(8, 2, 512, 4096, 4096, T, group=128) == (128, 64, 256, 64, 32, 4)
     assert picked(8, 2, 128, 4096, 11008, T, group=128) == (128, 64, 256, 64, 32, 4)
     assert picked(8, 2, 128, 12288, 4096, T, group=128) == (128, 64, 256, 64, 32, 4)
-    assert picked(8, 2, 192, 12288, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)   # 384 workgroups: two rounds of it
-    assert picked(8, 2, 128, 22016, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
+    # 384 workgroups would be two rounds of it: the 128x128 tile with the same split while that makes one round
+    assert picked(8, 2, 192, 12288, 4096, T, group=128) == (128, 128, 256, 64, 64, 4)
+    assert picked(8, 2, 128, 22016, 4096, T, group=128) == (128, 128, 256, 64, 64, 4)
+    assert picked(8, 2, 384, 12288, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)   # 288 tiles of 128x128: neither
     assert picked(8, 2, 64, 22016, 4096, T, group=128) == (64, 128, 256, 32, 64, 4)    # ... one round of the 64x128 one
-    assert picked(4, 4, 64, 22016, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)    # (built for activations wider than weights)
+    assert picked(4, 4, 64, 22016, 4096, T, group=128) == (128, 128, 256, 64, 64, 4)   # (built for activations wider than weights)
     # ... activations of at most 4 bits keep 128x64 up to 400 tiles
     assert picked(4, 4, 512, 11008, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
     assert picked(8, 2, 512, 11008, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
