@@ -494,7 +494,12 @@ static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 #define ABQ_SENTRY_K(SG, TM, TN, WM, WN, WK)                                                            \
     { 32, TM, TN, WM, WN, WK, 4, &launch_mfma_staged<ABQ_Q, ABQ_P, SG, false, TM, TN, WM, WN, false, WK>, 128, \
       StagedStages<ABQ_Q, ABQ_P, false, TM, TN, WM, WN, false, WK>::kLds },
+// (the 128 x 128 one where three stages of two K tiles fit the LDS: not W8A8)
+#if ABQ_Q == 8 && ABQ_P == 8
 #define ABQ_STAGED_KSPLIT(SG) ABQ_SENTRY_K(SG, 1, 1, 2, 2, 2) ABQ_SENTRY_K(SG, 2, 1, 2, 2, 2)
+#else
+#define ABQ_STAGED_KSPLIT(SG) ABQ_SENTRY_K(SG, 1, 1, 2, 2, 2) ABQ_SENTRY_K(SG, 2, 1, 2, 2, 2) ABQ_SENTRY_K(SG, 2, 2, 2, 2, 2)
+#endif
 // Activations wider than the weights: a 128 x 256 tile (eight waves of 64 x 64, 2 along M, 4 along N) moves fewer
 // bytes per MFMA than 256 x 128, since a row of activations is the longer record.
 #if ABQ_Q > ABQ_P

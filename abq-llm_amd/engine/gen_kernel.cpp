@@ -208,6 +208,8 @@ std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits, bool is_signed)
         if (field && (is_signed || (x_bits < 8 && w_bits < 8))) {
             out.push_back(Tile{ 64, 64, 256, 32, 32, 128, 32, 32, 32, 2, 4, { 4 } });
             out.push_back(Tile{ 128, 64, 256, 64, 32, 128, 32, 32, 32, 2, 4, { 4 } });
+            if (x_bits + w_bits < 16) // three stages of two K tiles of 128 x 128 fit the LDS
+                out.push_back(Tile{ 128, 128, 256, 64, 64, 128, 32, 32, 32, 2, 4, { 4 } });
         }
         if (field && x_bits > w_bits && (is_signed || x_bits < 8)) {
             out.push_back(Tile{ 64, 128, 128, 32, 64, 128, 32, 32, 32, 2, 2, { 4 } });
