@@ -176,11 +176,66 @@ __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__
     }
 }
 
+// The same with one word-set (32 elements) per thread: a workgroup converts 8 rows x 8 K tiles, 32 consecutive
+// threads read 128 contiguous bytes of a plane row.  Four times the workgroups for a quarter of the work each: for
+// the few hundred activation rows of a small prefill, where the kernel above would occupy a quarter of the chip
+// and its time is one thread's latency chain (512 x 4096 8-bit activations: 64 workgroups there, 256 here).
+template <int BITS>
+__global__ __launch_bounds__(256) void relayout_planes_ws_kernel(const uint32_t *__restrict__ planes,
+                                                                 uint32_t *__restrict__ tiled, int rows, int KW)
+{
+    constexpr int REC = BITS * 4;          // words per record
+    constexpr int SLAB = 8 * REC + 4;      // words per K tile in LDS (+16 bytes against bank conflicts)
+    __shared__ __align__(16) uint32_t buf[8 * SLAB];
+    const int tid = threadIdx.x;
+    const int kt_tiles = KW / 4;
+    const int row0 = blockIdx.x * 8, kt0 = blockIdx.y * 8;
+    const size_t plane_stride = (size_t)rows * KW;
+    {
+        const int i = tid >> 5, w = tid & 31; // row, word-set within the 8 K tiles
+        const int row = row0 + i, kw = 4 * kt0 + w;
+        if (row < rows && kw < KW) {
+            uint32_t pw[BITS], e[8], f[BITS];
+            const uint32_t *p = planes + (size_t)row * KW + kw;
+#pragma unroll
+            for (int b = 0; b < BITS; ++b)
+                pw[b] = p[b * plane_stride];
+            planes_to_int8<BITS, kLow>(pw, e);
+            compress_fields<BITS>(e, f);
+            store_fields<BITS>(buf + (w >> 2) * SLAB + i * REC, w & 3, f);
+        }
+    }
+    __syncthreads();
+    const int nrow = min(8, rows - row0);
+    const int per_tile = nrow * BITS; // 16-byte units of one K tile's records
+    for (int u = tid; u < 8 * per_tile; u += 256) {
+        const int j = u / per_tile, v = u - j * per_tile;
+        if (kt0 + j < kt_tiles)
+            reinterpret_cast<uint4 *>(tiled + ((size_t)(kt0 + j) * rows + row0) * REC)[v] =
+                reinterpret_cast<const uint4 *>(buf + j * SLAB)[v];
+    }
+}
+
 hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits,
                                   hipStream_t stream)
 {
     const int KW = k / 32;
     const dim3 grid((rows + 31) / 32, (KW / 4 + 7) / 8);
+    if ((long)grid.x * grid.y < 256) { // less than a workgroup per compute unit: the finer kernel
+        const dim3 fine((rows + 7) / 8, (KW / 4 + 7) / 8);
+        switch (bits) {
+#define ABQ_RELAYOUT_CASE(B)                                                                                     \
+    case B:                                                                                                      \
+        hipLaunchKernelGGL(relayout_planes_ws_kernel<B>, fine, dim3(256), 0, stream, planes, tiled, rows, KW);   \
+        break;
+            ABQ_RELAYOUT_CASE(1) ABQ_RELAYOUT_CASE(2) ABQ_RELAYOUT_CASE(3) ABQ_RELAYOUT_CASE(4)
+            ABQ_RELAYOUT_CASE(5) ABQ_RELAYOUT_CASE(6) ABQ_RELAYOUT_CASE(7) ABQ_RELAYOUT_CASE(8)
+#undef ABQ_RELAYOUT_CASE
+        default:
+            return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
     switch (bits) {
 #define ABQ_RELAYOUT_CASE(B)                                                                                     \
     case B:                                                                                                      \
