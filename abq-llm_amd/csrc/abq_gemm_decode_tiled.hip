@@ -796,6 +796,14 @@ template <int Q, int P, bool SIGNED, bool XDYN = false> static hipError_t launch
             return hipErrorInvalidValue;
         return launch_decode_tiled_grouped_t<Q, P, SIGNED, 2, XDYN>(a, stream);
     }
+    // More than 8 rows on wide outputs: two tiles per workgroup as well, so that the rows a workgroup stages (64 KB at
+    // 16 x 4096 8-bit activations, five times the weights of one tile) serve twice the weights; W2A8 16 x 12288 x 4096
+    // 9.9 against 11.1 us, 16 x 11008 x 4096 9.7 against 11.0 (at 8 rows 7.2 against 6.8: not taken).  Only where the
+    // rows of a block stay the same, and not for shapes the variant that quantises in the kernel takes (at most 16384
+    // elements), whose output has to stay that of this one bit for bit.
+    if (!XDYN && a.M > 8 && (size_t)a.M * a.K > 16384 && (a.N + 15) / 16 >= 512 && a.N % 32 == 0 &&
+        decode_tiled_grouped_rows(16, 2, a.M, a.K, Q) == decode_tiled_grouped_rows(16, 1, a.M, a.K, Q))
+        return launch_decode_tiled_grouped_t<Q, P, SIGNED, 2, XDYN>(a, stream);
     return launch_decode_tiled_grouped_t<Q, P, SIGNED, 1, XDYN>(a, stream);
 }
 

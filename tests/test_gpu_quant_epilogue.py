@@ -493,6 +493,35 @@ def test_group_scale_staged_kernel_every_tile(abq, oracle, q, p, signed):
             torch.cuda.synchronize()
             assert_close_rel(got.cpu().numpy(), want)
 
+@pytest.mark.parametrize("q,p", [(8, 2), (4, 4), (8, 8)])
+def test_group_scale_decode_kernel_on_wide_outputs_of_more_than_eight_rows(abq, oracle, q, p):
+    """9 to 16 rows on outputs of at least 512 tiles of 16 weight rows: the decode kernel's group-scale variant takes two
+    tiles per workgroup (the staged rows serve twice the weights); an output whose width is no multiple of 32 and a
+    last workgroup with one tile keep working, zero points on both sides."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(8800 + 10 * q + p)
+    lo_x, hi_x, lo_w, hi_w = -(1 << (q - 1)), 1 << (q - 1), -(1 << (p - 1)), 1 << (p - 1)
+    for (M, N, K) in [(16, 8224, 1152), (12, 8208, 1536), (9, 8200, 2048)]:
+        G = K // 128
+        x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        xs = rng.uniform(0.01, 0.05, M)
+        xz = rng.integers(lo_x // 2, hi_x // 2 + 1, M).astype(np.float64)
+        wsc = rng.uniform(0.001, 0.02, (N, G))
+        wz = rng.integers(lo_w, hi_w, (N, G)).astype(np.float64)
+        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, 128)
+        wp = planes_dev(oracle.pack_i32(w, p))
+        kw = dict(x_scale=fdev(xs), w_scale=fdev(wsc), group_size=128, w_zero=fdev(wz), x_zero=fdev(xz), x_tiled=True, w_tiled=True,
+                  x_group_sums=torch.from_numpy(x.reshape(M, G, 128).sum(axis=2).astype(np.int32)).cuda())
+        kw["w_zero_term"] = abq.weight_zero_term(wp, True, kw["w_scale"], kw["w_zero"], 128)
+        xt, wt = abq.relayout_planes(planes_dev(oracle.pack_i32(x, q))), abq.relayout_planes(wp)
+        g = abq.Gemm(xt, wt, True, out_kind=abq.OUT_F16_SCALED, **kw)
+        assert g.strategy == "decode_tiled", (M, N, K, g.strategy)
+        got = g.run()
+        torch.cuda.synchronize()
+        assert_close_rel(got.float().cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("q,p,act", [(8, 2, False), (4, 4, False), (8, 2, True)])
 def test_group_scale_tiles_whose_waves_split_k_are_the_default_on_grids_of_one_round(abq, oracle, q, p, act):
     """Grids of at most one workgroup per compute unit run the tile with two groups of waves that split K inside the
