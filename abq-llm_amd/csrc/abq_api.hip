@@ -942,11 +942,11 @@ static bool decode_tiled_pays(int x_bits, int w_bits, int M, int N, int K)
     const double melems = (double)N * K / 1e6 * mrows / 16.0;
     const double per_block = x_bits == 8 ? 0.11 * (w_mb + x_mb) + 0.5 : 0.037 * melems * (w_bits >= 4 && K > 8192 ? 1.5 : 1.0);
     const double decode_us = (x_bits == 8 ? 0.8 : 2.7) + blocks * per_block;
-    // (all pairs but W8A8 run that tile with two groups of waves that split K: 4.5 + 0.13 us per K tile, e.g. W2A8
-    // 128 x 4096 x 11008 15.5 against 20.9 us)
+    // (all pairs but W8A8 run that tile with two groups of waves that split K: 5.0 + 0.145 us per K tile on weights
+    // that come from HBM, e.g. W2A8 64 x 4096 x 4096 9.7, 64 x 4096 x 11008 17.5 us)
     const long tiles64 = (long)((M + 63) / 64) * ((N + 63) / 64);
     const int kt = K / 128;
-    const double tiled_us = (x_bits + w_bits < 16 ? 4.5 + 0.13 * kt : 2.3 + 0.23 * kt) * (tiles64 > 256 ? 1.35 : 1.0);
+    const double tiled_us = (x_bits + w_bits < 16 ? 5.0 + 0.145 * kt : 2.3 + 0.23 * kt) * (tiles64 > 256 ? 1.35 : 1.0);
     return decode_us < 0.9 * tiled_us;
 }
 
@@ -990,11 +990,11 @@ static abq_status switch_to_decode_tiled(abq_gemm_state *st)
 // Group scales on a decode-sized GEMM whose operands are (or are about to be declared) both prepared: whether the
 // decode kernel of that layout has a group-scale variant for the pair that fits this shape.
 // The same weighing for the group-scale variant (one tile per workgroup, two with the SiLU gate), against the
-// group-scale prefill kernel, whose smallest grids (128 x 64 tiles) take 0.48 us per K tile whatever M is
-// and 0.6 x 1.45 once they exceed one workgroup per compute unit.  Fits to a sweep of W2A8, W4A8 and W4A4 with
-// zero points over M = 24 ... 128 on the LLaMA-7B linears (4096 x 4096, QKV, gate + up with the gate fused, down);
-// taken when estimated 15 % ahead: W2A8 32 x 4096 x 4096 8.3 against 20.1 us, 32 x 4096 x 11008 23.2 against 48.8,
-// W4A4 32 x 12288 x 4096 13.2 against 20.6; the wide outputs of the 8-bit activations stay on the prefill kernel.
+// group-scale prefill kernel, whose smallest grids (128 x 64 tiles) take 4 + 0.42 us per K tile whatever M is and
+// 1 + 0.6 x 1.45 per K tile once they exceed one workgroup per compute unit.  Fits to a sweep of W2A8, W4A8 and W4A4
+// with zero points over M = 24 ... 128 on the LLaMA-7B linears (4096 x 4096, QKV, gate + up with the gate fused,
+// down); taken when estimated 10 % ahead: W2A8 32 x 4096 x 4096 8.3 against 17 us, 32 x 4096 x 11008 24 against 38;
+// the wide outputs of the 8-bit activations stay on the prefill kernel.
 static bool decode_tiled_grouped_pays(int x_bits, int w_bits, int M, int N, int K, int act)
 {
     if (M <= 16)
@@ -1010,10 +1010,11 @@ static bool decode_tiled_grouped_pays(int x_bits, int w_bits, int M, int N, int 
     const double x_mb = (double)((N + 16 * t - 1) / (16 * t)) * mrows * K * x_bits / 8e6;
     const double per_block = x_bits == 8 ? 0.165 * (w_mb + x_mb) : 0.11 * (w_mb + x_mb) + 0.7;
     const double decode_us = 1.0 + blocks * per_block;
-    // (up to one workgroup per compute unit the prefill kernel's waves split K: 0.48 us per K tile)
+    // (up to one workgroup per compute unit the prefill kernel's waves split K: 4 + 0.42 us per K tile on weights that
+    // come from HBM, W2A8 64 x 4096 x 4096 17.4, 64 x 4096 x 11008 38.2 us)
     const long wgs = (long)((N + 63) / 64) * ((M + 127) / 128);
-    const double tiled_us = 1.0 + (wgs > 256 ? 0.6 * 1.45 : 0.48) * (K / 128);
-    return decode_us < 0.85 * tiled_us;
+    const double tiled_us = wgs > 256 ? 1.0 + 0.6 * 1.45 * (K / 128) : 4.0 + 0.42 * (K / 128);
+    return decode_us < 0.9 * tiled_us;
 }
 
 static bool decode_tiled_grouped_fits(const abq_gemm_state *st, int group_size, int act)
