@@ -808,6 +808,12 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
             want[4] = 2;
             want[0] = n64x64 <= 256 ? 1 : along_n ? 1 : 2; // 64x64 up to one workgroup per compute unit
             want[1] = n64x64 <= 256 ? 1 : along_n ? 2 : 1;
+        } else if (tt->entries[pick].lds != 0 && t128 <= 256 && c.x_bits + c.w_bits < 16) {
+            // exactly one round of 128x128 tiles: that tile with the split (1024 x 4096 x 11008: W2A8 1725 against 1611
+            // TOPS on 64x128, W4A4 1686 against 1530 on 128x128; on K = 4096 level with the best)
+            want[4] = 2;
+            want[0] = 2;
+            want[1] = 2;
         } else if (tt->entries[pick].lds != 0 && along_n && t128 < 400 && tt->entries[pick].tm * tt->entries[pick].wm <= 4 &&
                    tt->entries[pick].tn * tt->entries[pick].wn <= 4) {
             want[4] = 1;
@@ -837,7 +843,7 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
     if (!fp6_eligible(c.x_bits, c.w_bits, c.is_signed, st->K))
         return ABQ_ERR_UNSUPPORTED;
     if (st->group_size) {
-        // group scales: one scale per K tile, i.e. groups of 128.  Below 300 tiles of 128x128: 128x64, the
+        // group scales: one scale per K tile, i.e. groups of 128.  Below 256 tiles of 128x128 (one round): 128x64, the
         // smallest tile with two MFMA tiles per wave; above, 256x128 runs 6 % faster than 128x128 where its
         // rounds of workgroups come out even (sweep of the three tiles over M = 512 .. 16384 and the LLaMA
         // widths: the choice is within 0.1 % of the best tile on average, 4 % at worst)
@@ -853,7 +859,7 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
             const int bm = 32 * ge[i].tm * ge[i].wm, bn = 32 * ge[i].tn * ge[i].wn;
             if (!st->auto_chosen ? (bm == c.block_m && bn == c.block_n && 32 * ge[i].tm == c.warp_m)
                                  : large >= 0 ? i == large
-                                              : ((t128 >= 300 && bm == 128 && bn == 128) || (t128 < 300 && bm == 128 && bn == 64)))
+                                              : ((t128 >= 256 && bm == 128 && bn == 128) || (t128 < 256 && bm == 128 && bn == 64)))
                 gpick = i;
         }
         if (gpick < 0)
@@ -874,7 +880,7 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
     // 128x128 (two workgroups per compute unit) is the fastest tile from 200 tiles up: with the grouped tile
     // mapping it beats 256x128 at every M of the sweep but the very largest, by 3-10 %; below that the
     // smaller ones: { TM, TN, waves along M, waves along N, workgroups needed }
-    static const int order[][5] = { { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 400 }, { 1, 1, 2, 2, 0 } };
+    static const int order[][5] = { { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 256 }, { 1, 1, 2, 2, 0 } };
     int pick = -1;
     for (const auto &o : order) {
         const int bm = 32 * o[0] * o[2], bn = 32 * o[1] * o[3];

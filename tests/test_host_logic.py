@@ -422,7 +422,8 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
 
     T, F6 = abq.LAYOUT_TILED, abq.LAYOUT_FP6
     # W4A4 on the FP6 route: 128x128 from a chip's worth of tiles up
-    assert picked(4, 4, 512, 4096, 4096, F6) == (64, 64, 128, 32, 32, 5)
+    assert picked(4, 4, 512, 4096, 4096, F6) == (128, 64, 128, 64, 32, 5)
+    assert picked(4, 4, 256, 4096, 4096, F6) == (64, 64, 128, 32, 32, 5)
     assert picked(4, 4, 512, 11008, 4096, F6) == (128, 128, 128, 64, 64, 5)
     assert picked(4, 4, 2048, 12288, 4096, F6) == (128, 128, 128, 64, 64, 5)
     assert picked(4, 4, 16384, 4096, 4096, F6) == (128, 128, 128, 64, 64, 5)
@@ -437,8 +438,10 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(8, 2, 256, 4096, 4096, T) == (64, 64, 256, 32, 32, 4)
     assert picked(4, 4, 512, 4096, 4096, T) == (128, 64, 256, 64, 32, 4)
     assert picked(8, 2, 512, 11008, 4096, T) == (64, 128, 128, 32, 64, 4)
-    assert picked(8, 2, 1024, 4096, 4096, T) == (64, 128, 128, 32, 64, 4)
-    assert picked(4, 4, 1024, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)
+    assert picked(8, 2, 384, 12288, 4096, T) == (64, 128, 128, 32, 64, 4)
+    assert picked(8, 2, 1024, 4096, 4096, T) == (128, 128, 256, 64, 64, 4)     # one round of 128x128 tiles: with the split
+    assert picked(4, 4, 1024, 4096, 11008, T) == (128, 128, 256, 64, 64, 4)
+    assert picked(8, 8, 1024, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)     # (not built for W8A8)
     # signed W8A8: 256x128 as soon as it fills the chip
     assert picked(8, 8, 2048, 4096, 4096, T) == (256, 128, 128, 64, 64, 4)
     assert picked(8, 8, 1024, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)
@@ -468,4 +471,5 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(4, 4, 2048, 4096, 4096, F6, group=128) == (256, 128, 128, 64, 64, 5)
     assert picked(4, 4, 1024, 11008, 4096, F6, group=128) == (128, 128, 128, 64, 64, 5)   # 344 tiles of 256x128: 1.3 rounds
     assert picked(4, 4, 16384, 4096, 11008, F6, group=128) == (256, 128, 128, 64, 64, 5)
-    assert picked(4, 4, 1024, 4096, 4096, F6, group=128) == (128, 64, 128, 64, 32, 5)
+    assert picked(4, 4, 1024, 4096, 4096, F6, group=128) == (128, 128, 128, 64, 64, 5)
+    assert picked(4, 4, 512, 4096, 4096, F6, group=128) == (128, 64, 128, 64, 32, 5)
