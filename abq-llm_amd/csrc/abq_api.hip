@@ -784,7 +784,9 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
             continue;
         const int bm = 32 * o[0] * o[2], bn = 32 * o[1] * o[3];
         const long tiles = (long)((st->M + bm - 1) / bm) * ((st->N + bn - 1) / bn);
-        const long need = (staged && o[0] == 2 && o[1] == 2 && o[2] == 4) ? 160 : o[4];
+        // (signed W8A8, which keeps its one-group tiles on small grids: 128x64 from one workgroup per compute unit,
+        // 512 x 4096 x 4096 844 against 794 TOPS on 64x64)
+        const long need = (staged && o[0] == 2 && o[1] == 2 && o[2] == 4) ? 160 : (staged && o[0] == 2 && o[1] == 1) ? 256 : o[4];
         for (int i = 0; i < tt->count; ++i)
             if (tt->entries[i].tm == o[0] && tt->entries[i].tn == o[1] && tt->entries[i].kb == 128 && tt->entries[i].wk == 1 &&
                 tt->entries[i].wm == o[2] && tt->entries[i].wn == o[3] && tiles >= need && pick < 0)
@@ -877,12 +879,16 @@ static abq_status switch_to_fp6(abq_gemm_state *st)
     }
     int count = 0;
     const KernelEntry *es = fp6_entries(&count);
-    // 128x128 (two workgroups per compute unit) is the fastest tile from 200 tiles up: with the grouped tile
-    // mapping it beats 256x128 at every M of the sweep but the very largest, by 3-10 %; below that the
+    // 128x128 (two workgroups per compute unit) from 200 tiles up unless 256x128 is estimated ahead, below that the
     // smaller ones: { TM, TN, waves along M, waves along N, workgroups needed }
     static const int order[][5] = { { 2, 2, 2, 2, 200 }, { 2, 1, 2, 2, 256 }, { 1, 1, 2, 2, 0 } };
-    int pick = -1;
+    // (at the clock the chip sustains the 256x128 tile runs 6-10 % ahead of 128x128 wherever its rounds of workgroups
+    // come out even: weighed by the same model as on the int8 route)
+    static const LargeTile fp6_large[] = { { 2, 2, 4, 2, 1.07, 1.07 } };
+    int pick = (long)((st->M + 127) / 128) * ((st->N + 127) / 128) >= 200 ? pick_large_tile(es, count, fp6_large, 1, st->M, st->N) : -1;
     for (const auto &o : order) {
+        if (pick >= 0)
+            break;
         const int bm = 32 * o[0] * o[2], bn = 32 * o[1] * o[3];
         const long tiles = (long)((st->M + bm - 1) / bm) * ((st->N + bn - 1) / bn);
         for (int i = 0; i < count; ++i)

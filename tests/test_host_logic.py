@@ -421,12 +421,15 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
         return (c.block_m, c.block_n, c.block_k, c.warp_m, c.warp_n, c.nstage)
 
     T, F6 = abq.LAYOUT_TILED, abq.LAYOUT_FP6
-    # W4A4 on the FP6 route: 128x128 from a chip's worth of tiles up
+    # W4A4 on the FP6 route: 128x128 from a chip's worth of tiles up where the larger tile's grid is ragged
     assert picked(4, 4, 512, 4096, 4096, F6) == (128, 64, 128, 64, 32, 5)
     assert picked(4, 4, 256, 4096, 4096, F6) == (64, 64, 128, 32, 32, 5)
-    assert picked(4, 4, 512, 11008, 4096, F6) == (128, 128, 128, 64, 64, 5)
-    assert picked(4, 4, 2048, 12288, 4096, F6) == (128, 128, 128, 64, 64, 5)
-    assert picked(4, 4, 16384, 4096, 4096, F6) == (128, 128, 128, 64, 64, 5)
+    assert picked(4, 4, 1024, 11008, 4096, F6) == (128, 128, 128, 64, 64, 5)
+    assert picked(4, 4, 1024, 4096, 4096, F6) == (128, 128, 128, 64, 64, 5)
+    # ... and 256x128 where its rounds of workgroups come out even
+    assert picked(4, 4, 512, 11008, 4096, F6) == (256, 128, 128, 64, 64, 5)
+    assert picked(4, 4, 2048, 12288, 4096, F6) == (256, 128, 128, 64, 64, 5)
+    assert picked(4, 4, 16384, 4096, 4096, F6) == (256, 128, 128, 64, 64, 5)
     # W2A8: 256x256 only where its grid is whole rounds of the chip
     assert picked(8, 2, 2048, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)
     assert picked(8, 2, 4096, 11008, 4096, T) == (128, 128, 128, 64, 64, 4)       # 688 tiles of 256x256: a third round mostly empty
