@@ -624,8 +624,7 @@ int main(int argc, char **argv)
                 body(repeat);
                 HIP_OK(hipStreamEndCapture(stream, &g));
                 HIP_OK(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0));
-                HIP_OK(hipGraphLaunch(ge, stream));
-                HIP_OK(hipStreamSynchronize(stream));
+                warm_replays(ge, stream);
             }
             HIP_OK(hipEventRecord(e0, stream));
             if (use_graph)
