@@ -445,11 +445,15 @@ template <int P, bool SIGNED> __device__ __forceinline__ void dtg_operands(const
 // rows it multiplies (at most XP * 64 NW units of eight halves), takes their extrema through LDS, writes the int8
 // records and the group sums into LDS and keeps the rows' scales and zero points there for the epilogue.  The
 // quantising launch in front of every decode GEMM, and the memory round trip between the two, fall away.
-template <int Q, int P, bool SIGNED, int NW, int D, int T, bool XDYN = false>
+// XDYN is the number of units a thread holds (0: the activations arrive packed): 1, 2 or, with eight waves, 4, i.e. up
+// to 16384 elements per workgroup; the launcher takes the smallest that covers the rows (a row of 4096 needs one unit
+// per thread of eight waves: 52 + 25 registers instead of 52 + 49, three workgroups per compute unit instead of two).
+template <int Q, int P, bool SIGNED, int NW, int D, int T, int XDYN = 0>
 __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmArgs a, int mrows)
 {
     static_assert(!XDYN || (Q == 8 && SIGNED), "in-kernel quantisation writes signed 8-bit records");
-    constexpr int XP = NW == 16 ? 2 : 4; // XDYN: units per thread (16384 elements per workgroup either way)
+    static_assert(XDYN == 0 || XDYN == 1 || XDYN == 2 || (XDYN == 4 && NW == 8), "units per thread");
+    constexpr int XP = XDYN > 0 ? XDYN : 1; // XDYN: units per thread
     constexpr int NT = 64 * NW;
     constexpr int QLOG = Q == 8 ? 3 : Q == 4 ? 2 : 1;
     constexpr int LPS = DtgShare<P>::kLoads; // loads per step and tile
@@ -749,6 +753,20 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
     }
 }
 
+template <int Q, int P, bool SIGNED, int NW, int D, int T, int XD>
+static hipError_t launch_decode_tiled_grouped_instance(const GemmArgs &a, int mrows, hipStream_t stream)
+{
+    const size_t lds = decode_tiled_grouped_lds(NW, T, mrows, a.K, Q);
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T, XD>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr != hipSuccess)
+        return attr;
+    const int tiles = (a.N + 15) / 16;
+    const dim3 grid((tiles + T - 1) / T, (a.M + mrows - 1) / mrows);
+    hipLaunchKernelGGL((gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T, XD>), grid, dim3(64 * NW), lds, stream, a, mrows);
+    return hipGetLastError();
+}
+
 // (waves, loads in flight per wave, tiles) by shape; the fused gate needs a tile pair per workgroup.
 template <int Q, int P, bool SIGNED, int NW, int D, int T, bool XDYN = false>
 static hipError_t launch_decode_tiled_grouped_as(const GemmArgs &a, hipStream_t stream)
@@ -759,15 +777,17 @@ static hipError_t launch_decode_tiled_grouped_as(const GemmArgs &a, hipStream_t 
     // in-kernel quantisation: a workgroup's rows fit its threads' registers (two or four units of eight halves each)
     if (XDYN && (size_t)mrows * a.K > 16384)
         return hipErrorInvalidValue;
-    const size_t lds = decode_tiled_grouped_lds(NW, T, mrows, a.K, Q);
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T, XDYN>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (attr != hipSuccess)
-        return attr;
-    const int tiles = (a.N + 15) / 16;
-    const dim3 grid((tiles + T - 1) / T, (a.M + mrows - 1) / mrows);
-    hipLaunchKernelGGL((gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T, XDYN>), grid, dim3(64 * NW), lds, stream, a, mrows);
-    return hipGetLastError();
+    if constexpr (XDYN) {
+        // the fewest units per thread that cover the workgroup's rows
+        const int need = (int)(((size_t)mrows * a.K / 8 + 64 * NW - 1) / (64 * NW));
+        if (need <= 1)
+            return launch_decode_tiled_grouped_instance<Q, P, SIGNED, NW, D, T, 1>(a, mrows, stream);
+        if (need <= 2 || NW == 16)
+            return launch_decode_tiled_grouped_instance<Q, P, SIGNED, NW, D, T, 2>(a, mrows, stream);
+        return launch_decode_tiled_grouped_instance<Q, P, SIGNED, NW, D, T, NW == 8 ? 4 : 2>(a, mrows, stream);
+    } else {
+        return launch_decode_tiled_grouped_instance<Q, P, SIGNED, NW, D, T, 0>(a, mrows, stream);
+    }
 }
 
 template <int Q, int P, bool SIGNED, int T, bool XDYN = false>
