@@ -117,11 +117,15 @@ template <int BITS, bool SIGNED> __device__ __forceinline__ void dt_unpack(const
 // (int)(half(x) * half(scale)) as pack_half of the reference does (abq_gemm_wrapper.cu:29-54), straight into the
 // int8 records in LDS: the pack kernel and its launch in front of every decode GEMM of the FT wrapper fall away.
 // Every workgroup converts the rows it multiplies (M x K halves, from L2 after the first).  8-bit activations.
-template <int Q, int P, bool SIGNED, int NW, int D, int T, bool XF16 = false>
+// XF16 is the number of 16-byte units of eight halves a thread holds per pass (0: the activations arrive packed; 1, 2
+// or 4, the launcher takes the fewest that cover the rows in one pass, at most 4: eight rows of 4096 with sixteen waves;
+// more spills, and with four the instances need 95 - 104 registers against 52 - 67, which costs workgroups per unit).
+template <int Q, int P, bool SIGNED, int NW, int D, int T, int XF16 = 0>
 __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, int mrows)
 {
     static_assert(!XF16 || Q == 8, "in-kernel quantisation writes 8-bit records");
-    constexpr int XP = 4;        // XF16: 16-byte units of eight halves per thread and pass (eight rows of 4096 in one pass; more spills)
+    static_assert(XF16 == 0 || XF16 == 1 || XF16 == 2 || XF16 == 4, "units per thread and pass");
+    constexpr int XP = XF16 > 0 ? XF16 : 1;
     constexpr int NXL = Q / P;   // activation chunks (16 bytes) per weight unit
     constexpr int NM = 8 / P;    // MFMAs per weight unit
     constexpr int MX = 8 / Q;    // MFMAs per activation chunk
@@ -346,6 +350,20 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
     }
 }
 
+template <int Q, int P, bool SIGNED, int NW, int D, int T, int XU>
+static hipError_t launch_decode_tiled_instance(const GemmArgs &a, int mrows, hipStream_t stream)
+{
+    const size_t lds = decode_tiled_lds(NW, T, mrows, a.K, Q);
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled<Q, P, SIGNED, NW, D, T, XU>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr != hipSuccess)
+        return attr;
+    const int tiles = (a.N + 15) / 16;
+    const dim3 grid((tiles + T - 1) / T, (a.M + mrows - 1) / mrows);
+    hipLaunchKernelGGL((gemm_decode_tiled<Q, P, SIGNED, NW, D, T, XU>), grid, dim3(64 * NW), lds, stream, a, mrows);
+    return hipGetLastError();
+}
+
 template <int Q, int P, bool SIGNED, int NW, int D, int T, bool XF16 = false>
 static hipError_t launch_decode_tiled(const GemmArgs &a, hipStream_t stream)
 {
@@ -354,15 +372,16 @@ static hipError_t launch_decode_tiled(const GemmArgs &a, hipStream_t stream)
         return hipErrorInvalidValue;
     if (XF16 && !a.x_pack_scale)
         return hipErrorInvalidValue;
-    const size_t lds = decode_tiled_lds(NW, T, mrows, a.K, Q);
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled<Q, P, SIGNED, NW, D, T, XF16>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (attr != hipSuccess)
-        return attr;
-    const int tiles = (a.N + 15) / 16;
-    const dim3 grid((tiles + T - 1) / T, (a.M + mrows - 1) / mrows);
-    hipLaunchKernelGGL((gemm_decode_tiled<Q, P, SIGNED, NW, D, T, XF16>), grid, dim3(64 * NW), lds, stream, a, mrows);
-    return hipGetLastError();
+    if constexpr (XF16) {
+        const int need = (int)(((size_t)mrows * a.K / 8 + 64 * NW - 1) / (64 * NW)); // units per thread for one pass
+        if (need <= 1)
+            return launch_decode_tiled_instance<Q, P, SIGNED, NW, D, T, 1>(a, mrows, stream);
+        if (need <= 2)
+            return launch_decode_tiled_instance<Q, P, SIGNED, NW, D, T, 2>(a, mrows, stream);
+        return launch_decode_tiled_instance<Q, P, SIGNED, NW, D, T, 4>(a, mrows, stream);
+    } else {
+        return launch_decode_tiled_instance<Q, P, SIGNED, NW, D, T, 0>(a, mrows, stream);
+    }
 }
 
 // ---- the same plan with group-wise weight scales -------------------------------------------------

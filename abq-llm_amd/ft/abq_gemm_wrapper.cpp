@@ -135,9 +135,12 @@ void ABQGEMMWrapper::gemm(const int M, const int N, const int K, const _Float16 
     }
     // quant + packing; for a prepared weight straight into the layout its kernels read, or, for decode-sized calls
     // with 8-bit activations, inside the GEMM kernel itself (one launch instead of two)
-    // (where a workgroup quantises its rows in one pass, M * K <= 32768: 4.0 against 5.8 us at M = 2, 4.7 against 5.8
-    // at M = 8 on 4096 x 4096; at M = 16 the repeated conversion costs more than the launch it saves)
-    if (tiled && (long)M * K <= 32768 && abq_gemm_set_f16_activations(&state, A, scale) == ABQ_OK) {
+    // (where a workgroup quantises its rows in one pass, M * K <= 32768, and the workgroups that all repeat that are
+    // few enough: 3.9 against 5.2 us at M = 1 and 5.0 against 5.5 at M = 8 on 4096 x 4096, 5.8 against 6.5 at M = 1 on
+    // 11008 x 4096; on wider outputs, or from M = 4 on outputs beyond 4096, the packing launch is the cheaper way:
+    // 22016 x 4096 at M = 1 8.6 against 9.4 us, 11008 x 4096 at M = 8 6.9 against 10.2)
+    const bool in_kernel = (long)M * K <= 32768 && (N <= 4096 || (M == 1 && N <= 12288));
+    if (tiled && in_kernel && abq_gemm_set_f16_activations(&state, A, scale) == ABQ_OK) {
         // nothing to pack
     } else if (tiled) {
         const abq_status prc = abq_pack_f16_tiled(A, scale, reinterpret_cast<uint32_t *>(abq_gemm_workspace), M, K, x_bits_, stream);
@@ -223,7 +226,10 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     abq_gemm_state state;
     // the smallest calls on the prepared-operand decode kernel: the kernel quantises the rows itself (one launch
     // instead of two; the quantising launch costs as much as the GEMM at these sizes), same result bit for bit
-    if (decode_prepared && M <= 16 && (size_t)M * K <= 16384) {
+    // (one token, or several on outputs of at most 4096 columns: every workgroup repeats the quantisation, which on
+    // the wide linears costs more than the launch from two tokens on: QKV of LLaMA-7B at two tokens 11.6 against
+    // 10.1 us, at four 18.0 against 10.7; 4096 x 4096 at four tokens 8.1 against 8.6)
+    if (decode_prepared && M <= 16 && (size_t)M * K <= 16384 && (M == 1 || N <= 4096)) {
         rc = abq_gemm_init(nullptr, x_bits_, w_bits_, 1, planes, reinterpret_cast<const uint32_t *>(W.planes_tiled), M, N, K, D,
                            nullptr, 0, ABQ_OUT_F16_SCALED, &state);
         if (rc == ABQ_OK)

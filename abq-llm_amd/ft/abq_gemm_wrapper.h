@@ -82,8 +82,9 @@ public:
     // silu_gate: W holds a gate / up pair interleaved in blocks of 16 rows (abq_weight_blob_interleave_gate_up),
     // N counts the rows of both and D is [M][N/2] = silu(gate) * up: the two GEMMs and the elementwise
     // kernel of the reference's gated MLP (FfnLayer.cc:341-374,575-577) in one launch.
-    // The smallest calls (at most 16 rows, M * K <= 16384, 8-bit activations, groups of 128, a pair the
-    // prepared-operand decode kernel is built for) are ONE launch: that kernel quantises the rows itself, the
+    // The smallest calls (one token, or up to 16 rows on outputs of at most 4096 columns; M * K <= 16384, 8-bit
+    // activations, groups of 128, a pair the prepared-operand decode kernel is built for) are ONE launch: that kernel
+    // quantises the rows itself, the
     // workspace is not written, the output is the same bit for bit.
     void gemm_dynamic(const int M, const int N, const int K, const _Float16 *A, const ABQGroupedWeight &W,
                       _Float16 *D, bool x_symmetric, char *abq_gemm_workspace, size_t abq_gemm_ws_bytes,

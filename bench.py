@@ -589,7 +589,7 @@ def main():
                     gm.run()
                 step()
                 torch.cuda.synchronize()
-                reps = 3
+                reps = 3 if tokens >= 1024 else 20  # (a replay's own launch cost is spread over the steps of the graph)
                 gr = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(gr):
                     for _ in range(reps):
