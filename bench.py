@@ -317,7 +317,7 @@ def main():
                     gm = abq.Gemm(xpl, wtl, signed, w_tiled=True, workspace=ws)  # activations converted per call
                     gm.run()
                     torch.cuda.synchronize()
-                    reps = 5
+                    reps = 20  # (a replay's own launch cost is spread over the steps of the graph)
                     gr = torch.cuda.CUDAGraph()  # replayed like the decode GEMMs: no host launch cost in the figure
                     with torch.cuda.graph(gr):
                         for _ in range(reps):
@@ -384,7 +384,7 @@ def main():
                                                                    x_scale=xsc, w_scale=wsc))):
                         gm.run()
                         torch.cuda.synchronize()
-                        reps = 5
+                        reps = 20
                         gr = torch.cuda.CUDAGraph()
                         with torch.cuda.graph(gr):
                             for _ in range(reps):
@@ -589,7 +589,7 @@ def main():
                     gm.run()
                 step()
                 torch.cuda.synchronize()
-                reps = 3 if tokens >= 1024 else 20  # (a replay's own launch cost is spread over the steps of the graph)
+                reps = 20 if tokens < 1024 else 10 if tokens < 8192 else 3  # (a replay's own launch cost is spread over its steps)
                 gr = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(gr):
                     for _ in range(reps):
