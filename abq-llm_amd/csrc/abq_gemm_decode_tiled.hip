@@ -62,6 +62,14 @@ __device__ __forceinline__ v4u dt_load16(const char *base, uint32_t off)
     asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(v) : "v"(off), "s"(base) : "memory");
     return v;
 }
+// the same for weight records, which nothing reads a second time: marked non-temporal, so that the lines do not
+// displace the activations and scales every workgroup shares in the L2
+__device__ __forceinline__ v4u dt_load16_once(const char *base, uint32_t off)
+{
+    v4u v;
+    asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(v) : "v"(off), "s"(base) : "memory");
+    return v;
+}
 
 template <int N> __device__ __forceinline__ void dt_wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 // the same with a count that is constant only after unrolling
@@ -251,7 +259,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
             const uint32_t bk = (ragged && s == S - 1 && 4 * s + g >= U) ? back : 0u;
 #pragma unroll
             for (int t = 0; t < T; ++t)
-                wb[d][t] = dt_load16(wp, woff[t] - bk);
+                wb[d][t] = dt_load16_once(wp, woff[t] - bk);
         }
         if (round == 0) {
             dt_wait_loads<D * T>(); // the activation loads are older than these
@@ -419,7 +427,7 @@ template <int P> struct DtgShare {
     {
 #pragma unroll
         for (int i = 0; i < P / 4; ++i)
-            v[i] = dt_load16(base, off + 16u * i);
+            v[i] = dt_load16_once(base, off + 16u * i);
     }
     __device__ __forceinline__ void landed()
     {
@@ -433,7 +441,7 @@ template <> struct DtgShare<2> {
     static constexpr int kLoads = 1;
     __device__ __forceinline__ void issue(const char *base, uint32_t off)
     {
-        asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(v) : "v"(off), "s"(base) : "memory");
+        asm volatile("global_load_dwordx2 %0, %1, %2 nt" : "=&v"(v) : "v"(off), "s"(base) : "memory");
     }
     __device__ __forceinline__ void landed() { asm volatile("" : "+v"(v)); }
 };

@@ -61,10 +61,11 @@ __device__ __forceinline__ void store_wave_tile_f16(_Float16 *out, int row_len, 
 #pragma unroll
     for (int it = 0; it < 32 * TM / T::kRowsPerPass; ++it) {
         const int row = it * T::kRowsPerPass + lr;
-        const uint4 v = *reinterpret_cast<const uint4 *>(wave_lds + row * T::kStride + lc * 16);
+        typedef unsigned int line_piece __attribute__((ext_vector_type(4)));
+        const line_piece v = *reinterpret_cast<const line_piece *>(wave_lds + row * T::kStride + lc * 16);
         const int m = row0 + row, n = col0 + lc * 8;
-        if (m < rows_end && n < cols_end)
-            *reinterpret_cast<uint4 *>(out + (size_t)m * row_len + n) = v;
+        if (m < rows_end && n < cols_end) // written once, read by another kernel: non-temporal
+            __builtin_nontemporal_store(v, reinterpret_cast<line_piece *>(out + (size_t)m * row_len + n));
     }
 }
 

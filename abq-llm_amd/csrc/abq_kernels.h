@@ -210,7 +210,7 @@ __device__ __attribute__((noinline)) static void store_result_call(void *D, cons
 __device__ __forceinline__ void store_result_compact(const StoreOperands &o, int m, int n, int acc)
 {
     if (o.out_kind == 0)
-        reinterpret_cast<int *>(o.D)[(size_t)m * o.N + n] = acc;
+        __builtin_nontemporal_store(acc, reinterpret_cast<int *>(o.D) + ((size_t)m * o.N + n));
     else
         store_result_call(o.D, o.C, o.x_scale, o.w_scale, o.N, o.out_kind, m, n, acc);
 }

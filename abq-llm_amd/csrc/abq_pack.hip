@@ -550,7 +550,10 @@ __global__ __launch_bounds__(256) void quant_pack_wave_rows_kernel(const uint4 *
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
         const int u = lane + 64 * i;
-        raw[i] = xr[u < units ? u : 0]; // past the end: the row's first unit once more (it changes no extremum)
+        // (read once: non-temporal; past the end: the row's first unit once more, it changes no extremum)
+        typedef unsigned int unit_words __attribute__((ext_vector_type(4)));
+        const unit_words w = __builtin_nontemporal_load(reinterpret_cast<const unit_words *>(xr + (u < units ? u : 0)));
+        raw[i] = make_uint4(w.x, w.y, w.z, w.w);
     }
     half2_t mx2 = { (_Float16)-INFINITY, (_Float16)-INFINITY }, mn2 = { (_Float16)INFINITY, (_Float16)INFINITY };
 #pragma unroll
