@@ -62,12 +62,24 @@ __device__ __forceinline__ v4u dt_load16(const char *base, uint32_t off)
     asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(v) : "v"(off), "s"(base) : "memory");
     return v;
 }
-// the same for weight records, which nothing reads a second time: marked non-temporal, so that the lines do not
-// displace the activations and scales every workgroup shares in the L2
-__device__ __forceinline__ v4u dt_load16_once(const char *base, uint32_t off)
+// the same for weight records.  once: nothing reads the record a second time (the grid has one block of rows), and the
+// load is marked non-temporal, so that the lines do not displace what the workgroups share in the L2; with several
+// blocks of rows the other blocks' workgroups read the record again and it is loaded like anything else.  (wave-uniform)
+// (One statement with a scalar branch inside, not two statements under an if: the destination is then one register
+// whichever way the load is issued, and no copy of a register still in flight can come between load and wait.)
+__device__ __forceinline__ v4u dt_load16_weights(const char *base, uint32_t off, int once)
 {
     v4u v;
-    asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(v) : "v"(off), "s"(base) : "memory");
+    asm volatile("s_cmp_eq_u32 %3, 0\n\t"
+                 "s_cbranch_scc1 .Ldt_plain_%=\n\t"
+                 "global_load_dwordx4 %0, %1, %2 nt\n\t"
+                 "s_branch .Ldt_issued_%=\n"
+                 ".Ldt_plain_%=:\n\t"
+                 "global_load_dwordx4 %0, %1, %2\n"
+                 ".Ldt_issued_%=:"
+                 : "=&v"(v)
+                 : "v"(off), "s"(base), "s"(__builtin_amdgcn_readfirstlane(once))
+                 : "memory", "scc");
     return v;
 }
 
@@ -154,6 +166,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
     const int S = (U + 3) >> 2;      // steps
     const int tile0 = blockIdx.x * T;
     const int m0 = blockIdx.y * mrows;
+    const int once = gridDim.y == 1; // no other workgroup reads this one's weight records
     const int Mb = min(mrows, M - m0);
     const char *Xt = reinterpret_cast<const char *>(a.X);
     const char *Wt = reinterpret_cast<const char *>(a.W);
@@ -259,7 +272,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
             const uint32_t bk = (ragged && s == S - 1 && 4 * s + g >= U) ? back : 0u;
 #pragma unroll
             for (int t = 0; t < T; ++t)
-                wb[d][t] = dt_load16_once(wp, woff[t] - bk);
+                wb[d][t] = dt_load16_weights(wp, woff[t] - bk, once);
         }
         if (round == 0) {
             dt_wait_loads<D * T>(); // the activation loads are older than these
@@ -423,11 +436,11 @@ __device__ __forceinline__ void dt_dma_dword(const void *src, unsigned lds_addr)
 template <int P> struct DtgShare {
     v4u v[P / 4];
     static constexpr int kLoads = P / 4;
-    __device__ __forceinline__ void issue(const char *base, uint32_t off)
+    __device__ __forceinline__ void issue(const char *base, uint32_t off, int once)
     {
 #pragma unroll
         for (int i = 0; i < P / 4; ++i)
-            v[i] = dt_load16_once(base, off + 16u * i);
+            v[i] = dt_load16_weights(base, off + 16u * i, once);
     }
     __device__ __forceinline__ void landed()
     {
@@ -439,9 +452,18 @@ template <int P> struct DtgShare {
 template <> struct DtgShare<2> {
     v2u v;
     static constexpr int kLoads = 1;
-    __device__ __forceinline__ void issue(const char *base, uint32_t off)
+    __device__ __forceinline__ void issue(const char *base, uint32_t off, int once)
     {
-        asm volatile("global_load_dwordx2 %0, %1, %2 nt" : "=&v"(v) : "v"(off), "s"(base) : "memory");
+        asm volatile("s_cmp_eq_u32 %3, 0\n\t"
+                     "s_cbranch_scc1 .Ldt_plain_%=\n\t"
+                     "global_load_dwordx2 %0, %1, %2 nt\n\t"
+                     "s_branch .Ldt_issued_%=\n"
+                     ".Ldt_plain_%=:\n\t"
+                     "global_load_dwordx2 %0, %1, %2\n"
+                     ".Ldt_issued_%=:"
+                     : "=&v"(v)
+                     : "v"(off), "s"(base), "s"(__builtin_amdgcn_readfirstlane(once))
+                     : "memory", "scc");
     }
     __device__ __forceinline__ void landed() { asm volatile("" : "+v"(v)); }
 };
@@ -496,6 +518,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
     const int KT = a.K >> 7; // K tiles = scale groups = steps
     const int tile0 = blockIdx.x * T;
     const int m0 = blockIdx.y * mrows;
+    const int once = gridDim.y == 1; // no other workgroup reads this one's weight records
     const int Mb = min(mrows, M - m0);
     const char *Xt = reinterpret_cast<const char *>(a.X);
     const char *Wt = reinterpret_cast<const char *>(a.W);
@@ -593,7 +616,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
             const char *wp = Wt + (size_t)s * step_bytes;
 #pragma unroll
             for (int t = 0; t < T; ++t)
-                wb[d][t].issue(wp, woff[t]);
+                wb[d][t].issue(wp, woff[t], once);
         }
         if (round == 0) {
             dt_wait_loads<D * T * LPS>(); // the DMA loads (and the rows' fp16 units) are older than these
