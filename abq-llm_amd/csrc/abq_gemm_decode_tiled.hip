@@ -70,12 +70,12 @@ __device__ __forceinline__ v4u dt_load16(const char *base, uint32_t off)
 __device__ __forceinline__ v4u dt_load16_weights(const char *base, uint32_t off, int once)
 {
     v4u v;
-    asm volatile("s_cmp_eq_u32 %3, 0\n\t"
-                 "s_cbranch_scc1 .Ldt_plain_%=\n\t"
-                 "global_load_dwordx4 %0, %1, %2 nt\n\t"
+    asm volatile("s_cmp_lg_u32 %3, 0\n\t"
+                 "s_cbranch_scc1 .Ldt_once_%=\n\t"
+                 "global_load_dwordx4 %0, %1, %2\n\t"
                  "s_branch .Ldt_issued_%=\n"
-                 ".Ldt_plain_%=:\n\t"
-                 "global_load_dwordx4 %0, %1, %2\n"
+                 ".Ldt_once_%=:\n\t"
+                 "global_load_dwordx4 %0, %1, %2 nt\n"
                  ".Ldt_issued_%=:"
                  : "=&v"(v)
                  : "v"(off), "s"(base), "s"(__builtin_amdgcn_readfirstlane(once))
@@ -454,12 +454,12 @@ template <> struct DtgShare<2> {
     static constexpr int kLoads = 1;
     __device__ __forceinline__ void issue(const char *base, uint32_t off, int once)
     {
-        asm volatile("s_cmp_eq_u32 %3, 0\n\t"
-                     "s_cbranch_scc1 .Ldt_plain_%=\n\t"
-                     "global_load_dwordx2 %0, %1, %2 nt\n\t"
+        asm volatile("s_cmp_lg_u32 %3, 0\n\t"
+                     "s_cbranch_scc1 .Ldt_once_%=\n\t"
+                     "global_load_dwordx2 %0, %1, %2\n\t"
                      "s_branch .Ldt_issued_%=\n"
-                     ".Ldt_plain_%=:\n\t"
-                     "global_load_dwordx2 %0, %1, %2\n"
+                     ".Ldt_once_%=:\n\t"
+                     "global_load_dwordx2 %0, %1, %2 nt\n"
                      ".Ldt_issued_%=:"
                      : "=&v"(v)
                      : "v"(off), "s"(base), "s"(__builtin_amdgcn_readfirstlane(once))
