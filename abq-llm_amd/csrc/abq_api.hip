@@ -1472,7 +1472,8 @@ size_t abq_gemm_workspace_bytes(const abq_gemm_state *st)
     if (st->strategy == ABQ_STRATEGY_FP6)
         return (st->x_layout == ABQ_LAYOUT_FP6 ? 0 : fp6_bytes(st->M, st->K)) +
                (st->w_layout == ABQ_LAYOUT_FP6 ? 0 : fp6_bytes(st->N, st->K));
-    const size_t xb = st->x_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->M, st->K, st->cfg.x_bits);
+    // (fp16 activations are quantised inside the decode kernel: nothing is converted for them)
+    const size_t xb = (st->x_layout == ABQ_LAYOUT_TILED || st->x_layout == ABQ_LAYOUT_F16) ? 0 : planes_bytes(st->M, st->K, st->cfg.x_bits);
     const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, st->cfg.w_bits);
     return xb + wb;
 }
@@ -1580,10 +1581,13 @@ abq_status abq_gemm_set_workspace(abq_gemm_state *st, void *workspace, size_t by
     st->workspace_bytes = bytes;
     // (up to 64 rows, 32 on wide outputs, the conversion launch costs more than the LDS-staged kernel gains over the
     // 16-row tiles on plane operands: W2A8 32 x 4096 x 4096 12.6 against 8.7 us)
+    // A state on the decode kernel of prepared operands converts nothing and was weighed against the prefill kernel when
+    // it got there: it stays.  A state with group scales moves to the group-scale variants of the prefill kernel (the
+    // plain table's variant numbers mean other tiles there).
     const bool pays = st->group_size != 0 || st->M > 64 || (st->M > 32 && st->N >= 8192);
-    if (st->strategy != ABQ_STRATEGY_TILED && st->strategy != ABQ_STRATEGY_FP6 && st->auto_chosen && st->M > 16 && pays &&
-        workspace && bytes >= abq_gemm_workspace_bytes(st))
-        return switch_to_tiled(st);
+    if (st->strategy != ABQ_STRATEGY_TILED && st->strategy != ABQ_STRATEGY_FP6 && st->strategy != ABQ_STRATEGY_DECODE_TILED &&
+        st->auto_chosen && st->M > 16 && pays && workspace && bytes >= abq_gemm_workspace_bytes(st))
+        return st->group_size ? pick_grouped_tiled(st) : switch_to_tiled(st);
     return ABQ_OK;
 }
 

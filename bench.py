@@ -19,7 +19,8 @@ GEMM, recorded on the launch stream, brackets exactly that kernel's K launches; 
 is the same as K interleaved steps.  Each group of K launches is replayed from a HIP graph so
 the host launch rate does not bound the measurement.
 
-Prints ONE JSON line on stdout (everything else goes to stderr).
+Prints ONE short JSON line on stdout.  Progress and the side measurements go to stderr, the side measurements also
+as JSON into --extra-out (default gpurun_out/bench_extra.json).
 """
 import argparse
 import importlib.util
@@ -38,15 +39,83 @@ Q_BITS, P_BITS, SIGNED = 8, 2, True
 ROTATE_BYTES = 512 << 20
 
 
-# HBM bytes per launch of the dominant kernel, averaged over this workload's nine GEMMs, from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled by a plain copy of known size
-# (the summary with the commands is kept under profiles/, decode_w2a8_prepared_bench_hbm_traffic).  Reported only for the
-# kernel it was measured on.
-MEASURED_TRAFFIC_BYTES = {
-    "decode:AqBMMA_8x2xtrue_16x16x8192_16x16x512_16x16x64_3": 9358234,
-}
-# one figure for the whole headline workload when its GEMMs run on several tile tuples of one kernel family
-MEASURED_TRAFFIC_BYTES_DECODE_TILED = 9306992
+# HBM bytes per launch of the dominant kernel come from the rocprofv3 --pmc summary kept under profiles/ (two counter
+# runs of this script scaled by a plain copy of known size): the summary carries one line
+# `bench.py reads: kernel=<family> traffic_bytes_per_launch=<n>` (the kernel trace: `avg_dispatch_ns=<n>`) per measured
+# kernel family, and the figure is reported only for the family it was taken on.
+PROFILE_SUMMARIES = ("decode_w2a8_prepared_bench_hbm_traffic.md", "decode_w2a8_prepared_bench_kernel_trace.md")
+LINE_LIMIT = 4096  # the one stdout line must stay far below what a log tail keeps
+
+
+def profile_figures(family, directory=None):
+    """{'traffic_bytes_per_launch': n, 'avg_dispatch_ns': n, 'source': [...]} for a kernel family, from profiles/*.md."""
+    directory = directory or os.path.join(ROOT, "profiles")
+    out = {}
+    for name in PROFILE_SUMMARIES:
+        try:
+            text = open(os.path.join(directory, name)).read()
+        except OSError:
+            continue
+        for line in text.splitlines():
+            if "bench.py reads:" not in line:
+                continue
+            fields = dict(f.split("=", 1) for f in line.split("bench.py reads:", 1)[1].replace("`", " ").split() if "=" in f)
+            if fields.get("kernel") != family:
+                continue
+            for key in ("traffic_bytes_per_launch", "avg_dispatch_ns"):
+                if key in fields:
+                    out[key] = int(fields[key])
+                    out.setdefault("source", []).append("profiles/" + name)
+    return out
+
+
+def headline(value, steps, warmup, total_s, n_gemms, clock_settle_s, dominant, tuples, launches, bytes_per_launch,
+             avg_launch_us, cpu_tops, cpu_threads, cpu_sample, plane_operand_tops=None, extra_file=None, figures=None):
+    """The one JSON object bench.py prints on stdout.  Side measurements never go in here: they are written to a file
+    of their own (and logged on stderr), so that this line stays a few hundred bytes."""
+    figures = profile_figures(dominant) if figures is None else figures
+    achieved = bytes_per_launch / (avg_launch_us * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": figures.get("traffic_bytes_per_launch"),
+                "kernel": dominant + ":" + ",".join(sorted(set(t.split(":")[1] for t in tuples))),
+                "launches_per_step": launches,
+                "algorithmic_bytes_per_launch_avg": round(bytes_per_launch),
+                "avg_launch_us": round(avg_launch_us, 3)}
+    if "avg_dispatch_ns" in figures:
+        # an isolated dispatch under the profiler (no overlap with the next launch's ramp): the conservative figure
+        iso = bytes_per_launch / (figures["avg_dispatch_ns"] * 1e-9) / 1e9
+        roofline["kernel_trace_avg_us"] = round(figures["avg_dispatch_ns"] / 1e3, 3)
+        roofline["frac_kernel_trace"] = round(iso / HBM_PEAK_GBS, 4)
+    result = {
+        "metric": "effective int TOPS (2*M*N*K / t) over the LLaMA-7B W2A8 decode GEMMs, M in {1,4,8}",
+        "value": round(value, 4),
+        "unit": "TOPS",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(total_s * 1e3 / steps, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",  # packed fields unpacked to int8, int8 MFMA with int32 accumulation
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: W2A8 signed decode GEMM, M in {1,4,8} x (N,K) in "
+                               "{(4096,4096),(11008,4096),(4096,11008)}, int32 out, packed operands resident in HBM "
+                               "(K-tiled layout: weights prepared once, activations as the quantising kernel writes them)",
+                   "gemms_per_step": n_gemms, "x_bits": Q_BITS, "w_bits": P_BITS, "signed": SIGNED,
+                   "clock_settle_s": clock_settle_s},
+        "roofline": roofline,
+        "cpu_baseline": {"value": round(cpu_tops, 5), "unit": "TOPS", "cores": int(cpu_threads), "kind": "port",
+                         "sample": cpu_sample},
+    }
+    if plane_operand_tops is not None:  # the same GEMMs on the reference's plane layout (what this line measured at first)
+        result["plane_operands_value"] = round(plane_operand_tops, 4)
+    if extra_file:
+        result["extra_file"] = extra_file
+    line = json.dumps(result)
+    assert len(line) < LINE_LIMIT, "headline line grew to %d bytes" % len(line)
+    return line
 
 
 def log(*a):
@@ -101,6 +170,8 @@ def main():
     ap.add_argument("--extras", default=None,
                     help="comma-separated side measurements to run (default all): decode_plane_operands, prefill, prefill_fp6, library_int8_gemm, "
                          "decode_fused_linears, decode_group_scales, small_batch, decoder_layer_w2a8_group128")
+    ap.add_argument("--extra-out", default=os.path.join(ROOT, "gpurun_out", "bench_extra.json"),
+                    help="file the side measurements are written to as JSON ('' for none); they never go on stdout")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (the known-size kernel that "
                          "calibrates FETCH_SIZE / WRITE_SIZE in a counter run)")
@@ -233,12 +304,10 @@ def main():
         f["tuples"].append(name)
     dominant = max(families, key=lambda k: families[k]["us"])
     dg = families[dominant]
-    achieved = dg["bytes"] / (dg["us"] * 1e-6) / 1e9
     total_ops = sum(c["ops"] for c in cases) * K_STEPS
     value = total_ops / total_s / 1e12
-    for r in per_gemm:
-        log("M=%d N=%d K=%d  %.2f us  %.2f TOPS  %.0f GB/s (%.1f%% of HBM peak)  %s"
-            % (r["M"], r["N"], r["K"], r["us"], r["tops"], r["hbm_gbs"], 100 * r["hbm_frac"], r["kernel"]))
+    log("headline: %.2f TOPS over %d GEMMs x %d steps, %.3f us per launch (rows are logged at the end)"
+        % (value, len(cases), K_STEPS, dg["us"] / dg["launches"]))
 
     # ---------------------------------------------------------------- CPU baseline (bounded sample) + parity
     sys.path.insert(0, ROOT)
@@ -625,38 +694,28 @@ def main():
         extra["decoder_layer_w2a8_group128"] = layer
 
 
-    result = {
-        "metric": "effective int TOPS (2*M*N*K / t) over the LLaMA-7B W2A8 decode GEMMs, M in {1,4,8}",
-        "value": round(value, 4),
-        "unit": "TOPS",
-        "n_gpus": 1,
-        "steps": K_STEPS,
-        "warmup": W_STEPS,
-        "ms_per_step": round(total_s * 1e3 / K_STEPS, 5),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "int8",  # bit planes unpacked to int8, int8 MFMA with int32 accumulation
-        "data": "synthetic",
-        "config": {"workload": "BASELINE configs[1]: W2A8 signed decode GEMM, M in {1,4,8} x (N,K) in "
-                               "{(4096,4096),(11008,4096),(4096,11008)}, int32 out, packed operands resident in HBM "
-                               "(K-tiled layout: weights prepared once, activations as the quantising kernel writes them)",
-                   "gemms_per_step": len(cases), "x_bits": Q_BITS, "w_bits": P_BITS, "signed": SIGNED,
-                   "clock_settle_s": args.clock_settle_s},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": (MEASURED_TRAFFIC_BYTES_DECODE_TILED if dominant == "decode_tiled"
-                                 else MEASURED_TRAFFIC_BYTES.get(dg["tuples"][0]) if len(dg["tuples"]) == 1 else None),
-                     "kernel": dominant + ":" + ",".join(sorted(set(t.split(":")[1] for t in dg["tuples"]))),
-                     "launches_per_step": dg["launches"],
-                     "algorithmic_bytes_per_launch_avg": round(dg["bytes"] / dg["launches"]),
-                     "avg_launch_us": round(dg["us"] / dg["launches"], 3)},
-        "cpu_baseline": {"value": round(cpu_ops / cpu_s / 1e12, 5), "unit": "TOPS", "cores": int(cpu_threads),
-                         "kind": "port",
-                         "sample": "%d passes over the same 9 GEMMs (%.1f s), oracle popcount GEMM with OpenMP" % (reps, cpu_s)},
-        "extra": extra,
-    }
-    print(json.dumps(result), flush=True)
+    # ---------------------------------------------------------------- output
+    # side measurements: a file of their own (stderr already carries them line by line); the headline rows are logged
+    # last so that they are what a tail of stderr keeps
+    extra_file = None
+    if args.extra_out:
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(args.extra_out)), exist_ok=True)
+            with open(args.extra_out, "w") as f:
+                json.dump(extra, f, indent=1)
+            extra_file = os.path.relpath(os.path.abspath(args.extra_out), ROOT)
+        except OSError as exc:
+            log("side measurements not written (%r)" % (exc,))
+    for r in per_gemm:
+        log("M=%d N=%d K=%d  %.2f us  %.2f TOPS  %.0f GB/s (%.1f%% of HBM peak)  %s"
+            % (r["M"], r["N"], r["K"], r["us"], r["tops"], r["hbm_gbs"], 100 * r["hbm_frac"], r["kernel"]))
+    plane_tops = None
+    if "decode_plane_operands" in extra:
+        plane_tops = sum(c["ops"] for c in cases) / sum(r["us"] * 1e-6 for r in extra["decode_plane_operands"]) / 1e12
+    print(headline(value, K_STEPS, W_STEPS, total_s, len(cases), args.clock_settle_s, dominant, dg["tuples"],
+                   dg["launches"], dg["bytes"] / dg["launches"], dg["us"] / dg["launches"], cpu_ops / cpu_s, cpu_threads,
+                   "%d passes over the same 9 GEMMs (%.1f s), oracle popcount GEMM with OpenMP" % (reps, cpu_s),
+                   plane_operand_tops=plane_tops, extra_file=extra_file), flush=True)
 
 
 if __name__ == "__main__":

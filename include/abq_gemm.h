@@ -348,9 +348,10 @@ abq_status abq_gemm_set_f16_activations(abq_gemm_state *state, const void *x_f16
  * reference, whose activations are quantised by a kernel of their own (abq_gemm_wrapper.cu:29-69). */
 abq_status abq_gemm_set_dynamic_f16_activations(abq_gemm_state *state, const void *x_f16, int symmetric);
 
-/* Workspace needed by abq_gemm_exec if the state ran as ABQ_STRATEGY_TILED (ABQ_STRATEGY_FP6)
- * with its current operand layouts: the converted copies of the operands still in the reference
- * layout (0 if neither is). */
+/* Workspace needed by abq_gemm_exec if the state ran as ABQ_STRATEGY_TILED, ABQ_STRATEGY_DECODE_TILED
+ * (ABQ_STRATEGY_FP6) with its current operand layouts: the converted copies of the operands still in
+ * the reference layout.  Operands declared K-tiled (FP6 records) count 0, and so do fp16 activations
+ * handed to the decode kernel (ABQ_LAYOUT_F16: quantised inside the kernel, nothing is converted). */
 size_t abq_gemm_workspace_bytes(const abq_gemm_state *state);
 
 /* Hands a caller-owned device buffer to the state.  If the tile was the library's choice, M > 64

@@ -277,6 +277,12 @@ def test_group_scale_decode_kernel_over_row_blocks(abq, oracle, q, p, signed):
         got = g.run()
         torch.cuda.synchronize()
         assert_close_rel(got.cpu().numpy(), want)
+        if (M, N, K) == (32, 4096, 4096):
+            # layouts -> scales -> workspace: a workspace the state does not need leaves it on the same kernel
+            ws = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+            g2 = abq.Gemm(xt, wt, signed, out_kind=abq.OUT_F16_SCALED, workspace=ws, **kw)
+            assert (g2.strategy, g2.config_name) == (g.strategy, g.config_name)
+            assert torch.equal(g2.run(), got)
     # what the estimate decides on the decoder-layer linears (W2A8: the narrow outputs only)
     if (q, p, signed) == (8, 2, True):
         assert abq.prepared_decode_pays(8, 2, True, 32, 4096, 4096, 128) and abq.prepared_decode_pays(8, 2, True, 32, 4096, 11008, 128)

@@ -405,6 +405,42 @@ def test_group_scales_move_a_state_to_the_kernel_that_carries_them(abq):
     assert bytes(st) == before
 
 
+def test_workspace_after_layouts_and_scales_keeps_a_consistent_state(abq):
+    """layouts -> scales -> workspace at 32 rows: a state on the prepared-operand decode kernel stays there (it converts
+    nothing), and a group-scale state that does move lands on a variant of the group-scale table."""
+    lib = abq.lib()
+    T = abq.LAYOUT_TILED
+    names = abq.STRATEGY_NAMES
+    for (N, K) in ((4096, 4096), (4096, 11008)):
+        rc, st = _init(abq, q=8, p=2, M=32, signed=1, N=N, K=K, out_kind=abq.OUT_F16_SCALED)
+        assert rc == 0
+        assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0
+        assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 128) == 0
+        assert names[st.strategy] == "decode_tiled" and st.variant == 0
+        before = (st.strategy, st.variant, st.cfg.as_tuple())
+        assert lib.abq_gemm_set_workspace(ctypes.byref(st), 0x100000, 1 << 20) == 0
+        assert (st.strategy, st.variant, st.cfg.as_tuple()) == before
+        assert lib.abq_gemm_workspace_bytes(ctypes.byref(st)) == 0
+    # without group scales: 65 to 128 rows on the decode kernel stay there as well
+    rc, st = _init(abq, q=4, p=4, M=64, signed=1, N=4096, K=4096)
+    assert rc == 0 and lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0
+    assert names[st.strategy] == "decode_tiled"
+    assert lib.abq_gemm_set_workspace(ctypes.byref(st), 0x100000, 1 << 20) == 0 and names[st.strategy] == "decode_tiled"
+    # plane operands with group scales at 32 rows (the group-scale prefill kernel from the start): the workspace call
+    # keeps the variant inside the group-scale table
+    rc, st = _init(abq, q=8, p=2, M=32, signed=1, N=4096, K=4096, out_kind=abq.OUT_F16_SCALED)
+    assert rc == 0 and lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 128) == 0
+    assert names[st.strategy] == "tiled"
+    v = st.variant
+    assert lib.abq_gemm_set_workspace(ctypes.byref(st), 0x100000, 64 << 20) == 0
+    assert names[st.strategy] == "tiled" and st.variant == v
+    # fp16 activations handed to the decode kernel are not converted: no workspace asked for them
+    rc, st = _init(abq, q=8, p=2, M=4, signed=1, N=4096, K=4096)
+    assert rc == 0 and lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0
+    assert lib.abq_gemm_set_f16_activations(ctypes.byref(st), 0x200000, 0x300000) == 0
+    assert lib.abq_gemm_workspace_bytes(ctypes.byref(st)) == 0
+
+
 def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     """The tile the library picks for prepared operands, pinned on shapes of BASELINE.json configs[2] and
     configs[4] and on a few where the measured sweep of all tiles separates them clearly:
