@@ -36,6 +36,7 @@ EXPORTED = [
     "abq_gemm_set_workspace", "abq_fp6_bytes", "abq_fp6_eligible", "abq_prepared_decode_pays", "abq_gemm_set_dynamic_f16_activations", "abq_relayout_planes_fp6",
     "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16", "abq_gemm_set_activation",
     "abq_probe_launch", "abq_gemm_exec_static", "abq_gemm_set_f16_activations",
+    "abq_row_sums", "abq_gemm_set_row_sums", "abq_gemm_row_sums_ready",
 ]
 
 
@@ -74,6 +75,7 @@ class GemmState(ctypes.Structure):
         ("x_group_sums", ctypes.c_void_p), ("w_zero_term", ctypes.c_void_p),
         ("act", ctypes.c_int),
         ("x_pack_scale", ctypes.c_void_p),
+        ("x_row_sums", ctypes.c_void_p), ("w_row_sums", ctypes.c_void_p),
     ]
 
 
@@ -130,6 +132,10 @@ def lib():
         L.abq_gemm_workspace_bytes.restype = ctypes.c_size_t
         L.abq_gemm_set_workspace.argtypes = [ctypes.POINTER(GemmState), vp, ctypes.c_size_t]
         L.abq_gemm_set_zero_points.argtypes = [ctypes.POINTER(GemmState), vp, vp, vp, vp]
+        L.abq_row_sums.argtypes = [vp, ci, ci, ci, vp, vp]
+        L.abq_gemm_set_row_sums.argtypes = [ctypes.POINTER(GemmState), vp, vp]
+        L.abq_gemm_row_sums_ready.argtypes = [ctypes.POINTER(GemmState)]
+        L.abq_gemm_row_sums_ready.restype = ci
         L.abq_gemm_set_activation.argtypes = [ctypes.POINTER(GemmState), ci]
         L.abq_weight_zero_term.argtypes = [vp, ci, ci, ci, ci, vp, vp, ci, vp, vp]
         L.abq_quant_pack_f16.argtypes = [vp, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, vp]
@@ -227,6 +233,17 @@ def relayout_planes(planes, out=None, stream=None):
     return out
 
 
+def row_sums(planes, stream=None):
+    """planes int32 tensor [bits, rows, k/32] -> int32 [rows]: the sum over k of each row's unsigned codes (what the
+    staged kernel wants handed in for pairs with an unsigned 8-bit operand)."""
+    import torch
+    bits, rows, kw = planes.shape
+    assert planes.is_cuda and planes.is_contiguous()
+    out = torch.empty(rows, dtype=torch.int32, device=planes.device)
+    _check(lib().abq_row_sums(planes.data_ptr(), rows, kw * 32, bits, out.data_ptr(), _stream_ptr(stream)), "abq_row_sums")
+    return out
+
+
 def fp6_eligible(x_bits, w_bits, signed, k):
     """Whether the FP6 matrix-core route is exact for this bit pair and K (host-side check)."""
     return bool(lib().abq_fp6_eligible(x_bits, w_bits, int(bool(signed)), k))
@@ -292,7 +309,7 @@ class Gemm:
     def __init__(self, x_planes, w_planes, signed, out=None, cfg=None, out_kind=OUT_I32, c_scale=None,
                  x_scale=None, w_scale=None, group_size=0, x_tiled=False, w_tiled=False, workspace=None,
                  x_zero=None, w_zero=None, x_group_sums=None, w_zero_term=None, act=ACT_NONE,
-                 x_fp6=0, w_fp6=0):
+                 x_fp6=0, w_fp6=0, x_row_sums=None, w_row_sums=None):
         import torch
         if x_fp6:
             kt, M, _ = x_planes.shape
@@ -338,6 +355,10 @@ class Gemm:
             _check(lib().abq_gemm_set_operand_layout(ctypes.byref(self.state), xl, wl), "abq_gemm_set_operand_layout")
         if act != ACT_NONE:
             _check(lib().abq_gemm_set_activation(ctypes.byref(self.state), act), "abq_gemm_set_activation")
+        self.row_sums = (x_row_sums, w_row_sums)
+        if x_row_sums is not None or w_row_sums is not None:
+            _check(lib().abq_gemm_set_row_sums(ctypes.byref(self.state), x_row_sums.data_ptr() if x_row_sums is not None else None,
+                                               w_row_sums.data_ptr() if w_row_sums is not None else None), "abq_gemm_set_row_sums")
         self.workspace = workspace
         if workspace is not None:
             _check(lib().abq_gemm_set_workspace(ctypes.byref(self.state), workspace.data_ptr(),
@@ -346,6 +367,11 @@ class Gemm:
     @property
     def workspace_bytes(self):
         return lib().abq_gemm_workspace_bytes(ctypes.byref(self.state))
+
+    @property
+    def row_sums_ready(self):
+        """True if run() launches the staged kernel that takes the row sums of an unsigned 8-bit pair handed in."""
+        return bool(lib().abq_gemm_row_sums_ready(ctypes.byref(self.state)))
 
     @property
     def strategy(self):

@@ -19,6 +19,7 @@ hipError_t launch_pack_f16_tiled(const void *, const float *, uint32_t *, int, i
 hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes_fp6(const uint32_t *, uint32_t *, int, int, int, int, hipStream_t);
+hipError_t launch_row_sums(const uint32_t *, int *, int, int, int, hipStream_t);
 const KernelEntry *fp6_entries(int *count);
 const KernelEntry *fp6_grouped_entries(int *count);
 hipError_t launch_quant_pack_rows(const void *, uint32_t *, float *, float *, int *, int, int, int, int, int, int,
@@ -604,8 +605,12 @@ static int native_config(int x_bits, int w_bits, int is_signed, int index, abq_t
         const KernelEntry &e = tm->entries[index - (n - tm->count)];
         entry_to_config(e, e.mi == 16 ? ABQ_STRATEGY_MFMA16 : ABQ_STRATEGY_MFMA32, x_bits, w_bits, is_signed, 0, cfg);
     }
-    if (in(tt->count))
-        entry_to_config(tt->entries[index - (n - tt->count)], ABQ_STRATEGY_TILED, x_bits, w_bits, is_signed, 0, cfg);
+    // (entries that want row sums handed in stand behind the kernel of the same tuple, at the end: no tuples of their own)
+    int tt_count = tt->count;
+    while (tt_count > 0 && (tt->entries[tt_count - 1].flags & kNeedsRowSums))
+        --tt_count;
+    if (in(tt_count))
+        entry_to_config(tt->entries[index - (n - tt_count)], ABQ_STRATEGY_TILED, x_bits, w_bits, is_signed, 0, cfg);
     if (fp6_eligible(x_bits, w_bits, is_signed, 128)) {
         int nfp6 = 0;
         const KernelEntry *es = fp6_entries(&nfp6);
@@ -742,11 +747,12 @@ static int large_tiles_int8(int x_bits, int w_bits, int is_signed, const LargeTi
     static const LargeTile wide_n[] = { { 2, 4, 4, 2, 1.06, 1.06 } };
     static const LargeTile w8a8[] = { { 2, 2, 4, 2, 1.20, 1.20 } };
     const bool field = (x_bits == 2 || x_bits == 4 || x_bits == 8) && (w_bits == 2 || w_bits == 4 || w_bits == 8);
+    (void)is_signed; // (the staged kernel serves unsigned 8-bit operands too, given their row sums)
     if (x_bits == 8 && w_bits == 8) {
         *out = w8a8;
-        return is_signed ? 1 : 0;
+        return 1;
     }
-    if (field && x_bits >= w_bits && (is_signed || x_bits < 8)) {
+    if (field && x_bits >= w_bits) {
         *out = wide_n;
         return 1;
     }
@@ -770,7 +776,7 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
                                     { 1, 1, 2, 2, 0 } };
     // signed W8A8 below 200 tiles of 128x128: the staged kernel's 256x128 tile pays as soon as it covers about two
     // thirds of the compute units
-    const bool staged = c.x_bits == 8 && c.w_bits == 8 && c.is_signed;
+    const bool staged = c.x_bits == 8 && c.w_bits == 8;
     int pick = -1;
     const LargeTile *cands = nullptr;
     const int ncands = large_tiles_int8(c.x_bits, c.w_bits, c.is_signed, &cands);
@@ -1299,6 +1305,67 @@ abq_status abq_gemm_exec_static(const abq_gemm_state *st, void *stream)
     return abq_gemm_exec(&local, stream);
 }
 
+// Row sums of the operands of a state whose kernel wants them handed in (kNeedsRowSums): which are needed, which
+// the caller has set, and where in the workspace (behind `converted` bytes of converted operands) those are put that
+// the library can take itself, which it can only from an operand still in the reference's plane layout.
+struct RowSumPlan {
+    bool ok;             // every needed sum is set or can be taken into the workspace the state holds
+    size_t x_off, w_off; // byte offsets into the workspace
+    size_t bytes;        // workspace the sums need on top of the converted operands
+};
+
+static RowSumPlan row_sum_plan(const abq_gemm_state *st, size_t converted)
+{
+    const abq_tile_config &c = st->cfg;
+    RowSumPlan p{ true, 0, 0, 0 };
+    const bool take_x = c.w_bits == 8 && !st->x_row_sums, take_w = c.x_bits == 8 && !st->w_row_sums;
+    if ((take_x && st->x_layout != ABQ_LAYOUT_PLANES) || (take_w && st->w_layout != ABQ_LAYOUT_PLANES))
+        p.ok = false;
+    p.x_off = (converted + 255) / 256 * 256;
+    p.w_off = p.x_off + (take_x ? ((size_t)st->M * 4 + 255) / 256 * 256 : 0);
+    const size_t end = p.w_off + (take_w ? (size_t)st->N * 4 : 0);
+    p.bytes = (take_x || take_w) ? end - converted : 0;
+    if (p.bytes && (!st->workspace || converted + p.bytes > st->workspace_bytes))
+        p.ok = false;
+    return p;
+}
+
+// Whether the state's kernel is one that wants row sums handed in.
+static bool wants_row_sums(const abq_gemm_state *st)
+{
+    if (st->strategy != ABQ_STRATEGY_TILED || st->group_size || st->cfg.is_signed || (st->cfg.x_bits != 8 && st->cfg.w_bits != 8))
+        return false;
+    const KernelTable *t = find_table(registry().tiled, st->cfg.x_bits, st->cfg.w_bits, 0);
+    return t && st->variant >= 0 && st->variant < t->count && (t->entries[st->variant].flags & kNeedsRowSums);
+}
+
+abq_status abq_row_sums(const uint32_t *planes, int rows, int k, int bits, int32_t *sums, void *stream)
+{
+    if (!planes || !sums || rows <= 0 || bits < 1 || bits > 8)
+        return ABQ_ERR_INVALID_ARG;
+    if (k < 128 || k % 128 != 0)
+        return ABQ_ERR_BAD_K;
+    return hip_status(launch_row_sums(planes, sums, rows, k, bits, (hipStream_t)stream));
+}
+
+int abq_gemm_row_sums_ready(const abq_gemm_state *st)
+{
+    if (!st || !st->init_success || !wants_row_sums(st))
+        return 0;
+    const size_t xb = st->x_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->M, st->K, st->cfg.x_bits);
+    const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, st->cfg.w_bits);
+    return row_sum_plan(st, xb + wb).ok ? 1 : 0;
+}
+
+abq_status abq_gemm_set_row_sums(abq_gemm_state *st, const int32_t *x_row_sums, const int32_t *w_row_sums)
+{
+    if (!st || !st->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    st->x_row_sums = x_row_sums;
+    st->w_row_sums = w_row_sums;
+    return ABQ_OK;
+}
+
 abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
 {
     if (!st || !st->init_success)
@@ -1327,6 +1394,8 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     a.w_zero_term = st->w_zero_term;
     a.x_pack_scale = st->x_pack_scale;
     a.x_dynamic = st->x_layout == ABQ_LAYOUT_F16 ? st->reserved[1] : 0;
+    a.x_row_sums = st->x_row_sums;
+    a.w_row_sums = st->w_row_sums;
     const Registry &reg = registry();
     const abq_tile_config &c = st->cfg;
     hipError_t e;
@@ -1396,7 +1465,41 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
                                           c.x_bits, c.w_bits, c.is_signed);
         if (!t || st->variant < 0 || st->variant >= t->count)
             return ABQ_ERR_NOT_INITIALIZED;
-        e = t->entries[st->variant].launch(a, (hipStream_t)stream);
+        int variant = st->variant;
+        if (t->entries[variant].flags & kNeedsRowSums) {
+            // An unsigned 8-bit operand is fed as value - 128 and the other operand's row sums put the result right.
+            // The sums the caller set are taken; those of an operand still in planes are taken here, into the
+            // workspace behind the converted copies, if it has the room.  Otherwise the kernel of the same tile
+            // that gathers the sums itself runs.
+            const bool need_x = c.w_bits == 8, need_w = c.x_bits == 8;
+            const RowSumPlan plan = row_sum_plan(st, xb + wb);
+            if (plan.ok) {
+                if (need_x && !st->x_row_sums) {
+                    e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, c.x_bits, (hipStream_t)stream);
+                    if (e != hipSuccess)
+                        return hip_status(e);
+                }
+                if (need_w && !st->w_row_sums) {
+                    e = launch_row_sums(st->W, reinterpret_cast<int *>(ws + plan.w_off), st->N, st->K, c.w_bits, (hipStream_t)stream);
+                    if (e != hipSuccess)
+                        return hip_status(e);
+                }
+                a.x_row_sums = !need_x ? nullptr : st->x_row_sums ? st->x_row_sums : reinterpret_cast<const int *>(ws + plan.x_off);
+                a.w_row_sums = !need_w ? nullptr : st->w_row_sums ? st->w_row_sums : reinterpret_cast<const int *>(ws + plan.w_off);
+            } else {
+                variant = -1;
+                const KernelEntry &want = t->entries[st->variant];
+                for (int i = 0; i < st->variant; ++i) {
+                    const KernelEntry &o = t->entries[i];
+                    if (!(o.flags & kNeedsRowSums) && o.tm == want.tm && o.tn == want.tn && o.wm == want.wm && o.wn == want.wn &&
+                        o.wk == want.wk && o.kb == want.kb)
+                        variant = i;
+                }
+                if (variant < 0)
+                    return ABQ_ERR_NOT_INITIALIZED;
+            }
+        }
+        e = t->entries[variant].launch(a, (hipStream_t)stream);
     } else {
         if (st->group_size && st->strategy != ABQ_STRATEGY_DECODE)
             return ABQ_ERR_NOT_INITIALIZED; // group scales live on the decode and tiled kernels only
@@ -1475,7 +1578,8 @@ size_t abq_gemm_workspace_bytes(const abq_gemm_state *st)
     // (fp16 activations are quantised inside the decode kernel: nothing is converted for them)
     const size_t xb = (st->x_layout == ABQ_LAYOUT_TILED || st->x_layout == ABQ_LAYOUT_F16) ? 0 : planes_bytes(st->M, st->K, st->cfg.x_bits);
     const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, st->cfg.w_bits);
-    return xb + wb;
+    // (pairs with an unsigned 8-bit operand on the staged kernel: the row sums of the operands still in planes)
+    return xb + wb + (wants_row_sums(st) ? row_sum_plan(st, xb + wb).bytes : 0);
 }
 
 abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_layout)

@@ -12,9 +12,12 @@
 //             stay packed in LDS; a wave turns the field words of its own fragments into int8 with a
 //             shift and a mask per four elements right before the MFMA that uses them (8-bit
 //             operands need nothing).  Signed operands are placed at the top of the byte and the
-//             result shifted right by 16 - q - p, unsigned ones (at most 4 bits here) are fed as they
-//             are.  Pairs with an unsigned 8-bit operand (bit 7 to flip and row sums to take after
-//             every LDS read: measured slower than what the staging saves) and the widths made of
+//             result shifted right by 16 - q - p, unsigned ones of at most 4 bits are fed as they
+//             are.  An unsigned 8-bit operand is fed as value - 128 (bit 7 flipped after the LDS read,
+//             one xor per dword of the operand) and the result corrected in the epilogue with 128 x the
+//             other operand's row sums, which the kernel does not take itself (gathering them beside
+//             the MFMAs cost more than the staging saved): they come in through GemmArgs, computed once
+//             per weight matrix and once per activation block by abq_row_sums.  The widths made of
 //             several fields (3, 5, 6, 7 bits) stay on the kernel of abq_gemm_tiled.hip.
 //
 // global_load_lds_dwordx4 writes a wave's 64 x 16 bytes straight into LDS (at M0 + 16 * lane): no
@@ -77,7 +80,11 @@ template <int BITS, bool FP6> struct StagedOperand {
 template <int BITS, bool SIGNED> __device__ __forceinline__ v4i staged_int8_operand(const v4i *piece, int c)
 {
     if constexpr (BITS == 8) {
-        return piece[c];
+        if constexpr (SIGNED)
+            return piece[c];
+        else // value - 128
+            return v4i{ piece[c][0] ^ (int)0x80808080u, piece[c][1] ^ (int)0x80808080u, piece[c][2] ^ (int)0x80808080u,
+                        piece[c][3] ^ (int)0x80808080u };
     } else if constexpr (BITS == 4) {
         // step c <- words 2c, 2c + 1 of the lane's eight; each word holds two expanded dwords
         const uint32_t w0 = (uint32_t)piece[c / 2][2 * (c % 2)], w1 = (uint32_t)piece[c / 2][2 * (c % 2) + 1];
@@ -166,7 +173,8 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     constexpr int NPW = NPR + (GROUPED ? 1 : 0);               // GROUPED: and one load of 64 scales (256 bytes)
     static_assert(!GROUPED || (TM * TN >= 2 && BN / 64 <= WM * WN), "group scales: two MFMA tiles per wave or more");
     constexpr int kSteps = FP6 ? 2 : 4;                        // MFMA K steps per tile of 128
-    static_assert(FP6 || SIGNED || (QB < 8 && PB < 8), "unsigned 8-bit operands are not handled here");
+    constexpr bool FLIP_X = !FP6 && !SIGNED && QB == 8, FLIP_W = !FP6 && !SIGNED && PB == 8; // fed as value - 128
+    static_assert(!GROUPED || !(FLIP_X || FLIP_W), "no group scales on unsigned 8-bit operands");
     static_assert(S >= 3 && S <= 4, "three or four LDS stages");
     static_assert(NPW * S < 64, "the load counter has six bits");
     static_assert(BUF_BYTES % 512 == 0 && (BM * TA::kRow) % 512 == 0 && (32 * TA::kRow) % 256 == 0 && (32 * TB::kRow) % 256 == 0,
@@ -497,6 +505,27 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
         return;
     }
 
+    // Unsigned 8-bit operands were fed as value - 128: sum (x - 128) w = sum x w - 128 sum w, and likewise for the
+    // weights; with both, 2^14 K comes on top.  The correction of a column (row) is the same for all its elements.
+    if constexpr (FLIP_X || FLIP_W) {
+        int col_fix[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            unsigned v = FLIP_X ? 128u * (unsigned)a.w_row_sums[min(n0 + wn * 32 * TN + j * 32 + r, N - 1)] : 0u;
+            if (FLIP_X && FLIP_W)
+                v -= 16384u * (unsigned)(ktot * 128);
+            col_fix[j] = (int)v;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int row_fix = FLIP_W ? (int)(128u * (unsigned)a.x_row_sums[min(m0 + wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4), M - 1)]) : 0;
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j][e] = (int)((unsigned)acc[i][j][e] + (unsigned)row_fix + (unsigned)col_fix[j]);
+            }
+    }
     auto result = [&](int i, int j, int e) -> int {
         if constexpr (FP6)
             return (int)(acc[i][j][e] * 64.0f); // both operands carry 1/8 as their unit: the sum is the result / 64, exactly

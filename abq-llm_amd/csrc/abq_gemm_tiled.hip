@@ -482,7 +482,7 @@ static hipError_t launch_mfma_tiled(const GemmArgs &a, hipStream_t stream)
 #define ABQ_GENTRY_T(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, true, TM, TN, true, 128>, 128 },
 #define ABQ_GENTRY_F(TM, TN) { 32, TM, TN, 2, 2, 1, 4, &launch_mfma_tiled<ABQ_Q, ABQ_P, false, TM, TN, true, 128>, 128 },
 
-// Pairs of single-field widths (2, 4, 8 bits; unsigned only up to 4) run the tiles that the staged kernel
+// Pairs of single-field widths (2, 4, 8 bits) run the tiles that the staged kernel
 // (abq_gemm_staged.h: records loaded straight into LDS, unpacked by the waves after the LDS read) is built
 // for on that kernel, under the same tile tuples; the other tiles and pairs keep the kernel above.
 #define ABQ_FIELD1(B) ((B) == 2 || (B) == 4 || (B) == 8)
@@ -528,8 +528,21 @@ static const KernelEntry kUnsigned[] = { ABQ_ENTRY_F(4, 4) ABQ_ENTRY_F(2, 4) ABQ
                                          ABQ_SENTRY(false, 2, 2, 4, 2) ABQ_WENTRY_F(2, 2, 4, 4) ABQ_STAGED_256(false)
                                          ABQ_STAGED_WIDE_N(false) ABQ_STAGED_KSPLIT(false) };
 #else
+// Pairs with an unsigned 8-bit operand: the kernel above under every tuple, which takes the row sums of the
+// correction itself, and behind it, under the same tuples, the staged kernel for the tiles it is built for, which
+// wants them handed in (abq_row_sums; the host launches it when it has them).
+#define ABQ_SENTRY_U8(TM, TN, WM, WN)                                                           \
+    { 32, TM, TN, WM, WN, 1, 4, &launch_mfma_staged<ABQ_Q, ABQ_P, false, false, TM, TN, WM, WN>, 128, \
+      StagedStages<ABQ_Q, ABQ_P, false, TM, TN, WM, WN>::kLds, kNeedsRowSums },
+#if ABQ_Q == 8 && ABQ_P == 8
+#define ABQ_STAGED_U8_LARGE
+#else
+#define ABQ_STAGED_U8_LARGE ABQ_SENTRY_U8(2, 4, 4, 2)
+#endif
 static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_F)
-                                         ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_F) };
+                                         ABQ_TILED_WIDE_VARIANTS(ABQ_WENTRY_F)
+                                         ABQ_SENTRY_U8(2, 2, 2, 2) ABQ_SENTRY_U8(2, 1, 2, 2) ABQ_SENTRY_U8(1, 1, 2, 2)
+                                         ABQ_SENTRY_U8(2, 2, 4, 2) ABQ_STAGED_U8_LARGE };
 #endif
 #else
 static const KernelEntry kSigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_T) ABQ_TILED_HALF_VARIANTS(ABQ_HENTRY_T)

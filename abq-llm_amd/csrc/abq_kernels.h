@@ -29,6 +29,11 @@ struct GemmArgs {
     const float *w_zero_term;  // [N] sum_g w_scale * (sum of weight codes - group_size * w_zero) (needed with x_zero)
     const float *x_pack_scale; // kernels that quantise fp16 activations themselves: X is fp16 [M][K], this the static scale
     int x_dynamic;             // ... or, per token from the rows' own extrema: 1 symmetric, 2 with a zero point; 0: not
+    // sums over K of the unsigned codes of every row, for kernels that feed an unsigned 8-bit operand as value - 128
+    // and take no sums themselves (entries with kNeedsRowSums): D = acc + 128 (w sums if X is 8 bits wide)
+    // + 128 (x sums if W is) - 2^14 K (if both are)
+    const int *x_row_sums;     // [M]
+    const int *w_row_sums;     // [N]
 };
 
 typedef hipError_t (*GemmLauncher)(const GemmArgs &, hipStream_t);
@@ -42,7 +47,10 @@ struct KernelEntry {
     GemmLauncher launch;
     int kb;                 // K elements per LDS stage (tiled kernel); 0 where it does not apply
     size_t lds;             // dynamic LDS of the launch where the kernel fixes it itself; 0: derived from the tile
+    int flags;              // kNeedsRowSums: reads GemmArgs::x_row_sums / w_row_sums; the entry of the same tile tuple
+                            // in front of it in the table is the kernel that runs when the sums are not to be had
 };
+constexpr int kNeedsRowSums = 1;
 
 struct KernelTable {
     int x_bits, w_bits, is_signed;

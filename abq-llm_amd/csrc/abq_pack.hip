@@ -335,6 +335,40 @@ __global__ __launch_bounds__(256) void relayout_planes_fp6_kernel(const uint32_t
     }
 }
 
+// sums[row] = sum over K of the unsigned codes of a row (bit b of an element counts 2^b): one wave per row, the
+// plane words read as 16-byte units along the lanes, a popcount per word and plane.  What the kernels that feed an
+// unsigned 8-bit operand as value - 128 add back in their epilogue (GemmArgs::x_row_sums / w_row_sums).
+__global__ __launch_bounds__(256) void row_sums_kernel(const uint32_t *__restrict__ planes, int *__restrict__ sums, int rows,
+                                                       int KW, int bits)
+{
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows)
+        return; // whole waves, no barrier below
+    const size_t plane_stride = (size_t)rows * KW;
+    unsigned total = 0;
+    for (int b = 0; b < bits; ++b) {
+        const uint4 *p = reinterpret_cast<const uint4 *>(planes + b * plane_stride + (size_t)row * KW);
+        unsigned ones = 0;
+        for (int u = lane; u < KW / 4; u += 64) {
+            const uint4 v = p[u];
+            ones += __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
+        }
+        total += ones << b;
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1)
+        total += __shfl_xor(total, d);
+    if (lane == 0)
+        sums[row] = (int)total;
+}
+
+hipError_t launch_row_sums(const uint32_t *planes, int *sums, int rows, int k, int bits, hipStream_t stream)
+{
+    hipLaunchKernelGGL(row_sums_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, planes, sums, rows, k / 32, bits);
+    return hipGetLastError();
+}
+
 hipError_t launch_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int rows, int k, int bits, int is_signed,
                                       hipStream_t stream)
 {

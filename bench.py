@@ -13,11 +13,10 @@ The 256 MB Infinity Cache is defeated by rotation: every shape owns >= 512 MiB o
 weight buffers and consecutive launches walk through them, so a buffer is revisited only after
 more than the cache's capacity of other weights has streamed through.
 
-Timed region: K steps = K launches of each of the 9 GEMMs.  The launches are issued GEMM by
-GEMM (K launches of the first, then K of the second, ...) so that one pair of HIP events per
-GEMM, recorded on the launch stream, brackets exactly that kernel's K launches; the total work
-is the same as K interleaved steps.  Each group of K launches is replayed from a HIP graph so
-the host launch rate does not bound the measurement.
+Timed region: exactly K steps, a step being one launch of each of the 9 GEMMs in turn, replayed from one HIP
+graph so the host launch rate does not bound the measurement, bracketed by one pair of HIP events on the launch
+stream: the average launch duration of the roofline is that interval over 9 K launches.  The per-GEMM rows on
+stderr come from one graph per GEMM (K launches of it), replayed after the timed region.
 
 Prints ONE short JSON line on stdout.  Progress and the side measurements go to stderr, the side measurements also
 as JSON into --extra-out (default gpurun_out/bench_extra.json).
@@ -225,14 +224,26 @@ def main():
         for s in range(count):
             g[(offset + s) % len(g)].run()
 
-    # ---------------------------------------------------------------- HIP graphs (one per GEMM)
+    # ---------------------------------------------------------------- HIP graphs
+    # The timed region is ONE graph that holds the K steps as they run in a model (GEMM 1 .. 9, then again), so a
+    # replay's own launch cost is spread over 9 K launches; one graph per GEMM (K launches of it) gives the per-GEMM
+    # rows afterwards, outside the timed region.
     use_graph = not args.no_graph
-    graphs = []
+    graphs, step_graph = [], None
+
+    def launch_steps(count, offset=0):
+        for s in range(count):
+            for case in cases:
+                g = case["gemms"]
+                g[(offset + s) % len(g)].run()
+
     if use_graph:
         try:
-            for case in cases:
-                launch_group(case, 2)
+            launch_steps(2)
             torch.cuda.synchronize()
+            step_graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(step_graph):
+                launch_steps(K_STEPS)
             for case in cases:
                 gr = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(gr):
@@ -240,7 +251,7 @@ def main():
                 graphs.append(gr)
         except Exception as e:  # noqa: BLE001
             log("HIP graph capture failed (%r); falling back to plain stream launches" % (e,))
-            use_graph, graphs = False, []
+            use_graph, graphs, step_graph = False, [], None
             torch.cuda.synchronize()
 
     if args.pmc_copy_mib:
@@ -256,21 +267,31 @@ def main():
     # milliseconds of work to get there; the first launch of a graph also uploads it): untimed passes over the same
     # launches for CLOCK_SETTLE_S, then the W warm-up steps of the contract.
     def one_pass():
-        for i, case in enumerate(cases):
-            if use_graph:
-                graphs[i].replay()
-            else:
-                launch_group(case, K_STEPS)
+        if use_graph:
+            step_graph.replay()
+        else:
+            launch_steps(K_STEPS)
     if args.clock_settle_s > 0:
         settle(one_pass, args.clock_settle_s)
-    for case in cases:
-        launch_group(case, W_STEPS, offset=7)
+    launch_steps(W_STEPS, offset=7)
     torch.cuda.synchronize()
 
-    # ---------------------------------------------------------------- timed region
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in cases]
+    # ---------------------------------------------------------------- timed region: exactly K steps
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    e0.record()
+    one_pass()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    total_s = t1 - t0
+    timed_us_per_launch = e0.elapsed_time(e1) * 1e3 / (K_STEPS * len(cases))
+
+    # ---------------------------------------------------------------- per-GEMM rows (outside the timed region)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in cases]
+    if use_graph:
+        settle(lambda: [gr.replay() for gr in graphs], 0.05)
     for i, case in enumerate(cases):
         ev[i][0].record()
         if use_graph:
@@ -279,8 +300,6 @@ def main():
             launch_group(case, K_STEPS)
         ev[i][1].record()
     torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    total_s = t1 - t0
 
     per_gemm = []
     groups = {}
@@ -304,10 +323,13 @@ def main():
         f["tuples"].append(name)
     dominant = max(families, key=lambda k: families[k]["us"])
     dg = families[dominant]
+    # launch duration of the dominant kernel: the timed region's own events when every GEMM of a step runs that kernel
+    # family (the case), else the family's share of the per-GEMM rows
+    avg_launch_us = timed_us_per_launch if len(families) == 1 else dg["us"] / dg["launches"]
     total_ops = sum(c["ops"] for c in cases) * K_STEPS
     value = total_ops / total_s / 1e12
-    log("headline: %.2f TOPS over %d GEMMs x %d steps, %.3f us per launch (rows are logged at the end)"
-        % (value, len(cases), K_STEPS, dg["us"] / dg["launches"]))
+    log("headline: %.2f TOPS over %d GEMMs x %d steps, %.3f us per launch in the timed region, %.3f as K launches per GEMM "
+        "(rows are logged at the end)" % (value, len(cases), K_STEPS, avg_launch_us, dg["us"] / dg["launches"]))
 
     # ---------------------------------------------------------------- CPU baseline (bounded sample) + parity
     sys.path.insert(0, ROOT)
@@ -380,10 +402,14 @@ def main():
             for (N, K) in SHAPES:
                 wpl = random_planes(torch, (p, N, K // 32))
                 wtl = abq.relayout_planes(wpl)  # weights prepared once in the K-tiled layout
+                # (pairs with an unsigned 8-bit operand: the weights' row sums are prepared with them; the activations'
+                # are taken inside the timed call when they arrive as planes, and come with them when they arrive tiled)
+                u8 = not signed and 8 in (q, p)
+                wrs = abq.row_sums(wpl) if u8 else None
                 for M in (512, 2048):
                     xpl = random_planes(torch, (q, M, K // 32))
-                    ws = torch.empty(xpl.numel() * 4, dtype=torch.uint8, device="cuda")
-                    gm = abq.Gemm(xpl, wtl, signed, w_tiled=True, workspace=ws)  # activations converted per call
+                    ws = torch.empty(xpl.numel() * 4 + 4 * M + 512, dtype=torch.uint8, device="cuda")
+                    gm = abq.Gemm(xpl, wtl, signed, w_tiled=True, workspace=ws, w_row_sums=wrs)  # activations converted per call
                     gm.run()
                     torch.cuda.synchronize()
                     reps = 20  # (a replay's own launch cost is spread over the steps of the graph)
@@ -403,7 +429,8 @@ def main():
                     # the same GEMM with the activations already in the K-tiled layout, which is how the fused
                     # quantise + pack kernel hands them over: no conversion launch in the timed call
                     xtl = abq.relayout_planes(xpl)
-                    gt = abq.Gemm(xtl, wtl, signed, x_tiled=True, w_tiled=True)
+                    gt = abq.Gemm(xtl, wtl, signed, x_tiled=True, w_tiled=True, w_row_sums=wrs,
+                                  x_row_sums=abq.row_sums(xpl) if u8 else None)
                     gt.run()
                     torch.cuda.synchronize()
                     gr = torch.cuda.CUDAGraph()
@@ -713,7 +740,7 @@ def main():
     if "decode_plane_operands" in extra:
         plane_tops = sum(c["ops"] for c in cases) / sum(r["us"] * 1e-6 for r in extra["decode_plane_operands"]) / 1e12
     print(headline(value, K_STEPS, W_STEPS, total_s, len(cases), args.clock_settle_s, dominant, dg["tuples"],
-                   dg["launches"], dg["bytes"] / dg["launches"], dg["us"] / dg["launches"], cpu_ops / cpu_s, cpu_threads,
+                   dg["launches"], dg["bytes"] / dg["launches"], avg_launch_us, cpu_ops / cpu_s / 1e12, cpu_threads,
                    "%d passes over the same 9 GEMMs (%.1f s), oracle popcount GEMM with OpenMP" % (reps, cpu_s),
                    plane_operand_tops=plane_tops, extra_file=extra_file), flush=True)
 

@@ -189,6 +189,9 @@ typedef struct abq_gemm_state {
     const float *w_zero_term;
     int act;                 /* abq_activation fused into the epilogue */
     const float *x_pack_scale; /* x_layout == ABQ_LAYOUT_F16: the static quantisation scale, see abq_gemm_set_f16_activations */
+    /* row sums of unsigned operands, see abq_gemm_set_row_sums */
+    const int32_t *x_row_sums;
+    const int32_t *w_row_sums;
 } abq_gemm_state;
 
 /* Replaces AqBMMAInitFn / AqBWMMAInitFn (engine/mma_any/aq_bmma_op.h:141-147,163 and
@@ -347,6 +350,26 @@ abq_status abq_gemm_set_f16_activations(abq_gemm_state *state, const void *x_f16
  * shape does not qualify (the caller then quantises with abq_quant_pack_f16 as before).  No counterpart in the
  * reference, whose activations are quantised by a kernel of their own (abq_gemm_wrapper.cu:29-69). */
 abq_status abq_gemm_set_dynamic_f16_activations(abq_gemm_state *state, const void *x_f16, int symmetric);
+
+/* sums[row] = sum over k of the unsigned codes of a row of an operand in the plane layout ([bits][rows][k/32]).
+ * For pairs with an unsigned 8-bit operand: the LDS-staged kernel feeds such an operand to the signed matrix
+ * cores as value - 128 and adds 128 x the OTHER operand's row sums to the result (and takes off 2^14 K when both
+ * operands are 8 bits wide); it does not gather the sums itself.  Once per weight matrix, beside
+ * abq_relayout_planes; once per call for the activations.  No counterpart in the reference, whose binary tensor
+ * cores need no such correction (its unsigned instances: engine/test_w4a4_uint_wmma.cu:228-229, FT
+ * abqgemm/mma_any/aq_bmma_impl/aq_bmma_w2a8.cu:4-9). */
+abq_status abq_row_sums(const uint32_t *planes, int rows, int k, int bits, int32_t *sums, void *stream);
+
+/* Hands the row sums of an unsigned pair's operands to a state (either may be NULL): x_row_sums[M] is read when the
+ * weights are 8 bits wide, w_row_sums[N] when the activations are.  abq_gemm_exec on ABQ_STRATEGY_TILED then runs
+ * the staged kernel for the tiles it is built for.  Sums that are not set are taken by abq_gemm_exec itself for an
+ * operand still in the plane layout if the workspace has the room (abq_gemm_workspace_bytes counts them); when a
+ * needed sum is neither set nor to be had, the kernel that gathers the sums inside its K loop runs instead (same
+ * tile, same result, slower).  Ignored by signed pairs and by pairs without an 8-bit operand. */
+abq_status abq_gemm_set_row_sums(abq_gemm_state *state, const int32_t *x_row_sums, const int32_t *w_row_sums);
+/* 1 if abq_gemm_exec on this state, as it stands, runs the kernel that takes the row sums handed in (every needed
+ * sum set, or to be had from plane operands into the workspace the state holds), 0 otherwise. */
+int abq_gemm_row_sums_ready(const abq_gemm_state *state);
 
 /* Workspace needed by abq_gemm_exec if the state ran as ABQ_STRATEGY_TILED, ABQ_STRATEGY_DECODE_TILED
  * (ABQ_STRATEGY_FP6) with its current operand layouts: the converted copies of the operands still in

@@ -175,11 +175,22 @@ def test_relayout_planes_matches_closed_form(abq, oracle):
         assert np.array_equal(got.reshape(want.shape), want), (bits, rows, k)
 
 
+def test_row_sums_of_plane_operands(abq, oracle):
+    rng = np.random.default_rng(14)
+    for bits, rows, k in [(8, 1, 128), (8, 37, 1152), (2, 300, 4096), (4, 5, 13824), (3, 66, 384), (8, 2048, 4096)]:
+        v = rng.integers(0, 1 << bits, size=(rows, k), dtype=np.int32)
+        if rows > 1:
+            v[1] = (1 << bits) - 1  # a row of maximal codes
+        got = abq.row_sums(planes_dev(oracle.pack_i32(v, bits))).cpu().numpy()
+        assert np.array_equal(got, v.sum(axis=1)), (bits, rows, k)
+
+
 def test_tiled_kernels_with_prepared_operands(abq, oracle):
     """K-tiled kernels fed tiled activations and/or tiled weights directly, ragged shapes."""
     rng = np.random.default_rng(13)
     for q, p, signed, M, N, K in [(8, 2, True, 300, 200, 640), (4, 4, False, 70, 513, 1152), (8, 8, False, 257, 129, 384),
-                                  (8, 4, True, 130, 200, 768), (8, 8, True, 70, 129, 128)]:
+                                  (8, 4, True, 130, 200, 768), (8, 8, True, 70, 129, 128), (8, 2, False, 300, 290, 640),
+                                  (8, 4, False, 130, 200, 768), (8, 8, False, 300, 513, 1152)]:
         x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
         xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
         xt, wt = abq.relayout_planes(xd), abq.relayout_planes(wd)
@@ -190,6 +201,20 @@ def test_tiled_kernels_with_prepared_operands(abq, oracle):
             ws = torch.empty(xd.numel() * 4, dtype=torch.uint8, device="cuda")
             got = abq.gemm(xd, wt, signed, cfg=cfg, w_tiled=True, workspace=ws).cpu().numpy()
             assert np.array_equal(got, want), abq.format_kernel_name(cfg)
+            if not signed and 8 in (q, p):
+                # unsigned 8-bit operands with their row sums handed in: the staged kernel where it has the tile
+                # (the other tiles keep the kernel that gathers the sums itself, whatever is handed in)
+                g = abq.Gemm(xt, wt, signed, cfg=cfg, x_tiled=True, w_tiled=True, x_row_sums=abq.row_sums(xd), w_row_sums=abq.row_sums(wd))
+                staged_tile = cfg.warp_k == 128 and cfg.block_k == 128 and (cfg.block_m, cfg.block_n, cfg.warp_m, cfg.warp_n) in (
+                    (128, 128, 64, 64), (128, 64, 64, 32), (64, 64, 32, 32), (256, 128, 64, 64)) + (
+                    ((256, 256, 64, 128),) if (q, p) != (8, 8) else ())
+                assert g.row_sums_ready == staged_tile, abq.format_kernel_name(cfg)
+                assert np.array_equal(g.run().cpu().numpy(), want), abq.format_kernel_name(cfg)
+                # activations as planes with a workspace that holds their sums too, weight sums handed in
+                ws2 = torch.empty(xd.numel() * 4 + 4 * M + 512, dtype=torch.uint8, device="cuda")
+                g = abq.Gemm(xd, wt, signed, cfg=cfg, w_tiled=True, workspace=ws2, w_row_sums=abq.row_sums(wd))
+                assert g.row_sums_ready == staged_tile and g.workspace_bytes <= ws2.numel()
+                assert np.array_equal(g.run().cpu().numpy(), want), abq.format_kernel_name(cfg)
         # a state with an explicit non-tiled tile refuses tiled operands; exec without workspace is refused
         cfg = [c for c in abq.native_configs(q, p, signed) if c.nstage == 2][0]
         with pytest.raises(abq.AbqError):
@@ -663,9 +688,11 @@ def test_config2_prefill_full_size(abq, oracle, q, p, signed):
             x = rand_vals(rng, M, K, q, signed)
             xp = oracle.pack_i32(x, q)
             xd = planes_dev(xp)
-            ws = torch.empty(xd.numel() * 4, dtype=torch.uint8, device="cuda")
-            g = abq.Gemm(xd, wt, signed, w_tiled=True, workspace=ws)
-            assert g.strategy == "tiled"
+            ws = torch.empty(xd.numel() * 4 + 4 * M + 512, dtype=torch.uint8, device="cuda")
+            # (unsigned 8-bit operands: the weights' row sums come with the prepared weights, the activations' are
+            # taken per call into the workspace; the staged kernel then runs them like the signed pairs)
+            g = abq.Gemm(xd, wt, signed, w_tiled=True, workspace=ws, w_row_sums=None if signed else abq.row_sums(wd))
+            assert g.strategy == "tiled" and g.row_sums_ready == ((q, p, signed) == (8, 8, False))
             got_d = g.run()
             ref = torch.from_numpy(x).cuda().double() @ wf.T
             assert torch.equal(got_d.double(), ref), (q, p, signed, M, N, K)
