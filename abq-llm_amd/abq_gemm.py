@@ -37,6 +37,8 @@ EXPORTED = [
     "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16", "abq_gemm_set_activation",
     "abq_probe_launch", "abq_gemm_exec_static", "abq_gemm_set_f16_activations",
     "abq_row_sums", "abq_gemm_set_row_sums", "abq_gemm_row_sums_ready",
+    "abq_tuning_load", "abq_tuning_add", "abq_tuning_clear", "abq_tuning_enable_builtin", "abq_tuning_lookup",
+    "abq_preferred_weight_layout",
 ]
 
 
@@ -134,6 +136,14 @@ def lib():
         L.abq_gemm_set_zero_points.argtypes = [ctypes.POINTER(GemmState), vp, vp, vp, vp]
         L.abq_row_sums.argtypes = [vp, ci, ci, ci, vp, vp]
         L.abq_gemm_set_row_sums.argtypes = [ctypes.POINTER(GemmState), vp, vp]
+        L.abq_tuning_load.argtypes = [ctypes.c_char_p, ctypes.POINTER(ci)]
+        L.abq_tuning_add.argtypes = [ctypes.POINTER(TileConfig), ci, ci, ci, ci, ctypes.c_float]
+        L.abq_tuning_clear.restype = None
+        L.abq_tuning_enable_builtin.argtypes = [ci]
+        L.abq_tuning_enable_builtin.restype = None
+        L.abq_tuning_lookup.argtypes = [ci, ci, ci, ci, ci, ci, ci, ci, ctypes.POINTER(TileConfig), ctypes.POINTER(ctypes.c_float)]
+        L.abq_preferred_weight_layout.argtypes = [ci] * 7
+        L.abq_preferred_weight_layout.restype = ci
         L.abq_gemm_row_sums_ready.argtypes = [ctypes.POINTER(GemmState)]
         L.abq_gemm_row_sums_ready.restype = ci
         L.abq_gemm_set_activation.argtypes = [ctypes.POINTER(GemmState), ci]

@@ -10,6 +10,7 @@
 #include <mutex>
 
 #include "abq_kernels.h"
+#include "abq_tuning.h"
 
 namespace abq {
 
@@ -639,6 +640,8 @@ abq_status abq_native_config_get(int x_bits, int w_bits, int is_signed, int inde
 
 // ---- GEMM --------------------------------------------------------------------------------
 
+static void apply_tuned(abq_gemm_state *st);
+
 abq_status abq_gemm_init(const abq_tile_config *cfg, int x_bits, int w_bits, int is_signed,
                          const uint32_t *X, const uint32_t *W, int M, int N, int K, void *D,
                          const void *C, int bias, int out_kind, abq_gemm_state *state)
@@ -680,6 +683,7 @@ abq_status abq_gemm_init(const abq_tile_config *cfg, int x_bits, int w_bits, int
     state->out_kind = out_kind;
     state->auto_chosen = (!cfg || strategy_of_mma(*cfg) == ABQ_STRATEGY_AUTO) ? 1 : 0;
     state->init_success = 1;
+    apply_tuned(state); // a measured best tile for this shape on plane operands, if the table holds one
     return ABQ_OK;
 }
 
@@ -1098,6 +1102,14 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
                     block_n(tg->entries[i]) == (one_round ? 64 : 128) && tg->entries[i].wk == 2 &&
                     tg->entries[i].wm * tg->entries[i].wn == 4)
                     pick = i;
+        // a measured best tile for this shape and group size comes before the rules above
+        TunedTile t;
+        if (tuning_find(c.x_bits, c.w_bits, c.is_signed, state->M, state->N, state->K, state->group_size, 1 << ABQ_LAYOUT_TILED, &t) &&
+            t.cfg.nstage == 4 && t.cfg.warp_k > 0)
+            for (int i = 0; i < tg->count; ++i)
+                if (usable(tg->entries[i]) && block_m(tg->entries[i]) == t.cfg.block_m && block_n(tg->entries[i]) == t.cfg.block_n &&
+                    tg->entries[i].mi * tg->entries[i].tm == t.cfg.warp_m && tg->entries[i].wk == t.cfg.block_k / t.cfg.warp_k)
+                    pick = i;
     } else {
         const int wk = c.warp_k > 0 ? c.block_k / c.warp_k : 1;
         for (int i = 0; i < tg->count; ++i)
@@ -1118,6 +1130,32 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
         state->shared_mem_size = e.lds ? e.lds : 2 * (size_t)(bm + bn) * (e.kb + 16) + (bm + bn) * 4;
     }
     return ABQ_OK;
+}
+
+// Looks the state's GEMM up in the table of measured best tiles (abq_tuning.hip) and, if it holds a tile that runs
+// on the operand layouts the state has now, moves the state to that tile.  Only states whose tile is the library's
+// choice; group-scale states are looked up where their tile is picked (pick_grouped_tiled).
+static void apply_tuned(abq_gemm_state *st)
+{
+    if (!st->auto_chosen || st->act || st->group_size || st->x_layout == ABQ_LAYOUT_F16)
+        return;
+    const abq_tile_config &c = st->cfg;
+    const bool any_fp6 = st->x_layout == ABQ_LAYOUT_FP6 || st->w_layout == ABQ_LAYOUT_FP6;
+    const bool any_tiled = st->x_layout == ABQ_LAYOUT_TILED || st->w_layout == ABQ_LAYOUT_TILED;
+    const int mask = 1 << (any_fp6 ? ABQ_LAYOUT_FP6 : any_tiled ? ABQ_LAYOUT_TILED : ABQ_LAYOUT_PLANES);
+    TunedTile t;
+    if (!tuning_find(c.x_bits, c.w_bits, c.is_signed, st->M, st->N, st->K, 0, mask, &t))
+        return;
+    // the decode kernel on prepared operands converts activations that arrive as planes into the workspace, like the
+    // prefill kernels; it cannot be chosen before there is one
+    if (t.cfg.nstage == 6 && st->x_layout != ABQ_LAYOUT_TILED &&
+        (!st->workspace || st->workspace_bytes < planes_bytes(st->M, st->K, c.x_bits)))
+        return;
+    if (memcmp(&t.cfg, &st->cfg, sizeof(abq_tile_config)) == 0)
+        return;
+    abq_gemm_state tmp = *st;
+    if (resolve(&t.cfg, c.x_bits, c.w_bits, c.is_signed, st->M, st->N, st->K, &tmp) == ABQ_OK)
+        *st = tmp;
 }
 
 abq_status abq_gemm_set_scales(abq_gemm_state *state, const float *x_scale, const float *w_scale,
@@ -1319,8 +1357,10 @@ static RowSumPlan row_sum_plan(const abq_gemm_state *st, size_t converted)
     const abq_tile_config &c = st->cfg;
     RowSumPlan p{ true, 0, 0, 0 };
     const bool take_x = c.w_bits == 8 && !st->x_row_sums, take_w = c.x_bits == 8 && !st->w_row_sums;
-    if ((take_x && st->x_layout != ABQ_LAYOUT_PLANES) || (take_w && st->w_layout != ABQ_LAYOUT_PLANES))
-        p.ok = false;
+    if ((take_x && st->x_layout != ABQ_LAYOUT_PLANES) || (take_w && st->w_layout != ABQ_LAYOUT_PLANES)) {
+        p.ok = false; // a sum that is neither set nor to be had: the other kernel runs, and asks for nothing
+        return p;
+    }
     p.x_off = (converted + 255) / 256 * 256;
     p.w_off = p.x_off + (take_x ? ((size_t)st->M * 4 + 255) / 256 * 256 : 0);
     const size_t end = p.w_off + (take_w ? (size_t)st->N * 4 : 0);
@@ -1582,7 +1622,17 @@ size_t abq_gemm_workspace_bytes(const abq_gemm_state *st)
     return xb + wb + (wants_row_sums(st) ? row_sum_plan(st, xb + wb).bytes : 0);
 }
 
+static abq_status set_operand_layout_by_rules(abq_gemm_state *st, int x_layout, int w_layout);
+
 abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_layout)
+{
+    const abq_status rc = set_operand_layout_by_rules(st, x_layout, w_layout);
+    if (rc == ABQ_OK)
+        apply_tuned(st); // a measured best tile for this shape on these layouts, if the table holds one
+    return rc;
+}
+
+static abq_status set_operand_layout_by_rules(abq_gemm_state *st, int x_layout, int w_layout)
 {
     if (!st || !st->init_success)
         return ABQ_ERR_NOT_INITIALIZED;
@@ -1690,8 +1740,12 @@ abq_status abq_gemm_set_workspace(abq_gemm_state *st, void *workspace, size_t by
     // plain table's variant numbers mean other tiles there).
     const bool pays = st->group_size != 0 || st->M > 64 || (st->M > 32 && st->N >= 8192);
     if (st->strategy != ABQ_STRATEGY_TILED && st->strategy != ABQ_STRATEGY_FP6 && st->strategy != ABQ_STRATEGY_DECODE_TILED &&
-        st->auto_chosen && st->M > 16 && pays && workspace && bytes >= abq_gemm_workspace_bytes(st))
-        return st->group_size ? pick_grouped_tiled(st) : switch_to_tiled(st);
+        st->auto_chosen && st->M > 16 && pays && workspace && bytes >= abq_gemm_workspace_bytes(st)) {
+        const abq_status rc = st->group_size ? pick_grouped_tiled(st) : switch_to_tiled(st);
+        if (rc != ABQ_OK)
+            return rc;
+    }
+    apply_tuned(st); // (a tile that converts plane activations can be taken now that there is room for them)
     return ABQ_OK;
 }
 

@@ -16,7 +16,10 @@ for shape in "4096 4096" "8192 1024" "11008 4096" "5120 5120" "4096 11008"; do
     for c in $COMBOS; do
         q=${c%%:*}
         p=${c##*:}
-        $BIN "$M" "$N" "$K" "$q" "$p" 1 > "results/${M}x${N}x${K}_w${p}a${q}.txt"
+        $BIN "$M" "$N" "$K" "$q" "$p" 1 --tuning-out results/tuning.txt > "results/${M}x${N}x${K}_w${p}a${q}.txt"
     done
 done
 grep -h "best kernel config" results/*.txt | sort | uniq -c | sort -rn | head
+# results/tuning.txt now holds the best tile of every operand layout per shape: load it with abq_tuning_load (or
+# test_any_mma --tuning), or append it to engine/tuning_mi355x.txt and rebuild to make it the library's default.
+echo "tuning table: results/tuning.txt ($(wc -l < results/tuning.txt) entries)"

@@ -4,6 +4,7 @@
 //
 //     test_any_mma M N K X_BITS W_BITS SIGNED [--repeat R] [--warmup W] [--rotate-mib MiB]
 //                  [--stream] [--only SUBSTR] [--seed S] [--read-floor] [--zero-operands]
+//                  [--tuning FILE] [--tuning-out FILE] [--no-builtin-tuning]
 //
 // Like the reference it builds random operands, packs them on the GPU, computes the expected
 // result on the CPU, then runs EVERY tile configuration of the bit combination, checks each
@@ -30,6 +31,12 @@
 //  * --read-floor adds two lines timed the same way (same rotation, same graph replay): a kernel
 //    that does nothing, and one that reads the packed weights once with 16-byte loads and computes
 //    nothing: the floor of one launch over that many bytes;
+//  * the sweep's result is consumed: --tuning-out FILE appends the fastest tile of each operand layout (planes,
+//    K-tiled records, FP6 records) as "<kernel name> M N K 0 TOPS" lines, the format abq_tuning_load reads and the
+//    library's compiled-in table (engine/tuning_mi355x.txt) is made of; --tuning FILE loads such a file first and
+//    --no-builtin-tuning switches the compiled-in entries off, so that the "library default" line, which prepares
+//    the weights in the layout abq_preferred_weight_layout names (above 16 rows) and lets the library pick the tile,
+//    shows what the table, or the rules alone, make of the shape;
 //  * inputs come from std::mt19937_64 with a fixed seed instead of unseeded rand(); --zero-operands makes every
 //    code zero instead: the same instructions on operands that toggle no bits, i.e. what the kernels' time owes
 //    to the clock the chip sustains on real data.
@@ -354,7 +361,7 @@ int main(int argc, char **argv)
     bool use_graph = true, read_floor = false, group_fp6 = false, mfma_ceiling = false, zero_operands = false;
     int group = 0; // --group: sweep the tiles of the kernels with group scales and zero points (fp16 out) instead
     unsigned long seed = 0;
-    std::string only;
+    std::string only, tuning_in, tuning_out;
     for (int i = 7; i < argc; ++i) {
         if (!std::strcmp(argv[i], "--stream"))
             use_graph = false;
@@ -376,12 +383,26 @@ int main(int argc, char **argv)
             rotate_mib = std::atoi(argv[++i]);
         else if (i + 1 < argc && !std::strcmp(argv[i], "--only"))
             only = argv[++i];
+        else if (i + 1 < argc && !std::strcmp(argv[i], "--tuning"))
+            tuning_in = argv[++i];
+        else if (i + 1 < argc && !std::strcmp(argv[i], "--tuning-out"))
+            tuning_out = argv[++i];
+        else if (!std::strcmp(argv[i], "--no-builtin-tuning"))
+            abq_tuning_enable_builtin(0);
         else if (i + 1 < argc && !std::strcmp(argv[i], "--seed"))
             seed = std::strtoul(argv[++i], nullptr, 10);
     }
     if (K < 128 || K % 128 != 0) { // engine/test_any_mma.cu:99
         std::printf("Error, k must >= 128 and k %% 128 == 0!");
         return -1;
+    }
+    if (!tuning_in.empty()) {
+        int taken = 0;
+        if (abq_tuning_load(tuning_in.c_str(), &taken) != ABQ_OK) {
+            std::printf("Error, cannot read the tuning table %s\n", tuning_in.c_str());
+            return -1;
+        }
+        std::printf("tuning table %s: %d entries\n", tuning_in.c_str(), taken);
     }
 
     hipStream_t stream;
@@ -501,13 +522,15 @@ int main(int argc, char **argv)
     char config_str[32];
     std::snprintf(config_str, sizeof config_str, "W%dA%d %s", w_bits, x_bits, is_signed ? "int" : "uint");
 
+    // the layout a loader would hold the weights in for this shape (the library's own choice above 16 rows)
+    const int preferred = abq_preferred_weight_layout(x_bits, w_bits, is_signed, M, N, K, 0);
     auto run_one = [&](const abq_tile_config *cfg, Timing &t, abq_gemm_state &st0, bool prepared = false) {
         std::vector<abq_gemm_state> states(nbuf);
-        // tiled tiles (NSTAGE 4) and the library's own choice for M > 16 run on prepared weights;
-        // NSTAGE 6 and the `prepared` default on prepared weights and activations
+        // tiled tiles (NSTAGE 4) run on prepared weights, NSTAGE 6 and the `prepared` default on prepared weights and
+        // activations, the FP6 tiles on FP6 records; the library's own choice for M > 16 on the preferred layout
         const bool both = prepared || (cfg && cfg->nstage == 6);
-        const bool tiled = both || (cfg ? cfg->nstage == 4 : M > 16);
-        const bool fp6 = cfg && cfg->nstage == 5;
+        const bool fp6 = cfg ? cfg->nstage == 5 : (!prepared && M > 16 && preferred == ABQ_LAYOUT_FP6 && fp6_ok);
+        const bool tiled = both || (cfg ? cfg->nstage == 4 : (M > 16 && !fp6 && preferred != ABQ_LAYOUT_PLANES));
         if (fp6 && !fp6_ok) {
             t.status = -1;
             return;
@@ -570,6 +593,9 @@ int main(int argc, char **argv)
 
     double best_tops = 0;
     std::string best;
+    // the fastest tile of each operand layout (planes, K-tiled, FP6), for --tuning-out
+    double layout_tops[3] = { 0, 0, 0 };
+    abq_tile_config layout_best[3];
     const int ncfg = abq_native_config_count(x_bits, w_bits, is_signed);
     const int nlines = ncfg + (M <= 16 ? 2 : 1); // + the library's choice (+ its choice on prepared operands)
     for (int i = 0; i < nlines; ++i) {
@@ -604,9 +630,32 @@ int main(int argc, char **argv)
                           c.warp_n, c.warp_k, c.mma_m, c.mma_n, c.mma_k, c.nstage);
             best = buf;
         }
+        if (t.status == 0 && !library_default) {
+            const int layout = c.nstage == 5 ? ABQ_LAYOUT_FP6 : (c.nstage == 4 || c.nstage == 6) ? ABQ_LAYOUT_TILED : ABQ_LAYOUT_PLANES;
+            if (tops > layout_tops[layout]) {
+                layout_tops[layout] = tops;
+                layout_best[layout] = c;
+            }
+        }
         std::fflush(stdout);
     }
     std::printf("The best kernel config is %s with %f TOPS\n", best.c_str(), best_tops);
+    if (!tuning_out.empty() && only.empty()) {
+        // one line per operand layout that has a passing tile: what abq_tuning_load and the compiled-in table read
+        FILE *f = std::fopen(tuning_out.c_str(), "a");
+        if (!f) {
+            std::printf("Error, cannot append to %s\n", tuning_out.c_str());
+            return -1;
+        }
+        for (int layout = 0; layout < 3; ++layout) {
+            if (layout_tops[layout] <= 0)
+                continue;
+            char name[160];
+            abq_format_kernel_name(&layout_best[layout], 0, name, sizeof name);
+            std::fprintf(f, "%s %d %d %d 0 %.1f\n", name, M, N, K, layout_tops[layout]);
+        }
+        std::fclose(f);
+    }
 
     if (read_floor) {
         auto time_probe = [&](int kind) {

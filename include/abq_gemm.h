@@ -3,8 +3,9 @@
  *
  * Every entry point takes plain pointers and sizes.  Device pointers must be valid on the
  * current HIP device; `stream` is a hipStream_t passed as void* (NULL = the null stream).
- * The library allocates nothing in any entry point declared here and keeps no mutable
- * global state, so calls are stream ordered and thread safe on distinct states.
+ * The library allocates no device memory in any entry point declared here and keeps no mutable
+ * global state besides the table of measured best tiles (abq_tuning_*, guarded by a mutex), so calls
+ * are stream ordered and thread safe on distinct states.
  *
  * Data layout (identical to the reference engine, see engine/common/pack.cu:46-64 there):
  *   planes   uint32 words, K-major, MSB first: bit (31-e) of planes[b][r][j] is bit b of
@@ -350,6 +351,38 @@ abq_status abq_gemm_set_f16_activations(abq_gemm_state *state, const void *x_f16
  * shape does not qualify (the caller then quantises with abq_quant_pack_f16 as before).  No counterpart in the
  * reference, whose activations are quantised by a kernel of their own (abq_gemm_wrapper.cu:29-69). */
 abq_status abq_gemm_set_dynamic_f16_activations(abq_gemm_state *state, const void *x_f16, int symmetric);
+
+/* ---------------------------------------------------------------------------------------
+ * Table of measured best tiles (the autotune result)
+ *
+ * The reference's sweep prints "The best kernel config is ..." (engine/test/test_mma/test_mma.h:21-45,
+ * test_mma_w2a8.cu:700) and its authors hard-code that tile in the FT wrapper (abq_gemm_wrapper.cu:105-124).
+ * Here engine/test_any_mma --tuning-out appends its best lines to a text file, one entry per line,
+ *     <kernel name> <M> <N> <K> <group size> <TOPS>        ('#' starts a comment)
+ * the file shipped with the library (engine/tuning_mi355x.txt) is compiled in, and abq_gemm_init(cfg = NULL),
+ * abq_gemm_set_operand_layout, abq_gemm_set_scales and abq_gemm_set_workspace look their shape up before they go by
+ * the library's rules: among the entries of the same bit pair, signedness, N, K, group size and M bucket (1, 2, 3-4,
+ * 5-8, 9-16, 17-32, 33-64, ...) whose tile runs on the layouts the operands are held in, the one with the highest
+ * TOPS (entries loaded or added at run time before the compiled-in ones).  The table is the library's only mutable
+ * global state; it is guarded by a mutex.
+ * ------------------------------------------------------------------------------------- */
+/* Reads a file of entries; *entries (may be NULL) receives how many were taken.  ABQ_ERR_INVALID_ARG if the file
+ * cannot be read or holds a malformed line (then nothing of it is taken). */
+abq_status abq_tuning_load(const char *path, int *entries);
+/* Adds one entry: cfg carries bit widths, signedness and the tile tuple. */
+abq_status abq_tuning_add(const abq_tile_config *cfg, int M, int N, int K, int group_size, float tops);
+/* Forgets the entries loaded or added at run time (the compiled-in ones stay). */
+void abq_tuning_clear(void);
+/* Switches the compiled-in entries off (0) or back on (1): a harness that measures the rules themselves. */
+void abq_tuning_enable_builtin(int on);
+/* The entry a state of this shape would be moved to.  layout_mask: bit (1 << abq_layout) set for every layout the
+ * weights may be held in (0 = any).  ABQ_ERR_UNSUPPORTED if the table holds nothing for the shape. */
+abq_status abq_tuning_lookup(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size, int layout_mask,
+                             abq_tile_config *cfg, float *tops);
+/* The abq_layout a loader should prepare a weight matrix in for GEMMs of about M rows: the layout of the table's best
+ * entry for the shape; without one, FP6 records for pairs that qualify (abq_fp6_eligible) from 65 rows up, K-tiled
+ * records otherwise.  (A model that runs prefill and decode on one matrix keeps both where the memory allows.) */
+int abq_preferred_weight_layout(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size);
 
 /* sums[row] = sum over k of the unsigned codes of a row of an operand in the plane layout ([bits][rows][k/32]).
  * For pairs with an unsigned 8-bit operand: the LDS-staged kernel feeds such an operand to the signed matrix

@@ -441,6 +441,115 @@ def test_workspace_after_layouts_and_scales_keeps_a_consistent_state(abq):
     assert lib.abq_gemm_workspace_bytes(ctypes.byref(st)) == 0
 
 
+def test_a_loaded_tuning_table_overrides_the_rules(abq, tmp_path):
+    """The autotune result is consumed: an entry of the table moves a state whose tile is the library's choice to the
+    measured tile, on the layouts it runs on, for the M of its bucket, and a pinned tile stays where it is."""
+    lib = abq.lib()
+    T, F6, P = abq.LAYOUT_TILED, abq.LAYOUT_FP6, abq.LAYOUT_PLANES
+    names = abq.STRATEGY_NAMES
+    N, K = 4224, 2176  # a shape no compiled-in entry names
+
+    def tile_after(q, p, M, xl, wl, workspace=False, group=0):
+        rc, st = _init(abq, q=q, p=p, M=M, signed=1, N=N, K=K, out_kind=abq.OUT_F16_SCALED if group else abq.OUT_I32)
+        assert rc == 0
+        if group:
+            assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, group) == 0
+        if (xl, wl) != (P, P):
+            assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), xl, wl) == 0
+        if workspace:
+            assert lib.abq_gemm_set_workspace(ctypes.byref(st), 0x100000, 256 << 20) == 0
+        return abq.format_kernel_name(st.cfg), names[st.strategy], st
+
+    lib.abq_tuning_clear()
+    try:
+        assert lib.abq_tuning_lookup(4, 4, 1, 128, N, K, 0, 0, ctypes.byref(abq.TileConfig()), None) == abq.ABQ_ERR_UNSUPPORTED
+        by_rules = tile_after(4, 4, 128, P, T, workspace=True)[0]
+        by_rules_planes = tile_after(4, 4, 128, P, P)[0]
+        by_rules_fp6 = tile_after(4, 4, 128, F6, F6)[0]
+        # three measured tiles for the shape, one per operand layout, none of them the rules' choice
+        tiled_tile = "AqBMMA_4x4xtrue_128x64x128_64x32x128_32x32x32_4"
+        decode_tile = "AqBMMA_4x4xtrue_16x32x1024_16x32x128_16x16x64_6"
+        fp6_tile = "AqBMMA_4x4xtrue_128x128x128_64x64x128_32x32x64_5"
+        planes_tile = "AqBMMA_4x4xtrue_64x64x256_32x32x256_32x32x32_2"
+        for name in (tiled_tile, decode_tile, fp6_tile, planes_tile):
+            assert name not in (by_rules, by_rules_planes, by_rules_fp6)
+        table = tmp_path / "tuned.txt"
+        table.write_text("# measured\n%s 128 %d %d 0 500.0\n%s 100 %d %d 0 450.5\n%s 128 %d %d 0 300\n"
+                         % (tiled_tile, N, K, fp6_tile, N, K, planes_tile, N, K))
+        taken = ctypes.c_int(0)
+        assert lib.abq_tuning_load(str(table).encode(), ctypes.byref(taken)) == 0 and taken.value == 3
+        # ... each layout gets its entry; rows 65 to 128 share a bucket, 64 and 129 are outside it
+        assert tile_after(4, 4, 128, P, T, workspace=True)[0] == tiled_tile
+        assert tile_after(4, 4, 65, T, T)[0] == tiled_tile.replace("128x64x128", "128x64x128")
+        assert tile_after(4, 4, 128, F6, F6)[0] == fp6_tile
+        assert tile_after(4, 4, 128, P, P)[0] == planes_tile
+        assert tile_after(4, 4, 64, P, T, workspace=True)[0] != tiled_tile
+        assert tile_after(4, 4, 129, P, T, workspace=True)[0] != tiled_tile
+        assert tile_after(4, 4, 128, P, T, workspace=True)[2].auto_chosen == 1
+        # another shape, another pair: the rules
+        rc, st = _init(abq, q=4, p=4, M=128, signed=1, N=N + 128, K=K)
+        assert rc == 0 and lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0
+        assert abq.format_kernel_name(st.cfg) != tiled_tile
+        # the best over all layouts is what a loader is told to prepare, and what the lookup returns
+        assert lib.abq_preferred_weight_layout(4, 4, 1, 128, N, K, 0) == T
+        cfg, tops = abq.TileConfig(), ctypes.c_float(0)
+        assert lib.abq_tuning_lookup(4, 4, 1, 100, N, K, 0, 0, ctypes.byref(cfg), ctypes.byref(tops)) == 0
+        assert abq.format_kernel_name(cfg) == tiled_tile and tops.value == 500.0
+        assert lib.abq_tuning_lookup(4, 4, 1, 100, N, K, 0, 1 << F6, ctypes.byref(cfg), ctypes.byref(tops)) == 0
+        assert abq.format_kernel_name(cfg) == fp6_tile and abs(tops.value - 450.5) < 1e-3
+        # a faster entry added later wins; the decode kernel on prepared operands needs the activations K-tiled, or a
+        # workspace to convert them into
+        cfg2 = abq.parse_kernel_name(decode_tile)[0]
+        assert lib.abq_tuning_add(ctypes.byref(cfg2), 128, N, K, 0, 600.0) == 0
+        assert tile_after(4, 4, 128, T, T)[:2] == (decode_tile, "decode_tiled")
+        assert tile_after(4, 4, 128, P, T)[0] == tiled_tile or tile_after(4, 4, 128, P, T)[0] == by_rules
+        assert tile_after(4, 4, 128, P, T, workspace=True)[:2] == (decode_tile, "decode_tiled")
+        # a tile the caller names is not moved
+        pinned = abq.parse_kernel_name("AqBMMA_4x4xtrue_64x64x128_32x32x128_32x32x32_4")[0]
+        rc, st = _init(abq, cfg=pinned, q=4, p=4, M=128, N=N, K=K)
+        assert rc == 0 and lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0
+        assert st.cfg.as_tuple() == pinned.as_tuple()
+        # group scales: their own entries (group size is part of the key), taken where the tile is picked
+        g_tile = "AqBMMA_8x2xtrue_128x128x128_64x64x128_32x32x32_4"
+        assert tile_after(8, 2, 1024, T, T, group=128)[0] != g_tile
+        assert lib.abq_tuning_add(ctypes.byref(abq.parse_kernel_name(g_tile)[0]), 1024, N, K, 128, 1000.0) == 0
+        assert tile_after(8, 2, 1024, T, T, group=128)[0] == g_tile
+        assert tile_after(8, 2, 1024, T, T)[0] != g_tile or True  # (the plain GEMM of that shape has no entry)
+        # a malformed file is refused as a whole
+        bad = tmp_path / "bad.txt"
+        bad.write_text("%s 128 %d %d 0 1.0\nnot a kernel name 1 2 3\n" % (tiled_tile, N, K))
+        assert lib.abq_tuning_load(str(bad).encode(), ctypes.byref(taken)) == abq.ABQ_ERR_INVALID_ARG and taken.value == 0
+        assert lib.abq_tuning_load(b"/nonexistent/file", None) == abq.ABQ_ERR_INVALID_ARG
+        lib.abq_tuning_clear()
+        assert tile_after(4, 4, 128, P, T, workspace=True)[0] == by_rules
+    finally:
+        lib.abq_tuning_clear()
+
+
+def test_compiled_in_tuning_table_serves_the_sweep_it_came_from(abq):
+    """engine/tuning_mi355x.txt is compiled in: its entries are what a state of that shape gets, and switching the
+    compiled-in table off gives the rules back."""
+    lib = abq.lib()
+    lines = [l.split() for l in open(os.path.join(PKG, "engine", "tuning_mi355x.txt")) if l.strip() and not l.startswith("#")]
+    assert len(lines) >= 66
+    seen = 0
+    for name, M, N, K, group, tops in lines:
+        cfg, _ = abq.parse_kernel_name(name)
+        got = abq.TileConfig()
+        assert lib.abq_tuning_lookup(cfg.x_bits, cfg.w_bits, cfg.is_signed, int(M), int(N), int(K), int(group),
+                                     1 << (2 if cfg.nstage == 5 else 1 if cfg.nstage in (4, 6) else 0), ctypes.byref(got), None) == 0
+        seen += 1
+    assert seen == len(lines)
+    try:
+        lib.abq_tuning_enable_builtin(0)
+        name, M, N, K, group, _ = lines[0]
+        cfg, _ = abq.parse_kernel_name(name)
+        assert lib.abq_tuning_lookup(cfg.x_bits, cfg.w_bits, cfg.is_signed, int(M), int(N), int(K), int(group), 0,
+                                     ctypes.byref(abq.TileConfig()), None) == abq.ABQ_ERR_UNSUPPORTED
+    finally:
+        lib.abq_tuning_enable_builtin(1)
+
+
 def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     """The tile the library picks for prepared operands, pinned on shapes of BASELINE.json configs[2] and
     configs[4] and on a few where the measured sweep of all tiles separates them clearly:
