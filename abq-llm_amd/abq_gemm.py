@@ -38,7 +38,7 @@ EXPORTED = [
     "abq_probe_launch", "abq_gemm_exec_static", "abq_gemm_set_f16_activations",
     "abq_row_sums", "abq_gemm_set_row_sums", "abq_gemm_row_sums_ready",
     "abq_tuning_load", "abq_tuning_add", "abq_tuning_clear", "abq_tuning_enable_builtin", "abq_tuning_lookup",
-    "abq_preferred_weight_layout",
+    "abq_preferred_weight_layout", "abq_padded_bits", "abq_relayout_planes_padded", "abq_gemm_set_value_bits",
 ]
 
 
@@ -144,6 +144,10 @@ def lib():
         L.abq_tuning_lookup.argtypes = [ci, ci, ci, ci, ci, ci, ci, ci, ctypes.POINTER(TileConfig), ctypes.POINTER(ctypes.c_float)]
         L.abq_preferred_weight_layout.argtypes = [ci] * 7
         L.abq_preferred_weight_layout.restype = ci
+        L.abq_padded_bits.argtypes = [ci]
+        L.abq_padded_bits.restype = ci
+        L.abq_relayout_planes_padded.argtypes = [vp, vp, ci, ci, ci, ci, vp]
+        L.abq_gemm_set_value_bits.argtypes = [ctypes.POINTER(GemmState), ci, ci]
         L.abq_gemm_row_sums_ready.argtypes = [ctypes.POINTER(GemmState)]
         L.abq_gemm_row_sums_ready.restype = ci
         L.abq_gemm_set_activation.argtypes = [ctypes.POINTER(GemmState), ci]
@@ -254,6 +258,22 @@ def row_sums(planes, stream=None):
     return out
 
 
+def padded_bits(bits):
+    return lib().abq_padded_bits(bits)
+
+
+def relayout_planes_padded(planes, signed, stream=None):
+    """planes int32 tensor [bits, rows, k/32] -> K-tiled records of the next width of one field (2, 4 or 8 bits),
+    [k/128, rows, padded bits, 4], the codes extended to that width."""
+    import torch
+    bits, rows, kw = planes.shape
+    assert planes.is_cuda and planes.is_contiguous() and kw % 4 == 0
+    out = torch.empty((kw // 4, rows, padded_bits(bits), 4), dtype=torch.int32, device=planes.device)
+    _check(lib().abq_relayout_planes_padded(planes.data_ptr(), out.data_ptr(), rows, kw * 32, bits, int(bool(signed)),
+                                            _stream_ptr(stream)), "abq_relayout_planes_padded")
+    return out
+
+
 def fp6_eligible(x_bits, w_bits, signed, k):
     """Whether the FP6 matrix-core route is exact for this bit pair and K (host-side check)."""
     return bool(lib().abq_fp6_eligible(x_bits, w_bits, int(bool(signed)), k))
@@ -319,7 +339,7 @@ class Gemm:
     def __init__(self, x_planes, w_planes, signed, out=None, cfg=None, out_kind=OUT_I32, c_scale=None,
                  x_scale=None, w_scale=None, group_size=0, x_tiled=False, w_tiled=False, workspace=None,
                  x_zero=None, w_zero=None, x_group_sums=None, w_zero_term=None, act=ACT_NONE,
-                 x_fp6=0, w_fp6=0, x_row_sums=None, w_row_sums=None):
+                 x_fp6=0, w_fp6=0, x_row_sums=None, w_row_sums=None, value_bits=None):
         import torch
         if x_fp6:
             kt, M, _ = x_planes.shape
@@ -365,6 +385,9 @@ class Gemm:
             _check(lib().abq_gemm_set_operand_layout(ctypes.byref(self.state), xl, wl), "abq_gemm_set_operand_layout")
         if act != ACT_NONE:
             _check(lib().abq_gemm_set_activation(ctypes.byref(self.state), act), "abq_gemm_set_activation")
+        if value_bits is not None:  # (x, w): the codes' real widths inside padded records
+            _check(lib().abq_gemm_set_value_bits(ctypes.byref(self.state), int(value_bits[0]), int(value_bits[1])),
+                   "abq_gemm_set_value_bits")
         self.row_sums = (x_row_sums, w_row_sums)
         if x_row_sums is not None or w_row_sums is not None:
             _check(lib().abq_gemm_set_row_sums(ctypes.byref(self.state), x_row_sums.data_ptr() if x_row_sums is not None else None,

@@ -19,6 +19,7 @@ hipError_t launch_pack_f16(const void *, const float *, uint32_t *, int, int, in
 hipError_t launch_pack_f16_tiled(const void *, const float *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
+hipError_t launch_relayout_planes_padded(const uint32_t *, uint32_t *, int, int, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes_fp6(const uint32_t *, uint32_t *, int, int, int, int, hipStream_t);
 hipError_t launch_row_sums(const uint32_t *, int *, int, int, int, hipStream_t);
 const KernelEntry *fp6_entries(int *count);
@@ -976,11 +977,36 @@ static bool decode_tiled_pays(int x_bits, int w_bits, int M, int N, int K)
 // pair.  Variant by shape (measured on MI355X, W2A8, LLaMA-7B widths): sixteen waves with one weight load each
 // in flight while a compute unit holds at most two workgroups; with more tiles than that, eight waves with two
 // loads each (twice the workgroups fit a compute unit).
+// Unsigned 8-bit records on the decode kernel of prepared operands: codes up to 255 are fed as value - 128 and need
+// the other operand's row sums (abq_gemm_set_row_sums); records declared to hold narrower codes
+// (abq_gemm_set_value_bits: padded records) are fed as they are.  flip_x / flip_w: which operands are flipped.
+static void decode_tiled_flips(const abq_gemm_state *st, int *flip_x, int *flip_w)
+{
+    const abq_tile_config &c = st->cfg;
+    *flip_x = !c.is_signed && c.x_bits == 8 && (st->reserved[2] == 0 || st->reserved[2] == 8);
+    *flip_w = !c.is_signed && c.w_bits == 8 && (st->reserved[3] == 0 || st->reserved[3] == 8);
+}
+
+// Whether that kernel can run the state as it stands: the sums are there, and two 8-bit operands are either both
+// flipped or both not (there is no instance for a mix).
+static bool decode_tiled_flips_ok(const abq_gemm_state *st)
+{
+    int fx, fw;
+    decode_tiled_flips(st, &fx, &fw);
+    if (fx && !st->w_row_sums)
+        return false;
+    if (fw && !st->x_row_sums)
+        return false;
+    if (!st->cfg.is_signed && st->cfg.x_bits == 8 && st->cfg.w_bits == 8 && fx != fw)
+        return false;
+    return true;
+}
+
 static abq_status switch_to_decode_tiled(abq_gemm_state *st)
 {
     const abq_tile_config &c = st->cfg;
     const KernelTable *tdt = find_table(registry().decode_tiled, c.x_bits, c.w_bits, c.is_signed);
-    if (!tdt || tdt->count == 0)
+    if (!tdt || tdt->count == 0 || !decode_tiled_flips_ok(st))
         return ABQ_ERR_UNSUPPORTED;
     const int tiles = (st->N + 15) / 16;
     const int steps = (st->K / 128 * c.w_bits + 3) / 4;
@@ -1150,6 +1176,8 @@ static void apply_tuned(abq_gemm_state *st)
     // prefill kernels; it cannot be chosen before there is one
     if (t.cfg.nstage == 6 && st->x_layout != ABQ_LAYOUT_TILED &&
         (!st->workspace || st->workspace_bytes < planes_bytes(st->M, st->K, c.x_bits)))
+        return;
+    if (t.cfg.nstage == 6 && !decode_tiled_flips_ok(st))
         return;
     if (memcmp(&t.cfg, &st->cfg, sizeof(abq_tile_config)) == 0)
         return;
@@ -1397,13 +1425,54 @@ int abq_gemm_row_sums_ready(const abq_gemm_state *st)
     return row_sum_plan(st, xb + wb).ok ? 1 : 0;
 }
 
+static abq_status switch_to_decode_tiled(abq_gemm_state *st);
+static bool decode_tiled_pays(int x_bits, int w_bits, int M, int N, int K);
+static void apply_tuned(abq_gemm_state *st);
+
+// A state on the prefill kernel whose operands are both prepared, once the decode kernel of that layout has become
+// possible for it (row sums or value bits declared after the layouts): the move abq_gemm_set_operand_layout would
+// have made.
+static void reconsider_decode_tiled(abq_gemm_state *st)
+{
+    if (st->strategy == ABQ_STRATEGY_TILED && st->auto_chosen && !st->group_size && !st->act && st->x_layout == ABQ_LAYOUT_TILED &&
+        st->w_layout == ABQ_LAYOUT_TILED && decode_tiled_pays(st->cfg.x_bits, st->cfg.w_bits, st->M, st->N, st->K))
+        (void)switch_to_decode_tiled(st);
+    apply_tuned(st);
+}
+
 abq_status abq_gemm_set_row_sums(abq_gemm_state *st, const int32_t *x_row_sums, const int32_t *w_row_sums)
 {
     if (!st || !st->init_success)
         return ABQ_ERR_NOT_INITIALIZED;
     st->x_row_sums = x_row_sums;
     st->w_row_sums = w_row_sums;
+    reconsider_decode_tiled(st);
     return ABQ_OK;
+}
+
+abq_status abq_gemm_set_value_bits(abq_gemm_state *st, int x_value_bits, int w_value_bits)
+{
+    if (!st || !st->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    if (x_value_bits < 1 || x_value_bits > st->cfg.x_bits || w_value_bits < 1 || w_value_bits > st->cfg.w_bits)
+        return ABQ_ERR_INVALID_ARG;
+    st->reserved[2] = x_value_bits;
+    st->reserved[3] = w_value_bits;
+    reconsider_decode_tiled(st);
+    return ABQ_OK;
+}
+
+int abq_padded_bits(int bits) { return bits < 1 || bits > 8 ? 0 : bits <= 2 ? 2 : bits <= 4 ? 4 : 8; }
+
+abq_status abq_relayout_planes_padded(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits, int is_signed,
+                                      void *stream)
+{
+    if (!planes || !tiled || rows <= 0 || bits < 1 || bits > 8)
+        return ABQ_ERR_INVALID_ARG;
+    if (k < 128 || k % 128 != 0)
+        return ABQ_ERR_BAD_K;
+    return hip_status(launch_relayout_planes_padded(planes, tiled, rows, k, abq_padded_bits(bits), bits, is_signed ? 1 : 0,
+                                                    (hipStream_t)stream));
 }
 
 abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
@@ -1436,6 +1505,9 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     a.x_dynamic = st->x_layout == ABQ_LAYOUT_F16 ? st->reserved[1] : 0;
     a.x_row_sums = st->x_row_sums;
     a.w_row_sums = st->w_row_sums;
+    decode_tiled_flips(st, &a.flip_x, &a.flip_w);
+    if (st->strategy == ABQ_STRATEGY_DECODE_TILED && !decode_tiled_flips_ok(st))
+        return ABQ_ERR_INVALID_ARG; // unsigned 8-bit codes on this kernel need their row sums
     const Registry &reg = registry();
     const abq_tile_config &c = st->cfg;
     hipError_t e;

@@ -42,11 +42,8 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 constexpr bool decode_tiled_width(int b) { return b == 2 || b == 4 || b == 8; }
-// single-field widths; an unsigned 8-bit operand would need the row-sum corrections of the other kernels
-constexpr bool decode_tiled_built(int q, int p, bool is_signed)
-{
-    return decode_tiled_width(q) && decode_tiled_width(p) && q >= p && (is_signed || (q < 8 && p < 8));
-}
+// single-field widths, activations at least as wide as the weights
+constexpr bool decode_tiled_built(int q, int p) { return decode_tiled_width(q) && decode_tiled_width(p) && q >= p; }
 
 __device__ __forceinline__ void dt_load_to_lds(const void *src, unsigned lds_addr)
 {
@@ -140,10 +137,16 @@ template <int BITS, bool SIGNED> __device__ __forceinline__ void dt_unpack(const
 // XF16 is the number of 16-byte units of eight halves a thread holds per pass (0: the activations arrive packed; 1, 2
 // or 4, the launcher takes the fewest that cover the rows in one pass, at most 4: eight rows of 4096 with sixteen waves;
 // more spills, and with four the instances need 95 - 104 registers against 52 - 67, which costs workgroups per unit).
-template <int Q, int P, bool SIGNED, int NW, int D, int T, int XF16 = 0>
+// FLIP (unsigned pairs): the 8-bit records hold codes up to 255, which the signed matrix cores take as value - 128
+// (bit 7 flipped: one xor per dword after the load); the result is put right with 128 x the other operand's row
+// sums (GemmArgs::x_row_sums / w_row_sums, abq_row_sums) and, when both operands are 8 bits wide, - 2^14 K.  Without
+// FLIP the bytes of an unsigned 8-bit record are fed as they are: padded records of narrower codes (below 128).
+template <int Q, int P, bool SIGNED, int NW, int D, int T, int XF16 = 0, bool FLIP = false>
 __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, int mrows)
 {
     static_assert(!XF16 || Q == 8, "in-kernel quantisation writes 8-bit records");
+    static_assert(!FLIP || (!SIGNED && Q == 8 && !XF16), "flipping is for unsigned 8-bit records");
+    constexpr bool FLIP_X = FLIP && Q == 8, FLIP_W = FLIP && P == 8;
     static_assert(XF16 == 0 || XF16 == 1 || XF16 == 2 || XF16 == 4, "units per thread and pass");
     constexpr int XP = XF16 > 0 ? XF16 : 1;
     constexpr int NXL = Q / P;   // activation chunks (16 bytes) per weight unit
@@ -317,6 +320,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
                     const v4u xv = *reinterpret_cast<const v4u *>(xs + ((uint32_t)rowi * Q + part) * 16u);
                     v4i tt[MX];
                     dt_unpack<Q, SIGNED>(xv, tt);
+                    if constexpr (FLIP_X)
+                        tt[0] = v4i{ tt[0][0] ^ (int)0x80808080u, tt[0][1] ^ (int)0x80808080u, tt[0][2] ^ (int)0x80808080u,
+                                     tt[0][3] ^ (int)0x80808080u };
 #pragma unroll
                     for (int k = 0; k < MX; ++k)
                         av[i * MX + k] = tt[k];
@@ -332,7 +338,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
                 const bool ok = 4 * cs + g < U;
 #pragma unroll
                 for (int t = 0; t < T; ++t) {
-                    const v4u wv = ok ? wb[d][t] : v4u{ 0u, 0u, 0u, 0u };
+                    // (lanes past the end of K feed zeros, also where the weights are flipped)
+                    constexpr unsigned kFlipW = FLIP_W ? 0x80808080u : 0u;
+                    const v4u wv = ok ? v4u{ wb[d][t][0] ^ kFlipW, wb[d][t][1] ^ kFlipW, wb[d][t][2] ^ kFlipW, wb[d][t][3] ^ kFlipW }
+                                      : v4u{ 0u, 0u, 0u, 0u };
                     v4i bv[NM];
                     dt_unpack<P, SIGNED>(wv, bv);
 #pragma unroll
@@ -366,22 +375,28 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
                 v += part[w];
             if (SIGNED)
                 v >>= 16 - Q - P; // both operands were fed at the top of the byte
+            if constexpr (FLIP_X)
+                v = (int)((unsigned)v + 128u * (unsigned)a.w_row_sums[n]);
+            if constexpr (FLIP_W)
+                v = (int)((unsigned)v + 128u * (unsigned)a.x_row_sums[m0 + (rem >> 4)]);
+            if constexpr (FLIP_X && FLIP_W)
+                v = (int)((unsigned)v - 16384u * (unsigned)a.K);
             store_result(a, m0 + (rem >> 4), n, v);
         }
     }
 }
 
-template <int Q, int P, bool SIGNED, int NW, int D, int T, int XU>
+template <int Q, int P, bool SIGNED, int NW, int D, int T, int XU, bool FLIP = false>
 static hipError_t launch_decode_tiled_instance(const GemmArgs &a, int mrows, hipStream_t stream)
 {
     const size_t lds = decode_tiled_lds(NW, T, mrows, a.K, Q);
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled<Q, P, SIGNED, NW, D, T, XU>),
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled<Q, P, SIGNED, NW, D, T, XU, FLIP>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess)
         return attr;
     const int tiles = (a.N + 15) / 16;
     const dim3 grid((tiles + T - 1) / T, (a.M + mrows - 1) / mrows);
-    hipLaunchKernelGGL((gemm_decode_tiled<Q, P, SIGNED, NW, D, T, XU>), grid, dim3(64 * NW), lds, stream, a, mrows);
+    hipLaunchKernelGGL((gemm_decode_tiled<Q, P, SIGNED, NW, D, T, XU, FLIP>), grid, dim3(64 * NW), lds, stream, a, mrows);
     return hipGetLastError();
 }
 
@@ -400,6 +415,15 @@ static hipError_t launch_decode_tiled(const GemmArgs &a, hipStream_t stream)
         if (need <= 2)
             return launch_decode_tiled_instance<Q, P, SIGNED, NW, D, T, 2>(a, mrows, stream);
         return launch_decode_tiled_instance<Q, P, SIGNED, NW, D, T, 4>(a, mrows, stream);
+    } else if constexpr (!SIGNED && Q == 8) {
+        // unsigned 8-bit records: codes up to 255 in every 8-bit operand (flipped, row sums needed), or padded
+        // narrower codes in every one (fed as they are); a mix of the two has no instance
+        const bool flip_x = a.flip_x != 0, flip_w = P == 8 && a.flip_w != 0;
+        if (!flip_x && !flip_w)
+            return launch_decode_tiled_instance<Q, P, SIGNED, NW, D, T, 0>(a, mrows, stream);
+        if (!flip_x || (P == 8 && !flip_w) || !a.w_row_sums || (P == 8 && !a.x_row_sums))
+            return hipErrorInvalidValue;
+        return launch_decode_tiled_instance<Q, P, SIGNED, NW, D, T, 0, true>(a, mrows, stream);
     } else {
         return launch_decode_tiled_instance<Q, P, SIGNED, NW, D, T, 0>(a, mrows, stream);
     }
@@ -910,13 +934,8 @@ static const KernelEntry kUnsignedGrouped[] = { { 16, 1, 1, 1, 1, 16, 6, &launch
 #else
 static const KernelEntry *const kUnsignedGrouped = nullptr;
 #endif
-#if ABQ_Q < 8
 static const KernelEntry kUnsigned[] = { ABQ_DT_VARIANTS(ABQ_DT_ENTRY_F) };
 #define ABQ_DT_NUNSIGNED ((int)(sizeof(kUnsigned) / sizeof(kUnsigned[0])))
-#else
-static const KernelEntry *const kUnsigned = nullptr;
-#define ABQ_DT_NUNSIGNED 0
-#endif
 #define ABQ_DT_NSIGNED ((int)(sizeof(kSigned) / sizeof(kSigned[0])))
 #else
 static const KernelEntry *const kSigned = nullptr;

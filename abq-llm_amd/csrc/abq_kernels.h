@@ -34,6 +34,9 @@ struct GemmArgs {
     // + 128 (x sums if W is) - 2^14 K (if both are)
     const int *x_row_sums;     // [M]
     const int *w_row_sums;     // [N]
+    // the decode kernel on prepared operands, unsigned pairs: whether the 8-bit records of X (W) hold codes up to 255
+    // (fed as value - 128, with the row sums above) or padded narrower codes, which are fed as they are
+    int flip_x, flip_w;
 };
 
 typedef hipError_t (*GemmLauncher)(const GemmArgs &, hipStream_t);

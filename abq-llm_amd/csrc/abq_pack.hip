@@ -131,9 +131,13 @@ __device__ __forceinline__ void store_fields(uint32_t *rec, int ws, const uint32
 // reads 16 bytes per plane (eight threads cover 128 contiguous bytes of a plane row), converts its
 // four word-sets in registers, and parks the record in LDS; the records of one K tile are then
 // contiguous in memory over the 32 rows and leave with coalesced 16-byte stores.
+// in_bits < BITS: the operand has in_bits planes and is written as records of the wider field (padded records, for
+// the widths made of several fields): the planes above it repeat its top plane (signed codes: sign extension) or
+// are zero.
 template <int BITS>
 __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__restrict__ planes,
-                                                              uint32_t *__restrict__ tiled, int rows, int KW)
+                                                              uint32_t *__restrict__ tiled, int rows, int KW, int in_bits,
+                                                              int sign_extend)
 {
     constexpr int REC = BITS * 4;          // words per record
     constexpr int SLAB = 32 * REC + 4;     // words per K tile in LDS (+16 bytes against bank conflicts)
@@ -150,7 +154,9 @@ __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__
             const uint32_t *p = planes + (size_t)row * KW + 4 * kt;
 #pragma unroll
             for (int b = 0; b < BITS; ++b) {
-                const uint4 v = *reinterpret_cast<const uint4 *>(p + b * plane_stride);
+                uint4 v = *reinterpret_cast<const uint4 *>(p + min(b, in_bits - 1) * plane_stride);
+                if (b >= in_bits && !sign_extend)
+                    v = make_uint4(0u, 0u, 0u, 0u);
                 pw[0][b] = v.x; pw[1][b] = v.y; pw[2][b] = v.z; pw[3][b] = v.w;
             }
             uint32_t *rec = buf + j * SLAB + i * REC;
@@ -182,7 +188,8 @@ __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__
 // and its time is one thread's latency chain (512 x 4096 8-bit activations: 64 workgroups there, 256 here).
 template <int BITS>
 __global__ __launch_bounds__(256) void relayout_planes_ws_kernel(const uint32_t *__restrict__ planes,
-                                                                 uint32_t *__restrict__ tiled, int rows, int KW)
+                                                                 uint32_t *__restrict__ tiled, int rows, int KW, int in_bits,
+                                                                 int sign_extend)
 {
     constexpr int REC = BITS * 4;          // words per record
     constexpr int SLAB = 8 * REC + 4;      // words per K tile in LDS (+16 bytes against bank conflicts)
@@ -199,7 +206,7 @@ __global__ __launch_bounds__(256) void relayout_planes_ws_kernel(const uint32_t 
             const uint32_t *p = planes + (size_t)row * KW + kw;
 #pragma unroll
             for (int b = 0; b < BITS; ++b)
-                pw[b] = p[b * plane_stride];
+                pw[b] = (b >= in_bits && !sign_extend) ? 0u : p[min(b, in_bits - 1) * plane_stride];
             planes_to_int8<BITS, kLow>(pw, e);
             compress_fields<BITS>(e, f);
             store_fields<BITS>(buf + (w >> 2) * SLAB + i * REC, w & 3, f);
@@ -216,8 +223,9 @@ __global__ __launch_bounds__(256) void relayout_planes_ws_kernel(const uint32_t 
     }
 }
 
-hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits,
-                                  hipStream_t stream)
+// bits: width of the records written; in_bits <= bits: planes the operand has (sign_extend: what the rest repeats)
+hipError_t launch_relayout_planes_padded(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits, int in_bits,
+                                         int sign_extend, hipStream_t stream)
 {
     const int KW = k / 32;
     const dim3 grid((rows + 31) / 32, (KW / 4 + 7) / 8);
@@ -226,7 +234,7 @@ hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int r
         switch (bits) {
 #define ABQ_RELAYOUT_CASE(B)                                                                                     \
     case B:                                                                                                      \
-        hipLaunchKernelGGL(relayout_planes_ws_kernel<B>, fine, dim3(256), 0, stream, planes, tiled, rows, KW);   \
+        hipLaunchKernelGGL(relayout_planes_ws_kernel<B>, fine, dim3(256), 0, stream, planes, tiled, rows, KW, in_bits, sign_extend); \
         break;
             ABQ_RELAYOUT_CASE(1) ABQ_RELAYOUT_CASE(2) ABQ_RELAYOUT_CASE(3) ABQ_RELAYOUT_CASE(4)
             ABQ_RELAYOUT_CASE(5) ABQ_RELAYOUT_CASE(6) ABQ_RELAYOUT_CASE(7) ABQ_RELAYOUT_CASE(8)
@@ -239,7 +247,7 @@ hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int r
     switch (bits) {
 #define ABQ_RELAYOUT_CASE(B)                                                                                     \
     case B:                                                                                                      \
-        hipLaunchKernelGGL(relayout_planes_kernel<B>, grid, dim3(256), 0, stream, planes, tiled, rows, KW);      \
+        hipLaunchKernelGGL(relayout_planes_kernel<B>, grid, dim3(256), 0, stream, planes, tiled, rows, KW, in_bits, sign_extend); \
         break;
         ABQ_RELAYOUT_CASE(1) ABQ_RELAYOUT_CASE(2) ABQ_RELAYOUT_CASE(3) ABQ_RELAYOUT_CASE(4)
         ABQ_RELAYOUT_CASE(5) ABQ_RELAYOUT_CASE(6) ABQ_RELAYOUT_CASE(7) ABQ_RELAYOUT_CASE(8)
@@ -248,6 +256,11 @@ hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int r
         return hipErrorInvalidValue;
     }
     return hipGetLastError();
+}
+
+hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits, hipStream_t stream)
+{
+    return launch_relayout_planes_padded(planes, tiled, rows, k, bits, bits, 0, stream);
 }
 
 // ---- FP6 records ---------------------------------------------------------------------------

@@ -524,11 +524,15 @@ int main(int argc, char **argv)
 
     // the layout a loader would hold the weights in for this shape (the library's own choice above 16 rows)
     const int preferred = abq_preferred_weight_layout(x_bits, w_bits, is_signed, M, N, K, 0);
+    // ... and when the table's tile for the shape is the decode kernel of prepared operands, the activations come
+    // K-tiled too, as the quantising kernel writes them (what that tile's own line of the sweep is timed on)
+    abq_tile_config tuned;
+    const bool tuned_decode = M > 16 && abq_tuning_lookup(x_bits, w_bits, is_signed, M, N, K, 0, 0, &tuned, nullptr) == ABQ_OK && tuned.nstage == 6;
     auto run_one = [&](const abq_tile_config *cfg, Timing &t, abq_gemm_state &st0, bool prepared = false) {
         std::vector<abq_gemm_state> states(nbuf);
         // tiled tiles (NSTAGE 4) run on prepared weights, NSTAGE 6 and the `prepared` default on prepared weights and
         // activations, the FP6 tiles on FP6 records; the library's own choice for M > 16 on the preferred layout
-        const bool both = prepared || (cfg && cfg->nstage == 6);
+        const bool both = prepared || (cfg ? cfg->nstage == 6 : tuned_decode);
         const bool fp6 = cfg ? cfg->nstage == 5 : (!prepared && M > 16 && preferred == ABQ_LAYOUT_FP6 && fp6_ok);
         const bool tiled = both || (cfg ? cfg->nstage == 4 : (M > 16 && !fp6 && preferred != ABQ_LAYOUT_PLANES));
         if (fp6 && !fp6_ok) {

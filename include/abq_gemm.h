@@ -111,7 +111,9 @@ typedef enum abq_strategy {
                                  of at most 4 bits unsigned / 5 bits signed (see
                                  abq_relayout_planes_fp6); tile tuples with NSTAGE = 5, MMA 32x32x64 */
     ABQ_STRATEGY_DECODE_TILED = 8 /* int8 MFMA 16x16x64 for decode-sized M on operands that are both in the
-                                 K-tiled layout (widths 2, 4 or 8 bits; no unsigned 8-bit operand):
+                                 K-tiled layout (widths 2, 4 or 8 bits; unsigned 8-bit codes with their row
+                                 sums set, abq_gemm_set_row_sums; other widths as padded records,
+                                 abq_relayout_planes_padded):
                                  nothing is expanded or transposed inside the kernel; tile tuples with
                                  NSTAGE = 6.  A state with M <= 16 whose operands are both declared
                                  ABQ_LAYOUT_TILED moves here by itself, and so does one of up to 128 rows
@@ -177,7 +179,8 @@ typedef struct abq_gemm_state {
     const float *x_scale;  /* [M] per token            */
     const float *w_scale;  /* [N] or [N][K/group_size] */
     int group_size;        /* 0 = per channel          */
-    int reserved[5];
+    int reserved[5];       /* [0] popcount kernels: log2 of the lanes per weight row; [1] see
+                              abq_gemm_set_dynamic_f16_activations; [2], [3] see abq_gemm_set_value_bits */
     /* K-tiled operands (ABQ_STRATEGY_TILED) */
     int x_layout, w_layout;  /* abq_layout of X and W as handed to init                    */
     int auto_chosen;         /* 1 if the tile was the library's choice                     */
@@ -403,6 +406,23 @@ abq_status abq_gemm_set_row_sums(abq_gemm_state *state, const int32_t *x_row_sum
 /* 1 if abq_gemm_exec on this state, as it stands, runs the kernel that takes the row sums handed in (every needed
  * sum set, or to be had from plane operands into the workspace the state holds), 0 otherwise. */
 int abq_gemm_row_sums_ready(const abq_gemm_state *state);
+
+/* Padded records for the widths made of several fields.  The decode kernel on prepared operands reads records of one
+ * field per element (2, 4 or 8 bits).  An operand of 3, 5, 6 or 7 bits is brought to it as records of the next such
+ * width, abq_padded_bits(bits) (1, 2 -> 2; 3, 4 -> 4; 5..8 -> 8), the code of every element extended to that width
+ * (sign extension for signed codes): the values, and therefore the GEMM, are the same, the records are
+ * abq_planes_bytes(rows, k, abq_padded_bits(bits)) long.  The GEMM is then initialised with the padded widths, its
+ * operands declared ABQ_LAYOUT_TILED, and (unsigned pairs whose records are 8 bits wide) told through
+ * abq_gemm_set_value_bits how many bits the codes really have: 8-bit records of at most 7-bit codes are fed to the
+ * matrix cores as they are, while true 8-bit codes need the value - 128 route and its row sums.  For widths of one
+ * field the call equals abq_relayout_planes.  No counterpart in the reference (its binary tensor cores take any
+ * number of planes; its decode sweep over these widths: engine/test.sh:8-206). */
+int abq_padded_bits(int bits);
+abq_status abq_relayout_planes_padded(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits, int is_signed,
+                                      void *stream);
+/* Declares that the codes of X (W) use only the low x_value_bits (w_value_bits) of their fields (1 .. the state's
+ * widths): see above. */
+abq_status abq_gemm_set_value_bits(abq_gemm_state *state, int x_value_bits, int w_value_bits);
 
 /* Workspace needed by abq_gemm_exec if the state ran as ABQ_STRATEGY_TILED, ABQ_STRATEGY_DECODE_TILED
  * (ABQ_STRATEGY_FP6) with its current operand layouts: the converted copies of the operands still in

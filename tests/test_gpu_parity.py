@@ -492,7 +492,7 @@ def test_decode_kernel_k_chunking_and_many_tiles(abq, oracle):
             assert np.array_equal(got, want), (abq.format_kernel_name(cfg), M, N, K)
 
 
-DECODE_TILED_PAIRS = [(2, 2), (4, 2), (8, 2), (4, 4), (8, 4), (8, 8)]
+DECODE_TILED_PAIRS = COMBOS  # all twelve pairs of the reference's library
 
 
 @pytest.mark.parametrize("q,p", DECODE_TILED_PAIRS)
@@ -501,29 +501,54 @@ def test_decode_on_prepared_operands(abq, oracle, q, p, signed):
     """Decode-sized GEMM with both operands K-tiled: the library moves to the decode kernel of that layout by
     itself (no workspace, one launch); every tile tuple of that kernel on ragged shapes: partial tiles of N, an odd
     number of K tiles (half-filled last step), M past 16 (several row blocks), long K (rows per workgroup limited
-    by the LDS), more steps than the waves hold in flight."""
-    built = signed or q < 8
+    by the LDS), more steps than the waves hold in flight.  Widths made of several fields (3, 5, 6, 7 bits) come as
+    padded records of the next single-field width; unsigned 8-bit codes bring their row sums."""
+    qp, pp = abq.padded_bits(q), abq.padded_bits(p)
+    padded = (qp, pp) != (q, p)
     rng = np.random.default_rng(500 + 10 * q + p + int(signed))
     shapes = [(1, 64, 128), (1, 4096, 4096), (3, 37, 384), (4, 200, 1408), (8, 130, 1152), (8, 64, 11008), (13, 72, 4096),
               (16, 100, 13824), (16, 48, 2048), (17, 64, 512), (40, 96, 640), (2, 300, 24576)]
     for (M, N, K) in shapes:
         x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+        if M > 1:
+            x[1] = (1 << (q - 1)) - 1 if signed else (1 << q) - 1  # a row of the largest code ...
+            w[0] = -(1 << (p - 1)) if signed else (1 << p) - 1      # ... against one of the code furthest from zero
         xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
-        xt, wt = abq.relayout_planes(xd), abq.relayout_planes(wd)
+        xt, wt = abq.relayout_planes_padded(xd, signed), abq.relayout_planes_padded(wd, signed)
+        assert xt.shape == (K // 128, M, qp, 4) and wt.shape == (K // 128, N, pp, 4)
+        if not padded:  # for the widths of one field the padded records are the K-tiled records
+            assert torch.equal(xt, abq.relayout_planes(xd)) and torch.equal(wt, abq.relayout_planes(wd))
         want = oracle.np_gemm(x, w)
-        g = abq.Gemm(xt, wt, signed, x_tiled=True, w_tiled=True)
+        kw = dict(x_tiled=True, w_tiled=True)
+        if padded:
+            kw["value_bits"] = (q, p)
+        needs_sums = not signed and 8 in (q, p)
+        if needs_sums:
+            # without the row sums a state of unsigned 8-bit codes stays on the prefill kernel, which takes them itself
+            g = abq.Gemm(xt, wt, signed, **kw)
+            assert g.strategy == "tiled"
+            assert np.array_equal(g.run().cpu().numpy(), want), (g.config_name, M, N, K)
+            kw.update(x_row_sums=abq.row_sums(xd), w_row_sums=abq.row_sums(wd))
+        g = abq.Gemm(xt, wt, signed, **kw)
+        assert (g.state.cfg.x_bits, g.state.cfg.w_bits) == (qp, pp)
         # up to 16 rows always; up to 128 rows where the library estimates the decode kernel ahead (several blocks of rows)
-        assert g.strategy == "decode_tiled" if built and M <= 16 else g.strategy in ("decode_tiled", "tiled"), (g.strategy, M, N, K)
-        assert built or g.strategy == "tiled"
+        assert g.strategy == "decode_tiled" if M <= 16 else g.strategy in ("decode_tiled", "tiled"), (g.strategy, M, N, K)
         assert g.workspace_bytes == 0
         assert np.array_equal(g.run().cpu().numpy(), want), (g.config_name, M, N, K)
-        for cfg in abq.native_configs(q, p, signed):
+        ran = 0
+        for cfg in abq.native_configs(qp, pp, signed):
             if cfg.nstage != 6:
                 continue
             out = torch.full((M, N), -12345, dtype=torch.int32, device="cuda")
-            got = abq.Gemm(xt, wt, signed, cfg=cfg, out=out, x_tiled=True, w_tiled=True).run().cpu().numpy()
+            got = abq.Gemm(xt, wt, signed, cfg=cfg, out=out, **kw).run().cpu().numpy()
             assert np.array_equal(got, want), (abq.format_kernel_name(cfg), M, N, K)
-    assert built == any(c.nstage == 6 for c in abq.native_configs(q, p, signed))
+            ran += 1
+        assert ran == 5
+        if needs_sums:  # a tile of this kernel named by the caller, but no sums: refused before any launch
+            cfg = [c for c in abq.native_configs(qp, pp, signed) if c.nstage == 6][0]
+            with pytest.raises(abq.AbqError) as e:
+                abq.Gemm(xt, wt, signed, cfg=cfg, x_tiled=True, w_tiled=True, **({"value_bits": (q, p)} if padded else {})).run()
+            assert e.value.status == abq.ABQ_ERR_INVALID_ARG
 
 
 def test_decode_kernel_over_row_blocks_is_the_default_where_it_pays(abq, oracle):

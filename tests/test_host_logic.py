@@ -550,6 +550,42 @@ def test_compiled_in_tuning_table_serves_the_sweep_it_came_from(abq):
         lib.abq_tuning_enable_builtin(1)
 
 
+def test_unsigned_8bit_codes_reach_the_prepared_decode_kernel_with_their_row_sums(abq):
+    """Unsigned 8-bit codes are fed as value - 128: the decode kernel on prepared operands takes such a state only once
+    the row sums are set; padded records of narrower codes (value bits declared) need none."""
+    lib = abq.lib()
+    T = abq.LAYOUT_TILED
+    names = abq.STRATEGY_NAMES
+
+    def state(q, p, M=4):
+        rc, st = _init(abq, q=q, p=p, M=M, signed=0, N=4096, K=4096)
+        assert rc == 0 and lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0
+        return st
+
+    st = state(8, 8)
+    assert names[st.strategy] == "tiled"
+    assert lib.abq_gemm_set_row_sums(ctypes.byref(st), 0x7000, None) == 0 and names[st.strategy] == "tiled"  # both are needed
+    assert lib.abq_gemm_set_row_sums(ctypes.byref(st), 0x7000, 0x8000) == 0 and names[st.strategy] == "decode_tiled"
+    st = state(8, 2)
+    assert names[st.strategy] == "tiled"
+    assert lib.abq_gemm_set_row_sums(ctypes.byref(st), None, 0x8000) == 0 and names[st.strategy] == "decode_tiled"
+    # padded records: 7-bit codes in 8-bit fields need no sums; a mix of real and padded 8-bit operands has no kernel there
+    st = state(8, 8)
+    assert lib.abq_gemm_set_value_bits(ctypes.byref(st), 7, 7) == 0 and names[st.strategy] == "decode_tiled"
+    st = state(8, 8)
+    assert lib.abq_gemm_set_value_bits(ctypes.byref(st), 8, 7) == 0
+    assert lib.abq_gemm_set_row_sums(ctypes.byref(st), 0x7000, 0x8000) == 0 and names[st.strategy] == "tiled"
+    st = state(8, 2)
+    assert lib.abq_gemm_set_value_bits(ctypes.byref(st), 6, 2) == 0 and names[st.strategy] == "decode_tiled"
+    assert lib.abq_gemm_set_value_bits(ctypes.byref(st), 9, 2) == abq.ABQ_ERR_INVALID_ARG
+    assert lib.abq_gemm_set_value_bits(ctypes.byref(st), 6, 0) == abq.ABQ_ERR_INVALID_ARG
+    # more than 16 rows: where the prefill kernel is the better choice the sums change nothing about the strategy
+    st = state(8, 8, M=512)
+    assert lib.abq_gemm_set_row_sums(ctypes.byref(st), 0x7000, 0x8000) == 0 and names[st.strategy] == "tiled"
+    assert lib.abq_gemm_row_sums_ready(ctypes.byref(st)) == 1
+    assert [abq.padded_bits(b) for b in range(0, 10)] == [0, 2, 2, 4, 4, 8, 8, 8, 8, 0]
+
+
 def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     """The tile the library picks for prepared operands, pinned on shapes of BASELINE.json configs[2] and
     configs[4] and on a few where the measured sweep of all tiles separates them clearly:
