@@ -1384,7 +1384,12 @@ static RowSumPlan row_sum_plan(const abq_gemm_state *st, size_t converted)
 {
     const abq_tile_config &c = st->cfg;
     RowSumPlan p{ true, 0, 0, 0 };
-    const bool take_x = c.w_bits == 8 && !st->x_row_sums, take_w = c.x_bits == 8 && !st->w_row_sums;
+    // which operands are fed as value - 128: every unsigned 8-bit one on the prefill kernel; on the decode kernel of
+    // prepared operands those whose codes are not declared narrower
+    int flip_x = c.x_bits == 8, flip_w = c.w_bits == 8;
+    if (st->strategy == ABQ_STRATEGY_DECODE_TILED)
+        decode_tiled_flips(st, &flip_x, &flip_w);
+    const bool take_x = flip_w && !st->x_row_sums, take_w = flip_x && !st->w_row_sums;
     if ((take_x && st->x_layout != ABQ_LAYOUT_PLANES) || (take_w && st->w_layout != ABQ_LAYOUT_PLANES)) {
         p.ok = false; // a sum that is neither set nor to be had: the other kernel runs, and asks for nothing
         return p;
@@ -1401,7 +1406,14 @@ static RowSumPlan row_sum_plan(const abq_gemm_state *st, size_t converted)
 // Whether the state's kernel is one that wants row sums handed in.
 static bool wants_row_sums(const abq_gemm_state *st)
 {
-    if (st->strategy != ABQ_STRATEGY_TILED || st->group_size || st->cfg.is_signed || (st->cfg.x_bits != 8 && st->cfg.w_bits != 8))
+    if (st->group_size || st->cfg.is_signed || (st->cfg.x_bits != 8 && st->cfg.w_bits != 8))
+        return false;
+    if (st->strategy == ABQ_STRATEGY_DECODE_TILED) {
+        int fx, fw;
+        decode_tiled_flips(st, &fx, &fw);
+        return fx || fw;
+    }
+    if (st->strategy != ABQ_STRATEGY_TILED)
         return false;
     const KernelTable *t = find_table(registry().tiled, st->cfg.x_bits, st->cfg.w_bits, 0);
     return t && st->variant >= 0 && st->variant < t->count && (t->entries[st->variant].flags & kNeedsRowSums);
@@ -1506,8 +1518,6 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     a.x_row_sums = st->x_row_sums;
     a.w_row_sums = st->w_row_sums;
     decode_tiled_flips(st, &a.flip_x, &a.flip_w);
-    if (st->strategy == ABQ_STRATEGY_DECODE_TILED && !decode_tiled_flips_ok(st))
-        return ABQ_ERR_INVALID_ARG; // unsigned 8-bit codes on this kernel need their row sums
     const Registry &reg = registry();
     const abq_tile_config &c = st->cfg;
     hipError_t e;
@@ -1578,7 +1588,25 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
         if (!t || st->variant < 0 || st->variant >= t->count)
             return ABQ_ERR_NOT_INITIALIZED;
         int variant = st->variant;
-        if (t->entries[variant].flags & kNeedsRowSums) {
+        if (st->strategy == ABQ_STRATEGY_DECODE_TILED && (a.flip_x || a.flip_w) && !c.is_signed) {
+            // unsigned 8-bit codes on the decode kernel: the sums the caller set, or those of an operand that arrived
+            // as planes, taken into the workspace behind its converted copy; there is no kernel to fall back to
+            const RowSumPlan plan = row_sum_plan(st, xb + wb);
+            if (!plan.ok || (c.x_bits == 8 && c.w_bits == 8 && a.flip_x != a.flip_w))
+                return ABQ_ERR_INVALID_ARG;
+            if (a.flip_w && !st->x_row_sums) {
+                e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, c.x_bits, (hipStream_t)stream);
+                if (e != hipSuccess)
+                    return hip_status(e);
+                a.x_row_sums = reinterpret_cast<const int *>(ws + plan.x_off);
+            }
+            if (a.flip_x && !st->w_row_sums) {
+                e = launch_row_sums(st->W, reinterpret_cast<int *>(ws + plan.w_off), st->N, st->K, c.w_bits, (hipStream_t)stream);
+                if (e != hipSuccess)
+                    return hip_status(e);
+                a.w_row_sums = reinterpret_cast<const int *>(ws + plan.w_off);
+            }
+        } else if (t->entries[variant].flags & kNeedsRowSums) {
             // An unsigned 8-bit operand is fed as value - 128 and the other operand's row sums put the result right.
             // The sums the caller set are taken; those of an operand still in planes are taken here, into the
             // workspace behind the converted copies, if it has the room.  Otherwise the kernel of the same tile
