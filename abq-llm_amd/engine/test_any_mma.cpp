@@ -488,6 +488,33 @@ int main(int argc, char **argv)
         HIP_OK(hipStreamSynchronize(stream));
     }
 
+    // Decode-sized M: the "prepared operands" line of the widths made of several fields (3, 5, 6, 7 bits) runs on padded
+    // records (abq_relayout_planes_padded: the next width of 2, 4 or 8 bits), and unsigned 8-bit codes bring their row
+    // sums (abq_row_sums), which is how the decode kernel of prepared operands serves those pairs.
+    const int xq = abq_padded_bits(x_bits), wq = abq_padded_bits(w_bits);
+    const bool padded = xq != x_bits || wq != w_bits;
+    const bool with_sums = !is_signed && (x_bits == 8 || w_bits == 8);
+    const size_t wpad_bytes = abq_planes_bytes(N, K, wq);
+    size_t nbuf_pad = std::min<size_t>(4096, std::max<size_t>(1, ((size_t)rotate_mib << 20) / wpad_bytes));
+    uint32_t *d_xpad = nullptr, *d_wpad = nullptr;
+    int *d_xsum = nullptr, *d_wsum = nullptr;
+    if (M <= 16 && (padded || with_sums)) {
+        HIP_OK(hipMalloc(&d_xpad, abq_planes_bytes(M, K, xq)));
+        HIP_OK(hipMalloc(&d_wpad, wpad_bytes * nbuf_pad));
+        HIP_OK(hipMalloc(&d_xsum, (size_t)M * 4));
+        HIP_OK(hipMalloc(&d_wsum, (size_t)N * 4));
+        if (abq_relayout_planes_padded(d_xp, d_xpad, M, K, x_bits, is_signed, stream) != ABQ_OK ||
+            abq_relayout_planes_padded(d_wp, d_wpad, N, K, w_bits, is_signed, stream) != ABQ_OK ||
+            abq_row_sums(d_xp, M, K, x_bits, d_xsum, stream) != ABQ_OK || abq_row_sums(d_wp, N, K, w_bits, d_wsum, stream) != ABQ_OK) {
+            std::printf("preparing padded records failed (hip error %d)\n", abq_last_hip_error());
+            return -1;
+        }
+        HIP_OK(hipStreamSynchronize(stream));
+        for (size_t b = 1; b < nbuf_pad; ++b)
+            HIP_OK(hipMemcpyAsync((char *)d_wpad + b * wpad_bytes, d_wpad, wpad_bytes, hipMemcpyDeviceToDevice, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+    }
+
     if (group)
         return sweep_group_scales(M, N, K, x_bits, w_bits, is_signed, group, group_fp6, h_x, h_w, d_xp, d_xt, d_wt, d_wf, wp_bytes,
                                   wf_bytes, nbuf, repeat, warmup, only, stream);
@@ -539,11 +566,21 @@ int main(int argc, char **argv)
             t.status = -1;
             return;
         }
-        for (size_t b = 0; b < nbuf; ++b) {
-            const char *wbase = fp6 ? (const char *)d_wf + b * wf_bytes
-                                    : (tiled ? (const char *)d_wt : (const char *)d_wp) + b * wp_bytes;
-            abq_status s = abq_gemm_init(cfg, x_bits, w_bits, is_signed, both ? d_xt : d_xp, (const uint32_t *)wbase,
+        // (the prepared default of pairs the decode kernel serves through padded records or row sums)
+        const bool via_padded = prepared && d_wpad != nullptr;
+        if (via_padded)
+            states.resize(nbuf_pad);
+        for (size_t b = 0; b < states.size(); ++b) {
+            const char *wbase = via_padded ? (const char *)d_wpad + b * wpad_bytes
+                                : fp6      ? (const char *)d_wf + b * wf_bytes
+                                           : (tiled ? (const char *)d_wt : (const char *)d_wp) + b * wp_bytes;
+            abq_status s = abq_gemm_init(cfg, via_padded ? xq : x_bits, via_padded ? wq : w_bits, is_signed,
+                                         via_padded ? d_xpad : both ? d_xt : d_xp, (const uint32_t *)wbase,
                                          M, N, K, d_out, nullptr, 0, ABQ_OUT_I32, &states[b]);
+            if (s == ABQ_OK && via_padded && padded)
+                s = abq_gemm_set_value_bits(&states[b], x_bits, w_bits);
+            if (s == ABQ_OK && via_padded && with_sums)
+                s = abq_gemm_set_row_sums(&states[b], d_xsum, d_wsum);
             if (s == ABQ_OK && tiled)
                 s = abq_gemm_set_operand_layout(&states[b], both ? ABQ_LAYOUT_TILED : ABQ_LAYOUT_PLANES, ABQ_LAYOUT_TILED);
             if (s == ABQ_OK && fp6)
@@ -564,7 +601,7 @@ int main(int argc, char **argv)
         HIP_OK(hipMemcpy(h_out.data(), d_out, (size_t)M * N * 4, hipMemcpyDeviceToHost));
         t.status = std::memcmp(h_out.data(), h_ref.data(), (size_t)M * N * 4) == 0 ? 0 : -2;
         for (int i = 0; i < warmup; ++i)
-            abq_gemm_exec(&states[i % nbuf], stream);
+            abq_gemm_exec(&states[i % states.size()], stream);
         HIP_OK(hipStreamSynchronize(stream));
         float ms = 0;
         if (use_graph) {
@@ -572,7 +609,7 @@ int main(int argc, char **argv)
             hipGraphExec_t ge;
             HIP_OK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
             for (int i = 0; i < repeat; ++i)
-                abq_gemm_exec(&states[i % nbuf], stream);
+                abq_gemm_exec(&states[i % states.size()], stream);
             HIP_OK(hipStreamEndCapture(stream, &g));
             HIP_OK(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0));
             warm_replays(ge, stream);
@@ -586,7 +623,7 @@ int main(int argc, char **argv)
         } else {
             HIP_OK(hipEventRecord(e0, stream));
             for (int i = 0; i < repeat; ++i)
-                abq_gemm_exec(&states[i % nbuf], stream);
+                abq_gemm_exec(&states[i % states.size()], stream);
             HIP_OK(hipEventRecord(e1, stream));
             HIP_OK(hipStreamSynchronize(stream));
             HIP_OK(hipEventElapsedTime(&ms, e0, e1));
@@ -610,7 +647,7 @@ int main(int argc, char **argv)
             continue;
         char name[160] = "library default";
         if (prepared)
-            std::snprintf(name, sizeof name, "library default, prepared operands");
+            std::snprintf(name, sizeof name, "library default, prepared operands%s", d_wpad ? (padded ? " (padded records)" : " (with row sums)") : "");
         if (!library_default)
             abq_format_kernel_name(&cfg, 0, name, sizeof name);
         if (!only.empty() && std::string(name).find(only) == std::string::npos)
@@ -626,7 +663,9 @@ int main(int argc, char **argv)
         std::printf("packing %f (us) exec %f (us) %f TOPS | %f B-TOPS | %s | %.1f%% HBM %.1f%% MFMA%s\n", t.pack_us,
                     t.exec_us, tops, tops * x_bits * w_bits, t.status == 0 ? "PASSED" : t.status == -1 ? "ERROR" : "FAILED",
                     t.status == 0 ? 100.0 * alg_bytes / (t.exec_us * 1e-6) / 8e12 : 0.0, 100.0 * tops / 5000.0,
-                    prepared ? " | library default, prepared operands" : library_default ? " | library default" : "");
+                    prepared ? (d_wpad ? (padded ? " | library default, prepared operands (padded records)" : " | library default, prepared operands (with row sums)")
+                                       : " | library default, prepared operands")
+                             : library_default ? " | library default" : "");
         if (t.status == 0 && !library_default && tops > best_tops) {
             best_tops = tops;
             char buf[128];
