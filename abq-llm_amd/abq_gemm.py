@@ -35,7 +35,7 @@ EXPORTED = [
     "abq_planes_bytes", "abq_relayout_planes", "abq_gemm_set_operand_layout", "abq_gemm_workspace_bytes",
     "abq_gemm_set_workspace", "abq_fp6_bytes", "abq_fp6_eligible", "abq_prepared_decode_pays", "abq_gemm_set_dynamic_f16_activations", "abq_relayout_planes_fp6",
     "abq_gemm_set_zero_points", "abq_weight_zero_term", "abq_quant_pack_f16", "abq_gemm_set_activation",
-    "abq_probe_launch", "abq_gemm_exec_static", "abq_gemm_set_f16_activations",
+    "abq_gemm_exec_static", "abq_gemm_set_f16_activations",
     "abq_row_sums", "abq_gemm_set_row_sums", "abq_gemm_row_sums_ready",
     "abq_tuning_load", "abq_tuning_add", "abq_tuning_clear", "abq_tuning_enable_builtin", "abq_tuning_lookup",
     "abq_preferred_weight_layout", "abq_padded_bits", "abq_relayout_planes_padded", "abq_gemm_set_value_bits",
@@ -153,7 +153,6 @@ def lib():
         L.abq_gemm_set_activation.argtypes = [ctypes.POINTER(GemmState), ci]
         L.abq_weight_zero_term.argtypes = [vp, ci, ci, ci, ci, vp, vp, ci, vp, vp]
         L.abq_quant_pack_f16.argtypes = [vp, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, vp]
-        L.abq_probe_launch.argtypes = [ci, vp, ctypes.c_size_t, vp]
         _lib = L
     return _lib
 

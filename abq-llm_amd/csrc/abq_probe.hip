@@ -3,7 +3,7 @@
 // touches nothing but registers, on operand bits the caller chooses (the clock of the matrix cores follows the
 // power their data makes them draw: the rate on random bits is the ceiling of a GEMM on such data, not the
 // datasheet figure).  No counterpart in the reference.
-#include "abq_gemm.h"
+#include "abq_probe.h"
 
 #include <hip/hip_runtime.h>
 

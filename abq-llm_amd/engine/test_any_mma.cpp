@@ -53,6 +53,7 @@
 #include <vector>
 
 #include "abq_gemm.h"
+#include "abq_probe.h" // measurement probes, not part of the library's interface
 
 #define HIP_OK(x)                                                                        \
     do {                                                                                 \

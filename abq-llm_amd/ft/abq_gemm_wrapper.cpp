@@ -5,6 +5,8 @@
 
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
 
 #include <mutex>
 #include <unordered_map>
@@ -15,6 +17,8 @@ namespace {
 
 struct PreparedWeight {
     int N, K, bits;
+    bool ready;              // false while prepare_weight is still converting (the entry reserves the pointer)
+    uint32_t fingerprint[16]; // the first 64 bytes of the prepared records, for verify_prepared
 };
 
 std::mutex g_prepared_mutex;
@@ -29,10 +33,22 @@ bool find_prepared(const void *B, PreparedWeight *out)
 {
     std::lock_guard<std::mutex> lock(g_prepared_mutex);
     const auto it = prepared_table().find(B);
-    if (it == prepared_table().end())
+    if (it == prepared_table().end() || !it->second.ready)
         return false;
     *out = it->second;
     return true;
+}
+
+// ABQ_VERIFY_PREPARED=1 in the environment: every gemm() on a prepared weight first compares the weight's first
+// record with what prepare_weight left there (a device read and a synchronisation per call: for debugging a
+// loader that frees or refills weight buffers without release_weight, not for production).
+bool verify_on_every_call()
+{
+    static const bool on = [] {
+        const char *v = getenv("ABQ_VERIFY_PREPARED");
+        return v && v[0] == '1';
+    }();
+    return on;
 }
 
 } // namespace
@@ -45,25 +61,52 @@ bool ABQGEMMWrapper::prepare_weight(int *B, int N, int K, int W_BITS, int *scrat
         printf("[ABQ][Error] prepare_weight: bad argument (N, K, bits = %d, %d, %d)\n", N, K, W_BITS);
         return false;
     }
-    PreparedWeight seen;
-    if (find_prepared(B, &seen)) {
-        printf("[ABQ][Error] prepare_weight: %p is prepared already\n", (void *)B);
-        return false;
+    {
+        // check and insert in one critical section: of two threads that prepare the same B one is refused; the
+        // entry is not ready (gemm() does not see it) until the records are in place
+        std::lock_guard<std::mutex> lock(g_prepared_mutex);
+        if (prepared_table().count(B)) {
+            printf("[ABQ][Error] prepare_weight: %p is prepared already\n", (void *)B);
+            return false;
+        }
+        prepared_table()[B] = PreparedWeight{ N, K, W_BITS, false, { 0 } };
     }
+    auto fail = [&](const char *what) {
+        printf("[ABQ][Error] prepare_weight failed: %s\n", what);
+        std::lock_guard<std::mutex> lock(g_prepared_mutex);
+        prepared_table().erase(B);
+        return false;
+    };
     const abq_status rc = abq_relayout_planes(reinterpret_cast<const uint32_t *>(B), reinterpret_cast<uint32_t *>(scratch),
                                               N, K, W_BITS, stream);
-    if (rc != ABQ_OK) {
-        printf("[ABQ][Error] prepare_weight failed: %s\n", abq_status_string(rc));
-        return false;
-    }
-    const hipError_t e = hipMemcpyAsync(B, scratch, abq_planes_bytes(N, K, W_BITS), hipMemcpyDeviceToDevice, stream);
-    if (e != hipSuccess) {
-        printf("[ABQ][Error] prepare_weight failed: %s\n", hipGetErrorString(e));
-        return false;
-    }
+    if (rc != ABQ_OK)
+        return fail(abq_status_string(rc));
+    hipError_t e = hipMemcpyAsync(B, scratch, abq_planes_bytes(N, K, W_BITS), hipMemcpyDeviceToDevice, stream);
+    if (e != hipSuccess)
+        return fail(hipGetErrorString(e));
+    // the first record's bytes as they now are (one small read and a synchronisation, once per weight matrix)
+    PreparedWeight entry{ N, K, W_BITS, true, { 0 } };
+    const size_t nfp = abq_planes_bytes(N, K, W_BITS) < sizeof entry.fingerprint ? abq_planes_bytes(N, K, W_BITS) : sizeof entry.fingerprint;
+    e = hipMemcpyAsync(entry.fingerprint, B, nfp, hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess)
+        e = hipStreamSynchronize(stream);
+    if (e != hipSuccess)
+        return fail(hipGetErrorString(e));
     std::lock_guard<std::mutex> lock(g_prepared_mutex);
-    prepared_table()[B] = PreparedWeight{ N, K, W_BITS };
+    prepared_table()[B] = entry;
     return true;
+}
+
+bool ABQGEMMWrapper::verify_prepared(const int *B, hipStream_t stream)
+{
+    PreparedWeight w;
+    if (!find_prepared(B, &w))
+        return false;
+    uint32_t now[16] = { 0 };
+    const size_t nfp = abq_planes_bytes(w.N, w.K, w.bits) < sizeof now ? abq_planes_bytes(w.N, w.K, w.bits) : sizeof now;
+    if (hipMemcpyAsync(now, B, nfp, hipMemcpyDeviceToHost, stream) != hipSuccess || hipStreamSynchronize(stream) != hipSuccess)
+        return false;
+    return memcmp(now, w.fingerprint, nfp) == 0;
 }
 
 void ABQGEMMWrapper::release_weight(const int *B)
@@ -113,6 +156,11 @@ void ABQGEMMWrapper::gemm(const int M, const int N, const int K, const _Float16 
     }
     PreparedWeight prepared;
     const bool tiled = find_prepared(B, &prepared);
+    if (tiled && verify_on_every_call() && !verify_prepared(B, stream)) {
+        printf("[ABQ][Error] %p is in the table of prepared weights but no longer holds the prepared records "
+               "(freed or refilled without release_weight?)\n", (const void *)B);
+        return;
+    }
     if (tiled && (prepared.N != N || prepared.K != K || prepared.bits != w_bits_)) {
         printf("[ABQ][Error] weight prepared as N, K, bits = %d, %d, %d, called with %d, %d, %d\n", prepared.N, prepared.K,
                prepared.bits, N, K, w_bits_);
@@ -163,6 +211,10 @@ void ABQGEMMWrapper::gemm_scaled(const int M, const int N, const int K, const in
         printf("[ABQ][Error] unsupport K = %d\n", K);
         return;
     }
+    if (is_prepared(B)) { // its words are K-tiled records now: read as planes they would give wrong numbers silently
+        printf("[ABQ][Error] gemm_scaled takes weight planes; %p has been rewritten by prepare_weight\n", (const void *)B);
+        return;
+    }
     abq_gemm_state state;
     abq_status rc = abq_gemm_init(nullptr, x_bits_, w_bits_, signed_ ? 1 : 0, reinterpret_cast<const uint32_t *>(X_packed),
                                   reinterpret_cast<const uint32_t *>(B), M, N, K, D, nullptr, 0, ABQ_OUT_F16_SCALED, &state);
@@ -200,6 +252,11 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     }
     if (!signed_ || (W.group_size != 64 && W.group_size != 128) || (!x_symmetric && !W.zero_term)) {
         printf("[ABQ][Error] unsupport dynamic quantisation setup\n");
+        return;
+    }
+    if (W.planes && is_prepared(W.planes)) {
+        printf("[ABQ][Error] ABQGroupedWeight::planes %p has been rewritten by prepare_weight: hand it over as planes_tiled\n",
+               (const void *)W.planes);
         return;
     }
     if (abq_gemm_ws_bytes < dynamic_workspace_bytes(M, K, W.group_size)) {

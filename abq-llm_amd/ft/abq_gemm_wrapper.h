@@ -58,13 +58,20 @@ public:
     // activations into the same layout and runs the LDS-staged prefill kernel (M > 16) or the decode kernel on
     // prepared operands (M <= 16, and small batches above that where the library estimates it ahead) with no
     // conversion inside the call; a B that was never prepared keeps the plane
-    // kernels.  B must not be handed to gemm_scaled() or to ABQGroupedWeight::planes afterwards.  Returns false
-    // (after "[ABQ][Error] ...") on a bad argument or a failed launch.  release_weight() takes B out of the table
-    // (before its memory is freed or refilled).  The table is guarded by a mutex.
+    // kernels.  gemm_scaled() and ABQGroupedWeight::planes refuse a B that has been prepared (its words are records
+    // now).  Returns false (after "[ABQ][Error] ...") on a bad argument, a failed launch, or a B that is prepared already
+    // (check and entry are one critical section: of two threads preparing one B one is refused).  release_weight()
+    // takes B out of the table and MUST be called before the memory is freed or refilled: the table goes by the
+    // pointer, and a buffer re-allocated at the same address would be read as records.  What the library can do
+    // about that without reading device memory in every call: prepare_weight keeps the first 64 bytes of the
+    // records (one synchronisation per weight matrix at load time), verify_prepared() compares them with what B
+    // holds now (a loader or a test calls it after it has moved weights around), and with ABQ_VERIFY_PREPARED=1 in the
+    // environment every gemm() on a prepared weight does so first (one device read and synchronisation per call).
     static size_t prepared_weight_bytes(int N, int K, int W_BITS);
     static bool prepare_weight(int *B, int N, int K, int W_BITS, int *scratch, hipStream_t stream);
     static void release_weight(const int *B);
     static bool is_prepared(const int *B);
+    static bool verify_prepared(const int *B, hipStream_t stream);
 
     // A: fp16 activations [M][K]; B: packed weight planes [w_bits][N][K/32]; C unused;
     // D: fp16 [M][N]; scale: activation quantisation scale (1 float, device);

@@ -4,6 +4,7 @@
 // (oracle/abq_oracle.h) bit for bit.  `--no-gpu` runs only the host-side error paths.
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -218,8 +219,8 @@ static void gpu_paths()
         HIP_OK(hipFree(d_ws));
     }
 
-    {   // FT wrapper on a prepared weight: gemm() with unchanged arguments, prefill- and decode-sized, bit-equal
-        // to the same call on the plane weight; timed beside it
+    {   // FT wrapper on a prepared weight: gemm() with unchanged arguments, prefill- and decode-sized, against the
+        // CPU oracle (pack_half restated, popcount GEMM, the FT epilogue) bit for bit, and the plane weight beside it
         const int N = 4096, K = 4096, Mmax = 1024;
         std::mt19937 r32(11);
         std::normal_distribution<float> nd(0.f, 2.f);
@@ -246,7 +247,8 @@ static void gpu_paths()
         HIP_OK(hipMemcpy(d_a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
         HIP_OK(hipMemcpy(d_b0, wpl.data(), wbytes, hipMemcpyHostToDevice));
         HIP_OK(hipMemcpy(d_b1, wpl.data(), wbytes, hipMemcpyHostToDevice));
-        const float scales[2] = { 21.0f, 0.0123f };
+        const float in_scale = 21.0f, out_scale = 0.0123f;
+        const float scales[2] = { in_scale, out_scale };
         HIP_OK(hipMemcpy(d_scales, scales, 8, hipMemcpyHostToDevice));
         CHECK(!ABQGEMMWrapper::is_prepared(d_b1));
         CHECK(!ABQGEMMWrapper::prepare_weight(d_b1, N, 100, 2, d_scratch, stream)); // K not a multiple of 128
@@ -254,33 +256,43 @@ static void gpu_paths()
         CHECK(ABQGEMMWrapper::is_prepared(d_b1) && !ABQGEMMWrapper::is_prepared(d_b0));
         CHECK(!ABQGEMMWrapper::prepare_weight(d_b1, N, K, 2, d_scratch, stream)); // twice
         ABQGEMMWrapper wrap(8, 2, true);
-        hipEvent_t e0, e1;
-        HIP_OK(hipEventCreate(&e0));
-        HIP_OK(hipEventCreate(&e1));
+        // expected: all Mmax rows once (the rows of a smaller call are its first rows)
+        std::vector<uint32_t> ap((size_t)8 * Mmax * K / 32);
+        abq_oracle_pack_f16(ha.data(), in_scale, ap.data(), Mmax, K, 8);
+        std::vector<int> acc((size_t)Mmax * N);
+        abq_oracle_gemm_popc(wpl.data(), ap.data(), acc.data(), Mmax, N, K, 2, 8, 1, 0);
+        std::vector<uint16_t> want((size_t)Mmax * N);
+        abq_oracle_epilogue_f16(acc.data(), abq_oracle_f32_to_f16(out_scale), want.data(), (int)acc.size());
         for (int M : { 1024, 300, 16, 8, 4, 2, 1 }) {
-            float us[2] = { 0.f, 0.f };
             for (int prepared = 0; prepared < 2; ++prepared) {
                 _Float16 *d_d = prepared ? d_d1 : d_d0;
-                const int *d_b = prepared ? d_b1 : d_b0;
                 HIP_OK(hipMemsetAsync(d_d, 0xff, (size_t)M * N * 2, stream));
-                const int reps = 200;
-                for (int it = 0; it < reps + 2; ++it) {
-                    if (it == 2)
-                        HIP_OK(hipEventRecord(e0, stream));
-                    wrap.gemm(M, N, K, d_a, d_b, nullptr, d_d, d_scales, nullptr, d_scales + 1, false, d_ws, ws_bytes, stream);
-                }
-                HIP_OK(hipEventRecord(e1, stream));
+                wrap.gemm(M, N, K, d_a, prepared ? d_b1 : d_b0, nullptr, d_d, d_scales, nullptr, d_scales + 1, false, d_ws, ws_bytes, stream);
                 HIP_OK(hipStreamSynchronize(stream));
-                float ms = 0.f;
-                HIP_OK(hipEventElapsedTime(&ms, e0, e1));
-                us[prepared] = ms * 1000.f / reps;
+                std::vector<uint16_t> got((size_t)M * N);
+                HIP_OK(hipMemcpy(got.data(), d_d, got.size() * 2, hipMemcpyDeviceToHost));
+                CHECK(std::equal(got.begin(), got.end(), want.begin()));
             }
-            std::vector<uint16_t> got0((size_t)M * N), got1((size_t)M * N);
-            HIP_OK(hipMemcpy(got0.data(), d_d0, got0.size() * 2, hipMemcpyDeviceToHost));
-            HIP_OK(hipMemcpy(got1.data(), d_d1, got1.size() * 2, hipMemcpyDeviceToHost));
-            CHECK(got0 == got1);
-            printf("  gemm() W2A8 M = %4d, N = K = 4096 (pack + GEMM per call): plane weight %.1f us, prepared weight %.1f us\n", M,
-                   us[0], us[1]);
+        }
+        // the records are where prepare_weight left them; refilled behind the table's back they are not
+        CHECK(ABQGEMMWrapper::verify_prepared(d_b1, stream));
+        {
+            std::vector<uint32_t> keep(16), junk(16, 0x12345678u);
+            HIP_OK(hipMemcpy(keep.data(), d_b1, 64, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(d_b1, junk.data(), 64, hipMemcpyHostToDevice));
+            CHECK(!ABQGEMMWrapper::verify_prepared(d_b1, stream));
+            HIP_OK(hipMemcpy(d_b1, keep.data(), 64, hipMemcpyHostToDevice));
+            CHECK(ABQGEMMWrapper::verify_prepared(d_b1, stream));
+            CHECK(!ABQGEMMWrapper::verify_prepared(d_b0, stream)); // never prepared
+        }
+        // gemm_scaled reads planes: a prepared weight is refused (D stays as it was)
+        HIP_OK(hipMemset(d_d1, 0xff, 64));
+        wrap.gemm_scaled(1, N, K, reinterpret_cast<const int *>(d_ws), d_b1, d_d1, d_scales, d_scales, stream);
+        HIP_OK(hipStreamSynchronize(stream));
+        {
+            uint16_t first = 0;
+            HIP_OK(hipMemcpy(&first, d_d1, 2, hipMemcpyDeviceToHost));
+            CHECK(first == 0xffff);
         }
         // a prepared weight is checked against the shape it was prepared for: D stays as it was
         HIP_OK(hipMemset(d_d1, 0xff, 64));
@@ -291,8 +303,6 @@ static void gpu_paths()
         CHECK(first == 0xffff);
         ABQGEMMWrapper::release_weight(d_b1);
         CHECK(!ABQGEMMWrapper::is_prepared(d_b1));
-        HIP_OK(hipEventDestroy(e0));
-        HIP_OK(hipEventDestroy(e1));
         HIP_OK(hipFree(d_a));
         HIP_OK(hipFree(d_d0));
         HIP_OK(hipFree(d_d1));

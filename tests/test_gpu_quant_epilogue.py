@@ -649,7 +649,7 @@ def test_group_scales_on_the_fp6_route(abq, oracle, q, p, signed):
 LAYER_LINEARS = [("qkv", 12288, 4096), ("o", 4096, 4096), ("gate_up", 2 * 11008, 4096), ("down", 4096, 11008)]
 
 
-def _layer_linear(abq, oracle, name, N, K, tokens, x_symmetric, seed, sample_rows, bit_balance=False):
+def _layer_linear(abq, oracle, name, N, K, tokens, x_symmetric, seed, sample_rows, bit_balance=False, full_check=False):
     """One W2A8 linear: fp16 weights N(0, 0.02) quantised to 2 bits per (channel, group of 128),
     fp16 activations quantised per token on the device; checks `sample_rows` output rows.
     bit_balance: the reference's default 2-bit weight quantiser (five levels, quantizer.py:66-68,169-171),
@@ -690,6 +690,29 @@ def _layer_linear(abq, oracle, name, N, K, tokens, x_symmetric, seed, sample_row
     assert_close_rel(got[rows], want)
     if got2 is not None:
         assert_close_rel(got2[rows], want)
+    if full_check:
+        # every row, on the GPU in fp64: the codes the kernel itself packed (read back from its planes, which hold the
+        # same codes as the K-tiled records: the sampled rows above pin them to the restated quantiser), dequantised,
+        # times the dequantised weights; every product and partial sum is far inside fp64's exact range
+        xp_d, xs_p, xz_p, _ = abq.quant_pack_f16(x, 8, symmetric=x_symmetric, tiled=False, group_size=128)
+        assert torch.equal(xs_p, xs)
+        shifts = torch.arange(31, -1, -1, device="cuda", dtype=torch.int32)
+        codes_d = torch.zeros((tokens, K), dtype=torch.int32, device="cuda")
+        for b in range(8):
+            bits = ((xp_d[b].unsqueeze(-1) >> shifts) & 1).reshape(tokens, K)
+            codes_d += bits * (-(1 << b) if b == 7 else (1 << b))  # two's complement: the top plane is negative
+        zero_d = xz_p.double().unsqueeze(1) if xz_p is not None else 0.0
+        x_dq = (codes_d.double() - zero_d) * xs.double().unsqueeze(1)
+        w_dq = ((torch.from_numpy(w_codes).cuda().double().reshape(N, K // 128, 128) - wz_d.double().unsqueeze(2)) *
+                ws_d.double().unsqueeze(2)).reshape(N, K)
+        want_d = x_dq @ w_dq.T
+        got_d = torch.from_numpy(got).cuda().double()
+        rms = torch.sqrt(torch.mean(want_d ** 2))
+        err = torch.abs(got_d - want_d)
+        assert bool(torch.all(torch.isfinite(got_d)))
+        assert bool(torch.all(err <= REL_TOL * torch.abs(want_d) + 1e-3 * rms)), float((err / (torch.abs(want_d) + 1e-1 * rms)).max())
+        assert float(torch.linalg.norm(got_d - want_d)) <= 2e-3 * float(torch.linalg.norm(want_d))
+        del x_dq, w_dq, want_d, got_d, err, codes_d
     # and the quantised result tracks the unquantised fp16 linear as 2-bit weights allow: the
     # dequantised weights are within scale/2 of the originals, so this is only a sanity bound
     full = x_rows.astype(np.float64) @ w.astype(np.float64).T
@@ -712,4 +735,4 @@ def test_config4_linear_with_bit_balanced_2bit_weights(abq, oracle, tokens, x_sy
 
 @pytest.mark.parametrize("name,N,K", LAYER_LINEARS)
 def test_config4_decoder_layer_linears_batch16(abq, oracle, name, N, K):
-    _layer_linear(abq, oracle, name, N, K, 16 * 1024, True, seed=7 + len(name), sample_rows=32)
+    _layer_linear(abq, oracle, name, N, K, 16 * 1024, True, seed=7 + len(name), sample_rows=32, full_check=True)
