@@ -39,6 +39,7 @@ EXPORTED = [
     "abq_row_sums", "abq_gemm_set_row_sums", "abq_gemm_row_sums_ready",
     "abq_tuning_load", "abq_tuning_add", "abq_tuning_clear", "abq_tuning_enable_builtin", "abq_tuning_lookup",
     "abq_preferred_weight_layout", "abq_padded_bits", "abq_relayout_planes_padded", "abq_gemm_set_value_bits",
+    "abq_relayout_planes_biased", "abq_gemm_set_biased_records",
 ]
 
 
@@ -144,6 +145,8 @@ def lib():
         L.abq_tuning_lookup.argtypes = [ci, ci, ci, ci, ci, ci, ci, ci, ctypes.POINTER(TileConfig), ctypes.POINTER(ctypes.c_float)]
         L.abq_preferred_weight_layout.argtypes = [ci] * 7
         L.abq_preferred_weight_layout.restype = ci
+        L.abq_relayout_planes_biased.argtypes = [vp, vp, ci, ci, vp]
+        L.abq_gemm_set_biased_records.argtypes = [ctypes.POINTER(GemmState), ci, ci]
         L.abq_padded_bits.argtypes = [ci]
         L.abq_padded_bits.restype = ci
         L.abq_relayout_planes_padded.argtypes = [vp, vp, ci, ci, ci, ci, vp]
@@ -257,6 +260,17 @@ def row_sums(planes, stream=None):
     return out
 
 
+def relayout_planes_biased(planes, stream=None):
+    """planes int32 tensor [8, rows, k/32] of unsigned codes -> K-tiled records [k/128, rows, 8, 4] holding code - 128."""
+    import torch
+    bits, rows, kw = planes.shape
+    assert bits == 8 and planes.is_cuda and planes.is_contiguous() and kw % 4 == 0
+    out = torch.empty((kw // 4, rows, 8, 4), dtype=torch.int32, device=planes.device)
+    _check(lib().abq_relayout_planes_biased(planes.data_ptr(), out.data_ptr(), rows, kw * 32, _stream_ptr(stream)),
+           "abq_relayout_planes_biased")
+    return out
+
+
 def padded_bits(bits):
     return lib().abq_padded_bits(bits)
 
@@ -338,7 +352,7 @@ class Gemm:
     def __init__(self, x_planes, w_planes, signed, out=None, cfg=None, out_kind=OUT_I32, c_scale=None,
                  x_scale=None, w_scale=None, group_size=0, x_tiled=False, w_tiled=False, workspace=None,
                  x_zero=None, w_zero=None, x_group_sums=None, w_zero_term=None, act=ACT_NONE,
-                 x_fp6=0, w_fp6=0, x_row_sums=None, w_row_sums=None, value_bits=None):
+                 x_fp6=0, w_fp6=0, x_row_sums=None, w_row_sums=None, value_bits=None, biased=None):
         import torch
         if x_fp6:
             kt, M, _ = x_planes.shape
@@ -387,6 +401,9 @@ class Gemm:
         if value_bits is not None:  # (x, w): the codes' real widths inside padded records
             _check(lib().abq_gemm_set_value_bits(ctypes.byref(self.state), int(value_bits[0]), int(value_bits[1])),
                    "abq_gemm_set_value_bits")
+        if biased is not None:  # (x, w): which K-tiled operands of an unsigned W8A8 pair hold code - 128
+            _check(lib().abq_gemm_set_biased_records(ctypes.byref(self.state), int(bool(biased[0])), int(bool(biased[1]))),
+                   "abq_gemm_set_biased_records")
         self.row_sums = (x_row_sums, w_row_sums)
         if x_row_sums is not None or w_row_sums is not None:
             _check(lib().abq_gemm_set_row_sums(ctypes.byref(self.state), x_row_sums.data_ptr() if x_row_sums is not None else None,

@@ -977,6 +977,10 @@ static bool decode_tiled_pays(int x_bits, int w_bits, int M, int N, int K)
 // pair.  Variant by shape (measured on MI355X, W2A8, LLaMA-7B widths): sixteen waves with one weight load each
 // in flight while a compute unit holds at most two workgroups; with more tiles than that, eight waves with two
 // loads each (twice the workgroups fit a compute unit).
+// reserved[4]: bit 0 / bit 1: the K-tiled 8-bit records of X / W hold code - 128 (abq_gemm_set_biased_records)
+static bool biased_x(const abq_gemm_state *st) { return (st->reserved[4] & 1) != 0; }
+static bool biased_w(const abq_gemm_state *st) { return (st->reserved[4] & 2) != 0; }
+
 // Unsigned 8-bit records on the decode kernel of prepared operands: codes up to 255 are fed as value - 128 and need
 // the other operand's row sums (abq_gemm_set_row_sums); records declared to hold narrower codes
 // (abq_gemm_set_value_bits: padded records) are fed as they are.  flip_x / flip_w: which operands are flipped.
@@ -993,6 +997,8 @@ static bool decode_tiled_flips_ok(const abq_gemm_state *st)
 {
     int fx, fw;
     decode_tiled_flips(st, &fx, &fw);
+    if (biased_x(st) || biased_w(st))
+        return false; // biased records are read by the prefill kernel only
     if (fx && !st->w_row_sums)
         return false;
     if (fw && !st->x_row_sums)
@@ -1475,6 +1481,29 @@ abq_status abq_gemm_set_value_bits(abq_gemm_state *st, int x_value_bits, int w_v
     return ABQ_OK;
 }
 
+abq_status abq_gemm_set_biased_records(abq_gemm_state *st, int x_biased, int w_biased)
+{
+    if (!st || !st->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    if ((x_biased || w_biased) && (st->cfg.is_signed || st->cfg.x_bits != 8 || st->cfg.w_bits != 8 || st->group_size))
+        return ABQ_ERR_UNSUPPORTED;
+    if (x_biased && !w_biased)
+        return ABQ_ERR_INVALID_ARG;
+    st->reserved[4] = (x_biased ? 1 : 0) | (w_biased ? 2 : 0);
+    if (w_biased && st->strategy == ABQ_STRATEGY_DECODE_TILED && st->auto_chosen)
+        return switch_to_tiled(st); // biased records are read by the prefill kernel only
+    return ABQ_OK;
+}
+
+abq_status abq_relayout_planes_biased(const uint32_t *planes, uint32_t *tiled, int rows, int k, void *stream)
+{
+    if (!planes || !tiled || rows <= 0)
+        return ABQ_ERR_INVALID_ARG;
+    if (k < 128 || k % 128 != 0)
+        return ABQ_ERR_BAD_K;
+    return hip_status(launch_relayout_planes_padded(planes, tiled, rows, k, 8, 8, 2, (hipStream_t)stream));
+}
+
 int abq_padded_bits(int bits) { return bits < 1 || bits > 8 ? 0 : bits <= 2 ? 2 : bits <= 4 ? 4 : 8; }
 
 abq_status abq_relayout_planes_padded(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits, int is_signed,
@@ -1516,8 +1545,8 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     a.w_zero_term = st->w_zero_term;
     a.x_pack_scale = st->x_pack_scale;
     a.x_dynamic = st->x_layout == ABQ_LAYOUT_F16 ? st->reserved[1] : 0;
-    a.x_row_sums = st->x_row_sums;
-    a.w_row_sums = st->w_row_sums;
+    a.x_row_sums = nullptr; // (handed to a kernel only by the branches below that need them)
+    a.w_row_sums = nullptr;
     decode_tiled_flips(st, &a.flip_x, &a.flip_w);
     const Registry &reg = registry();
     const abq_tile_config &c = st->cfg;
@@ -1566,8 +1595,17 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
         if (xb + wb > st->workspace_bytes || ((xb + wb) && !st->workspace))
             return ABQ_ERR_INVALID_ARG;
         char *ws = static_cast<char *>(st->workspace);
+        // Unsigned W8A8 whose weights were prepared with the 128 already taken off (abq_relayout_planes_biased): the
+        // activations are brought to the same form (converted that way here when they arrive as planes), and the
+        // signed kernel of the same tile runs on them, handed both operands' row sums for the correction.
+        const bool biased = st->strategy == ABQ_STRATEGY_TILED && biased_w(st);
+        if (biased && (c.is_signed || c.x_bits != 8 || c.w_bits != 8 || st->group_size || wb || (!xb && !biased_x(st)) || (xb && biased_x(st))))
+            return ABQ_ERR_INVALID_ARG;
+        if (!biased && biased_x(st))
+            return ABQ_ERR_INVALID_ARG; // biased activations only make sense against biased weights
         if (xb) {
-            e = launch_relayout_planes(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, c.x_bits, (hipStream_t)stream);
+            e = launch_relayout_planes_padded(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, c.x_bits, c.x_bits, biased ? 2 : 0,
+                                              (hipStream_t)stream);
             if (e != hipSuccess)
                 return hip_status(e);
             a.X = reinterpret_cast<const uint32_t *>(ws);
@@ -1589,12 +1627,38 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
         if (!t || st->variant < 0 || st->variant >= t->count)
             return ABQ_ERR_NOT_INITIALIZED;
         int variant = st->variant;
+        if (biased) {
+            const RowSumPlan plan = row_sum_plan(st, xb + wb);
+            if (!plan.ok)
+                return ABQ_ERR_INVALID_ARG; // both operands' sums are needed; the weights' must be set
+            if (!st->x_row_sums) {
+                e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, c.x_bits, (hipStream_t)stream);
+                if (e != hipSuccess)
+                    return hip_status(e);
+            }
+            a.x_row_sums = st->x_row_sums ? st->x_row_sums : reinterpret_cast<const int *>(ws + plan.x_off);
+            a.w_row_sums = st->w_row_sums;
+            // the signed pair's staged entry of the same tile
+            const KernelTable *ts = find_table(reg.tiled, 8, 8, 1);
+            const KernelEntry &want = t->entries[st->variant];
+            const KernelEntry *run = nullptr;
+            for (int i = 0; ts && i < ts->count; ++i) {
+                const KernelEntry &o = ts->entries[i];
+                if (o.lds != 0 && o.tm == want.tm && o.tn == want.tn && o.wm == want.wm && o.wn == want.wn && o.wk == want.wk && o.kb == want.kb)
+                    run = &o;
+            }
+            if (!run)
+                return ABQ_ERR_UNSUPPORTED; // a tile the staged kernel is not built for
+            return hip_status(run->launch(a, (hipStream_t)stream));
+        }
         if (st->strategy == ABQ_STRATEGY_DECODE_TILED && (a.flip_x || a.flip_w) && !c.is_signed) {
             // unsigned 8-bit codes on the decode kernel: the sums the caller set, or those of an operand that arrived
             // as planes, taken into the workspace behind its converted copy; there is no kernel to fall back to
             const RowSumPlan plan = row_sum_plan(st, xb + wb);
-            if (!plan.ok || (c.x_bits == 8 && c.w_bits == 8 && a.flip_x != a.flip_w))
+            if (!plan.ok || (c.x_bits == 8 && c.w_bits == 8 && a.flip_x != a.flip_w) || biased_x(st) || biased_w(st))
                 return ABQ_ERR_INVALID_ARG;
+            a.x_row_sums = st->x_row_sums;
+            a.w_row_sums = st->w_row_sums;
             if (a.flip_w && !st->x_row_sums) {
                 e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, c.x_bits, (hipStream_t)stream);
                 if (e != hipSuccess)

@@ -507,24 +507,31 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
 
     // Unsigned 8-bit operands were fed as value - 128: sum (x - 128) w = sum x w - 128 sum w, and likewise for the
     // weights; with both, 2^14 K comes on top.  The correction of a column (row) is the same for all its elements.
-    if constexpr (FLIP_X || FLIP_W) {
-        int col_fix[TN];
+    // The signed W8A8 instances do the same when the host hands them row sums: then their records are those of an
+    // unsigned pair written with the 128 already taken off (abq_relayout_planes_biased), and nothing was flipped here.
+    constexpr bool MAY_BE_BIASED = !FP6 && SIGNED && QB == 8 && PB == 8 && !GROUPED;
+    if constexpr (FLIP_X || FLIP_W || MAY_BE_BIASED) {
+        const bool fix_x = FLIP_X || (MAY_BE_BIASED && a.w_row_sums != nullptr); // X was fed as value - 128
+        const bool fix_w = FLIP_W || (MAY_BE_BIASED && a.x_row_sums != nullptr);
+        if (fix_x || fix_w) {
+            int col_fix[TN];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            unsigned v = FLIP_X ? 128u * (unsigned)a.w_row_sums[min(n0 + wn * 32 * TN + j * 32 + r, N - 1)] : 0u;
-            if (FLIP_X && FLIP_W)
-                v -= 16384u * (unsigned)(ktot * 128);
-            col_fix[j] = (int)v;
-        }
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int row_fix = FLIP_W ? (int)(128u * (unsigned)a.x_row_sums[min(m0 + wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4), M - 1)]) : 0;
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j][e] = (int)((unsigned)acc[i][j][e] + (unsigned)row_fix + (unsigned)col_fix[j]);
+            for (int j = 0; j < TN; ++j) {
+                unsigned v = fix_x ? 128u * (unsigned)a.w_row_sums[min(n0 + wn * 32 * TN + j * 32 + r, N - 1)] : 0u;
+                if (fix_x && fix_w)
+                    v -= 16384u * (unsigned)(ktot * 128);
+                col_fix[j] = (int)v;
             }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int row_fix = fix_w ? (int)(128u * (unsigned)a.x_row_sums[min(m0 + wm * 32 * TM + i * 32 + 8 * (e / 4) + 4 * g + (e % 4), M - 1)]) : 0;
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j][e] = (int)((unsigned)acc[i][j][e] + (unsigned)row_fix + (unsigned)col_fix[j]);
+                }
+        }
     }
     auto result = [&](int i, int j, int e) -> int {
         if constexpr (FP6)

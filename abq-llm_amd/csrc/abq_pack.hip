@@ -132,8 +132,9 @@ __device__ __forceinline__ void store_fields(uint32_t *rec, int ws, const uint32
 // four word-sets in registers, and parks the record in LDS; the records of one K tile are then
 // contiguous in memory over the 32 rows and leave with coalesced 16-byte stores.
 // in_bits < BITS: the operand has in_bits planes and is written as records of the wider field (padded records, for
-// the widths made of several fields): the planes above it repeat its top plane (signed codes: sign extension) or
-// are zero.
+// the widths made of several fields): the planes above it repeat its top plane (sign_extend & 1: signed codes) or
+// are zero.  sign_extend & 2 (8-bit records): bit 7 of every code is flipped, i.e. the record holds code - 128
+// (biased records of unsigned 8-bit operands, which the signed matrix cores take as they are).
 template <int BITS>
 __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__restrict__ planes,
                                                               uint32_t *__restrict__ tiled, int rows, int KW, int in_bits,
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__
 #pragma unroll
             for (int b = 0; b < BITS; ++b) {
                 uint4 v = *reinterpret_cast<const uint4 *>(p + min(b, in_bits - 1) * plane_stride);
-                if (b >= in_bits && !sign_extend)
+                if (b >= in_bits && !(sign_extend & 1))
                     v = make_uint4(0u, 0u, 0u, 0u);
                 pw[0][b] = v.x; pw[1][b] = v.y; pw[2][b] = v.z; pw[3][b] = v.w;
             }
@@ -164,6 +165,11 @@ __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__
             for (int ws = 0; ws < 4; ++ws) {
                 uint32_t e[8], f[BITS];
                 planes_to_int8<BITS, kLow>(pw[ws], e);
+                if (BITS == 8 && (sign_extend & 2)) {
+#pragma unroll
+                    for (int d = 0; d < 8; ++d)
+                        e[d] ^= 0x80808080u;
+                }
                 compress_fields<BITS>(e, f);
                 store_fields<BITS>(rec, ws, f);
             }
@@ -206,8 +212,13 @@ __global__ __launch_bounds__(256) void relayout_planes_ws_kernel(const uint32_t 
             const uint32_t *p = planes + (size_t)row * KW + kw;
 #pragma unroll
             for (int b = 0; b < BITS; ++b)
-                pw[b] = (b >= in_bits && !sign_extend) ? 0u : p[min(b, in_bits - 1) * plane_stride];
+                pw[b] = (b >= in_bits && !(sign_extend & 1)) ? 0u : p[min(b, in_bits - 1) * plane_stride];
             planes_to_int8<BITS, kLow>(pw, e);
+            if (BITS == 8 && (sign_extend & 2)) {
+#pragma unroll
+                for (int d = 0; d < 8; ++d)
+                    e[d] ^= 0x80808080u;
+            }
             compress_fields<BITS>(e, f);
             store_fields<BITS>(buf + (w >> 2) * SLAB + i * REC, w & 3, f);
         }

@@ -406,10 +406,16 @@ def main():
                 # are taken inside the timed call when they arrive as planes, and come with them when they arrive tiled)
                 u8 = not signed and 8 in (q, p)
                 wrs = abq.row_sums(wpl) if u8 else None
+                # unsigned W8A8: the weights as biased records (code - 128 written at preparation), which the signed
+                # pair's kernel runs without flipping anything after its LDS reads
+                biased = u8 and (q, p) == (8, 8)
+                if biased:
+                    wtl = abq.relayout_planes_biased(wpl)
                 for M in (512, 2048):
                     xpl = random_planes(torch, (q, M, K // 32))
                     ws = torch.empty(xpl.numel() * 4 + 4 * M + 512, dtype=torch.uint8, device="cuda")
-                    gm = abq.Gemm(xpl, wtl, signed, w_tiled=True, workspace=ws, w_row_sums=wrs)  # activations converted per call
+                    gm = abq.Gemm(xpl, wtl, signed, w_tiled=True, workspace=ws, w_row_sums=wrs,
+                                  biased=(False, True) if biased else None)  # activations converted per call
                     gm.run()
                     torch.cuda.synchronize()
                     reps = 20  # (a replay's own launch cost is spread over the steps of the graph)
@@ -428,9 +434,9 @@ def main():
                     tops = 2.0 * M * N * K / (us * 1e-6) / 1e12
                     # the same GEMM with the activations already in the K-tiled layout, which is how the fused
                     # quantise + pack kernel hands them over: no conversion launch in the timed call
-                    xtl = abq.relayout_planes(xpl)
+                    xtl = abq.relayout_planes_biased(xpl) if biased else abq.relayout_planes(xpl)
                     gt = abq.Gemm(xtl, wtl, signed, x_tiled=True, w_tiled=True, w_row_sums=wrs,
-                                  x_row_sums=abq.row_sums(xpl) if u8 else None)
+                                  x_row_sums=abq.row_sums(xpl) if u8 else None, biased=(True, True) if biased else None)
                     gt.run()
                     torch.cuda.synchronize()
                     gr = torch.cuda.CUDAGraph()

@@ -180,7 +180,8 @@ typedef struct abq_gemm_state {
     const float *w_scale;  /* [N] or [N][K/group_size] */
     int group_size;        /* 0 = per channel          */
     int reserved[5];       /* [0] popcount kernels: log2 of the lanes per weight row; [1] see
-                              abq_gemm_set_dynamic_f16_activations; [2], [3] see abq_gemm_set_value_bits */
+                              abq_gemm_set_dynamic_f16_activations; [2], [3] see abq_gemm_set_value_bits; [4] see
+                              abq_gemm_set_biased_records */
     /* K-tiled operands (ABQ_STRATEGY_TILED) */
     int x_layout, w_layout;  /* abq_layout of X and W as handed to init                    */
     int auto_chosen;         /* 1 if the tile was the library's choice                     */
@@ -406,6 +407,18 @@ abq_status abq_gemm_set_row_sums(abq_gemm_state *state, const int32_t *x_row_sum
 /* 1 if abq_gemm_exec on this state, as it stands, runs the kernel that takes the row sums handed in (every needed
  * sum set, or to be had from plane operands into the workspace the state holds), 0 otherwise. */
 int abq_gemm_row_sums_ready(const abq_gemm_state *state);
+
+/* Biased records of unsigned W8A8.  abq_relayout_planes_biased writes the K-tiled records of an unsigned 8-bit
+ * operand with 128 taken off every code (bit 7 flipped): the byte is then the int8 the signed matrix cores want, and
+ * the staged kernel spends nothing on flipping it after every LDS read (W8A8 uint then runs the signed pair's
+ * kernel).  abq_gemm_set_biased_records(state, x_biased, w_biased) declares which K-tiled operands of an unsigned
+ * W8A8 state are such records: the weights (prepared once, with their row sums set through abq_gemm_set_row_sums),
+ * and the activations if the caller prepared them the same way; activations that arrive as planes are converted
+ * that way by abq_gemm_exec itself, and their row sums taken, in the workspace.  Only the prefill kernel
+ * (ABQ_STRATEGY_TILED) on the tiles the staged kernel is built for reads them; x_biased without w_biased is refused.
+ * ABQ_ERR_UNSUPPORTED for any other pair.  No counterpart in the reference. */
+abq_status abq_relayout_planes_biased(const uint32_t *planes, uint32_t *tiled, int rows, int k, void *stream);
+abq_status abq_gemm_set_biased_records(abq_gemm_state *state, int x_biased, int w_biased);
 
 /* Padded records for the widths made of several fields.  The decode kernel on prepared operands reads records of one
  * field per element (2, 4 or 8 bits).  An operand of 3, 5, 6 or 7 bits is brought to it as records of the next such

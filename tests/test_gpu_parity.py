@@ -215,6 +215,25 @@ def test_tiled_kernels_with_prepared_operands(abq, oracle):
                 g = abq.Gemm(xd, wt, signed, cfg=cfg, w_tiled=True, workspace=ws2, w_row_sums=abq.row_sums(wd))
                 assert g.row_sums_ready == staged_tile and g.workspace_bytes <= ws2.numel()
                 assert np.array_equal(g.run().cpu().numpy(), want), abq.format_kernel_name(cfg)
+                if (q, p) == (8, 8):
+                    # biased records (code - 128 written at preparation): the signed pair's staged kernel runs them, the
+                    # activations arriving biased too or as planes (converted that way into the workspace); a tile that
+                    # kernel is not built for is refused
+                    xb_, wb_ = abq.relayout_planes_biased(xd), abq.relayout_planes_biased(wd)
+                    assert torch.equal(wb_, abq.relayout_planes(wd) ^ torch.tensor(-2139062144, dtype=torch.int32, device="cuda"))
+                    g1 = abq.Gemm(xb_, wb_, signed, cfg=cfg, x_tiled=True, w_tiled=True, x_row_sums=abq.row_sums(xd),
+                                  w_row_sums=abq.row_sums(wd), biased=(True, True))
+                    g2 = abq.Gemm(xd, wb_, signed, cfg=cfg, w_tiled=True, workspace=ws2, w_row_sums=abq.row_sums(wd), biased=(False, True))
+                    for gb in (g1, g2):
+                        if staged_tile:
+                            gb.out.fill_(-7)
+                            assert np.array_equal(gb.run().cpu().numpy(), want), abq.format_kernel_name(cfg)
+                        else:
+                            with pytest.raises(abq.AbqError):
+                                gb.run()
+                    with pytest.raises(abq.AbqError):  # plain activations against biased weights
+                        abq.Gemm(xt, wb_, signed, cfg=cfg, x_tiled=True, w_tiled=True, x_row_sums=abq.row_sums(xd),
+                                 w_row_sums=abq.row_sums(wd), biased=(False, True)).run()
         # a state with an explicit non-tiled tile refuses tiled operands; exec without workspace is refused
         cfg = [c for c in abq.native_configs(q, p, signed) if c.nstage == 2][0]
         with pytest.raises(abq.AbqError):
@@ -719,6 +738,11 @@ def test_config2_prefill_full_size(abq, oracle, q, p, signed):
             g = abq.Gemm(xd, wt, signed, w_tiled=True, workspace=ws, w_row_sums=None if signed else abq.row_sums(wd))
             assert g.strategy == "tiled" and g.row_sums_ready == ((q, p, signed) == (8, 8, False))
             got_d = g.run()
+            if (q, p, signed) == (8, 8, False):  # the same on weights prepared as biased records (code - 128)
+                gb = abq.Gemm(xd, abq.relayout_planes_biased(wd), signed, w_tiled=True, workspace=ws, w_row_sums=abq.row_sums(wd),
+                              biased=(False, True))
+                assert gb.strategy == "tiled" and gb.config_name == g.config_name
+                assert torch.equal(gb.run(), got_d)
             ref = torch.from_numpy(x).cuda().double() @ wf.T
             assert torch.equal(got_d.double(), ref), (q, p, signed, M, N, K)
             _sampled_oracle_check(oracle, xp, wp, signed, got_d.cpu().numpy(), rng, rows=2)
