@@ -39,7 +39,7 @@ EXPORTED = [
     "abq_row_sums", "abq_gemm_set_row_sums", "abq_gemm_row_sums_ready",
     "abq_tuning_load", "abq_tuning_add", "abq_tuning_clear", "abq_tuning_enable_builtin", "abq_tuning_lookup",
     "abq_preferred_weight_layout", "abq_padded_bits", "abq_relayout_planes_padded", "abq_gemm_set_value_bits",
-    "abq_relayout_planes_biased", "abq_gemm_set_biased_records",
+    "abq_relayout_planes_biased", "abq_gemm_set_biased_records", "abq_pack_f16_fp6",
 ]
 
 
@@ -108,6 +108,7 @@ def lib():
         L.abq_pack_u4.argtypes = [vp, vp, ci, ci, ci, vp]
         L.abq_pack_f16.argtypes = [vp, vp, vp, ci, ci, ci, vp]
         L.abq_pack_f16_tiled.argtypes = [vp, vp, vp, ci, ci, ci, vp]
+        L.abq_pack_f16_fp6.argtypes = [vp, vp, vp, ci, ci, ci, ci, vp]
         L.abq_parse_kernel_name.argtypes = [ctypes.c_char_p, ctypes.POINTER(TileConfig), ctypes.POINTER(ci)]
         L.abq_format_kernel_name.argtypes = [ctypes.POINTER(TileConfig), ci, ctypes.c_char_p, ctypes.c_size_t]
         L.abq_native_config_count.argtypes = [ci, ci, ci]
@@ -234,6 +235,17 @@ def pack_f16(values, scale, bits, out=None, stream=None, tiled=False):
                else planes_empty(bits, rows, k, values.device))
     fn, name = (lib().abq_pack_f16_tiled, "abq_pack_f16_tiled") if tiled else (lib().abq_pack_f16, "abq_pack_f16")
     _check(fn(values.data_ptr(), scale.data_ptr(), out.data_ptr(), rows, k, bits, _stream_ptr(stream)), name)
+    return out
+
+
+def pack_f16_fp6(values, scale, bits, signed, stream=None):
+    """The same values as pack_f16 written as FP6 records [k/128, rows, 24] (bits <= 5 signed, <= 4 unsigned)."""
+    import torch
+    assert values.dtype == torch.float16 and values.is_cuda and values.is_contiguous()
+    rows, k = values.shape
+    out = torch.empty((k // 128, rows, 24), dtype=torch.int32, device=values.device)
+    _check(lib().abq_pack_f16_fp6(values.data_ptr(), scale.data_ptr(), out.data_ptr(), rows, k, bits, int(bool(signed)),
+                                  _stream_ptr(stream)), "abq_pack_f16_fp6")
     return out
 
 

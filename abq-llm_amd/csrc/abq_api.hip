@@ -17,6 +17,7 @@ namespace abq {
 hipError_t launch_pack_i32(const int32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_pack_f16(const void *, const float *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_pack_f16_tiled(const void *, const float *, uint32_t *, int, int, int, hipStream_t);
+hipError_t launch_pack_f16_fp6(const void *, const float *, uint32_t *, int, int, int, int, hipStream_t);
 hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes_padded(const uint32_t *, uint32_t *, int, int, int, int, int, hipStream_t);
@@ -527,6 +528,21 @@ abq_status abq_pack_f16_tiled(const void *in_f16, const float *scale_dev, uint32
     if (!scale_dev || bits > 8)
         return ABQ_ERR_INVALID_ARG;
     return hip_status(launch_pack_f16_tiled(in_f16, scale_dev, tiled, rows, k, bits, (hipStream_t)stream));
+}
+
+abq_status abq_pack_f16_fp6(const void *in_f16, const float *scale_dev, uint32_t *records, int rows, int k, int bits,
+                            int is_signed, void *stream)
+{
+    abq_status s = check_pack(in_f16, records, rows, k, bits);
+    if (s != ABQ_OK)
+        return s;
+    if (!scale_dev)
+        return ABQ_ERR_INVALID_ARG;
+    if (bits > (is_signed ? 5 : 4))
+        return ABQ_ERR_UNSUPPORTED;
+    if (k % 128 != 0)
+        return ABQ_ERR_BAD_K;
+    return hip_status(launch_pack_f16_fp6(in_f16, scale_dev, records, rows, k, bits, is_signed ? 1 : 0, (hipStream_t)stream));
 }
 
 // ---- names -------------------------------------------------------------------------------

@@ -475,11 +475,45 @@ __device__ __forceinline__ void emit_tiled(const int (&v)[8], uint32_t *tiled, i
         store_fields_any(tiled + ((size_t)(w >> 2) * rows + row) * (bits * 4), w & 3, e, bits);
 }
 
+// Eight codes of magnitude at most 16 (this lane's unit: elements 8 u .. 8 u + 7 of `row`, u = 4 w + quad_lane) ->
+// their share of the row's FP6 record; the four lanes of a quad assemble one word-set of 192 bits.
+__device__ __forceinline__ void emit_fp6(const int (&v)[8], uint32_t *records, int rows, int row, int w, int quad_lane, bool active)
+{
+    // position p = 4 s + c of the word-set's 192-bit string holds element 31 - (8c + s): this lane's
+    // element j goes to position 4 (7 - j) + 3 - quad_lane as the code (sign << 5) | magnitude
+    uint32_t o[6] = { 0u, 0u, 0u, 0u, 0u, 0u };
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t code = v[j] < 0 ? (32u | (uint32_t)(-v[j])) : (uint32_t)v[j];
+        constexpr int kBase[8] = { 168, 144, 120, 96, 72, 48, 24, 0 }; // 24 (7 - j)
+        const int d0 = kBase[j] >> 5;                                   // first dword the code can touch
+        const uint64_t wide = (uint64_t)code << ((kBase[j] & 31) + 6 * (3 - quad_lane));
+        o[d0] |= (uint32_t)wide;
+        if (d0 + 1 < 6)
+            o[d0 + 1] |= (uint32_t)(wide >> 32);
+    }
+#pragma unroll
+    for (int d = 0; d < 6; ++d)
+        o[d] = quad_or(o[d]);
+    if (active && quad_lane == 0) {
+        const int ws = w & 3;
+        uint32_t *rec = records + ((size_t)(w >> 2) * rows + row) * 24 + 12 * (ws & 1) + 6 * (ws >> 1);
+        *reinterpret_cast<uint2 *>(rec) = make_uint2(o[0], o[1]);
+        *reinterpret_cast<uint2 *>(rec + 2) = make_uint2(o[2], o[3]);
+        *reinterpret_cast<uint2 *>(rec + 4) = make_uint2(o[4], o[5]);
+    }
+}
+
 // pack_f16_kernel's values (fp16 product with the scale, truncated, no clamp: abq_gemm_wrapper.cu:29-54 of the
 // reference), written as field-packed K-tiled records instead of planes: what relayout_planes_kernel makes of
 // pack_f16_kernel's output, in one pass.
+// FP6: the same values written as FP6 records (codes of at most 5 bits signed / 4 unsigned): the low `bits` bits of
+// the truncated product, read as the signed or unsigned code they are in the planes (values beyond the range alias
+// there as well: the reference packs the low bits and does not clamp).
+template <bool FP6>
 __global__ __launch_bounds__(256) void pack_f16_tiled_kernel(const uint4 *__restrict__ in, const float *__restrict__ scale,
-                                                             uint32_t *__restrict__ tiled, int rows, int units, int bits)
+                                                             uint32_t *__restrict__ tiled, int rows, int units, int bits,
+                                                             int is_signed)
 {
     const _Float16 hs = (_Float16)scale[0];
     const size_t n_units = (size_t)rows * units; // units per row: a multiple of 16, so a quad is active as one
@@ -502,7 +536,16 @@ __global__ __launch_bounds__(256) void pack_f16_tiled_kernel(const uint4 *__rest
             }
         }
         const int row = (int)(t / units), u = (int)(t % units);
-        emit_tiled(v, tiled, rows, active ? row : 0, u >> 2, u & 3, bits, active, sel_pair, sel_half);
+        if constexpr (FP6) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const int low = v[c] & ((1 << bits) - 1);
+                v[c] = (is_signed && (low >> (bits - 1))) ? low - (1 << bits) : low;
+            }
+            emit_fp6(v, tiled, rows, active ? row : 0, u >> 2, u & 3, active);
+        } else {
+            emit_tiled(v, tiled, rows, active ? row : 0, u >> 2, u & 3, bits, active, sel_pair, sel_half);
+        }
     }
 }
 
@@ -549,29 +592,7 @@ __device__ __forceinline__ void quant_emit_unit(const uint4 &rawq, bool active, 
     }
     const int quad_lane = u & 3, w = u >> 2; // w: word-set (32 elements) within the row
     if (LAYOUT == 2) {
-        // position p = 4 s + c of the word-set's 192-bit string holds element 31 - (8c + s): this lane's
-        // element j goes to position 4 (7 - j) + 3 - quad_lane as the code (sign << 5) | magnitude
-        uint32_t o[6] = { 0u, 0u, 0u, 0u, 0u, 0u };
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const uint32_t code = v[j] < 0 ? (32u | (uint32_t)(-v[j])) : (uint32_t)v[j];
-            constexpr int kBase[8] = { 168, 144, 120, 96, 72, 48, 24, 0 }; // 24 (7 - j)
-            const int d0 = kBase[j] >> 5;                                   // first dword the code can touch
-            const uint64_t wide = (uint64_t)code << ((kBase[j] & 31) + 6 * (3 - quad_lane));
-            o[d0] |= (uint32_t)wide;
-            if (d0 + 1 < 6)
-                o[d0 + 1] |= (uint32_t)(wide >> 32);
-        }
-#pragma unroll
-        for (int d = 0; d < 6; ++d)
-            o[d] = quad_or(o[d]);
-        if (active && quad_lane == 0) {
-            const int ws = w & 3;
-            uint32_t *rec = planes + ((size_t)(w >> 2) * M + row) * 24 + 12 * (ws & 1) + 6 * (ws >> 1);
-            *reinterpret_cast<uint2 *>(rec) = make_uint2(o[0], o[1]);
-            *reinterpret_cast<uint2 *>(rec + 2) = make_uint2(o[2], o[3]);
-            *reinterpret_cast<uint2 *>(rec + 4) = make_uint2(o[4], o[5]);
-        }
+        emit_fp6(v, planes, M, row, w, quad_lane, active);
     } else if (LAYOUT == 1) {
         emit_tiled(v, planes, M, row, w, quad_lane, bits, active, sel_pair, sel_half);
     } else {
@@ -895,8 +916,17 @@ hipError_t launch_pack_f16_tiled(const void *in, const float *scale, uint32_t *t
                                  hipStream_t stream)
 {
     const size_t n_units = (size_t)rows * k / 8;
-    hipLaunchKernelGGL(pack_f16_tiled_kernel, dim3(grid_for(n_units)), dim3(256), 0, stream,
-                       reinterpret_cast<const uint4 *>(in), scale, tiled, rows, k / 8, bits);
+    hipLaunchKernelGGL(pack_f16_tiled_kernel<false>, dim3(grid_for(n_units)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint4 *>(in), scale, tiled, rows, k / 8, bits, 0);
+    return hipGetLastError();
+}
+
+hipError_t launch_pack_f16_fp6(const void *in, const float *scale, uint32_t *records, int rows, int k, int bits, int is_signed,
+                               hipStream_t stream)
+{
+    const size_t n_units = (size_t)rows * k / 8;
+    hipLaunchKernelGGL(pack_f16_tiled_kernel<true>, dim3(grid_for(n_units)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint4 *>(in), scale, records, rows, k / 8, bits, is_signed);
     return hipGetLastError();
 }
 

@@ -21,6 +21,19 @@ struct PreparedWeight {
     uint32_t fingerprint[16]; // the first 64 bytes of the prepared records, for verify_prepared
 };
 
+// FP6 records registered for a weight pointer (prepare_weight_fp6): a second copy for prefill-sized calls
+struct Fp6Weight {
+    const int *records;
+    int N, K, bits;
+    bool is_signed;
+};
+
+std::unordered_map<const void *, Fp6Weight> &fp6_table()
+{
+    static std::unordered_map<const void *, Fp6Weight> table;
+    return table;
+}
+
 std::mutex g_prepared_mutex;
 
 std::unordered_map<const void *, PreparedWeight> &prepared_table()
@@ -109,10 +122,34 @@ bool ABQGEMMWrapper::verify_prepared(const int *B, hipStream_t stream)
     return memcmp(now, w.fingerprint, nfp) == 0;
 }
 
+size_t ABQGEMMWrapper::fp6_weight_bytes(int N, int K) { return abq_fp6_bytes(N, K); }
+
+bool ABQGEMMWrapper::prepare_weight_fp6(const int *B, int N, int K, int W_BITS, bool SIGNED, int *records, hipStream_t stream)
+{
+    if (!B || !records || N <= 0 || K < 128 || K % 128 != 0 || W_BITS < 1 || W_BITS > (SIGNED ? 5 : 4)) {
+        printf("[ABQ][Error] prepare_weight_fp6: bad argument (N, K, bits = %d, %d, %d)\n", N, K, W_BITS);
+        return false;
+    }
+    if (is_prepared(B)) { // its planes are gone
+        printf("[ABQ][Error] prepare_weight_fp6: %p has been rewritten by prepare_weight already; call this one first\n", (const void *)B);
+        return false;
+    }
+    const abq_status rc = abq_relayout_planes_fp6(reinterpret_cast<const uint32_t *>(B), reinterpret_cast<uint32_t *>(records), N, K,
+                                                  W_BITS, SIGNED ? 1 : 0, stream);
+    if (rc != ABQ_OK) {
+        printf("[ABQ][Error] prepare_weight_fp6 failed: %s\n", abq_status_string(rc));
+        return false;
+    }
+    std::lock_guard<std::mutex> lock(g_prepared_mutex);
+    fp6_table()[B] = Fp6Weight{ records, N, K, W_BITS, SIGNED };
+    return true;
+}
+
 void ABQGEMMWrapper::release_weight(const int *B)
 {
     std::lock_guard<std::mutex> lock(g_prepared_mutex);
     prepared_table().erase(B);
+    fp6_table().erase(B);
 }
 
 bool ABQGEMMWrapper::is_prepared(const int *B)
@@ -153,6 +190,40 @@ void ABQGEMMWrapper::gemm(const int M, const int N, const int K, const _Float16 
     if (abq_gemm_ws_bytes < (size_t)x_bits_ * M * K / 8) {
         printf("[ABQ][Error] workspace too small: %zu bytes for M,K,bits = %d,%d,%d\n", abq_gemm_ws_bytes, M, K, x_bits_);
         return;
+    }
+    // Prefill-sized calls on a pair that qualifies for the FP6 matrix cores, when the loader registered FP6 records
+    // for this weight and the workspace holds the activations as such records (6 bits per element): twice the
+    // matrix-core rate of the int8 route, and nothing to unpack.
+    {
+        Fp6Weight f6{};
+        bool have = false;
+        {
+            std::lock_guard<std::mutex> lock(g_prepared_mutex);
+            const auto it = fp6_table().find(B);
+            if (it != fp6_table().end()) {
+                f6 = it->second;
+                have = true;
+            }
+        }
+        if (have && M > 16 && f6.N == N && f6.K == K && f6.bits == w_bits_ && f6.is_signed == signed_ &&
+            abq_fp6_eligible(x_bits_, w_bits_, signed_ ? 1 : 0, K) && abq_gemm_ws_bytes >= abq_fp6_bytes(M, K) &&
+            abq_preferred_weight_layout(x_bits_, w_bits_, signed_ ? 1 : 0, M, N, K, 0) == ABQ_LAYOUT_FP6) {
+            abq_gemm_state st;
+            abq_status rc = abq_pack_f16_fp6(A, scale, reinterpret_cast<uint32_t *>(abq_gemm_workspace), M, K, x_bits_, signed_ ? 1 : 0, stream);
+            if (rc == ABQ_OK)
+                rc = abq_gemm_init(nullptr, x_bits_, w_bits_, signed_ ? 1 : 0, reinterpret_cast<const uint32_t *>(abq_gemm_workspace),
+                                   reinterpret_cast<const uint32_t *>(f6.records), M, N, K, D, scale_out, bias ? 1 : 0,
+                                   ABQ_OUT_F16_TENSOR_F32SCALE, &st);
+            if (rc == ABQ_OK)
+                rc = abq_gemm_set_operand_layout(&st, ABQ_LAYOUT_FP6, ABQ_LAYOUT_FP6);
+            if (rc == ABQ_OK && st.init_success) {
+                const abq_status ex = abq_gemm_exec(&st, stream);
+                if (ex != ABQ_OK)
+                    printf("[ABQ][Error] launch failed: %s\n", abq_status_string(ex));
+                return;
+            }
+            // (anything the FP6 route refuses: the routes below)
+        }
     }
     PreparedWeight prepared;
     const bool tiled = find_prepared(B, &prepared);

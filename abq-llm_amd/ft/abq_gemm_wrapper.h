@@ -72,6 +72,15 @@ public:
     static void release_weight(const int *B);
     static bool is_prepared(const int *B);
     static bool verify_prepared(const int *B, hipStream_t stream);
+    // A second copy of a weight matrix for prefill-sized calls on pairs that qualify for the FP6 matrix cores
+    // (abq_fp6_eligible: at most 5 bits signed, 4 unsigned, e.g. W4A4): FP6 records of fp6_weight_bytes(N, K) bytes,
+    // written to caller-owned `records` from the planes at B and entered into a table under B.  Call it BEFORE
+    // prepare_weight (which rewrites the planes).  gemm() on B with more than 16 rows then packs its activations
+    // as FP6 records as well (workspace of at least 0.75 M K bytes) and runs the FP6 kernel where
+    // abq_preferred_weight_layout names that layout for the shape (the table of measured tiles, else from 65 rows
+    // up); every other call keeps the routes of prepare_weight.  release_weight(B) forgets both.
+    static size_t fp6_weight_bytes(int N, int K);
+    static bool prepare_weight_fp6(const int *B, int N, int K, int W_BITS, bool SIGNED, int *records, hipStream_t stream);
 
     // A: fp16 activations [M][K]; B: packed weight planes [w_bits][N][K/32]; C unused;
     // D: fp16 [M][N]; scale: activation quantisation scale (1 float, device);

@@ -305,6 +305,12 @@ abq_status abq_relayout_planes(const uint32_t *planes, uint32_t *tiled, int rows
  * second pass.  bits <= 8, k % 128 == 0. */
 abq_status abq_pack_f16_tiled(const void *in_f16, const float *scale_dev, uint32_t *tiled, int rows, int k, int bits,
                               void *stream);
+/* The same values written as FP6 records (abq_relayout_planes_fp6's layout; bits <= 5 signed, <= 4 unsigned): bit for
+ * bit what abq_relayout_planes_fp6 makes of abq_pack_f16's planes, i.e. the low `bits` bits of the truncated product
+ * read as the code they are (the reference does not clamp, pack_half, abq_gemm_wrapper.cu:42-49).  What
+ * ABQGEMMWrapper::gemm packs its activations into when the weight was also prepared as FP6 records. */
+abq_status abq_pack_f16_fp6(const void *in_f16, const float *scale_dev, uint32_t *records, int rows, int k, int bits,
+                            int is_signed, void *stream);
 
 /* FP6 records (no counterpart in the reference): the operand format of ABQ_STRATEGY_FP6.
  * CDNA4's matrix cores multiply 6-bit floats (E2M3) at twice their int8 rate, and an integer of

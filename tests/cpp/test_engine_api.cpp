@@ -313,6 +313,63 @@ static void gpu_paths()
         HIP_OK(hipFree(d_ws));
     }
 
+    {   // FT wrapper, W4A4 with the weight also registered as FP6 records: prefill-sized gemm() runs the FP6 matrix
+        // cores (activations packed as FP6 records), decode-sized calls keep the other routes; both against the oracle
+        const int N = 320, K = 640, Mmax = 300;
+        std::mt19937 r32(23);
+        std::normal_distribution<float> nd(0.f, 2.f);
+        std::vector<uint16_t> ha((size_t)Mmax * K);
+        for (auto &h : ha)
+            h = abq_oracle_f32_to_f16(nd(r32));
+        std::vector<uint32_t> wpl((size_t)4 * N * K / 32);
+        for (auto &v : wpl)
+            v = r32();
+        _Float16 *d_a, *d_d;
+        int *d_b, *d_rec, *d_scratch;
+        float *d_scales;
+        char *d_ws;
+        const size_t ws_bytes = (size_t)Mmax * K, wbytes = wpl.size() * 4; // 0.75 M K needed for FP6 records
+        HIP_OK(hipMalloc(&d_a, ha.size() * 2));
+        HIP_OK(hipMalloc(&d_d, (size_t)Mmax * N * 2));
+        HIP_OK(hipMalloc(&d_b, wbytes));
+        HIP_OK(hipMalloc(&d_scratch, wbytes));
+        HIP_OK(hipMalloc(&d_rec, ABQGEMMWrapper::fp6_weight_bytes(N, K)));
+        HIP_OK(hipMalloc(&d_scales, 8));
+        HIP_OK(hipMalloc(&d_ws, ws_bytes));
+        HIP_OK(hipMemcpy(d_a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(d_b, wpl.data(), wbytes, hipMemcpyHostToDevice));
+        const float in_scale = 1.7f, out_scale = 0.031f;
+        const float scales[2] = { in_scale, out_scale };
+        HIP_OK(hipMemcpy(d_scales, scales, 8, hipMemcpyHostToDevice));
+        CHECK(!ABQGEMMWrapper::prepare_weight_fp6(d_b, N, K, 6, true, d_rec, stream)); // too wide for FP6 codes
+        CHECK(ABQGEMMWrapper::prepare_weight_fp6(d_b, N, K, 4, true, d_rec, stream));
+        CHECK(ABQGEMMWrapper::prepare_weight(d_b, N, K, 4, d_scratch, stream));
+        CHECK(!ABQGEMMWrapper::prepare_weight_fp6(d_b, N, K, 4, true, d_rec, stream)); // the planes are gone
+        std::vector<uint32_t> ap((size_t)4 * Mmax * K / 32);
+        abq_oracle_pack_f16(ha.data(), in_scale, ap.data(), Mmax, K, 4);
+        std::vector<int> acc((size_t)Mmax * N);
+        abq_oracle_gemm_popc(wpl.data(), ap.data(), acc.data(), Mmax, N, K, 4, 4, 1, 0);
+        std::vector<uint16_t> want((size_t)Mmax * N);
+        abq_oracle_epilogue_f16(acc.data(), abq_oracle_f32_to_f16(out_scale), want.data(), (int)acc.size());
+        ABQGEMMWrapper wrap(4, 4, true);
+        for (int M : { 300, 128, 16, 1 }) {
+            HIP_OK(hipMemsetAsync(d_d, 0xff, (size_t)M * N * 2, stream));
+            wrap.gemm(M, N, K, d_a, d_b, nullptr, d_d, d_scales, nullptr, d_scales + 1, false, d_ws, ws_bytes, stream);
+            HIP_OK(hipStreamSynchronize(stream));
+            std::vector<uint16_t> got((size_t)M * N);
+            HIP_OK(hipMemcpy(got.data(), d_d, got.size() * 2, hipMemcpyDeviceToHost));
+            CHECK(std::equal(got.begin(), got.end(), want.begin()));
+        }
+        ABQGEMMWrapper::release_weight(d_b);
+        HIP_OK(hipFree(d_a));
+        HIP_OK(hipFree(d_d));
+        HIP_OK(hipFree(d_b));
+        HIP_OK(hipFree(d_scratch));
+        HIP_OK(hipFree(d_rec));
+        HIP_OK(hipFree(d_scales));
+        HIP_OK(hipFree(d_ws));
+    }
+
     {   // FT wrapper, dynamic path: per-token int8 activations, 2-bit weights with group scales and
         // zero points; expected values from a double-precision loop over the dequantised operands
         const int M = 40, N = 192, K = 512, G = 128, groups = K / G;

@@ -98,6 +98,22 @@ def test_pack_f16_tiled_equals_the_relayout_of_the_planes(abq, rows, k):
         assert torch.equal(got.view(-1), want.view(-1)), bits
 
 
+@pytest.mark.parametrize("rows,k", [(1, 128), (5, 4096), (300, 512), (1024, 4096)])
+def test_pack_f16_fp6_equals_the_fp6_relayout_of_the_planes(abq, rows, k):
+    """abq_pack_f16_fp6 writes in one pass what abq_relayout_planes_fp6 makes of abq_pack_f16's planes, values that
+    overflow the code width included (the reference packs the low bits and does not clamp)."""
+    g = torch.Generator(device="cuda").manual_seed(rows + k + 1)
+    x = (torch.randn((rows, k), generator=g, device="cuda") * 3).to(torch.float16)
+    s = torch.tensor([2.5], dtype=torch.float32, device="cuda")
+    for bits, signed in [(4, True), (5, True), (2, True), (3, True), (4, False), (2, False), (1, False)]:
+        want = abq.relayout_planes_fp6(abq.pack_f16(x, s, bits), signed)
+        got = abq.pack_f16_fp6(x, s, bits, signed)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), (bits, signed)
+    with pytest.raises(abq.AbqError):
+        abq.pack_f16_fp6(x, s, 6, True)
+
+
 @pytest.mark.parametrize("p", [2, 4, 8])
 def test_decode_quantises_fp16_activations_itself(abq, oracle, p):
     """abq_gemm_set_f16_activations: the decode kernel on prepared weights reads fp16 activations and quantises them
