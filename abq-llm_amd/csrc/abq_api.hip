@@ -1092,8 +1092,8 @@ static bool decode_tiled_grouped_fits(const abq_gemm_state *st, int group_size, 
 {
     const abq_tile_config &c = st->cfg;
     const KernelTable *t = find_table(registry().decode_tiled_grouped, c.x_bits, c.w_bits, c.is_signed);
-    return t && t->count > 0 && st->auto_chosen && group_size == 128 && (!act || st->N % 32 == 0) &&
-           decode_tiled_grouped_rows(16, act ? 2 : 1, st->M, st->K, c.x_bits) != 0 &&
+    return t && t->count > 0 && st->auto_chosen && (group_size == 128 || group_size == 64) && (!act || st->N % 32 == 0) &&
+           decode_tiled_grouped_rows(16, act ? 2 : 1, st->M, st->K, c.x_bits, group_size) != 0 &&
            decode_tiled_grouped_pays(c.x_bits, c.w_bits, st->M, st->N, st->K, act);
 }
 
@@ -1767,8 +1767,8 @@ int abq_prepared_decode_pays(int x_bits, int w_bits, int is_signed, int M, int N
     const Registry &reg = registry();
     if (group_size) {
         const KernelTable *t = find_table(reg.decode_tiled_grouped, x_bits, w_bits, is_signed);
-        return t && t->count > 0 && group_size == 128 && (!act || N % 32 == 0) &&
-                       decode_tiled_grouped_rows(16, act ? 2 : 1, M, K, x_bits) != 0 &&
+        return t && t->count > 0 && (group_size == 128 || group_size == 64) && (!act || N % 32 == 0) &&
+                       decode_tiled_grouped_rows(16, act ? 2 : 1, M, K, x_bits, group_size) != 0 &&
                        decode_tiled_grouped_pays(x_bits, w_bits, M, N, K, act)
                    ? 1
                    : 0;

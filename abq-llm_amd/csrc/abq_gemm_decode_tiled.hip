@@ -521,10 +521,16 @@ template <int P, bool SIGNED> __device__ __forceinline__ void dtg_operands(const
 // XDYN is the number of units a thread holds (0: the activations arrive packed): 1, 2 or, with eight waves, 4, i.e. up
 // to 16384 elements per workgroup; the launcher takes the smallest that covers the rows (a row of 4096 needs one unit
 // per thread of eight waves: 52 + 25 registers instead of 52 + 49, three workgroups per compute unit instead of two).
-template <int Q, int P, bool SIGNED, int NW, int D, int T, int XDYN = 0>
+// G64: groups of 64, two to a K tile: lane groups 0, 1 hold the elements of the first, 2, 3 those of the second, and
+// the matrix core sums over all four, so a step runs its two instructions twice: once on all lanes and once with
+// the activations of lane groups 2, 3 zeroed; the difference is the second group's dot product.  Scales, zero
+// points and group sums are staged as [2 K tiles' worth of groups][16] and folded per half.
+template <int Q, int P, bool SIGNED, int NW, int D, int T, int XDYN = 0, bool G64 = false>
 __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmArgs a, int mrows)
 {
     static_assert(!XDYN || (Q == 8 && SIGNED), "in-kernel quantisation writes signed 8-bit records");
+    static_assert(!(XDYN && G64), "in-kernel quantisation takes group sums over 128 elements");
+    constexpr int GPT = G64 ? 2 : 1; // scale groups per K tile
     static_assert(XDYN == 0 || XDYN == 1 || XDYN == 2 || (XDYN == 4 && NW == 8), "units per thread");
     constexpr int XP = XDYN > 0 ? XDYN : 1; // XDYN: units per thread
     constexpr int NT = 64 * NW;
@@ -548,7 +554,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
     const char *Wt = reinterpret_cast<const char *>(a.W);
     const unsigned xs_addr = (unsigned)(size_t)xs;
     const int xchunks = KT * Mb * Q;
-    const int per_arr = (KT * 16 + 63) & ~63; // floats of one [group][16] array, in whole wave loads
+    const int NG = KT * GPT;                   // scale groups along K
+    const int per_arr = (NG * 16 + 63) & ~63;  // floats of one [group][16] array, in whole wave loads
     float *sws = reinterpret_cast<float *>(xs + (size_t)mrows * (KT + 1) * Q * 16 + 1024); // [T][group][16]
     float *zws = sws + T * per_arr;                                                       // [T][group][16]
     int *sxs = reinterpret_cast<int *>(zws + T * per_arr);                                // [group][16]
@@ -583,13 +590,13 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
     }
     // ---- scales, zero points of the tiles' rows and group sums of the activation rows: [group][16] ----
     {
-        const int nfl = KT * 16;
+        const int nfl = NG * 16;
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             for (int pb = wid * 64; pb < nfl; pb += NT) {
                 const int p = min(pb + lane, nfl - 1);
                 const int n = min((tile0 + t) * 16 + (p & 15), N - 1);
-                const size_t src = (size_t)n * KT + (p >> 4);
+                const size_t src = (size_t)n * NG + (p >> 4);
                 dt_dma_dword(a.w_scale + src, (unsigned)(size_t)(sws + t * per_arr + pb));
                 if (zp)
                     dt_dma_dword(a.w_zero + src, (unsigned)(size_t)(zws + t * per_arr + pb));
@@ -599,7 +606,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
             for (int pb = wid * 64; pb < nfl; pb += NT) {
                 const int p = min(pb + lane, nfl - 1);
                 const int m = m0 + min(p & 15, Mb - 1);
-                dt_dma_dword(a.x_group_sums + (size_t)m * KT + (p >> 4), (unsigned)(size_t)(sxs + pb));
+                dt_dma_dword(a.x_group_sums + (size_t)m * NG + (p >> 4), (unsigned)(size_t)(sxs + pb));
             }
         }
     }
@@ -736,6 +743,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
             const bool have = cs < KT; // wave-uniform
             v4i av[2];
             float sw[T], zs[T], sxf[4];
+            float sw2[G64 ? T : 1], zs2[G64 ? T : 1], sxf2[4]; // G64: the K tile's second group
             if (have) {
                 const int rowi = cs * Mb + ml; // row index in LDS: K tile * rows + row
                 const unsigned char *xrow = xs + (uint32_t)rowi * (Q * 16u);
@@ -755,17 +763,29 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
                 }
 #pragma unroll
                 for (int t = 0; t < T; ++t) {
-                    sw[t] = sws[t * per_arr + cs * 16 + r];
-                    zs[t] = zp ? sw[t] * zws[t * per_arr + cs * 16 + r] : 0.f;
+                    sw[t] = sws[t * per_arr + (GPT * cs) * 16 + r];
+                    zs[t] = zp ? sw[t] * zws[t * per_arr + (GPT * cs) * 16 + r] : 0.f;
                     sw[t] *= unshift;
+                    if constexpr (G64) {
+                        sw2[t] = sws[t * per_arr + (2 * cs + 1) * 16 + r];
+                        zs2[t] = zp ? sw2[t] * zws[t * per_arr + (2 * cs + 1) * 16 + r] : 0.f;
+                        sw2[t] *= unshift;
+                    }
                 }
                 if (zp) {
-                    const v4i sx = *reinterpret_cast<const v4i *>(sxs + cs * 16 + 4 * g);
+                    const v4i sx = *reinterpret_cast<const v4i *>(sxs + (GPT * cs) * 16 + 4 * g);
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         sxf[e] = (float)sx[e];
+                    if constexpr (G64) {
+                        const v4i sx2 = *reinterpret_cast<const v4i *>(sxs + (2 * cs + 1) * 16 + 4 * g);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            sxf2[e] = (float)sx2[e];
+                    }
                 } else {
                     sxf[0] = sxf[1] = sxf[2] = sxf[3] = 0.f;
+                    sxf2[0] = sxf2[1] = sxf2[2] = sxf2[3] = 0.f;
                 }
             }
             // Waited for and marked as landed on every path: a register with a load still in flight must not
@@ -781,9 +801,20 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
                     dtg_operands<P, SIGNED>(wb[d][t], bv);
                     v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[0], bv[0], v4i{ 0, 0, 0, 0 }, 0, 0, 0);
                     acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[1], bv[1], acc, 0, 0, 0);
+                    if constexpr (G64) {
+                        // the first group alone: the activations of lane groups 2, 3 zeroed
+                        const v4i zero = v4i{ 0, 0, 0, 0 };
+                        const v4i a0 = g < 2 ? av[0] : zero, a1 = g < 2 ? av[1] : zero;
+                        v4i lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, bv[0], zero, 0, 0, 0);
+                        lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, bv[1], lo, 0, 0, 0);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        facc[t][e] += sw[t] * (float)acc[e] - zs[t] * sxf[e];
+                        for (int e = 0; e < 4; ++e)
+                            facc[t][e] += sw[t] * (float)lo[e] - zs[t] * sxf[e] + sw2[t] * (float)(acc[e] - lo[e]) - zs2[t] * sxf2[e];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            facc[t][e] += sw[t] * (float)acc[e] - zs[t] * sxf[e];
+                    }
                 }
             }
         }
@@ -827,17 +858,17 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
     }
 }
 
-template <int Q, int P, bool SIGNED, int NW, int D, int T, int XD>
+template <int Q, int P, bool SIGNED, int NW, int D, int T, int XD, bool G64 = false>
 static hipError_t launch_decode_tiled_grouped_instance(const GemmArgs &a, int mrows, hipStream_t stream)
 {
-    const size_t lds = decode_tiled_grouped_lds(NW, T, mrows, a.K, Q);
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T, XD>),
+    const size_t lds = decode_tiled_grouped_lds(NW, T, mrows, a.K, Q, G64 ? 64 : 128);
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T, XD, G64>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess)
         return attr;
     const int tiles = (a.N + 15) / 16;
     const dim3 grid((tiles + T - 1) / T, (a.M + mrows - 1) / mrows);
-    hipLaunchKernelGGL((gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T, XD>), grid, dim3(64 * NW), lds, stream, a, mrows);
+    hipLaunchKernelGGL((gemm_decode_tiled_grouped<Q, P, SIGNED, NW, D, T, XD, G64>), grid, dim3(64 * NW), lds, stream, a, mrows);
     return hipGetLastError();
 }
 
@@ -845,12 +876,18 @@ static hipError_t launch_decode_tiled_grouped_instance(const GemmArgs &a, int mr
 template <int Q, int P, bool SIGNED, int NW, int D, int T, bool XDYN = false>
 static hipError_t launch_decode_tiled_grouped_as(const GemmArgs &a, hipStream_t stream)
 {
-    const int mrows = decode_tiled_grouped_rows(NW, T, a.M, a.K, Q);
+    const int mrows = decode_tiled_grouped_rows(NW, T, a.M, a.K, Q, a.group_size);
     if (mrows == 0)
         return hipErrorInvalidValue;
     // in-kernel quantisation: a workgroup's rows fit its threads' registers (two or four units of eight halves each)
     if (XDYN && (size_t)mrows * a.K > 16384)
         return hipErrorInvalidValue;
+    if (a.group_size == 64) {
+        if constexpr (XDYN)
+            return hipErrorInvalidValue;
+        else
+            return launch_decode_tiled_grouped_instance<Q, P, SIGNED, NW, D, T, 0, true>(a, mrows, stream);
+    }
     if constexpr (XDYN) {
         // the fewest units per thread that cover the workgroup's rows
         const int need = (int)(((size_t)mrows * a.K / 8 + 64 * NW - 1) / (64 * NW));
@@ -882,7 +919,7 @@ static hipError_t launch_decode_tiled_grouped_t(const GemmArgs &a, hipStream_t s
 
 template <int Q, int P, bool SIGNED, bool XDYN = false> static hipError_t launch_decode_tiled_grouped(const GemmArgs &a, hipStream_t stream)
 {
-    if (a.group_size != 128 || !a.w_scale || (!XDYN && !a.x_scale) || (size_t)a.N * a.K * P / 8 >= (1ull << 32) ||
+    if ((a.group_size != 128 && !(a.group_size == 64 && !XDYN)) || !a.w_scale || (!XDYN && !a.x_scale) || (size_t)a.N * a.K * P / 8 >= (1ull << 32) ||
         (size_t)a.M * a.K * Q / 8 >= (1ull << 32) || (XDYN && (a.x_dynamic < 1 || a.x_dynamic > 2 || (a.x_dynamic == 2 && !a.w_zero_term))))
         return hipErrorInvalidValue;
     if (a.act) {
@@ -896,7 +933,7 @@ template <int Q, int P, bool SIGNED, bool XDYN = false> static hipError_t launch
     // rows of a block stay the same, and not for shapes the variant that quantises in the kernel takes (at most 16384
     // elements), whose output has to stay that of this one bit for bit.
     if (!XDYN && a.M > 8 && (size_t)a.M * a.K > 16384 && (a.N + 15) / 16 >= 512 && a.N % 32 == 0 &&
-        decode_tiled_grouped_rows(16, 2, a.M, a.K, Q) == decode_tiled_grouped_rows(16, 1, a.M, a.K, Q))
+        decode_tiled_grouped_rows(16, 2, a.M, a.K, Q, a.group_size) == decode_tiled_grouped_rows(16, 1, a.M, a.K, Q, a.group_size))
         return launch_decode_tiled_grouped_t<Q, P, SIGNED, 2, XDYN>(a, stream);
     return launch_decode_tiled_grouped_t<Q, P, SIGNED, 1, XDYN>(a, stream);
 }

@@ -96,18 +96,19 @@ inline int decode_tiled_rows(int nw, int t, int M, int K, int q)
 // The same kernel with group scales (groups of 128 = one K tile): fp32 partial tiles, and after the activations the
 // tile's weight scales and zero points ([group][16 rows] each, T tiles) and the activation group sums
 // ([group][16 rows]), every array padded to whole wave loads of four bytes per lane.
-inline size_t decode_tiled_grouped_lds(int nw, int t, int mrows, int K, int q)
+// (group: 128, or 64 = two scale groups per K tile)
+inline size_t decode_tiled_grouped_lds(int nw, int t, int mrows, int K, int q, int group = 128)
 {
-    const size_t groups = (size_t)K / 128;
+    const size_t groups = (size_t)K / group;
     const size_t per_tile = (groups * 16 + 63) / 64 * 256; // bytes of one [group][16] float array
     return decode_tiled_lds(nw, t, mrows, K, q) + (2 * t + 1) * per_tile + 1024;
 }
-inline int decode_tiled_grouped_rows(int nw, int t, int M, int K, int q)
+inline int decode_tiled_grouped_rows(int nw, int t, int M, int K, int q, int group = 128)
 {
     int mrows = M < 16 ? M : 16;
-    while (mrows > 1 && decode_tiled_grouped_lds(nw, t, mrows, K, q) > 150 * 1024)
+    while (mrows > 1 && decode_tiled_grouped_lds(nw, t, mrows, K, q, group) > 150 * 1024)
         mrows = (mrows + 1) / 2;
-    return decode_tiled_grouped_lds(nw, t, mrows, K, q) <= 160 * 1024 ? mrows : 0;
+    return decode_tiled_grouped_lds(nw, t, mrows, K, q, group) <= 160 * 1024 ? mrows : 0;
 }
 
 // Workgroup id -> output tile.  XCD x = id % 8 owns n blocks [x * npx, (x + 1) * npx); inside an XCD the

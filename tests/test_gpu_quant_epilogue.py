@@ -212,9 +212,10 @@ def test_decode_kernel_with_group_scales_and_zero_points(abq, oracle, q, p, sign
 
 @pytest.mark.parametrize("q,p,signed", [(8, 2, True), (8, 4, True), (8, 8, True), (4, 4, True), (4, 2, True), (2, 2, True),
                                         (4, 4, False), (4, 2, False), (2, 2, False)])
-def test_decode_on_prepared_operands_with_group_scales(abq, oracle, q, p, signed):
-    """At most 16 activation rows with both operands K-tiled and groups of 128: the prepared-operand decode
-    kernel's group-scale variant (one K tile = one scale group per step), with zero points on both sides."""
+@pytest.mark.parametrize("group_size", [128, 64])
+def test_decode_on_prepared_operands_with_group_scales(abq, oracle, q, p, signed, group_size):
+    """At most 16 activation rows with both operands K-tiled and groups of 128 or 64: the prepared-operand decode
+    kernel's group-scale variant (one K tile = one or two scale groups per step), with zero points on both sides."""
     from oracle import quantizer as Q
     rng = np.random.default_rng(3 * q + 11 * p + signed)
     for (M, N, K, zeros) in [(1, 64, 128, 0), (5, 200, 384, 1), (16, 4096 + 8, 4096, 2), (8, 300, 11008, 2), (3, 4096, 1152, 1),
@@ -223,18 +224,18 @@ def test_decode_on_prepared_operands_with_group_scales(abq, oracle, q, p, signed
         lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed else (0, 1 << p)
         x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
         w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
-        G = K // 128
+        G = K // group_size
         xs = rng.uniform(0.01, 0.05, M)
         wsc = rng.uniform(0.001, 0.02, (N, G))
         wz = rng.integers(lo_w, hi_w, (N, G)).astype(np.float64) if zeros >= 1 else np.zeros((N, G))
         xz = rng.integers(lo_x // 2, hi_x // 2, M).astype(np.float64) if zeros >= 2 else np.zeros(M)
-        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, 128)
+        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, group_size)
         wp = planes_dev(oracle.pack_i32(w, p))
-        kw = dict(x_scale=fdev(xs), w_scale=fdev(wsc), group_size=128, x_tiled=True, w_tiled=True)
+        kw = dict(x_scale=fdev(xs), w_scale=fdev(wsc), group_size=group_size, x_tiled=True, w_tiled=True)
         if zeros >= 1:
-            kw.update(w_zero=fdev(wz), x_group_sums=torch.from_numpy(x.reshape(M, G, 128).sum(axis=2).astype(np.int32)).cuda())
+            kw.update(w_zero=fdev(wz), x_group_sums=torch.from_numpy(x.reshape(M, G, group_size).sum(axis=2).astype(np.int32)).cuda())
         if zeros >= 2:
-            kw.update(x_zero=fdev(xz), w_zero_term=abq.weight_zero_term(wp, signed, kw["w_scale"], kw["w_zero"], 128))
+            kw.update(x_zero=fdev(xz), w_zero_term=abq.weight_zero_term(wp, signed, kw["w_scale"], kw["w_zero"], group_size))
         out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
         xt, wt = abq.relayout_planes(planes_dev(oracle.pack_i32(x, q))), abq.relayout_planes(wp)
         got = run_grouped(abq, xt, wt, signed, strategy="decode_tiled", out=out, **kw)
@@ -289,7 +290,7 @@ def test_group_scale_decode_kernel_over_row_blocks(abq, oracle, q, p, signed):
         assert not abq.prepared_decode_pays(8, 2, True, 32, 12288, 4096, 128)
         assert not abq.prepared_decode_pays(8, 2, True, 96, 4096, 4096, 128)
         assert not abq.prepared_decode_pays(8, 2, True, 200, 4096, 4096, 128)
-        assert not abq.prepared_decode_pays(8, 2, True, 32, 4096, 4096, 64)
+        assert abq.prepared_decode_pays(8, 2, True, 32, 4096, 4096, 64)  # groups of 64: two to a K tile
 
 
 def test_decode_kernel_quantises_fp16_activations_per_token_itself(abq, oracle):
@@ -373,10 +374,13 @@ def test_decode_on_prepared_operands_group_scales_either_call_order(abq, oracle)
     out = g.run()
     torch.cuda.synchronize()
     assert_close_rel(out.cpu().numpy(), Q.dequant_matmul(x, xs, np.zeros(M), w, wsc, np.zeros_like(wsc), 128))
-    # groups of 64 have no variant there: the state moves to the tiled kernel
+    # groups of 64 run on the same kernel (two groups to a K tile)
     g2 = abq.Gemm(xt, wt, True, out_kind=abq.OUT_F16_SCALED, x_scale=fdev(xs), w_scale=fdev(np.repeat(wsc, 2, axis=1)),
                   group_size=64, x_tiled=True, w_tiled=True)
-    assert g2.strategy == "tiled"
+    assert g2.strategy == "decode_tiled"
+    out2 = g2.run()
+    torch.cuda.synchronize()
+    assert_close_rel(out2.cpu().numpy(), Q.dequant_matmul(x, xs, np.zeros(M), w, wsc, np.zeros_like(wsc), 128))
 
 
 def interleave16(gate, up):
@@ -417,8 +421,6 @@ def test_silu_gate_epilogue(abq, oracle, M, strategy, group_size):
     if strategy == "tiled":
         got = run_grouped(abq, planes_dev(oracle.pack_i32(x, q)), abq.relayout_planes(wp), True, w_tiled=True, out=out, **kw)
     elif strategy == "decode_tiled":
-        if group_size == 64:
-            pytest.skip("the prepared-operand decode kernel has groups of 128 only")
         got = run_grouped(abq, abq.relayout_planes(planes_dev(oracle.pack_i32(x, q))), abq.relayout_planes(wp), True,
                           strategy="decode_tiled", x_tiled=True, w_tiled=True, out=out, **kw)
     else:

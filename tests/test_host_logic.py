@@ -380,10 +380,10 @@ def test_group_scales_move_a_state_to_the_kernel_that_carries_them(abq):
     assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 128) == 0
     assert names[st.strategy] == "decode_tiled" and st.variant == 0
     assert lib.abq_gemm_set_activation(ctypes.byref(st), abq.ACT_SILU_GATE) == 0 and names[st.strategy] == "decode_tiled"
-    # groups of 64, or widths of several fields, have no variant there: the tiled kernel
+    # groups of 64 run there too (two groups to a K tile); widths of several fields have no variant there: the tiled kernel
     st = state(M=8)
     assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0
-    assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 64) == 0 and names[st.strategy] == "tiled"
+    assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 64) == 0 and names[st.strategy] == "decode_tiled"
     st = state(q=6, p=2, M=8)
     assert lib.abq_gemm_set_scales(ctypes.byref(st), 0x4000, 0x5000, 128) == 0
     assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0 and names[st.strategy] == "tiled"
