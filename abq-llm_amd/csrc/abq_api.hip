@@ -1024,7 +1024,7 @@ static bool decode_tiled_flips_ok(const abq_gemm_state *st)
     return true;
 }
 
-static abq_status switch_to_decode_tiled(abq_gemm_state *st)
+static abq_status switch_to_decode_tiled(abq_gemm_state *st, bool one_tile = false)
 {
     const abq_tile_config &c = st->cfg;
     const KernelTable *tdt = find_table(registry().decode_tiled, c.x_bits, c.w_bits, c.is_signed);
@@ -1036,10 +1036,15 @@ static abq_status switch_to_decode_tiled(abq_gemm_state *st)
     // at K = 11008); with more rows the activation traffic comes first and one load at a time is as fast.  Several
     // blocks of 16 rows (M > 16): eight waves on two tiles, so that a workgroup's activations serve twice the weights.
     const bool row_blocks = st->M > 16;
-    const int want_t = row_blocks ? kDecodeTiledBlocksTiles : 1;
-    const int want_wk = row_blocks ? kDecodeTiledBlocksWaves : tiles > 512 ? 8 : 16;
+    // Nine to sixteen rows: the activations a workgroup stages (every workgroup all of them) outweigh the weights of
+    // one tile, so a workgroup takes several tiles: three on wide outputs, two on long K (W2A8 at 16 rows, 11008 x 4096:
+    // 5.4 against 6.2 us; 4096 x 11008: 6.5 against 9.1).
+    // (one_tile: the caller needs an instance of one tile per workgroup, the ones that quantise fp16 activations)
+    const bool many_rows = !one_tile && !row_blocks && st->M > 8 && (tiles > 512 || steps > 32);
+    const int want_t = row_blocks ? kDecodeTiledBlocksTiles : many_rows ? (tiles > 512 ? 3 : 2) : 1;
+    const int want_wk = row_blocks ? kDecodeTiledBlocksWaves : many_rows ? 16 : tiles > 512 ? 8 : 16;
     // (8-bit weights keep one load in flight: W8A8 4096 x 4096 at one row 5.3 against 6.5 us, 4096 x 11008 10.2 against 11.7)
-    const int want_d = row_blocks ? 1 : tiles > 512 ? 2 : (steps > 32 && st->M <= 2 && c.w_bits < 8) ? 3 : 1;
+    const int want_d = row_blocks || many_rows ? 1 : tiles > 512 ? 2 : (steps > 32 && st->M <= 2 && c.w_bits < 8) ? 3 : 1;
     int pick = -1;
     for (int i = 0; i < tdt->count; ++i) {
         const KernelEntry &e = tdt->entries[i];
@@ -1460,7 +1465,7 @@ int abq_gemm_row_sums_ready(const abq_gemm_state *st)
     return row_sum_plan(st, xb + wb).ok ? 1 : 0;
 }
 
-static abq_status switch_to_decode_tiled(abq_gemm_state *st);
+static abq_status switch_to_decode_tiled(abq_gemm_state *st, bool one_tile);
 static bool decode_tiled_pays(int x_bits, int w_bits, int M, int N, int K);
 static void apply_tuned(abq_gemm_state *st);
 
@@ -1875,7 +1880,11 @@ abq_status abq_gemm_set_f16_activations(abq_gemm_state *st, const void *x_f16, c
         return ABQ_ERR_INVALID_ARG;
     const abq_tile_config &c = st->cfg;
     const KernelTable *t = find_table(registry().decode_tiled_f16, c.x_bits, c.w_bits, c.is_signed);
-    // the quantising instances mirror the first entries of the kernel's table
+    // the quantising instances mirror the first entries of the kernel's table, those of one tile per workgroup; a
+    // state whose tile is the library's choice moves to the one its rules pick among them
+    if (st->strategy == ABQ_STRATEGY_DECODE_TILED && st->auto_chosen && t && st->variant >= t->count && st->M <= 16 &&
+        switch_to_decode_tiled(st, true) != ABQ_OK)
+        return ABQ_ERR_UNSUPPORTED;
     if (st->strategy != ABQ_STRATEGY_DECODE_TILED || st->group_size || st->act || st->w_layout != ABQ_LAYOUT_TILED || !t ||
         st->variant < 0 || st->variant >= t->count || (size_t)st->M * st->K * 2 >= (1ull << 32))
         return ABQ_ERR_UNSUPPORTED;

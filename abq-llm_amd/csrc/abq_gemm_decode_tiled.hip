@@ -940,7 +940,7 @@ template <int Q, int P, bool SIGNED, bool XDYN = false> static hipError_t launch
 
 // Native tile space of this kernel: (waves, weight loads in flight per wave, tiles per workgroup).  Entries name
 // MFMA 16x16x64 with NSTAGE = 6; wk = waves, tn = tiles, kb = K elements a wave has in flight (D steps).
-#define ABQ_DT_VARIANTS(V) V(16, 1, 1) V(16, 3, 1) V(8, 2, 1) V(16, 1, 3) V(8, 1, 2)
+#define ABQ_DT_VARIANTS(V) V(16, 1, 1) V(16, 3, 1) V(8, 2, 1) V(16, 1, 3) V(8, 1, 2) V(8, 2, 2) V(16, 1, 2)
 
 #define ABQ_DT_ENTRY_T(NW, D, T) { 16, 1, T, 1, 1, NW, 6, &launch_decode_tiled<ABQ_Q, ABQ_P, true, NW, D, T>, (512 / ABQ_P) * D },
 #define ABQ_DT_ENTRY_F(NW, D, T) { 16, 1, T, 1, 1, NW, 6, &launch_decode_tiled<ABQ_Q, ABQ_P, false, NW, D, T>, (512 / ABQ_P) * D },

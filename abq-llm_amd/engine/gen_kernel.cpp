@@ -233,7 +233,7 @@ std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits, bool is_signed)
     {
         const bool field = (x_bits == 2 || x_bits == 4 || x_bits == 8) && (w_bits == 2 || w_bits == 4 || w_bits == 8);
         if (field && x_bits >= w_bits) {
-            const int dt[][3] = { { 16, 1, 1 }, { 16, 3, 1 }, { 8, 2, 1 }, { 16, 1, 3 }, { 8, 1, 2 } };
+            const int dt[][3] = { { 16, 1, 1 }, { 16, 3, 1 }, { 8, 2, 1 }, { 16, 1, 3 }, { 8, 1, 2 }, { 8, 2, 2 }, { 16, 1, 2 } };
             const int stepk = 512 / w_bits;
             for (const auto &v : dt)
                 out.push_back(Tile{ 16, 16 * v[2], stepk * v[1] * v[0], 16, 16 * v[2], stepk * v[1], 16, 16, 64, 1, v[0], { 6 } });

@@ -672,7 +672,7 @@ def main():
         # activations quantised per token on the device inside the timed call, fp16 output; gate and up run
         # as one GEMM with the fused SiLU-gate epilogue.  Time = quantise+pack kernel + GEMM, graph replay.
         layer = []
-        for tokens in (1, 16, 1024, 16384):  # a decode step of batch 1 and 16 (weights stay in the Infinity Cache), two prefills
+        for tokens in (1, 16, 1024, 16384):  # a decode step of batch 1 and 16 (weights rotating, like every decode row), two prefills
             for name, N, K, act in (("qkv", 12288, 4096, 0), ("o", 4096, 4096, 0), ("gate_up_silu", 22016, 4096, 1),
                                     ("down", 4096, 11008, 0)):
                 G = K // 128
@@ -682,16 +682,28 @@ def main():
                 x = torch.randn((tokens, K), device="cuda", dtype=torch.float16)
                 xt, xsc, _, sums = abq.quant_pack_f16(x, Q_BITS, symmetric=True, tiled=True, group_size=128)
                 out = torch.empty((tokens, N // 2 if act else N), dtype=torch.float16, device="cuda")
-                gm = abq.Gemm(xt, wt, SIGNED, out=out, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc, group_size=128,
-                              w_zero=wz, x_group_sums=sums, x_tiled=True, w_tiled=True, act=act)
+                kwl = dict(out=out, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc, group_size=128,
+                           w_zero=wz, x_group_sums=sums, x_tiled=True, w_tiled=True, act=act)
+                gm = abq.Gemm(xt, wt, SIGNED, **kwl)
+                # decode steps: the weights rotate over >= 512 MiB of copies, so that the Infinity Cache does not serve them
+                # (a prefill streams its activations and outputs through the cache anyway)
+                copies = [wt]
+                if tokens <= 16:
+                    wbytes = wt.numel() * 4
+                    wrot = wt.unsqueeze(0).repeat(max(2, math.ceil(ROTATE_BYTES / wbytes)), 1, 1, 1, 1)
+                    copies = [wrot[r] for r in range(wrot.shape[0])]
+                gms = [gm] if len(copies) == 1 else [abq.Gemm(xt, c, SIGNED, **kwl) for c in copies]
+                calls = [0]
 
                 def step():
                     abq._check(abq.lib().abq_quant_pack_f16(x.data_ptr(), tokens, K, Q_BITS, 1, 1, xt.data_ptr(), xsc.data_ptr(),
                                                             None, sums.data_ptr(), 128, abq._stream_ptr(None)), "quant_pack")
-                    gm.run()
+                    gms[calls[0] % len(gms)].run()
+                    calls[0] += 1
                 step()
                 torch.cuda.synchronize()
-                reps = 20 if tokens < 1024 else 10 if tokens < 8192 else 3  # (a replay's own launch cost is spread over its steps)
+                # (a replay's own launch cost is spread over its steps; a decode graph walks through all weight copies)
+                reps = max(20, len(gms)) if tokens < 1024 else 10 if tokens < 8192 else 3
                 gr = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(gr):
                     for _ in range(reps):
@@ -711,19 +723,22 @@ def main():
                 if tokens <= 16 and tokens * K <= 16384 and gm.strategy == "decode_tiled":
                     # the smallest calls: the decode kernel quantises the rows itself, one launch, same output bit for bit
                     out1 = torch.empty_like(out)
-                    g1 = abq.Gemm(xt, wt, SIGNED, out=out1, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc, group_size=128,
-                                  x_tiled=True, w_tiled=True, act=act)
-                    g1.set_dynamic_f16_activations(x, True, w_zero=wz)
-                    g1.run()
+                    g1s = []
+                    for c in copies:
+                        g1 = abq.Gemm(xt, c, SIGNED, out=out1, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc, group_size=128,
+                                      x_tiled=True, w_tiled=True, act=act)
+                        g1.set_dynamic_f16_activations(x, True, w_zero=wz)
+                        g1s.append(g1)
+                    g1s[0].run()
                     torch.cuda.synchronize()
                     if not torch.equal(out1, out):
                         raise RuntimeError("one-launch dynamic GEMM differs from quantise + GEMM (%s, tokens=%d)" % (name, tokens))
-                    us1 = time_rotating([g1], reps=20)
+                    us1 = time_rotating(g1s, reps=max(20, len(g1s)))
                     entry["one_launch_us"] = round(us1, 1)
                     log("layer %s tokens=%d: one launch (kernel quantises the rows) %.1f us" % (name, tokens, us1))
-                    del g1, out1
+                    del g1, g1s, out1
                 layer.append(entry)
-                del gr, gm, out, x, xt, wt
+                del gr, gm, gms, copies, out, x, xt, wt
         extra["decoder_layer_w2a8_group128"] = layer
 
 

@@ -578,7 +578,7 @@ def test_decode_on_prepared_operands(abq, oracle, q, p, signed):
             got = abq.Gemm(xt, wt, signed, cfg=cfg, out=out, **kw).run().cpu().numpy()
             assert np.array_equal(got, want), (abq.format_kernel_name(cfg), M, N, K)
             ran += 1
-        assert ran == 5
+        assert ran == 7
         if needs_sums:  # a tile of this kernel named by the caller, but no sums: refused before any launch
             cfg = [c for c in abq.native_configs(qp, pp, signed) if c.nstage == 6][0]
             with pytest.raises(abq.AbqError) as e:
