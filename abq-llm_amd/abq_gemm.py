@@ -39,6 +39,7 @@ EXPORTED = [
     "abq_row_sums", "abq_gemm_set_row_sums", "abq_gemm_row_sums_ready",
     "abq_tuning_load", "abq_tuning_add", "abq_tuning_clear", "abq_tuning_enable_builtin", "abq_tuning_lookup",
     "abq_preferred_weight_layout", "abq_padded_bits", "abq_relayout_planes_padded", "abq_gemm_set_value_bits",
+    "abq_gemm_set_padded_activations",
     "abq_relayout_planes_biased", "abq_gemm_set_biased_records", "abq_pack_f16_fp6",
 ]
 
@@ -152,6 +153,7 @@ def lib():
         L.abq_padded_bits.restype = ci
         L.abq_relayout_planes_padded.argtypes = [vp, vp, ci, ci, ci, ci, vp]
         L.abq_gemm_set_value_bits.argtypes = [ctypes.POINTER(GemmState), ci, ci]
+        L.abq_gemm_set_padded_activations.argtypes = [ctypes.POINTER(GemmState), ci]
         L.abq_gemm_row_sums_ready.argtypes = [ctypes.POINTER(GemmState)]
         L.abq_gemm_row_sums_ready.restype = ci
         L.abq_gemm_set_activation.argtypes = [ctypes.POINTER(GemmState), ci]
@@ -364,7 +366,7 @@ class Gemm:
     def __init__(self, x_planes, w_planes, signed, out=None, cfg=None, out_kind=OUT_I32, c_scale=None,
                  x_scale=None, w_scale=None, group_size=0, x_tiled=False, w_tiled=False, workspace=None,
                  x_zero=None, w_zero=None, x_group_sums=None, w_zero_term=None, act=ACT_NONE,
-                 x_fp6=0, w_fp6=0, x_row_sums=None, w_row_sums=None, value_bits=None, biased=None):
+                 x_fp6=0, w_fp6=0, x_row_sums=None, w_row_sums=None, value_bits=None, biased=None, x_padded_from=None):
         import torch
         if x_fp6:
             kt, M, _ = x_planes.shape
@@ -372,6 +374,9 @@ class Gemm:
         elif x_tiled:
             kt, M, q, _ = x_planes.shape
             kw = kt * 4
+            if x_padded_from is not None:  # records of padded_bits(q) bits holding codes of q = x_padded_from bits
+                assert q == padded_bits(int(x_padded_from))
+                q = int(x_padded_from)
         else:
             q, M, kw = x_planes.shape
         if w_fp6:
@@ -404,6 +409,8 @@ class Gemm:
             _check(lib().abq_gemm_set_zero_points(ctypes.byref(self.state),
                                                   *[t.data_ptr() if t is not None else None
                                                     for t in self.zero_operands]), "abq_gemm_set_zero_points")
+        if x_padded_from is not None:
+            _check(lib().abq_gemm_set_padded_activations(ctypes.byref(self.state), 1), "abq_gemm_set_padded_activations")
         if x_tiled or w_tiled or x_fp6 or w_fp6:
             xl = LAYOUT_FP6 if x_fp6 else int(x_tiled)
             wl = LAYOUT_FP6 if w_fp6 else int(w_tiled)

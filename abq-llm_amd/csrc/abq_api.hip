@@ -373,9 +373,10 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         if (v < 0)
             return ABQ_ERR_UNSUPPORTED;
         const KernelEntry &e = tdt->entries[v];
-        const int mrows = decode_tiled_rows(e.wk, e.tn, M, K, x_bits);
+        const int xq = abq_padded_bits(x_bits); // width of the activation records the kernel reads
+        const int mrows = decode_tiled_rows(e.wk, e.tn, M, K, xq);
         // byte offsets inside the kernel are 32 bits wide
-        if (mrows == 0 || K >= (1 << 17) || (size_t)N * K * w_bits / 8 >= (1ull << 32) || (size_t)M * K * x_bits / 8 >= (1ull << 32) ||
+        if (mrows == 0 || K >= (1 << 17) || (size_t)N * K * w_bits / 8 >= (1ull << 32) || (size_t)M * K * xq / 8 >= (1ull << 32) ||
             (M + mrows - 1) / mrows > 65535)
             return ABQ_ERR_TOO_LARGE;
         st->strategy = strategy;
@@ -383,7 +384,7 @@ static abq_status resolve(const abq_tile_config *cfg, int x_bits, int w_bits, in
         entry_to_config(e, strategy, x_bits, w_bits, is_signed, 0, &st->cfg);
         st->grid_dim = abq_dim3{ (unsigned)(((N + 15) / 16 + e.tn - 1) / e.tn), (unsigned)((M + mrows - 1) / mrows), 1 };
         st->block_dim = abq_dim3{ (unsigned)(64 * e.wk), 1, 1 };
-        st->shared_mem_size = decode_tiled_lds(e.wk, e.tn, mrows, K, x_bits);
+        st->shared_mem_size = decode_tiled_lds(e.wk, e.tn, mrows, K, xq);
         return ABQ_OK;
     }
 
@@ -967,8 +968,8 @@ static bool decode_tiled_pays(int x_bits, int w_bits, int M, int N, int K)
 {
     if (M <= 16)
         return true;
-    if (M > 128)
-        return false;
+    if (M > 128 || !(x_bits == 2 || x_bits == 4 || x_bits == 8) || !(w_bits == 2 || w_bits == 4 || w_bits == 8))
+        return false; // (the instances that walk several blocks of rows exist for operands of one field)
     const int mrows = decode_tiled_rows(kDecodeTiledBlocksWaves, kDecodeTiledBlocksTiles, M, K, x_bits);
     if (mrows == 0)
         return false;
@@ -996,6 +997,22 @@ static bool decode_tiled_pays(int x_bits, int w_bits, int M, int N, int K)
 // reserved[4]: bit 0 / bit 1: the K-tiled 8-bit records of X / W hold code - 128 (abq_gemm_set_biased_records)
 static bool biased_x(const abq_gemm_state *st) { return (st->reserved[4] & 1) != 0; }
 static bool biased_w(const abq_gemm_state *st) { return (st->reserved[4] & 2) != 0; }
+// reserved[4] bit 2: the K-tiled activation records are those of the next single-field width
+// (abq_relayout_planes_padded), which is how the decode kernel on prepared operands reads activations of 3, 5, 6 or
+// 7 bits (abq_gemm_set_padded_activations)
+static bool padded_x(const abq_gemm_state *st) { return (st->reserved[4] & 4) != 0; }
+static bool one_field(int bits) { return bits == 2 || bits == 4 || bits == 8; }
+// Width of the activation records the decode kernel on prepared operands reads for a pair.
+static int decode_tiled_x_bits(int x_bits) { return abq_padded_bits(x_bits); }
+// Whether that kernel can read the state's activations as they are declared: planes (converted by exec), records of
+// one field, or padded records for the widths of several fields.
+static bool decode_tiled_x_ok(const abq_gemm_state *st, int x_layout)
+{
+    if (x_layout != ABQ_LAYOUT_TILED)
+        return true; // (a declaration of padded records says nothing about planes or fp16)
+    return one_field(st->cfg.x_bits) ? true : padded_x(st);
+}
+static bool decode_tiled_x_ok(const abq_gemm_state *st) { return decode_tiled_x_ok(st, st->x_layout); }
 
 // Unsigned 8-bit records on the decode kernel of prepared operands: codes up to 255 are fed as value - 128 and need
 // the other operand's row sums (abq_gemm_set_row_sums); records declared to hold narrower codes
@@ -1015,6 +1032,8 @@ static bool decode_tiled_flips_ok(const abq_gemm_state *st)
     decode_tiled_flips(st, &fx, &fw);
     if (biased_x(st) || biased_w(st))
         return false; // biased records are read by the prefill kernel only
+    if (!decode_tiled_x_ok(st))
+        return false; // activation records of several fields: the prefill kernel reads those
     if (fx && !st->w_row_sums)
         return false;
     if (fw && !st->x_row_sums)
@@ -1046,10 +1065,24 @@ static abq_status switch_to_decode_tiled(abq_gemm_state *st, bool one_tile = fal
     // (8-bit weights keep one load in flight: W8A8 4096 x 4096 at one row 5.3 against 6.5 us, 4096 x 11008 10.2 against 11.7)
     const int want_d = row_blocks || many_rows ? 1 : tiles > 512 ? 2 : (steps > 32 && st->M <= 2 && c.w_bits < 8) ? 3 : 1;
     int pick = -1;
-    for (int i = 0; i < tdt->count; ++i) {
-        const KernelEntry &e = tdt->entries[i];
-        if (e.tn == want_t && e.wk == want_wk && e.kb == (512 / c.w_bits) * want_d)
-            pick = i;
+    if (one_field(c.w_bits)) {
+        for (int i = 0; i < tdt->count; ++i) {
+            const KernelEntry &e = tdt->entries[i];
+            if (e.tn == want_t && e.wk == want_wk && e.kb == (512 / c.w_bits) * want_d)
+                pick = i;
+        }
+    } else {
+        // weights of several fields (gemm_decode_fields; warp K of the entry = 128 x loads in flight per wave), up to 16
+        // rows.  Sixteen waves with two loads each, except 3-bit weights on outputs that give a compute unit more than
+        // two workgroups: eight waves with four (W3A3 11008 x 4096 at one row 7.9 against 8.6 us; from 5 bits up the
+        // kernel is bound by the work per field and sixteen waves stay ahead: W5A5 12.0 against 15.5, W7A7 17.7
+        // against 20.6).
+        if (row_blocks)
+            return ABQ_ERR_UNSUPPORTED;
+        const int wk = (tiles > 512 && c.w_bits == 3) ? 8 : 16, d = wk == 8 ? 4 : 2;
+        for (int i = 0; i < tdt->count; ++i)
+            if (tdt->entries[i].wk == wk && tdt->entries[i].kb == 128 * d)
+                pick = i;
     }
     if (pick < 0)
         return ABQ_ERR_UNSUPPORTED;
@@ -1460,7 +1493,8 @@ int abq_gemm_row_sums_ready(const abq_gemm_state *st)
 {
     if (!st || !st->init_success || !wants_row_sums(st))
         return 0;
-    const size_t xb = st->x_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->M, st->K, st->cfg.x_bits);
+    const int xrec = st->strategy == ABQ_STRATEGY_DECODE_TILED ? decode_tiled_x_bits(st->cfg.x_bits) : st->cfg.x_bits;
+    const size_t xb = st->x_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->M, st->K, xrec);
     const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, st->cfg.w_bits);
     return row_sum_plan(st, xb + wb).ok ? 1 : 0;
 }
@@ -1499,6 +1533,29 @@ abq_status abq_gemm_set_value_bits(abq_gemm_state *st, int x_value_bits, int w_v
     st->reserved[2] = x_value_bits;
     st->reserved[3] = w_value_bits;
     reconsider_decode_tiled(st);
+    return ABQ_OK;
+}
+
+abq_status abq_gemm_set_padded_activations(abq_gemm_state *st, int padded)
+{
+    if (!st || !st->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    if (padded && one_field(st->cfg.x_bits))
+        padded = 0; // records of one field are their own padding
+    st->reserved[4] = (st->reserved[4] & ~4) | (padded ? 4 : 0);
+    if (st->x_layout == ABQ_LAYOUT_TILED) {
+        if (padded && st->strategy != ABQ_STRATEGY_DECODE_TILED) {
+            reconsider_decode_tiled(st);
+            if (st->strategy != ABQ_STRATEGY_DECODE_TILED) {
+                st->reserved[4] &= ~4;
+                return ABQ_ERR_UNSUPPORTED; // only the decode kernel on prepared operands reads such records
+            }
+        } else if (!padded && st->strategy == ABQ_STRATEGY_DECODE_TILED && !decode_tiled_x_ok(st)) {
+            if (!st->auto_chosen)
+                return ABQ_ERR_UNSUPPORTED;
+            return st->group_size ? pick_grouped_tiled(st) : switch_to_tiled(st);
+        }
+    }
     return ABQ_OK;
 }
 
@@ -1605,10 +1662,14 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
     } else if (st->strategy == ABQ_STRATEGY_TILED || st->strategy == ABQ_STRATEGY_DECODE_TILED) {
         // operands still in the reference layout are converted into the caller's workspace
         const bool x_f16 = st->x_layout == ABQ_LAYOUT_F16; // quantised inside the decode kernel
-        const size_t xb = (st->x_layout == ABQ_LAYOUT_TILED || x_f16) ? 0 : planes_bytes(st->M, st->K, c.x_bits);
+        // (the decode kernel reads activations of 3, 5, 6 or 7 bits as records of the next single-field width)
+        const int xrec = st->strategy == ABQ_STRATEGY_DECODE_TILED ? decode_tiled_x_bits(c.x_bits) : c.x_bits;
+        const size_t xb = (st->x_layout == ABQ_LAYOUT_TILED || x_f16) ? 0 : planes_bytes(st->M, st->K, xrec);
         const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, c.w_bits);
         if (st->x_layout == ABQ_LAYOUT_FP6 || st->w_layout == ABQ_LAYOUT_FP6)
             return ABQ_ERR_NOT_INITIALIZED;
+        if (st->strategy == ABQ_STRATEGY_DECODE_TILED ? !decode_tiled_x_ok(st) : (st->x_layout == ABQ_LAYOUT_TILED && padded_x(st)))
+            return ABQ_ERR_INVALID_ARG; // records of the width this kernel does not read
         if (x_f16 && (st->strategy != ABQ_STRATEGY_DECODE_TILED ||
                       (x_dynamic ? st->group_size != 128 || (st->reserved[1] == 2 && !st->w_zero_term)
                                  : st->group_size != 0 || !st->x_pack_scale)))
@@ -1625,8 +1686,8 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
         if (!biased && biased_x(st))
             return ABQ_ERR_INVALID_ARG; // biased activations only make sense against biased weights
         if (xb) {
-            e = launch_relayout_planes_padded(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, c.x_bits, c.x_bits, biased ? 2 : 0,
-                                              (hipStream_t)stream);
+            e = launch_relayout_planes_padded(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, xrec, c.x_bits,
+                                              biased ? 2 : (xrec != c.x_bits && c.is_signed ? 1 : 0), (hipStream_t)stream);
             if (e != hipSuccess)
                 return hip_status(e);
             a.X = reinterpret_cast<const uint32_t *>(ws);
@@ -1802,7 +1863,8 @@ size_t abq_gemm_workspace_bytes(const abq_gemm_state *st)
         return (st->x_layout == ABQ_LAYOUT_FP6 ? 0 : fp6_bytes(st->M, st->K)) +
                (st->w_layout == ABQ_LAYOUT_FP6 ? 0 : fp6_bytes(st->N, st->K));
     // (fp16 activations are quantised inside the decode kernel: nothing is converted for them)
-    const size_t xb = (st->x_layout == ABQ_LAYOUT_TILED || st->x_layout == ABQ_LAYOUT_F16) ? 0 : planes_bytes(st->M, st->K, st->cfg.x_bits);
+    const int xrec = st->strategy == ABQ_STRATEGY_DECODE_TILED ? decode_tiled_x_bits(st->cfg.x_bits) : st->cfg.x_bits;
+    const size_t xb = (st->x_layout == ABQ_LAYOUT_TILED || st->x_layout == ABQ_LAYOUT_F16) ? 0 : planes_bytes(st->M, st->K, xrec);
     const size_t wb = st->w_layout == ABQ_LAYOUT_TILED ? 0 : planes_bytes(st->N, st->K, st->cfg.w_bits);
     // (pairs with an unsigned 8-bit operand on the staged kernel: the row sums of the operands still in planes)
     return xb + wb + (wants_row_sums(st) ? row_sum_plan(st, xb + wb).bytes : 0);
@@ -1845,7 +1907,15 @@ static abq_status set_operand_layout_by_rules(abq_gemm_state *st, int x_layout, 
     }
     // decode-sized M (and up to 128 rows where it pays) with both operands prepared: the decode kernel of that layout
     // (plain and per-channel epilogues)
-    if (x_layout == ABQ_LAYOUT_TILED && w_layout == ABQ_LAYOUT_TILED && st->auto_chosen &&
+    if (st->strategy == ABQ_STRATEGY_DECODE_TILED && !decode_tiled_x_ok(st, x_layout)) {
+        // activation records of several fields: the prefill kernel reads those
+        if (!st->auto_chosen)
+            return ABQ_ERR_UNSUPPORTED;
+        const abq_status rc = st->group_size ? pick_grouped_tiled(st) : switch_to_tiled(st);
+        if (rc != ABQ_OK)
+            return rc;
+    }
+    if (x_layout == ABQ_LAYOUT_TILED && w_layout == ABQ_LAYOUT_TILED && st->auto_chosen && decode_tiled_x_ok(st, x_layout) &&
         decode_tiled_pays(st->cfg.x_bits, st->cfg.w_bits, st->M, st->N, st->K) && !st->group_size &&
         !st->act && st->strategy != ABQ_STRATEGY_DECODE_TILED && switch_to_decode_tiled(st) == ABQ_OK) {
         st->x_layout = x_layout;

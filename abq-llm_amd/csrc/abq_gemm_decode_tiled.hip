@@ -29,7 +29,10 @@
 //   * per-wave partial tiles meet in LDS and are summed by the threads that store them (integer adds:
 //     any order gives the same bits).
 // K longer than NW * D steps runs further rounds of the same loop (their latency is exposed).
+#include <type_traits>
+
 #include "abq_kernels.h"
+#include "abq_bits.h"
 #include "abq_quant.h"
 
 #ifndef ABQ_Q
@@ -384,6 +387,244 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled(const GemmArgs a, i
             store_result(a, m0 + (rem >> 4), n, v);
         }
     }
+}
+
+// ---- weights of several fields ------------------------------------------------------------------
+//
+// Widths of 3, 5, 6 and 7 bits are records of a 4-bit, a 2-bit and a 1-bit field (abq_bits.h: a row's K tile is
+// P * 16 bytes, the field of width F the F units of 16 bytes at byte 16 * (P & ~(2F - 1))).  Inside its region a
+// field is laid out exactly as a single-field record of that width, so the plan above carries over field by field:
+// a step of field F is one 16-byte load per lane, lane group g taking unit 4 cs + g of the field's units along K
+// (K tile (4 cs + g) / F, unit (4 cs + g) % F of it), 8 / F MFMAs against the 128 / F activations the unit covers.
+// A field is fed at the place its bits have in the code (signed: in the code moved to the top of the byte, so that
+// the widest field carries the sign and the others are non-negative), all fields into one accumulator: the sum is
+// the dot product times 2^(16 - QP - P) as for a single field.  The steps of all fields form one list (4-bit
+// field first), wave w takes steps w, w + NW, ...; which field a step belongs to is the same for the whole wave.
+// The weights are the records the prefill kernels read (abq_relayout_planes): one copy serves both.  The
+// activations are records of a single field of QP bits: their own width, or for 3, 5, 6 and 7 bits the next such
+// width with the codes extended (abq_relayout_planes_padded); activation bytes are small at decode.
+template <int F, int POS, bool TOP> __device__ __forceinline__ void dt_unpack_field(const v4u &u, v4i (&out)[8 / F])
+{
+    // word j of the unit carries in byte c, at bits [F s, F s + F), the field of expanded dword (8 / F) j + s;
+    // operand i = expanded dwords 4 i .. 4 i + 3.  The field goes to bits [POS, POS + F) of the byte.
+    constexpr uint32_t mask = field_mask(F) << POS;
+    constexpr int per = 8 / F; // expanded dwords per word
+#pragma unroll
+    for (int i = 0; i < 8 / F; ++i)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int d = 4 * i + c, j = d / per, sft = POS - F * (d % per);
+            const uint32_t w = u[j];
+            out[i][c] = (int)((sft >= 0 ? w << (sft >= 0 ? sft : 0) : w >> (sft < 0 ? -sft : 0)) & mask);
+        }
+    (void)TOP;
+}
+
+constexpr int dt_field_steps(int kt, int p, int f) { return (p & f) ? (kt * f + 3) / 4 : 0; }
+
+template <int QP, int P, bool SIGNED, int NW, int D, bool FLIP_X = false>
+__global__ __launch_bounds__(64 * NW) void gemm_decode_fields(const GemmArgs a, int mrows)
+{
+    static_assert(QP == 4 || QP == 8, "activations as records of one field");
+    static_assert(P == 3 || P == 5 || P == 6 || P == 7, "weights of several fields");
+    static_assert(!FLIP_X || (!SIGNED && QP == 8), "flipping is for unsigned 8-bit records");
+    constexpr int MX = 8 / QP; // MFMAs per activation chunk
+    constexpr int NT = 64 * NW;
+    constexpr int QLOG = QP == 8 ? 3 : 2;
+    constexpr int XC = 6;
+    constexpr int WPOS = SIGNED ? 8 - P : 0; // place of the code's lowest bit in the byte
+    extern __shared__ __align__(16) unsigned char smem[];
+    int *red = reinterpret_cast<int *>(smem); // [NW][16][16]
+    unsigned char *xs = smem + NW * 1024;     // [kt][row][QP chunks], chunks permuted within a row
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int M = a.M, N = a.N;
+    const int KT = a.K >> 7;
+    const int S4 = dt_field_steps(KT, P, 4), S2 = dt_field_steps(KT, P, 2), S1 = dt_field_steps(KT, P, 1);
+    const int S = S4 + S2 + S1;
+    const int tile0 = blockIdx.x;
+    const int m0 = blockIdx.y * mrows;
+    const int once = gridDim.y == 1;
+    const int Mb = min(mrows, M - m0);
+    const char *Xt = reinterpret_cast<const char *>(a.X);
+    const char *Wt = reinterpret_cast<const char *>(a.W);
+    const unsigned xs_addr = (unsigned)(size_t)xs;
+    const int xchunks = KT * Mb * QP;
+
+    // ---- activations: as in gemm_decode_tiled ---------------------------------------------------------
+    if (Mb == M) {
+#pragma unroll
+        for (int i = 0; i < XC; ++i) {
+            const int pb = wid * 64 + i * NT;
+            if (pb < xchunks) {
+                const int p = pb + lane;
+                const int src = min(p ^ ((p >> QLOG) & (QP - 1)), xchunks - 1);
+                dt_load_to_lds(Xt + (uint32_t)src * 16u, xs_addr + (unsigned)pb * 16u);
+            }
+        }
+        for (int pb = wid * 64 + XC * NT; pb < xchunks; pb += NT) {
+            const int p = pb + lane;
+            const int src = min(p ^ ((p >> QLOG) & (QP - 1)), xchunks - 1);
+            dt_load_to_lds(Xt + (uint32_t)src * 16u, xs_addr + (unsigned)pb * 16u);
+        }
+    } else {
+        const int per = Mb * QP;
+        for (int pb = wid * 64; pb < xchunks; pb += NT) {
+            const int p = min(pb + lane, xchunks - 1);
+            const int q = p ^ ((p >> QLOG) & (QP - 1));
+            const int kt = q / per, rem = q - kt * per;
+            dt_load_to_lds(Xt + ((size_t)(kt * M + m0) * QP + rem) * 16u, xs_addr + (unsigned)pb * 16u);
+        }
+    }
+
+    // ---- weights: byte offset of (lane, field F, step cs) = K tile * tile_bytes + row_off + field_off[F] ----
+    const uint32_t tile_bytes = (uint32_t)N * (P * 16u);
+    const uint32_t row_off = (uint32_t)min(tile0 * 16 + r, N - 1) * (P * 16u);
+    // flat step t -> field (4: t < S4; 2: t < S4 + S2; else 1) and the field's own step; wave-uniform
+    auto weight_offset = [&](int t) -> uint32_t {
+        int kt;
+        uint32_t fo;
+        if (t < S4) {
+            kt = t;
+            fo = 16u * field_list_index(P, 4) + 16u * g;
+        } else if (t < S4 + S2) {
+            kt = 2 * (t - S4) + (g >> 1);
+            fo = 16u * field_list_index(P, 2) + 16u * (g & 1);
+        } else {
+            kt = 4 * (t - S4 - S2) + g;
+            fo = 16u * field_list_index(P, 1);
+        }
+        return (uint32_t)min(kt, KT - 1) * tile_bytes + row_off + fo; // lanes past the end of K repeat the last K tile
+    };
+
+    v4i acc[2];
+    acc[0] = acc[1] = v4i{ 0, 0, 0, 0 };
+    const int ml = min(r, Mb - 1);
+
+    // the activations of the unit (field F, step cs) of this lane group -> 8 / F MFMA operands
+    auto read_x = [&](auto fc, int cs, v4i(&av)[8]) {
+        constexpr int F = decltype(fc)::value;
+        constexpr int NXL = QP >= F ? QP / F : 1; // activation chunks per weight unit
+        const int uu = min(4 * cs + g, KT * F - 1);
+        const int u0 = uu * NXL;
+        const int rowi = (u0 >> QLOG) * Mb + ml;
+#pragma unroll
+        for (int i = 0; i < NXL; ++i) {
+            const int part = ((u0 + i) & (QP - 1)) ^ (rowi & (QP - 1));
+            const v4u xv = *reinterpret_cast<const v4u *>(xs + ((uint32_t)rowi * QP + part) * 16u);
+            v4i tt[MX];
+            dt_unpack<QP, SIGNED>(xv, tt);
+            if constexpr (FLIP_X)
+                tt[0] = v4i{ tt[0][0] ^ (int)0x80808080u, tt[0][1] ^ (int)0x80808080u, tt[0][2] ^ (int)0x80808080u,
+                             tt[0][3] ^ (int)0x80808080u };
+#pragma unroll
+            for (int k = 0; k < MX; ++k)
+                av[i * MX + k] = tt[k];
+        }
+    };
+    auto multiply = [&](auto fc, int cs, const v4u &wraw, const v4i(&av)[8]) {
+        constexpr int F = decltype(fc)::value;
+        const bool ok = 4 * cs + g < KT * F;
+        const v4u wv = ok ? wraw : v4u{ 0u, 0u, 0u, 0u };
+        v4i bv[8 / F];
+        dt_unpack_field<F, WPOS + field_base(P, F), SIGNED>(wv, bv);
+#pragma unroll
+        for (int i = 0; i < 8 / F; ++i)
+            acc[i & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[i], bv[i], acc[i & 1], 0, 0, 0);
+    };
+
+    int round = 0;
+    do {
+        v4u wb[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int t = min(wid + (round * D + d) * NW, S - 1);
+            wb[d] = dt_load16_weights(Wt, weight_offset(t), once);
+        }
+        if (round == 0) {
+            dt_wait_loads<D>(); // the activation loads are older than these
+            __syncthreads();
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int t = wid + (round * D + d) * NW;
+            const bool have = t < S; // wave-uniform
+            v4i av[8];
+            if (have) {
+                if ((P & 4) && t < S4)
+                    read_x(std::integral_constant<int, 4>{}, t, av);
+                else if ((P & 2) && t < S4 + S2)
+                    read_x(std::integral_constant<int, 2>{}, t - S4, av);
+                else if (P & 1)
+                    read_x(std::integral_constant<int, 1>{}, t - S4 - S2, av);
+            }
+            dt_wait_loads_n(D - 1 - d);
+            dt_landed(wb[d]);
+            if (have) {
+                if ((P & 4) && t < S4)
+                    multiply(std::integral_constant<int, 4>{}, t, wb[d], av);
+                else if ((P & 2) && t < S4 + S2)
+                    multiply(std::integral_constant<int, 2>{}, t - S4, wb[d], av);
+                else if (P & 1)
+                    multiply(std::integral_constant<int, 1>{}, t - S4 - S2, wb[d], av);
+            }
+        }
+        ++round;
+    } while (wid + round * D * NW < S);
+
+    // ---- the waves' partial tiles meet in LDS ----------------------------------------------------------
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        if (4 * g + e < Mb)
+            red[(wid * 16 + 4 * g + e) * 16 + r] = acc[0][e] + acc[1][e];
+    __syncthreads();
+    for (int o = tid; o < 256; o += NT) {
+        const int n = tile0 * 16 + (o & 15);
+        if ((o >> 4) < Mb && n < N) {
+            int part[NW];
+#pragma unroll
+            for (int w = 0; w < NW; ++w)
+                part[w] = red[w * 256 + o];
+            int v = 0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w)
+                v += part[w];
+            if (SIGNED)
+                v >>= 16 - QP - P;
+            if constexpr (FLIP_X)
+                v = (int)((unsigned)v + 128u * (unsigned)a.w_row_sums[n]);
+            store_result(a, m0 + (o >> 4), n, v);
+        }
+    }
+}
+
+template <int QP, int P, bool SIGNED, int NW, int D, bool MAY_FLIP>
+static hipError_t launch_decode_fields(const GemmArgs &a, hipStream_t stream)
+{
+    const int mrows = decode_tiled_rows(NW, 1, a.M, a.K, QP);
+    if (mrows == 0 || (size_t)a.N * a.K * P / 8 >= (1ull << 32) || (size_t)a.M * a.K * QP / 8 >= (1ull << 32))
+        return hipErrorInvalidValue;
+    const size_t lds = decode_tiled_lds(NW, 1, mrows, a.K, QP);
+    const int tiles = (a.N + 15) / 16;
+    const dim3 grid(tiles, (a.M + mrows - 1) / mrows);
+    auto go = [&](auto kernel) -> hipError_t {
+        const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (attr != hipSuccess)
+            return attr;
+        hipLaunchKernelGGL(kernel, grid, dim3(64 * NW), lds, stream, a, mrows);
+        return hipGetLastError();
+    };
+    if constexpr (!SIGNED && QP == 8 && MAY_FLIP) {
+        if (a.flip_x) { // true 8-bit codes (fed as value - 128); padded narrower codes go as they are
+            if (!a.w_row_sums)
+                return hipErrorInvalidValue;
+            return go(&gemm_decode_fields<QP, P, SIGNED, NW, D, true>);
+        }
+    }
+    return go(&gemm_decode_fields<QP, P, SIGNED, NW, D, false>);
 }
 
 template <int Q, int P, bool SIGNED, int NW, int D, int T, int XU, bool FLIP = false>
@@ -945,7 +1186,12 @@ template <int Q, int P, bool SIGNED, bool XDYN = false> static hipError_t launch
 #define ABQ_DT_ENTRY_T(NW, D, T) { 16, 1, T, 1, 1, NW, 6, &launch_decode_tiled<ABQ_Q, ABQ_P, true, NW, D, T>, (512 / ABQ_P) * D },
 #define ABQ_DT_ENTRY_F(NW, D, T) { 16, 1, T, 1, 1, NW, 6, &launch_decode_tiled<ABQ_Q, ABQ_P, false, NW, D, T>, (512 / ABQ_P) * D },
 
-#if (ABQ_Q == 2 || ABQ_Q == 4 || ABQ_Q == 8) && (ABQ_P == 2 || ABQ_P == 4 || ABQ_P == 8)
+// activations of 3, 5, 6 or 7 bits reach these kernels as records of the next single-field width
+#define ABQ_QP (ABQ_Q == 3 ? 4 : (ABQ_Q >= 5 && ABQ_Q <= 7) ? 8 : ABQ_Q)
+#define ABQ_P_ONE_FIELD (ABQ_P == 2 || ABQ_P == 4 || ABQ_P == 8)
+#define ABQ_Q_ONE_FIELD (ABQ_Q == 2 || ABQ_Q == 4 || ABQ_Q == 8)
+
+#if ABQ_Q_ONE_FIELD && ABQ_P_ONE_FIELD
 static const KernelEntry kSigned[] = { ABQ_DT_VARIANTS(ABQ_DT_ENTRY_T) };
 // the single-tile instances with in-kernel quantisation of fp16 activations (8-bit activations, signed), same order
 #if ABQ_Q == 8
@@ -975,16 +1221,28 @@ static const KernelEntry kUnsigned[] = { ABQ_DT_VARIANTS(ABQ_DT_ENTRY_F) };
 #define ABQ_DT_NUNSIGNED ((int)(sizeof(kUnsigned) / sizeof(kUnsigned[0])))
 #define ABQ_DT_NSIGNED ((int)(sizeof(kSigned) / sizeof(kSigned[0])))
 #else
-static const KernelEntry *const kSigned = nullptr;
-static const KernelEntry *const kUnsigned = nullptr;
 static const KernelEntry *const kSignedGrouped = nullptr;
 static const KernelEntry *const kUnsignedGrouped = nullptr;
 static const KernelEntry *const kSignedGroupedDyn = nullptr;
 #define ABQ_DT_NDYN 0
 static const KernelEntry *const kSignedF16 = nullptr;
 #define ABQ_DT_NF16 0
-#define ABQ_DT_NSIGNED 0
-#define ABQ_DT_NUNSIGNED 0
+#if ABQ_P_ONE_FIELD
+// activations of several fields over weights of one (W2A6): the kernel above on activation records padded to ABQ_QP bits
+#define ABQ_DT_ENTRY_PT(NW, D, T) { 16, 1, T, 1, 1, NW, 6, &launch_decode_tiled<ABQ_QP, ABQ_P, true, NW, D, T>, (512 / ABQ_P) * D },
+#define ABQ_DT_ENTRY_PF(NW, D, T) { 16, 1, T, 1, 1, NW, 6, &launch_decode_tiled<ABQ_QP, ABQ_P, false, NW, D, T>, (512 / ABQ_P) * D },
+static const KernelEntry kSigned[] = { ABQ_DT_VARIANTS(ABQ_DT_ENTRY_PT) };
+static const KernelEntry kUnsigned[] = { ABQ_DT_VARIANTS(ABQ_DT_ENTRY_PF) };
+#else
+// weights of several fields: (waves, weight loads in flight per wave); warp K in the tile's name = 128 D
+#define ABQ_DF_VARIANTS(V) V(16, 2) V(16, 4) V(8, 4)
+#define ABQ_DF_ENTRY_T(NW, D) { 16, 1, 1, 1, 1, NW, 6, &launch_decode_fields<ABQ_QP, ABQ_P, true, NW, D, false>, 128 * D },
+#define ABQ_DF_ENTRY_F(NW, D) { 16, 1, 1, 1, 1, NW, 6, &launch_decode_fields<ABQ_QP, ABQ_P, false, NW, D, ABQ_Q == 8>, 128 * D },
+static const KernelEntry kSigned[] = { ABQ_DF_VARIANTS(ABQ_DF_ENTRY_T) };
+static const KernelEntry kUnsigned[] = { ABQ_DF_VARIANTS(ABQ_DF_ENTRY_F) };
+#endif
+#define ABQ_DT_NUNSIGNED ((int)(sizeof(kUnsigned) / sizeof(kUnsigned[0])))
+#define ABQ_DT_NSIGNED ((int)(sizeof(kSigned) / sizeof(kSigned[0])))
 #endif
 
 #define ABQ_CAT_(a, b, c, d) a##b##c##d

@@ -227,16 +227,21 @@ std::vector<Tile> enumerate_gfx950(int x_bits, int w_bits, bool is_signed)
         for (const auto &t : fp6)
             out.push_back(Tile{ 32 * t[0] * t[2], 32 * t[1] * t[3], 128, 32 * t[0], 32 * t[1], 128, 32, 32, 64, t[2], t[3], { 5 } });
     }
-    // Decode kernel on K-tiled operands (NSTAGE = 6): single-field widths (unsigned 8-bit codes with their row sums
-    // handed in; other widths run it as padded records under the padded pair's tuples);
-    // { waves, weight loads in flight per wave, 16-row tiles per workgroup }; a load covers 512 / W_BITS elements of K
+    // Decode kernel on K-tiled operands (NSTAGE = 6).  Weights of one field (2, 4, 8 bits; activations of several
+    // fields reach it as records of the next single-field width): { waves, weight loads in flight per wave, 16-row
+    // tiles per workgroup }, a load covers 512 / W_BITS elements of K.  Weights of several fields (3, 5, 6, 7 bits,
+    // read field by field): { waves, loads in flight }, warp K in the name = 128 x loads.
     {
-        const bool field = (x_bits == 2 || x_bits == 4 || x_bits == 8) && (w_bits == 2 || w_bits == 4 || w_bits == 8);
-        if (field && x_bits >= w_bits) {
+        const bool w_field = w_bits == 2 || w_bits == 4 || w_bits == 8;
+        if (w_field && x_bits >= w_bits) {
             const int dt[][3] = { { 16, 1, 1 }, { 16, 3, 1 }, { 8, 2, 1 }, { 16, 1, 3 }, { 8, 1, 2 }, { 8, 2, 2 }, { 16, 1, 2 } };
             const int stepk = 512 / w_bits;
             for (const auto &v : dt)
                 out.push_back(Tile{ 16, 16 * v[2], stepk * v[1] * v[0], 16, 16 * v[2], stepk * v[1], 16, 16, 64, 1, v[0], { 6 } });
+        } else if (!w_field && x_bits >= w_bits) {
+            const int df[][2] = { { 16, 2 }, { 16, 4 }, { 8, 4 } };
+            for (const auto &v : df)
+                out.push_back(Tile{ 16, 16, 128 * v[1] * v[0], 16, 16, 128 * v[1], 16, 16, 64, 1, v[0], { 6 } });
         }
     }
     return out;

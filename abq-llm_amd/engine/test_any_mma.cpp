@@ -489,9 +489,10 @@ int main(int argc, char **argv)
         HIP_OK(hipStreamSynchronize(stream));
     }
 
-    // Decode-sized M: the "prepared operands" line of the widths made of several fields (3, 5, 6, 7 bits) runs on padded
-    // records (abq_relayout_planes_padded: the next width of 2, 4 or 8 bits), and unsigned 8-bit codes bring their row
-    // sums (abq_row_sums), which is how the decode kernel of prepared operands serves those pairs.
+    // Decode-sized M, prepared operands.  Weights of several fields (3, 5, 6, 7 bits) are read by the decode kernel as
+    // the records above; activations of such widths come as padded records (abq_relayout_planes_padded: the next width
+    // of 2, 4 or 8 bits), and unsigned 8-bit codes bring their row sums (abq_row_sums).  A second "prepared operands"
+    // line times the same pairs with the weights padded as well (the padded pair's kernel).
     const int xq = abq_padded_bits(x_bits), wq = abq_padded_bits(w_bits);
     const bool padded = xq != x_bits || wq != w_bits;
     const bool with_sums = !is_signed && (x_bits == 8 || w_bits == 8);
@@ -556,7 +557,8 @@ int main(int argc, char **argv)
     // K-tiled too, as the quantising kernel writes them (what that tile's own line of the sweep is timed on)
     abq_tile_config tuned;
     const bool tuned_decode = M > 16 && abq_tuning_lookup(x_bits, w_bits, is_signed, M, N, K, 0, 0, &tuned, nullptr) == ABQ_OK && tuned.nstage == 6;
-    auto run_one = [&](const abq_tile_config *cfg, Timing &t, abq_gemm_state &st0, bool prepared = false) {
+    const bool x_fields = xq != x_bits; // activations the decode kernel reads as padded records
+    auto run_one = [&](const abq_tile_config *cfg, Timing &t, abq_gemm_state &st0, bool prepared = false, bool pad_weights = false) {
         std::vector<abq_gemm_state> states(nbuf);
         // tiled tiles (NSTAGE 4) run on prepared weights, NSTAGE 6 and the `prepared` default on prepared weights and
         // activations, the FP6 tiles on FP6 records; the library's own choice for M > 16 on the preferred layout
@@ -567,20 +569,26 @@ int main(int argc, char **argv)
             t.status = -1;
             return;
         }
-        // (the prepared default of pairs the decode kernel serves through padded records or row sums)
-        const bool via_padded = prepared && d_wpad != nullptr;
+        // (the prepared default with the weights as padded records too: the padded pair's kernel)
+        const bool via_padded = prepared && pad_weights && d_wpad != nullptr;
         if (via_padded)
             states.resize(nbuf_pad);
+        if (both && (x_fields || with_sums) && !d_xpad) { // more than 16 rows: no padded activations were made
+            t.status = -1;
+            return;
+        }
         for (size_t b = 0; b < states.size(); ++b) {
             const char *wbase = via_padded ? (const char *)d_wpad + b * wpad_bytes
                                 : fp6      ? (const char *)d_wf + b * wf_bytes
                                            : (tiled ? (const char *)d_wt : (const char *)d_wp) + b * wp_bytes;
             abq_status s = abq_gemm_init(cfg, via_padded ? xq : x_bits, via_padded ? wq : w_bits, is_signed,
-                                         via_padded ? d_xpad : both ? d_xt : d_xp, (const uint32_t *)wbase,
+                                         via_padded ? d_xpad : both ? (x_fields ? d_xpad : d_xt) : d_xp, (const uint32_t *)wbase,
                                          M, N, K, d_out, nullptr, 0, ABQ_OUT_I32, &states[b]);
             if (s == ABQ_OK && via_padded && padded)
                 s = abq_gemm_set_value_bits(&states[b], x_bits, w_bits);
-            if (s == ABQ_OK && via_padded && with_sums)
+            if (s == ABQ_OK && both && !via_padded && x_fields)
+                s = abq_gemm_set_padded_activations(&states[b], 1);
+            if (s == ABQ_OK && both && with_sums)
                 s = abq_gemm_set_row_sums(&states[b], d_xsum, d_wsum);
             if (s == ABQ_OK && tiled)
                 s = abq_gemm_set_operand_layout(&states[b], both ? ABQ_LAYOUT_TILED : ABQ_LAYOUT_PLANES, ABQ_LAYOUT_TILED);
@@ -639,16 +647,18 @@ int main(int argc, char **argv)
     double layout_tops[3] = { 0, 0, 0 };
     abq_tile_config layout_best[3];
     const int ncfg = abq_native_config_count(x_bits, w_bits, is_signed);
-    const int nlines = ncfg + (M <= 16 ? 2 : 1); // + the library's choice (+ its choice on prepared operands)
+    // + the library's choice (+ its choice on prepared operands (+ the same with the weights padded as well))
+    const int nlines = ncfg + (M <= 16 ? (padded && wq != w_bits ? 3 : 2) : 1);
     for (int i = 0; i < nlines; ++i) {
         abq_tile_config cfg;
         const bool library_default = i >= ncfg;
-        const bool prepared = i == ncfg + 1;
+        const bool prepared = i >= ncfg + 1, pad_weights = i == ncfg + 2;
         if (!library_default && abq_native_config_get(x_bits, w_bits, is_signed, i, &cfg) != ABQ_OK)
             continue;
         char name[160] = "library default";
+        const char *how = pad_weights ? " (padded records)" : (with_sums && d_wpad) ? " (with row sums)" : "";
         if (prepared)
-            std::snprintf(name, sizeof name, "library default, prepared operands%s", d_wpad ? (padded ? " (padded records)" : " (with row sums)") : "");
+            std::snprintf(name, sizeof name, "library default, prepared operands%s", how);
         if (!library_default)
             abq_format_kernel_name(&cfg, 0, name, sizeof name);
         if (!only.empty() && std::string(name).find(only) == std::string::npos)
@@ -656,7 +666,7 @@ int main(int argc, char **argv)
         Timing t;
         abq_gemm_state st;
         std::memset(&st, 0, sizeof st);
-        run_one(library_default ? nullptr : &cfg, t, st, prepared);
+        run_one(library_default ? nullptr : &cfg, t, st, prepared, pad_weights);
         const abq_tile_config &c = st.cfg;
         const double tops = t.status == 0 ? ops / (t.exec_us * 1e-6) / 1e12 : 0;
         std::printf("gfx950 %s %d %d %d %d %d %d %d %d %d %d ", config_str, c.block_m, c.block_n, c.block_k, c.warp_m,
@@ -664,8 +674,9 @@ int main(int argc, char **argv)
         std::printf("packing %f (us) exec %f (us) %f TOPS | %f B-TOPS | %s | %.1f%% HBM %.1f%% MFMA%s\n", t.pack_us,
                     t.exec_us, tops, tops * x_bits * w_bits, t.status == 0 ? "PASSED" : t.status == -1 ? "ERROR" : "FAILED",
                     t.status == 0 ? 100.0 * alg_bytes / (t.exec_us * 1e-6) / 8e12 : 0.0, 100.0 * tops / 5000.0,
-                    prepared ? (d_wpad ? (padded ? " | library default, prepared operands (padded records)" : " | library default, prepared operands (with row sums)")
-                                       : " | library default, prepared operands")
+                    prepared ? (pad_weights ? " | library default, prepared operands (padded records)"
+                                : (with_sums && d_wpad) ? " | library default, prepared operands (with row sums)"
+                                                        : " | library default, prepared operands")
                              : library_default ? " | library default" : "");
         if (t.status == 0 && !library_default && tops > best_tops) {
             best_tops = tops;

@@ -180,8 +180,8 @@ typedef struct abq_gemm_state {
     const float *w_scale;  /* [N] or [N][K/group_size] */
     int group_size;        /* 0 = per channel          */
     int reserved[5];       /* [0] popcount kernels: log2 of the lanes per weight row; [1] see
-                              abq_gemm_set_dynamic_f16_activations; [2], [3] see abq_gemm_set_value_bits; [4] see
-                              abq_gemm_set_biased_records */
+                              abq_gemm_set_dynamic_f16_activations; [2], [3] see abq_gemm_set_value_bits; [4] bits 0, 1 see
+                              abq_gemm_set_biased_records, bit 2 abq_gemm_set_padded_activations */
     /* K-tiled operands (ABQ_STRATEGY_TILED) */
     int x_layout, w_layout;  /* abq_layout of X and W as handed to init                    */
     int auto_chosen;         /* 1 if the tile was the library's choice                     */
@@ -442,6 +442,16 @@ abq_status abq_relayout_planes_padded(const uint32_t *planes, uint32_t *tiled, i
 /* Declares that the codes of X (W) use only the low x_value_bits (w_value_bits) of their fields (1 .. the state's
  * widths): see above. */
 abq_status abq_gemm_set_value_bits(abq_gemm_state *state, int x_value_bits, int w_value_bits);
+/* Weights of 3, 5, 6 or 7 bits need no padded copy for decode: the decode kernel on prepared operands reads the
+ * records abq_relayout_planes writes (the ones the prefill kernels read), field by field.  Its activations are records
+ * of one field; a state whose ACTIVATIONS are 3, 5, 6 or 7 bits wide therefore takes them as padded records
+ * (abq_relayout_planes_padded, abq_planes_bytes(M, k, abq_padded_bits(x_bits)) bytes), declared ABQ_LAYOUT_TILED and
+ * marked with this call (before or after abq_gemm_set_operand_layout; activations handed over as planes are converted
+ * that way by abq_gemm_exec itself, abq_gemm_workspace_bytes counts the padded size).  The state is initialised with
+ * the pair's own widths.  Up to 16 rows; ABQ_ERR_UNSUPPORTED where only the prefill kernel could run, which reads
+ * records of the activations' own width.  No effect for activations of 2, 4 or 8 bits.  No counterpart in the
+ * reference (its decode sweep over these widths: engine/test.sh:8-206). */
+abq_status abq_gemm_set_padded_activations(abq_gemm_state *state, int padded);
 
 /* Workspace needed by abq_gemm_exec if the state ran as ABQ_STRATEGY_TILED, ABQ_STRATEGY_DECODE_TILED
  * (ABQ_STRATEGY_FP6) with its current operand layouts: the converted copies of the operands still in

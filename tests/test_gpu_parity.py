@@ -586,6 +586,75 @@ def test_decode_on_prepared_operands(abq, oracle, q, p, signed):
             assert e.value.status == abq.ABQ_ERR_INVALID_ARG
 
 
+FIELD_PAIRS = [(3, 3), (5, 5), (6, 6), (7, 7), (8, 3), (6, 2)]  # a width of several fields on either side
+
+
+@pytest.mark.parametrize("q,p", FIELD_PAIRS)
+@pytest.mark.parametrize("signed", [True, False])
+def test_decode_on_prepared_operands_of_several_fields(abq, oracle, q, p, signed):
+    """Weights of 3, 5, 6 or 7 bits on the decode kernel as the records the prefill kernels read (no padded copy), the
+    state initialised with the pair's own widths; activations of such widths as padded records, declared so, or as
+    planes, which exec converts.  Every tile tuple of the kernel on ragged shapes (partial tiles of N, numbers of K
+    tiles that leave the last step of the 2-bit and of the 1-bit field partly empty, long K), the rows of the largest
+    codes against the code furthest from zero, unsigned 8-bit activations with the weights' row sums."""
+    qp = abq.padded_bits(q)
+    rng = np.random.default_rng(900 + 10 * q + p + int(signed))
+    shapes = [(1, 64, 128), (1, 4096, 4096), (3, 37, 384), (4, 200, 1408), (8, 130, 1152), (8, 64, 11008), (13, 72, 4096),
+              (16, 100, 13824), (16, 48, 2048), (2, 300, 24576), (5, 16, 640), (7, 1000, 896)]
+    for (M, N, K) in shapes:
+        x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+        if M > 1:
+            x[1] = (1 << (q - 1)) - 1 if signed else (1 << q) - 1
+            w[0] = -(1 << (p - 1)) if signed else (1 << p) - 1
+        xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
+        wt = abq.relayout_planes(wd)                      # the weights' own records
+        xt = abq.relayout_planes_padded(xd, signed)       # activations: records of one field
+        assert wt.shape == (K // 128, N, p, 4) and xt.shape == (K // 128, M, qp, 4)
+        want = oracle.np_gemm(x, w)
+        kw = dict(x_tiled=True, w_tiled=True)
+        if qp != q:
+            kw["x_padded_from"] = q
+        needs_sums = not signed and q == 8
+        if needs_sums:
+            g = abq.Gemm(xt, wt, signed, **kw)  # no sums: the prefill kernel, which takes them itself
+            assert g.strategy == "tiled"
+            assert np.array_equal(g.run().cpu().numpy(), want), (g.config_name, M, N, K)
+            kw["w_row_sums"] = abq.row_sums(wd)
+        g = abq.Gemm(xt, wt, signed, **kw)
+        assert (g.state.cfg.x_bits, g.state.cfg.w_bits) == (q, p)
+        assert g.strategy == "decode_tiled" and g.workspace_bytes == 0, (g.strategy, M, N, K)
+        assert np.array_equal(g.run().cpu().numpy(), want), (g.config_name, M, N, K)
+        ran = 0
+        for cfg in abq.native_configs(q, p, signed):
+            if cfg.nstage != 6:
+                continue
+            out = torch.full((M, N), -12345, dtype=torch.int32, device="cuda")
+            got = abq.Gemm(xt, wt, signed, cfg=cfg, out=out, **kw).run().cpu().numpy()
+            assert np.array_equal(got, want), (abq.format_kernel_name(cfg), M, N, K)
+            ran += 1
+        assert ran == (7 if p == 2 else 3)
+        # activations handed over as planes: exec writes the padded records into the workspace
+        cfg = [c for c in abq.native_configs(q, p, signed) if c.nstage == 6][0]
+        sums = {"w_row_sums": kw["w_row_sums"]} if needs_sums else {}
+        g = abq.Gemm(xd, wt, signed, cfg=cfg, w_tiled=True, **sums)
+        assert g.workspace_bytes == xt.numel() * 4
+        g = abq.Gemm(xd, wt, signed, cfg=cfg, w_tiled=True, workspace=torch.empty(g.workspace_bytes, dtype=torch.uint8, device="cuda"), **sums)
+        assert np.array_equal(g.run().cpu().numpy(), want), ("planes in", M, N, K)
+    if qp != q:
+        # records of the activations' own width are what the prefill kernel reads: the state stays there, and a tile of
+        # the decode kernel named by the caller is refused on them
+        M, N, K = 4, 64, 256
+        x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+        xe = abq.relayout_planes(planes_dev(oracle.pack_i32(x, q)))
+        wt = abq.relayout_planes(planes_dev(oracle.pack_i32(w, p)))
+        g = abq.Gemm(xe, wt, signed, x_tiled=True, w_tiled=True)
+        assert g.strategy == "tiled"
+        assert np.array_equal(g.run().cpu().numpy(), oracle.np_gemm(x, w))
+        cfg = [c for c in abq.native_configs(q, p, signed) if c.nstage == 6][0]
+        with pytest.raises(abq.AbqError):
+            abq.Gemm(xe, wt, signed, cfg=cfg, x_tiled=True, w_tiled=True).run()
+
+
 def test_decode_kernel_over_row_blocks_is_the_default_where_it_pays(abq, oracle):
     """Between 17 and 128 rows on prepared operands the library weighs the decode kernel over blocks of 16 rows
     against the prefill kernel's 64 x 64 tile: the choices its fit makes on the LLaMA-7B width, the result either

@@ -586,6 +586,46 @@ def test_unsigned_8bit_codes_reach_the_prepared_decode_kernel_with_their_row_sum
     assert [abq.padded_bits(b) for b in range(0, 10)] == [0, 2, 2, 4, 4, 8, 8, 8, 8, 0]
 
 
+def test_weights_of_several_fields_reach_the_prepared_decode_kernel_as_they_are(abq):
+    """Weights of 3, 5, 6, 7 bits: the decode kernel on prepared operands reads the prefill kernels' records, so a
+    decode-sized state with both operands K-tiled moves there with the pair's own widths.  Activations of such widths
+    only as padded records: declared before or after the layouts; undeclared, the state stays on the prefill kernel;
+    the workspace of plane activations counts the padded size; more than 16 rows stay on the prefill kernel."""
+    lib = abq.lib()
+    T, P = abq.LAYOUT_TILED, abq.LAYOUT_PLANES
+    names = abq.STRATEGY_NAMES
+
+    def fresh(q, p, M=4, signed=1):
+        rc, st = _init(abq, q=q, p=p, M=M, signed=signed, N=4096, K=4096)
+        assert rc == 0
+        return st
+
+    st = fresh(8, 3)  # activations of one field: nothing to declare
+    assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0 and names[st.strategy] == "decode_tiled"
+    assert (st.cfg.x_bits, st.cfg.w_bits, st.cfg.nstage) == (8, 3, 6) and lib.abq_gemm_workspace_bytes(ctypes.byref(st)) == 0
+    for q, p in [(3, 3), (5, 5), (6, 6), (7, 7), (6, 2)]:
+        st = fresh(q, p)
+        assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0 and names[st.strategy] == "tiled"
+        assert lib.abq_gemm_set_padded_activations(ctypes.byref(st), 1) == 0 and names[st.strategy] == "decode_tiled"
+        assert (st.cfg.x_bits, st.cfg.w_bits, st.cfg.nstage) == (q, p, 6)
+        assert lib.abq_gemm_set_padded_activations(ctypes.byref(st), 0) == 0 and names[st.strategy] == "tiled"
+        st = fresh(q, p)  # the other order
+        assert lib.abq_gemm_set_padded_activations(ctypes.byref(st), 1) == 0
+        assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0 and names[st.strategy] == "decode_tiled"
+        # plane activations under a tile of that kernel: exec pads them into the workspace
+        cfg = [c for c in abq.native_configs(q, p, True) if c.nstage == 6][0]
+        rc, st = _init(abq, q=q, p=p, M=4, signed=1, N=4096, K=4096, cfg=cfg)
+        assert rc == 0 and lib.abq_gemm_set_operand_layout(ctypes.byref(st), P, T) == 0
+        assert lib.abq_gemm_workspace_bytes(ctypes.byref(st)) == 4 * 4096 * abq.padded_bits(q) // 8
+        # ... and records of the activations' own width are refused for it
+        assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == abq.ABQ_ERR_UNSUPPORTED
+        st = fresh(q, p, M=64)  # more than 16 rows: only the prefill kernel, which reads no padded records
+        assert lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0 and names[st.strategy] == "tiled"
+        assert lib.abq_gemm_set_padded_activations(ctypes.byref(st), 1) == abq.ABQ_ERR_UNSUPPORTED and names[st.strategy] == "tiled"
+    st = fresh(8, 2)
+    assert lib.abq_gemm_set_padded_activations(ctypes.byref(st), 1) == 0 and st.reserved[4] == 0  # one field: its own padding
+
+
 def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     """The tile the library picks for prepared operands, pinned on shapes of BASELINE.json configs[2] and
     configs[4] and on a few where the measured sweep of all tiles separates them clearly:
