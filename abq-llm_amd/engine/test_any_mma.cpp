@@ -453,7 +453,8 @@ int main(int argc, char **argv)
     uint32_t *d_wt;
     char *d_ws;
     HIP_OK(hipMalloc(&d_wt, wp_bytes * nbuf));
-    const size_t ws_bytes = std::max((size_t)xp_words * 4, abq_fp6_bytes(M, K));
+    // (+ the activations' row sums, which exec takes for unsigned pairs with 8-bit weights when the activations arrive as planes)
+    const size_t ws_bytes = std::max((size_t)xp_words * 4, abq_fp6_bytes(M, K)) + (size_t)M * 4 + 1024;
     HIP_OK(hipMalloc(&d_ws, ws_bytes));
     if (abq_relayout_planes(d_wp, d_wt, N, K, w_bits, stream) != ABQ_OK) {
         std::printf("abq_relayout_planes failed (hip error %d)\n", abq_last_hip_error());
@@ -500,14 +501,19 @@ int main(int argc, char **argv)
     size_t nbuf_pad = std::min<size_t>(4096, std::max<size_t>(1, ((size_t)rotate_mib << 20) / wpad_bytes));
     uint32_t *d_xpad = nullptr, *d_wpad = nullptr;
     int *d_xsum = nullptr, *d_wsum = nullptr;
+    if (with_sums) { // the weights' row sums belong to their preparation, whatever M is
+        HIP_OK(hipMalloc(&d_xsum, (size_t)M * 4));
+        HIP_OK(hipMalloc(&d_wsum, (size_t)N * 4));
+        if (abq_row_sums(d_xp, M, K, x_bits, d_xsum, stream) != ABQ_OK || abq_row_sums(d_wp, N, K, w_bits, d_wsum, stream) != ABQ_OK) {
+            std::printf("abq_row_sums failed (hip error %d)\n", abq_last_hip_error());
+            return -1;
+        }
+    }
     if (M <= 16 && (padded || with_sums)) {
         HIP_OK(hipMalloc(&d_xpad, abq_planes_bytes(M, K, xq)));
         HIP_OK(hipMalloc(&d_wpad, wpad_bytes * nbuf_pad));
-        HIP_OK(hipMalloc(&d_xsum, (size_t)M * 4));
-        HIP_OK(hipMalloc(&d_wsum, (size_t)N * 4));
         if (abq_relayout_planes_padded(d_xp, d_xpad, M, K, x_bits, is_signed, stream) != ABQ_OK ||
-            abq_relayout_planes_padded(d_wp, d_wpad, N, K, w_bits, is_signed, stream) != ABQ_OK ||
-            abq_row_sums(d_xp, M, K, x_bits, d_xsum, stream) != ABQ_OK || abq_row_sums(d_wp, N, K, w_bits, d_wsum, stream) != ABQ_OK) {
+            abq_relayout_planes_padded(d_wp, d_wpad, N, K, w_bits, is_signed, stream) != ABQ_OK) {
             std::printf("preparing padded records failed (hip error %d)\n", abq_last_hip_error());
             return -1;
         }
@@ -573,7 +579,7 @@ int main(int argc, char **argv)
         const bool via_padded = prepared && pad_weights && d_wpad != nullptr;
         if (via_padded)
             states.resize(nbuf_pad);
-        if (both && (x_fields || with_sums) && !d_xpad) { // more than 16 rows: no padded activations were made
+        if (both && x_fields && !d_xpad) { // more than 16 rows: no padded activations were made
             t.status = -1;
             return;
         }
@@ -588,8 +594,10 @@ int main(int argc, char **argv)
                 s = abq_gemm_set_value_bits(&states[b], x_bits, w_bits);
             if (s == ABQ_OK && both && !via_padded && x_fields)
                 s = abq_gemm_set_padded_activations(&states[b], 1);
-            if (s == ABQ_OK && both && with_sums)
-                s = abq_gemm_set_row_sums(&states[b], d_xsum, d_wsum);
+            // unsigned 8-bit codes: the weights' row sums come with the prepared weights; the activations' with prepared
+            // activations, else exec takes them from the planes into the workspace
+            if (s == ABQ_OK && (both || tiled) && with_sums)
+                s = abq_gemm_set_row_sums(&states[b], both ? d_xsum : nullptr, d_wsum);
             if (s == ABQ_OK && tiled)
                 s = abq_gemm_set_operand_layout(&states[b], both ? ABQ_LAYOUT_TILED : ABQ_LAYOUT_PLANES, ABQ_LAYOUT_TILED);
             if (s == ABQ_OK && fp6)
