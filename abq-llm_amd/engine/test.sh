@@ -18,6 +18,7 @@ for shape in "4096 4096" "8192 1024" "11008 4096" "5120 5120" "4096 11008"; do
         p=${c##*:}
         $BIN "$M" "$N" "$K" "$q" "$p" 1 --tuning-out results/tuning.txt > "results/${M}x${N}x${K}_w${p}a${q}.txt"
     done
+    echo "M=$M N=$N K=$K: $(cat results/${M}x${N}x${K}_*.txt | grep -c PASSED) lines PASSED, $(cat results/${M}x${N}x${K}_*.txt | grep -c 'FAILED\|ERROR') FAILED or ERROR"
 done
 grep -h "best kernel config" results/*.txt | sort | uniq -c | sort -rn | head
 # results/tuning.txt now holds the best tile of every operand layout per shape: load it with abq_tuning_load (or
