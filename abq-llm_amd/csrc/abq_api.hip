@@ -175,6 +175,10 @@ static size_t fp6_bytes(int rows, int k) { return (size_t)rows * (k / 128) * 96;
 static int best_lpr_log2(int K)
 {
     const int units = K / 128;
+    // A row of at most 64 units: the fewest lanes that cover it in one pass, every load of the row in flight at once
+    // (K = 5120, 40 units: 64 lanes ahead of three passes of 16 by up to 20 % on the wide pairs, level on the narrow ones).
+    if (units <= 64)
+        return units <= 16 ? 4 : units <= 32 ? 5 : 6;
     int best = 6;
     double best_eff = 0;
     for (int l = 4; l <= 6; ++l) {
@@ -224,8 +228,11 @@ static void choose_default(int M, int N, int K, int x_bits, int w_bits, int *str
         *strategy = ABQ_STRATEGY_BCNT;
         *mi = 1; *tm = M <= 1 ? 1 : M <= 2 ? 2 : 4; *tn = 1; *wm = 1; *wn = 8; *wk = 1;
     } else if (M <= 16) {
+        // sixteen waves split K, eight where both operands are at least 5 bits wide (the transposes of that many planes
+        // in sixteen waves: W8A8 8 x 4096 x 4096 15.5 against 7.6 us, W6A6 9.9 against 6.7, W5A5 6.9 against 5.5) or K is
+        // short (8192 x 1024: 10 - 15 % on every pair); measured over M = 3 ... 16 on five shapes
         *strategy = ABQ_STRATEGY_DECODE;
-        *mi = 16; *tm = 1; *tn = 1; *wm = 1; *wn = 1; *wk = 16;
+        *mi = 16; *tm = 1; *tn = 1; *wm = 1; *wn = 1; *wk = ((x_bits >= 5 && w_bits >= 5) || K <= 2048) ? 8 : 16;
     } else if (M <= 64 ? (N < 8192 || w_bits <= 4 || M <= 32)
                        : (w_bits < 8 && (M <= 128 || (M <= 256 && K >= 8192)) && N < 8192)) {
         // 17 to 128 rows: blocks of 16 rows whose waves split K (16-row MFMA tiles, two per wave), which fill the chip
