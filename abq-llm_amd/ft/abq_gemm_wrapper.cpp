@@ -343,8 +343,12 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     // prepared operands where it is built for the pair (widths of 2, 4 or 8 bits, groups of 128; the library moves
     // the state there once both layouts are declared), else the decode kernel on plane operands if the caller kept
     // the planes; otherwise the tiled kernel on the prefill layout
-    const bool decode_prepared = W.planes_tiled != nullptr &&
-                                 abq_prepared_decode_pays(x_bits_, w_bits_, 1, M, N, K, W.group_size, silu_gate ? 1 : 0) != 0;
+    // (weights of several fields: as padded records, on the padded pair's kernel, the codes' own width declared)
+    const int w_rec_bits = abq_padded_bits(w_bits_);
+    const bool w_padded = w_rec_bits != w_bits_;
+    const uint32_t *w_records = reinterpret_cast<const uint32_t *>(w_padded ? W.records_padded : W.planes_tiled);
+    const bool decode_prepared = w_records != nullptr &&
+                                 abq_prepared_decode_pays(x_bits_, w_rec_bits, 1, M, N, K, W.group_size, silu_gate ? 1 : 0) != 0;
     // (if the expanded activations fit the decode kernel's LDS: partial tiles, group sums, M padded rows)
     const bool decode = !decode_prepared && M <= 16 && W.planes != nullptr &&
                         (silu_gate ? 32 : 16) * 1024 + (size_t)64 * (K / W.group_size) + 128 + (size_t)M * ((K + 511) / 512 * 512 + 16) <= 160 * 1024;
@@ -358,8 +362,9 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     // the wide linears costs more than the launch from two tokens on: QKV of LLaMA-7B at two tokens 11.6 against
     // 10.1 us, at four 18.0 against 10.7; 4096 x 4096 at four tokens 8.1 against 8.6)
     if (decode_prepared && M <= 16 && (size_t)M * K <= 16384 && (M == 1 || N <= 4096)) {
-        rc = abq_gemm_init(nullptr, x_bits_, w_bits_, 1, planes, reinterpret_cast<const uint32_t *>(W.planes_tiled), M, N, K, D,
-                           nullptr, 0, ABQ_OUT_F16_SCALED, &state);
+        rc = abq_gemm_init(nullptr, x_bits_, w_rec_bits, 1, planes, w_records, M, N, K, D, nullptr, 0, ABQ_OUT_F16_SCALED, &state);
+        if (rc == ABQ_OK && w_padded)
+            rc = abq_gemm_set_value_bits(&state, x_bits_, w_bits_);
         if (rc == ABQ_OK)
             rc = abq_gemm_set_operand_layout(&state, ABQ_LAYOUT_TILED, ABQ_LAYOUT_TILED);
         if (rc == ABQ_OK)
@@ -384,9 +389,17 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
         printf("[ABQ][Error] pack failed: %s\n", abq_status_string(rc));
         return;
     }
-    rc = abq_gemm_init(nullptr, x_bits_, w_bits_, 1, planes,
-                       reinterpret_cast<const uint32_t *>(decode ? W.planes : fp6 ? W.records_fp6 : W.planes_tiled), M, N, K,
+    const bool on_padded = decode_prepared && w_padded;
+    if (!decode && !fp6 && !on_padded && !W.planes_tiled) {
+        printf("[ABQ][Error] ABQGroupedWeight::planes_tiled is needed for M,N,K = %d,%d,%d\n", M, N, K);
+        return;
+    }
+    rc = abq_gemm_init(nullptr, x_bits_, on_padded ? w_rec_bits : w_bits_, 1, planes,
+                       decode ? reinterpret_cast<const uint32_t *>(W.planes) : fp6 ? reinterpret_cast<const uint32_t *>(W.records_fp6)
+                       : on_padded ? w_records : reinterpret_cast<const uint32_t *>(W.planes_tiled), M, N, K,
                        D, nullptr, 0, ABQ_OUT_F16_SCALED, &state);
+    if (rc == ABQ_OK && on_padded)
+        rc = abq_gemm_set_value_bits(&state, x_bits_, w_bits_);
     if (rc == ABQ_OK && !decode)
         rc = abq_gemm_set_operand_layout(&state, layout, layout);
     if (rc == ABQ_OK)

@@ -35,6 +35,10 @@ struct ABQGroupedWeight {
     const int *records_fp6;   // the same weights as FP6 records (abq_relayout_planes_fp6), or nullptr; with it,
                               // groups of 128 and a bit pair that qualifies (abq_fp6_eligible, e.g. W4A4), calls of
                               // more than 16 rows run on the FP6 matrix cores
+    const int *records_padded; // weights of 3, 5, 6 or 7 bits (e.g. the reference's bit-balanced 2-bit weights, three
+                              // planes): the same weights as records of the next single-field width
+                              // (abq_relayout_planes_padded), or nullptr; with it, the decode-sized calls run the
+                              // prepared-operand decode kernel of that width instead of the one on plane operands
 };
 
 class ABQGEMMWrapper {

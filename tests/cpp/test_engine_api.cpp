@@ -370,10 +370,14 @@ static void gpu_paths()
         HIP_OK(hipFree(d_ws));
     }
 
-    {   // FT wrapper, dynamic path: per-token int8 activations, 2-bit weights with group scales and
-        // zero points; expected values from a double-precision loop over the dequantised operands
-        const int M = 40, N = 192, K = 512, G = 128, groups = K / G;
-        std::mt19937 r32(5);
+    // FT wrapper, dynamic path: per-token int8 activations, weights with group scales and zero points; expected
+    // values from a double-precision loop over the dequantised operands.  2-bit weights (prefill- and decode-sized
+    // calls), and 3-bit weights (the reference's bit-balanced 2-bit quantiser writes three planes): at decode sizes as
+    // padded records on the prepared-operand decode kernel of the 4-bit width, as planes on the plane-operand one,
+    // above that on the prefill kernel.
+    auto dynamic_case = [&](const int WB, const int M, const bool padded_records, const bool keep_planes) {
+        const int N = 192, K = 512, G = 128, groups = K / G;
+        std::mt19937 r32(5 + WB + M);
         std::normal_distribution<float> nd(0.f, 1.5f);
         std::uniform_real_distribution<float> ud(0.002f, 0.02f);
         std::vector<uint16_t> ha((size_t)M * K);
@@ -381,24 +385,25 @@ static void gpu_paths()
             h = abq_oracle_f32_to_f16(nd(r32));
         std::vector<int> wq((size_t)N * K);
         for (auto &v : wq)
-            v = (int)(r32() % 4) - 2;
+            v = (int)(r32() % (1u << WB)) - (1 << (WB - 1));
         std::vector<float> wscale((size_t)N * groups), wzero((size_t)N * groups);
         for (auto &v : wscale)
             v = ud(r32);
         for (auto &v : wzero)
-            v = (float)((int)(r32() % 4) - 2);
-        std::vector<uint32_t> wpl((size_t)2 * N * K / 32);
-        abq_oracle_pack_i32(wq.data(), wpl.data(), N, K, 2);
+            v = (float)((int)(r32() % (1u << WB)) - (1 << (WB - 1)));
+        std::vector<uint32_t> wpl((size_t)WB * N * K / 32);
+        abq_oracle_pack_i32(wq.data(), wpl.data(), N, K, WB);
         _Float16 *d_a, *d_d;
-        uint32_t *d_wpl, *d_wt;
+        uint32_t *d_wpl, *d_wt, *d_wpad;
         float *d_wscale, *d_wzero, *d_term;
         char *d_ws;
-        ABQGEMMWrapper wrap(8, 2, true);
+        ABQGEMMWrapper wrap(8, WB, true);
         const size_t ws_bytes = wrap.dynamic_workspace_bytes(M, K, G);
         HIP_OK(hipMalloc(&d_a, ha.size() * 2));
         HIP_OK(hipMalloc(&d_d, (size_t)M * N * 2));
         HIP_OK(hipMalloc(&d_wpl, wpl.size() * 4));
         HIP_OK(hipMalloc(&d_wt, wpl.size() * 4));
+        HIP_OK(hipMalloc(&d_wpad, abq_planes_bytes(N, K, abq_padded_bits(WB))));
         HIP_OK(hipMalloc(&d_wscale, wscale.size() * 4));
         HIP_OK(hipMalloc(&d_wzero, wzero.size() * 4));
         HIP_OK(hipMalloc(&d_term, N * 4));
@@ -407,9 +412,12 @@ static void gpu_paths()
         HIP_OK(hipMemcpy(d_wpl, wpl.data(), wpl.size() * 4, hipMemcpyHostToDevice));
         HIP_OK(hipMemcpy(d_wscale, wscale.data(), wscale.size() * 4, hipMemcpyHostToDevice));
         HIP_OK(hipMemcpy(d_wzero, wzero.data(), wzero.size() * 4, hipMemcpyHostToDevice));
-        CHECK(abq_relayout_planes(d_wpl, d_wt, N, K, 2, stream) == ABQ_OK);
-        CHECK(abq_weight_zero_term(d_wpl, N, K, 2, 1, d_wscale, d_wzero, G, d_term, stream) == ABQ_OK);
-        const ABQGroupedWeight weight = { reinterpret_cast<const int *>(d_wt), d_wscale, d_wzero, d_term, G, nullptr };
+        CHECK(abq_relayout_planes(d_wpl, d_wt, N, K, WB, stream) == ABQ_OK);
+        CHECK(abq_relayout_planes_padded(d_wpl, d_wpad, N, K, WB, 1, stream) == ABQ_OK);
+        CHECK(abq_weight_zero_term(d_wpl, N, K, WB, 1, d_wscale, d_wzero, G, d_term, stream) == ABQ_OK);
+        const ABQGroupedWeight weight = { reinterpret_cast<const int *>(d_wt), d_wscale, d_wzero, d_term, G,
+                                          keep_planes ? reinterpret_cast<const int *>(d_wpl) : nullptr, nullptr,
+                                          padded_records ? reinterpret_cast<const int *>(d_wpad) : nullptr };
         for (int symmetric = 1; symmetric >= 0; --symmetric) {
             wrap.gemm_dynamic(M, N, K, d_a, weight, d_d, symmetric != 0, d_ws, ws_bytes, stream);
             HIP_OK(hipStreamSynchronize(stream));
@@ -459,11 +467,19 @@ static void gpu_paths()
         HIP_OK(hipFree(d_d));
         HIP_OK(hipFree(d_wpl));
         HIP_OK(hipFree(d_wt));
+        HIP_OK(hipFree(d_wpad));
         HIP_OK(hipFree(d_wscale));
         HIP_OK(hipFree(d_wzero));
         HIP_OK(hipFree(d_term));
         HIP_OK(hipFree(d_ws));
-    }
+    };
+    dynamic_case(2, 40, false, false);
+    dynamic_case(2, 1, false, false);
+    dynamic_case(3, 40, true, false);  // blocks of 16 rows on the 4-bit decode kernel (or the prefill kernel on the 3-bit records)
+    dynamic_case(3, 1, true, false);   // one launch: the 4-bit decode kernel quantises the row itself
+    dynamic_case(3, 8, true, false);   // quantiser + the 4-bit decode kernel on the padded records
+    dynamic_case(3, 8, false, true);   // no padded records: the decode kernel on plane operands
+    dynamic_case(5, 4, true, false);   // 5-bit weights as 8-bit records
 
     {   // weight file -> device weight -> dynamic GEMM: the file round-trips, and the GEMM on the loaded
         // weight equals a double-precision loop over the blob's own dequantised codes
