@@ -629,7 +629,33 @@ def main():
                 log("dequant decode M=%d N=%d K=%d  %.2f us  %.0f GB/s (%.1f%% of HBM peak)  %s; plane operands %.2f us"
                     % (M, N, K, us, gbs, 100 * gbs / HBM_PEAK_GBS, gs[0].strategy, us_planes))
                 del gs, out
+        # the same with 3-bit weights (what the reference's default 2-bit quantiser, bit balance, writes): as padded
+        # 4-bit records on the prepared-operand kernel, and on plane operands
+        deq3 = []
+        for (N, K) in SHAPES:
+            G = K // 128
+            R3 = max(2, math.ceil(ROTATE_BYTES / (4 * N * K // 8)))
+            w3 = random_planes(torch, (3, N, K // 32))
+            w3p = abq.relayout_planes_padded(w3, SIGNED)
+            Wp3 = w3p.unsqueeze(0).repeat(R3, 1, 1, 1, 1)
+            W3 = w3.unsqueeze(0).repeat(R3, 1, 1, 1)
+            wsc = torch.rand((N, G), device="cuda") * 0.01 + 0.001
+            wz = torch.randint(-4, 4, (N, G), device="cuda").float()
+            for M in (1, 8):
+                xsc = torch.rand(M, device="cuda") * 0.05 + 0.01
+                sums = torch.randint(-1000, 1000, (M, G), dtype=torch.int32, device="cuda")
+                out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+                kw = dict(out=out, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc, group_size=128, w_zero=wz, x_group_sums=sums)
+                gs = [abq.Gemm(xs_tiled[(M, K)], Wp3[r], SIGNED, x_tiled=True, w_tiled=True, value_bits=(Q_BITS, 3), **kw) for r in range(R3)]
+                us = time_rotating(gs)
+                us_planes = time_rotating([abq.Gemm(xs[(M, K)], W3[r], SIGNED, **kw) for r in range(R3)])
+                deq3.append(dict(M=M, N=N, K=K, w_bits=3, group_size=128, us=round(us, 3), kernel="%s:%s" % (gs[0].strategy, gs[0].config_name),
+                                 plane_operands_us=round(us_planes, 3)))
+                log("dequant decode W3A8 M=%d N=%d K=%d  %.2f us (%s, padded records); plane operands %.2f us" % (M, N, K, us, gs[0].strategy, us_planes))
+                del gs, out
+            del Wp3, W3
         extra["decode_group_scales"] = deq
+        extra["decode_group_scales_w3a8"] = deq3
 
     if want("small_batch"):
         # ------------------------------------------------------------ side measurement: 32 and 64 rows on prepared operands
