@@ -19,7 +19,7 @@ stream: the average launch duration of the roofline is that interval over 9 K la
 stderr come from one graph per GEMM (K launches of it), replayed after the timed region.
 
 Prints ONE short JSON line on stdout.  Progress and the side measurements go to stderr, the side measurements also
-as JSON into --extra-out (default gpurun_out/bench_extra.json).
+as JSON into the file --extra-out names (default: bench_extra.json in the output folder beside this script).
 """
 import argparse
 import importlib.util
