@@ -917,12 +917,27 @@ __global__ __launch_bounds__(64 * NW) void gemm_decode_tiled_grouped(const GemmA
                         const int last = __builtin_amdgcn_readfirstlane(min(p - lane + 63, nunits - 1) / upr);
                         auto ordered = [](float f) { const int k = __builtin_bit_cast(int, f); return k ^ ((k >> 31) & 0x7FFFFFFF); };
                         if (first == last) {
-#pragma unroll
-                            for (int o = 32; o > 0; o >>= 1) {
-                                mx = fmaxf(mx, __shfl_xor(mx, o));
-                                mn = fminf(mn, __shfl_xor(mn, o));
-                            }
-                            if (lane == 0) {
+                            // across the wave with lane permutations inside the vector ALU (a shuffle through the LDS
+                            // crossbar per step would be six dependent round trips): quads, halves of a row of 16, the
+                            // row, then the rows' last lanes handed on; lane 63 ends up with the wave's extrema
+                            auto dpp = [](float v, auto ctrl, auto row_mask) {
+                                return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v),
+                                                                                             decltype(ctrl)::value, decltype(row_mask)::value, 0xF, false));
+                            };
+                            using std::integral_constant;
+                            mx = fmaxf(mx, dpp(mx, integral_constant<int, 0xB1>{}, integral_constant<int, 0xF>{}));  // quad_perm [1,0,3,2]
+                            mn = fminf(mn, dpp(mn, integral_constant<int, 0xB1>{}, integral_constant<int, 0xF>{}));
+                            mx = fmaxf(mx, dpp(mx, integral_constant<int, 0x4E>{}, integral_constant<int, 0xF>{}));  // quad_perm [2,3,0,1]
+                            mn = fminf(mn, dpp(mn, integral_constant<int, 0x4E>{}, integral_constant<int, 0xF>{}));
+                            mx = fmaxf(mx, dpp(mx, integral_constant<int, 0x141>{}, integral_constant<int, 0xF>{})); // row_half_mirror
+                            mn = fminf(mn, dpp(mn, integral_constant<int, 0x141>{}, integral_constant<int, 0xF>{}));
+                            mx = fmaxf(mx, dpp(mx, integral_constant<int, 0x140>{}, integral_constant<int, 0xF>{})); // row_mirror
+                            mn = fminf(mn, dpp(mn, integral_constant<int, 0x140>{}, integral_constant<int, 0xF>{}));
+                            mx = fmaxf(mx, dpp(mx, integral_constant<int, 0x142>{}, integral_constant<int, 0xA>{})); // row_bcast 15 into rows 1, 3
+                            mn = fminf(mn, dpp(mn, integral_constant<int, 0x142>{}, integral_constant<int, 0xA>{}));
+                            mx = fmaxf(mx, dpp(mx, integral_constant<int, 0x143>{}, integral_constant<int, 0xC>{})); // row_bcast 31 into rows 2, 3
+                            mn = fminf(mn, dpp(mn, integral_constant<int, 0x143>{}, integral_constant<int, 0xC>{}));
+                            if (lane == 63) {
                                 atomicMax(&row_ext[row], ordered(mx));
                                 atomicMin(&row_ext[16 + row], ordered(mn));
                             }
