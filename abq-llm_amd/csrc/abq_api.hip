@@ -1881,9 +1881,17 @@ static abq_status set_operand_layout_by_rules(abq_gemm_state *st, int x_layout, 
 
 abq_status abq_gemm_set_operand_layout(abq_gemm_state *st, int x_layout, int w_layout)
 {
-    const abq_status rc = set_operand_layout_by_rules(st, x_layout, w_layout);
+    if (!st || !st->init_success)
+        return ABQ_ERR_NOT_INITIALIZED;
+    abq_gemm_state next = *st; // the caller's state changes only if the declaration is taken
+    abq_status rc = set_operand_layout_by_rules(&next, x_layout, w_layout);
     if (rc == ABQ_OK)
-        apply_tuned(st); // a measured best tile for this shape on these layouts, if the table holds one
+        apply_tuned(&next); // a measured best tile for this shape on these layouts, if the table holds one
+    // activation records declared padded are read by the decode kernel on prepared operands only
+    if (rc == ABQ_OK && next.x_layout == ABQ_LAYOUT_TILED && padded_x(&next) && next.strategy != ABQ_STRATEGY_DECODE_TILED)
+        rc = ABQ_ERR_UNSUPPORTED;
+    if (rc == ABQ_OK)
+        *st = next;
     return rc;
 }
 
