@@ -366,7 +366,8 @@ class Gemm:
     def __init__(self, x_planes, w_planes, signed, out=None, cfg=None, out_kind=OUT_I32, c_scale=None,
                  x_scale=None, w_scale=None, group_size=0, x_tiled=False, w_tiled=False, workspace=None,
                  x_zero=None, w_zero=None, x_group_sums=None, w_zero_term=None, act=ACT_NONE,
-                 x_fp6=0, w_fp6=0, x_row_sums=None, w_row_sums=None, value_bits=None, biased=None, x_padded_from=None):
+                 x_fp6=0, w_fp6=0, x_row_sums=None, w_row_sums=None, value_bits=None, biased=None, x_padded_from=None,
+                 x_planes_of=None):
         import torch
         if x_fp6:
             kt, M, _ = x_planes.shape
@@ -379,6 +380,9 @@ class Gemm:
                 q = int(x_padded_from)
         else:
             q, M, kw = x_planes.shape
+            if x_planes_of is not None:  # planes of fewer bits than the state's width (value_bits says how many)
+                assert q == int(value_bits[0]) and q <= int(x_planes_of)
+                q = int(x_planes_of)
         if w_fp6:
             kt2, N, _ = w_planes.shape
             p, kw2 = int(w_fp6), kt2 * 4

@@ -1021,6 +1021,15 @@ static bool decode_tiled_x_ok(const abq_gemm_state *st, int x_layout)
 }
 static bool decode_tiled_x_ok(const abq_gemm_state *st) { return decode_tiled_x_ok(st, st->x_layout); }
 
+// Planes an operand arrives in: as many as its codes have bits, which abq_gemm_set_value_bits may have declared fewer
+// than the state's (record) width.
+static int x_plane_bits(const abq_gemm_state *st) {
+    return st->reserved[2] > 0 && st->reserved[2] < st->cfg.x_bits ? st->reserved[2] : st->cfg.x_bits;
+}
+static int w_plane_bits(const abq_gemm_state *st) {
+    return st->reserved[3] > 0 && st->reserved[3] < st->cfg.w_bits ? st->reserved[3] : st->cfg.w_bits;
+}
+
 // Unsigned 8-bit records on the decode kernel of prepared operands: codes up to 255 are fed as value - 128 and need
 // the other operand's row sums (abq_gemm_set_row_sums); records declared to hold narrower codes
 // (abq_gemm_set_value_bits: padded records) are fed as they are.  flip_x / flip_w: which operands are flipped.
@@ -1648,14 +1657,14 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
             return ABQ_ERR_INVALID_ARG;
         char *ws = static_cast<char *>(st->workspace);
         if (xb) {
-            e = launch_relayout_planes_fp6(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, c.x_bits, c.is_signed,
+            e = launch_relayout_planes_fp6(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, x_plane_bits(st), c.is_signed,
                                            (hipStream_t)stream);
             if (e != hipSuccess)
                 return hip_status(e);
             a.X = reinterpret_cast<const uint32_t *>(ws);
         }
         if (wb) {
-            e = launch_relayout_planes_fp6(st->W, reinterpret_cast<uint32_t *>(ws + xb), st->N, st->K, c.w_bits,
+            e = launch_relayout_planes_fp6(st->W, reinterpret_cast<uint32_t *>(ws + xb), st->N, st->K, w_plane_bits(st),
                                            c.is_signed, (hipStream_t)stream);
             if (e != hipSuccess)
                 return hip_status(e);
@@ -1693,14 +1702,16 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
         if (!biased && biased_x(st))
             return ABQ_ERR_INVALID_ARG; // biased activations only make sense against biased weights
         if (xb) {
-            e = launch_relayout_planes_padded(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, xrec, c.x_bits,
-                                              biased ? 2 : (xrec != c.x_bits && c.is_signed ? 1 : 0), (hipStream_t)stream);
+            // (planes of fewer bits than the records: the codes are extended to the record's width)
+            e = launch_relayout_planes_padded(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, xrec, x_plane_bits(st),
+                                              biased ? 2 : (xrec != x_plane_bits(st) && c.is_signed ? 1 : 0), (hipStream_t)stream);
             if (e != hipSuccess)
                 return hip_status(e);
             a.X = reinterpret_cast<const uint32_t *>(ws);
         }
         if (wb) {
-            e = launch_relayout_planes(st->W, reinterpret_cast<uint32_t *>(ws + xb), st->N, st->K, c.w_bits, (hipStream_t)stream);
+            e = launch_relayout_planes_padded(st->W, reinterpret_cast<uint32_t *>(ws + xb), st->N, st->K, c.w_bits, w_plane_bits(st),
+                                              w_plane_bits(st) != c.w_bits && c.is_signed ? 1 : 0, (hipStream_t)stream);
             if (e != hipSuccess)
                 return hip_status(e);
             a.W = reinterpret_cast<const uint32_t *>(ws + xb);
@@ -1716,12 +1727,24 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
         if (!t || st->variant < 0 || st->variant >= t->count)
             return ABQ_ERR_NOT_INITIALIZED;
         int variant = st->variant;
+        if (st->strategy == ABQ_STRATEGY_TILED && !c.is_signed && !biased && x_plane_bits(st) < c.x_bits && w_plane_bits(st) < c.w_bits) {
+            // Unsigned codes that leave the top bit of their records clear are signed codes of the records' width as
+            // well: the signed pair's kernel of the same tile reads them as they are (no value - 128, no row sums).
+            const KernelTable *ts = find_table(st->group_size ? reg.tiled_grouped : reg.tiled, c.x_bits, c.w_bits, 1);
+            const KernelEntry &want = t->entries[st->variant];
+            for (int i = 0; ts && i < ts->count; ++i) {
+                const KernelEntry &o = ts->entries[i];
+                if ((o.lds != 0) == (want.lds != 0) && !(o.flags & kNeedsRowSums) && o.mi == want.mi && o.tm == want.tm && o.tn == want.tn &&
+                    o.wm == want.wm && o.wn == want.wn && o.wk == want.wk && o.kb == want.kb && o.nstage == want.nstage)
+                    return hip_status(o.launch(a, (hipStream_t)stream));
+            }
+        }
         if (biased) {
             const RowSumPlan plan = row_sum_plan(st, xb + wb);
             if (!plan.ok)
                 return ABQ_ERR_INVALID_ARG; // both operands' sums are needed; the weights' must be set
             if (!st->x_row_sums) {
-                e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, c.x_bits, (hipStream_t)stream);
+                e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, x_plane_bits(st), (hipStream_t)stream);
                 if (e != hipSuccess)
                     return hip_status(e);
             }
@@ -1749,13 +1772,13 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
             a.x_row_sums = st->x_row_sums;
             a.w_row_sums = st->w_row_sums;
             if (a.flip_w && !st->x_row_sums) {
-                e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, c.x_bits, (hipStream_t)stream);
+                e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, x_plane_bits(st), (hipStream_t)stream);
                 if (e != hipSuccess)
                     return hip_status(e);
                 a.x_row_sums = reinterpret_cast<const int *>(ws + plan.x_off);
             }
             if (a.flip_x && !st->w_row_sums) {
-                e = launch_row_sums(st->W, reinterpret_cast<int *>(ws + plan.w_off), st->N, st->K, c.w_bits, (hipStream_t)stream);
+                e = launch_row_sums(st->W, reinterpret_cast<int *>(ws + plan.w_off), st->N, st->K, w_plane_bits(st), (hipStream_t)stream);
                 if (e != hipSuccess)
                     return hip_status(e);
                 a.w_row_sums = reinterpret_cast<const int *>(ws + plan.w_off);
@@ -1769,12 +1792,12 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
             const RowSumPlan plan = row_sum_plan(st, xb + wb);
             if (plan.ok) {
                 if (need_x && !st->x_row_sums) {
-                    e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, c.x_bits, (hipStream_t)stream);
+                    e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, x_plane_bits(st), (hipStream_t)stream);
                     if (e != hipSuccess)
                         return hip_status(e);
                 }
                 if (need_w && !st->w_row_sums) {
-                    e = launch_row_sums(st->W, reinterpret_cast<int *>(ws + plan.w_off), st->N, st->K, c.w_bits, (hipStream_t)stream);
+                    e = launch_row_sums(st->W, reinterpret_cast<int *>(ws + plan.w_off), st->N, st->K, w_plane_bits(st), (hipStream_t)stream);
                     if (e != hipSuccess)
                         return hip_status(e);
                 }

@@ -454,7 +454,7 @@ int main(int argc, char **argv)
     char *d_ws;
     HIP_OK(hipMalloc(&d_wt, wp_bytes * nbuf));
     // (+ the activations' row sums, which exec takes for unsigned pairs with 8-bit weights when the activations arrive as planes)
-    const size_t ws_bytes = std::max((size_t)xp_words * 4, abq_fp6_bytes(M, K)) + (size_t)M * 4 + 1024;
+    const size_t ws_bytes = std::max(abq_planes_bytes(M, K, abq_padded_bits(x_bits)), abq_fp6_bytes(M, K)) + (size_t)M * 4 + 1024;
     HIP_OK(hipMalloc(&d_ws, ws_bytes));
     if (abq_relayout_planes(d_wp, d_wt, N, K, w_bits, stream) != ABQ_OK) {
         std::printf("abq_relayout_planes failed (hip error %d)\n", abq_last_hip_error());
@@ -493,7 +493,8 @@ int main(int argc, char **argv)
     // Decode-sized M, prepared operands.  Weights of several fields (3, 5, 6, 7 bits) are read by the decode kernel as
     // the records above; activations of such widths come as padded records (abq_relayout_planes_padded: the next width
     // of 2, 4 or 8 bits), and unsigned 8-bit codes bring their row sums (abq_row_sums).  A second "prepared operands"
-    // line times the same pairs with the weights padded as well (the padded pair's kernel).
+    // line times the same pairs with the weights padded as well (the padded pair's kernel).  Above 16 rows the padded
+// weights get a line too: the padded pair's prefill kernel, the activations arriving as planes of their own width.
     const int xq = abq_padded_bits(x_bits), wq = abq_padded_bits(w_bits);
     const bool padded = xq != x_bits || wq != w_bits;
     const bool with_sums = !is_signed && (x_bits == 8 || w_bits == 8);
@@ -509,7 +510,9 @@ int main(int argc, char **argv)
             return -1;
         }
     }
-    if (M <= 16 && (padded || with_sums)) {
+    // (above 16 rows only where the padded pair's weights are K-tiled records as well)
+    const bool padded_prefill = M > 16 && padded && !group && abq_preferred_weight_layout(xq, wq, is_signed, M, N, K, 0) == ABQ_LAYOUT_TILED;
+    if (M <= 16 ? (padded || with_sums) : padded_prefill) {
         HIP_OK(hipMalloc(&d_xpad, abq_planes_bytes(M, K, xq)));
         HIP_OK(hipMalloc(&d_wpad, wpad_bytes * nbuf_pad));
         if (abq_relayout_planes_padded(d_xp, d_xpad, M, K, x_bits, is_signed, stream) != ABQ_OK ||
@@ -568,15 +571,15 @@ int main(int argc, char **argv)
         std::vector<abq_gemm_state> states(nbuf);
         // tiled tiles (NSTAGE 4) run on prepared weights, NSTAGE 6 and the `prepared` default on prepared weights and
         // activations, the FP6 tiles on FP6 records; the library's own choice for M > 16 on the preferred layout
-        const bool both = prepared || (cfg ? cfg->nstage == 6 : tuned_decode);
-        const bool fp6 = cfg ? cfg->nstage == 5 : (!prepared && M > 16 && preferred == ABQ_LAYOUT_FP6 && fp6_ok);
-        const bool tiled = both || (cfg ? cfg->nstage == 4 : (M > 16 && !fp6 && preferred != ABQ_LAYOUT_PLANES));
+        // (the default with the weights as padded records: the padded pair's kernel)
+        const bool via_padded = !cfg && pad_weights && d_wpad != nullptr;
+        const bool both = prepared || (cfg ? cfg->nstage == 6 : (tuned_decode && !via_padded));
+        const bool fp6 = cfg ? cfg->nstage == 5 : (!prepared && !via_padded && M > 16 && preferred == ABQ_LAYOUT_FP6 && fp6_ok);
+        const bool tiled = both || via_padded || (cfg ? cfg->nstage == 4 : (M > 16 && !fp6 && preferred != ABQ_LAYOUT_PLANES));
         if (fp6 && !fp6_ok) {
             t.status = -1;
             return;
         }
-        // (the prepared default with the weights as padded records too: the padded pair's kernel)
-        const bool via_padded = prepared && pad_weights && d_wpad != nullptr;
         if (via_padded)
             states.resize(nbuf_pad);
         if (both && x_fields && !d_xpad) { // more than 16 rows: no padded activations were made
@@ -588,7 +591,7 @@ int main(int argc, char **argv)
                                 : fp6      ? (const char *)d_wf + b * wf_bytes
                                            : (tiled ? (const char *)d_wt : (const char *)d_wp) + b * wp_bytes;
             abq_status s = abq_gemm_init(cfg, via_padded ? xq : x_bits, via_padded ? wq : w_bits, is_signed,
-                                         via_padded ? d_xpad : both ? (x_fields ? d_xpad : d_xt) : d_xp, (const uint32_t *)wbase,
+                                         !both ? d_xp : via_padded ? d_xpad : (x_fields ? d_xpad : d_xt), (const uint32_t *)wbase,
                                          M, N, K, d_out, nullptr, 0, ABQ_OUT_I32, &states[b]);
             if (s == ABQ_OK && via_padded && padded)
                 s = abq_gemm_set_value_bits(&states[b], x_bits, w_bits);
@@ -656,17 +659,19 @@ int main(int argc, char **argv)
     abq_tile_config layout_best[3];
     const int ncfg = abq_native_config_count(x_bits, w_bits, is_signed);
     // + the library's choice (+ its choice on prepared operands (+ the same with the weights padded as well))
-    const int nlines = ncfg + (M <= 16 ? (padded && wq != w_bits ? 3 : 2) : 1);
+    const int nlines = ncfg + (M <= 16 ? (padded && wq != w_bits ? 3 : 2) : (padded_prefill ? 2 : 1));
     for (int i = 0; i < nlines; ++i) {
         abq_tile_config cfg;
         const bool library_default = i >= ncfg;
-        const bool prepared = i >= ncfg + 1, pad_weights = i == ncfg + 2;
+        const bool prepared = M <= 16 && i >= ncfg + 1, pad_weights = i == ncfg + (M <= 16 ? 2 : 1);
         if (!library_default && abq_native_config_get(x_bits, w_bits, is_signed, i, &cfg) != ABQ_OK)
             continue;
         char name[160] = "library default";
         const char *how = pad_weights ? " (padded records)" : (with_sums && d_wpad) ? " (with row sums)" : "";
         if (prepared)
             std::snprintf(name, sizeof name, "library default, prepared operands%s", how);
+        else if (pad_weights)
+            std::snprintf(name, sizeof name, "library default (padded records)");
         if (!library_default)
             abq_format_kernel_name(&cfg, 0, name, sizeof name);
         if (!only.empty() && std::string(name).find(only) == std::string::npos)
@@ -685,7 +690,8 @@ int main(int argc, char **argv)
                     prepared ? (pad_weights ? " | library default, prepared operands (padded records)"
                                 : (with_sums && d_wpad) ? " | library default, prepared operands (with row sums)"
                                                         : " | library default, prepared operands")
-                             : library_default ? " | library default" : "");
+                    : pad_weights   ? " | library default (padded records)"
+                    : library_default ? " | library default" : "");
         if (t.status == 0 && !library_default && tops > best_tops) {
             best_tops = tops;
             char buf[128];

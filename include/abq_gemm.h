@@ -440,7 +440,12 @@ int abq_padded_bits(int bits);
 abq_status abq_relayout_planes_padded(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits, int is_signed,
                                       void *stream);
 /* Declares that the codes of X (W) use only the low x_value_bits (w_value_bits) of their fields (1 .. the state's
- * widths): see above. */
+ * widths): see above.  An operand of such a state that is still in the reference plane layout has that many planes,
+ * and abq_gemm_exec extends its codes to the records' width while it converts them into the workspace.  This makes
+ * padded weight records serve every M: above 16 rows the padded pair's prefill kernels run (the LDS-staged int8
+ * kernel for 8-bit records, which the widths of several fields do not have), and an unsigned pair whose codes are
+ * narrower than the records on both sides runs the signed pair's kernel of the same tile: such codes are signed codes
+ * of the records' width as well, so neither the value - 128 route nor row sums are needed. */
 abq_status abq_gemm_set_value_bits(abq_gemm_state *state, int x_value_bits, int w_value_bits);
 /* Weights of 3, 5, 6 or 7 bits need no padded copy for decode: the decode kernel on prepared operands reads the
  * records abq_relayout_planes writes (the ones the prefill kernels read), field by field.  Its activations are records

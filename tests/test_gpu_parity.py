@@ -586,6 +586,34 @@ def test_decode_on_prepared_operands(abq, oracle, q, p, signed):
             assert e.value.status == abq.ABQ_ERR_INVALID_ARG
 
 
+@pytest.mark.parametrize("q,p", [(3, 3), (5, 5), (6, 6), (7, 7), (8, 3), (6, 2)])
+@pytest.mark.parametrize("signed", [True, False])
+def test_prefill_on_padded_weight_records(abq, oracle, q, p, signed):
+    """Weights of 3, 5, 6 or 7 bits held as padded records serve the prefill as well: the state is initialised with
+    the padded pair and told the codes' widths, the activations arrive as planes of their own width and exec extends
+    them to the records' width in the workspace (sign extension for signed codes; the row sums of unsigned codes in
+    8-bit records are those of the codes)."""
+    qp, pp = abq.padded_bits(q), abq.padded_bits(p)
+    rng = np.random.default_rng(900 + 10 * q + p + int(signed))
+    for (M, N, K) in [(17, 64, 512), (40, 200, 1408), (128, 256, 4096), (300, 130, 1152)]:
+        x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+        x[1] = (1 << (q - 1)) - 1 if signed else (1 << q) - 1
+        x[2] = -(1 << (q - 1)) if signed else 0
+        w[0] = -(1 << (p - 1)) if signed else (1 << p) - 1
+        xd, wd = planes_dev(oracle.pack_i32(x, q)), planes_dev(oracle.pack_i32(w, p))
+        wt = abq.relayout_planes_padded(wd, signed)
+        want = oracle.np_gemm(x, w)
+        ws = torch.empty(M * K * qp // 8 + 4 * (M + N) + 1024, dtype=torch.uint8, device="cuda")
+        g = abq.Gemm(xd, wt, signed, w_tiled=True, value_bits=(q, p), x_planes_of=qp, workspace=ws)
+        assert (g.state.cfg.x_bits, g.state.cfg.w_bits) == (qp, pp) and g.strategy in ("tiled", "decode_tiled")
+        assert g.workspace_bytes <= ws.numel()
+        assert np.array_equal(g.run().cpu().numpy(), want), (g.config_name, M, N, K)
+        assert np.array_equal(g.run().cpu().numpy(), want)
+        if not signed and 8 in (qp, pp):  # the same with the weights' sums from their preparation
+            g = abq.Gemm(xd, wt, signed, w_tiled=True, value_bits=(q, p), x_planes_of=qp, workspace=ws, w_row_sums=abq.row_sums(wd))
+            assert np.array_equal(g.run().cpu().numpy(), want), (g.config_name, M, N, K)
+
+
 FIELD_PAIRS = [(3, 3), (5, 5), (6, 6), (7, 7), (8, 3), (6, 2)]  # a width of several fields on either side
 
 
