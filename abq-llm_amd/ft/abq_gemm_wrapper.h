@@ -37,8 +37,10 @@ struct ABQGroupedWeight {
                               // more than 16 rows run on the FP6 matrix cores
     const int *records_padded; // weights of 3, 5, 6 or 7 bits (e.g. the reference's bit-balanced 2-bit weights, three
                               // planes): the same weights as records of the next single-field width
-                              // (abq_relayout_planes_padded), or nullptr; with it, the decode-sized calls run the
-                              // prepared-operand decode kernel of that width instead of the one on plane operands
+                              // (abq_relayout_planes_padded), or nullptr; with it, every call runs the padded
+                              // pair's kernels on them: the prepared-operand decode kernel instead of the one on plane
+                              // operands, the LDS-staged prefill kernel instead of the register-staged one of the
+                              // odd widths; planes_tiled may then be nullptr
 };
 
 class ABQGEMMWrapper {

@@ -654,8 +654,31 @@ def main():
                 log("dequant decode W3A8 M=%d N=%d K=%d  %.2f us (%s, padded records); plane operands %.2f us" % (M, N, K, us, gs[0].strategy, us_planes))
                 del gs, out
             del Wp3, W3
+        # ... and a prefill of 1024 tokens on the same 3-bit weights: padded 4-bit records (the 4-bit pair's LDS-staged
+        # kernel) against the 3-bit records (the register-staged kernel of the odd widths)
+        pre3 = []
+        for (N, K) in SHAPES:
+            G = K // 128
+            w3 = random_planes(torch, (3, N, K // 32))
+            w3p, w3t = abq.relayout_planes_padded(w3, SIGNED), abq.relayout_planes(w3)
+            wsc = torch.rand((N, G), device="cuda") * 0.01 + 0.001
+            wz = torch.randint(-4, 4, (N, G), device="cuda").float()
+            x = torch.randn((1024, K), device="cuda", dtype=torch.float16)
+            xt, xsc, _, sums = abq.quant_pack_f16(x, Q_BITS, symmetric=True, tiled=True, group_size=128)
+            out = torch.empty((1024, N), dtype=torch.float16, device="cuda")
+            kw = dict(out=out, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc, group_size=128, w_zero=wz, x_group_sums=sums,
+                      x_tiled=True, w_tiled=True)
+            gp = abq.Gemm(xt, w3p, SIGNED, value_bits=(Q_BITS, 3), **kw)
+            us = time_rotating([gp])
+            us_own = time_rotating([abq.Gemm(xt, w3t, SIGNED, **kw)])
+            tops = 2.0 * 1024 * N * K / (us * 1e-6) / 1e12
+            pre3.append(dict(M=1024, N=N, K=K, w_bits=3, group_size=128, us=round(us, 2), tops=round(tops, 1),
+                             kernel="%s:%s" % (gp.strategy, gp.config_name), own_width_records_us=round(us_own, 2)))
+            log("dequant prefill W3A8 M=1024 N=%d K=%d  %.1f us  %.0f TOPS (padded records); 3-bit records %.1f us" % (N, K, us, tops, us_own))
+            del w3, w3p, w3t, out, xt
         extra["decode_group_scales"] = deq
         extra["decode_group_scales_w3a8"] = deq3
+        extra["prefill_group_scales_w3a8"] = pre3
 
     if want("small_batch"):
         # ------------------------------------------------------------ side measurement: 32 and 64 rows on prepared operands

@@ -374,7 +374,8 @@ static void gpu_paths()
     // values from a double-precision loop over the dequantised operands.  2-bit weights (prefill- and decode-sized
     // calls), and 3-bit weights (the reference's bit-balanced 2-bit quantiser writes three planes): at decode sizes as
     // padded records on the prepared-operand decode kernel of the 4-bit width, as planes on the plane-operand one,
-    // above that on the prefill kernel.
+    // above that on the prefill kernel of the padded pair (padded records, which then are the only copy handed over)
+    // or of the 3-bit records.
     auto dynamic_case = [&](const int WB, const int M, const bool padded_records, const bool keep_planes) {
         const int N = 192, K = 512, G = 128, groups = K / G;
         std::mt19937 r32(5 + WB + M);
@@ -415,7 +416,7 @@ static void gpu_paths()
         CHECK(abq_relayout_planes(d_wpl, d_wt, N, K, WB, stream) == ABQ_OK);
         CHECK(abq_relayout_planes_padded(d_wpl, d_wpad, N, K, WB, 1, stream) == ABQ_OK);
         CHECK(abq_weight_zero_term(d_wpl, N, K, WB, 1, d_wscale, d_wzero, G, d_term, stream) == ABQ_OK);
-        const ABQGroupedWeight weight = { reinterpret_cast<const int *>(d_wt), d_wscale, d_wzero, d_term, G,
+        const ABQGroupedWeight weight = { padded_records ? nullptr : reinterpret_cast<const int *>(d_wt), d_wscale, d_wzero, d_term, G,
                                           keep_planes ? reinterpret_cast<const int *>(d_wpl) : nullptr, nullptr,
                                           padded_records ? reinterpret_cast<const int *>(d_wpad) : nullptr };
         for (int symmetric = 1; symmetric >= 0; --symmetric) {
@@ -480,6 +481,9 @@ static void gpu_paths()
     dynamic_case(3, 8, true, false);   // quantiser + the 4-bit decode kernel on the padded records
     dynamic_case(3, 8, false, true);   // no padded records: the decode kernel on plane operands
     dynamic_case(5, 4, true, false);   // 5-bit weights as 8-bit records
+    dynamic_case(3, 300, true, false); // prefill on the padded records: the 4-bit pair's LDS-staged kernel
+    dynamic_case(3, 300, false, false); // ... and on the 3-bit records
+    dynamic_case(6, 130, true, false); // 6-bit weights as 8-bit records, prefill
 
     {   // weight file -> device weight -> dynamic GEMM: the file round-trips, and the GEMM on the loaded
         // weight equals a double-precision loop over the blob's own dequantised codes
