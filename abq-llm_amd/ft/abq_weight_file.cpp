@@ -186,10 +186,10 @@ ABQDeviceWeight::~ABQDeviceWeight() { release(); }
 
 void ABQDeviceWeight::release()
 {
-    for (void *p : { (void *)planes_, (void *)tiled_, (void *)fp6_, (void *)scale_, (void *)zero_, (void *)zero_term_ })
+    for (void *p : { (void *)planes_, (void *)tiled_, (void *)fp6_, (void *)padded_, (void *)scale_, (void *)zero_, (void *)zero_term_ })
         if (p)
             (void)hipFree(p);
-    planes_ = tiled_ = fp6_ = nullptr;
+    planes_ = tiled_ = fp6_ = padded_ = nullptr;
     scale_ = zero_ = zero_term_ = nullptr;
 }
 
@@ -226,6 +226,12 @@ bool ABQDeviceWeight::load(const ABQWeightBlob &blob, hipStream_t stream, std::s
             return false;
         rc = abq_relayout_planes_fp6(planes_, fp6_, (int)info_.n, (int)info_.k, (int)info_.bits, (int)info_.is_signed, stream);
     }
+    // padded records for the widths of several fields: the kernels of the next single-field width read those
+    if (rc == ABQ_OK && abq_padded_bits((int)info_.bits) != (int)info_.bits) {
+        if (!hip_ok(hipMalloc(&padded_, abq_planes_bytes((int)info_.n, (int)info_.k, abq_padded_bits((int)info_.bits))), "hipMalloc padded"))
+            return false;
+        rc = abq_relayout_planes_padded(planes_, padded_, (int)info_.n, (int)info_.k, (int)info_.bits, (int)info_.is_signed, stream);
+    }
     if (rc != ABQ_OK)
         return fail(error, std::string("weight preparation failed: ") + abq_status_string(rc));
     return hip_ok(hipStreamSynchronize(stream), "synchronise");
@@ -234,5 +240,6 @@ bool ABQDeviceWeight::load(const ABQWeightBlob &blob, hipStream_t stream, std::s
 ABQGroupedWeight ABQDeviceWeight::grouped() const
 {
     return ABQGroupedWeight{ reinterpret_cast<const int *>(tiled_), scale_, zero_, zero_term_, (int)info_.group_size,
-                             reinterpret_cast<const int *>(planes_), reinterpret_cast<const int *>(fp6_) };
+                             reinterpret_cast<const int *>(planes_), reinterpret_cast<const int *>(fp6_),
+                             reinterpret_cast<const int *>(padded_) };
 }

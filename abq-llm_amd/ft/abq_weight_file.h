@@ -68,7 +68,8 @@ bool abq_weight_file_read(const std::string &path, ABQWeightBlob *blob, std::str
 bool abq_weight_file_write_ft_bin(const std::string &path, const ABQWeightBlob &blob, std::string *error);
 
 // A weight matrix resident on the device, ready for both kernel families: the planes as they
-// are (decode kernels), the prefill layout, scales, zero points and the zero-point term.
+// are (decode kernels), the prefill layout, scales, zero points and the zero-point term; for the
+// widths the kernels read fastest in another form (FP6 records, padded records) that form as well.
 class ABQDeviceWeight {
 public:
     ABQDeviceWeight() = default;
@@ -89,5 +90,6 @@ public:
 private:
     ABQWeightHeader info_{};
     uint32_t *planes_ = nullptr, *tiled_ = nullptr, *fp6_ = nullptr; // fp6_: only for groups of 128 and at most 5 (4 unsigned) bits
+    uint32_t *padded_ = nullptr;                                     // only for 3, 5, 6, 7 bits: records of the next width of one field
     float *scale_ = nullptr, *zero_ = nullptr, *zero_term_ = nullptr;
 };

@@ -485,17 +485,20 @@ static void gpu_paths()
     dynamic_case(3, 300, false, false); // ... and on the 3-bit records
     dynamic_case(6, 130, true, false); // 6-bit weights as 8-bit records, prefill
 
-    {   // weight file -> device weight -> dynamic GEMM: the file round-trips, and the GEMM on the loaded
-        // weight equals a double-precision loop over the blob's own dequantised codes
-        const int M = 24, N = 160, K = 384, G = 64, groups = K / G;
-        std::mt19937 r32(11);
+    for (const int WB : { 4, 3 })
+    for (const int M : { 24, 3 }) {
+        // weight file -> device weight -> dynamic GEMM: the file round-trips, and the GEMM on the loaded
+        // weight equals a double-precision loop over the blob's own dequantised codes (3-bit weights: the loaded
+        // weight carries padded records, which the calls of every size run on)
+        const int N = 160, K = 384, G = 64, groups = K / G;
+        std::mt19937 r32(11 + WB + M);
         std::normal_distribution<float> nd(0.f, 0.05f), xd_(0.f, 1.f);
         std::vector<float> wf((size_t)N * K);
         for (auto &v : wf)
             v = nd(r32);
         ABQWeightBlob blob, back;
         std::string err;
-        CHECK(abq_quantize_weights(wf.data(), N, K, 4, false, G, &blob, &err));
+        CHECK(abq_quantize_weights(wf.data(), N, K, WB, false, G, &blob, &err));
         const std::string path = "/tmp/abq_test_weight.abqw";
         CHECK(abq_weight_file_write(path, blob, &err));
         CHECK(abq_weight_file_read(path, &back, &err));
@@ -505,12 +508,13 @@ static void gpu_paths()
         std::remove(path.c_str());
         ABQDeviceWeight dw;
         CHECK(dw.load(blob, stream, &err));
+        CHECK((dw.grouped().records_padded != nullptr) == (WB == 3));
         std::vector<int> codes((size_t)N * K);
-        abq_oracle_unpack(blob.planes.data(), codes.data(), N, K, 4, 1);
+        abq_oracle_unpack(blob.planes.data(), codes.data(), N, K, WB, 1);
         std::vector<uint16_t> ha((size_t)M * K);
         for (auto &h : ha)
             h = abq_oracle_f32_to_f16(xd_(r32));
-        ABQGEMMWrapper wrap(8, 4, true);
+        ABQGEMMWrapper wrap(8, WB, true);
         const size_t ws_bytes = wrap.dynamic_workspace_bytes(M, K, G);
         _Float16 *d_a, *d_d;
         char *d_ws;
