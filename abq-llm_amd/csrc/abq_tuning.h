@@ -19,4 +19,10 @@ int tile_operand_layout(const abq_tile_config &c);
 // loaded at run time come before the compiled-in ones.
 bool tuning_find(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group, int layout_mask, TunedTile *out);
 
+// A signed prefill-sized GEMM (more than 16 rows, no group scales) whose activations have 3, 5, 6 or 7 bits and whose
+// weights have 2, 4 or 8: the library runs it as the pair (activations padded to the next width of one field, the same
+// weights) when that pair has kernels on K-tiled records; the activations are converted per call anyway, the weight
+// records are the pair's own (abq_api.hip).
+bool activations_run_padded(int x_bits, int w_bits, int is_signed, int M, int group_size);
+
 } // namespace abq

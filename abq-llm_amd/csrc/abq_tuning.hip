@@ -205,6 +205,8 @@ abq_status abq_tuning_lookup(int x_bits, int w_bits, int is_signed, int M, int N
 
 int abq_preferred_weight_layout(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size)
 {
+    if (activations_run_padded(x_bits, w_bits, is_signed, M, group_size))
+        return ABQ_LAYOUT_TILED; // (whatever was measured on the pair's own kernels: the padded pair's run on these)
     TunedTile t;
     if (tuning_find(x_bits, w_bits, is_signed, M, N, K, group_size, 7, &t))
         return tile_operand_layout(t.cfg);

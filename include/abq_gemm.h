@@ -338,7 +338,12 @@ abq_status abq_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int ro
  * ABQ_STRATEGY_DECODE_TILED where that kernel exists for the pair and epilogue; a state
  * initialised with an explicit tile tuple of another strategy is refused (ABQ_ERR_UNSUPPORTED),
  * and so are a tiled and an FP6 operand together, an FP6 operand with group scales of groups other
- * than 128, and an FP6 operand of a bit pair or K that does not qualify. */
+ * than 128, and an FP6 operand of a bit pair or K that does not qualify.  A call that is refused leaves the state as
+ * it was.  One case changes the pair: signed activations of 3, 5, 6 or 7 bits that stay in planes, above 16 rows,
+ * against K-tiled weights of 2, 4 or 8 bits (W2A6): exec converts the activations anyway, so it writes them as records
+ * of the next width of one field and the state becomes that pair's (cfg.x_bits = abq_padded_bits, the codes' width
+ * kept as by abq_gemm_set_value_bits), which runs the LDS-staged kernel instead of the register-staged one of the odd
+ * widths; size the workspace with abq_gemm_workspace_bytes AFTER this call. */
 abq_status abq_gemm_set_operand_layout(abq_gemm_state *state, int x_layout, int w_layout);
 
 /* Decode without a packing launch (ABQGEMMWrapper::gemm of the reference packs A and runs the GEMM, two launches,

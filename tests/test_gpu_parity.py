@@ -614,6 +614,29 @@ def test_prefill_on_padded_weight_records(abq, oracle, q, p, signed):
             assert np.array_equal(g.run().cpu().numpy(), want), (g.config_name, M, N, K)
 
 
+def test_prefill_pads_activations_of_several_fields_by_itself(abq, oracle):
+    """Signed W2A6 above 16 rows, activations as planes, weights as their own K-tiled records: the library runs the pair
+    as W2A8 (exec extends the activation codes while it converts them), says so in the state, and sizes the workspace
+    for the wider records.  Unsigned pairs and decode-sized calls keep the pair's own kernels."""
+    rng = np.random.default_rng(77)
+    for (M, N, K) in [(17, 64, 512), (128, 200, 1408), (300, 130, 1152)]:
+        x, w = rand_vals(rng, M, K, 6, True), rand_vals(rng, N, K, 2, True)
+        x[1], x[2], w[0] = 31, -32, -2
+        xd, wd = planes_dev(oracle.pack_i32(x, 6)), planes_dev(oracle.pack_i32(w, 2))
+        g = abq.Gemm(xd, abq.relayout_planes(wd), True, w_tiled=True)
+        assert (g.state.cfg.x_bits, g.state.cfg.w_bits, g.strategy) == (8, 2, "tiled")
+        assert g.workspace_bytes >= M * K
+        ws = torch.empty(g.workspace_bytes, dtype=torch.uint8, device="cuda")
+        g = abq.Gemm(xd, abq.relayout_planes(wd), True, w_tiled=True, workspace=ws)
+        assert np.array_equal(g.run().cpu().numpy(), oracle.np_gemm(x, w)), (g.config_name, M, N, K)
+    x, w = rand_vals(rng, 40, 512, 6, False), rand_vals(rng, 64, 512, 2, False)
+    g = abq.Gemm(planes_dev(oracle.pack_i32(x, 6)), abq.relayout_planes(planes_dev(oracle.pack_i32(w, 2))), False, w_tiled=True)
+    assert g.state.cfg.x_bits == 6
+    x = rand_vals(rng, 8, 512, 6, True)
+    g = abq.Gemm(planes_dev(oracle.pack_i32(x, 6)), abq.relayout_planes(planes_dev(oracle.pack_i32(w, 2))), True, w_tiled=True)
+    assert g.state.cfg.x_bits == 6
+
+
 FIELD_PAIRS = [(3, 3), (5, 5), (6, 6), (7, 7), (8, 3), (6, 2)]  # a width of several fields on either side
 
 
