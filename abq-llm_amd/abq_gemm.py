@@ -38,7 +38,7 @@ EXPORTED = [
     "abq_gemm_exec_static", "abq_gemm_set_f16_activations",
     "abq_row_sums", "abq_gemm_set_row_sums", "abq_gemm_row_sums_ready",
     "abq_tuning_load", "abq_tuning_add", "abq_tuning_clear", "abq_tuning_enable_builtin", "abq_tuning_lookup",
-    "abq_preferred_weight_layout", "abq_padded_bits", "abq_relayout_planes_padded", "abq_gemm_set_value_bits",
+    "abq_preferred_weight_layout", "abq_preferred_weight_records", "abq_padded_bits", "abq_relayout_planes_padded", "abq_gemm_set_value_bits",
     "abq_gemm_set_padded_activations",
     "abq_relayout_planes_biased", "abq_gemm_set_biased_records", "abq_pack_f16_fp6",
 ]
@@ -147,6 +147,8 @@ def lib():
         L.abq_tuning_lookup.argtypes = [ci, ci, ci, ci, ci, ci, ci, ci, ctypes.POINTER(TileConfig), ctypes.POINTER(ctypes.c_float)]
         L.abq_preferred_weight_layout.argtypes = [ci] * 7
         L.abq_preferred_weight_layout.restype = ci
+        L.abq_preferred_weight_records.argtypes = [ci] * 7 + [ctypes.POINTER(ci)]
+        L.abq_preferred_weight_records.restype = ci
         L.abq_relayout_planes_biased.argtypes = [vp, vp, ci, ci, vp]
         L.abq_gemm_set_biased_records.argtypes = [ctypes.POINTER(GemmState), ci, ci]
         L.abq_padded_bits.argtypes = [ci]

@@ -218,4 +218,27 @@ int abq_preferred_weight_layout(int x_bits, int w_bits, int is_signed, int M, in
     return ABQ_LAYOUT_TILED;
 }
 
+int abq_preferred_weight_records(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size, int *record_bits)
+{
+    const int wq = abq_padded_bits(w_bits);
+    int bits = w_bits, layout;
+    if (wq == w_bits || wq == 0) {
+        layout = abq_preferred_weight_layout(x_bits, w_bits, is_signed, M, N, K, group_size);
+    } else if (M > 16 && is_signed && w_bits == 5 && abq_fp6_eligible(x_bits, w_bits, is_signed, K) && (group_size == 0 || group_size == 128)) {
+        layout = ABQ_LAYOUT_FP6; // twice the int8 rate beats the 8-bit records' staged kernel
+    } else {
+        // the padded pair's answer; FP6 records hold the codes themselves, whatever width they were declared with
+        layout = abq_preferred_weight_layout(abq_padded_bits(x_bits), wq, is_signed, M, N, K, group_size);
+        if (layout == ABQ_LAYOUT_FP6 && !abq_fp6_eligible(x_bits, w_bits, is_signed, K))
+            layout = ABQ_LAYOUT_TILED;
+        if (layout != ABQ_LAYOUT_FP6) {
+            layout = ABQ_LAYOUT_TILED;
+            bits = wq;
+        }
+    }
+    if (record_bits)
+        *record_bits = bits;
+    return layout;
+}
+
 } // extern "C"

@@ -398,6 +398,13 @@ abq_status abq_tuning_lookup(int x_bits, int w_bits, int is_signed, int M, int N
  * entry for the shape; without one, FP6 records for pairs that qualify (abq_fp6_eligible) from 65 rows up, K-tiled
  * records otherwise.  (A model that runs prefill and decode on one matrix keeps both where the memory allows.) */
 int abq_preferred_weight_layout(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size);
+/* The same for a loader that can also write padded records (abq_relayout_planes_padded): *record_bits receives the
+ * width of the records to write, w_bits or abq_padded_bits(w_bits).  Weights of 2, 4 or 8 bits: as above.  Weights of
+ * 3, 5, 6 or 7 bits run fastest on the kernels of the padded pair at every M, so the answer is that pair's
+ * (K-tiled records of the padded width, GEMM initialised with the padded pair and abq_gemm_set_value_bits; or FP6
+ * records, which are the same for both widths), except signed 5-bit weights under activations of at most 5 bits
+ * above 16 rows, which stay on FP6 records.  No counterpart in the reference. */
+int abq_preferred_weight_records(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size, int *record_bits);
 
 /* sums[row] = sum over k of the unsigned codes of a row of an operand in the plane layout ([bits][rows][k/32]).
  * For pairs with an unsigned 8-bit operand: the LDS-staged kernel feeds such an operand to the signed matrix

@@ -697,3 +697,31 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(4, 4, 16384, 4096, 11008, F6, group=128) == (256, 128, 128, 64, 64, 5)
     assert picked(4, 4, 1024, 4096, 4096, F6, group=128) == (128, 128, 128, 64, 64, 5)
     assert picked(4, 4, 512, 4096, 4096, F6, group=128) == (128, 64, 128, 64, 32, 5)
+
+
+def test_preferred_weight_records_name_the_padded_pair_for_widths_of_several_fields(abq):
+    """What a loader is told to write: for weights of 2, 4, 8 bits the layout abq_preferred_weight_layout names, at their
+    own width; for 3, 5, 6, 7 bits K-tiled records of the next single-field width at every M (the padded pair's
+    kernels), or FP6 records where that pair's answer is FP6 and the codes qualify; signed 5-bit weights under
+    narrow activations keep FP6 records above 16 rows."""
+    lib = abq.lib()
+    T, F6 = abq.LAYOUT_TILED, abq.LAYOUT_FP6
+    bits = ctypes.c_int(0)
+
+    def ask(q, p, signed, M, N=5120, K=5120, group=0):
+        layout = lib.abq_preferred_weight_records(q, p, signed, M, N, K, group, ctypes.byref(bits))
+        return layout, bits.value
+
+    for (q, p) in [(8, 2), (4, 4), (8, 8), (2, 2), (8, 4)]:
+        for M in (1, 8, 128, 2048):
+            assert ask(q, p, 1, M) == (lib.abq_preferred_weight_layout(q, p, 1, M, 5120, 5120, 0), p)
+    for M in (1, 8, 16, 128, 2048):
+        assert ask(6, 6, 1, M) == (T, 8) and ask(7, 7, 0, M) == (T, 8) and ask(5, 5, 0, M) == (T, 8)
+        assert ask(8, 3, 1, M) == (T, 4) and ask(8, 3, 1, M, group=128) == (T, 4)
+    assert ask(5, 5, 1, 128) == (F6, 5) and ask(5, 5, 1, 8) == (T, 8)
+    assert ask(8, 5, 1, 128) == (T, 8)            # activations too wide for FP6
+    # 3-bit weights under 3-bit activations: whatever the 4-bit pair is told, at the width that layout holds
+    for M in (8, 128, 2048):
+        want = lib.abq_preferred_weight_layout(4, 4, 1, M, 5120, 5120, 0)
+        assert ask(3, 3, 1, M) == ((F6, 3) if want == F6 else (T, 4))
+    assert lib.abq_preferred_weight_records(6, 6, 1, 128, 5120, 5120, 0, None) == T
