@@ -1120,7 +1120,7 @@ static abq_status switch_to_decode_tiled(abq_gemm_state *st, bool one_tile = fal
 // with zero points over M = 24 ... 128 on the LLaMA-7B linears (4096 x 4096, QKV, gate + up with the gate fused,
 // down); taken when estimated 10 % ahead: W2A8 32 x 4096 x 4096 8.3 against 17 us, 32 x 4096 x 11008 24 against 38;
 // the wide outputs of the 8-bit activations stay on the prefill kernel.
-static bool decode_tiled_grouped_pays(int x_bits, int w_bits, int M, int N, int K, int act)
+static bool decode_tiled_grouped_pays(int x_bits, int w_bits, int M, int N, int K, int act, int group_size)
 {
     if (M <= 16)
         return true;
@@ -1137,8 +1137,12 @@ static bool decode_tiled_grouped_pays(int x_bits, int w_bits, int M, int N, int 
     const double decode_us = 1.0 + blocks * per_block;
     // (up to one workgroup per compute unit the prefill kernel's waves split K: 4 + 0.42 us per K tile on weights that
     // come from HBM, W2A8 64 x 4096 x 4096 17.4, 64 x 4096 x 11008 38.2 us)
-    const long wgs = (long)((N + 63) / 64) * ((M + 127) / 128);
-    const double tiled_us = wgs > 256 ? 1.0 + 0.6 * 1.45 * (K / 128) : 4.0 + 0.42 * (K / 128);
+    // (groups of 128, up to one 64x64 workgroup per compute unit: that tile with the split, 5 + 0.26 us per K tile:
+    // 64 x 4096 x 4096 12.9, 64 x 4096 x 11008 26.8 us)
+    const long wgs = (long)((N + 63) / 64) * ((M + 127) / 128), wgs64 = (long)((N + 63) / 64) * ((M + 63) / 64);
+    const double tiled_us = group_size == 128 && wgs64 <= 256 ? 5.0 + 0.26 * (K / 128)
+                            : wgs > 256                        ? 1.0 + 0.6 * 1.45 * (K / 128)
+                                                               : 4.0 + 0.42 * (K / 128);
     return decode_us < 0.9 * tiled_us;
 }
 
@@ -1148,7 +1152,7 @@ static bool decode_tiled_grouped_fits(const abq_gemm_state *st, int group_size, 
     const KernelTable *t = find_table(registry().decode_tiled_grouped, c.x_bits, c.w_bits, c.is_signed);
     return t && t->count > 0 && st->auto_chosen && (group_size == 128 || group_size == 64) && (!act || st->N % 32 == 0) &&
            decode_tiled_grouped_rows(16, act ? 2 : 1, st->M, st->K, c.x_bits, group_size) != 0 &&
-           decode_tiled_grouped_pays(c.x_bits, c.w_bits, st->M, st->N, st->K, act);
+           decode_tiled_grouped_pays(c.x_bits, c.w_bits, st->M, st->N, st->K, act, group_size);
 }
 
 // Moves a state with group scales onto the tiled kernel's group-scale variants.
@@ -1204,6 +1208,14 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
                 if (usable(tg->entries[i]) && tg->entries[i].lds != 0 && block_m(tg->entries[i]) == (along_n ? 64 : 128) &&
                     block_n(tg->entries[i]) == (one_round ? 64 : 128) && tg->entries[i].wk == 2 &&
                     tg->entries[i].wm * tg->entries[i].wn == 4)
+                    pick = i;
+        // Grids of at most one 64x64 workgroup per compute unit (batches of 17 to 64 rows up to QKV's width, 256 rows on
+        // 4096 columns): that tile with the split, one MFMA tile per wave.  W2A8 with zero points, K = 4096: 12.6-13.5 us
+        // against 15.5-17.1 on 128x64 with the split; K = 11008 at 64-256 rows 26.8-28.8 against 33.4-34.7.
+        if ((long)((state->M + 63) / 64) * ((state->N + 63) / 64) <= 256)
+            for (int i = 0; i < tg->count; ++i)
+                if (usable(tg->entries[i]) && tg->entries[i].lds != 0 && block_m(tg->entries[i]) == 64 && block_n(tg->entries[i]) == 64 &&
+                    tg->entries[i].wk == 2)
                     pick = i;
         // a measured best tile for this shape and group size comes before the rules above
         TunedTile t;
@@ -1865,7 +1877,7 @@ int abq_prepared_decode_pays(int x_bits, int w_bits, int is_signed, int M, int N
         const KernelTable *t = find_table(reg.decode_tiled_grouped, x_bits, w_bits, is_signed);
         return t && t->count > 0 && (group_size == 128 || group_size == 64) && (!act || N % 32 == 0) &&
                        decode_tiled_grouped_rows(16, act ? 2 : 1, M, K, x_bits, group_size) != 0 &&
-                       decode_tiled_grouped_pays(x_bits, w_bits, M, N, K, act)
+                       decode_tiled_grouped_pays(x_bits, w_bits, M, N, K, act, group_size)
                    ? 1
                    : 0;
     }

@@ -147,7 +147,8 @@ template <int TM, int TN, int WM, int WN, int STAGE_BYTES> struct StagedOutputLd
 // row into the same accumulator), and while the matrix core works on one MFMA tile the vector ALU folds
 // the one finished before it into the fp32 accumulators (a convert and a multiply-add per element: as
 // many cycles as the four MFMAs take).  The last MFMA tile of a K tile is folded during the first of the
-// next K tile.
+// next K tile.  A wave of ONE MFMA tile (the 64 x 64 workgroup tile of small batches) keeps two int32
+// accumulators and alternates between them from K tile to K tile, folding the other one.
 //
 // WK > 1: WK groups of WM x WN waves share the workgroup's output tile and split K between them: a stage holds WK
 // consecutive K tiles, group wk loads and multiplies the wk-th of them, and the groups' partial tiles meet in LDS
@@ -171,7 +172,7 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     constexpr int NI = NIA + BN * TB::kUnits / 64;             // ... and in all
     constexpr int NPR = (NI + NW - 1) / NW;                    // per wave
     constexpr int NPW = NPR + (GROUPED ? 1 : 0);               // GROUPED: and one load of 64 scales (256 bytes)
-    static_assert(!GROUPED || (TM * TN >= 2 && BN / 64 <= WM * WN), "group scales: two MFMA tiles per wave or more");
+    static_assert(!GROUPED || BN / 64 <= WM * WN || BN < 64, "group scales: a wave per block of 64 scales");
     constexpr int kSteps = FP6 ? 2 : 4;                        // MFMA K steps per tile of 128
     constexpr bool FLIP_X = !FP6 && !SIGNED && QB == 8, FLIP_W = !FP6 && !SIGNED && PB == 8; // fed as value - 128
     static_assert(!GROUPED || !(FLIP_X || FLIP_W), "no group scales on unsigned 8-bit operands");
@@ -237,13 +238,14 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
 
     using Acc = typename std::conditional<FP6, v16f, v16i>::type;
     Acc acc[TM][TN];
+    Acc acc_alt[TM][TN]; // GROUPED with one MFMA tile per wave: the accumulator of the odd K tiles
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e)
-                acc[i][j][e] = 0;
+                acc[i][j][e] = acc_alt[i][j][e] = 0;
 
     unsigned char *lds_a = smem + wk * BUF_BYTES; // the K group's tile within a stage
     unsigned char *lds_b = lds_a + BM * TA::kRow;
@@ -386,21 +388,21 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     // step k % kSteps, the first one starting from zero); beside it the vector ALU folds its share (a
     // quarter, or half for FP6) of the tile finished before u: tile u - 1 of this K tile, or for u = 0 the last tile of the previous K tile (all
     // zeros, with a zero scale, when there is none).
-#define ABQ_STAGED_K_TILE_G(KT, QC, QN)                                                                         \
+#define ABQ_STAGED_K_TILE_G(KT, QC, QN, ACC, ACC_PREV)                                                          \
     {                                                                                                           \
         constexpr int NU = TM * TN;                                                                             \
         read_scales(sc_next, st_rd);                                                                            \
         _Pragma("unroll") for (int k = 0; k < NM; ++k)                                                          \
         {                                                                                                       \
             const int u = k / kSteps, ks = k % kSteps, uf = (u + NU - 1) % NU;                                  \
-            mfma(acc[u / TN][u % TN], QC, u / TN, u % TN, ks, ks == 0);                                         \
+            mfma(ACC[u / TN][u % TN], QC, u / TN, u % TN, ks, ks == 0);                                         \
             _Pragma("unroll") for (int d = k * NPW / NM; d < (k + 1) * NPW / NM; ++d)                           \
                 request(st_req, d);                                                                             \
             _Pragma("unroll") for (int p = k * NR / NM; p < (k + 1) * NR / NM; ++p)                             \
                 read_piece(QN, st_rd, p);                                                                       \
             const float scf = u == 0 ? sc_last : sc_cur[uf % TN];                                               \
             _Pragma("unroll") for (int e = (16 / kSteps) * ks; e < (16 / kSteps) * (ks + 1); ++e)               \
-                facc[uf / TN][uf % TN][e] += (float)acc[uf / TN][uf % TN][e] * scf;                             \
+                facc[uf / TN][uf % TN][e] += (float)ACC_PREV[uf / TN][uf % TN][e] * scf;                        \
             __builtin_amdgcn_sched_barrier(0);                                                                  \
         }                                                                                                       \
         sc_last = sc_cur[TN - 1];                                                                               \
@@ -414,13 +416,20 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     }
 
     int kt = 0;
-    if constexpr (GROUPED) {
+    if constexpr (GROUPED && TM * TN == 1) {
         for (; kt + 2 <= ktiles; kt += 2) {
-            ABQ_STAGED_K_TILE_G(kt, q0, q1)
-            ABQ_STAGED_K_TILE_G(kt + 1, q1, q0)
+            ABQ_STAGED_K_TILE_G(kt, q0, q1, acc, acc_alt)
+            ABQ_STAGED_K_TILE_G(kt + 1, q1, q0, acc_alt, acc)
         }
         if (kt < ktiles)
-            ABQ_STAGED_K_TILE_G(kt, q0, q1)
+            ABQ_STAGED_K_TILE_G(kt, q0, q1, acc, acc_alt)
+    } else if constexpr (GROUPED) {
+        for (; kt + 2 <= ktiles; kt += 2) {
+            ABQ_STAGED_K_TILE_G(kt, q0, q1, acc, acc)
+            ABQ_STAGED_K_TILE_G(kt + 1, q1, q0, acc, acc)
+        }
+        if (kt < ktiles)
+            ABQ_STAGED_K_TILE_G(kt, q0, q1, acc, acc)
     } else if constexpr (WK == 1) {
         for (; kt + 2 <= ktiles; kt += 2) {
             ABQ_STAGED_K_TILE(kt, q0, q1, true)
@@ -449,10 +458,12 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
     staged_wait_loads<0>(); // the clamped requests past the last tile: nothing of ours may be in flight below
 
     if constexpr (GROUPED) {
-        // the last MFMA tile of the last K tile is still to be folded
+        // the last MFMA tile of the last K tile is still to be folded (one tile per wave: the accumulator of that
+        // K tile's parity)
+        const bool in_alt = TM * TN == 1 && (ktiles & 1) == 0;
 #pragma unroll
         for (int e = 0; e < 16; ++e)
-            facc[TM - 1][TN - 1][e] += (float)acc[TM - 1][TN - 1][e] * sc_last;
+            facc[TM - 1][TN - 1][e] += (float)(in_alt ? acc_alt[0][0][e] : acc[TM - 1][TN - 1][e]) * sc_last;
     }
     if constexpr (WK > 1) {
         // The K groups' partial tiles: group 1, 2, .. in turn leave theirs in LDS (lane-contiguous 16-byte pieces,
@@ -501,7 +512,8 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
             return;
     }
     if constexpr (GROUPED) {
-        group_scale_epilogue<TM, TN, WM, WN, LDS_BYTES>(a, facc, smem, M, N, m0, n0, wm, wn, r, g, tid);
+        // (the integer tiles have the registers to run the zero-point loads ahead of their use)
+        group_scale_epilogue<TM, TN, WM, WN, LDS_BYTES, FP6 ? 0 : TM * TN == 1 ? 2 : TM * TN == 2 ? 1 : 0>(a, facc, smem, M, N, m0, n0, wm, wn, r, g, tid);
         return;
     }
 

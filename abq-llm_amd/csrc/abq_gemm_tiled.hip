@@ -556,17 +556,18 @@ static const KernelEntry kUnsigned[] = { ABQ_TILED_VARIANTS(ABQ_ENTRY_F) ABQ_TIL
 #define ABQ_SGENTRY(SG, TM, TN, WM, WN)                                                                  \
     { 32, TM, TN, WM, WN, 1, 4, &launch_mfma_staged<ABQ_Q, ABQ_P, SG, false, TM, TN, WM, WN, true>, 128, \
       StagedStages<ABQ_Q, ABQ_P, false, TM, TN, WM, WN, true>::kLds },
-// (the 128 x 64 and 128 x 128 tiles also with two groups of waves that split K, for grids of one round)
+// (the 128 x 64 and 128 x 128 tiles also with two groups of waves that split K, for grids of one round; the 64 x 64
+// tile, one MFMA tile per wave, plain and split, for batches of 17 to 64 rows)
 #define ABQ_SGENTRY_K(SG, TM, TN, WM, WN, WK)                                                                  \
     { 32, TM, TN, WM, WN, WK, 4, &launch_mfma_staged<ABQ_Q, ABQ_P, SG, false, TM, TN, WM, WN, true, WK>, 128, \
       StagedStages<ABQ_Q, ABQ_P, false, TM, TN, WM, WN, true, WK>::kLds },
 #if ABQ_Q == 8 && ABQ_P == 8
 // two fragment sets of 64x64 8-bit operands, the int32 and the fp32 accumulators do not fit 256 registers
-#define ABQ_STAGED_GROUPED(SG) ABQ_SGENTRY(SG, 2, 1, 2, 2) ABQ_SGENTRY_K(SG, 2, 1, 2, 2, 2)
+#define ABQ_STAGED_GROUPED(SG) ABQ_SGENTRY(SG, 2, 1, 2, 2) ABQ_SGENTRY_K(SG, 2, 1, 2, 2, 2) ABQ_SGENTRY(SG, 1, 1, 2, 2) ABQ_SGENTRY_K(SG, 1, 1, 2, 2, 2)
 #else
 #define ABQ_STAGED_GROUPED(SG)                                                                                          \
     ABQ_SGENTRY(SG, 2, 2, 4, 2) ABQ_SGENTRY(SG, 2, 2, 2, 2) ABQ_SGENTRY(SG, 2, 1, 2, 2) ABQ_STAGED_WIDE_N_GROUPED(SG) \
-    ABQ_SGENTRY_K(SG, 2, 1, 2, 2, 2) ABQ_SGENTRY_K(SG, 2, 2, 2, 2, 2)
+    ABQ_SGENTRY_K(SG, 2, 1, 2, 2, 2) ABQ_SGENTRY_K(SG, 2, 2, 2, 2, 2) ABQ_SGENTRY(SG, 1, 1, 2, 2) ABQ_SGENTRY_K(SG, 1, 1, 2, 2, 2)
 #endif
 static const KernelEntry kSignedGrouped[] = { ABQ_GROUPED_VARIANTS(ABQ_GENTRY_T) ABQ_STAGED_GROUPED(true) };
 #if ABQ_Q < 8 && ABQ_P < 8

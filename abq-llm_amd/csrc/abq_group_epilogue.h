@@ -73,18 +73,19 @@ typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 
-// Eight consecutive per-group values of one row, groups [gb, gb + 8) of `groups`, zeros past the end.  `whole`:
-// the eight exist and rows start on 16-byte boundaries (wave-uniform), so two 16-byte loads do.
-template <typename T> __device__ __forceinline__ void load_groups8(const T *row, int gb, int groups, bool whole, T (&v)[8])
+// Eight consecutive per-group values of one row, groups [gb, gb + 8) of `groups`, zeros past the end.  Where the
+// eight exist they come as two 16-byte loads that ask for 4-byte alignment only (rows of 86 groups, K = 11008, start
+// anywhere); the lanes of a last, partial chunk load one by one.
+template <typename T> __device__ __forceinline__ void load_groups8(const T *row, int gb, int groups, T (&v)[8])
 {
-    if (whole) {
-        struct alignas(16) Q { T q[4]; };
+    typedef T quad __attribute__((ext_vector_type(4), aligned(4)));
+    if (gb + 8 <= groups) {
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
-            const Q t = *reinterpret_cast<const Q *>(row + gb + 4 * c);
+            const quad t = *reinterpret_cast<const quad *>(row + gb + 4 * c);
 #pragma unroll
             for (int d = 0; d < 4; ++d)
-                v[4 * c + d] = t.q[d];
+                v[4 * c + d] = t[d];
         }
     } else {
 #pragma unroll
@@ -93,19 +94,32 @@ template <typename T> __device__ __forceinline__ void load_groups8(const T *row,
     }
 }
 
-// Eight groups (from gb on) of the lane's TM activation rows and TN weight rows: group sums, scales, zero points.
+// Sixteen groups (from gb on) of the lane's TM activation rows and TN weight rows: group sums, scales, zero points.
+template <int TM, int TN> struct ZeroPointChunk {
+    int sx[2][TM][8];
+    float ws[2][TN][8], wz[2][TN][8];
+};
+
 template <int TM, int TN>
-__device__ __forceinline__ void zero_point_loads(const GemmArgs &a, const uint32_t (&arow)[TM], const uint32_t (&brow)[TN], int gb,
-                                                 int groups, bool whole, int (&sx)[TM][8], float (&ws)[TN][8], float (&wz)[TN][8])
+__device__ __forceinline__ void zero_point_loads_half(const GemmArgs &a, const uint32_t (&arow)[TM], const uint32_t (&brow)[TN], int gb,
+                                                      int groups, ZeroPointChunk<TM, TN> &c, int h)
 {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-        load_groups8(a.x_group_sums + arow[i], gb, groups, whole, sx[i]);
+        load_groups8(a.x_group_sums + arow[i], gb + 8 * h, groups, c.sx[h][i]);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        load_groups8(a.w_scale + brow[j], gb, groups, whole, ws[j]);
-        load_groups8(a.w_zero + brow[j], gb, groups, whole, wz[j]);
+        load_groups8(a.w_scale + brow[j], gb + 8 * h, groups, c.ws[h][j]);
+        load_groups8(a.w_zero + brow[j], gb + 8 * h, groups, c.wz[h][j]);
     }
+}
+
+template <int TM, int TN>
+__device__ __forceinline__ void zero_point_loads(const GemmArgs &a, const uint32_t (&arow)[TM], const uint32_t (&brow)[TN], int gb,
+                                                 int groups, ZeroPointChunk<TM, TN> &c)
+{
+    zero_point_loads_half<TM, TN>(a, arow, brow, gb, groups, c, 0);
+    zero_point_loads_half<TM, TN>(a, arow, brow, gb, groups, c, 1);
 }
 
 // facc -= (the eight groups' sums) x (their w_scale * w_zero)^T: four bf16 MFMAs per MFMA tile, see below.
@@ -161,9 +175,11 @@ __device__ __forceinline__ void zero_point_product(const int (&sx)[TM][8], const
 // for the K slots 8 g .. 8 g + 7, i.e. for two groups; which two is free as long as both operands agree, and the
 // choice here, groups 16 g + 2 q and 16 g + 2 q + 1 for instruction q of the chunk, lets every lane read its
 // sixteen groups of a row as 64 contiguous bytes straight from global memory: no staging, no barrier.
-// LDS_BYTES: size of the workgroup's LDS at smem.  LOADS_FIRST: a chunk's loads are all requested before any is
-// used (one memory latency per chunk instead of two, 48 more registers).
-template <int TM, int TN, int WM, int WN, int LDS_BYTES, bool LOADS_FIRST = false>
+// LDS_BYTES: size of the workgroup's LDS at smem.  AHEAD: how far the loads of the zero-point term run ahead of their
+// use, for the kernels that have the registers: 0 = half a chunk is loaded, multiplied, then the other half (two memory
+// latencies per chunk); 1 = a chunk's loads are all requested before any is used; 2 = and the next chunk's before the
+// current one is multiplied (K = 11008 has three chunks).
+template <int TM, int TN, int WM, int WN, int LDS_BYTES, int AHEAD = 0>
 __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&facc)[TM][TN], unsigned char *smem, int M,
                                                      int N, int m0, int n0, int wm, int wn, int r, int g, int tid)
 {
@@ -189,8 +205,6 @@ __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&f
 
     if (a.w_zero) {
         const int groups = a.K / a.group_size;
-        const bool rows16 = (groups & 3) == 0 && ((reinterpret_cast<size_t>(a.x_group_sums) | reinterpret_cast<size_t>(a.w_scale) |
-                                                   reinterpret_cast<size_t>(a.w_zero)) & 15) == 0;
         // rows of this lane in the three arrays (32-bit element offsets: the arrays hold fewer than 2^32 elements)
         uint32_t arow[TM], brow[TN];
 #pragma unroll
@@ -199,19 +213,37 @@ __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&f
 #pragma unroll
         for (int j = 0; j < TN; ++j)
             brow[j] = (uint32_t)min(n0 + wn * 32 * TN + j * 32 + r, N - 1) * (uint32_t)groups;
-        for (int g0 = 0; g0 < groups; g0 += 32) {
-            const bool whole = rows16 && g0 + 32 <= groups; // wave-uniform
-            // half of the lane's sixteen groups at a time
-            const int gb = g0 + 16 * g;
-            int sx0[TM][8], sx1[TM][8];
-            float ws0[TN][8], wz0[TN][8], ws1[TN][8], wz1[TN][8];
-            zero_point_loads<TM, TN>(a, arow, brow, gb, groups, whole, sx0, ws0, wz0);
-            if constexpr (LOADS_FIRST)
-                zero_point_loads<TM, TN>(a, arow, brow, gb + 8, groups, whole, sx1, ws1, wz1);
-            zero_point_product<TM, TN>(sx0, ws0, wz0, facc);
-            if constexpr (!LOADS_FIRST)
-                zero_point_loads<TM, TN>(a, arow, brow, gb + 8, groups, whole, sx1, ws1, wz1);
-            zero_point_product<TM, TN>(sx1, ws1, wz1, facc);
+        ZeroPointChunk<TM, TN> c0, c1;
+        auto multiply = [&](const ZeroPointChunk<TM, TN> &c) {
+            zero_point_product<TM, TN>(c.sx[0], c.ws[0], c.wz[0], facc);
+            zero_point_product<TM, TN>(c.sx[1], c.ws[1], c.wz[1], facc);
+        };
+        // (a lane's sixteen groups of chunk g0: from g0 + 16 g on)
+        if constexpr (AHEAD == 2) {
+            zero_point_loads<TM, TN>(a, arow, brow, 16 * g, groups, c0);
+            for (int g0 = 0; g0 < groups; g0 += 64) {
+                const bool second = g0 + 32 < groups; // wave-uniform
+                if (second)
+                    zero_point_loads<TM, TN>(a, arow, brow, g0 + 32 + 16 * g, groups, c1);
+                multiply(c0);
+                if (second) {
+                    if (g0 + 64 < groups)
+                        zero_point_loads<TM, TN>(a, arow, brow, g0 + 64 + 16 * g, groups, c0);
+                    multiply(c1);
+                }
+            }
+        } else if constexpr (AHEAD == 1) {
+            for (int g0 = 0; g0 < groups; g0 += 32) {
+                zero_point_loads<TM, TN>(a, arow, brow, g0 + 16 * g, groups, c0);
+                multiply(c0);
+            }
+        } else {
+            for (int g0 = 0; g0 < groups; g0 += 32) {
+                zero_point_loads_half<TM, TN>(a, arow, brow, g0 + 16 * g, groups, c0, 0);
+                zero_point_product<TM, TN>(c0.sx[0], c0.ws[0], c0.wz[0], facc);
+                zero_point_loads_half<TM, TN>(a, arow, brow, g0 + 16 * g, groups, c0, 1);
+                zero_point_product<TM, TN>(c0.sx[1], c0.ws[1], c0.wz[1], facc);
+            }
         }
     }
     if (a.x_zero) {

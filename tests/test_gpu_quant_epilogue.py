@@ -464,21 +464,24 @@ def _staged_grouped_lds(cfg):
 def test_group_scale_staged_kernel_every_tile(abq, oracle, q, p, signed):
     """Groups of 128 on pairs of 2-, 4- and 8-bit fields run on the kernel that loads the records and
     the scales straight into LDS; every tile it is built for, picked by its tuple, with zero points
-    on both sides, on shapes with ragged edges, fewer K tiles than LDS stages and an odd tile count."""
+    on both sides, on shapes with ragged edges, fewer K tiles than LDS stages, odd and even tile counts (the 64 x 64
+    tile, one MFMA tile per wave, alternates between two accumulators) and a K of 86 groups (three chunks of the
+    zero-point term, rows of the scale arrays that start off 16-byte boundaries)."""
     from oracle import quantizer as Q
     rng = np.random.default_rng(100 * q + 10 * p + signed)
     tiles = [c for c in abq.native_configs(q, p, signed)
-             if c.nstage == 4 and c.warp_k == 128 and (c.warp_m, c.warp_n) in ((64, 64), (64, 32), (32, 64)) and
-             (c.block_m, c.block_n) in ((256, 128), (128, 128), (128, 64), (128, 256), (64, 128))]
+             if c.nstage == 4 and c.warp_k == 128 and (c.warp_m, c.warp_n) in ((64, 64), (64, 32), (32, 64), (32, 32)) and
+             (c.block_m, c.block_n) in ((256, 128), (128, 128), (128, 64), (128, 256), (64, 128), (64, 64))]
     assert ((128, 256) in [(c.block_m, c.block_n) for c in tiles]) == (q > p)
     assert [c.block_k for c in tiles if (c.block_m, c.block_n) == (64, 128)] == ([128, 256] if q > p else [])
     if (q, p) == (8, 8):
-        tiles = [c for c in tiles if (c.block_m, c.block_n) == (128, 64)]
+        tiles = [c for c in tiles if (c.block_m, c.block_n) in ((128, 64), (64, 64))]
     assert tiles
+    assert [c.block_k for c in tiles if (c.block_m, c.block_n) == (64, 64)] == [128, 256]
     assert [c.block_k for c in tiles if (c.block_m, c.block_n) == (128, 64)] == [128, 256]  # plain, and waves that split K
     lo_x, hi_x = (-(1 << (q - 1)), 1 << (q - 1)) if signed else (0, 1 << q)
     lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed else (0, 1 << p)
-    for (M, N, K) in [(300, 200, 640), (70, 330, 256), (129, 65, 128), (200, 136, 1536)]:
+    for (M, N, K) in [(300, 200, 640), (70, 330, 256), (129, 65, 128), (200, 136, 1536), (70, 100, 11008)]:
         G = K // 128
         x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
         w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
@@ -533,13 +536,14 @@ def test_group_scale_decode_kernel_on_wide_outputs_of_more_than_eight_rows(abq, 
 @pytest.mark.parametrize("q,p,act", [(8, 2, False), (4, 4, False), (8, 2, True)])
 def test_group_scale_tiles_whose_waves_split_k_are_the_default_on_grids_of_one_round(abq, oracle, q, p, act):
     """Grids of at most one workgroup per compute unit run the tile with two groups of waves that split K inside the
-    workgroup: 128x64 while that makes at most 256 workgroups, 128x128 beyond while that does, 64x128 for wide outputs
+    workgroup: 64x64 while that makes at most 256 workgroups, then 128x64, 128x128 beyond while that does, 64x128 for wide outputs
     of at most 64 rows (activations wider than the weights); an odd number of K tiles (the last trip has one group
     without a tile), zero points on both sides, ragged edges, the fused SiLU gate."""
     from oracle import quantizer as Q
     rng = np.random.default_rng(7100 + 10 * q + p + act)
     lo_x, hi_x, lo_w, hi_w = -(1 << (q - 1)), 1 << (q - 1), -(1 << (p - 1)), 1 << (p - 1)
-    cases = [(300, 192, 640, (128, 64, 256)), (1040, 2144, 384, (128, 128, 256)), (130, 16000, 256, (128, 128, 256))]
+    cases = [(300, 192, 640, (64, 64, 256)), (300, 3840, 384, (128, 64, 256)), (1040, 2144, 384, (128, 128, 256)),
+             (130, 16000, 256, (128, 128, 256))]
     if q > p:
         cases.append((40, 16640, 384, (64, 128, 256)))
     for (M, N, K, tile) in cases:

@@ -679,8 +679,12 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(8, 2, 128, 4096, 4096, T, group=64) == (64, 64, 128, 32, 32, 4)
     # up to one 128x64 workgroup per compute unit: the tile whose waves split K (its stages fill a compute unit's LDS)
     assert picked(8, 2, 512, 4096, 4096, T, group=128) == (128, 64, 256, 64, 32, 4)
-    assert picked(8, 2, 128, 4096, 11008, T, group=128) == (128, 64, 256, 64, 32, 4)
     assert picked(8, 2, 128, 12288, 4096, T, group=128) == (128, 64, 256, 64, 32, 4)
+    # up to one 64x64 workgroup per compute unit: that tile with the split (one MFMA tile per wave)
+    assert picked(8, 2, 128, 4096, 11008, T, group=128) == (64, 64, 256, 32, 32, 4)
+    assert picked(8, 2, 64, 12288, 4096, T, group=128) == (64, 64, 256, 32, 32, 4)
+    assert picked(8, 2, 256, 4096, 4096, T, group=128) == (64, 64, 256, 32, 32, 4)
+    assert picked(8, 8, 64, 4096, 4096, T, group=128) == (64, 64, 256, 32, 32, 4)
     # 384 workgroups would be two rounds of it: the 128x128 tile with the same split while that makes one round
     assert picked(8, 2, 192, 12288, 4096, T, group=128) == (128, 128, 256, 64, 64, 4)
     assert picked(8, 2, 128, 22016, 4096, T, group=128) == (128, 128, 256, 64, 64, 4)
