@@ -161,6 +161,46 @@ __device__ __forceinline__ void zero_point_product(const int (&sx)[TM][8], const
             }
 }
 
+// A wave's 64 x 16 bytes from global memory straight into LDS at lds_addr + 16 * lane (`base` the same in every lane,
+// `offset` the lane's byte offset from it), and the wait for every such load of the wave.
+__device__ __forceinline__ void epilogue_load_to_lds(const void *base, uint32_t offset, unsigned lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(offset),
+                 "s"(base)
+                 : "memory");
+}
+
+// Half h of a chunk that the workgroup has staged in LDS (see group_scale_epilogue): the lane's eight groups of its TM
+// activation rows and TN weight rows.  A staged row is 128 bytes at row_at(row), its 16-byte pieces permuted by the
+// row number.
+template <int TM, int TN, typename RowAt>
+__device__ __forceinline__ void zero_point_reads_half(RowAt row_at, int row_a, int row_s, int row_z, int g, int h,
+                                                      ZeroPointChunk<TM, TN> &c)
+{
+    typedef int quad_i __attribute__((ext_vector_type(4)));
+    typedef float quad_f __attribute__((ext_vector_type(4)));
+    auto at = [&](int row, int piece) { return row_at(row) + 16 * (piece ^ ((row >> 1) & 7)); };
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        const int piece = 4 * g + 2 * h + p;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const quad_i v = *reinterpret_cast<const quad_i *>(at(row_a + 32 * i, piece));
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                c.sx[h][i][4 * p + d] = v[d];
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const quad_f s4 = *reinterpret_cast<const quad_f *>(at(row_s + 32 * j, piece));
+            const quad_f z4 = *reinterpret_cast<const quad_f *>(at(row_z + 32 * j, piece));
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                c.ws[h][j][4 * p + d] = s4[d], c.wz[h][j][4 * p + d] = z4[d];
+        }
+    }
+}
+
 // facc[i][j][e]: MFMA tile (i, j) of this wave, element e in the 32x32 accumulator layout (row
 // 8 * (e / 4) + 4 * g + e % 4, column r).  smem: the workgroup's LDS, free for reuse once a barrier has
 // been passed (only the fp16 store uses it).
@@ -179,7 +219,35 @@ __device__ __forceinline__ void zero_point_product(const int (&sx)[TM][8], const
 // use, for the kernels that have the registers: 0 = half a chunk is loaded, multiplied, then the other half (two memory
 // latencies per chunk); 1 = a chunk's loads are all requested before any is used; 2 = and the next chunk's before the
 // current one is multiplied (K = 11008 has three chunks).
-template <int TM, int TN, int WM, int WN, int LDS_BYTES, int AHEAD = 0>
+// VIA_LDS (kernels whose K loop leaves the whole LDS free, every wave of the workgroup here): the whole chunks of rows
+// that start on 16-byte boundaries come through LDS instead.  A lane's 16-byte pieces of 32 different rows touch 32
+// cache lines per load instruction and use 32 bytes of each; with all waves of a compute unit doing that over some
+// 100 KB of lines the 32 KB L1 fetches every line several times (QKV of LLaMA-7B at 16384 tokens: the term cost 10 %
+// of the GEMM).  Staged, a load instruction takes eight whole rows of the workgroup's tile (every line once, no
+// registers), and the lanes pick their pieces out of LDS.
+// (Requesting the first chunk from inside the K loop's last trips, whose load slots and stages go to waste, was built
+// and dropped: branches in the loop body, or copies of it with other requests, cost the integer tiles 40-90 spilled
+// registers.)
+template <int RA, int RB>
+__device__ __forceinline__ uint32_t zero_point_unit_offset(const GemmArgs &a, int u, int lane, int m0, int n0, int M, int N, int groups,
+                                                           int first, const void **base)
+{
+    const int row = 8 * u + (lane >> 3);
+    const int piece = (lane & 7) ^ ((row >> 1) & 7);
+    // (a unit lies in one of the three arrays: RA and RB are multiples of 32)
+    *base = 8 * u < RA ? (const void *)a.x_group_sums : 8 * u < RA + RB ? (const void *)a.w_scale : (const void *)a.w_zero;
+    const int grow = row < RA ? min(m0 + row, M - 1) : min(n0 + (row < RA + RB ? row - RA : row - RA - RB), N - 1);
+    // (a last, partial chunk: pieces past the row's end bring its last piece once more; the reader drops them)
+    return ((uint32_t)grow * (uint32_t)groups + (uint32_t)min(first + 4 * piece, groups - 4)) * 4u;
+}
+
+__device__ __forceinline__ bool zero_point_rows_aligned(const GemmArgs &a, int groups)
+{
+    return (groups & 3) == 0 && ((reinterpret_cast<size_t>(a.x_group_sums) | reinterpret_cast<size_t>(a.w_scale) |
+                                  reinterpret_cast<size_t>(a.w_zero)) & 15) == 0;
+}
+
+template <int TM, int TN, int WM, int WN, int LDS_BYTES, int AHEAD = 0, bool VIA_LDS = false>
 __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&facc)[TM][TN], unsigned char *smem, int M,
                                                      int N, int m0, int n0, int wm, int wn, int r, int g, int tid)
 {
@@ -218,10 +286,92 @@ __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&f
             zero_point_product<TM, TN>(c.sx[0], c.ws[0], c.wz[0], facc);
             zero_point_product<TM, TN>(c.sx[1], c.ws[1], c.wz[1], facc);
         };
+        int first = 0; // first group of the chunks still to do
+        constexpr int RA = 32 * TM * WM, RB = 32 * TN * WN; // rows of the workgroup's tile
+        if constexpr (VIA_LDS && (RA + 2 * RB) * 128 <= LDS_BYTES) {
+            const int ra = wm * 32 * TM + r, rs = RA + wn * 32 * TN + r; // the lane's rows among the staged ones
+            {
+                const bool rows16 = zero_point_rows_aligned(a, groups);
+                const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+                const unsigned lds0 = (unsigned)(size_t)smem;
+                // LDS: the tile's RA rows of group sums, its RB rows of scales, its RB rows of zero points, 128 bytes
+                // each; a load instruction brings eight rows, the waves take them in turn
+                constexpr int UNITS = (RA + 2 * RB) / 8;
+                for (; first < groups; first += 32) {
+                    __syncthreads(); // every wave is through with what the LDS held (the stages; the chunk before)
+                    if (rows16) {
+                        for (int u = wave; u < UNITS; u += WM * WN) { // wave-uniform
+                            const void *base;
+                            const uint32_t off = zero_point_unit_offset<RA, RB>(a, u, lane, m0, n0, M, N, groups, first, &base);
+                            epilogue_load_to_lds(base, off, lds0 + u * 1024);
+                        }
+                    } else {
+                        // rows that start off 16-byte boundaries (K = 11008: 86 groups): the same units through registers,
+                        // three loads of a wave in flight at a time (a 16-byte load into registers asks for 4-byte alignment
+                        // only); the piece that straddles the end of a row comes word by word
+                        typedef unsigned int quad_u __attribute__((ext_vector_type(4)));
+                        typedef unsigned int quad_u4 __attribute__((ext_vector_type(4), aligned(4)));
+                        for (int u0 = wave; u0 < UNITS; u0 += 3 * WM * WN) {
+                            quad_u v[3];
+#pragma unroll
+                            for (int b = 0; b < 3; ++b) {
+                                const int u = u0 + b * WM * WN;
+                                if (u < UNITS) { // wave-uniform
+                                    const int row = 8 * u + (lane >> 3);
+                                    const int piece = (lane & 7) ^ ((row >> 1) & 7);
+                                    const int grow = row < RA ? min(m0 + row, M - 1) : min(n0 + (row < RA + RB ? row - RA : row - RA - RB), N - 1);
+                                    const int s0 = first + 4 * piece;
+                                    const uint32_t e0 = (uint32_t)grow * (uint32_t)groups + (uint32_t)s0; // element of the row's array
+                                    auto fetch = [&](const unsigned int *array) {
+                                        if (s0 + 4 <= groups) {
+                                            v[b] = *reinterpret_cast<const quad_u4 *>(array + e0);
+                                        } else {
+#pragma unroll
+                                            for (int d = 0; d < 4; ++d)
+                                                v[b][d] = array[e0 + (uint32_t)(min(s0 + d, groups - 1) - s0)];
+                                        }
+                                    };
+                                    if (8 * u < RA) // (a unit lies in one of the three arrays; wave-uniform)
+                                        fetch(reinterpret_cast<const unsigned int *>(a.x_group_sums));
+                                    else if (8 * u < RA + RB)
+                                        fetch(reinterpret_cast<const unsigned int *>(a.w_scale));
+                                    else
+                                        fetch(reinterpret_cast<const unsigned int *>(a.w_zero));
+                                }
+                            }
+#pragma unroll
+                            for (int b = 0; b < 3; ++b) {
+                                const int u = u0 + b * WM * WN;
+                                if (u < UNITS)
+                                    *reinterpret_cast<quad_u *>(smem + u * 1024 + lane * 16) = v[b];
+                            }
+                        }
+                    }
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __syncthreads();
+                    auto row_at = [&](int row) { return smem + row * 128; };
+                    zero_point_reads_half<TM, TN>(row_at, ra, rs, rs + RB, g, 0, c0);
+                    zero_point_reads_half<TM, TN>(row_at, ra, rs, rs + RB, g, 1, c0);
+                    if (first + 32 > groups) { // a partial chunk: groups past the end count nothing (their scales are some group's: finite)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h)
+#pragma unroll
+                            for (int t = 0; t < 8; ++t)
+                                if (first + 16 * g + 8 * h + t >= groups) {
+#pragma unroll
+                                    for (int i = 0; i < TM; ++i)
+                                        c0.sx[h][i][t] = 0;
+                                }
+                    }
+                    multiply(c0);
+                }
+            }
+        }
         // (a lane's sixteen groups of chunk g0: from g0 + 16 g on)
         if constexpr (AHEAD == 2) {
-            zero_point_loads<TM, TN>(a, arow, brow, 16 * g, groups, c0);
-            for (int g0 = 0; g0 < groups; g0 += 64) {
+            if (first < groups)
+                zero_point_loads<TM, TN>(a, arow, brow, first + 16 * g, groups, c0);
+            for (int g0 = first; g0 < groups; g0 += 64) {
                 const bool second = g0 + 32 < groups; // wave-uniform
                 if (second)
                     zero_point_loads<TM, TN>(a, arow, brow, g0 + 32 + 16 * g, groups, c1);
@@ -233,12 +383,12 @@ __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&f
                 }
             }
         } else if constexpr (AHEAD == 1) {
-            for (int g0 = 0; g0 < groups; g0 += 32) {
+            for (int g0 = first; g0 < groups; g0 += 32) {
                 zero_point_loads<TM, TN>(a, arow, brow, g0 + 16 * g, groups, c0);
                 multiply(c0);
             }
         } else {
-            for (int g0 = 0; g0 < groups; g0 += 32) {
+            for (int g0 = first; g0 < groups; g0 += 32) {
                 zero_point_loads_half<TM, TN>(a, arow, brow, g0 + 16 * g, groups, c0, 0);
                 zero_point_product<TM, TN>(c0.sx[0], c0.ws[0], c0.wz[0], facc);
                 zero_point_loads_half<TM, TN>(a, arow, brow, g0 + 16 * g, groups, c0, 1);
