@@ -21,6 +21,7 @@ hipError_t launch_pack_f16_fp6(const void *, const float *, uint32_t *, int, int
 hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes_padded(const uint32_t *, uint32_t *, int, int, int, int, int, hipStream_t);
+hipError_t launch_relayout_planes_folded(const uint32_t *, const float *, int, uint32_t *, int, int, int, int, int, int *, hipStream_t);
 hipError_t launch_relayout_planes_fp6(const uint32_t *, uint32_t *, int, int, int, int, hipStream_t);
 hipError_t launch_row_sums(const uint32_t *, int *, int, int, int, hipStream_t);
 const KernelEntry *fp6_entries(int *count);
@@ -1621,6 +1622,21 @@ abq_status abq_relayout_planes_padded(const uint32_t *planes, uint32_t *tiled, i
         return ABQ_ERR_BAD_K;
     return hip_status(launch_relayout_planes_padded(planes, tiled, rows, k, abq_padded_bits(bits), bits, is_signed ? 1 : 0,
                                                     (hipStream_t)stream));
+}
+
+int abq_folded_bits(int bits) { return bits < 1 || bits > 7 ? 0 : abq_padded_bits(bits + 1); }
+
+abq_status abq_relayout_planes_folded(const uint32_t *planes, const float *w_zero, int group_size, uint32_t *tiled, int rows, int k,
+                                      int bits, int is_signed, int *misfit_dev, void *stream)
+{
+    if (!planes || !w_zero || !tiled || rows <= 0 || bits < 1 || bits > 8 || group_size < 32 || group_size % 32 != 0)
+        return ABQ_ERR_INVALID_ARG;
+    if (k < 128 || k % 128 != 0 || k % group_size != 0 || (group_size > 128 && group_size % 128 != 0))
+        return ABQ_ERR_BAD_K;
+    if (!abq_folded_bits(bits))
+        return ABQ_ERR_UNSUPPORTED; // 8-bit codes less their zero points need nine bits
+    return hip_status(launch_relayout_planes_folded(planes, w_zero, group_size, tiled, rows, k, abq_folded_bits(bits), bits,
+                                                    is_signed ? 1 : 0, misfit_dev, (hipStream_t)stream));
 }
 
 abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)

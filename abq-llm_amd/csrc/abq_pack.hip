@@ -127,6 +127,30 @@ __device__ __forceinline__ void store_fields(uint32_t *rec, int ws, const uint32
         rec[field_word_offset(BITS, 1) + ws] = f[field_list_index(BITS, 1)];
 }
 
+// Folds a weight zero point into the codes of one word-set: e holds 32 codes, one per byte, as the low `in_bits` bits
+// (two's complement when `is_signed`); every code becomes code - z in the low BITS bits.  Returns false where a
+// result does not fit BITS bits as a signed number.
+template <int BITS> __device__ __forceinline__ bool fold_zero_point(uint32_t (&e)[8], int z, int in_bits, bool is_signed)
+{
+    bool fits = true;
+    const int lo = -(1 << (BITS - 1)), hi = (1 << (BITS - 1)) - 1;
+#pragma unroll
+    for (int d = 0; d < 8; ++d) {
+        uint32_t out = 0;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            int code = (int)((e[d] >> (8 * c)) & ((1u << in_bits) - 1u));
+            if (is_signed && (code >> (in_bits - 1)))
+                code -= 1 << in_bits;
+            const int v = code - z;
+            fits = fits && v >= lo && v <= hi;
+            out |= ((uint32_t)v & ((1u << BITS) - 1u)) << (8 * c);
+        }
+        e[d] = out;
+    }
+    return fits;
+}
+
 // One workgroup converts 32 rows x 8 K tiles.  A thread owns one record (one row, one K tile): it
 // reads 16 bytes per plane (eight threads cover 128 contiguous bytes of a plane row), converts its
 // four word-sets in registers, and parks the record in LDS; the records of one K tile are then
@@ -135,10 +159,14 @@ __device__ __forceinline__ void store_fields(uint32_t *rec, int ws, const uint32
 // the widths made of several fields): the planes above it repeat its top plane (sign_extend & 1: signed codes) or
 // are zero.  sign_extend & 2 (8-bit records): bit 7 of every code is flipped, i.e. the record holds code - 128
 // (biased records of unsigned 8-bit operands, which the signed matrix cores take as they are).
+// zero != nullptr (weights with group-wise zero points, group_size a multiple of 32): every code has its group's zero
+// point, zero[row][k / group_size], taken off, and the records hold the signed differences; *flag is set where a
+// zero point is no whole number or a difference does not fit the records.
 template <int BITS>
 __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__restrict__ planes,
                                                               uint32_t *__restrict__ tiled, int rows, int KW, int in_bits,
-                                                              int sign_extend)
+                                                              int sign_extend, const float *__restrict__ zero = nullptr,
+                                                              int group_size = 0, int *flag = nullptr)
 {
     constexpr int REC = BITS * 4;          // words per record
     constexpr int SLAB = 32 * REC + 4;     // words per K tile in LDS (+16 bytes against bank conflicts)
@@ -169,6 +197,13 @@ __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__
 #pragma unroll
                     for (int d = 0; d < 8; ++d)
                         e[d] ^= 0x80808080u;
+                }
+                if (zero) {
+                    const float zf = zero[(size_t)row * (KW * 32 / group_size) + (kt * 128 + ws * 32) / group_size];
+                    const float zr = rintf(zf);
+                    const bool ok = zr == zf && fabsf(zr) <= 256.f && fold_zero_point<BITS>(e, (int)zr, in_bits, (sign_extend & 1) != 0);
+                    if (!ok && flag)
+                        *flag = 1;
                 }
                 compress_fields<BITS>(e, f);
                 store_fields<BITS>(rec, ws, f);
@@ -262,6 +297,26 @@ hipError_t launch_relayout_planes_padded(const uint32_t *planes, uint32_t *tiled
         break;
         ABQ_RELAYOUT_CASE(1) ABQ_RELAYOUT_CASE(2) ABQ_RELAYOUT_CASE(3) ABQ_RELAYOUT_CASE(4)
         ABQ_RELAYOUT_CASE(5) ABQ_RELAYOUT_CASE(6) ABQ_RELAYOUT_CASE(7) ABQ_RELAYOUT_CASE(8)
+#undef ABQ_RELAYOUT_CASE
+    default:
+        return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// Records of `bits` bits holding code - zero point (see relayout_planes_kernel).
+hipError_t launch_relayout_planes_folded(const uint32_t *planes, const float *zero, int group_size, uint32_t *tiled, int rows, int k,
+                                         int bits, int in_bits, int is_signed, int *flag, hipStream_t stream)
+{
+    const int KW = k / 32;
+    const dim3 grid((rows + 31) / 32, (KW / 4 + 7) / 8);
+    switch (bits) {
+#define ABQ_RELAYOUT_CASE(B)                                                                                     \
+    case B:                                                                                                      \
+        hipLaunchKernelGGL(relayout_planes_kernel<B>, grid, dim3(256), 0, stream, planes, tiled, rows, KW, in_bits, is_signed ? 1 : 0, \
+                           zero, group_size, flag);                                                              \
+        break;
+        ABQ_RELAYOUT_CASE(2) ABQ_RELAYOUT_CASE(4) ABQ_RELAYOUT_CASE(8)
 #undef ABQ_RELAYOUT_CASE
     default:
         return hipErrorInvalidValue;

@@ -392,22 +392,30 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     // (padded records serve every M: above the decode sizes the padded pair's LDS-staged prefill kernel reads them,
     // which the widths of several fields do not have: W3A8 with groups of 128 at 1024 tokens 1.3-1.7 times faster)
     const bool on_padded = w_padded && W.records_padded != nullptr && !decode && !fp6;
-    if (!decode && !fp6 && !on_padded && !W.planes_tiled) {
+    // (prefill-sized calls on weights whose zero points were folded into the records: no zero-point term)
+    const bool on_folded = W.records_folded != nullptr && W.zero != nullptr && !decode && !decode_prepared && !fp6 && M > 16 &&
+                           abq_folded_bits(w_bits_) != 0;
+    if (!decode && !fp6 && !on_padded && !on_folded && !W.planes_tiled) {
         printf("[ABQ][Error] ABQGroupedWeight::planes_tiled is needed for M,N,K = %d,%d,%d\n", M, N, K);
         return;
     }
-    rc = abq_gemm_init(nullptr, x_bits_, on_padded ? w_rec_bits : w_bits_, 1, planes,
+    rc = abq_gemm_init(nullptr, x_bits_, on_folded ? abq_folded_bits(w_bits_) : on_padded ? w_rec_bits : w_bits_, 1, planes,
                        decode ? reinterpret_cast<const uint32_t *>(W.planes) : fp6 ? reinterpret_cast<const uint32_t *>(W.records_fp6)
+                       : on_folded ? reinterpret_cast<const uint32_t *>(W.records_folded)
                        : on_padded ? w_records : reinterpret_cast<const uint32_t *>(W.planes_tiled), M, N, K,
                        D, nullptr, 0, ABQ_OUT_F16_SCALED, &state);
-    if (rc == ABQ_OK && on_padded)
+    if (rc == ABQ_OK && on_padded && !on_folded)
         rc = abq_gemm_set_value_bits(&state, x_bits_, w_bits_);
     if (rc == ABQ_OK && !decode)
         rc = abq_gemm_set_operand_layout(&state, layout, layout);
     if (rc == ABQ_OK)
         rc = abq_gemm_set_scales(&state, x_scale, W.scale, W.group_size);
-    if (rc == ABQ_OK && (W.zero || !x_symmetric))
+    if (rc == ABQ_OK && on_folded) {
+        if (!x_symmetric)
+            rc = abq_gemm_set_zero_points(&state, x_zero, nullptr, nullptr, W.zero_term);
+    } else if (rc == ABQ_OK && (W.zero || !x_symmetric)) {
         rc = abq_gemm_set_zero_points(&state, x_symmetric ? nullptr : x_zero, W.zero, sums, W.zero_term);
+    }
     if (rc == ABQ_OK && silu_gate)
         rc = abq_gemm_set_activation(&state, ABQ_ACT_SILU_GATE);
     if (rc == ABQ_ERR_UNSUPPORTED) {

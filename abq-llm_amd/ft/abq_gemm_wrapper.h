@@ -41,6 +41,10 @@ struct ABQGroupedWeight {
                               // pair's kernels on them: the prepared-operand decode kernel instead of the one on plane
                               // operands, the LDS-staged prefill kernel instead of the register-staged one of the
                               // odd widths; planes_tiled may then be nullptr
+    const int *records_folded; // weights with whole-number zero points, at most 7 bits: the same weights as records of
+                              // code - zero point (abq_relayout_planes_folded; twice the bytes of 2-bit weights), or
+                              // nullptr; with it, prefill-sized calls (those that leave the decode kernels) run on
+                              // them without the zero-point term, 3-19 % faster (most at K = 11008)
 };
 
 class ABQGEMMWrapper {

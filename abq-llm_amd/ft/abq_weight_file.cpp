@@ -186,10 +186,11 @@ ABQDeviceWeight::~ABQDeviceWeight() { release(); }
 
 void ABQDeviceWeight::release()
 {
-    for (void *p : { (void *)planes_, (void *)tiled_, (void *)fp6_, (void *)padded_, (void *)scale_, (void *)zero_, (void *)zero_term_ })
+    for (void *p : { (void *)planes_, (void *)tiled_, (void *)fp6_, (void *)padded_, (void *)folded_, (void *)scale_, (void *)zero_,
+                     (void *)zero_term_ })
         if (p)
             (void)hipFree(p);
-    planes_ = tiled_ = fp6_ = padded_ = nullptr;
+    planes_ = tiled_ = fp6_ = padded_ = folded_ = nullptr;
     scale_ = zero_ = zero_term_ = nullptr;
 }
 
@@ -232,6 +233,26 @@ bool ABQDeviceWeight::load(const ABQWeightBlob &blob, hipStream_t stream, std::s
             return false;
         rc = abq_relayout_planes_padded(planes_, padded_, (int)info_.n, (int)info_.k, (int)info_.bits, (int)info_.is_signed, stream);
     }
+    // zero points folded into the records, for prefill-sized calls: kept only if every zero point is a whole number
+    // and the differences fit (the quantiser's rounded zero points do)
+    if (rc == ABQ_OK && info_.has_zero && (info_.group_size == 64 || info_.group_size == 128) && abq_folded_bits((int)info_.bits) != 0) {
+        int *misfit = nullptr, host_misfit = 1;
+        if (!hip_ok(hipMalloc(&folded_, abq_planes_bytes((int)info_.n, (int)info_.k, abq_folded_bits((int)info_.bits))), "hipMalloc folded") ||
+            !hip_ok(hipMalloc(&misfit, sizeof(int)), "hipMalloc flag") || !hip_ok(hipMemsetAsync(misfit, 0, sizeof(int), stream), "clear flag"))
+            return false;
+        rc = abq_relayout_planes_folded(planes_, zero_, (int)info_.group_size, folded_, (int)info_.n, (int)info_.k, (int)info_.bits,
+                                        (int)info_.is_signed, misfit, stream);
+        const bool copied = hip_ok(hipMemcpyAsync(&host_misfit, misfit, sizeof(int), hipMemcpyDeviceToHost, stream), "read flag") &&
+                            hip_ok(hipStreamSynchronize(stream), "synchronise");
+        (void)hipFree(misfit);
+        if (!copied)
+            return false;
+        if (rc != ABQ_OK || host_misfit) { // such weights keep the zero-point term
+            (void)hipFree(folded_);
+            folded_ = nullptr;
+            rc = rc == ABQ_ERR_UNSUPPORTED ? ABQ_OK : rc;
+        }
+    }
     if (rc != ABQ_OK)
         return fail(error, std::string("weight preparation failed: ") + abq_status_string(rc));
     return hip_ok(hipStreamSynchronize(stream), "synchronise");
@@ -241,5 +262,5 @@ ABQGroupedWeight ABQDeviceWeight::grouped() const
 {
     return ABQGroupedWeight{ reinterpret_cast<const int *>(tiled_), scale_, zero_, zero_term_, (int)info_.group_size,
                              reinterpret_cast<const int *>(planes_), reinterpret_cast<const int *>(fp6_),
-                             reinterpret_cast<const int *>(padded_) };
+                             reinterpret_cast<const int *>(padded_), reinterpret_cast<const int *>(folded_) };
 }

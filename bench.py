@@ -725,7 +725,8 @@ def main():
             for name, N, K, act in (("qkv", 12288, 4096, 0), ("o", 4096, 4096, 0), ("gate_up_silu", 22016, 4096, 1),
                                     ("down", 4096, 11008, 0)):
                 G = K // 128
-                wt = abq.relayout_planes(random_planes(torch, (P_BITS, N, K // 32)))
+                wpl = random_planes(torch, (P_BITS, N, K // 32))
+                wt = abq.relayout_planes(wpl)
                 wsc = torch.rand((N, G), device="cuda") * 0.01 + 0.001
                 wz = torch.randint(-2, 2, (N, G), device="cuda").float()
                 x = torch.randn((tokens, K), device="cuda", dtype=torch.float16)
@@ -742,28 +743,34 @@ def main():
                     wrot = wt.unsqueeze(0).repeat(max(2, math.ceil(ROTATE_BYTES / wbytes)), 1, 1, 1, 1)
                     copies = [wrot[r] for r in range(wrot.shape[0])]
                 gms = [gm] if len(copies) == 1 else [abq.Gemm(xt, c, SIGNED, **kwl) for c in copies]
-                calls = [0]
 
-                def step():
-                    abq._check(abq.lib().abq_quant_pack_f16(x.data_ptr(), tokens, K, Q_BITS, 1, 1, xt.data_ptr(), xsc.data_ptr(),
-                                                            None, sums.data_ptr(), 128, abq._stream_ptr(None)), "quant_pack")
-                    gms[calls[0] % len(gms)].run()
-                    calls[0] += 1
-                step()
-                torch.cuda.synchronize()
-                # (a replay's own launch cost is spread over its steps; a decode graph walks through all weight copies)
-                reps = max(20, len(gms)) if tokens < 1024 else 10 if tokens < 8192 else 3
-                gr = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(gr):
-                    for _ in range(reps):
-                        step()
-                settle(gr.replay)
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                gr.replay()
-                e1.record()
-                torch.cuda.synchronize()
-                us = e0.elapsed_time(e1) * 1e3 / reps
+                def quantise_and_run(gemms):
+                    """us per step of: quantise + pack the fp16 rows, then the GEMM (the next of `gemms`), graph replay"""
+                    calls = [0]
+
+                    def step():
+                        abq._check(abq.lib().abq_quant_pack_f16(x.data_ptr(), tokens, K, Q_BITS, 1, 1, xt.data_ptr(), xsc.data_ptr(),
+                                                                None, sums.data_ptr(), 128, abq._stream_ptr(None)), "quant_pack")
+                        gemms[calls[0] % len(gemms)].run()
+                        calls[0] += 1
+                    step()
+                    torch.cuda.synchronize()
+                    # (a replay's own launch cost is spread over its steps; a decode graph walks through all weight copies)
+                    reps = max(20, len(gemms)) if tokens < 1024 else 10 if tokens < 8192 else 3
+                    gr = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(gr):
+                        for _ in range(reps):
+                            step()
+                    settle(gr.replay)
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    gr.replay()
+                    e1.record()
+                    torch.cuda.synchronize()
+                    del gr
+                    return e0.elapsed_time(e1) * 1e3 / reps
+
+                us = quantise_and_run(gms)
                 tops = 2.0 * tokens * N * K / (us * 1e-6) / 1e12
                 entry = dict(linear=name, tokens=tokens, N=N, K=K, us=round(us, 1), tops=round(tops, 1),
                              mfma_frac=round(tops / INT8_MFMA_PEAK_TOPS, 4), kernel="%s:%s" % (gm.strategy, gm.config_name))
@@ -786,8 +793,24 @@ def main():
                     entry["one_launch_us"] = round(us1, 1)
                     log("layer %s tokens=%d: one launch (kernel quantises the rows) %.1f us" % (name, tokens, us1))
                     del g1, g1s, out1
+                if tokens >= 1024:
+                    # the same prefill on a second copy of the weights with the zero points folded into 4-bit records
+                    # (abq_relayout_planes_folded): no zero-point term in the epilogue
+                    wf = abq.relayout_planes_folded(wpl, wz, 128, SIGNED)
+                    outf = torch.empty_like(out)
+                    gf = abq.Gemm(xt, wf, SIGNED, out=outf, out_kind=abq.OUT_F16_SCALED, x_scale=xsc, w_scale=wsc, group_size=128,
+                                  x_tiled=True, w_tiled=True, act=act)
+                    usf = quantise_and_run([gf])
+                    torch.cuda.synchronize()
+                    worst = float((outf.float() - out.float()).abs().max() / out.float().abs().max().clamp_min(1e-6))
+                    if worst > 5e-3:
+                        raise RuntimeError("GEMM on folded zero points differs from the zero-point term (%s, tokens=%d): %g" % (name, tokens, worst))
+                    entry["folded_zero_points"] = dict(us=round(usf, 1), tops=round(2.0 * tokens * N * K / (usf * 1e-6) / 1e12, 1),
+                                                       kernel="%s:%s" % (gf.strategy, gf.config_name))
+                    log("layer %s tokens=%d: zero points folded into 4-bit records %.1f us  %.0f TOPS" % (name, tokens, usf, entry["folded_zero_points"]["tops"]))
+                    del gf, wf, outf
                 layer.append(entry)
-                del gr, gm, gms, copies, out, x, xt, wt
+                del gm, gms, copies, out, x, xt, wt, wpl
         extra["decoder_layer_w2a8_group128"] = layer
 
 

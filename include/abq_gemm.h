@@ -451,6 +451,21 @@ abq_status abq_gemm_set_biased_records(abq_gemm_state *state, int x_biased, int 
 int abq_padded_bits(int bits);
 abq_status abq_relayout_planes_padded(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits, int is_signed,
                                       void *stream);
+/* Weights with group-wise zero points as records that need no zero-point term: every code has its group's zero point
+ * taken off, w_zero[row][k / group_size] (a whole number, as the quantiser's rounding leaves it), and the signed
+ * differences, one bit wider than the codes, are written as K-tiled records of abq_folded_bits(bits) bits (2 -> 4,
+ * 3 -> 4, 4 ... 7 -> 8; 0 for 8: not supported).  A GEMM on them is initialised as the signed pair (x_bits,
+ * abq_folded_bits(bits)) with the group scales and WITHOUT weight zero points (abq_gemm_set_zero_points: w_zero and
+ * x_group_sums NULL; the activation zero points' w_zero_term stays what abq_weight_zero_term made of the original
+ * weights): out = sum_g sx sw[n,g] sum_k x (w - z) is the same number, and the epilogue's zero-point term, 10-20 %
+ * of a prefill GEMM with group scales, is gone, for records twice the size of 2-bit weights: a copy for prefill-sized
+ * calls where the memory is there.  group_size: a multiple of 32 that divides k (and of 128, or a divisor of it).
+ * misfit_dev (may be NULL): a device int the caller has zeroed, set to 1 if a zero point is no whole number or a
+ * difference does not fit the records.  No counterpart in the reference (its zero points: quantizer.py:111-132). */
+int abq_folded_bits(int bits);
+abq_status abq_relayout_planes_folded(const uint32_t *planes, const float *w_zero, int group_size, uint32_t *tiled, int rows, int k,
+                                      int bits, int is_signed, int *misfit_dev, void *stream);
+
 /* Declares that the codes of X (W) use only the low x_value_bits (w_value_bits) of their fields (1 .. the state's
  * widths): see above.  An operand of such a state that is still in the reference plane layout has that many planes,
  * and abq_gemm_exec extends its codes to the records' width while it converts them into the workspace.  This makes

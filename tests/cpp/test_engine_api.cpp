@@ -376,7 +376,7 @@ static void gpu_paths()
     // padded records on the prepared-operand decode kernel of the 4-bit width, as planes on the plane-operand one,
     // above that on the prefill kernel of the padded pair (padded records, which then are the only copy handed over)
     // or of the 3-bit records.
-    auto dynamic_case = [&](const int WB, const int M, const bool padded_records, const bool keep_planes) {
+    auto dynamic_case = [&](const int WB, const int M, const bool padded_records, const bool keep_planes, const bool folded_records = false) {
         const int N = 192, K = 512, G = 128, groups = K / G;
         std::mt19937 r32(5 + WB + M);
         std::normal_distribution<float> nd(0.f, 1.5f);
@@ -395,7 +395,8 @@ static void gpu_paths()
         std::vector<uint32_t> wpl((size_t)WB * N * K / 32);
         abq_oracle_pack_i32(wq.data(), wpl.data(), N, K, WB);
         _Float16 *d_a, *d_d;
-        uint32_t *d_wpl, *d_wt, *d_wpad;
+        uint32_t *d_wpl, *d_wt, *d_wpad, *d_wfold;
+        int *d_misfit;
         float *d_wscale, *d_wzero, *d_term;
         char *d_ws;
         ABQGEMMWrapper wrap(8, WB, true);
@@ -405,6 +406,9 @@ static void gpu_paths()
         HIP_OK(hipMalloc(&d_wpl, wpl.size() * 4));
         HIP_OK(hipMalloc(&d_wt, wpl.size() * 4));
         HIP_OK(hipMalloc(&d_wpad, abq_planes_bytes(N, K, abq_padded_bits(WB))));
+        HIP_OK(hipMalloc(&d_wfold, abq_planes_bytes(N, K, abq_folded_bits(WB))));
+        HIP_OK(hipMalloc(&d_misfit, sizeof(int)));
+        HIP_OK(hipMemset(d_misfit, 0, sizeof(int)));
         HIP_OK(hipMalloc(&d_wscale, wscale.size() * 4));
         HIP_OK(hipMalloc(&d_wzero, wzero.size() * 4));
         HIP_OK(hipMalloc(&d_term, N * 4));
@@ -416,9 +420,14 @@ static void gpu_paths()
         CHECK(abq_relayout_planes(d_wpl, d_wt, N, K, WB, stream) == ABQ_OK);
         CHECK(abq_relayout_planes_padded(d_wpl, d_wpad, N, K, WB, 1, stream) == ABQ_OK);
         CHECK(abq_weight_zero_term(d_wpl, N, K, WB, 1, d_wscale, d_wzero, G, d_term, stream) == ABQ_OK);
+        CHECK(abq_relayout_planes_folded(d_wpl, d_wzero, G, d_wfold, N, K, WB, 1, d_misfit, stream) == ABQ_OK);
+        int misfit = 1;
+        HIP_OK(hipMemcpy(&misfit, d_misfit, sizeof(int), hipMemcpyDeviceToHost));
+        CHECK(misfit == 0);
         const ABQGroupedWeight weight = { padded_records ? nullptr : reinterpret_cast<const int *>(d_wt), d_wscale, d_wzero, d_term, G,
                                           keep_planes ? reinterpret_cast<const int *>(d_wpl) : nullptr, nullptr,
-                                          padded_records ? reinterpret_cast<const int *>(d_wpad) : nullptr };
+                                          padded_records ? reinterpret_cast<const int *>(d_wpad) : nullptr,
+                                          folded_records ? reinterpret_cast<const int *>(d_wfold) : nullptr };
         for (int symmetric = 1; symmetric >= 0; --symmetric) {
             wrap.gemm_dynamic(M, N, K, d_a, weight, d_d, symmetric != 0, d_ws, ws_bytes, stream);
             HIP_OK(hipStreamSynchronize(stream));
@@ -469,6 +478,8 @@ static void gpu_paths()
         HIP_OK(hipFree(d_wpl));
         HIP_OK(hipFree(d_wt));
         HIP_OK(hipFree(d_wpad));
+        HIP_OK(hipFree(d_wfold));
+        HIP_OK(hipFree(d_misfit));
         HIP_OK(hipFree(d_wscale));
         HIP_OK(hipFree(d_wzero));
         HIP_OK(hipFree(d_term));
@@ -484,6 +495,9 @@ static void gpu_paths()
     dynamic_case(3, 300, true, false); // prefill on the padded records: the 4-bit pair's LDS-staged kernel
     dynamic_case(3, 300, false, false); // ... and on the 3-bit records
     dynamic_case(6, 130, true, false); // 6-bit weights as 8-bit records, prefill
+    dynamic_case(2, 300, false, false, true); // prefill on records with the zero points folded in (4-bit records of 2-bit weights)
+    dynamic_case(3, 300, true, false, true);  // ... of 3-bit weights
+    dynamic_case(2, 8, false, false, true);   // decode-sized: the weights' own records
 
     for (const int WB : { 4, 3 })
     for (const int M : { 24, 3 }) {

@@ -574,6 +574,54 @@ def test_group_scale_tiles_whose_waves_split_k_are_the_default_on_grids_of_one_r
         assert_close_rel(got.float().cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("p,signed_codes", [(2, True), (3, True), (4, True), (2, False), (3, False), (6, True)])
+@pytest.mark.parametrize("group_size", [128, 64])
+def test_zero_points_folded_into_the_weight_records(abq, oracle, p, signed_codes, group_size):
+    """Weights with whole-number zero points as records of code - zero point, one field wider: the GEMM runs the signed
+    pair of that width with group scales and no weight zero points, and gives what the zero-point term gives: against
+    the dequantised reference, and against the same GEMM on the plain records with the zero points handed in.
+    Decode- and prefill-sized calls, activation zero points (whose weight-side term comes from the original weights),
+    ragged shapes; zero points that are no whole numbers or push a difference out of the records are reported."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(4000 + 10 * p + signed_codes + group_size)
+    q, rb = 8, abq.lib().abq_folded_bits(p)
+    assert rb == (4 if p <= 3 else 8)
+    lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed_codes else (0, 1 << p)
+    for (M, N, K) in [(4, 96, 512), (40, 200, 640), (300, 130, 1152), (130, 264, 4096)]:
+        G = K // group_size
+        x = rng.integers(-128, 128, (M, K)).astype(np.int32)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        xs = rng.uniform(0.01, 0.05, M)
+        xz = rng.integers(-64, 65, M).astype(np.float64)
+        wsc = rng.uniform(0.001, 0.02, (N, G))
+        wz = rng.integers(lo_w, hi_w + (0 if signed_codes else 1), (N, G)).astype(np.float64)
+        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, group_size)
+        wp = planes_dev(oracle.pack_i32(w, p))
+        folded = abq.relayout_planes_folded(wp, fdev(wz), group_size, signed_codes)
+        assert folded.shape == (K // 128, N, rb, 4)
+        xsum = torch.from_numpy(x.reshape(M, G, group_size).sum(axis=2).astype(np.int32)).cuda()
+        term = abq.weight_zero_term(wp, signed_codes, fdev(wsc), fdev(wz), group_size)
+        xt = abq.relayout_planes(planes_dev(oracle.pack_i32(x, q)))
+        g = abq.Gemm(xt, folded, True, out_kind=abq.OUT_F16_SCALED, x_tiled=True, w_tiled=True, x_scale=fdev(xs), w_scale=fdev(wsc),
+                     group_size=group_size, x_zero=fdev(xz), w_zero_term=term)
+        assert (g.state.cfg.x_bits, g.state.cfg.w_bits) == (8, rb)
+        got = g.run().float().cpu().numpy()
+        assert_close_rel(got, want)
+        if signed_codes and p in (2, 4):  # the same through the zero-point term, on the weights' own records
+            ref = abq.Gemm(xt, abq.relayout_planes(wp), True, out_kind=abq.OUT_F16_SCALED, x_tiled=True, w_tiled=True, x_scale=fdev(xs),
+                           w_scale=fdev(wsc), group_size=group_size, x_zero=fdev(xz), w_zero=fdev(wz), x_group_sums=xsum,
+                           w_zero_term=term).run().float().cpu().numpy()
+            assert_close_rel(got, ref)
+    wz_bad = wz.copy()
+    wz_bad[3, 1] += 0.25
+    with pytest.raises(ValueError):
+        abq.relayout_planes_folded(wp, fdev(wz_bad), group_size, signed_codes)
+    wz_bad = wz.copy()
+    wz_bad[5, 0] = -(1 << rb)
+    with pytest.raises(ValueError):
+        abq.relayout_planes_folded(wp, fdev(wz_bad), group_size, signed_codes)
+
+
 @pytest.mark.parametrize("M,K", [(200, 4096), (130, 4608), (136, 8192)])
 @pytest.mark.parametrize("q,p,fp6", [(8, 2, False), (4, 4, False), (4, 4, True)])
 def test_zero_points_over_whole_chunks_of_groups(abq, oracle, M, K, q, p, fp6):
