@@ -512,8 +512,9 @@ void gemm_mfma_staged(const GemmArgs a, const v4u *xt, const v4u *wt, int m_bloc
             return;
     }
     if constexpr (GROUPED) {
-        // (the integer tiles have the registers to run the zero-point loads ahead of their use, and stage them through LDS)
-        group_scale_epilogue<TM, TN, WM, WN, LDS_BYTES, FP6 ? 0 : TM * TN == 1 ? 2 : TM * TN == 2 ? 1 : 0, !FP6>(a, facc, smem, M, N, m0, n0, wm,
+        // (the integer tiles have the registers to run the zero-point loads ahead of their use; the term's operands come
+        // through LDS except on the 128 x 128 tile whose waves split K, which has no registers left for that either)
+        group_scale_epilogue<TM, TN, WM, WN, LDS_BYTES, FP6 ? 0 : TM * TN == 1 ? 2 : TM * TN == 2 ? 1 : 0, WK == 1 || TM * TN < 4>(a, facc, smem, M, N, m0, n0, wm,
                                                                                                                wn, r, g, tid);
         return;
     }

@@ -290,8 +290,9 @@ __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&f
         constexpr int RA = 32 * TM * WM, RB = 32 * TN * WN; // rows of the workgroup's tile
         if constexpr (VIA_LDS && (RA + 2 * RB) * 128 <= LDS_BYTES) {
             const int ra = wm * 32 * TM + r, rs = RA + wn * 32 * TN + r; // the lane's rows among the staged ones
-            {
-                const bool rows16 = zero_point_rows_aligned(a, groups);
+            // (rows that start off 16-byte boundaries, K = 11008 with its 86 groups, keep the loads below: bringing them
+            // through registers or four bytes a lane into the same LDS layout was no faster, and slower on the FP6 tiles)
+            if (zero_point_rows_aligned(a, groups)) {
                 const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
                 const unsigned lds0 = (unsigned)(size_t)smem;
                 // LDS: the tile's RA rows of group sums, its RB rows of scales, its RB rows of zero points, 128 bytes
@@ -299,53 +300,10 @@ __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&f
                 constexpr int UNITS = (RA + 2 * RB) / 8;
                 for (; first < groups; first += 32) {
                     __syncthreads(); // every wave is through with what the LDS held (the stages; the chunk before)
-                    if (rows16) {
-                        for (int u = wave; u < UNITS; u += WM * WN) { // wave-uniform
-                            const void *base;
-                            const uint32_t off = zero_point_unit_offset<RA, RB>(a, u, lane, m0, n0, M, N, groups, first, &base);
-                            epilogue_load_to_lds(base, off, lds0 + u * 1024);
-                        }
-                    } else {
-                        // rows that start off 16-byte boundaries (K = 11008: 86 groups): the same units through registers,
-                        // three loads of a wave in flight at a time (a 16-byte load into registers asks for 4-byte alignment
-                        // only); the piece that straddles the end of a row comes word by word
-                        typedef unsigned int quad_u __attribute__((ext_vector_type(4)));
-                        typedef unsigned int quad_u4 __attribute__((ext_vector_type(4), aligned(4)));
-                        for (int u0 = wave; u0 < UNITS; u0 += 3 * WM * WN) {
-                            quad_u v[3];
-#pragma unroll
-                            for (int b = 0; b < 3; ++b) {
-                                const int u = u0 + b * WM * WN;
-                                if (u < UNITS) { // wave-uniform
-                                    const int row = 8 * u + (lane >> 3);
-                                    const int piece = (lane & 7) ^ ((row >> 1) & 7);
-                                    const int grow = row < RA ? min(m0 + row, M - 1) : min(n0 + (row < RA + RB ? row - RA : row - RA - RB), N - 1);
-                                    const int s0 = first + 4 * piece;
-                                    const uint32_t e0 = (uint32_t)grow * (uint32_t)groups + (uint32_t)s0; // element of the row's array
-                                    auto fetch = [&](const unsigned int *array) {
-                                        if (s0 + 4 <= groups) {
-                                            v[b] = *reinterpret_cast<const quad_u4 *>(array + e0);
-                                        } else {
-#pragma unroll
-                                            for (int d = 0; d < 4; ++d)
-                                                v[b][d] = array[e0 + (uint32_t)(min(s0 + d, groups - 1) - s0)];
-                                        }
-                                    };
-                                    if (8 * u < RA) // (a unit lies in one of the three arrays; wave-uniform)
-                                        fetch(reinterpret_cast<const unsigned int *>(a.x_group_sums));
-                                    else if (8 * u < RA + RB)
-                                        fetch(reinterpret_cast<const unsigned int *>(a.w_scale));
-                                    else
-                                        fetch(reinterpret_cast<const unsigned int *>(a.w_zero));
-                                }
-                            }
-#pragma unroll
-                            for (int b = 0; b < 3; ++b) {
-                                const int u = u0 + b * WM * WN;
-                                if (u < UNITS)
-                                    *reinterpret_cast<quad_u *>(smem + u * 1024 + lane * 16) = v[b];
-                            }
-                        }
+                    for (int u = wave; u < UNITS; u += WM * WN) { // wave-uniform
+                        const void *base;
+                        const uint32_t off = zero_point_unit_offset<RA, RB>(a, u, lane, m0, n0, M, N, groups, first, &base);
+                        epilogue_load_to_lds(base, off, lds0 + u * 1024);
                     }
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     __syncthreads();
