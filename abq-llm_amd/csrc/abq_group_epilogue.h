@@ -162,7 +162,7 @@ __device__ __forceinline__ void zero_point_product(const int (&sx)[TM][8], const
 }
 
 // A wave's 64 x 16 bytes from global memory straight into LDS at lds_addr + 16 * lane (`base` the same in every lane,
-// `offset` the lane's byte offset from it), and the wait for every such load of the wave.
+// `offset` the lane's byte offset from it).
 __device__ __forceinline__ void epilogue_load_to_lds(const void *base, uint32_t offset, unsigned lds_addr)
 {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(offset),
@@ -201,33 +201,9 @@ __device__ __forceinline__ void zero_point_reads_half(RowAt row_at, int row_a, i
     }
 }
 
-// facc[i][j][e]: MFMA tile (i, j) of this wave, element e in the 32x32 accumulator layout (row
-// 8 * (e / 4) + 4 * g + e % 4, column r).  smem: the workgroup's LDS, free for reuse once a barrier has
-// been passed (only the fp16 store uses it).
-//
-// The weight zero points are a small matrix product of their own, out -= Sx (M x groups) times
-// (w_scale * w_zero)^T (groups x N), done on the bf16 matrix cores (v_mfma_f32_32x32x16_bf16, an eighth of the
-// time of the fp32 instruction per product) without loss: a group sum of at most 128 8-bit codes splits exactly
-// into two bf16 numbers (its multiple of 128 and the remainder below 128), c = -w_scale * w_zero into bf16(c) and
-// bf16(c - bf16(c)), both rounded to nearest, which carries c to 2^-18 relative; the four products of the pieces
-// take four of the instruction's sixteen K slots, so one instruction covers four groups and a chunk of 32 groups
-// takes eight per MFMA tile.  Lane (r, g) supplies row r of the activation block and column r of the weight block
-// for the K slots 8 g .. 8 g + 7, i.e. for two groups; which two is free as long as both operands agree, and the
-// choice here, groups 16 g + 2 q and 16 g + 2 q + 1 for instruction q of the chunk, lets every lane read its
-// sixteen groups of a row as 64 contiguous bytes straight from global memory: no staging, no barrier.
-// LDS_BYTES: size of the workgroup's LDS at smem.  AHEAD: how far the loads of the zero-point term run ahead of their
-// use, for the kernels that have the registers: 0 = half a chunk is loaded, multiplied, then the other half (two memory
-// latencies per chunk); 1 = a chunk's loads are all requested before any is used; 2 = and the next chunk's before the
-// current one is multiplied (K = 11008 has three chunks).
-// VIA_LDS (kernels whose K loop leaves the whole LDS free, every wave of the workgroup here): the whole chunks of rows
-// that start on 16-byte boundaries come through LDS instead.  A lane's 16-byte pieces of 32 different rows touch 32
-// cache lines per load instruction and use 32 bytes of each; with all waves of a compute unit doing that over some
-// 100 KB of lines the 32 KB L1 fetches every line several times (QKV of LLaMA-7B at 16384 tokens: the term cost 10 %
-// of the GEMM).  Staged, a load instruction takes eight whole rows of the workgroup's tile (every line once, no
-// registers), and the lanes pick their pieces out of LDS.
-// (Requesting the first chunk from inside the K loop's last trips, whose load slots and stages go to waste, was built
-// and dropped: branches in the loop body, or copies of it with other requests, cost the integer tiles 40-90 spilled
-// registers.)
+// Byte offset, from *base, of what a lane requests for unit u (eight rows) of a chunk staged through LDS (see
+// group_scale_epilogue): rows 0 .. RA - 1 of the units are the tile's rows of group sums, then RB rows of scales, then RB
+// rows of zero points; lane l brings the 16-byte piece (l % 8) ^ ((row / 2) % 8) of row 8 u + l / 8.
 template <int RA, int RB>
 __device__ __forceinline__ uint32_t zero_point_unit_offset(const GemmArgs &a, int u, int lane, int m0, int n0, int M, int N, int groups,
                                                            int first, const void **base)
@@ -247,6 +223,33 @@ __device__ __forceinline__ bool zero_point_rows_aligned(const GemmArgs &a, int g
                                   reinterpret_cast<size_t>(a.w_zero)) & 15) == 0;
 }
 
+// facc[i][j][e]: MFMA tile (i, j) of this wave, element e in the 32x32 accumulator layout (row
+// 8 * (e / 4) + 4 * g + e % 4, column r).  smem: the workgroup's LDS, free for reuse once a barrier has
+// been passed (only the fp16 store uses it).
+//
+// The weight zero points are a small matrix product of their own, out -= Sx (M x groups) times
+// (w_scale * w_zero)^T (groups x N), done on the bf16 matrix cores (v_mfma_f32_32x32x16_bf16, an eighth of the
+// time of the fp32 instruction per product) without loss: a group sum of at most 128 8-bit codes splits exactly
+// into two bf16 numbers (its multiple of 128 and the remainder below 128), c = -w_scale * w_zero into bf16(c) and
+// bf16(c - bf16(c)), both rounded to nearest, which carries c to 2^-18 relative; the four products of the pieces
+// take four of the instruction's sixteen K slots, so one instruction covers four groups and a chunk of 32 groups
+// takes eight per MFMA tile.  Lane (r, g) supplies row r of the activation block and column r of the weight block
+// for the K slots 8 g .. 8 g + 7, i.e. for two groups; which two is free as long as both operands agree, and the
+// choice here, groups 16 g + 2 q and 16 g + 2 q + 1 for instruction q of the chunk, lets every lane read its
+// sixteen groups of a row as 64 contiguous bytes straight from global memory: no staging, no barrier.
+// LDS_BYTES: size of the workgroup's LDS at smem.  AHEAD: how far the loads of the zero-point term run ahead of their
+// use, for the kernels that have the registers: 0 = half a chunk is loaded, multiplied, then the other half (two memory
+// latencies per chunk); 1 = a chunk's loads are all requested before any is used; 2 = and the next chunk's before the
+// current one is multiplied (K = 11008 has three chunks).
+// VIA_LDS (kernels whose K loop leaves the whole LDS free, every wave of the workgroup here): where the arrays' rows
+// start on 16-byte boundaries the chunks come through LDS instead.  A lane's 16-byte pieces of 32 different rows touch 32
+// cache lines per load instruction and use 32 bytes of each; with all waves of a compute unit doing that over some
+// 100 KB of lines the 32 KB L1 fetches every line several times (QKV of LLaMA-7B at 16384 tokens: the term cost 10 %
+// of the GEMM).  Staged, a load instruction takes eight whole rows of the workgroup's tile (every line once, no
+// registers), and the lanes pick their pieces out of LDS.
+// (Requesting the first chunk from inside the K loop's last trips, whose load slots and stages go to waste, was built
+// and dropped: branches in the loop body, or copies of it with other requests, cost the integer tiles 40-90 spilled
+// registers.)
 template <int TM, int TN, int WM, int WN, int LDS_BYTES, int AHEAD = 0, bool VIA_LDS = false>
 __device__ __forceinline__ void group_scale_epilogue(const GemmArgs &a, v16f (&facc)[TM][TN], unsigned char *smem, int M,
                                                      int N, int m0, int n0, int wm, int wn, int r, int g, int tid)
