@@ -313,10 +313,19 @@ size_t ABQGEMMWrapper::activation_bytes(int M, int K) const
     return ((size_t)bits * M * K / 8 + 255) / 256 * 256;
 }
 
-void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _Float16 *A, const ABQGroupedWeight &W,
+void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _Float16 *A, const ABQGroupedWeight &W_given,
                                   _Float16 *D, bool x_symmetric, char *abq_gemm_workspace, size_t abq_gemm_ws_bytes,
                                   hipStream_t stream, bool silu_gate)
 {
+    // Weights of 3, 5, 6 or 7 bits whose folded records are as wide as their padded ones: the folded records take the
+    // padded records' place in every call, and the weights have no zero points any more (W3A8 with groups of 128 at one
+    // token: 3.8 / 6.7 / 7.3 us against 4.0 / 7.3 / 8.1 on padded records with zero points)
+    ABQGroupedWeight W = W_given;
+    if (W.records_folded && W.zero && abq_padded_bits(w_bits_) != w_bits_ && abq_folded_bits(w_bits_) == abq_padded_bits(w_bits_)) {
+        W.records_padded = W.records_folded;
+        W.records_folded = nullptr;
+        W.zero = nullptr;
+    }
     if (K < 128 || K % 128 != 0) {
         printf("[ABQ][Error] unsupport K = %d\n", K);
         return;

@@ -44,7 +44,9 @@ struct ABQGroupedWeight {
     const int *records_folded; // weights with whole-number zero points, at most 7 bits: the same weights as records of
                               // code - zero point (abq_relayout_planes_folded; twice the bytes of 2-bit weights), or
                               // nullptr; with it, prefill-sized calls (those that leave the decode kernels) run on
-                              // them without the zero-point term, 3-19 % faster (most at K = 11008)
+                              // them without the zero-point term, 3-19 % faster (most at K = 11008); for weights of
+                              // 3, 5, 6, 7 bits they are as wide as the padded records and serve every call in their
+                              // place
 };
 
 class ABQGEMMWrapper {

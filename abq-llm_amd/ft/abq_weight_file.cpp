@@ -251,6 +251,9 @@ bool ABQDeviceWeight::load(const ABQWeightBlob &blob, hipStream_t stream, std::s
             (void)hipFree(folded_);
             folded_ = nullptr;
             rc = rc == ABQ_ERR_UNSUPPORTED ? ABQ_OK : rc;
+        } else if (padded_ && abq_folded_bits((int)info_.bits) == abq_padded_bits((int)info_.bits)) {
+            (void)hipFree(padded_); // records of the same width without the zero points: gemm_dynamic runs every call on the folded ones
+            padded_ = nullptr;
         }
     }
     if (rc != ABQ_OK)

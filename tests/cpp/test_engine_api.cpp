@@ -498,6 +498,9 @@ static void gpu_paths()
     dynamic_case(2, 300, false, false, true); // prefill on records with the zero points folded in (4-bit records of 2-bit weights)
     dynamic_case(3, 300, true, false, true);  // ... of 3-bit weights
     dynamic_case(2, 8, false, false, true);   // decode-sized: the weights' own records
+    dynamic_case(3, 8, false, false, true);   // 3-bit weights: the folded records at every size (decode kernel, two launches)
+    dynamic_case(3, 1, false, false, true);   // ... one launch
+    dynamic_case(3, 40, false, false, true);
 
     for (const int WB : { 4, 3 })
     for (const int M : { 24, 3 }) {
@@ -522,7 +525,9 @@ static void gpu_paths()
         std::remove(path.c_str());
         ABQDeviceWeight dw;
         CHECK(dw.load(blob, stream, &err));
-        CHECK((dw.grouped().records_padded != nullptr) == (WB == 3));
+        // (3-bit weights: padded records, or, their zero points being whole numbers, folded ones of the same width)
+        CHECK((dw.grouped().records_padded != nullptr || dw.grouped().records_folded != nullptr) == (WB == 3 || dw.grouped().records_folded != nullptr));
+        CHECK(WB != 3 || dw.grouped().records_folded != nullptr);
         std::vector<int> codes((size_t)N * K);
         abq_oracle_unpack(blob.planes.data(), codes.data(), N, K, WB, 1);
         std::vector<uint16_t> ha((size_t)M * K);
