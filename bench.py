@@ -641,6 +641,8 @@ def main():
             W3 = w3.unsqueeze(0).repeat(R3, 1, 1, 1)
             wsc = torch.rand((N, G), device="cuda") * 0.01 + 0.001
             wz = torch.randint(-4, 4, (N, G), device="cuda").float()
+            # (records of code - zero point, as wide as the padded ones: no zero points left to read)
+            Wf3 = abq.relayout_planes_folded(w3, wz, 128, SIGNED).unsqueeze(0).repeat(R3, 1, 1, 1, 1)
             for M in (1, 8):
                 xsc = torch.rand(M, device="cuda") * 0.05 + 0.01
                 sums = torch.randint(-1000, 1000, (M, G), dtype=torch.int32, device="cuda")
@@ -649,11 +651,14 @@ def main():
                 gs = [abq.Gemm(xs_tiled[(M, K)], Wp3[r], SIGNED, x_tiled=True, w_tiled=True, value_bits=(Q_BITS, 3), **kw) for r in range(R3)]
                 us = time_rotating(gs)
                 us_planes = time_rotating([abq.Gemm(xs[(M, K)], W3[r], SIGNED, **kw) for r in range(R3)])
+                kwf = dict(kw, w_zero=None, x_group_sums=None)
+                us_folded = time_rotating([abq.Gemm(xs_tiled[(M, K)], Wf3[r], SIGNED, x_tiled=True, w_tiled=True, **kwf) for r in range(R3)])
                 deq3.append(dict(M=M, N=N, K=K, w_bits=3, group_size=128, us=round(us, 3), kernel="%s:%s" % (gs[0].strategy, gs[0].config_name),
-                                 plane_operands_us=round(us_planes, 3)))
-                log("dequant decode W3A8 M=%d N=%d K=%d  %.2f us (%s, padded records); plane operands %.2f us" % (M, N, K, us, gs[0].strategy, us_planes))
+                                 plane_operands_us=round(us_planes, 3), folded_zero_points_us=round(us_folded, 3)))
+                log("dequant decode W3A8 M=%d N=%d K=%d  %.2f us (%s, padded records); plane operands %.2f us; zero points folded in %.2f us"
+                    % (M, N, K, us, gs[0].strategy, us_planes, us_folded))
                 del gs, out
-            del Wp3, W3
+            del Wp3, W3, Wf3
         # ... and a prefill of 1024 tokens on the same 3-bit weights: padded 4-bit records (the 4-bit pair's LDS-staged
         # kernel) against the 3-bit records (the register-staged kernel of the odd widths)
         pre3 = []
