@@ -512,11 +512,18 @@ int main(int argc, char **argv)
     }
     // (above 16 rows only where the padded pair's weights are K-tiled records as well)
     const bool padded_prefill = M > 16 && padded && !group && abq_preferred_weight_layout(xq, wq, is_signed, M, N, K, 0) == ABQ_LAYOUT_TILED;
-    if (M <= 16 ? (padded || with_sums) : padded_prefill) {
+    const bool want_wpad = M <= 16 ? (padded || with_sums) : padded_prefill;
+    if (want_wpad || xq != x_bits) { // (activations of several fields: what the NSTAGE 6 tiles read at any M)
         HIP_OK(hipMalloc(&d_xpad, abq_planes_bytes(M, K, xq)));
+        if (abq_relayout_planes_padded(d_xp, d_xpad, M, K, x_bits, is_signed, stream) != ABQ_OK) {
+            std::printf("preparing padded records failed (hip error %d)\n", abq_last_hip_error());
+            return -1;
+        }
+        HIP_OK(hipStreamSynchronize(stream));
+    }
+    if (want_wpad) {
         HIP_OK(hipMalloc(&d_wpad, wpad_bytes * nbuf_pad));
-        if (abq_relayout_planes_padded(d_xp, d_xpad, M, K, x_bits, is_signed, stream) != ABQ_OK ||
-            abq_relayout_planes_padded(d_wp, d_wpad, N, K, w_bits, is_signed, stream) != ABQ_OK) {
+        if (abq_relayout_planes_padded(d_wp, d_wpad, N, K, w_bits, is_signed, stream) != ABQ_OK) {
             std::printf("preparing padded records failed (hip error %d)\n", abq_last_hip_error());
             return -1;
         }
