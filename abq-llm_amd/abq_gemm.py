@@ -38,7 +38,7 @@ EXPORTED = [
     "abq_gemm_exec_static", "abq_gemm_set_f16_activations",
     "abq_row_sums", "abq_gemm_set_row_sums", "abq_gemm_row_sums_ready",
     "abq_tuning_load", "abq_tuning_add", "abq_tuning_clear", "abq_tuning_enable_builtin", "abq_tuning_lookup",
-    "abq_preferred_weight_layout", "abq_preferred_weight_records", "abq_padded_bits", "abq_folded_bits", "abq_relayout_planes_folded", "abq_relayout_planes_padded", "abq_gemm_set_value_bits",
+    "abq_preferred_weight_layout", "abq_preferred_weight_records", "abq_padded_bits", "abq_folded_bits", "abq_relayout_planes_folded", "abq_relayout_planes_fp6_folded", "abq_relayout_planes_padded", "abq_gemm_set_value_bits",
     "abq_gemm_set_padded_activations",
     "abq_relayout_planes_biased", "abq_gemm_set_biased_records", "abq_pack_f16_fp6",
 ]
@@ -155,6 +155,7 @@ def lib():
         L.abq_padded_bits.restype = ci
         L.abq_relayout_planes_padded.argtypes = [vp, vp, ci, ci, ci, ci, vp]
         L.abq_relayout_planes_folded.argtypes = [vp, vp, ci, vp, ci, ci, ci, ci, vp, vp]
+        L.abq_relayout_planes_fp6_folded.argtypes = [vp, vp, ci, vp, ci, ci, ci, ci, vp, vp]
         L.abq_folded_bits.argtypes = [ci]
         L.abq_gemm_set_value_bits.argtypes = [ctypes.POINTER(GemmState), ci, ci]
         L.abq_gemm_set_padded_activations.argtypes = [ctypes.POINTER(GemmState), ci]
@@ -320,6 +321,21 @@ def relayout_planes_folded(planes, w_zero, group_size, signed, stream=None):
                                             int(bool(signed)), misfit.data_ptr(), _stream_ptr(stream)), "abq_relayout_planes_folded")
     if int(misfit.item()):
         raise ValueError("zero points that are no whole numbers, or differences that do not fit the records")
+    return out
+
+
+def relayout_planes_fp6_folded(planes, w_zero, group_size, signed, stream=None):
+    """The same as FP6 records [k/128, rows, 24] (codes of at most 4 bits); used under the pair's own widths on a signed GEMM."""
+    import torch
+    bits, rows, kw = planes.shape
+    assert planes.is_cuda and planes.is_contiguous() and kw % 4 == 0
+    assert w_zero.dtype == torch.float32 and w_zero.is_contiguous() and tuple(w_zero.shape) == (rows, kw * 32 // group_size)
+    out = torch.empty((kw // 4, rows, 24), dtype=torch.int32, device=planes.device)
+    misfit = torch.zeros(1, dtype=torch.int32, device=planes.device)
+    _check(lib().abq_relayout_planes_fp6_folded(planes.data_ptr(), w_zero.data_ptr(), group_size, out.data_ptr(), rows, kw * 32, bits,
+                                                int(bool(signed)), misfit.data_ptr(), _stream_ptr(stream)), "abq_relayout_planes_fp6_folded")
+    if int(misfit.item()):
+        raise ValueError("zero points that are no whole numbers, or differences without an FP6 code")
     return out
 
 

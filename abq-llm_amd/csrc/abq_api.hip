@@ -22,7 +22,8 @@ hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream
 hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes_padded(const uint32_t *, uint32_t *, int, int, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes_folded(const uint32_t *, const float *, int, uint32_t *, int, int, int, int, int, int *, hipStream_t);
-hipError_t launch_relayout_planes_fp6(const uint32_t *, uint32_t *, int, int, int, int, hipStream_t);
+hipError_t launch_relayout_planes_fp6(const uint32_t *, uint32_t *, int, int, int, int, hipStream_t, const float *zero = nullptr,
+                                      int group_size = 0, int *flag = nullptr);
 hipError_t launch_row_sums(const uint32_t *, int *, int, int, int, hipStream_t);
 const KernelEntry *fp6_entries(int *count);
 const KernelEntry *fp6_grouped_entries(int *count);
@@ -1911,6 +1912,19 @@ abq_status abq_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int ro
     if (k < 128 || k % 128 != 0)
         return ABQ_ERR_BAD_K;
     return hip_status(launch_relayout_planes_fp6(planes, fp6, rows, k, bits, is_signed ? 1 : 0, (hipStream_t)stream));
+}
+
+abq_status abq_relayout_planes_fp6_folded(const uint32_t *planes, const float *w_zero, int group_size, uint32_t *fp6, int rows, int k,
+                                          int bits, int is_signed, int *misfit_dev, void *stream)
+{
+    if (!planes || !w_zero || !fp6 || rows <= 0 || bits < 1 || group_size < 32 || group_size % 32 != 0)
+        return ABQ_ERR_INVALID_ARG;
+    if (bits > 4)
+        return ABQ_ERR_UNSUPPORTED; // wider codes less their zero points leave the range of the FP6 codes
+    if (k < 128 || k % 128 != 0 || k % group_size != 0)
+        return ABQ_ERR_BAD_K;
+    return hip_status(launch_relayout_planes_fp6(planes, fp6, rows, k, bits, is_signed ? 1 : 0, (hipStream_t)stream, w_zero, group_size,
+                                                 misfit_dev));
 }
 
 size_t abq_gemm_workspace_bytes(const abq_gemm_state *st)

@@ -340,6 +340,22 @@ hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int r
 // [12 (ws & 1) + 6 (ws >> 1), +6): the two word-sets that lanes 0-31 feed to the two MFMA
 // K steps come first, then the two of lanes 32-63.  Records are stored fp6[kt][row][24].
 
+// r[0..4]: bit-sliced magnitude, r[5]: sign, r[6], r[7]: zero -> the word-set's string of 6-bit codes.
+__device__ __forceinline__ void fp6_string_of_codes(uint32_t (&r)[8], uint32_t (&out)[6])
+{
+    transpose8x8x4(r); // dword d, byte c: the code of the element at plane bit 8c + d
+    uint32_t y[8];
+#pragma unroll
+    for (int d = 0; d < 8; ++d)
+        y[d] = (r[d] & 0x3Fu) | ((r[d] >> 2) & 0xFC0u) | ((r[d] >> 4) & 0x3F000u) | ((r[d] >> 6) & 0xFC0000u);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        out[3 * h + 0] = y[4 * h] | (y[4 * h + 1] << 24);
+        out[3 * h + 1] = (y[4 * h + 1] >> 8) | (y[4 * h + 2] << 16);
+        out[3 * h + 2] = (y[4 * h + 2] >> 16) | (y[4 * h + 3] << 8);
+    }
+}
+
 // Bit-sliced |value| and sign of 32 elements: p[t] = plane t, planes at and above bits - 1 read
 // as the sign plane (two's complement sign extension) when the operand is signed.
 __device__ __forceinline__ void fp6_string(const uint32_t (&p)[5], int bits, bool is_signed, uint32_t (&out)[6])
@@ -356,26 +372,49 @@ __device__ __forceinline__ void fp6_string(const uint32_t (&p)[5], int bits, boo
     r[5] = s;
     r[6] = 0u;
     r[7] = 0u;
-    transpose8x8x4(r); // dword d, byte c: the code of the element at plane bit 8c + d
-    uint32_t y[8];
-#pragma unroll
-    for (int d = 0; d < 8; ++d)
-        y[d] = (r[d] & 0x3Fu) | ((r[d] >> 2) & 0xFC0u) | ((r[d] >> 4) & 0x3F000u) | ((r[d] >> 6) & 0xFC0000u);
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        out[3 * h + 0] = y[4 * h] | (y[4 * h + 1] << 24);
-        out[3 * h + 1] = (y[4 * h + 1] >> 8) | (y[4 * h + 2] << 16);
-        out[3 * h + 2] = (y[4 * h + 2] >> 16) | (y[4 * h + 3] << 8);
-    }
+    fp6_string_of_codes(r, out);
 }
+
+// The same for code - z (a weight zero point folded in): the difference of the bit-sliced codes and the constant as six
+// planes of two's complement, then sign and magnitude as above.  Returns a word with a bit set for every element whose
+// difference has a magnitude above 16 (no E2M3 number).  |z| <= 32.
+__device__ __forceinline__ uint32_t fp6_string_folded(const uint32_t (&p)[5], int bits, bool is_signed, int z, uint32_t (&out)[6])
+{
+    uint32_t d[6], borrow = 0u;
+#pragma unroll
+    for (int t = 0; t < 6; ++t) {
+        const uint32_t a = t < bits ? p[t] : (is_signed ? p[bits - 1] : 0u);
+        const uint32_t zb = ((z >> t) & 1) ? 0xFFFFFFFFu : 0u;
+        d[t] = a ^ zb ^ borrow;
+        borrow = (~a & zb) | (~(a ^ zb) & borrow);
+    }
+    const uint32_t s = d[5];
+    uint32_t r[8], carry = s;
+#pragma unroll
+    for (int t = 0; t < 5; ++t) {
+        const uint32_t x = d[t] ^ s;
+        r[t] = x ^ carry;
+        carry &= x;
+    }
+    const uint32_t misfit = carry | (r[4] & (r[0] | r[1] | r[2] | r[3])); // -32, or a magnitude of 17 .. 31
+    r[5] = s;
+    r[6] = 0u;
+    r[7] = 0u;
+    fp6_string_of_codes(r, out);
+    return misfit;
+}
+
 
 // One thread per word-set; a workgroup covers 8 rows x 8 K tiles (32 consecutive plane words of a
 // row are one coalesced 128-byte read per plane) and writes each tile's 8 records (contiguous in
 // memory) with 16-byte stores out of LDS.
+// zero != nullptr (weights with group-wise zero points, group_size a multiple of 32): the records hold code - zero
+// point, zero[row][k / group_size]; *flag is set where a zero point is no whole number or a difference has no FP6 code.
 template <int BITS>
 __global__ __launch_bounds__(256) void relayout_planes_fp6_kernel(const uint32_t *__restrict__ planes,
                                                                   uint32_t *__restrict__ fp6, int rows, int KW,
-                                                                  int is_signed)
+                                                                  int is_signed, const float *__restrict__ zero = nullptr,
+                                                                  int group_size = 0, int *flag = nullptr)
 {
     constexpr int REC = 24;
     constexpr int SLAB = 8 * REC + 4; // words per K tile in LDS (+16 bytes against bank conflicts)
@@ -394,7 +433,16 @@ __global__ __launch_bounds__(256) void relayout_planes_fp6_kernel(const uint32_t
             for (int b = 0; b < 5; ++b)
                 pw[b] = b < BITS ? p[b * plane_stride] : 0u;
             uint32_t o[6];
-            fp6_string(pw, BITS, is_signed != 0, o);
+            if (zero) {
+                const float zf = zero[(size_t)row * (KW * 32 / group_size) + kw * 32 / group_size];
+                const float zr = rintf(zf);
+                const bool whole = zr == zf && fabsf(zr) <= 31.f;
+                const uint32_t misfit = fp6_string_folded(pw, BITS, is_signed != 0, whole ? (int)zr : 0, o);
+                if ((!whole || misfit) && flag)
+                    *flag = 1;
+            } else {
+                fp6_string(pw, BITS, is_signed != 0, o);
+            }
             const int ws = w & 3;
             uint32_t *rec = buf + (w >> 2) * SLAB + i * REC + 12 * (ws & 1) + 6 * (ws >> 1);
             *reinterpret_cast<uint2 *>(rec) = make_uint2(o[0], o[1]);
@@ -449,14 +497,15 @@ hipError_t launch_row_sums(const uint32_t *planes, int *sums, int rows, int k, i
 }
 
 hipError_t launch_relayout_planes_fp6(const uint32_t *planes, uint32_t *fp6, int rows, int k, int bits, int is_signed,
-                                      hipStream_t stream)
+                                      hipStream_t stream, const float *zero, int group_size, int *flag)
 {
     const int KW = k / 32;
     const dim3 grid((rows + 7) / 8, (KW / 4 + 7) / 8);
     switch (bits) {
 #define ABQ_FP6_CASE(B)                                                                                                  \
     case B:                                                                                                              \
-        hipLaunchKernelGGL(relayout_planes_fp6_kernel<B>, grid, dim3(256), 0, stream, planes, fp6, rows, KW, is_signed); \
+        hipLaunchKernelGGL(relayout_planes_fp6_kernel<B>, grid, dim3(256), 0, stream, planes, fp6, rows, KW, is_signed, zero, \
+                           group_size, flag);                                                                            \
         break;
         ABQ_FP6_CASE(1) ABQ_FP6_CASE(2) ABQ_FP6_CASE(3) ABQ_FP6_CASE(4) ABQ_FP6_CASE(5)
 #undef ABQ_FP6_CASE

@@ -321,11 +321,16 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     // padded records' place in every call, and the weights have no zero points any more (W3A8 with groups of 128 at one
     // token: 3.8 / 6.7 / 7.3 us against 4.0 / 7.3 / 8.1 on padded records with zero points)
     ABQGroupedWeight W = W_given;
+    if (W.records_folded && abq_native_config_count(x_bits_, abq_folded_bits(w_bits_), 1) <= 0)
+        W.records_folded = nullptr; // (no kernels for the activations' width against the folded records')
     if (W.records_folded && W.zero && abq_padded_bits(w_bits_) != w_bits_ && abq_folded_bits(w_bits_) == abq_padded_bits(w_bits_)) {
         W.records_padded = W.records_folded;
         W.records_folded = nullptr;
         W.zero = nullptr;
     }
+    // (FP6 records with the zero points folded in stand for the plain ones on the FP6 route)
+    const bool fp6_folded = W.records_fp6_folded != nullptr && W.zero != nullptr && w_bits_ <= 4;
+    const int *const records_fp6 = fp6_folded ? W.records_fp6_folded : W.records_fp6;
     if (K < 128 || K % 128 != 0) {
         printf("[ABQ][Error] unsupport K = %d\n", K);
         return;
@@ -361,7 +366,7 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     // (if the expanded activations fit the decode kernel's LDS: partial tiles, group sums, M padded rows)
     const bool decode = !decode_prepared && M <= 16 && W.planes != nullptr &&
                         (silu_gate ? 32 : 16) * 1024 + (size_t)64 * (K / W.group_size) + 128 + (size_t)M * ((K + 511) / 512 * 512 + 16) <= 160 * 1024;
-    const bool fp6 = !decode && !decode_prepared && W.records_fp6 != nullptr && W.group_size == 128 && abq_fp6_eligible(x_bits_, w_bits_, 1, K);
+    const bool fp6 = !decode && !decode_prepared && records_fp6 != nullptr && W.group_size == 128 && abq_fp6_eligible(x_bits_, w_bits_, 1, K);
     const int layout = decode ? ABQ_LAYOUT_PLANES : fp6 ? ABQ_LAYOUT_FP6 : ABQ_LAYOUT_TILED;
     abq_status rc;
     abq_gemm_state state;
@@ -409,7 +414,7 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
         return;
     }
     rc = abq_gemm_init(nullptr, x_bits_, on_folded ? abq_folded_bits(w_bits_) : on_padded ? w_rec_bits : w_bits_, 1, planes,
-                       decode ? reinterpret_cast<const uint32_t *>(W.planes) : fp6 ? reinterpret_cast<const uint32_t *>(W.records_fp6)
+                       decode ? reinterpret_cast<const uint32_t *>(W.planes) : fp6 ? reinterpret_cast<const uint32_t *>(records_fp6)
                        : on_folded ? reinterpret_cast<const uint32_t *>(W.records_folded)
                        : on_padded ? w_records : reinterpret_cast<const uint32_t *>(W.planes_tiled), M, N, K,
                        D, nullptr, 0, ABQ_OUT_F16_SCALED, &state);
@@ -419,7 +424,7 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
         rc = abq_gemm_set_operand_layout(&state, layout, layout);
     if (rc == ABQ_OK)
         rc = abq_gemm_set_scales(&state, x_scale, W.scale, W.group_size);
-    if (rc == ABQ_OK && on_folded) {
+    if (rc == ABQ_OK && (on_folded || (fp6 && fp6_folded))) {
         if (!x_symmetric)
             rc = abq_gemm_set_zero_points(&state, x_zero, nullptr, nullptr, W.zero_term);
     } else if (rc == ABQ_OK && (W.zero || !x_symmetric)) {

@@ -191,6 +191,7 @@ void ABQDeviceWeight::release()
         if (p)
             (void)hipFree(p);
     planes_ = tiled_ = fp6_ = padded_ = folded_ = nullptr;
+    fp6_is_folded_ = false;
     scale_ = zero_ = zero_term_ = nullptr;
 }
 
@@ -226,6 +227,30 @@ bool ABQDeviceWeight::load(const ABQWeightBlob &blob, hipStream_t stream, std::s
         if (!hip_ok(hipMalloc(&fp6_, abq_fp6_bytes((int)info_.n, (int)info_.k)), "hipMalloc fp6"))
             return false;
         rc = abq_relayout_planes_fp6(planes_, fp6_, (int)info_.n, (int)info_.k, (int)info_.bits, (int)info_.is_signed, stream);
+        // with whole-number zero points (and at most 4 bits) the same records hold code - zero point instead
+        if (rc == ABQ_OK && info_.has_zero && info_.bits <= 4u) {
+            int *misfit = nullptr, host_misfit = 1;
+            uint32_t *folded = nullptr;
+            if (!hip_ok(hipMalloc(&folded, abq_fp6_bytes((int)info_.n, (int)info_.k)), "hipMalloc fp6 folded") ||
+                !hip_ok(hipMalloc(&misfit, sizeof(int)), "hipMalloc flag") || !hip_ok(hipMemsetAsync(misfit, 0, sizeof(int), stream), "clear flag"))
+                return false;
+            const abq_status frc = abq_relayout_planes_fp6_folded(planes_, zero_, 128, folded, (int)info_.n, (int)info_.k, (int)info_.bits,
+                                                                  (int)info_.is_signed, misfit, stream);
+            const bool copied = hip_ok(hipMemcpyAsync(&host_misfit, misfit, sizeof(int), hipMemcpyDeviceToHost, stream), "read flag") &&
+                                hip_ok(hipStreamSynchronize(stream), "synchronise");
+            (void)hipFree(misfit);
+            if (!copied) {
+                (void)hipFree(folded);
+                return false;
+            }
+            if (frc == ABQ_OK && !host_misfit) {
+                (void)hipFree(fp6_);
+                fp6_ = folded;
+                fp6_is_folded_ = true;
+            } else {
+                (void)hipFree(folded);
+            }
+        }
     }
     // padded records for the widths of several fields: the kernels of the next single-field width read those
     if (rc == ABQ_OK && abq_padded_bits((int)info_.bits) != (int)info_.bits) {
@@ -264,6 +289,7 @@ bool ABQDeviceWeight::load(const ABQWeightBlob &blob, hipStream_t stream, std::s
 ABQGroupedWeight ABQDeviceWeight::grouped() const
 {
     return ABQGroupedWeight{ reinterpret_cast<const int *>(tiled_), scale_, zero_, zero_term_, (int)info_.group_size,
-                             reinterpret_cast<const int *>(planes_), reinterpret_cast<const int *>(fp6_),
-                             reinterpret_cast<const int *>(padded_), reinterpret_cast<const int *>(folded_) };
+                             reinterpret_cast<const int *>(planes_), fp6_is_folded_ ? nullptr : reinterpret_cast<const int *>(fp6_),
+                             reinterpret_cast<const int *>(padded_), reinterpret_cast<const int *>(folded_),
+                             fp6_is_folded_ ? reinterpret_cast<const int *>(fp6_) : nullptr };
 }

@@ -92,5 +92,6 @@ private:
     uint32_t *planes_ = nullptr, *tiled_ = nullptr, *fp6_ = nullptr; // fp6_: only for groups of 128 and at most 5 (4 unsigned) bits
     uint32_t *padded_ = nullptr;                                     // only for 3, 5, 6, 7 bits: records of the next width of one field
     uint32_t *folded_ = nullptr;                                     // only with whole-number zero points: records of code - zero point
+    bool fp6_is_folded_ = false;                                     // fp6_ holds code - zero point as well
     float *scale_ = nullptr, *zero_ = nullptr, *zero_term_ = nullptr;
 };

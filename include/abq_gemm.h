@@ -466,6 +466,14 @@ int abq_folded_bits(int bits);
 abq_status abq_relayout_planes_folded(const uint32_t *planes, const float *w_zero, int group_size, uint32_t *tiled, int rows, int k,
                                       int bits, int is_signed, int *misfit_dev, void *stream);
 
+/* The same for FP6 records (abq_relayout_planes_fp6's layout, same size): codes of at most 4 bits less whole-number
+ * zero points have magnitudes of at most 16 and therefore FP6 codes.  A GEMM on them is initialised like one on
+ * abq_relayout_planes_fp6's records, under the pair's own widths, SIGNED (activations that are unsigned codes come as
+ * FP6 records too, which hold their values), without weight zero points; exact for K up to 65536.  misfit_dev as
+ * above. */
+abq_status abq_relayout_planes_fp6_folded(const uint32_t *planes, const float *w_zero, int group_size, uint32_t *fp6, int rows, int k,
+                                          int bits, int is_signed, int *misfit_dev, void *stream);
+
 /* Declares that the codes of X (W) use only the low x_value_bits (w_value_bits) of their fields (1 .. the state's
  * widths): see above.  An operand of such a state that is still in the reference plane layout has that many planes,
  * and abq_gemm_exec extends its codes to the records' width while it converts them into the workspace.  This makes

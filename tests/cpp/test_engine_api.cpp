@@ -587,8 +587,10 @@ static void gpu_paths()
         ABQDeviceWeight dw;
         CHECK(dw.load(blob, stream, &err));
         ABQGroupedWeight with_fp6 = dw.grouped(), without = dw.grouped();
-        CHECK(with_fp6.records_fp6 != nullptr);
-        without.records_fp6 = nullptr;
+        // (the zero points of the quantiser are whole numbers: the FP6 records hold code - zero point)
+        CHECK(with_fp6.records_fp6 == nullptr && with_fp6.records_fp6_folded != nullptr);
+        without.records_fp6 = without.records_fp6_folded = nullptr;
+        without.records_folded = nullptr; // (W4A4 has no pair for 8-bit folded records anyway)
         std::vector<uint16_t> ha((size_t)M * K);
         for (auto &h : ha)
             h = abq_oracle_f32_to_f16(xd_(r32));

@@ -622,6 +622,38 @@ def test_zero_points_folded_into_the_weight_records(abq, oracle, p, signed_codes
         abq.relayout_planes_folded(wp, fdev(wz_bad), group_size, signed_codes)
 
 
+@pytest.mark.parametrize("q,p,signed_codes", [(4, 4, True), (4, 2, True), (3, 3, True), (4, 4, False), (4, 2, False)])
+def test_zero_points_folded_into_fp6_records(abq, oracle, q, p, signed_codes):
+    """The same on the FP6 route: FP6 records of code - zero point (magnitudes of at most 16), a signed GEMM without
+    weight zero points under the pair's own widths; unsigned codes and activations ride along as the signed numbers
+    they are (their records hold the values).  Against the
+    dequantised reference; a difference of magnitude 17 is reported."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(4600 + 10 * q + p + signed_codes)
+    lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed_codes else (0, 1 << p)
+    lo_x, hi_x = (-(1 << (q - 1)), 1 << (q - 1)) if signed_codes else (0, 1 << q)
+    for (M, N, K) in [(40, 96, 512), (300, 200, 640), (130, 264, 4096), (8, 64, 1152)]:
+        G = K // 128
+        x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
+        w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+        xs = rng.uniform(0.01, 0.05, M)
+        xz = rng.integers(lo_x // 2, hi_x // 2 + 1, M).astype(np.float64)
+        wsc = rng.uniform(0.001, 0.02, (N, G))
+        wz = rng.integers(lo_w, hi_w + (0 if signed_codes else 1), (N, G)).astype(np.float64)
+        want = Q.dequant_matmul(x, xs, xz, w, wsc, wz, 128)
+        wp, xp = planes_dev(oracle.pack_i32(w, p)), planes_dev(oracle.pack_i32(x, q))
+        term = abq.weight_zero_term(wp, signed_codes, fdev(wsc), fdev(wz), 128)
+        wf = abq.relayout_planes_fp6_folded(wp, fdev(wz), 128, signed_codes)
+        g = abq.Gemm(abq.relayout_planes_fp6(xp, signed_codes), wf, True, out_kind=abq.OUT_F16_SCALED, x_fp6=q, w_fp6=p,
+                     x_scale=fdev(xs), w_scale=fdev(wsc), group_size=128, x_zero=fdev(xz), w_zero_term=term)
+        assert g.strategy == "fp6"
+        assert_close_rel(g.run().float().cpu().numpy(), want)
+    wz_bad = wz.copy()
+    wz_bad[2, 0] = lo_w - 17.0  # code - zero point reaches 17
+    with pytest.raises(ValueError):
+        abq.relayout_planes_fp6_folded(wp, fdev(wz_bad), 128, signed_codes)
+
+
 @pytest.mark.parametrize("M,K", [(200, 4096), (130, 4608), (136, 8192)])
 @pytest.mark.parametrize("q,p,fp6", [(8, 2, False), (4, 4, False), (4, 4, True)])
 def test_zero_points_over_whole_chunks_of_groups(abq, oracle, M, K, q, p, fp6):
