@@ -654,6 +654,44 @@ def test_zero_points_folded_into_fp6_records(abq, oracle, q, p, signed_codes):
         abq.relayout_planes_fp6_folded(wp, fdev(wz_bad), 128, signed_codes)
 
 
+@pytest.mark.parametrize("q,p,fp6", [(8, 2, False), (8, 3, False), (8, 4, False), (8, 7, False), (4, 4, True), (4, 2, True), (3, 3, True)])
+@pytest.mark.parametrize("signed_codes", [True, False])
+def test_folded_records_accept_exactly_what_they_can_hold(abq, oracle, q, p, fp6, signed_codes):
+    """Zero points chosen from the weights so that the largest or the smallest difference of a group lands on the
+    last value the records hold (two's complement of the folded width; magnitude 16 on the FP6 records): accepted, and
+    the GEMM agrees with the dequantised reference.  One group moved one step further, at either end: reported."""
+    from oracle import quantizer as Q
+    rng = np.random.default_rng(5200 + 10 * q + p + 2 * fp6 + signed_codes)
+    M, N, K, gs = 24, 72, 640, 128
+    G = K // gs
+    lo_w, hi_w = (-(1 << (p - 1)), 1 << (p - 1)) if signed_codes else (0, 1 << p)
+    lo_x, hi_x = (-(1 << (q - 1)), 1 << (q - 1)) if signed_codes or not fp6 else (0, 1 << q)
+    rb = abq.lib().abq_folded_bits(p)
+    lim_lo, lim_hi = (-16, 16) if fp6 else (-(1 << (rb - 1)), (1 << (rb - 1)) - 1)
+    x = rng.integers(lo_x, hi_x, (M, K)).astype(np.int32)
+    w = rng.integers(lo_w, hi_w, (N, K)).astype(np.int32)
+    wg = w.reshape(N, G, gs)
+    z_least, z_most = wg.max(axis=2) - lim_hi, wg.min(axis=2) - lim_lo  # the zero points a group can take
+    wz = np.where(rng.integers(0, 2, (N, G)) == 0, z_least, z_most).astype(np.float64)
+    xs, wsc = rng.uniform(0.01, 0.05, M), rng.uniform(0.001, 0.02, (N, G))
+    xz = rng.integers(lo_x // 2, hi_x // 2 + 1, M).astype(np.float64)
+    wp, xp = planes_dev(oracle.pack_i32(w, p)), planes_dev(oracle.pack_i32(x, q))
+    fold = abq.relayout_planes_fp6_folded if fp6 else abq.relayout_planes_folded
+    wf = fold(wp, fdev(wz), gs, signed_codes)
+    kw = dict(out_kind=abq.OUT_F16_SCALED, x_scale=fdev(xs), w_scale=fdev(wsc), group_size=gs, x_zero=fdev(xz),
+              w_zero_term=abq.weight_zero_term(wp, signed_codes, fdev(wsc), fdev(wz), gs))
+    if fp6:
+        g = abq.Gemm(abq.relayout_planes_fp6(xp, signed_codes), wf, True, x_fp6=q, w_fp6=p, **kw)
+    else:
+        g = abq.Gemm(abq.relayout_planes(xp), wf, True, x_tiled=True, w_tiled=True, **kw)
+    assert_close_rel(g.run().float().cpu().numpy(), Q.dequant_matmul(x, xs, xz, w, wsc, wz, gs))
+    for (i, j, beyond) in [(3, 1, z_least[3, 1] - 1), (70, 4, z_most[70, 4] + 1)]:
+        wz_bad = wz.copy()
+        wz_bad[i, j] = beyond
+        with pytest.raises(ValueError):
+            fold(wp, fdev(wz_bad), gs, signed_codes)
+
+
 @pytest.mark.parametrize("M,K", [(200, 4096), (130, 4608), (136, 8192)])
 @pytest.mark.parametrize("q,p,fp6", [(8, 2, False), (4, 4, False), (4, 4, True)])
 def test_zero_points_over_whole_chunks_of_groups(abq, oracle, M, K, q, p, fp6):
