@@ -695,6 +695,9 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(4, 4, 512, 11008, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
     assert picked(8, 2, 512, 11008, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
     assert picked(4, 4, 2048, 4096, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)
+    # W8A8 with group scales: the LDS-staged kernel has the 128x64 tile only, and it is the faster one on large grids too
+    assert picked(8, 8, 16384, 4096, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
+    assert picked(8, 8, 2048, 12288, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)
     # group scales on FP6 records: 256x128 where its rounds of workgroups come out even
     assert picked(4, 4, 2048, 4096, 4096, F6, group=128) == (256, 128, 128, 64, 64, 5)
     assert picked(4, 4, 1024, 11008, 4096, F6, group=128) == (128, 128, 128, 64, 64, 5)   # 344 tiles of 256x128: 1.3 rounds
