@@ -9,6 +9,7 @@
 // fp16), turns them into one byte per plane with an 8x8 bit transpose, and the four lanes of
 // a quad assemble the bytes into one word per plane with DPP moves.  Input bytes are read
 // once, every load is 16 bytes wide and consecutive lanes touch consecutive memory.
+#include <climits>
 #include "abq_kernels.h"
 #include "abq_quant.h"
 
@@ -717,22 +718,28 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 // own point of their rows, so loads, arithmetic and stores of different rows overlap.  (With one workgroup per
 // row, a row's loads were in flight only during the first third of the workgroup's life: 3.2 TB/s where a plain
 // copy of the same buffers reaches 5.5.)  Rows of up to NU * 512 elements, NU <= 24 (beyond, the row spills).
-template <int LAYOUT, int NU, int BITS>
+// WPR = 4: the four waves of a workgroup share one row (wave w takes the rounds of 64 units w, w + 4, ...; NU is then
+// what one wave holds) and exchange their extrema through LDS: for the few hundred to two thousand rows of a small
+// prefill, where one wave per row leaves a SIMD with one or two waves and the time is a wave's own chain of
+// instructions (914 at K = 4096, 2359 at K = 11008) behind the latency of its loads.
+template <int LAYOUT, int NU, int BITS, int WPR = 1>
 __global__ __launch_bounds__(256) void quant_pack_wave_rows_kernel(const uint4 *__restrict__ x, uint32_t *__restrict__ planes,
                                                                    float *__restrict__ scale_out, float *__restrict__ zero_out,
                                                                    int *__restrict__ group_sums, int M, int K, int bits,
                                                                    int symmetric, int group_size)
 {
+    static_assert(WPR == 1 || WPR == 4, "one wave or the whole workgroup per row");
     const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int wsub = WPR == 1 ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // the wave's place in its row
+    const int row = WPR == 1 ? blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
     if (row >= M)
-        return; // whole waves leave: nothing below synchronises across waves
+        return; // whole waves leave: nothing below synchronises across waves (WPR = 4: the grid has M workgroups)
     const int units = K / 8;
     const uint4 *xr = x + (size_t)row * units;
     uint4 raw[NU];
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
-        const int u = lane + 64 * i;
+        const int u = lane + 64 * (i * WPR + wsub);
         // (read once: non-temporal; past the end: the row's first unit once more, it changes no extremum)
         typedef unsigned int unit_words __attribute__((ext_vector_type(4)));
         const unit_words w = __builtin_nontemporal_load(reinterpret_cast<const unit_words *>(xr + (u < units ? u : 0)));
@@ -755,8 +762,21 @@ __global__ __launch_bounds__(256) void quant_pack_wave_rows_kernel(const uint4 *
     float mx = fmaxf((float)mx2.x, (float)mx2.y), mn = fminf((float)mn2.x, (float)mn2.y);
     mx = wave_max(mx);
     mn = -wave_max(-mn);
+    if constexpr (WPR > 1) {
+        __shared__ float red[2][WPR];
+        if (lane == 0) {
+            red[0][wsub] = mx;
+            red[1][wsub] = mn;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < WPR; ++w) {
+            mx = fmaxf(mx, red[0][w]);
+            mn = fminf(mn, red[1][w]);
+        }
+    }
     const QuantRow q = quant_row_params(mx, mn, bits, symmetric);
-    if (lane == 0) {
+    if (lane == 0 && wsub == 0) {
         scale_out[row] = q.scale;
         if (zero_out)
             zero_out[row] = q.zero_out;
@@ -769,7 +789,8 @@ __global__ __launch_bounds__(256) void quant_pack_wave_rows_kernel(const uint4 *
         // The common case written out: 8-bit codes into K-tiled records.  Per unit: eight quotients, two byte
         // packs, the group sum as two dot products with ones and a butterfly of row operations over the
         // group's 8 or 16 lanes, two 4 x 4 byte transposes across the quad, one 8-byte store.  Unit
-        // u = lane + 64 i lies in K tile (lane >> 4) + 4 i: a fixed stride between a lane's records.
+        // u = lane + 64 j (round j = i, or i * WPR + the wave's place) lies in K tile (lane >> 4) + 4 j: a fixed stride
+        // between a lane's records.
         // clamp(rint(q) + zp, lo, hi) = rint(clamp(q, lo - zp, hi - zp)) + zp (the bounds are integers), and
         // adding 1.5 * 2^23 to a float of magnitude below 2^22 rounds it to an integer, to nearest even like rint,
         // and leaves that integer in the low mantissa bits: clamp, add, integer subtract.
@@ -784,7 +805,8 @@ __global__ __launch_bounds__(256) void quant_pack_wave_rows_kernel(const uint4 *
         const bool gs_lane = (lane & ((1 << glog) - 1)) == 0;
 #pragma unroll
         for (int i = 0; i < NU; ++i) {
-            if (64 * (i + 1) <= units) { // wave-uniform: every lane has a unit
+            const int j = i * WPR + wsub; // the round of 64 units
+            if (64 * (j + 1) <= units) { // wave-uniform: every lane has a unit
                 union {
                     uint4 q;
                     _Float16 h[8];
@@ -807,21 +829,21 @@ __global__ __launch_bounds__(256) void quant_pack_wave_rows_kernel(const uint4 *
                     if (glog == 4)
                         sum += __builtin_amdgcn_update_dpp(0, sum, 0x140, 0xF, 0xF, true); // row_mirror
                     if (gs_lane)
-                        gs[i * gs_stride] = sum;
+                        gs[j * gs_stride] = sum;
                 }
                 const uint32_t e_even = quad_transpose_bytes(pa, sel_pair, sel_half);
                 const uint32_t e_odd = quad_transpose_bytes(pb, sel_pair, sel_half);
-                *reinterpret_cast<uint2 *>(rec + i * rec_stride) = make_uint2(e_even, e_odd);
-            } else if (64 * i < units) { // the row's last, partly filled round
-                const int u = lane + 64 * i;
+                *reinterpret_cast<uint2 *>(rec + j * rec_stride) = make_uint2(e_even, e_odd);
+            } else if (64 * j < units) { // the row's last, partly filled round
+                const int u = lane + 64 * j;
                 quant_emit_unit<LAYOUT, BITS>(raw[i], u < units, u, row, M, K, bits, q, planes, group_sums, group_size, sel_pair, sel_half);
             }
         }
     } else {
 #pragma unroll
         for (int i = 0; i < NU; ++i) {
-            const int u = lane + 64 * i;
-            if (64 * i < units) // wave-uniform: units is a multiple of 16, so quads and groups are active as one
+            const int j = i * WPR + wsub, u = lane + 64 * j;
+            if (64 * j < units) // wave-uniform: units is a multiple of 16, so quads and groups are active as one
                 quant_emit_unit<LAYOUT, BITS>(raw[i], u < units, u, row, M, K, bits, q, planes, group_sums, group_size, sel_pair, sel_half);
         }
     }
@@ -900,11 +922,54 @@ hipError_t launch_quant_pack_rows(const void *x, uint32_t *planes, float *scale,
                                   int M, int K, int bits, int symmetric, int group_size, int layout,
                                   hipStream_t stream)
 {
-    // Many rows, or rows of at most 4096 elements: one wave per row, the row in registers (up to 12288 elements).
-    // (Measured on MI355X, 8-bit codes into K-tiled records: ahead of the kernel below from 16 rows up at K = 4096,
-    // from 1024 rows at K = 11008, where a lone wave's 22 units in a row cost more than four waves' barrier.)
-    const int nu = (K + 511) / 512;
-    if (nu <= 24 && (M >= 1024 || nu <= 8)) {
+    const int nu = (K + 511) / 512; // rounds of 64 units (512 elements) in a row
+    // A workgroup per row, a quarter of the row's rounds per wave, while one wave per row would leave the SIMDs with a
+    // wave or two each; the longer the row, the more rows that is (a lone wave holding 16 to 24 units per lane runs at a
+    // lower occupancy as well).  8-bit codes into K-tiled records with group sums, one wave per row -> four, us:
+    // K = 4096: 64 rows 5.3 -> 3.6, 512 5.6 -> 4.4, 1024 6.1 -> 5.5, 2048 8.3 -> 8.6; K = 2048: 256 4.1 -> 3.3, 2048 5.4 -> 6.2;
+    // K = 5120: 1024 7.4 -> 6.4, 4096 16.9 -> 17.4; K = 8192: 4096 26.2 -> 24.1, 16384 75.9 -> 83.6; K = 11008: 1024
+    // 13.4 -> 10.3, 8192 60.1 -> 54.2, 16384 107.8 -> 113.5; K = 13824 (against the kernel that keeps the row in LDS):
+    // 1024 16.4 -> 11.9, 16384 177 -> 142.
+    const int split_rows = nu <= 2 ? 256 : nu <= 8 ? 1024 : nu <= 12 ? 2048 : nu <= 16 ? 4096 : nu <= 24 ? 8192 : INT_MAX;
+    if (nu <= 32 && M <= split_rows) {
+        const dim3 grid(M), block(256);
+        const int nu4 = (nu + 3) / 4;
+#define ABQ_QP_SPLIT(L, NU)                                                                                                 \
+    do {                                                                                                                    \
+        if (L == 1 && bits == 8)                                                                                            \
+            hipLaunchKernelGGL((quant_pack_wave_rows_kernel<L, NU, (L == 1 ? 8 : 0), 4>), grid, block, 0, stream,              \
+                               reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits, symmetric,  \
+                               group_size);                                                                                 \
+        else                                                                                                                \
+            hipLaunchKernelGGL((quant_pack_wave_rows_kernel<L, NU, 0, 4>), grid, block, 0, stream,                            \
+                               reinterpret_cast<const uint4 *>(x), planes, scale, zero, group_sums, M, K, bits, symmetric,  \
+                               group_size);                                                                                 \
+    } while (0)
+#define ABQ_QP_SPLIT_NU(L)       \
+    do {                         \
+        if (nu4 <= 1)            \
+            ABQ_QP_SPLIT(L, 1);  \
+        else if (nu4 <= 2)       \
+            ABQ_QP_SPLIT(L, 2);  \
+        else if (nu4 <= 4)       \
+            ABQ_QP_SPLIT(L, 4);  \
+        else if (nu4 <= 6)       \
+            ABQ_QP_SPLIT(L, 6);  \
+        else                     \
+            ABQ_QP_SPLIT(L, 8);  \
+    } while (0)
+        if (layout == 2)
+            ABQ_QP_SPLIT_NU(2);
+        else if (layout == 1)
+            ABQ_QP_SPLIT_NU(1);
+        else
+            ABQ_QP_SPLIT_NU(0);
+#undef ABQ_QP_SPLIT_NU
+#undef ABQ_QP_SPLIT
+        return hipGetLastError();
+    }
+    // More rows than that: one wave per row, the row in registers (up to 12288 elements).
+    if (nu <= 24) {
         const dim3 grid((M + 3) / 4), block(256);
 #define ABQ_QP_WAVE(L, NU)                                                                                                  \
     do {                                                                                                                    \

@@ -56,7 +56,11 @@ def run_grouped(abq, xp, wp, signed, strategy="tiled", **kw):
 @pytest.mark.parametrize("rows,k,bits,symmetric", [(1, 128, 8, True), (5, 4096, 8, True), (33, 11008, 8, False),
                                                    (7, 256, 4, True), (16, 1152, 4, False), (3, 384, 2, True),
                                                    (64, 4096, 6, False), (9, 640, 5, False), (12, 512, 3, True),
-                                                   (3, 24576, 8, True), (2, 24704, 8, False)])  # last row kept in LDS / first not
+                                                   (3, 24576, 8, True), (2, 24704, 8, False),  # last row kept in LDS / first not
+                                                   # a workgroup per row up to here; beyond, one wave per row:
+                                                   (1100, 4096, 8, True), (2100, 5120, 8, False), (1030, 1024, 4, False),
+                                                   # the longest rows a workgroup's four waves hold in registers
+                                                   (20, 13824, 8, False), (4, 16384, 8, True), (300, 2048, 8, False)])
 def test_quant_pack_matches_the_restated_quantizer(abq, oracle, rows, k, bits, symmetric):
     from oracle import quantizer as Q
     rng = np.random.default_rng(rows + k + bits)
@@ -74,6 +78,10 @@ def test_quant_pack_matches_the_restated_quantizer(abq, oracle, rows, k, bits, s
     # K-tiled output equals the relayout of the plane output
     tiled, _, _, _ = abq.quant_pack_f16(torch.from_numpy(x).cuda(), bits, symmetric=symmetric, tiled=True)
     assert torch.equal(tiled, abq.relayout_planes(planes))
+    # ... also when the group sums are taken in the same pass
+    tiled, s_t, _, sums_t = abq.quant_pack_f16(torch.from_numpy(x).cuda(), bits, symmetric=symmetric, tiled=True, group_size=128)
+    assert torch.equal(tiled, abq.relayout_planes(planes)) and torch.equal(s_t, s)
+    assert np.array_equal(sums_t.cpu().numpy(), codes.reshape(rows, k // 128, 128).sum(axis=2))
     # FP6 records (codes of at most 5 bits) equal the FP6 relayout of the plane output
     if bits <= 5:
         rec, s6, _, _ = abq.quant_pack_f16(torch.from_numpy(x).cuda(), bits, symmetric=symmetric, fp6=True)
