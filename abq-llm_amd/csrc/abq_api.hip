@@ -20,7 +20,7 @@ hipError_t launch_pack_f16_tiled(const void *, const float *, uint32_t *, int, i
 hipError_t launch_pack_f16_fp6(const void *, const float *, uint32_t *, int, int, int, int, hipStream_t);
 hipError_t launch_pack_u4(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
 hipError_t launch_relayout_planes(const uint32_t *, uint32_t *, int, int, int, hipStream_t);
-hipError_t launch_relayout_planes_padded(const uint32_t *, uint32_t *, int, int, int, int, int, hipStream_t);
+hipError_t launch_relayout_planes_padded(const uint32_t *, uint32_t *, int, int, int, int, int, hipStream_t, int *row_sums = nullptr);
 hipError_t launch_relayout_planes_folded(const uint32_t *, const float *, int, uint32_t *, int, int, int, int, int, int *, hipStream_t);
 hipError_t launch_relayout_planes_fp6(const uint32_t *, uint32_t *, int, int, int, int, hipStream_t, const float *zero = nullptr,
                                       int group_size = 0, int *flag = nullptr);
@@ -1733,7 +1733,35 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
             return ABQ_ERR_INVALID_ARG;
         if (!biased && biased_x(st))
             return ABQ_ERR_INVALID_ARG; // biased activations only make sense against biased weights
-        if (xb) {
+        const KernelTable *t = find_table(st->strategy == ABQ_STRATEGY_DECODE_TILED
+                                              ? (x_dynamic         ? reg.decode_tiled_grouped_dyn
+                                                 : st->group_size ? reg.decode_tiled_grouped
+                                                 : x_f16          ? reg.decode_tiled_f16
+                                                                  : reg.decode_tiled)
+                                          : st->group_size ? reg.tiled_grouped
+                                                           : reg.tiled,
+                                          c.x_bits, c.w_bits, c.is_signed);
+        if (!t || st->variant < 0 || st->variant >= t->count)
+            return ABQ_ERR_NOT_INITIALIZED;
+        // Activations that arrive as planes and whose row sums a branch below will take from those planes: the
+        // conversion's launch takes the sums as well (further workgroups of the same grid), where that branch puts them.
+        bool x_sums_taken = false;
+        if (xb && !c.is_signed && !st->x_row_sums) {
+            const bool narrow = st->strategy == ABQ_STRATEGY_TILED && !biased && x_plane_bits(st) < c.x_bits && w_plane_bits(st) < c.w_bits;
+            const bool wanted = biased ? true
+                                : st->strategy == ABQ_STRATEGY_DECODE_TILED ? a.flip_w != 0
+                                : !narrow && (t->entries[st->variant].flags & kNeedsRowSums) && c.w_bits == 8;
+            const RowSumPlan plan = row_sum_plan(st, xb + wb);
+            if (wanted && plan.ok) {
+                e = launch_relayout_planes_padded(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, xrec, x_plane_bits(st), biased ? 2 : 0,
+                                                  (hipStream_t)stream, reinterpret_cast<int *>(ws + plan.x_off));
+                if (e != hipSuccess)
+                    return hip_status(e);
+                a.X = reinterpret_cast<const uint32_t *>(ws);
+                x_sums_taken = true;
+            }
+        }
+        if (xb && !x_sums_taken) {
             // (planes of fewer bits than the records: the codes are extended to the record's width)
             e = launch_relayout_planes_padded(st->X, reinterpret_cast<uint32_t *>(ws), st->M, st->K, xrec, x_plane_bits(st),
                                               biased ? 2 : (xrec != x_plane_bits(st) && c.is_signed ? 1 : 0), (hipStream_t)stream);
@@ -1748,16 +1776,6 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
                 return hip_status(e);
             a.W = reinterpret_cast<const uint32_t *>(ws + xb);
         }
-        const KernelTable *t = find_table(st->strategy == ABQ_STRATEGY_DECODE_TILED
-                                              ? (x_dynamic         ? reg.decode_tiled_grouped_dyn
-                                                 : st->group_size ? reg.decode_tiled_grouped
-                                                 : x_f16          ? reg.decode_tiled_f16
-                                                                  : reg.decode_tiled)
-                                          : st->group_size ? reg.tiled_grouped
-                                                           : reg.tiled,
-                                          c.x_bits, c.w_bits, c.is_signed);
-        if (!t || st->variant < 0 || st->variant >= t->count)
-            return ABQ_ERR_NOT_INITIALIZED;
         int variant = st->variant;
         if (st->strategy == ABQ_STRATEGY_TILED && !c.is_signed && !biased && x_plane_bits(st) < c.x_bits && w_plane_bits(st) < c.w_bits) {
             // Unsigned codes that leave the top bit of their records clear are signed codes of the records' width as
@@ -1775,7 +1793,7 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
             const RowSumPlan plan = row_sum_plan(st, xb + wb);
             if (!plan.ok)
                 return ABQ_ERR_INVALID_ARG; // both operands' sums are needed; the weights' must be set
-            if (!st->x_row_sums) {
+            if (!st->x_row_sums && !x_sums_taken) {
                 e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, x_plane_bits(st), (hipStream_t)stream);
                 if (e != hipSuccess)
                     return hip_status(e);
@@ -1804,7 +1822,8 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
             a.x_row_sums = st->x_row_sums;
             a.w_row_sums = st->w_row_sums;
             if (a.flip_w && !st->x_row_sums) {
-                e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, x_plane_bits(st), (hipStream_t)stream);
+                e = x_sums_taken ? hipSuccess
+                                 : launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, x_plane_bits(st), (hipStream_t)stream);
                 if (e != hipSuccess)
                     return hip_status(e);
                 a.x_row_sums = reinterpret_cast<const int *>(ws + plan.x_off);
@@ -1823,7 +1842,7 @@ abq_status abq_gemm_exec(const abq_gemm_state *st, void *stream)
             const bool need_x = c.w_bits == 8, need_w = c.x_bits == 8;
             const RowSumPlan plan = row_sum_plan(st, xb + wb);
             if (plan.ok) {
-                if (need_x && !st->x_row_sums) {
+                if (need_x && !st->x_row_sums && !x_sums_taken) {
                     e = launch_row_sums(st->X, reinterpret_cast<int *>(ws + plan.x_off), st->M, st->K, x_plane_bits(st), (hipStream_t)stream);
                     if (e != hipSuccess)
                         return hip_status(e);

@@ -152,6 +152,35 @@ template <int BITS> __device__ __forceinline__ bool fold_zero_point(uint32_t (&e
     return fits;
 }
 
+// sums[row] = sum over K of the unsigned codes of a row (bit b of an element counts 2^b): one wave per row, the
+// plane words read as 16-byte units along the lanes, a popcount per word and plane.  What the kernels that feed an
+// unsigned 8-bit operand as value - 128 add back in their epilogue (GemmArgs::x_row_sums / w_row_sums).
+// job: which four rows this workgroup takes.
+__device__ __forceinline__ void row_sums_of_four_rows(const uint32_t *__restrict__ planes, int *__restrict__ sums, int rows, int KW,
+                                                      int bits, int job)
+{
+    const int lane = threadIdx.x & 63;
+    const int row = job * 4 + (threadIdx.x >> 6);
+    if (row >= rows)
+        return; // whole waves, no barrier below
+    const size_t plane_stride = (size_t)rows * KW;
+    unsigned total = 0;
+    for (int b = 0; b < bits; ++b) {
+        const uint4 *p = reinterpret_cast<const uint4 *>(planes + b * plane_stride + (size_t)row * KW);
+        unsigned ones = 0;
+        for (int u = lane; u < KW / 4; u += 64) {
+            const uint4 v = p[u];
+            ones += __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
+        }
+        total += ones << b;
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1)
+        total += __shfl_xor(total, d);
+    if (lane == 0)
+        sums[row] = (int)total;
+}
+
 // One workgroup converts 32 rows x 8 K tiles.  A thread owns one record (one row, one K tile): it
 // reads 16 bytes per plane (eight threads cover 128 contiguous bytes of a plane row), converts its
 // four word-sets in registers, and parks the record in LDS; the records of one K tile are then
@@ -167,13 +196,19 @@ template <int BITS>
 __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__restrict__ planes,
                                                               uint32_t *__restrict__ tiled, int rows, int KW, int in_bits,
                                                               int sign_extend, const float *__restrict__ zero = nullptr,
-                                                              int group_size = 0, int *flag = nullptr)
+                                                              int group_size = 0, int *flag = nullptr, int *__restrict__ row_sums = nullptr)
 {
     constexpr int REC = BITS * 4;          // words per record
     constexpr int SLAB = 32 * REC + 4;     // words per K tile in LDS (+16 bytes against bank conflicts)
     __shared__ __align__(16) uint32_t buf[8 * SLAB];
     const int tid = threadIdx.x;
     const int kt_tiles = KW / 4;
+    // row_sums: the grid has further layers of workgroups behind those that convert, which take the rows' sums of codes
+    // from the same planes (one launch instead of two for an operand that needs both)
+    if (row_sums && (int)blockIdx.y >= (kt_tiles + 7) / 8) {
+        row_sums_of_four_rows(planes, row_sums, rows, KW, in_bits, ((int)blockIdx.y - (kt_tiles + 7) / 8) * (int)gridDim.x + (int)blockIdx.x);
+        return;
+    }
     const int row0 = blockIdx.x * 32, kt0 = blockIdx.y * 8;
     const size_t plane_stride = (size_t)rows * KW;
     {
@@ -231,13 +266,17 @@ __global__ __launch_bounds__(256) void relayout_planes_kernel(const uint32_t *__
 template <int BITS>
 __global__ __launch_bounds__(256) void relayout_planes_ws_kernel(const uint32_t *__restrict__ planes,
                                                                  uint32_t *__restrict__ tiled, int rows, int KW, int in_bits,
-                                                                 int sign_extend)
+                                                                 int sign_extend, int *__restrict__ row_sums = nullptr)
 {
     constexpr int REC = BITS * 4;          // words per record
     constexpr int SLAB = 8 * REC + 4;      // words per K tile in LDS (+16 bytes against bank conflicts)
     __shared__ __align__(16) uint32_t buf[8 * SLAB];
     const int tid = threadIdx.x;
     const int kt_tiles = KW / 4;
+    if (row_sums && (int)blockIdx.y >= (kt_tiles + 7) / 8) { // (see relayout_planes_kernel)
+        row_sums_of_four_rows(planes, row_sums, rows, KW, in_bits, ((int)blockIdx.y - (kt_tiles + 7) / 8) * (int)gridDim.x + (int)blockIdx.x);
+        return;
+    }
     const int row0 = blockIdx.x * 8, kt0 = blockIdx.y * 8;
     const size_t plane_stride = (size_t)rows * KW;
     {
@@ -271,17 +310,20 @@ __global__ __launch_bounds__(256) void relayout_planes_ws_kernel(const uint32_t 
 }
 
 // bits: width of the records written; in_bits <= bits: planes the operand has (sign_extend: what the rest repeats)
+// row_sums != nullptr: the rows' sums of codes (as abq_row_sums takes them from the in_bits planes) in the same launch.
 hipError_t launch_relayout_planes_padded(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits, int in_bits,
-                                         int sign_extend, hipStream_t stream)
+                                         int sign_extend, hipStream_t stream, int *row_sums)
 {
     const int KW = k / 32;
-    const dim3 grid((rows + 31) / 32, (KW / 4 + 7) / 8);
+    dim3 grid((rows + 31) / 32, (KW / 4 + 7) / 8);
+    const int sum_jobs = row_sums ? (rows + 3) / 4 : 0; // workgroups of four waves, a row each
     if ((long)grid.x * grid.y < 256) { // less than a workgroup per compute unit: the finer kernel
-        const dim3 fine((rows + 7) / 8, (KW / 4 + 7) / 8);
+        dim3 fine((rows + 7) / 8, (KW / 4 + 7) / 8);
+        fine.y += (sum_jobs + fine.x - 1) / fine.x;
         switch (bits) {
 #define ABQ_RELAYOUT_CASE(B)                                                                                     \
     case B:                                                                                                      \
-        hipLaunchKernelGGL(relayout_planes_ws_kernel<B>, fine, dim3(256), 0, stream, planes, tiled, rows, KW, in_bits, sign_extend); \
+        hipLaunchKernelGGL(relayout_planes_ws_kernel<B>, fine, dim3(256), 0, stream, planes, tiled, rows, KW, in_bits, sign_extend, row_sums); \
         break;
             ABQ_RELAYOUT_CASE(1) ABQ_RELAYOUT_CASE(2) ABQ_RELAYOUT_CASE(3) ABQ_RELAYOUT_CASE(4)
             ABQ_RELAYOUT_CASE(5) ABQ_RELAYOUT_CASE(6) ABQ_RELAYOUT_CASE(7) ABQ_RELAYOUT_CASE(8)
@@ -291,10 +333,12 @@ hipError_t launch_relayout_planes_padded(const uint32_t *planes, uint32_t *tiled
         }
         return hipGetLastError();
     }
+    grid.y += (sum_jobs + grid.x - 1) / grid.x;
     switch (bits) {
 #define ABQ_RELAYOUT_CASE(B)                                                                                     \
     case B:                                                                                                      \
-        hipLaunchKernelGGL(relayout_planes_kernel<B>, grid, dim3(256), 0, stream, planes, tiled, rows, KW, in_bits, sign_extend); \
+        hipLaunchKernelGGL(relayout_planes_kernel<B>, grid, dim3(256), 0, stream, planes, tiled, rows, KW, in_bits, sign_extend, \
+                           (const float *)nullptr, 0, (int *)nullptr, row_sums);                                 \
         break;
         ABQ_RELAYOUT_CASE(1) ABQ_RELAYOUT_CASE(2) ABQ_RELAYOUT_CASE(3) ABQ_RELAYOUT_CASE(4)
         ABQ_RELAYOUT_CASE(5) ABQ_RELAYOUT_CASE(6) ABQ_RELAYOUT_CASE(7) ABQ_RELAYOUT_CASE(8)
@@ -327,7 +371,7 @@ hipError_t launch_relayout_planes_folded(const uint32_t *planes, const float *ze
 
 hipError_t launch_relayout_planes(const uint32_t *planes, uint32_t *tiled, int rows, int k, int bits, hipStream_t stream)
 {
-    return launch_relayout_planes_padded(planes, tiled, rows, k, bits, bits, 0, stream);
+    return launch_relayout_planes_padded(planes, tiled, rows, k, bits, bits, 0, stream, nullptr);
 }
 
 // ---- FP6 records ---------------------------------------------------------------------------
@@ -463,32 +507,10 @@ __global__ __launch_bounds__(256) void relayout_planes_fp6_kernel(const uint32_t
     }
 }
 
-// sums[row] = sum over K of the unsigned codes of a row (bit b of an element counts 2^b): one wave per row, the
-// plane words read as 16-byte units along the lanes, a popcount per word and plane.  What the kernels that feed an
-// unsigned 8-bit operand as value - 128 add back in their epilogue (GemmArgs::x_row_sums / w_row_sums).
 __global__ __launch_bounds__(256) void row_sums_kernel(const uint32_t *__restrict__ planes, int *__restrict__ sums, int rows,
                                                        int KW, int bits)
 {
-    const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= rows)
-        return; // whole waves, no barrier below
-    const size_t plane_stride = (size_t)rows * KW;
-    unsigned total = 0;
-    for (int b = 0; b < bits; ++b) {
-        const uint4 *p = reinterpret_cast<const uint4 *>(planes + b * plane_stride + (size_t)row * KW);
-        unsigned ones = 0;
-        for (int u = lane; u < KW / 4; u += 64) {
-            const uint4 v = p[u];
-            ones += __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
-        }
-        total += ones << b;
-    }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1)
-        total += __shfl_xor(total, d);
-    if (lane == 0)
-        sums[row] = (int)total;
+    row_sums_of_four_rows(planes, sums, rows, KW, bits, blockIdx.x);
 }
 
 hipError_t launch_row_sums(const uint32_t *planes, int *sums, int rows, int k, int bits, hipStream_t stream)
