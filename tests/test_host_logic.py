@@ -732,3 +732,26 @@ def test_preferred_weight_records_name_the_padded_pair_for_widths_of_several_fie
         want = lib.abq_preferred_weight_layout(4, 4, 1, M, 5120, 5120, 0)
         assert ask(3, 3, 1, M) == ((F6, 3) if want == F6 else (T, 4))
     assert lib.abq_preferred_weight_records(6, 6, 1, 128, 5120, 5120, 0, None) == T
+
+
+def test_folded_record_entry_points_check_their_arguments(abq):
+    """abq_relayout_planes_folded / abq_relayout_planes_fp6_folded refuse, before any launch: null pointers, rows <= 0,
+    bit widths they have no records for (8-bit codes less a zero point need nine bits; FP6 holds differences of codes of
+    at most 4 bits), groups that are no multiple of 32 or do not divide K, K that is no multiple of 128."""
+    lib = abq.lib()
+    P = ctypes.c_void_p(0x1000)  # never dereferenced on the host: every call below returns before a launch
+    OK_K, G = 4096, 128
+    assert lib.abq_folded_bits(2) == 4 and lib.abq_folded_bits(3) == 4 and lib.abq_folded_bits(4) == 8
+    assert lib.abq_folded_bits(7) == 8 and lib.abq_folded_bits(8) == 0 and lib.abq_folded_bits(0) == 0
+    for fn, widest in ((lib.abq_relayout_planes_folded, 7), (lib.abq_relayout_planes_fp6_folded, 4)):
+        assert fn(None, P, G, P, 16, OK_K, 2, 1, P, None) == 1
+        assert fn(P, None, G, P, 16, OK_K, 2, 1, P, None) == 1
+        assert fn(P, P, G, None, 16, OK_K, 2, 1, P, None) == 1
+        assert fn(P, P, G, P, 0, OK_K, 2, 1, P, None) == 1
+        assert fn(P, P, G, P, 16, OK_K, 0, 1, P, None) == 1
+        assert fn(P, P, 48, P, 16, OK_K, 2, 1, P, None) == 1       # groups of whole plane words only
+        assert fn(P, P, 0, P, 16, OK_K, 2, 1, P, None) == 1
+        assert fn(P, P, G, P, 16, OK_K, widest + 1, 1, P, None) == 3
+        assert fn(P, P, G, P, 16, 4096 + 64, 2, 1, P, None) == 2
+        assert fn(P, P, G, P, 16, 64, 2, 1, P, None) == 2
+        assert fn(P, P, 96, P, 16, OK_K, 2, 1, P, None) == 2       # 96 does not divide 4096
