@@ -2131,6 +2131,16 @@ abq_status abq_gemm_set_workspace(abq_gemm_state *st, void *workspace, size_t by
         if (rc != ABQ_OK)
             return rc;
     }
+    // Weights prepared, activations still planes, 17 to 128 rows: the decode kernel of prepared operands where it is
+    // estimated ahead of the prefill tile; either kernel has the activations converted into the workspace first, so the
+    // estimate is the one of prepared activations (W2A8 32 x 4096 x 4096 from planes: 8.1 against 11.8 us).
+    if (st->strategy == ABQ_STRATEGY_TILED && st->auto_chosen && !st->group_size && !st->act && st->M > 16 && workspace &&
+        st->x_layout == ABQ_LAYOUT_PLANES && st->w_layout == ABQ_LAYOUT_TILED &&
+        decode_tiled_pays(st->cfg.x_bits, st->cfg.w_bits, st->M, st->N, st->K)) {
+        abq_gemm_state tmp = *st;
+        if (switch_to_decode_tiled(&tmp) == ABQ_OK && decode_tiled_x_ok(&tmp) && bytes >= abq_gemm_workspace_bytes(&tmp))
+            *st = tmp;
+    }
     apply_tuned(st); // (a tile that converts plane activations can be taken now that there is room for them)
     return ABQ_OK;
 }

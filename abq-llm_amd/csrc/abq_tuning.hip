@@ -212,8 +212,11 @@ int abq_preferred_weight_layout(int x_bits, int w_bits, int is_signed, int M, in
         return tile_operand_layout(t.cfg);
     // no measurement: FP6 records for the pairs that qualify once the GEMM is prefill-sized (the FP6 matrix cores run
     // at twice the int8 rate and nothing is unpacked), K-tiled records otherwise (every decode and prefill kernel
-    // that is not the FP6 one runs fastest on them)
-    if (M > 64 && abq_fp6_eligible(x_bits, w_bits, is_signed, K) && (group_size == 0 || group_size == 128))
+    // that is not the FP6 one runs fastest on them).  Up to 256 rows the int8 route's small tiles, whose waves split
+    // K, are level or ahead (W4A4 / W2A2, activations converted in the call, int8 / FP6 us: 128 x 4096 x 4096 12.0 /
+    // 13.9, 128 x 4096 x 11008 20.4 / 26.0, 256 x 4096 x 4096 13.1 / 14.4, 256 x 11008 x 4096 22.8 / 23.1; 384 x 11008 x 4096
+    // 31.5 / 27.2, 512 x 4096 x 4096 with prepared activations 12.5 / 10.9).
+    if (M > 256 && abq_fp6_eligible(x_bits, w_bits, is_signed, K) && (group_size == 0 || group_size == 128))
         return ABQ_LAYOUT_FP6;
     return ABQ_LAYOUT_TILED;
 }

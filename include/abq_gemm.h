@@ -395,7 +395,7 @@ void abq_tuning_enable_builtin(int on);
 abq_status abq_tuning_lookup(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size, int layout_mask,
                              abq_tile_config *cfg, float *tops);
 /* The abq_layout a loader should prepare a weight matrix in for GEMMs of about M rows: the layout of the table's best
- * entry for the shape; without one, FP6 records for pairs that qualify (abq_fp6_eligible) from 65 rows up, K-tiled
+ * entry for the shape; without one, FP6 records for pairs that qualify (abq_fp6_eligible) from 257 rows up, K-tiled
  * records otherwise.  (A model that runs prefill and decode on one matrix keeps both where the memory allows.) */
 int abq_preferred_weight_layout(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size);
 /* The same for a loader that can also write padded records (abq_relayout_planes_padded): *record_bits receives the
@@ -502,7 +502,10 @@ size_t abq_gemm_workspace_bytes(const abq_gemm_state *state);
 /* Hands a caller-owned device buffer to the state.  If the tile was the library's choice, M > 64
  * (32 for outputs of 8192 columns or more; 16 with group scales) and the buffer is large enough, the
  * state moves to ABQ_STRATEGY_TILED; otherwise it keeps its kernel (which needs no workspace:
- * below those sizes the conversion launch costs more than the LDS-staged kernel gains). */
+ * below those sizes the conversion launch costs more than the LDS-staged kernel gains).  A state on
+ * ABQ_STRATEGY_TILED whose weights are K-tiled and whose activations are planes, 17 to 128 rows, moves to
+ * ABQ_STRATEGY_DECODE_TILED where that kernel is estimated ahead (either converts the activations into the
+ * workspace first; size the buffer with abq_gemm_workspace_bytes before and after: the need does not grow). */
 abq_status abq_gemm_set_workspace(abq_gemm_state *state, void *workspace, size_t bytes);
 
 /* Replaces AqBMMAExecFn / AqBWMMAExecFn (engine/mma_any/aq_bmma_op.h:155-161,164): one

@@ -637,6 +637,30 @@ def test_prefill_pads_activations_of_several_fields_by_itself(abq, oracle):
     assert g.state.cfg.x_bits == 6
 
 
+@pytest.mark.parametrize("q,p,signed", [(8, 2, True), (4, 4, True), (2, 2, True), (8, 8, True), (4, 4, False), (8, 4, True)])
+def test_small_batches_from_planes_on_the_prepared_decode_kernel(abq, oracle, q, p, signed):
+    """Weights prepared, activations handed over as planes, 17 to 128 rows: once the state has a workspace it runs the
+    decode kernel of prepared operands wherever it would on prepared activations (exec converts the planes first, over
+    several blocks of rows); without a workspace it stays on the prefill kernel.  Bit exact either way."""
+    rng = np.random.default_rng(1700 + 10 * q + p + int(signed))
+    took_decode = 0
+    for (M, N, K) in [(17, 64, 512), (40, 200, 1408), (64, 4096, 1024), (100, 130, 4096), (128, 264, 1152), (33, 96, 11008)]:
+        x, w = rand_vals(rng, M, K, q, signed), rand_vals(rng, N, K, p, signed)
+        xd, wt = planes_dev(oracle.pack_i32(x, q)), abq.relayout_planes(planes_dev(oracle.pack_i32(w, p)))
+        want = oracle.np_gemm(x, w)
+        on_records = abq.Gemm(abq.relayout_planes(xd), wt, signed, x_tiled=True, w_tiled=True)
+        g = abq.Gemm(xd, wt, signed, w_tiled=True)
+        assert g.strategy == "tiled"
+        ws = torch.empty(max(g.workspace_bytes, M * K * q // 8 + 4096), dtype=torch.uint8, device="cuda")
+        g = abq.Gemm(xd, wt, signed, w_tiled=True, workspace=ws)
+        assert g.strategy == on_records.strategy, (M, N, K, g.strategy, on_records.strategy)
+        assert g.workspace_bytes <= ws.numel()
+        took_decode += g.strategy == "decode_tiled"
+        assert np.array_equal(g.run().cpu().numpy(), want), (g.config_name, M, N, K)
+        assert np.array_equal(on_records.run().cpu().numpy(), want), (on_records.config_name, M, N, K)
+    assert took_decode >= 2
+
+
 FIELD_PAIRS = [(3, 3), (5, 5), (6, 6), (7, 7), (8, 3), (6, 2)]  # a width of several fields on either side
 
 

@@ -464,15 +464,16 @@ def test_a_loaded_tuning_table_overrides_the_rules(abq, tmp_path):
     try:
         assert lib.abq_tuning_lookup(4, 4, 1, 128, N, K, 0, 0, ctypes.byref(abq.TileConfig()), None) == abq.ABQ_ERR_UNSUPPORTED
         by_rules = tile_after(4, 4, 128, P, T, workspace=True)[0]
+        by_rules_no_room = tile_after(4, 4, 128, P, T)[0]  # (nowhere to convert the activations: no decode kernel)
         by_rules_planes = tile_after(4, 4, 128, P, P)[0]
         by_rules_fp6 = tile_after(4, 4, 128, F6, F6)[0]
         # three measured tiles for the shape, one per operand layout, none of them the rules' choice
         tiled_tile = "AqBMMA_4x4xtrue_128x64x128_64x32x128_32x32x32_4"
-        decode_tile = "AqBMMA_4x4xtrue_16x32x1024_16x32x128_16x16x64_6"
+        decode_tile = "AqBMMA_4x4xtrue_16x16x2048_16x16x128_16x16x64_6"
         fp6_tile = "AqBMMA_4x4xtrue_128x128x128_64x64x128_32x32x64_5"
         planes_tile = "AqBMMA_4x4xtrue_64x64x256_32x32x256_32x32x32_2"
         for name in (tiled_tile, decode_tile, fp6_tile, planes_tile):
-            assert name not in (by_rules, by_rules_planes, by_rules_fp6)
+            assert name not in (by_rules, by_rules_no_room, by_rules_planes, by_rules_fp6)
         table = tmp_path / "tuned.txt"
         table.write_text("# measured\n%s 128 %d %d 0 500.0\n%s 100 %d %d 0 450.5\n%s 128 %d %d 0 300\n"
                          % (tiled_tile, N, K, fp6_tile, N, K, planes_tile, N, K))
@@ -502,7 +503,7 @@ def test_a_loaded_tuning_table_overrides_the_rules(abq, tmp_path):
         cfg2 = abq.parse_kernel_name(decode_tile)[0]
         assert lib.abq_tuning_add(ctypes.byref(cfg2), 128, N, K, 0, 600.0) == 0
         assert tile_after(4, 4, 128, T, T)[:2] == (decode_tile, "decode_tiled")
-        assert tile_after(4, 4, 128, P, T)[0] == tiled_tile or tile_after(4, 4, 128, P, T)[0] == by_rules
+        assert tile_after(4, 4, 128, P, T)[0] in (tiled_tile, by_rules_no_room)
         assert tile_after(4, 4, 128, P, T, workspace=True)[:2] == (decode_tile, "decode_tiled")
         # a tile the caller names is not moved
         pinned = abq.parse_kernel_name("AqBMMA_4x4xtrue_64x64x128_32x32x128_32x32x32_4")[0]
@@ -755,3 +756,33 @@ def test_folded_record_entry_points_check_their_arguments(abq):
         assert fn(P, P, G, P, 16, 4096 + 64, 2, 1, P, None) == 2
         assert fn(P, P, G, P, 16, 64, 2, 1, P, None) == 2
         assert fn(P, P, 96, P, 16, OK_K, 2, 1, P, None) == 2       # 96 does not divide 4096
+
+
+def test_small_batches_with_plane_activations_reach_the_prepared_decode_kernel_once_there_is_a_workspace(abq):
+    """Weights prepared, activations still planes, 17 to 128 rows: with a workspace to convert the activations into, the
+    state moves to the decode kernel of prepared operands wherever it would with prepared activations (either kernel
+    converts them first); without one, with group scales, or where the prefill tile is estimated ahead, it stays."""
+    lib = abq.lib()
+    T, P = abq.LAYOUT_TILED, abq.LAYOUT_PLANES
+    names = abq.STRATEGY_NAMES
+
+    def strategy(q, p, M, N, K, xl, workspace):
+        rc, st = _init(abq, q=q, p=p, M=M, signed=1, N=N, K=K)
+        assert rc == 0 and lib.abq_gemm_set_operand_layout(ctypes.byref(st), xl, T) == 0
+        if workspace:
+            assert lib.abq_gemm_set_workspace(ctypes.byref(st), 0x100000, 256 << 20) == 0
+            assert lib.abq_gemm_workspace_bytes(ctypes.byref(st)) <= 256 << 20
+        return names[st.strategy]
+
+    lib.abq_tuning_clear()
+    lib.abq_tuning_enable_builtin(0)  # the rules alone
+    try:
+        for (q, p, M, N, K) in [(8, 2, 32, 4096, 4096), (4, 4, 64, 4096, 4096), (2, 2, 48, 4096, 11008), (8, 2, 24, 4096, 11008),
+                                (8, 2, 128, 11008, 4096), (8, 8, 64, 4096, 4096), (8, 2, 300, 4096, 4096)]:
+            with_records = strategy(q, p, M, N, K, T, False)
+            assert strategy(q, p, M, N, K, P, True) == with_records
+            assert strategy(q, p, M, N, K, P, False) == "tiled"
+        assert strategy(8, 2, 32, 4096, 4096, P, True) == "decode_tiled" and strategy(2, 2, 48, 4096, 11008, P, True) == "decode_tiled"
+        assert strategy(8, 2, 128, 11008, 4096, P, True) == "tiled" and strategy(8, 2, 300, 4096, 4096, P, True) == "tiled"
+    finally:
+        lib.abq_tuning_enable_builtin(1)
