@@ -366,7 +366,11 @@ void ABQGEMMWrapper::gemm_dynamic(const int M, const int N, const int K, const _
     // (if the expanded activations fit the decode kernel's LDS: partial tiles, group sums, M padded rows)
     const bool decode = !decode_prepared && M <= 16 && W.planes != nullptr &&
                         (silu_gate ? 32 : 16) * 1024 + (size_t)64 * (K / W.group_size) + 128 + (size_t)M * ((K + 511) / 512 * 512 + 16) <= 160 * 1024;
-    const bool fp6 = !decode && !decode_prepared && records_fp6 != nullptr && W.group_size == 128 && abq_fp6_eligible(x_bits_, w_bits_, 1, K);
+    // (FP6 records where the library prefers them for the shape: from 257 rows unless a measured entry says otherwise; below,
+    // the int8 route's small tiles are ahead, W4A4 with groups of 128 at 128 x 4096 x 4096 13.7 against 19.7 us.  A weight
+    // that has no other records runs on them at every size.)
+    const bool fp6 = !decode && !decode_prepared && records_fp6 != nullptr && W.group_size == 128 && abq_fp6_eligible(x_bits_, w_bits_, 1, K) &&
+                     (w_records == nullptr || abq_preferred_weight_layout(x_bits_, w_bits_, 1, M, N, K, 128) == ABQ_LAYOUT_FP6);
     const int layout = decode ? ABQ_LAYOUT_PLANES : fp6 ? ABQ_LAYOUT_FP6 : ABQ_LAYOUT_TILED;
     abq_status rc;
     abq_gemm_state state;
