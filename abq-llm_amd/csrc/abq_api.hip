@@ -823,7 +823,14 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
         const long tiles = (long)((st->M + bm - 1) / bm) * ((st->N + bn - 1) / bn);
         // (signed W8A8, which keeps its one-group tiles on small grids: 128x64 from one workgroup per compute unit,
         // 512 x 4096 x 4096 844 against 794 TOPS on 64x64)
-        const long need = (staged && o[0] == 2 && o[1] == 2 && o[2] == 4) ? 160 : (staged && o[0] == 2 && o[1] == 1) ? 256 : o[4];
+        // (and both 128x128 and 128x64 from 160 workgroups: more than 256 of the smaller tile, whose stages fill a compute
+        // unit's LDS, are a second round on part of the chip: 256 x 11008 x 4096 28.1 on 128x128 against 35.4 us on 128x64,
+        // 768 x 4096 x 4096 29.2 against 32.1; 128 x 11008 x 4096 22.0 on 128x64 against 25.9 on 64x64, 384 x 4096 x 4096 21.2
+        // against 21.9; 256 x 4096 x 4096, 128 workgroups of 128x64, stays on 64x64: 16.2)
+        const long need = (staged && o[0] == 2 && o[1] == 2 && o[2] == 4) ? 160
+                          : (staged && o[0] == 2 && o[1] == 2 && o[2] == 2) ? 160
+                          : (staged && o[0] == 2 && o[1] == 1)              ? 160
+                                                                            : o[4];
         for (int i = 0; i < tt->count; ++i)
             if (tt->entries[i].tm == o[0] && tt->entries[i].tn == o[1] && tt->entries[i].kb == 128 && tt->entries[i].wk == 1 &&
                 tt->entries[i].wm == o[2] && tt->entries[i].wn == o[3] && tiles >= need && pick < 0)
@@ -847,6 +854,12 @@ static abq_status switch_to_tiled(abq_gemm_state *st)
             want[4] = 2;
             want[0] = n64x64 <= 256 ? 1 : along_n ? 1 : 2; // 64x64 up to one workgroup per compute unit
             want[1] = n64x64 <= 256 ? 1 : along_n ? 2 : 1;
+            // The stages of these tiles fill most of a compute unit's LDS: more than 256 workgroups of the 64x128 (128x64)
+            // tile are a second round on part of the chip, and the 128x128 tile with the same split, one round below 200
+            // tiles, is ahead (256 x 11008 x 4096: W4A8 23.2 against 30.2 us, W2A8 22.1 against 24.0, W4A4 22.3 against 24.3;
+            // 768 x 4096 x 4096: W4A8 24.5 against 29.7).
+            if ((long)((st->M + 32 * want[0] * 2 - 1) / (32 * want[0] * 2)) * ((st->N + 32 * want[1] * 2 - 1) / (32 * want[1] * 2)) > 256)
+                want[0] = want[1] = 2;
         } else if (tt->entries[pick].lds != 0 && t128 <= 256 && c.x_bits + c.w_bits < 16) {
             // exactly one round of 128x128 tiles: that tile with the split (1024 x 4096 x 11008: W2A8 1725 against 1611
             // TOPS on 64x128, W4A4 1686 against 1530 on 128x128; on K = 4096 level with the best)

@@ -216,7 +216,10 @@ int abq_preferred_weight_layout(int x_bits, int w_bits, int is_signed, int M, in
     // K, are level or ahead (W4A4 / W2A2, activations converted in the call, int8 / FP6 us: 128 x 4096 x 4096 12.0 /
     // 13.9, 128 x 4096 x 11008 20.4 / 26.0, 256 x 4096 x 4096 13.1 / 14.4, 256 x 11008 x 4096 22.8 / 23.1; 384 x 11008 x 4096
     // 31.5 / 27.2, 512 x 4096 x 4096 with prepared activations 12.5 / 10.9).
-    if (M > 256 && abq_fp6_eligible(x_bits, w_bits, is_signed, K) && (group_size == 0 || group_size == 128))
+    // Weights of at most 2 bits are 32 bytes per row and K tile on the int8 route against 96 as FP6 records: level only
+    // from 2048 rows (W2A2 768 x 4096 x 4096 20.1 / 26.2, 1024 x 11008 x 4096 42.6 / 51.9, 2048 x 4096 x 4096 33.0 / 28.9,
+    // 2048 x 11008 x 4096 72.8 / 75.7).
+    if (M > (w_bits <= 2 ? 1024 : 256) && abq_fp6_eligible(x_bits, w_bits, is_signed, K) && (group_size == 0 || group_size == 128))
         return ABQ_LAYOUT_FP6;
     return ABQ_LAYOUT_TILED;
 }

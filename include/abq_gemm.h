@@ -395,7 +395,7 @@ void abq_tuning_enable_builtin(int on);
 abq_status abq_tuning_lookup(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size, int layout_mask,
                              abq_tile_config *cfg, float *tops);
 /* The abq_layout a loader should prepare a weight matrix in for GEMMs of about M rows: the layout of the table's best
- * entry for the shape; without one, FP6 records for pairs that qualify (abq_fp6_eligible) from 257 rows up, K-tiled
+ * entry for the shape; without one, FP6 records for pairs that qualify (abq_fp6_eligible) from 257 rows up (1025 for weights of at most 2 bits), K-tiled
  * records otherwise.  (A model that runs prefill and decode on one matrix keeps both where the memory allows.) */
 int abq_preferred_weight_layout(int x_bits, int w_bits, int is_signed, int M, int N, int K, int group_size);
 /* The same for a loader that can also write padded records (abq_relayout_planes_padded): *record_bits receives the

@@ -667,6 +667,17 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(8, 2, 1024, 4096, 4096, T) == (128, 128, 256, 64, 64, 4)     # one round of 128x128 tiles: with the split
     assert picked(4, 4, 1024, 4096, 11008, T) == (128, 128, 256, 64, 64, 4)
     assert picked(8, 8, 1024, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)     # (not built for W8A8)
+    # the tiles whose waves split K stay within one round of workgroups: past 256 of the 64x128 (128x64) tile, 128x128
+    assert picked(8, 4, 256, 11008, 4096, T) == (128, 128, 256, 64, 64, 4)
+    assert picked(8, 2, 192, 11008, 4096, T) == (128, 128, 256, 64, 64, 4)
+    assert picked(4, 4, 256, 11008, 4096, T) == (128, 128, 256, 64, 64, 4)
+    assert picked(8, 4, 768, 4096, 4096, T) == (128, 128, 256, 64, 64, 4)
+    assert picked(8, 4, 384, 4096, 4096, T) == (64, 128, 256, 32, 64, 4)      # 192 workgroups: as before
+    # signed W8A8: 128x64 and 128x128 from 160 workgroups (more than 256 of the smaller tile would be a second round)
+    assert picked(8, 8, 128, 11008, 4096, T) == (128, 64, 128, 64, 32, 4)
+    assert picked(8, 8, 256, 11008, 4096, T) == (128, 128, 128, 64, 64, 4)
+    assert picked(8, 8, 768, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)
+    assert picked(8, 8, 256, 4096, 4096, T) == (64, 64, 128, 32, 32, 4)
     # signed W8A8: 256x128 as soon as it fills the chip
     assert picked(8, 8, 2048, 4096, 4096, T) == (256, 128, 128, 64, 64, 4)
     assert picked(8, 8, 1024, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)
