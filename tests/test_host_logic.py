@@ -678,6 +678,9 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     assert picked(8, 8, 256, 11008, 4096, T) == (128, 128, 128, 64, 64, 4)
     assert picked(8, 8, 768, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)
     assert picked(8, 8, 256, 4096, 4096, T) == (64, 64, 128, 32, 32, 4)
+    # ... and on long K, up to one round of 128x64 tiles, that tile with its waves splitting K
+    assert picked(8, 8, 512, 4096, 11008, T) == (128, 64, 256, 64, 32, 4)
+    assert picked(8, 8, 512, 4096, 4096, T) == (128, 64, 128, 64, 32, 4)
     # signed W8A8: 256x128 as soon as it fills the chip
     assert picked(8, 8, 2048, 4096, 4096, T) == (256, 128, 128, 64, 64, 4)
     assert picked(8, 8, 1024, 4096, 4096, T) == (128, 128, 128, 64, 64, 4)
