@@ -1204,12 +1204,13 @@ static abq_status pick_grouped_tiled(abq_gemm_state *state)
         // The fold of the int32 tiles into fp32 bounds these kernels more than the tile traffic does, so tile
         // sizes from 128x128 up run within a few percent of each other (sweep over M = 256 .. 16384 and the
         // LLaMA widths): 128x128 once it fills the chip, below that 128x64, then 64x64.  With activations of
-        // at most 4 bits three workgroups of 128x64 fit a compute unit and stay ahead up to 400 tiles.
+        // at most 4 bits three workgroups of 128x64 fit a compute unit and stay ahead up to 400 tiles.  (8-bit activations:
+        // from the first tile past one round, 384 x 11008 x 4096 = 258 tiles: W2A8 40.3 against 46.9 us on 128x64.)
         const long t128 = (long)((state->M + 127) / 128) * ((state->N + 127) / 128);
         // W8A8 has the staged kernel at 128x64 only, and that runs 7-9 % ahead of the register-staged 128x128
         // (16384 x 4096 x 4096 / x 11008, 2048 x 12288 x 4096: 1098 / 1146 / 1038 against 1027 / 1038 / 1004 TOPS).
         const bool both8 = c.x_bits == 8 && c.w_bits == 8;
-        const int order[][3] = { { 128, 128, both8 ? 1 << 30 : c.x_bits <= 4 ? 400 : 300 }, { 128, 64, 64 }, { 64, 64, 0 } };
+        const int order[][3] = { { 128, 128, both8 ? 1 << 30 : c.x_bits <= 4 ? 400 : 257 }, { 128, 64, 64 }, { 64, 64, 0 } };
         for (const auto &o : order) {
             if (pick >= 0 || t128 < o[2])
                 continue;

@@ -511,7 +511,7 @@ def test_a_loaded_tuning_table_overrides_the_rules(abq, tmp_path):
         assert rc == 0 and lib.abq_gemm_set_operand_layout(ctypes.byref(st), T, T) == 0
         assert st.cfg.as_tuple() == pinned.as_tuple()
         # group scales: their own entries (group size is part of the key), taken where the tile is picked
-        g_tile = "AqBMMA_8x2xtrue_128x128x128_64x64x128_32x32x32_4"
+        g_tile = "AqBMMA_8x2xtrue_256x128x128_64x64x128_32x32x32_4"
         assert tile_after(8, 2, 1024, T, T, group=128)[0] != g_tile
         assert lib.abq_tuning_add(ctypes.byref(abq.parse_kernel_name(g_tile)[0]), 1024, N, K, 128, 1000.0) == 0
         assert tile_after(8, 2, 1024, T, T, group=128)[0] == g_tile
@@ -703,7 +703,8 @@ def test_prefill_tile_choice_on_the_baseline_shapes(abq):
     # 384 workgroups would be two rounds of it: the 128x128 tile with the same split while that makes one round
     assert picked(8, 2, 192, 12288, 4096, T, group=128) == (128, 128, 256, 64, 64, 4)
     assert picked(8, 2, 128, 22016, 4096, T, group=128) == (128, 128, 256, 64, 64, 4)
-    assert picked(8, 2, 384, 12288, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)   # 288 tiles of 128x128: neither
+    assert picked(8, 2, 384, 12288, 4096, T, group=128) == (128, 128, 128, 64, 64, 4)  # 288 tiles of 128x128: that tile, no split
+    assert picked(4, 4, 384, 12288, 4096, T, group=128) == (128, 64, 128, 64, 32, 4)   # (narrow activations: 128x64 up to 400)
     assert picked(8, 2, 64, 22016, 4096, T, group=128) == (64, 128, 256, 32, 64, 4)    # ... one round of the 64x128 one
     assert picked(4, 4, 64, 22016, 4096, T, group=128) == (128, 128, 256, 64, 64, 4)   # (built for activations wider than weights)
     # ... activations of at most 4 bits keep 128x64 up to 400 tiles
